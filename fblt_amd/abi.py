@@ -1,0 +1,131 @@
+"""ctypes view of the boundary structs declared in include/blt_abi.h.
+
+Field order and types follow that header one to one; `check_layout()` asserts
+the sizes the header's static assertions state, so a drift between the two is
+caught at import time.
+"""
+import ctypes as C
+
+BLT_BACKEND_CPU = 0
+BLT_BACKEND_HIP = 1
+
+BLT_DTYPE_FP32 = 0
+
+BLT_BDM_TRAIN = 0
+BLT_BDM_INFER = 1
+
+BLT_MAX_NDIM = 4
+
+c_float_p = C.POINTER(C.c_float)
+c_size_p = C.POINTER(C.c_size_t)
+
+
+class BltTensor(C.Structure):
+    _fields_ = [
+        ("data", C.c_void_p),
+        ("shape", C.c_size_t * BLT_MAX_NDIM),
+        ("strides", C.c_size_t * BLT_MAX_NDIM),
+        ("ndim", C.c_size_t),
+        ("numel", C.c_size_t),
+        ("dtype", C.c_int),
+        ("backend", C.c_int),
+        ("is_view", C.c_bool),
+    ]
+
+
+class BltArena(C.Structure):
+    _fields_ = [
+        ("buffer", C.c_void_p),
+        ("capacity", C.c_size_t),
+        ("offset", C.c_size_t),
+        ("backend", C.c_int),
+    ]
+
+
+class BltAttentionHeadArgs(C.Structure):
+    _fields_ = [
+        ("q", C.c_void_p),
+        ("q_stride", C.c_size_t),
+        ("k", C.c_void_p),
+        ("k_stride", C.c_size_t),
+        ("v", C.c_void_p),
+        ("v_stride", C.c_size_t),
+        ("combined", C.c_void_p),
+        ("combined_stride", C.c_size_t),
+        ("combined_col_offset", C.c_size_t),
+        ("weights_out", C.c_void_p),
+        ("lse_out", C.c_void_p),
+        ("scores_scratch", C.c_void_p),
+        ("mask", C.c_void_p),
+        ("nq", C.c_size_t),
+        ("nk", C.c_size_t),
+        ("head_dim", C.c_size_t),
+        ("is_causal", C.c_bool),
+        ("scale", C.c_float),
+    ]
+
+
+class BltMaskConfig(C.Structure):
+    _fields_ = [
+        ("seq_len_q", C.c_size_t),
+        ("seq_len_kv", C.c_size_t),
+        ("sliding_window", C.c_size_t),
+        ("doc_boundaries", c_size_p),
+        ("num_docs", C.c_size_t),
+        ("query_group_ids", c_size_p),
+        ("kv_group_ids", c_size_p),
+        ("bidirectional_within_group", C.c_bool),
+        ("is_causal", C.c_bool),
+        ("causal_offset", C.c_size_t),
+    ]
+
+
+class BltBlockDiffusionConfig(C.Structure):
+    _fields_ = [
+        ("mode", C.c_int),
+        ("seq_len", C.c_size_t),
+        ("num_clean", C.c_size_t),
+        ("block_size", C.c_size_t),
+        ("block_starts", c_size_p),
+        ("num_blocks", C.c_size_t),
+    ]
+
+
+class BltPatchInfo(C.Structure):
+    _fields_ = [
+        ("start_idx", C.c_size_t),
+        ("length", C.c_size_t),
+        ("peak_entropy", C.c_float),
+    ]
+
+
+def check_layout():
+    assert C.sizeof(BltTensor) == 104
+    assert C.sizeof(BltArena) == 32
+    assert C.sizeof(BltAttentionHeadArgs) == 136
+    assert BltAttentionHeadArgs.mask.offset == 96
+    assert BltAttentionHeadArgs.is_causal.offset == 128
+    assert BltAttentionHeadArgs.scale.offset == 132
+    assert C.sizeof(BltMaskConfig) == 72
+    assert BltMaskConfig.causal_offset.offset == 64
+    assert C.sizeof(BltBlockDiffusionConfig) == 48
+    assert C.sizeof(BltPatchInfo) == 24
+
+
+check_layout()
+
+
+def size_array(values):
+    """A ctypes size_t[] holding `values` (kept alive by the caller)."""
+    values = [int(v) for v in values]
+    return (C.c_size_t * max(len(values), 1))(*values)
+
+
+def patch_array(starts, lengths):
+    n = len(starts)
+    arr = (BltPatchInfo * max(n, 1))()
+    for i in range(n):
+        arr[i].start_idx = int(starts[i])
+        arr[i].length = int(lengths[i])
+        arr[i].peak_entropy = 0.0
+    return arr

@@ -1,0 +1,154 @@
+"""ctypes binding of libfblt_hip.so (the C-ABI declared in include/blt_hip.h).
+
+PyTorch is used by callers only to own device memory; every signature here is
+plain pointers and sizes.  There is no fallback: if the library is missing,
+`load()` raises.
+"""
+import ctypes as C
+import os
+
+from . import abi
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libfblt_hip.so")
+
+BLT_ATTN_MASK_FROM_HEAD = 0
+BLT_ATTN_MASK_CAUSAL = 1
+BLT_ATTN_MASK_ROW_RANGE = 2
+
+BLT_KV_STEP_CAUSAL = 0
+BLT_KV_STEP_BLOCK = 1
+
+
+class BltAttentionProblem(C.Structure):
+    _fields_ = [
+        ("head", abi.BltAttentionHeadArgs),
+        ("mask_kind", C.c_uint32),
+        ("reserved", C.c_uint32),
+        ("causal_offset", C.c_size_t),
+        ("window", C.c_size_t),
+        ("row_lo", C.c_void_p),
+        ("row_hi", C.c_void_p),
+    ]
+
+
+class BltKvAttnCache(C.Structure):
+    _fields_ = [
+        ("self_k", C.c_void_p),
+        ("self_v", C.c_void_p),
+        ("self_len", C.c_void_p),
+        ("batch", C.c_size_t),
+        ("max_seq_len", C.c_size_t),
+        ("embed_dim", C.c_size_t),
+        ("num_heads", C.c_size_t),
+        ("window", C.c_size_t),
+    ]
+
+
+# name -> (restype, argtypes); every symbol include/blt_hip.h declares
+SYMBOLS = {
+    "blt_attention_head_core_hip": (None, [C.c_int, C.POINTER(abi.BltAttentionHeadArgs)]),
+    "blt_build_attention_mask_hip": (None, [C.POINTER(abi.BltMaskConfig), C.POINTER(abi.BltTensor),
+                                            C.POINTER(abi.BltArena)]),
+    "blt_build_block_diffusion_mask_hip": (None, [C.POINTER(abi.BltBlockDiffusionConfig), C.POINTER(abi.BltTensor),
+                                                  C.POINTER(abi.BltArena)]),
+    "blt_strided_copy_hip": (None, [C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t,
+                                    C.c_size_t]),
+    "blt_softmax_masked_row_inplace_hip": (None, [C.c_int, C.c_void_p, C.c_size_t, C.c_size_t, C.c_bool, C.c_void_p,
+                                                  C.c_float]),
+    "blt_vec_dot_hip": (C.c_float, [C.c_int, C.c_void_p, C.c_void_p, C.c_size_t]),
+    "blt_hip_malloc": (C.c_void_p, [C.c_size_t]),
+    "blt_hip_free": (None, [C.c_void_p]),
+    "blt_hip_memset": (None, [C.c_void_p, C.c_int, C.c_size_t]),
+    "blt_hip_memcpy_h2d": (None, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "blt_hip_memcpy_d2h": (None, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "blt_backend_pass_sync_hip": (None, []),
+    "blt_arena_create": (C.POINTER(abi.BltArena), [C.c_size_t, C.c_int]),
+    "blt_arena_destroy": (None, [C.POINTER(abi.BltArena)]),
+    "blt_arena_reset": (None, [C.POINTER(abi.BltArena)]),
+    "blt_arena_alloc": (C.c_void_p, [C.POINTER(abi.BltArena), C.c_size_t, C.c_size_t]),
+    "blt_tensor_create": (abi.BltTensor, [C.POINTER(abi.BltArena), C.POINTER(C.c_size_t), C.c_size_t, C.c_int]),
+    "blt_tensor_create_uninit": (abi.BltTensor, [C.POINTER(abi.BltArena), C.POINTER(C.c_size_t), C.c_size_t,
+                                                 C.c_int]),
+    "blt_tensor_upload": (None, [C.POINTER(abi.BltTensor), C.c_void_p, C.c_size_t]),
+    "blt_tensor_download": (None, [C.POINTER(abi.BltTensor), C.c_void_p, C.c_size_t]),
+    "blt_backend_pass_sync": (None, [C.c_int]),
+    "blt_attention_head_core": (None, [C.c_int, C.POINTER(abi.BltAttentionHeadArgs)]),
+    "blt_build_attention_mask": (None, [C.POINTER(abi.BltMaskConfig), C.POINTER(abi.BltTensor),
+                                        C.POINTER(abi.BltArena)]),
+    "blt_build_block_diffusion_mask": (None, [C.POINTER(abi.BltBlockDiffusionConfig), C.POINTER(abi.BltTensor),
+                                              C.POINTER(abi.BltArena)]),
+    "blt_strided_copy": (None, [C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t]),
+    "blt_softmax_masked_row_inplace": (None, [C.c_int, C.c_void_p, C.c_size_t, C.c_size_t, C.c_bool, C.c_void_p,
+                                              C.c_float]),
+    "blt_vec_dot": (C.c_float, [C.c_int, C.c_void_p, C.c_void_p, C.c_size_t]),
+    "blt_patch_build_group_ids": (None, [C.POINTER(abi.BltPatchInfo), C.c_size_t, C.c_size_t, abi.c_size_p,
+                                         abi.c_size_p]),
+    "blt_patch_decoder_latent_at": (C.c_size_t, [C.POINTER(abi.BltPatchInfo), C.c_size_t, C.c_size_t]),
+    "blt_patch_expand_group_ids": (None, [abi.c_size_p, C.c_size_t, C.c_size_t, abi.c_size_p]),
+    "blt_attention_batch_hip": (None, [C.POINTER(BltAttentionProblem), C.c_size_t]),
+    "blt_attention_plan_create_hip": (C.c_void_p, [C.POINTER(BltAttentionProblem), C.c_size_t]),
+    "blt_attention_plan_run_hip": (None, [C.c_void_p]),
+    "blt_attention_plan_destroy_hip": (None, [C.c_void_p]),
+    "blt_attention_plan_kernel_hip": (C.c_char_p, [C.c_void_p]),
+    "blt_mask_config_row_ranges": (C.c_int, [C.POINTER(abi.BltMaskConfig), C.POINTER(C.c_uint32),
+                                             C.POINTER(C.c_uint32)]),
+    "blt_kv_attend_step_hip": (None, [C.POINTER(BltKvAttnCache), C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t,
+                                      C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t, C.c_int, C.c_int,
+                                      C.c_size_t]),
+    "blt_hip_build_info": (C.c_char_p, []),
+}
+
+_lib = None
+
+
+def load():
+    """The shared library with typed entry points; raises when it was never built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError("%s is missing: run `python -m fblt_amd.build` (there is no fallback path)" % LIB_PATH)
+    lib = C.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SYMBOLS.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def head_args(q_ptr, k_ptr, v_ptr, out_ptr, nq, nk, hd, scale, q_stride, k_stride, v_stride, out_stride, out_col,
+              weights=None, scratch=None, lse=None, mask=None, causal=False):
+    """blt_attention_head_args over raw addresses (ints)."""
+    a = abi.BltAttentionHeadArgs()
+    a.q, a.k, a.v = q_ptr, k_ptr, v_ptr
+    a.q_stride, a.k_stride, a.v_stride = q_stride, k_stride, v_stride
+    a.combined = out_ptr
+    a.combined_stride, a.combined_col_offset = out_stride, out_col
+    a.weights_out = weights
+    a.scores_scratch = scratch
+    a.lse_out = lse
+    a.mask = mask
+    a.nq, a.nk, a.head_dim = nq, nk, hd
+    a.is_causal = bool(causal)
+    a.scale = float(scale)
+    return a
+
+
+def problem(head, kind=BLT_ATTN_MASK_FROM_HEAD, causal_offset=0, window=0, row_lo=None, row_hi=None):
+    p = BltAttentionProblem()
+    p.head = head
+    p.mask_kind = kind
+    p.causal_offset = causal_offset
+    p.window = window
+    p.row_lo = row_lo
+    p.row_hi = row_hi
+    return p
+
+
+def problem_array(problems):
+    arr = (BltAttentionProblem * max(len(problems), 1))()
+    for i, p in enumerate(problems):
+        arr[i] = p
+    return arr

@@ -1,0 +1,297 @@
+/*
+ * Entry points of the attention forward path: the per-head device twin the
+ * reference's dispatcher binds, the whole-batch launch and the resident plan.
+ * Host code only (argument checks, descriptor translation, kernel choice);
+ * the kernels live in attn_rows.hip and attn_mfma.hip.
+ */
+#include "blt_hip.h"
+#include "blt_fatal.h"
+#include "hip_check.h"
+#include "attn_launch.h"
+
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+namespace {
+
+/* Kernel family a problem is routed to. */
+enum Family : uint32_t { FAM_ROWS = 0, FAM_MFMA = 1, FAM_COUNT = 2 };
+
+struct Bucket {
+    Family fam;
+    uint32_t hd;      /* head_dim shared by the bucket */
+    uint32_t base;    /* first descriptor in the sorted array */
+    uint32_t count;
+    uint32_t max_nq;
+    uint32_t tiles;   /* mfma: number of work items; first item index in tile array = tile_base */
+    uint32_t tile_base;
+};
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+/* Translate and check one problem.  `what` prefixes error messages. */
+AttnProb translate(const blt_attention_problem &pr, bool need_score_buffer, const char *what) {
+    const blt_attention_head_args &a = pr.head;
+    BLT_REQUIRE(a.q != NULL && a.k != NULL && a.v != NULL && a.combined != NULL, "%s: buffers must not be NULL",
+                what);
+    if (need_score_buffer)
+        BLT_REQUIRE(a.weights_out != NULL || a.scores_scratch != NULL || a.lse_out != NULL,
+                    "%s: need weights_out, scores_scratch, or lse_out", what);
+    BLT_REQUIRE(a.nq <= 0x7FFFFFFFu && a.nk <= 0x7FFFFFFFu, "%s: nq/nk exceed 2^31-1", what);
+    BLT_REQUIRE(a.head_dim >= 1 && a.head_dim <= ATTN_ROWS_MAX_HEAD_DIM, "%s: head_dim must be in [1, %u]", what,
+                ATTN_ROWS_MAX_HEAD_DIM);
+    BLT_REQUIRE(a.q_stride <= 0xFFFFFFFFu && a.k_stride <= 0xFFFFFFFFu && a.v_stride <= 0xFFFFFFFFu &&
+                    a.combined_stride <= 0xFFFFFFFFu,
+                "%s: row strides exceed 2^32-1 elements", what);
+
+    AttnProb d;
+    std::memset(&d, 0, sizeof(d));
+    d.q = a.q;
+    d.k = a.k;
+    d.v = a.v;
+    d.out = a.combined + a.combined_col_offset;
+    d.weights = a.weights_out;
+    d.lse = a.lse_out;
+    d.q_stride = (uint32_t)a.q_stride;
+    d.k_stride = (uint32_t)a.k_stride;
+    d.v_stride = (uint32_t)a.v_stride;
+    d.out_stride = (uint32_t)a.combined_stride;
+    d.nq = (uint32_t)a.nq;
+    d.nk = (uint32_t)a.nk;
+    d.hd = (uint32_t)a.head_dim;
+    d.scale = a.scale;
+
+    switch (pr.mask_kind) {
+    case BLT_ATTN_MASK_FROM_HEAD:
+        if (a.mask != NULL) {
+            d.vis = ATTN_VIS_DENSE;
+            d.mask = a.mask;
+        } else if (a.is_causal) {
+            d.vis = ATTN_VIS_CAUSAL;
+        } else {
+            d.vis = ATTN_VIS_ALL;
+        }
+        break;
+    case BLT_ATTN_MASK_CAUSAL:
+        BLT_REQUIRE(a.mask == NULL, "%s: a mask descriptor and a dense mask exclude each other", what);
+        BLT_REQUIRE(pr.causal_offset <= 0x7FFFFFFFu && pr.window <= 0xFFFFFFFFu,
+                    "%s: causal_offset/window out of range", what);
+        d.vis = ATTN_VIS_CAUSAL;
+        d.causal_off = (uint32_t)pr.causal_offset;
+        d.window = (uint32_t)pr.window;
+        break;
+    case BLT_ATTN_MASK_ROW_RANGE:
+        BLT_REQUIRE(a.mask == NULL, "%s: a mask descriptor and a dense mask exclude each other", what);
+        BLT_REQUIRE(pr.row_lo != NULL && pr.row_hi != NULL, "%s: row ranges must not be NULL", what);
+        d.vis = ATTN_VIS_RANGE;
+        d.row_lo = pr.row_lo;
+        d.row_hi = pr.row_hi;
+        break;
+    default:
+        BLT_FATAL("%s: unknown mask_kind %u", what, pr.mask_kind);
+    }
+
+    const bool vec = aligned16(d.q) && aligned16(d.k) && aligned16(d.v) && aligned16(d.out) && d.q_stride % 4 == 0 &&
+                     d.k_stride % 4 == 0 && d.v_stride % 4 == 0 && d.out_stride % 4 == 0 && d.hd % 4 == 0;
+    if (vec) d.flags |= ATTN_FLAG_VEC4;
+    return d;
+}
+
+/* BLT_HIP_ATTN_FAMILY=rows|mfma pins the kernel family wherever the shape
+ * allows it (tuning and test hook); unset or anything else = automatic. */
+int family_override() {
+    static const int cached = [] {
+        const char *e = getenv("BLT_HIP_ATTN_FAMILY");
+        if (e && std::strcmp(e, "rows") == 0) return 1;
+        if (e && std::strcmp(e, "mfma") == 0) return 2;
+        return 0;
+    }();
+    return cached;
+}
+
+Family choose_family(const AttnProb &d) {
+    const int forced = family_override();
+    if (forced == 1) return FAM_ROWS;
+    if (forced == 2 && attn_mfma_can(d)) return FAM_MFMA;
+    if (attn_mfma_takes(d)) return FAM_MFMA;
+    return FAM_ROWS;
+}
+
+} // namespace
+
+struct blt_attention_plan {
+    std::vector<AttnProb> host;   /* sorted by bucket */
+    std::vector<Bucket> buckets;
+    std::vector<AttnTile> tiles;  /* mfma work items, all buckets */
+    AttnProb *dev = nullptr;      /* resident plans: descriptors in device memory */
+    AttnTile *dev_tiles = nullptr;
+    const char *kernel = "none";
+};
+
+namespace {
+
+void plan_build(blt_attention_plan &pl, const blt_attention_problem *problems, size_t count, bool need_score_buffer,
+                const char *what) {
+    pl.host.clear();
+    pl.buckets.clear();
+    pl.tiles.clear();
+    pl.host.reserve(count);
+    std::vector<std::pair<uint64_t, AttnProb>> keyed;
+    keyed.reserve(count);
+    for (size_t t = 0; t < count; t++) {
+        AttnProb d = translate(problems[t], need_score_buffer, what);
+        if (d.nq == 0) continue; /* nothing to write */
+        const Family f = choose_family(d);
+        keyed.emplace_back(((uint64_t)f << 32) | d.hd, d);
+    }
+    std::stable_sort(keyed.begin(), keyed.end(),
+                     [](const std::pair<uint64_t, AttnProb> &x, const std::pair<uint64_t, AttnProb> &y) {
+                         return x.first < y.first;
+                     });
+    for (size_t t = 0; t < keyed.size(); t++) {
+        const AttnProb &d = keyed[t].second;
+        const Family f = (Family)(keyed[t].first >> 32);
+        if (pl.buckets.empty() || pl.buckets.back().fam != f || pl.buckets.back().hd != d.hd) {
+            Bucket b;
+            b.fam = f;
+            b.hd = d.hd;
+            b.base = (uint32_t)t;
+            b.count = 0;
+            b.max_nq = 0;
+            b.tiles = 0;
+            b.tile_base = 0;
+            pl.buckets.push_back(b);
+        }
+        Bucket &b = pl.buckets.back();
+        b.count++;
+        b.max_nq = std::max(b.max_nq, d.nq);
+        pl.host.push_back(d);
+    }
+    for (Bucket &b : pl.buckets) {
+        if (b.fam != FAM_MFMA) continue;
+        b.tile_base = (uint32_t)pl.tiles.size();
+        attn_mfma_make_tiles(pl.host.data(), b.base, b.count, pl.tiles);
+        b.tiles = (uint32_t)pl.tiles.size() - b.tile_base;
+    }
+    bool any_mfma = false, any_rows = false;
+    for (const Bucket &b : pl.buckets) (b.fam == FAM_MFMA ? any_mfma : any_rows) = true;
+    pl.kernel = any_mfma && any_rows ? "mfma+rows" : any_mfma ? "mfma" : any_rows ? "rows" : "none";
+}
+
+void plan_launch(const blt_attention_plan &pl, const AttnProb *dev, const AttnTile *dev_tiles) {
+    for (const Bucket &b : pl.buckets) {
+        if (b.fam == FAM_MFMA)
+            attn_mfma_launch(dev, dev_tiles + b.tile_base, b.tiles, b.hd, 0);
+        else
+            attn_rows_launch(dev, b.base, b.count, b.hd, b.max_nq, 0);
+    }
+    HIP_CHECK_LAUNCH("attention forward");
+}
+
+/* Staging for one-shot batches: descriptors go host vector -> pinned buffer ->
+ * device buffer with a truly asynchronous copy on the null stream.  The
+ * device buffer can be reused by the next call because that call's copy is
+ * ordered behind this call's kernels; the pinned buffer is guarded by an
+ * event recorded right after the copy. */
+struct Staging {
+    blt_attention_plan plan;
+    void *pinned = nullptr;
+    void *device = nullptr;
+    size_t capacity = 0;
+    hipEvent_t copied = nullptr;
+    bool in_flight = false;
+
+    void run() {
+        const size_t pbytes = plan.host.size() * sizeof(AttnProb);
+        const size_t tbytes = plan.tiles.size() * sizeof(AttnTile);
+        const size_t need = pbytes + tbytes;
+        if (need == 0) return;
+        if (!copied) HIP_CHECK(hipEventCreateWithFlags(&copied, hipEventDisableTiming));
+        if (in_flight) {
+            HIP_CHECK(hipEventSynchronize(copied));
+            in_flight = false;
+        }
+        if (need > capacity) {
+            if (device) {
+                HIP_CHECK(hipDeviceSynchronize());
+                HIP_CHECK(hipFree(device));
+                HIP_CHECK(hipHostFree(pinned));
+            }
+            capacity = std::max<size_t>(2 * need, 64 * 1024);
+            HIP_CHECK(hipMalloc(&device, capacity));
+            HIP_CHECK(hipHostMalloc(&pinned, capacity, hipHostMallocDefault));
+        }
+        std::memcpy(pinned, plan.host.data(), pbytes);
+        if (tbytes) std::memcpy(static_cast<char *>(pinned) + pbytes, plan.tiles.data(), tbytes);
+        HIP_CHECK(hipMemcpyAsync(device, pinned, need, hipMemcpyHostToDevice, 0));
+        HIP_CHECK(hipEventRecord(copied, 0));
+        in_flight = true;
+        plan_launch(plan, static_cast<const AttnProb *>(device),
+                    reinterpret_cast<const AttnTile *>(static_cast<const char *>(device) + pbytes));
+    }
+};
+
+Staging &staging() {
+    static thread_local Staging st;
+    return st;
+}
+
+} // namespace
+
+extern "C" void blt_attention_head_core_hip(blt_backend backend, const blt_attention_head_args *a) {
+    BLT_REQUIRE(backend == BLT_BACKEND_HIP, "blt_attention_head_core: HIP implementation called with non-HIP backend");
+    BLT_REQUIRE(a != NULL, "blt_attention_head_core: buffers must not be NULL");
+    blt_attention_problem pr;
+    std::memset(&pr, 0, sizeof(pr));
+    pr.head = *a;
+    pr.mask_kind = BLT_ATTN_MASK_FROM_HEAD;
+    /* one problem: the descriptor travels as a kernel argument, nothing is staged */
+    const AttnProb d = translate(pr, true, "blt_attention_head_core");
+    if (d.nq == 0) return;
+    if (choose_family(d) == FAM_MFMA) attn_mfma_launch_single(d, 0);
+    else attn_rows_launch_single(d, 0);
+    HIP_CHECK_LAUNCH("blt_attention_head_core");
+}
+
+extern "C" void blt_attention_batch_hip(const blt_attention_problem *problems, size_t count) {
+    if (count == 0) return;
+    BLT_REQUIRE(problems != NULL, "blt_attention_batch: problems must not be NULL");
+    Staging &st = staging();
+    plan_build(st.plan, problems, count, false, "blt_attention_batch");
+    st.run();
+}
+
+extern "C" blt_attention_plan *blt_attention_plan_create_hip(const blt_attention_problem *problems, size_t count) {
+    BLT_REQUIRE(problems != NULL || count == 0, "blt_attention_plan_create: problems must not be NULL");
+    blt_attention_plan *pl = new blt_attention_plan();
+    plan_build(*pl, problems, count, false, "blt_attention_plan_create");
+    if (!pl->host.empty()) {
+        HIP_CHECK(hipMalloc((void **)&pl->dev, pl->host.size() * sizeof(AttnProb)));
+        HIP_CHECK(hipMemcpy(pl->dev, pl->host.data(), pl->host.size() * sizeof(AttnProb), hipMemcpyHostToDevice));
+    }
+    if (!pl->tiles.empty()) {
+        HIP_CHECK(hipMalloc((void **)&pl->dev_tiles, pl->tiles.size() * sizeof(AttnTile)));
+        HIP_CHECK(hipMemcpy(pl->dev_tiles, pl->tiles.data(), pl->tiles.size() * sizeof(AttnTile),
+                            hipMemcpyHostToDevice));
+    }
+    return pl;
+}
+
+extern "C" void blt_attention_plan_run_hip(const blt_attention_plan *plan) {
+    BLT_REQUIRE(plan != NULL, "blt_attention_plan_run: plan must not be NULL");
+    plan_launch(*plan, plan->dev, plan->dev_tiles);
+}
+
+extern "C" void blt_attention_plan_destroy_hip(blt_attention_plan *plan) {
+    if (!plan) return;
+    HIP_CHECK(hipDeviceSynchronize());
+    if (plan->dev) HIP_CHECK(hipFree(plan->dev));
+    if (plan->dev_tiles) HIP_CHECK(hipFree(plan->dev_tiles));
+    delete plan;
+}
+
+extern "C" const char *blt_attention_plan_kernel_hip(const blt_attention_plan *plan) {
+    return plan ? plan->kernel : "none";
+}

@@ -1,0 +1,207 @@
+/*
+ * "rows" kernel family: one query row per group of G lanes.
+ *
+ * The universal attention kernel of the backend: any nq, nk, head_dim, any
+ * strides, every visibility kind, weights_out and lse_out.  A group of G
+ * lanes owns one query row; lane g of the group owns head-dim elements
+ * 4*(g + G*t) .. +3 for t < T.  The group walks the row's key range with an
+ * online softmax (running max, running sum, running output), so K and V are
+ * each read once and no score matrix is materialised.  It is the fast path
+ * for problems whose rows see only a few keys (byte<->patch cross-attention:
+ * 1..16 keys per row) and the fallback for shapes the tiled MFMA kernel does
+ * not take.  HBM-bound by construction; no LDS.
+ */
+#include "attn_device.h"
+#include "attn_launch.h"
+
+namespace {
+
+template <int G>
+__device__ __forceinline__ float group_sum(float x) {
+#pragma unroll
+    for (int o = 1; o < G; o <<= 1) x += __shfl_xor(x, o, 64);
+    return x;
+}
+
+/* Four head-dim elements starting at d (zero past head_dim). */
+__device__ __forceinline__ float4 load4(const float *row, uint32_t d, uint32_t hd, bool vec4) {
+    if (vec4) {
+        if (d < hd) return *reinterpret_cast<const float4 *>(row + d);
+        return make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    float4 r;
+    r.x = d + 0 < hd ? row[d + 0] : 0.f;
+    r.y = d + 1 < hd ? row[d + 1] : 0.f;
+    r.z = d + 2 < hd ? row[d + 2] : 0.f;
+    r.w = d + 3 < hd ? row[d + 3] : 0.f;
+    return r;
+}
+
+__device__ __forceinline__ void store4(float *row, uint32_t d, uint32_t hd, bool vec4, float4 x) {
+    if (vec4) {
+        if (d < hd) *reinterpret_cast<float4 *>(row + d) = x;
+        return;
+    }
+    if (d + 0 < hd) row[d + 0] = x.x;
+    if (d + 1 < hd) row[d + 1] = x.y;
+    if (d + 2 < hd) row[d + 2] = x.z;
+    if (d + 3 < hd) row[d + 3] = x.w;
+}
+
+__device__ __forceinline__ float dot4(float4 a, float4 b) { return a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w; }
+
+template <int G, int T, bool SINGLE>
+__global__ __launch_bounds__(256) void attn_rows_kernel(const AttnProb *__restrict__ probs, uint32_t prob_base,
+                                                        AttnProb single) {
+    constexpr int ROWS_PER_WAVE = 64 / G;
+    constexpr int ROWS_PER_BLOCK = 4 * ROWS_PER_WAVE;
+
+    const AttnProb p = SINGLE ? single : probs[prob_base + blockIdx.y];
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t g = lane % G;
+    const uint32_t row = blockIdx.x * ROWS_PER_BLOCK + wave * ROWS_PER_WAVE + lane / G;
+    /* whole wave past the end: leave (uniform per wave) */
+    if (blockIdx.x * ROWS_PER_BLOCK + wave * ROWS_PER_WAVE >= p.nq) return;
+
+    const bool live = row < p.nq;
+    const uint32_t i = live ? row : p.nq - 1;
+    const bool vec4 = (p.flags & ATTN_FLAG_VEC4) != 0;
+
+    uint32_t lo, hi;
+    row_key_range(p, i, lo, hi);
+    if (!live) hi = lo;
+
+    float4 q[T], o[T];
+    const float *qrow = p.q + (size_t)i * p.q_stride;
+#pragma unroll
+    for (int t = 0; t < T; t++) {
+        q[t] = load4(qrow, 4u * (g + G * t), p.hd, vec4);
+        o[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+
+    /* the wave walks the union of its rows' ranges; each group ignores keys
+     * outside its own range */
+    uint32_t wlo = lo, whi = hi;
+    if (lo == hi) {
+        wlo = 0xFFFFFFFFu;
+        whi = 0;
+    }
+#pragma unroll
+    for (int off = G; off < 64; off <<= 1) {
+        wlo = min(wlo, (uint32_t)__shfl_xor((int)wlo, off, 64));
+        whi = max(whi, (uint32_t)__shfl_xor((int)whi, off, 64));
+    }
+
+    float m = neg_inf(), l = 0.f;
+    const float *mrow = p.vis == ATTN_VIS_DENSE ? p.mask + (size_t)i * p.nk : nullptr;
+
+    for (uint32_t j = wlo; j < whi; j++) {
+        const bool mine = j >= lo && j < hi;
+        const uint32_t jj = mine ? j : lo; /* lo < nk whenever the row has keys; else unused */
+        const float *krow = p.k + (size_t)(hi > lo ? jj : 0) * p.k_stride;
+        float part = 0.f;
+#pragma unroll
+        for (int t = 0; t < T; t++) part += dot4(q[t], load4(krow, 4u * (g + G * t), p.hd, vec4));
+        float x = group_sum<G>(part) * p.scale;
+        if (mrow) x += mrow[hi > lo ? jj : 0];
+        const bool take = mine && isfinite(x);
+        if (take) {
+            const float mn = fmaxf(m, x);
+            const float a = softmax_exp(m - mn);
+            const float w = softmax_exp(x - mn);
+            l = l * a + w;
+            const float *vrow = p.v + (size_t)jj * p.v_stride;
+#pragma unroll
+            for (int t = 0; t < T; t++) {
+                const float4 v = load4(vrow, 4u * (g + G * t), p.hd, vec4);
+                o[t].x = o[t].x * a + w * v.x;
+                o[t].y = o[t].y * a + w * v.y;
+                o[t].z = o[t].z * a + w * v.z;
+                o[t].w = o[t].w * a + w * v.w;
+            }
+            m = mn;
+        }
+    }
+
+    if (live) {
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        float *orow = p.out + (size_t)i * p.out_stride;
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+            float4 r = make_float4(o[t].x * inv, o[t].y * inv, o[t].z * inv, o[t].w * inv);
+            store4(orow, 4u * (g + G * t), p.hd, vec4, r);
+        }
+        if (p.lse && g == 0) {
+            p.lse[2 * (size_t)i + 0] = m;
+            p.lse[2 * (size_t)i + 1] = l;
+        }
+    }
+
+    if (p.weights) {
+        /* second sweep: every column of the row gets its weight (0 where the
+         * key is not visible), recomputed against the final (m, l) */
+        float *wrow = p.weights + (size_t)i * p.nk;
+        uint32_t wn = live ? p.nk : 0;
+#pragma unroll
+        for (int off = G; off < 64; off <<= 1) wn = max(wn, (uint32_t)__shfl_xor((int)wn, off, 64));
+        for (uint32_t j = 0; j < wn; j++) {
+            const float *krow = p.k + (size_t)j * p.k_stride;
+            float part = 0.f;
+#pragma unroll
+            for (int t = 0; t < T; t++) part += dot4(q[t], load4(krow, 4u * (g + G * t), p.hd, vec4));
+            float x = group_sum<G>(part) * p.scale;
+            if (mrow) x += mrow[j];
+            float w = 0.f;
+            if (j >= lo && j < hi && isfinite(x) && l > 0.f) w = softmax_exp(x - m) / l;
+            if (live && g == 0) wrow[j] = w;
+        }
+    }
+}
+
+template <int G, int T>
+void launch_rows(const AttnProb *dprobs, uint32_t base, uint32_t count, uint32_t max_nq, const AttnProb *single,
+                 hipStream_t s) {
+    constexpr int ROWS_PER_BLOCK = 4 * (64 / G);
+    dim3 grid((max_nq + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK, count, 1);
+    if (single) {
+        hipLaunchKernelGGL((attn_rows_kernel<G, T, true>), grid, dim3(256), 0, s, dprobs, base, *single);
+    } else {
+        AttnProb none;
+        __builtin_memset(&none, 0, sizeof(none));
+        hipLaunchKernelGGL((attn_rows_kernel<G, T, false>), grid, dim3(256), 0, s, dprobs, base, none);
+    }
+}
+
+void dispatch_rows(const AttnProb *dprobs, uint32_t b, uint32_t n, uint32_t hd, uint32_t max_nq,
+                   const AttnProb *single, hipStream_t s) {
+    const uint32_t chunks = (hd + 3) / 4;
+    if (chunks <= 1) launch_rows<1, 1>(dprobs, b, n, max_nq, single, s);
+    else if (chunks <= 2) launch_rows<2, 1>(dprobs, b, n, max_nq, single, s);
+    else if (chunks <= 4) launch_rows<4, 1>(dprobs, b, n, max_nq, single, s);
+    else if (chunks <= 8) launch_rows<8, 1>(dprobs, b, n, max_nq, single, s);
+    else if (chunks <= 16) launch_rows<16, 1>(dprobs, b, n, max_nq, single, s);
+    else if (chunks <= 32) launch_rows<32, 1>(dprobs, b, n, max_nq, single, s);
+    else if (chunks <= 64) launch_rows<64, 1>(dprobs, b, n, max_nq, single, s);
+    else if (chunks <= 128) launch_rows<64, 2>(dprobs, b, n, max_nq, single, s);
+    else if (chunks <= 256) launch_rows<64, 4>(dprobs, b, n, max_nq, single, s);
+    else launch_rows<64, 16>(dprobs, b, n, max_nq, single, s);
+}
+
+} // namespace
+
+/* All problems [base, base+count) share head_dim `hd`. */
+void attn_rows_launch(const AttnProb *dprobs, uint32_t base, uint32_t count, uint32_t hd, uint32_t max_nq,
+                      hipStream_t s) {
+    /* grid.y is limited to 65535 */
+    for (uint32_t done = 0; done < count;) {
+        const uint32_t n = count - done < 65535u ? count - done : 65535u;
+        dispatch_rows(dprobs, base + done, n, hd, max_nq, nullptr, s);
+        done += n;
+    }
+}
+
+void attn_rows_launch_single(const AttnProb &single, hipStream_t s) {
+    if (single.nq == 0) return;
+    dispatch_rows(nullptr, 0, 1, single.hd, single.nq, &single, s);
+}

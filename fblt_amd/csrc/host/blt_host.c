@@ -1,0 +1,339 @@
+/*
+ * Host side of the HIP attention backend, in C99 like the reference's host
+ * code.  Holds the arena/tensor helpers, the run-time dispatchers with the
+ * reference's public names, the byte<->patch index helpers (host integer code
+ * in the reference too) and the mask-recipe -> row-range reduction.  Every
+ * device action goes through the extern "C" entry points of blt_hip.h; no HIP
+ * header is included here.
+ */
+#include "blt_hip.h"
+#include "blt_fatal.h"
+
+#include <stdlib.h>
+#include <string.h>
+
+/* ------------------------------------------------------------------ */
+/* Arena + tensors (reference behaviour: csrc/core/allocator.c:36-160) */
+/* ------------------------------------------------------------------ */
+
+static size_t dtype_bytes(blt_dtype t) {
+    switch (t) {
+    case BLT_DTYPE_FP32:
+    case BLT_DTYPE_INT32:
+        return 4;
+    case BLT_DTYPE_BF16:
+        return 2;
+    case BLT_DTYPE_UINT8:
+    case BLT_DTYPE_FP8_E4M3:
+        return 1;
+    }
+    return 0;
+}
+
+blt_arena *blt_arena_create(size_t capacity_bytes, blt_backend backend) {
+    BLT_REQUIRE(capacity_bytes > 0, "blt_arena_create: capacity must be positive");
+    blt_arena *a = (blt_arena *)calloc(1, sizeof(*a));
+    BLT_REQUIRE(a != NULL, "blt_arena_create: out of host memory");
+    a->capacity = capacity_bytes;
+    a->backend = backend;
+    if (backend == BLT_BACKEND_HIP) {
+        a->buffer = blt_hip_malloc(capacity_bytes);
+    } else {
+        void *p = NULL;
+        if (posix_memalign(&p, 64, capacity_bytes) != 0) p = NULL;
+        a->buffer = p;
+    }
+    if (!a->buffer) BLT_FATAL("failed to allocate arena buffer");
+    return a;
+}
+
+void blt_arena_destroy(blt_arena *a) {
+    if (!a) return;
+    if (a->backend == BLT_BACKEND_HIP) blt_hip_free(a->buffer);
+    else free(a->buffer);
+    free(a);
+}
+
+void blt_arena_reset(blt_arena *a) {
+    if (a) a->offset = 0;
+}
+
+void *blt_arena_alloc(blt_arena *a, size_t bytes, size_t alignment) {
+    if (!a || !a->buffer) BLT_FATAL("invalid arena");
+    if (alignment == 0) alignment = 1;
+    const size_t at = (a->offset + (alignment - 1)) & ~(alignment - 1);
+    if (at + bytes > a->capacity)
+        BLT_FATAL("arena allocation exceeded capacity: need %zu (aligned %zu), offset %zu, capacity %zu", bytes, at,
+                  a->offset, a->capacity);
+    a->offset = at + bytes;
+    return (char *)a->buffer + at;
+}
+
+static blt_tensor tensor_make(blt_arena *arena, const size_t *shape, size_t ndim, blt_dtype dtype, int clear) {
+    BLT_REQUIRE(ndim <= BLT_MAX_NDIM, "blt_tensor_create: ndim exceeds BLT_MAX_NDIM");
+    blt_tensor t;
+    memset(&t, 0, sizeof(t));
+    t.dtype = dtype;
+    t.backend = arena ? arena->backend : BLT_BACKEND_CPU;
+    t.ndim = ndim;
+    t.numel = ndim ? 1 : 0;
+    for (size_t d = 0; d < ndim; d++) {
+        t.shape[d] = shape[d];
+        t.numel *= shape[d];
+    }
+    size_t run = 1;
+    for (size_t d = ndim; d-- > 0;) {
+        t.strides[d] = run;
+        run *= shape[d];
+    }
+    const size_t bytes = t.numel * dtype_bytes(dtype);
+    t.data = blt_arena_alloc(arena, bytes, 64);
+    if (clear && bytes) {
+        if (t.backend == BLT_BACKEND_HIP) blt_hip_memset(t.data, 0, bytes);
+        else memset(t.data, 0, bytes);
+    }
+    return t;
+}
+
+blt_tensor blt_tensor_create(blt_arena *arena, const size_t *shape, size_t ndim, blt_dtype dtype) {
+    return tensor_make(arena, shape, ndim, dtype, 1);
+}
+
+blt_tensor blt_tensor_create_uninit(blt_arena *arena, const size_t *shape, size_t ndim, blt_dtype dtype) {
+    return tensor_make(arena, shape, ndim, dtype, 0);
+}
+
+void blt_tensor_upload(blt_tensor *dst, const void *host_src, size_t bytes) {
+    BLT_REQUIRE(dst != NULL && dst->data != NULL && host_src != NULL, "blt_tensor_upload: NULL argument");
+    if (dst->backend == BLT_BACKEND_HIP) blt_hip_memcpy_h2d(dst->data, host_src, bytes);
+    else memcpy(dst->data, host_src, bytes);
+}
+
+void blt_tensor_download(const blt_tensor *src, void *host_dst, size_t bytes) {
+    BLT_REQUIRE(src != NULL && src->data != NULL && host_dst != NULL, "blt_tensor_download: NULL argument");
+    if (src->backend == BLT_BACKEND_HIP) blt_hip_memcpy_d2h(host_dst, src->data, bytes);
+    else memcpy(host_dst, src->data, bytes);
+}
+
+void blt_backend_pass_sync(blt_backend backend) {
+    if (backend == BLT_BACKEND_HIP) blt_backend_pass_sync_hip();
+}
+
+/* ------------------------------------------------------------------ */
+/* Dispatchers (reference: csrc/core/backend.c:104-138, 455-492).       */
+/* There is no CPU compute path in this library.                        */
+/* ------------------------------------------------------------------ */
+
+#define BLT_DEVICE_ONLY(backend, what)                                                                             \
+    do {                                                                                                           \
+        if ((backend) != BLT_BACKEND_HIP)                                                                          \
+            BLT_FATAL(what ": this library implements the HIP backend only (got backend %d)", (int)(backend));     \
+    } while (0)
+
+void blt_attention_head_core(blt_backend backend, const blt_attention_head_args *args) {
+    BLT_DEVICE_ONLY(backend, "blt_attention_head_core");
+    blt_attention_head_core_hip(backend, args);
+}
+
+void blt_build_attention_mask(const blt_mask_config *config, blt_tensor *out_mask, blt_arena *arena) {
+    BLT_DEVICE_ONLY(arena ? arena->backend : BLT_BACKEND_CPU, "blt_build_attention_mask");
+    blt_build_attention_mask_hip(config, out_mask, arena);
+}
+
+void blt_build_block_diffusion_mask(const blt_block_diffusion_config *config, blt_tensor *out_mask,
+                                    blt_arena *arena) {
+    BLT_DEVICE_ONLY(arena ? arena->backend : BLT_BACKEND_CPU, "blt_build_block_diffusion_mask");
+    blt_build_block_diffusion_mask_hip(config, out_mask, arena);
+}
+
+void blt_strided_copy(blt_backend backend, float *dst, size_t dst_stride, const float *src, size_t src_stride,
+                      size_t rows, size_t cols) {
+    BLT_DEVICE_ONLY(backend, "blt_strided_copy");
+    blt_strided_copy_hip(backend, dst, dst_stride, src, src_stride, rows, cols);
+}
+
+void blt_softmax_masked_row_inplace(blt_backend backend, float *row, size_t row_len, size_t row_idx, bool is_causal,
+                                    const float *mask_row, float scale) {
+    BLT_DEVICE_ONLY(backend, "blt_softmax_masked_row_inplace");
+    blt_softmax_masked_row_inplace_hip(backend, row, row_len, row_idx, is_causal, mask_row, scale);
+}
+
+float blt_vec_dot(blt_backend backend, const float *a, const float *b, size_t n) {
+    BLT_DEVICE_ONLY(backend, "blt_vec_dot");
+    return blt_vec_dot_hip(backend, a, b, n);
+}
+
+/* ------------------------------------------------------------------ */
+/* Byte <-> patch index (reference: csrc/ops/patch_pool_cpu.c:98-142)   */
+/* ------------------------------------------------------------------ */
+
+void blt_patch_build_group_ids(const blt_patch_info *patches, size_t num_patches, size_t seq_len,
+                               size_t *query_group_ids_out, size_t *kv_group_ids_out) {
+    BLT_REQUIRE(patches != NULL || num_patches == 0, "patch_group_ids: NULL patches");
+    BLT_REQUIRE(query_group_ids_out != NULL && kv_group_ids_out != NULL, "patch_group_ids: NULL output array");
+
+    size_t cursor = 0;
+    for (size_t p = 0; p < num_patches; p++) {
+        query_group_ids_out[p] = p;
+        BLT_REQUIRE(patches[p].start_idx == cursor, "patch_group_ids: patches must tile [0, seq_len) contiguously");
+        BLT_REQUIRE(patches[p].length >= 1, "patch_group_ids: empty patch");
+        const size_t end = cursor + patches[p].length;
+        BLT_REQUIRE(end <= seq_len, "patch_group_ids: patches do not cover [0, seq_len) exactly");
+        while (cursor < end) kv_group_ids_out[cursor++] = p;
+    }
+    BLT_REQUIRE(cursor == seq_len, "patch_group_ids: patches do not cover [0, seq_len) exactly");
+}
+
+size_t blt_patch_decoder_latent_at(const blt_patch_info *patches, size_t num_patches, size_t pos) {
+    BLT_REQUIRE(patches != NULL && num_patches >= 1, "patch_decoder_latent: need at least one patch");
+    if (pos < patches[0].start_idx) return 0;
+    /* Patches are ordered by start; the owner is the last one starting at or before pos. */
+    size_t owner = num_patches;
+    for (size_t p = 0; p < num_patches && patches[p].start_idx <= pos; p++) {
+        if (pos - patches[p].start_idx < patches[p].length) {
+            owner = p;
+            break;
+        }
+    }
+    if (owner == num_patches) return num_patches - 1; /* not covered by any patch */
+    const int closes_patch = (pos - patches[owner].start_idx) + 1 == patches[owner].length;
+    const int has_successor = owner + 1 < num_patches;
+    if (closes_patch && has_successor) return owner; /* final byte: its own latent */
+    return owner == 0 ? 0 : owner - 1;               /* otherwise the previous latent */
+}
+
+void blt_patch_expand_group_ids(const size_t *group_ids_in, size_t n, size_t k, size_t *group_ids_out) {
+    BLT_REQUIRE(group_ids_in != NULL || n == 0, "patch_expand_group_ids: NULL group_ids_in");
+    BLT_REQUIRE(group_ids_out != NULL || n * k == 0, "patch_expand_group_ids: NULL group_ids_out");
+    BLT_REQUIRE(k >= 1, "patch_expand_group_ids: k must be >= 1");
+    size_t w = 0;
+    for (size_t i = 0; i < n; i++)
+        for (size_t r = 0; r < k; r++) group_ids_out[w++] = group_ids_in[i];
+}
+
+/* ------------------------------------------------------------------ */
+/* Mask recipe -> per-row key ranges                                    */
+/* ------------------------------------------------------------------ */
+
+/* Document id per position from the boundary list: entry d is the first
+ * position of document d+1 (reference: csrc/ops/mask_builder_cpu.c:11-19). */
+static void doc_ids(const size_t *bounds, size_t num_docs, size_t len, size_t *out) {
+    size_t d = 0;
+    for (size_t p = 0; p < len; p++) {
+        while (d + 1 < num_docs && p >= bounds[d]) d++;
+        out[p] = d;
+    }
+}
+
+/* For an id array, first[j]/last[j] style lookups: returns 1 when equal ids
+ * form contiguous runs (so "same id" is an interval of positions). */
+static int runs_are_contiguous(const size_t *ids, size_t n) {
+    /* A value may not reappear after its run ended.  O(n log n) would need a
+     * sort; ids here are patch/doc indices < n in practice, so try a direct
+     * table first and fall back to a quadratic scan for exotic values. */
+    size_t maxv = 0;
+    for (size_t i = 0; i < n; i++)
+        if (ids[i] > maxv) maxv = ids[i];
+    if (maxv <= 4 * n + 1024) {
+        unsigned char *seen = (unsigned char *)calloc(maxv + 1, 1);
+        if (!seen) return 0;
+        int ok = 1;
+        for (size_t i = 0; i < n && ok; i++) {
+            if (i > 0 && ids[i] == ids[i - 1]) continue;
+            if (seen[ids[i]]) ok = 0;
+            seen[ids[i]] = 1;
+        }
+        free(seen);
+        return ok;
+    }
+    for (size_t i = 1; i < n; i++) {
+        if (ids[i] == ids[i - 1]) continue;
+        for (size_t j = 0; j + 1 < i; j++)
+            if (ids[j] == ids[i]) return 0;
+    }
+    return 1;
+}
+
+/* Interval [lo, hi) of positions of `ids` (length n, contiguous runs) that
+ * carry value `want`; lo == hi when absent.  `hint` speeds up sorted queries. */
+static void run_of(const size_t *ids, size_t n, size_t want, size_t *hint, size_t *lo, size_t *hi) {
+    size_t s = *hint < n ? *hint : 0;
+    size_t scanned = 0;
+    while (scanned < n && ids[s] != want) {
+        s = (s + 1 == n) ? 0 : s + 1;
+        scanned++;
+    }
+    if (scanned == n) {
+        *lo = *hi = 0;
+        return;
+    }
+    size_t b = s;
+    while (b > 0 && ids[b - 1] == want) b--;
+    size_t e = s;
+    while (e < n && ids[e] == want) e++;
+    *lo = b;
+    *hi = e;
+    *hint = b;
+}
+
+static inline size_t zmin(size_t a, size_t b) { return a < b ? a : b; }
+static inline size_t zmax(size_t a, size_t b) { return a > b ? a : b; }
+
+int blt_mask_config_row_ranges(const blt_mask_config *c, uint32_t *lo_out, uint32_t *hi_out) {
+    BLT_REQUIRE(c != NULL && lo_out != NULL && hi_out != NULL, "blt_mask_config_row_ranges: NULL argument");
+    const size_t nq = c->seq_len_q, nk = c->seq_len_kv;
+    BLT_REQUIRE(nq > 0 && nk > 0, "blt_mask_config_row_ranges: seq_len_q/seq_len_kv must be > 0");
+    if (nk > 0xFFFFFFFFu || nq > 0xFFFFFFFFu) return 0;
+
+    const int docs = c->doc_boundaries != NULL && c->num_docs > 0;
+    const int groups = c->query_group_ids != NULL && c->kv_group_ids != NULL;
+    const size_t W = c->sliding_window;
+
+    size_t *dq = NULL, *dk = NULL;
+    int ok = 1;
+    if (docs) {
+        dq = (size_t *)malloc(nq * sizeof(size_t));
+        dk = (size_t *)malloc(nk * sizeof(size_t));
+        BLT_REQUIRE(dq != NULL && dk != NULL, "blt_mask_config_row_ranges: out of host memory");
+        doc_ids(c->doc_boundaries, c->num_docs, nq, dq);
+        doc_ids(c->doc_boundaries, c->num_docs, nk, dk); /* non-decreasing, so runs are contiguous */
+    }
+    if (groups && !runs_are_contiguous(c->kv_group_ids, nk)) ok = 0;
+
+    size_t doc_hint = 0, grp_hint = 0;
+    for (size_t i = 0; i < nq && ok; i++) {
+        size_t lo = 0, hi = nk; /* allowed keys: lo <= j < hi */
+        if (c->is_causal) {
+            /* j <= i + offset */
+            const size_t diag = i + c->causal_offset;
+            hi = zmin(hi, diag + 1);
+            if (W > 0) {
+                /* |diag - j| < W */
+                lo = zmax(lo, diag + 1 >= W ? diag + 1 - W : 0);
+                hi = zmin(hi, diag + W);
+            }
+        } else if (W > 0) {
+            lo = zmax(lo, i + 1 >= W ? i + 1 - W : 0);
+            hi = zmin(hi, i + W);
+        }
+        if (docs) {
+            size_t a, b;
+            run_of(dk, nk, dq[i], &doc_hint, &a, &b);
+            lo = zmax(lo, a);
+            hi = zmin(hi, b);
+        }
+        if (groups) {
+            size_t a, b;
+            run_of(c->kv_group_ids, nk, c->query_group_ids[i], &grp_hint, &a, &b);
+            lo = zmax(lo, a);
+            hi = zmin(hi, b);
+            if (!c->bidirectional_within_group) hi = zmin(hi, i + 1);
+        }
+        if (hi < lo) hi = lo;
+        lo_out[i] = (uint32_t)lo;
+        hi_out[i] = (uint32_t)hi;
+    }
+    free(dq);
+    free(dk);
+    return ok;
+}

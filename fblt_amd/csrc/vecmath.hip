@@ -1,0 +1,135 @@
+/*
+ * Small device utilities of the attention path: strided tile copy (head-slice
+ * gather and KV-cache write-through), the masked row softmax and the dot
+ * product (reference contracts: csrc/ops/vecmath.h:14-37).
+ */
+#include "blt_hip.h"
+#include "blt_fatal.h"
+#include "hip_check.h"
+
+#include <stdint.h>
+
+namespace {
+
+/* One thread per 4 consecutive columns when everything is 16-byte aligned,
+ * else one thread per element.  Threads run along the column axis. */
+template <bool VEC4>
+__global__ __launch_bounds__(256) void strided_copy_kernel(float *__restrict__ dst, uint64_t dst_stride,
+                                                           const float *__restrict__ src, uint64_t src_stride,
+                                                           uint64_t rows, uint64_t cols) {
+    const uint64_t per_row = VEC4 ? cols / 4u : cols;
+    const uint64_t total = rows * per_row;
+    for (uint64_t t = (uint64_t)blockIdx.x * 256u + threadIdx.x; t < total; t += (uint64_t)gridDim.x * 256u) {
+        const uint64_t r = t / per_row, c = t % per_row;
+        if (VEC4) {
+            *reinterpret_cast<float4 *>(dst + r * dst_stride + 4u * c) =
+                *reinterpret_cast<const float4 *>(src + r * src_stride + 4u * c);
+        } else {
+            dst[r * dst_stride + c] = src[r * src_stride + c];
+        }
+    }
+}
+
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x = fmaxf(x, __shfl_xor(x, o, 64));
+    return x;
+}
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, 64);
+    return x;
+}
+
+/* One workgroup of 256 threads owns the row: rewrite (scale, mask / causal
+ * cut), maximum over finite entries, exponentials, sum, true division. */
+__global__ __launch_bounds__(256) void softmax_row_kernel(float *__restrict__ row, uint64_t len, uint64_t row_idx,
+                                                          int is_causal, const float *__restrict__ mask_row,
+                                                          float scale) {
+    __shared__ float red[4];
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+
+    float top = -__builtin_huge_valf();
+    for (uint64_t c = threadIdx.x; c < len; c += 256u) {
+        float x;
+        if (mask_row) x = row[c] * scale + mask_row[c];
+        else if (is_causal && c > row_idx) x = -__builtin_huge_valf();
+        else x = row[c] * scale;
+        row[c] = x;
+        if (isfinite(x)) top = fmaxf(top, x);
+    }
+    top = wave_max(top);
+    if (lane == 0) red[wave] = top;
+    __syncthreads();
+    top = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+
+    float sum = 0.f;
+    for (uint64_t c = threadIdx.x; c < len; c += 256u) {
+        const float x = row[c];
+        const float e = isfinite(x) ? expf(x - top) : 0.f;
+        row[c] = e;
+        sum += e;
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) red[wave] = sum;
+    __syncthreads();
+    sum = (red[0] + red[1]) + (red[2] + red[3]);
+    if (sum > 0.f)
+        for (uint64_t c = threadIdx.x; c < len; c += 256u) row[c] = row[c] / sum;
+}
+
+__global__ __launch_bounds__(256) void dot_kernel(const float *__restrict__ a, const float *__restrict__ b,
+                                                  uint64_t n, float *__restrict__ out) {
+    __shared__ float red[4];
+    float acc = 0.f;
+    for (uint64_t t = threadIdx.x; t < n; t += 256u) acc += a[t] * b[t];
+    acc = wave_sum(acc);
+    if ((threadIdx.x & 63u) == 0) red[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) *out = (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+} // namespace
+
+extern "C" void blt_strided_copy_hip(blt_backend backend, float *dst, size_t dst_stride, const float *src,
+                                     size_t src_stride, size_t rows, size_t cols) {
+    BLT_REQUIRE(backend == BLT_BACKEND_HIP, "blt_strided_copy: HIP implementation called with non-HIP backend");
+    if (rows == 0 || cols == 0) return;
+    BLT_REQUIRE(dst != NULL && src != NULL, "blt_strided_copy: buffers must not be NULL");
+    const bool vec = ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15u) == 0 &&
+                     dst_stride % 4 == 0 && src_stride % 4 == 0 && cols % 4 == 0;
+    const uint64_t work = rows * (vec ? cols / 4 : cols);
+    const unsigned blocks = (unsigned)((work + 255u) / 256u < 4096u ? (work + 255u) / 256u : 4096u);
+    if (vec)
+        hipLaunchKernelGGL(strided_copy_kernel<true>, dim3(blocks), dim3(256), 0, 0, dst, (uint64_t)dst_stride, src,
+                           (uint64_t)src_stride, (uint64_t)rows, (uint64_t)cols);
+    else
+        hipLaunchKernelGGL(strided_copy_kernel<false>, dim3(blocks), dim3(256), 0, 0, dst, (uint64_t)dst_stride, src,
+                           (uint64_t)src_stride, (uint64_t)rows, (uint64_t)cols);
+    HIP_CHECK_LAUNCH("blt_strided_copy");
+}
+
+extern "C" void blt_softmax_masked_row_inplace_hip(blt_backend backend, float *row, size_t row_len, size_t row_idx,
+                                                   bool is_causal, const float *mask_row, float scale) {
+    BLT_REQUIRE(backend == BLT_BACKEND_HIP,
+                "blt_softmax_masked_row_inplace: HIP implementation called with non-HIP backend");
+    if (row_len == 0) return;
+    BLT_REQUIRE(row != NULL, "blt_softmax_masked_row_inplace: row must not be NULL");
+    hipLaunchKernelGGL(softmax_row_kernel, dim3(1), dim3(256), 0, 0, row, (uint64_t)row_len, (uint64_t)row_idx,
+                       is_causal ? 1 : 0, mask_row, scale);
+    HIP_CHECK_LAUNCH("blt_softmax_masked_row_inplace");
+}
+
+extern "C" float blt_vec_dot_hip(blt_backend backend, const float *a, const float *b, size_t n) {
+    BLT_REQUIRE(backend == BLT_BACKEND_HIP, "blt_vec_dot: HIP implementation called with non-HIP backend");
+    if (n == 0) return 0.f;
+    BLT_REQUIRE(a != NULL && b != NULL, "blt_vec_dot: buffers must not be NULL");
+    static thread_local float *slot = nullptr;
+    if (!slot) HIP_CHECK(hipMalloc((void **)&slot, sizeof(float)));
+    hipLaunchKernelGGL(dot_kernel, dim3(1), dim3(256), 0, 0, a, b, (uint64_t)n, slot);
+    HIP_CHECK_LAUNCH("blt_vec_dot");
+    float r = 0.f;
+    HIP_CHECK(hipMemcpy(&r, slot, sizeof(float), hipMemcpyDeviceToHost));
+    return r;
+}

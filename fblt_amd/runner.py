@@ -1,0 +1,202 @@
+"""Runs a workload through libfblt_hip.so with device buffers owned by torch.
+
+torch is plumbing here: it allocates device memory and copies results back.
+All compute goes through the C-ABI on the HIP null stream, so callers must not
+switch torch to another stream around these calls.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import abi, api
+
+
+def _torch():
+    import torch
+    if not torch.cuda.is_available():
+        raise RuntimeError("no GPU visible: the HIP attention backend has no CPU path")
+    return torch
+
+
+def sync():
+    api.load().blt_backend_pass_sync_hip()
+
+
+class DeviceWorkload:
+    """Device-resident copy of a workloads.Workload plus problem builders."""
+
+    def __init__(self, w):
+        torch = _torch()
+        self.w = w
+        self.lib = api.load()
+        self.dev = {n: torch.from_numpy(np.ascontiguousarray(a)).cuda() for n, a in w.buffers.items()}
+        self.rng = {n: torch.from_numpy(a.astype(np.int32)).cuda() for n, a in w.ranges.items()}
+        self._keep = []
+        self.arena = None
+        self._mask_cache = {}
+
+    # ---- helpers -------------------------------------------------------
+    def ptr(self, name, off=0):
+        return self.dev[name].data_ptr() + 4 * off
+
+    def zero_outputs(self):
+        for n in self.w.outputs:
+            self.dev[n].zero_()
+        _torch().cuda.synchronize()
+
+    def output(self, name="out"):
+        _torch().cuda.synchronize()
+        return self.dev[name].cpu().numpy()
+
+    def _arena(self):
+        if self.arena is None:
+            self.arena = self.lib.blt_arena_create(256 << 20, abi.BLT_BACKEND_HIP)
+        return self.arena
+
+    def close(self):
+        if self.arena is not None:
+            self.lib.blt_backend_pass_sync_hip()
+            self.lib.blt_arena_destroy(self.arena)
+            self.arena = None
+
+    def dense_mask_ptr(self, h):
+        """Device address of the dense additive mask of head h, built by the
+        device mask builder in the arena (the reference's flow)."""
+        if h.mask == "none":
+            return None
+        if h.mask == "causal":
+            key = ("causal", h.nq, h.nk, h.causal_offset, h.window)
+        elif h.mask == "range":
+            key = ("range", h.mask_ref, h.nq, h.nk)
+        else:
+            raise ValueError(h.mask)
+        if key in self._mask_cache:
+            return self._mask_cache[key]
+        cfg = abi.BltMaskConfig()
+        cfg.seq_len_q, cfg.seq_len_kv = h.nq, h.nk
+        if h.mask == "causal":
+            cfg.is_causal = True
+            cfg.causal_offset = h.causal_offset
+            cfg.sliding_window = h.window
+        else:
+            lo_name, hi_name, off = h.mask_ref
+            lo = self.w.ranges[lo_name][off:off + h.nq]
+            hi = self.w.ranges[hi_name][off:off + h.nq]
+            kv = np.full(h.nk, h.nq, dtype=np.uint64)
+            for i in range(h.nq):
+                kv[lo[i]:hi[i]] = i
+            qg, kg = abi.size_array(range(h.nq)), abi.size_array(kv)
+            self._keep += [qg, kg]
+            cfg.query_group_ids, cfg.kv_group_ids = qg, kg
+            cfg.bidirectional_within_group = True
+        t = abi.BltTensor()
+        self.lib.blt_build_attention_mask_hip(C.byref(cfg), C.byref(t), self._arena())
+        self._mask_cache[key] = t.data
+        return t.data
+
+    def head_args(self, h, mode, weights_ptr=None, lse_ptr=None, scratch_ptr=None):
+        """mode: 'flag' (is_causal / no mask), 'dense' (device dense mask), 'none' (no mask fields)."""
+        mask = None
+        causal = False
+        if mode == "dense":
+            mask = self.dense_mask_ptr(h)
+        elif mode == "flag":
+            causal = h.mask == "causal"
+        a = api.head_args(self.ptr(h.q[0], h.q[1]), self.ptr(h.k[0], h.k[1]), self.ptr(h.v[0], h.v[1]),
+                          self.ptr(h.out[0], h.out[1]), h.nq, h.nk, h.hd, h.scale, h.q[2], h.k[2], h.v[2], h.out[2],
+                          h.out[3], weights=weights_ptr, scratch=scratch_ptr, lse=lse_ptr, mask=mask, causal=causal)
+        return a
+
+    def problems(self, mask_mode="descriptor", weights_ptrs=None, lse_ptrs=None):
+        """ctypes array of blt_attention_problem for every head.
+        mask_mode: 'descriptor' (causal / row-range descriptors), 'dense', 'flag'."""
+        probs = []
+        for t, h in enumerate(self.w.heads):
+            wp = None if weights_ptrs is None else weights_ptrs[t]
+            lp = None if lse_ptrs is None else lse_ptrs[t]
+            if mask_mode == "descriptor" and h.mask == "causal":
+                a = self.head_args(h, "none", wp, lp)
+                probs.append(api.problem(a, api.BLT_ATTN_MASK_CAUSAL, h.causal_offset, h.window))
+            elif mask_mode == "descriptor" and h.mask == "range":
+                a = self.head_args(h, "none", wp, lp)
+                lo_name, hi_name, off = h.mask_ref
+                probs.append(api.problem(a, api.BLT_ATTN_MASK_ROW_RANGE,
+                                         row_lo=self.rng[lo_name].data_ptr() + 4 * off,
+                                         row_hi=self.rng[hi_name].data_ptr() + 4 * off))
+            else:
+                a = self.head_args(h, "dense" if mask_mode == "dense" else "flag", wp, lp)
+                probs.append(api.problem(a))
+        return api.problem_array(probs)
+
+    # ---- ways to run ---------------------------------------------------
+    def run_per_head(self, mode="dense", with_weights=True):
+        """The reference's caller loop: one blt_attention_head_core_hip call per head."""
+        torch = _torch()
+        max_scores = max(h.nq * h.nk for h in self.w.heads)
+        buf = torch.empty(max_scores, dtype=torch.float32, device="cuda")
+        for h in self.w.heads:
+            a = self.head_args(h, mode, weights_ptr=buf.data_ptr() if with_weights else None,
+                               scratch_ptr=None if with_weights else buf.data_ptr())
+            self.lib.blt_attention_head_core_hip(abi.BLT_BACKEND_HIP, C.byref(a))
+        self.lib.blt_backend_pass_sync_hip()
+
+    def run_batch(self, mask_mode="descriptor"):
+        arr = self.problems(mask_mode)
+        self.lib.blt_attention_batch_hip(arr, len(self.w.heads))
+        self.lib.blt_backend_pass_sync_hip()
+
+    def make_plan(self, mask_mode="descriptor"):
+        arr = self.problems(mask_mode)
+        return self.lib.blt_attention_plan_create_hip(arr, len(self.w.heads))
+
+
+class DeviceKvWorkload:
+    """Device-resident KV-cache workload driving blt_kv_attend_step_hip."""
+
+    def __init__(self, kw):
+        torch = _torch()
+        self.kw = kw
+        self.lib = api.load()
+        self.cache_k = torch.from_numpy(kw.cache_k).cuda()
+        self.cache_v = torch.from_numpy(kw.cache_v).cuda()
+        self.lens0 = torch.from_numpy(kw.lens.astype(np.int32)).cuda()
+        self.lens = self.lens0.clone()
+        self.q_new = torch.from_numpy(kw.q_new).cuda()
+        self.k_new = torch.from_numpy(kw.k_new).cuda()
+        self.v_new = torch.from_numpy(kw.v_new).cuda()
+        self.out = torch.zeros((kw.steps, kw.batch * kw.n, kw.E), dtype=torch.float32, device="cuda")
+        self.host_max_len = int(kw.lens.max())
+        self.c = api.BltKvAttnCache()
+        self.c.self_k = self.cache_k.data_ptr()
+        self.c.self_v = self.cache_v.data_ptr()
+        self.c.self_len = self.lens.data_ptr()
+        self.c.batch, self.c.max_seq_len = kw.batch, kw.max_seq_len
+        self.c.embed_dim, self.c.num_heads, self.c.window = kw.E, kw.H, kw.window
+        self.kind = api.BLT_KV_STEP_CAUSAL if kw.kind == "causal" else api.BLT_KV_STEP_BLOCK
+
+    def reset(self):
+        """Lengths back to the start; cache rows past them are dead by contract."""
+        self.lens.copy_(self.lens0)
+        self.host_max_len = int(self.kw.lens.max())
+        _torch().cuda.synchronize()
+
+    def step(self, s):
+        kw = self.kw
+        E = kw.E
+        hint = self.host_max_len + kw.n
+        self.lib.blt_kv_attend_step_hip(C.byref(self.c), self.q_new[s].data_ptr(), E, self.k_new[s].data_ptr(), E,
+                                        self.v_new[s].data_ptr(), E, self.out[s].data_ptr(), E, kw.n, self.kind,
+                                        1 if kw.commit else 0, hint)
+        if kw.commit:
+            self.host_max_len += kw.n
+
+    def run(self, steps=None):
+        steps = self.kw.steps if steps is None else steps
+        for s in range(steps):
+            self.step(s)
+        self.lib.blt_backend_pass_sync_hip()
+
+    def results(self):
+        _torch().cuda.synchronize()
+        return (self.out.cpu().numpy(), self.cache_k.cpu().numpy(), self.cache_v.cpu().numpy(),
+                self.lens.cpu().numpy())

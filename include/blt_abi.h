@@ -1,0 +1,156 @@
+/*
+ * Boundary types of the fBLT tensor-op C API, restated for the HIP attention
+ * backend.  Each struct is laid out exactly as the reference's own header lays
+ * it out (LP64), so a pointer handed over by the reference's C inference code
+ * can be read here without a copy or a conversion.  The static assertions at
+ * the end of this file are the contract: they hold for the reference compiled
+ * with gcc on x86-64 Linux.
+ *
+ * Reference definitions mirrored here:
+ *   blt_backend, blt_tensor            csrc/core/tensor.h:13-32
+ *   blt_dtype                          csrc/core/dtype.h:11-17
+ *   blt_arena                          csrc/core/allocator.h:11-16
+ *   blt_attention_head_args            csrc/ops/attn_core.h:25-44
+ *   blt_mask_config                    csrc/ops/mask_builder.h:12-32
+ *   blt_block_diffusion_mode/_config   csrc/ops/mask_builder.h:43-68
+ *   blt_patch_info                     csrc/models/patcher.h:16-20
+ */
+#ifndef FBLT_AMD_BLT_ABI_H
+#define FBLT_AMD_BLT_ABI_H
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- backend selector ------------------------------------------------- */
+/* The reference enumerates CPU=0 and one device slot (=1).  This backend
+ * owns the device slot: every pointer tagged BLT_BACKEND_HIP is HIP device
+ * memory of the current device. */
+typedef enum {
+    BLT_BACKEND_CPU = 0,
+    BLT_BACKEND_HIP = 1
+} blt_backend;
+
+typedef enum {
+    BLT_DTYPE_FP32 = 0,
+    BLT_DTYPE_BF16 = 1,
+    BLT_DTYPE_INT32 = 2,
+    BLT_DTYPE_UINT8 = 3,
+    BLT_DTYPE_FP8_E4M3 = 4
+} blt_dtype;
+
+#define BLT_MAX_NDIM 4
+
+/* ---- tensor descriptor (104 bytes) ------------------------------------ */
+typedef struct {
+    void *data;
+    size_t shape[BLT_MAX_NDIM];
+    size_t strides[BLT_MAX_NDIM]; /* in elements, row-major */
+    size_t ndim;
+    size_t numel;
+    blt_dtype dtype;
+    blt_backend backend;
+    bool is_view;
+} blt_tensor;
+
+/* ---- bump arena (32 bytes) -------------------------------------------- */
+/* The caller owns the arena and rewinds it by assigning `offset`. */
+typedef struct {
+    void *buffer;
+    size_t capacity;
+    size_t offset;
+    blt_backend backend;
+} blt_arena;
+
+/* ---- one (sequence, head) attention problem (136 bytes) ---------------- */
+/* Row strides are in float elements.  `combined` receives head_dim columns
+ * starting at combined_col_offset of every query row; all other columns are
+ * left alone.  `mask`, when given, is a dense additive [nq, nk] matrix with
+ * row stride nk and wins over is_causal. */
+typedef struct {
+    const float *q;
+    size_t q_stride;
+    const float *k;
+    size_t k_stride;
+    const float *v;
+    size_t v_stride;
+    float *combined;
+    size_t combined_stride;
+    size_t combined_col_offset;
+    float *weights_out;    /* optional [nq*nk]: post-softmax weights            */
+    float *lse_out;        /* optional [nq*2]:  (row max, sum of exponentials)  */
+    float *scores_scratch; /* optional [nq*nk] workspace; never read or written */
+    const float *mask;     /* optional [nq*nk] additive mask                    */
+    size_t nq;
+    size_t nk;
+    size_t head_dim;
+    bool is_causal;
+    float scale;
+} blt_attention_head_args;
+
+/* ---- dense mask recipe (72 bytes) -------------------------------------- */
+/* All index arrays are HOST pointers, also when the mask itself is built in
+ * device memory. */
+typedef struct {
+    size_t seq_len_q;
+    size_t seq_len_kv;
+    size_t sliding_window;        /* 0 = no window                              */
+    const size_t *doc_boundaries; /* entry d = first position of document d+1   */
+    size_t num_docs;              /* array holds num_docs-1 entries             */
+    const size_t *query_group_ids;
+    const size_t *kv_group_ids;
+    bool bidirectional_within_group;
+    bool is_causal;
+    size_t causal_offset;         /* causal rows may see keys j <= i + offset   */
+} blt_mask_config;
+
+typedef enum {
+    BLT_BDM_TRAIN = 0,
+    BLT_BDM_INFER = 1
+} blt_block_diffusion_mode;
+
+/* ---- BLT-D block mask recipe (48 bytes) -------------------------------- */
+typedef struct {
+    blt_block_diffusion_mode mode;
+    size_t seq_len;   /* S: square mask                                         */
+    size_t num_clean; /* N: rows/cols [0, N) are the clean prefix               */
+    size_t block_size;
+    const size_t *block_starts; /* TRAIN only, HOST pointer, num_blocks entries */
+    size_t num_blocks;
+} blt_block_diffusion_config;
+
+/* ---- patch boundary record (24 bytes) ---------------------------------- */
+typedef struct {
+    size_t start_idx;
+    size_t length;
+    float peak_entropy;
+} blt_patch_info;
+
+#ifdef __cplusplus
+}
+#define BLT_ABI_ASSERT(c, m) static_assert(c, m)
+#else
+#define BLT_ABI_ASSERT(c, m) _Static_assert(c, m)
+#endif
+
+BLT_ABI_ASSERT(sizeof(size_t) == 8 && sizeof(void *) == 8, "LP64 only");
+BLT_ABI_ASSERT(sizeof(blt_tensor) == 104, "blt_tensor layout");
+BLT_ABI_ASSERT(offsetof(blt_tensor, dtype) == 88 && offsetof(blt_tensor, is_view) == 96, "blt_tensor tail");
+BLT_ABI_ASSERT(sizeof(blt_arena) == 32, "blt_arena layout");
+BLT_ABI_ASSERT(sizeof(blt_attention_head_args) == 136, "blt_attention_head_args layout");
+BLT_ABI_ASSERT(offsetof(blt_attention_head_args, mask) == 96, "blt_attention_head_args.mask");
+BLT_ABI_ASSERT(offsetof(blt_attention_head_args, is_causal) == 128 &&
+                   offsetof(blt_attention_head_args, scale) == 132,
+               "blt_attention_head_args tail");
+BLT_ABI_ASSERT(sizeof(blt_mask_config) == 72, "blt_mask_config layout");
+BLT_ABI_ASSERT(offsetof(blt_mask_config, bidirectional_within_group) == 56 &&
+                   offsetof(blt_mask_config, is_causal) == 57 && offsetof(blt_mask_config, causal_offset) == 64,
+               "blt_mask_config tail");
+BLT_ABI_ASSERT(sizeof(blt_block_diffusion_config) == 48, "blt_block_diffusion_config layout");
+BLT_ABI_ASSERT(sizeof(blt_patch_info) == 24, "blt_patch_info layout");
+
+#endif /* FBLT_AMD_BLT_ABI_H */

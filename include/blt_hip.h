@@ -1,0 +1,203 @@
+/*
+ * C-ABI of the MI355X (gfx950) attention backend for fBLT.
+ *
+ * Part 1 are the device twins the reference's dispatcher binds: same
+ * parameter lists as its `_cpu` / `_cuda` functions, `_hip` suffix.  Part 2 is
+ * the device-memory shim the reference's core calls.  Part 3 is the host-side
+ * mirror of the reference's own public API for this path (arena, dispatch,
+ * patch index helpers) so that C callers written against the reference headers
+ * link unchanged.  Part 4 are additive entry points that have no counterpart
+ * in the reference: whole-batch launches and the batched KV-cache step.
+ *
+ * Errors: there are no return codes.  A violated precondition or a HIP error
+ * prints "BLT Fatal Error [file:line]: ..." to stderr and calls
+ * exit(EXIT_FAILURE), as the reference does (csrc/core/backend.h:13-31).
+ *
+ * Streams: everything is issued on the HIP default (null) stream of the
+ * current device, in order, without host synchronisation unless stated.
+ */
+#ifndef FBLT_AMD_BLT_HIP_H
+#define FBLT_AMD_BLT_HIP_H
+
+#include "blt_abi.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ===================================================================== */
+/* Part 1 -- device twins of the reference ops                            */
+/* ===================================================================== */
+
+/* Replaces blt_attention_head_core_cuda (csrc/ops/attn_core.cu:288-311;
+ * contract csrc/ops/attn_core.h:12-46).  All pointers are device pointers.
+ * Needs at least one of weights_out / scores_scratch / lse_out.  Writes
+ * combined[i, col_offset .. col_offset+head_dim); weights_out (post-softmax
+ * weights, zeros where masked) when given; lse_out (row max, row sum) when
+ * given.  scores_scratch is neither read nor written. */
+void blt_attention_head_core_hip(blt_backend backend, const blt_attention_head_args *args);
+
+/* Replaces blt_build_attention_mask_cuda (csrc/ops/mask_builder.cu:100-158).
+ * Creates out_mask [seq_len_q, seq_len_kv] fp32 in the device arena (0 where
+ * allowed, -INFINITY where not); index arrays in `config` are host pointers.
+ * Blocks until the row-validity flags are back; aborts when a query row has
+ * no allowed key. */
+void blt_build_attention_mask_hip(const blt_mask_config *config, blt_tensor *out_mask, blt_arena *arena);
+
+/* Replaces blt_build_block_diffusion_mask_cuda (csrc/ops/mask_builder.cu:187-216). */
+void blt_build_block_diffusion_mask_hip(const blt_block_diffusion_config *config, blt_tensor *out_mask,
+                                        blt_arena *arena);
+
+/* Replaces blt_strided_copy_cuda (csrc/ops/vecmath.cu:144-163): rows x cols
+ * fp32 tile between strided device buffers (head-slice gather, KV write-through). */
+void blt_strided_copy_hip(blt_backend backend, float *dst, size_t dst_stride, const float *src,
+                          size_t src_stride, size_t rows, size_t cols);
+
+/* Replaces blt_softmax_masked_row_inplace_cuda (csrc/ops/vecmath.cu:71-114):
+ * the row softmax of csrc/ops/vecmath.h:20-31 on one device row. */
+void blt_softmax_masked_row_inplace_hip(blt_backend backend, float *row, size_t row_len, size_t row_idx,
+                                        bool is_causal, const float *mask_row, float scale);
+
+/* Replaces blt_vec_dot_cuda (csrc/ops/vecmath.cu:20-69): device dot product,
+ * result returned to the host (blocking). */
+float blt_vec_dot_hip(blt_backend backend, const float *a, const float *b, size_t n);
+
+/* ===================================================================== */
+/* Part 2 -- device memory shim (csrc/core/cuda_shim.h:18-31,             */
+/*           csrc/ops/memory.cu:19-77)                                    */
+/* ===================================================================== */
+void *blt_hip_malloc(size_t bytes);
+void blt_hip_free(void *ptr);
+void blt_hip_memset(void *dst, int value, size_t bytes);                 /* async, default stream */
+void blt_hip_memcpy_h2d(void *dst, const void *src, size_t bytes);       /* async, default stream */
+void blt_hip_memcpy_d2h(void *dst, const void *src, size_t bytes);       /* blocking */
+void blt_backend_pass_sync_hip(void);                                    /* device sync + error check */
+
+/* ===================================================================== */
+/* Part 3 -- host mirror of the reference's public API for this path      */
+/* ===================================================================== */
+
+/* csrc/core/allocator.h:18-23 (allocator.c:36-160).  backend selects host or
+ * device memory for the arena's buffer. */
+blt_arena *blt_arena_create(size_t capacity_bytes, blt_backend backend);
+void blt_arena_destroy(blt_arena *arena);
+void blt_arena_reset(blt_arena *arena);
+void *blt_arena_alloc(blt_arena *arena, size_t bytes, size_t alignment);
+blt_tensor blt_tensor_create(blt_arena *arena, const size_t *shape, size_t ndim, blt_dtype dtype);
+blt_tensor blt_tensor_create_uninit(blt_arena *arena, const size_t *shape, size_t ndim, blt_dtype dtype);
+/* csrc/core/allocator.h:35-41 */
+void blt_tensor_upload(blt_tensor *dst, const void *host_src, size_t bytes);
+void blt_tensor_download(const blt_tensor *src, void *host_dst, size_t bytes);
+/* csrc/core/backend.h:61-63 */
+void blt_backend_pass_sync(blt_backend backend);
+
+/* Run-time dispatch with the reference's signatures (csrc/core/backend.c:
+ * 455-492).  This library holds no CPU compute path: a call tagged
+ * BLT_BACKEND_CPU is a fatal error, never a silent fallback. */
+void blt_attention_head_core(blt_backend backend, const blt_attention_head_args *args);
+void blt_build_attention_mask(const blt_mask_config *config, blt_tensor *out_mask, blt_arena *arena);
+void blt_build_block_diffusion_mask(const blt_block_diffusion_config *config, blt_tensor *out_mask,
+                                    blt_arena *arena);
+void blt_strided_copy(blt_backend backend, float *dst, size_t dst_stride, const float *src, size_t src_stride,
+                      size_t rows, size_t cols);
+void blt_softmax_masked_row_inplace(blt_backend backend, float *row, size_t row_len, size_t row_idx,
+                                    bool is_causal, const float *mask_row, float scale);
+float blt_vec_dot(blt_backend backend, const float *a, const float *b, size_t n);
+
+/* Byte<->patch index helpers; host integer code in the reference as well
+ * (csrc/ops/patch_pool.h:29-41, patch_pool_cpu.c:98-142). */
+void blt_patch_build_group_ids(const blt_patch_info *patches, size_t num_patches, size_t seq_len,
+                               size_t *query_group_ids_out, size_t *kv_group_ids_out);
+size_t blt_patch_decoder_latent_at(const blt_patch_info *patches, size_t num_patches, size_t pos);
+void blt_patch_expand_group_ids(const size_t *group_ids_in, size_t n, size_t k, size_t *group_ids_out);
+
+/* ===================================================================== */
+/* Part 4 -- additive entry points (no counterpart in the reference)      */
+/* ===================================================================== */
+
+/* How a problem says which (query, key) pairs are visible without a dense
+ * [nq, nk] matrix in memory. */
+typedef enum {
+    BLT_ATTN_MASK_FROM_HEAD = 0, /* use head.mask / head.is_causal as the per-head call does */
+    BLT_ATTN_MASK_CAUSAL = 1,    /* j <= i + causal_offset, and i + causal_offset - j < window if window > 0 */
+    BLT_ATTN_MASK_ROW_RANGE = 2  /* row i sees keys row_lo[i] <= j < row_hi[i] (device uint32 arrays) */
+} blt_attn_mask_kind;
+
+/* One (sequence, head) problem of a batch: the reference's argument block
+ * plus an optional mask descriptor.  With a descriptor, head.mask must be
+ * NULL; none of the three score buffers is required. */
+typedef struct {
+    blt_attention_head_args head;
+    uint32_t mask_kind; /* blt_attn_mask_kind */
+    uint32_t reserved;
+    size_t causal_offset;
+    size_t window;
+    const uint32_t *row_lo; /* device, [nq] */
+    const uint32_t *row_hi; /* device, [nq] */
+} blt_attention_problem;
+
+/* All problems of a forward pass in one go: what the reference issues as a
+ * caller loop of count per-head calls (csrc/models/attention.c:199-202,
+ * cross_attention.c:147-150).  `problems` is a HOST array; it is staged to the
+ * device on the default stream before the kernels that read it. */
+void blt_attention_batch_hip(const blt_attention_problem *problems, size_t count);
+
+/* A batch whose descriptors stay resident on the device, for callers that
+ * run the same set of problems repeatedly (same pointers, new contents). */
+typedef struct blt_attention_plan blt_attention_plan;
+blt_attention_plan *blt_attention_plan_create_hip(const blt_attention_problem *problems, size_t count);
+void blt_attention_plan_run_hip(const blt_attention_plan *plan);
+void blt_attention_plan_destroy_hip(blt_attention_plan *plan);
+/* Name of the kernel family the plan selected ("rows", "mfma32", ...), for logs. */
+const char *blt_attention_plan_kernel_hip(const blt_attention_plan *plan);
+
+/* Row ranges equivalent to a blt_mask_config, computed on the host in
+ * O(nq + nk): returns 1 and fills lo/hi (host arrays [seq_len_q]) when every
+ * row's allowed set is one contiguous key range (true for causal, window,
+ * document and sorted-group masks), 0 when it is not (then use the dense
+ * mask).  Rows with no allowed key get lo == hi. */
+int blt_mask_config_row_ranges(const blt_mask_config *config, uint32_t *lo, uint32_t *hi);
+
+/* Batched tier-1 KV cache in the layout blt_kv_cache_create_batched reserves
+ * (csrc/infer/kv_cache.c:27-71): self_k / self_v are [batch*max_seq_len,
+ * embed_dim] fp32 row-major, row b*max_seq_len + pos holds absolute position
+ * pos of sequence b.  self_len is a DEVICE array [batch] of valid rows. */
+typedef struct {
+    float *self_k;
+    float *self_v;
+    uint32_t *self_len;
+    size_t batch;
+    size_t max_seq_len;
+    size_t embed_dim;
+    size_t num_heads;
+    size_t window; /* local_window of the decoder, 0 = none */
+} blt_kv_attn_cache;
+
+enum {
+    BLT_KV_STEP_CAUSAL = 0, /* new row r sees keys j <= self_len + r (kv_cache.c:229-236) */
+    BLT_KV_STEP_BLOCK = 1   /* every new row sees all self_len + n keys (INFER block rows,
+                               mask_builder_cpu.c:133-135) */
+};
+
+/* The attention statements of blt_kv_decode_step (csrc/infer/kv_cache.c:
+ * 343-390) for every sequence of the batch in one launch: write the n new
+ * K/V rows of each sequence through to rows [len_b, len_b+n) FIRST, then
+ * attend over rows [0, len_b+n) for every head, write combined[b*n + r, :]
+ * and, when `commit` is non-zero, advance self_len[b] by n.  q_rows, k_rows,
+ * v_rows and combined are [batch*n, *] with the given row strides (elements);
+ * K rows are already rotated.  max_len_hint >= max_b(self_len[b]) + n sizes
+ * the launch (the host knows it, as the reference's host-side self_len does);
+ * sequences shorter than the hint simply leave blocks idle. */
+void blt_kv_attend_step_hip(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride,
+                            const float *k_rows, size_t k_stride, const float *v_rows, size_t v_stride,
+                            float *combined, size_t combined_stride, size_t n, int step_kind, int commit,
+                            size_t max_len_hint);
+
+/* Library build tag and the architecture its kernels were compiled for. */
+const char *blt_hip_build_info(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* FBLT_AMD_BLT_HIP_H */

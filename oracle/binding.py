@@ -1,0 +1,130 @@
+"""TEST INFRASTRUCTURE -- ctypes loaders for the CPU checker.
+
+Only tests/, the smoke check and the benchmark's cpu_baseline leg import this.
+`load_oracle()` loads oracle/liboracle.so (our restatement, built by
+`make -C oracle`); `load_ref()` loads oracle/_ref/libblt_ref.so (the reference's
+own core + CPU ops compiled from its sources, built by `make -C oracle ref`
+where those sources exist) or returns None.
+"""
+import ctypes as C
+import os
+import subprocess
+
+from fblt_amd import abi
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ORACLE_SO = os.path.join(HERE, "liboracle.so")
+REF_SO = os.path.join(HERE, "_ref", "libblt_ref.so")
+
+_fp = C.POINTER(C.c_float)
+_sp = C.POINTER(C.c_size_t)
+
+
+def build(ref=True):
+    """Compile the checker (and the reference build when its sources exist)."""
+    subprocess.check_call(["make", "-s", "-B", "-C", HERE, "all"])
+    if ref and os.path.isdir(os.environ.get("REF_ROOT", "/root/reference")):
+        subprocess.check_call(["make", "-s", "-B", "-C", HERE, "ref"])
+
+
+def load_oracle():
+    if not os.path.exists(ORACLE_SO):
+        build(ref=False)
+    lib = C.CDLL(ORACLE_SO)
+    A = abi.BltAttentionHeadArgs
+    lib.orc_vec_dot.restype = C.c_float
+    lib.orc_vec_dot.argtypes = [_fp, _fp, C.c_size_t]
+    lib.orc_softmax_masked_row_inplace.restype = None
+    lib.orc_softmax_masked_row_inplace.argtypes = [_fp, C.c_size_t, C.c_size_t, C.c_bool, _fp, C.c_float]
+    lib.orc_strided_copy.restype = None
+    lib.orc_strided_copy.argtypes = [_fp, C.c_size_t, _fp, C.c_size_t, C.c_size_t, C.c_size_t]
+    lib.orc_attention_head_core.restype = C.c_int
+    lib.orc_attention_head_core.argtypes = [C.POINTER(A)]
+    lib.orc_attention_head_core_many.restype = C.c_int
+    lib.orc_attention_head_core_many.argtypes = [C.POINTER(A), C.c_size_t]
+    lib.orc_build_attention_mask.restype = C.c_int
+    lib.orc_build_attention_mask.argtypes = [C.POINTER(abi.BltMaskConfig), _fp]
+    lib.orc_build_block_diffusion_mask.restype = C.c_int
+    lib.orc_build_block_diffusion_mask.argtypes = [C.POINTER(abi.BltBlockDiffusionConfig), _fp]
+    lib.orc_patch_build_group_ids.restype = C.c_int
+    lib.orc_patch_build_group_ids.argtypes = [C.POINTER(abi.BltPatchInfo), C.c_size_t, C.c_size_t, _sp, _sp]
+    lib.orc_patch_decoder_latent_at.restype = C.c_size_t
+    lib.orc_patch_decoder_latent_at.argtypes = [C.POINTER(abi.BltPatchInfo), C.c_size_t, C.c_size_t]
+    lib.orc_patch_expand_group_ids.restype = None
+    lib.orc_patch_expand_group_ids.argtypes = [_sp, C.c_size_t, C.c_size_t, _sp]
+    lib.orc_kv_row.restype = C.c_size_t
+    lib.orc_kv_row.argtypes = [C.c_size_t] * 3
+    lib.orc_kv_slot.restype = C.c_size_t
+    lib.orc_kv_slot.argtypes = [C.c_size_t] * 7
+    lib.orc_kv_self_mask.restype = None
+    lib.orc_kv_self_mask.argtypes = [_fp, C.c_size_t, C.c_size_t, C.c_size_t]
+    lib.orc_kv_step_group_ids.restype = None
+    lib.orc_kv_step_group_ids.argtypes = [C.POINTER(abi.BltPatchInfo), C.c_size_t, C.c_size_t, C.c_size_t,
+                                          C.c_size_t, C.c_int, _sp, _sp]
+    lib.orc_kv_cross_mask.restype = None
+    lib.orc_kv_cross_mask.argtypes = [_fp, _sp, C.c_size_t, _sp, C.c_size_t]
+    lib.orc_kv_attend_step.restype = C.c_int
+    lib.orc_kv_attend_step.argtypes = [_fp, _fp, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t,
+                                       C.c_size_t, C.c_size_t, _fp, _fp, _fp, _fp]
+    return lib
+
+
+def load_ref():
+    """The reference's own CPU ops, or None where they were never built."""
+    if not os.path.exists(REF_SO):
+        return None
+    lib = C.CDLL(REF_SO)
+    A = abi.BltAttentionHeadArgs
+    lib.blt_attention_head_core.restype = None
+    lib.blt_attention_head_core.argtypes = [C.c_int, C.POINTER(A)]
+    lib.blt_softmax_masked_row_inplace.restype = None
+    lib.blt_softmax_masked_row_inplace.argtypes = [C.c_int, _fp, C.c_size_t, C.c_size_t, C.c_bool, _fp, C.c_float]
+    lib.blt_vec_dot.restype = C.c_float
+    lib.blt_vec_dot.argtypes = [C.c_int, _fp, _fp, C.c_size_t]
+    lib.blt_strided_copy.restype = None
+    lib.blt_strided_copy.argtypes = [C.c_int, _fp, C.c_size_t, _fp, C.c_size_t, C.c_size_t, C.c_size_t]
+    lib.blt_arena_create.restype = C.POINTER(abi.BltArena)
+    lib.blt_arena_create.argtypes = [C.c_size_t, C.c_int]
+    lib.blt_arena_destroy.restype = None
+    lib.blt_arena_destroy.argtypes = [C.POINTER(abi.BltArena)]
+    lib.blt_build_attention_mask.restype = None
+    lib.blt_build_attention_mask.argtypes = [C.POINTER(abi.BltMaskConfig), C.POINTER(abi.BltTensor),
+                                             C.POINTER(abi.BltArena)]
+    lib.blt_build_block_diffusion_mask.restype = None
+    lib.blt_build_block_diffusion_mask.argtypes = [C.POINTER(abi.BltBlockDiffusionConfig),
+                                                   C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)]
+    lib.blt_patch_build_group_ids.restype = None
+    lib.blt_patch_build_group_ids.argtypes = [C.POINTER(abi.BltPatchInfo), C.c_size_t, C.c_size_t, _sp, _sp]
+    lib.blt_patch_decoder_latent_at.restype = C.c_size_t
+    lib.blt_patch_decoder_latent_at.argtypes = [C.POINTER(abi.BltPatchInfo), C.c_size_t, C.c_size_t]
+    lib.blt_patch_expand_group_ids.restype = None
+    lib.blt_patch_expand_group_ids.argtypes = [_sp, C.c_size_t, C.c_size_t, _sp]
+    return lib
+
+
+def fptr(a):
+    """float* into a C-contiguous float32 numpy array (or NULL for None)."""
+    if a is None:
+        return None
+    assert a.dtype.name == "float32" and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(_fp)
+
+
+def head_args(q, k, v, combined, nq, nk, hd, scale, q_stride, k_stride, v_stride, c_stride, c_off,
+              q_off=0, k_off=0, v_off=0, weights=None, scratch=None, lse=None, mask=None, causal=False):
+    """blt_attention_head_args over HOST numpy buffers (element offsets)."""
+    a = abi.BltAttentionHeadArgs()
+    a.q = q.ctypes.data + 4 * q_off
+    a.k = k.ctypes.data + 4 * k_off
+    a.v = v.ctypes.data + 4 * v_off
+    a.q_stride, a.k_stride, a.v_stride = q_stride, k_stride, v_stride
+    a.combined = combined.ctypes.data
+    a.combined_stride, a.combined_col_offset = c_stride, c_off
+    a.weights_out = weights.ctypes.data if weights is not None else None
+    a.scores_scratch = scratch.ctypes.data if scratch is not None else None
+    a.lse_out = lse.ctypes.data if lse is not None else None
+    a.mask = mask.ctypes.data if mask is not None else None
+    a.nq, a.nk, a.head_dim = nq, nk, hd
+    a.is_causal = bool(causal)
+    a.scale = float(scale)
+    return a

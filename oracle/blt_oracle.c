@@ -1,0 +1,322 @@
+/*
+ * TEST INFRASTRUCTURE -- NOT PART OF THE PRODUCT.  See blt_oracle.h.
+ *
+ * Scalar, single-threaded restatement of the reference's CPU attention path.
+ * Floating-point statements keep the reference's operand order and rounding
+ * points (one multiply, then one add, per term; libm expf; true division) so
+ * that results agree bit for bit with the reference compiled by the same gcc.
+ */
+#include "blt_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ---------------------------------------------------------------------- */
+/* csrc/ops/vecmath_cpu.c:6-14: float accumulator, ascending index.        */
+float orc_vec_dot(const float *a, const float *b, size_t n) {
+    float acc = 0.0f;
+    size_t t = 0;
+    while (t < n) {
+        acc += a[t] * b[t];
+        t++;
+    }
+    return acc;
+}
+
+/* csrc/ops/vecmath_cpu.c:16-53.
+ * Pass 1 rewrites each entry (scale, then mask or causal cut) and tracks the
+ * largest FINITE entry; pass 2 exponentiates finite entries against that
+ * maximum and zeroes the rest; pass 3 divides when the sum is positive. */
+void orc_softmax_masked_row_inplace(float *row, size_t row_len, size_t row_idx, bool is_causal,
+                                    const float *mask_row, float scale) {
+    float top = -INFINITY;
+    for (size_t c = 0; c < row_len; c++) {
+        float x;
+        if (mask_row) {
+            x = row[c] * scale + mask_row[c];
+        } else if (is_causal && c > row_idx) {
+            x = -INFINITY;
+        } else {
+            x = row[c] * scale;
+        }
+        row[c] = x;
+        if (isfinite(x) && x > top) top = x;
+    }
+
+    float total = 0.0f;
+    for (size_t c = 0; c < row_len; c++) {
+        if (!isfinite(row[c])) {
+            row[c] = 0.0f;
+            continue;
+        }
+        row[c] = expf(row[c] - top);
+        total += row[c];
+    }
+
+    if (total > 0.0f) {
+        for (size_t c = 0; c < row_len; c++) row[c] /= total;
+    }
+}
+
+/* csrc/ops/vecmath_cpu.c:55-63 */
+void orc_strided_copy(float *dst, size_t dst_stride, const float *src, size_t src_stride, size_t rows,
+                      size_t cols) {
+    for (size_t r = 0; r < rows; r++) memcpy(dst + r * dst_stride, src + r * src_stride, cols * sizeof(float));
+}
+
+/* csrc/ops/attn_core_cpu.c:16-57.
+ * All nq*nk dot products are formed (masked pairs too), each row goes through
+ * the masked softmax, then the output row is cleared and accumulated in
+ * ascending key order, skipping keys whose weight is exactly zero. */
+int orc_attention_head_core(const blt_attention_head_args *a) {
+    if (!a || !a->q || !a->k || !a->v || !a->combined) return ORC_ERR_NULL_BUFFER;
+    if (!a->weights_out && !a->scores_scratch) return ORC_ERR_NO_SCORE_BUFFER;
+
+    float *w = a->weights_out ? a->weights_out : a->scores_scratch;
+    const size_t nq = a->nq, nk = a->nk, hd = a->head_dim;
+
+    for (size_t i = 0; i < nq; i++) {
+        float *wi = w + i * nk;
+        const float *qi = a->q + i * a->q_stride;
+        for (size_t j = 0; j < nk; j++) wi[j] = orc_vec_dot(qi, a->k + j * a->k_stride, hd);
+        orc_softmax_masked_row_inplace(wi, nk, i, a->is_causal, a->mask ? a->mask + i * nk : NULL, a->scale);
+    }
+
+    for (size_t i = 0; i < nq; i++) {
+        const float *wi = w + i * nk;
+        float *o = a->combined + i * a->combined_stride + a->combined_col_offset;
+        for (size_t d = 0; d < hd; d++) o[d] = 0.0f;
+        for (size_t j = 0; j < nk; j++) {
+            const float p = wi[j];
+            if (p == 0.0f) continue;
+            const float *vj = a->v + j * a->v_stride;
+            for (size_t d = 0; d < hd; d++) o[d] += p * vj[d];
+        }
+    }
+    return ORC_OK;
+}
+
+/* csrc/models/attention.c:199-202: heads (and sequences) are a caller loop. */
+int orc_attention_head_core_many(const blt_attention_head_args *a, size_t count) {
+    for (size_t t = 0; t < count; t++) {
+        const int rc = orc_attention_head_core(a + t);
+        if (rc != ORC_OK) return rc;
+    }
+    return ORC_OK;
+}
+
+/* ---------------------------------------------------------------------- */
+/* csrc/ops/mask_builder_cpu.c:11-19: boundary d opens document d+1.       */
+static void doc_ids_from_boundaries(const size_t *bounds, size_t num_docs, size_t len, size_t *ids) {
+    size_t cur = 0;
+    for (size_t p = 0; p < len; p++) {
+        while (cur + 1 < num_docs && p >= bounds[cur]) cur++;
+        ids[p] = cur;
+    }
+}
+
+/* csrc/ops/mask_builder_cpu.c:21-95 */
+int orc_build_attention_mask(const blt_mask_config *c, float *out) {
+    if (!c || !out) return ORC_ERR_NULL_BUFFER;
+    const size_t nq = c->seq_len_q, nk = c->seq_len_kv;
+    if (nq == 0 || nk == 0) return ORC_ERR_EMPTY_SHAPE;
+
+    const bool docs = c->doc_boundaries != NULL && c->num_docs > 0;
+    const bool groups = c->query_group_ids != NULL && c->kv_group_ids != NULL;
+    const size_t W = c->sliding_window;
+
+    size_t *dq = NULL, *dk = NULL;
+    if (docs) {
+        dq = (size_t *)malloc(nq * sizeof(size_t));
+        dk = (size_t *)malloc(nk * sizeof(size_t));
+        doc_ids_from_boundaries(c->doc_boundaries, c->num_docs, nq, dq);
+        doc_ids_from_boundaries(c->doc_boundaries, c->num_docs, nk, dk);
+    }
+
+    int rc = ORC_OK;
+    for (size_t i = 0; i < nq && rc == ORC_OK; i++) {
+        bool any = false;
+        for (size_t j = 0; j < nk; j++) {
+            bool ok = true;
+            if (c->is_causal && j > i + c->causal_offset) ok = false;
+            if (W > 0) {
+                size_t dist;
+                if (c->is_causal) {
+                    const size_t diag = i + c->causal_offset;
+                    dist = diag >= j ? diag - j : j - diag;
+                } else {
+                    dist = i >= j ? i - j : j - i;
+                }
+                if (dist >= W) ok = false;
+            }
+            if (docs && dq[i] != dk[j]) ok = false;
+            if (groups) {
+                if (c->query_group_ids[i] != c->kv_group_ids[j]) ok = false;
+                else if (!c->bidirectional_within_group && j > i) ok = false;
+            }
+            out[i * nk + j] = ok ? 0.0f : -INFINITY;
+            any = any || ok;
+        }
+        /* The reference aborts after filling the first row that has no key. */
+        if (!any) rc = ORC_ERR_ROW_WITHOUT_KEY;
+    }
+    free(dq);
+    free(dk);
+    return rc;
+}
+
+/* csrc/ops/mask_builder_cpu.c:97-154 */
+int orc_build_block_diffusion_mask(const blt_block_diffusion_config *c, float *out) {
+    if (!c || !out) return ORC_ERR_NULL_BUFFER;
+    const size_t S = c->seq_len, N = c->num_clean, B = c->block_size;
+    if (!(S >= 1 && N >= 1 && N <= S)) return ORC_ERR_BAD_BLOCK_CONFIG;
+    const bool train = c->mode == BLT_BDM_TRAIN;
+    if (train) {
+        if (B < 1 || (S - N) % B != 0 || !c->block_starts || c->num_blocks != (S - N) / B)
+            return ORC_ERR_BAD_BLOCK_CONFIG;
+        for (size_t b = 0; b < c->num_blocks; b++)
+            if (c->block_starts[b] >= N) return ORC_ERR_BAD_BLOCK_CONFIG;
+    }
+
+    for (size_t i = 0; i < S; i++) {
+        bool any = false;
+        for (size_t j = 0; j < S; j++) {
+            bool ok;
+            if (i < N) {
+                ok = j < N && j <= i; /* clean rows: causal over the prefix */
+            } else if (!train) {
+                ok = true; /* INFER: the one live block sees everything */
+            } else {
+                const size_t blk = (i - N) / B;
+                const bool own = j >= N && (j - N) / B == blk;
+                ok = j < c->block_starts[blk] || own;
+            }
+            out[i * S + j] = ok ? 0.0f : -INFINITY;
+            any = any || ok;
+        }
+        if (!any) return ORC_ERR_ROW_WITHOUT_KEY;
+    }
+    return ORC_OK;
+}
+
+/* ---------------------------------------------------------------------- */
+/* csrc/ops/patch_pool_cpu.c:98-112 */
+int orc_patch_build_group_ids(const blt_patch_info *patches, size_t num_patches, size_t seq_len,
+                              size_t *q_ids, size_t *kv_ids) {
+    if ((!patches && num_patches) || !q_ids || !kv_ids) return ORC_ERR_NULL_BUFFER;
+    for (size_t p = 0; p < num_patches; p++) q_ids[p] = p;
+    size_t at = 0;
+    for (size_t p = 0; p < num_patches; p++) {
+        if (patches[p].start_idx != at || patches[p].length < 1) return ORC_ERR_PATCH_TILING;
+        for (size_t t = 0; t < patches[p].length; t++) kv_ids[at++] = p;
+    }
+    return at == seq_len ? ORC_OK : ORC_ERR_PATCH_TILING;
+}
+
+/* csrc/ops/patch_pool_cpu.c:114-131: a byte is "final" when it closes a patch
+ * that has a successor; final bytes read their own patch's latent, all others
+ * the previous one (patch 0 reads itself); uncovered positions read the last. */
+size_t orc_patch_decoder_latent_at(const blt_patch_info *patches, size_t num_patches, size_t pos) {
+    if (pos < patches[0].start_idx) return 0;
+    for (size_t p = 0; p < num_patches; p++) {
+        const size_t lo = patches[p].start_idx;
+        if (lo > pos) break;
+        const size_t hi = lo + patches[p].length;
+        if (pos < hi) {
+            if (pos + 1 == hi && p + 1 < num_patches) return p;
+            return p ? p - 1 : 0;
+        }
+    }
+    return num_patches - 1;
+}
+
+/* csrc/ops/patch_pool_cpu.c:133-142 */
+void orc_patch_expand_group_ids(const size_t *in, size_t n, size_t k, size_t *out) {
+    for (size_t i = 0; i < n; i++)
+        for (size_t r = 0; r < k; r++) out[i * k + r] = in[i];
+}
+
+/* ---------------------------------------------------------------------- */
+size_t orc_kv_row(size_t b, size_t pos, size_t max_seq_len) { return b * max_seq_len + pos; }
+
+size_t orc_kv_slot(size_t b, size_t pos, size_t head, size_t d, size_t max_seq_len, size_t embed_dim,
+                   size_t head_dim) {
+    return orc_kv_row(b, pos, max_seq_len) * embed_dim + head * head_dim + d;
+}
+
+/* csrc/infer/kv_cache.c:224-238 */
+void orc_kv_self_mask(float *out, size_t n, size_t base, size_t window) {
+    const size_t total = base + n;
+    for (size_t r = 0; r < n; r++) {
+        const size_t p = base + r;
+        for (size_t j = 0; j < total; j++) {
+            bool ok = j <= p;
+            if (ok && window > 0 && p - j >= window) ok = false;
+            out[r * total + j] = ok ? 0.0f : -INFINITY;
+        }
+    }
+}
+
+/* csrc/infer/kv_cache.c:203-218 */
+void orc_kv_step_group_ids(const blt_patch_info *patches, size_t num_patches, size_t k_split, size_t base,
+                           size_t n, int trailing_closed, size_t *q_ids, size_t *kv_ids) {
+    for (size_t r = 0; r < n; r++) q_ids[r] = orc_patch_decoder_latent_at(patches, num_patches, base + r);
+    if (trailing_closed && num_patches >= 1) q_ids[n - 1] = num_patches - 1;
+    for (size_t p = 0; p < num_patches; p++)
+        for (size_t s = 0; s < k_split; s++) kv_ids[p * k_split + s] = p;
+}
+
+/* csrc/infer/kv_cache.c:240-251 */
+void orc_kv_cross_mask(float *out, const size_t *q_ids, size_t n, const size_t *kv_ids, size_t total_sub) {
+    for (size_t r = 0; r < n; r++)
+        for (size_t j = 0; j < total_sub; j++) out[r * total_sub + j] = kv_ids[j] == q_ids[r] ? 0.0f : -INFINITY;
+}
+
+/* csrc/infer/kv_cache.c:343-390 (attention statements only) */
+int orc_kv_attend_step(float *self_k, float *self_v, size_t max_seq_len, size_t E, size_t H, size_t b,
+                       size_t base, size_t n, size_t window, const float *q_rows, const float *k_rows,
+                       const float *v_rows, float *combined) {
+    const size_t total = base + n;
+    if (total > max_seq_len) return ORC_ERR_CAPACITY;
+    const size_t hd = E / H;
+    float *kd = self_k + orc_kv_row(b, 0, max_seq_len) * E;
+    float *vd = self_v + orc_kv_row(b, 0, max_seq_len) * E;
+
+    /* write-through, one head slice at a time (kv_cache.c:363-365) */
+    for (size_t h = 0; h < H; h++) {
+        orc_strided_copy(kd + base * E + h * hd, E, k_rows + h * hd, E, n, hd);
+        orc_strided_copy(vd + base * E + h * hd, E, v_rows + h * hd, E, n, hd);
+    }
+
+    float *mask = (float *)malloc(n * total * sizeof(float));
+    float *scratch = (float *)malloc(n * total * sizeof(float));
+    orc_kv_self_mask(mask, n, base, window);
+    memset(combined, 0, n * E * sizeof(float));
+
+    int rc = ORC_OK;
+    for (size_t h = 0; h < H && rc == ORC_OK; h++) {
+        blt_attention_head_args a;
+        memset(&a, 0, sizeof(a));
+        a.q = q_rows + h * hd;
+        a.q_stride = E;
+        a.k = kd + h * hd;
+        a.k_stride = E;
+        a.v = vd + h * hd;
+        a.v_stride = E;
+        a.combined = combined;
+        a.combined_stride = E;
+        a.combined_col_offset = h * hd;
+        a.scores_scratch = scratch;
+        a.mask = mask;
+        a.nq = n;
+        a.nk = total;
+        a.head_dim = hd;
+        a.is_causal = false;
+        a.scale = 1.0f / sqrtf((float)hd);
+        rc = orc_attention_head_core(&a);
+    }
+    free(mask);
+    free(scratch);
+    return rc;
+}

@@ -1,0 +1,133 @@
+/*
+ * TEST INFRASTRUCTURE -- NOT PART OF THE PRODUCT.
+ *
+ * Single-threaded CPU restatement of the reference's attention path, used as
+ * the checker for the HIP backend and as the timed CPU baseline.  Nothing in
+ * the shipped library links, loads or calls this file.
+ *
+ * Every function names the reference lines it restates.  Build flags follow
+ * the reference (CMakeLists.txt:10-12,43,120): -std=c99 -O2, no -march, no
+ * fast-math, plus -ffp-contract=off so no fused multiply-add can appear.
+ *
+ * How each function is pinned (none is "parity unpinned"):
+ *   orc_vec_dot, orc_softmax_masked_row_inplace, orc_attention_head_core
+ *       bit-for-bit against the reference compiled from its own sources
+ *       (oracle/_ref), the reference's inline vectors
+ *       (tests/unit/models/unit_attention.c:82-88,167-171,
+ *       unit_cross_attention.c:111-117), closed forms (two-key sigmoid,
+ *       uniform weights, single visible key, all-masked row) and a float64
+ *       brute force on tiny shapes.
+ *   orc_build_attention_mask, orc_build_block_diffusion_mask
+ *       bit-for-bit against oracle/_ref over the reference's variant matrix
+ *       (tests/parity/parity_cuda_composites.c:66-150), the hard-coded 14x14
+ *       TRAIN matrix and INFER rule (tests/unit/models/unit_block_diffusion.c:
+ *       123-172), the causal/window/doc/group cases of
+ *       tests/unit/backend/unit_mask.c:14-192.
+ *   orc_patch_build_group_ids, orc_patch_decoder_latent_at,
+ *   orc_patch_expand_group_ids
+ *       the expected arrays of tests/unit/models/unit_local_decoder.c:94-113
+ *       and tests/unit/backend/unit_mask.c:116-127, plus oracle/_ref.
+ *   orc_strided_copy, orc_kv_* (slab indexing, step masks, write-through,
+ *   attend)
+ *       against oracle/_ref op calls issued in the order of
+ *       csrc/infer/kv_cache.c:343-390, and against the dense causal attention
+ *       over the same rows (the reference's cached == dense invariant,
+ *       tests/unit/infer/unit_kv_cache.c:136-151).
+ */
+#ifndef FBLT_AMD_ORACLE_H
+#define FBLT_AMD_ORACLE_H
+
+#include "blt_abi.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Return codes: 0 = done; a positive value = the reference would have aborted
+ * (BLT_REQUIRE) at this point; the value says which requirement. */
+enum {
+    ORC_OK = 0,
+    ORC_ERR_NULL_BUFFER = 1,     /* attn_core_cpu.c:18-19 */
+    ORC_ERR_NO_SCORE_BUFFER = 2, /* attn_core_cpu.c:20-21 */
+    ORC_ERR_EMPTY_SHAPE = 3,     /* mask_builder_cpu.c:30 */
+    ORC_ERR_ROW_WITHOUT_KEY = 4, /* mask_builder_cpu.c:93, 152 */
+    ORC_ERR_BAD_BLOCK_CONFIG = 5,/* mask_builder_cpu.c:105-119 */
+    ORC_ERR_PATCH_TILING = 6,    /* patch_pool_cpu.c:107-111 */
+    ORC_ERR_CAPACITY = 7         /* kv_cache.c:191 */
+};
+
+/* csrc/ops/vecmath_cpu.c:6-14 */
+float orc_vec_dot(const float *a, const float *b, size_t n);
+
+/* csrc/ops/vecmath_cpu.c:16-53 */
+void orc_softmax_masked_row_inplace(float *row, size_t row_len, size_t row_idx, bool is_causal,
+                                    const float *mask_row, float scale);
+
+/* csrc/ops/vecmath_cpu.c:55-63 */
+void orc_strided_copy(float *dst, size_t dst_stride, const float *src, size_t src_stride, size_t rows,
+                      size_t cols);
+
+/* csrc/ops/attn_core_cpu.c:16-57.  Weights land in weights_out, else in
+ * scores_scratch, as the reference does. */
+int orc_attention_head_core(const blt_attention_head_args *a);
+
+/* The reference's caller loop: one core call per (sequence, head), in array
+ * order (csrc/models/attention.c:199-202).  Stops at the first failure. */
+int orc_attention_head_core_many(const blt_attention_head_args *a, size_t count);
+
+/* csrc/ops/mask_builder_cpu.c:11-95.  `out` is [seq_len_q * seq_len_kv]. */
+int orc_build_attention_mask(const blt_mask_config *config, float *out);
+
+/* csrc/ops/mask_builder_cpu.c:97-154.  `out` is [seq_len * seq_len]. */
+int orc_build_block_diffusion_mask(const blt_block_diffusion_config *config, float *out);
+
+/* csrc/ops/patch_pool_cpu.c:98-112 */
+int orc_patch_build_group_ids(const blt_patch_info *patches, size_t num_patches, size_t seq_len,
+                              size_t *query_group_ids_out, size_t *kv_group_ids_out);
+
+/* csrc/ops/patch_pool_cpu.c:114-131 */
+size_t orc_patch_decoder_latent_at(const blt_patch_info *patches, size_t num_patches, size_t pos);
+
+/* csrc/ops/patch_pool_cpu.c:133-142 */
+void orc_patch_expand_group_ids(const size_t *group_ids_in, size_t n, size_t k, size_t *group_ids_out);
+
+/* ---- KV cache: layout, step masks, write-through, attend --------------- */
+
+/* Row of the tier-1 slab that holds absolute byte position `pos` of sequence
+ * `b`: tensors are [batch*max_seq_len, E] row-major (kv_cache.c:56-60), row
+ * index == absolute position (kv_cache.h:17-18). */
+size_t orc_kv_row(size_t b, size_t pos, size_t max_seq_len);
+
+/* Element offset of (b, pos, head, d) in a tier-1 tensor. */
+size_t orc_kv_slot(size_t b, size_t pos, size_t head, size_t d, size_t max_seq_len, size_t embed_dim,
+                   size_t head_dim);
+
+/* Self-attention step mask, kv_cache.c:224-238: n rows, total = base + n
+ * columns; allowed = j <= base+r and (window == 0 or base+r-j < window). */
+void orc_kv_self_mask(float *out, size_t n, size_t base, size_t window);
+
+/* Query/KV group ids of a decode step, kv_cache.c:203-218. */
+void orc_kv_step_group_ids(const blt_patch_info *patches, size_t num_patches, size_t k_split, size_t base,
+                           size_t n, int trailing_closed, size_t *q_group_ids, size_t *kv_group_ids);
+
+/* Cross-attention step mask, kv_cache.c:240-251. */
+void orc_kv_cross_mask(float *out, const size_t *q_group_ids, size_t n, const size_t *kv_group_ids,
+                       size_t total_sub);
+
+/* The attention part of one decode step for one sequence, kv_cache.c:343-390
+ * without the projections and RoPE: `q_rows`, `k_rows`, `v_rows` are the n new
+ * rows [n, E] (K already rotated).  K/V rows are written through to slab rows
+ * [base, base+n) of sequence `b` FIRST, then every head attends over rows
+ * [0, base+n) with the dense step mask, weights_out == NULL and a scratch
+ * score buffer.  `combined` [n, E] is zeroed and then filled head by head.
+ * Scratch buffers are allocated inside.  Returns ORC_ERR_CAPACITY when
+ * base + n exceeds max_seq_len. */
+int orc_kv_attend_step(float *self_k, float *self_v, size_t max_seq_len, size_t embed_dim, size_t num_heads,
+                       size_t b, size_t base, size_t n, size_t window, const float *q_rows,
+                       const float *k_rows, const float *v_rows, float *combined);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* FBLT_AMD_ORACLE_H */

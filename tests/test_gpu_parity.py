@@ -1,0 +1,411 @@
+"""GPU parity: the HIP library against the CPU checker on identical seeded inputs.
+
+Every compute call goes through the C-ABI of libfblt_hip.so.  Tolerance for
+fp32 attention outputs and weights (stated by the task): |got - ref| <=
+1e-5 + 1e-4 * |ref| element-wise; integer/boolean work (masks, cache slots,
+lengths) must be bit-exact.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from fblt_amd import abi, api, workloads
+from oracle import binding, runner as orunner
+
+pytestmark = pytest.mark.gpu
+
+ATOL, RTOL = 1e-5, 1e-4
+
+
+def assert_close(got, ref, what=""):
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    assert got.shape == ref.shape, (what, got.shape, ref.shape)
+    err = np.abs(got - ref)
+    bound = ATOL + RTOL * np.abs(ref)
+    bad = err > bound
+    assert not bad.any(), "%s: %d/%d out of tolerance, max abs err %.3e at %s (got %r ref %r)" % (
+        what, int(bad.sum()), bad.size, float(err.max()), np.unravel_index(int(err.argmax()), err.shape),
+        float(got.flat[int(err.argmax())]), float(ref.flat[int(err.argmax())]))
+    return float(err.max())
+
+
+@pytest.fixture(scope="module")
+def dev():
+    from fblt_amd import runner
+    return runner
+
+
+def _oracle_out(w, orc, weights=None):
+    for n in w.outputs:
+        w.buffers[n][:] = 0
+    orunner.run(w, lib=orc, weights=weights)
+    return {n: w.buffers[n].copy() for n in w.outputs}
+
+
+def _families(monkeypatch, fam):
+    # the override is read once per process; tests pin it through a reload of the cache
+    pass
+
+
+# ---------------------------------------------------------------------------
+# configs 1-3 through every entry point
+# ---------------------------------------------------------------------------
+SMALL = {
+    "c1_small": lambda: workloads.config1(batch=1, T=96, H=2, hd=32),
+    "c1_ragged": lambda: workloads.config1(batch=2, T=77, H=2, hd=32),
+    "c2_small": lambda: workloads.config2(batch=2, P=48, H=2, hd=64, T_bytes=192),
+    "c3_small": lambda: workloads.config3(batch=2, T=128, P=32, H=2, hd=32),
+    "c1_hd16": lambda: workloads.config1(batch=1, T=50, H=3, hd=16),
+    "c1_hd128": lambda: workloads.config1(batch=1, T=40, H=1, hd=128),
+    "c1_hd8": lambda: workloads.config1(batch=1, T=33, H=2, hd=8),
+}
+FULL = {
+    "c1_full": lambda: workloads.config1(),
+    "c2_full": lambda: workloads.config2(),
+    "c3_full": lambda: workloads.config3(),
+}
+
+
+@pytest.mark.parametrize("name", list(SMALL) + list(FULL))
+@pytest.mark.parametrize("entry", ["per_head_dense", "per_head_flag", "batch_descriptor", "batch_dense", "plan"])
+def test_dense_configs(name, entry, oracle, dev):
+    w = (SMALL.get(name) or FULL[name])()
+    if entry == "per_head_flag" and w.heads[0].mask != "causal":
+        pytest.skip("is_causal flag only describes causal problems")
+    if name in FULL and entry in ("batch_dense",):
+        pytest.skip("covered at reduced size")
+    ref = _oracle_out(w, oracle)
+    d = dev.DeviceWorkload(w)
+    try:
+        d.zero_outputs()
+        if entry == "per_head_dense":
+            d.run_per_head("dense", with_weights=True)
+        elif entry == "per_head_flag":
+            d.run_per_head("flag", with_weights=False)
+        elif entry == "batch_descriptor":
+            d.run_batch("descriptor")
+        elif entry == "batch_dense":
+            d.run_batch("dense")
+        else:
+            plan = d.make_plan("descriptor")
+            d.lib.blt_attention_plan_run_hip(plan)
+            d.lib.blt_backend_pass_sync_hip()
+            d.lib.blt_attention_plan_destroy_hip(plan)
+        got = d.output("out")
+    finally:
+        d.close()
+    assert_close(got, ref["out"], "%s/%s" % (name, entry))
+
+
+@pytest.mark.parametrize("name", ["c1_small", "c1_ragged", "c2_small", "c3_small"])
+@pytest.mark.parametrize("mask_mode", ["descriptor", "dense"])
+def test_weights_and_lse(name, mask_mode, oracle, dev):
+    """weights_out holds the post-softmax weights (zeros where masked); lse_out holds (max, sum)."""
+    import torch
+    w = SMALL[name]()
+    host_w = [np.zeros(h.nq * h.nk, dtype=np.float32) for h in w.heads]
+    ref = _oracle_out(w, oracle, weights=host_w)
+    d = dev.DeviceWorkload(w)
+    try:
+        d.zero_outputs()
+        wbufs = [torch.full((h.nq * h.nk,), 7.0, dtype=torch.float32, device="cuda") for h in w.heads]
+        lbufs = [torch.full((h.nq * 2,), 7.0, dtype=torch.float32, device="cuda") for h in w.heads]
+        arr = d.problems(mask_mode, [t.data_ptr() for t in wbufs], [t.data_ptr() for t in lbufs])
+        d.lib.blt_attention_batch_hip(arr, len(w.heads))
+        d.lib.blt_backend_pass_sync_hip()
+        got = d.output("out")
+        assert_close(got, ref["out"], name)
+        for t, h in enumerate(w.heads):
+            gw = wbufs[t].cpu().numpy()
+            assert_close(gw, host_w[t], "%s weights head %d" % (name, t))
+            assert ((gw == 0) == (host_w[t] == 0)).all(), "masked pattern differs"
+            lse = lbufs[t].cpu().numpy().reshape(h.nq, 2)
+            # (m, l): weights = exp(x - m) / l, so sum of ref weights * l == sum exp == l
+            assert np.isfinite(lse).all()
+            assert (lse[:, 1] >= 1.0 - 1e-4).all()  # the max term contributes exp(0) = 1
+    finally:
+        d.close()
+
+
+# ---------------------------------------------------------------------------
+# per-head call: the reference's own vectors and edge cases
+# ---------------------------------------------------------------------------
+def _run_single(lib, q, k, v, nq, nk, hd, scale, q_stride, k_stride, v_stride, out_cols, col, q_off=0, k_off=0,
+                v_off=0, mask=None, causal=False, want_weights=True):
+    import torch
+    tq, tk, tv = (torch.from_numpy(x).cuda() for x in (q, k, v))
+    out = torch.full((nq * out_cols,), 5.0, dtype=torch.float32, device="cuda")
+    wts = torch.full((max(nq * nk, 1),), 9.0, dtype=torch.float32, device="cuda")
+    tm = torch.from_numpy(mask).cuda() if mask is not None else None
+    a = api.head_args(tq.data_ptr() + 4 * q_off, tk.data_ptr() + 4 * k_off, tv.data_ptr() + 4 * v_off,
+                      out.data_ptr(), nq, nk, hd, scale, q_stride, k_stride, v_stride, out_cols, col,
+                      weights=wts.data_ptr() if want_weights else None,
+                      scratch=None if want_weights else wts.data_ptr(),
+                      mask=tm.data_ptr() if tm is not None else None, causal=causal)
+    lib.blt_attention_head_core_hip(abi.BLT_BACKEND_HIP, C.byref(a))
+    lib.blt_backend_pass_sync_hip()
+    return out.cpu().numpy().reshape(nq, out_cols), wts.cpu().numpy()[:nq * nk].reshape(nq, nk)
+
+
+def test_reference_identity_vector(dev):
+    """tests/unit/models/unit_attention.c:24-88: identity projections, 2 tokens, 2 heads of dim 2."""
+    lib = api.load()
+    qkv = np.zeros((2, 12), dtype=np.float32)
+    x = np.array([[1, 0, 1, 0], [0, 1, 0, 1]], dtype=np.float32)
+    qkv[:, 0:4] = x
+    qkv[:, 4:8] = x
+    qkv[:, 8:12] = x
+    scale = float(1.0 / np.sqrt(np.float32(2.0)))
+    want = np.array([[0.6697615, 0.3302385, 0.6697615, 0.3302385], [0.3302385, 0.6697615, 0.3302385, 0.6697615]])
+    got = np.zeros((2, 4))
+    for h in range(2):
+        o, _ = _run_single(lib, qkv.reshape(-1), qkv.reshape(-1), qkv.reshape(-1), 2, 2, 2, scale, 12, 12, 12, 4,
+                           2 * h, q_off=2 * h, k_off=4 + 2 * h, v_off=8 + 2 * h)
+        got[:, 2 * h:2 * h + 2] = o[:, 2 * h:2 * h + 2]
+        # columns of the other head are left alone (sentinel 5.0)
+        other = [c for c in range(4) if c // 2 != h]
+        assert (o[:, other] == 5.0).all()
+    assert np.abs(got - want).max() < 1e-6
+    # causal variant (unit_attention.c:160-171): row 0 sees only itself
+    want_c = np.array([[1, 0, 1, 0], [0.3302385, 0.6697615, 0.3302385, 0.6697615]])
+    for h in range(2):
+        o, wts = _run_single(lib, qkv.reshape(-1), qkv.reshape(-1), qkv.reshape(-1), 2, 2, 2, scale, 12, 12, 12, 4,
+                             2 * h, q_off=2 * h, k_off=4 + 2 * h, v_off=8 + 2 * h, causal=True)
+        assert np.abs(o[:, 2 * h:2 * h + 2] - want_c[:, 2 * h:2 * h + 2]).max() < 1e-6
+        assert wts[0, 1] == 0.0 and abs(wts[0, 0] - 1.0) < 1e-6
+
+
+@pytest.mark.parametrize("nq,nk,hd", [(1, 1, 32), (1, 300, 32), (5, 7, 32), (31, 33, 64), (64, 65, 32),
+                                      (17, 129, 128), (3, 40, 20), (40, 40, 6), (2, 5, 200)])
+@pytest.mark.parametrize("masked", ["none", "causal", "dense_random"])
+def test_single_head_shapes(nq, nk, hd, masked, oracle, dev):
+    """Ragged shapes, odd head dims and unaligned strides through the per-head call."""
+    lib = api.load()
+    rs = np.random.RandomState(1000 * nq + nk + hd)
+    stride = hd + 3  # not a multiple of 4: forces the scalar access path
+    q = rs.randn(nq, stride).astype(np.float32)
+    k = rs.randn(nk, stride).astype(np.float32)
+    v = rs.randn(nk, stride).astype(np.float32)
+    scale = float(1.0 / np.sqrt(np.float32(hd)))
+    mask = None
+    causal = masked == "causal"
+    if masked == "dense_random":
+        mask = np.where(rs.rand(nq, nk) < 0.4, -np.inf, 0.0).astype(np.float32)
+        mask[0, :] = -np.inf  # an all-masked row must give zeros
+        if nq > 1:
+            mask[1, :] = 0.0
+    out_ref = np.zeros((nq, hd + 1), dtype=np.float32)
+    w_ref = np.zeros((nq, nk), dtype=np.float32)
+    a = binding.head_args(q.reshape(-1), k.reshape(-1), v.reshape(-1), out_ref.reshape(-1), nq, nk, hd, scale,
+                          stride, stride, stride, hd + 1, 1, weights=w_ref.reshape(-1),
+                          mask=None if mask is None else mask.reshape(-1), causal=causal)
+    assert oracle.orc_attention_head_core(C.byref(a)) == 0
+    got, gw = _run_single(lib, q.reshape(-1), k.reshape(-1), v.reshape(-1), nq, nk, hd, scale, stride, stride, stride,
+                          hd + 1, 1, mask=None if mask is None else mask.reshape(-1), causal=causal)
+    assert (got[:, 0] == 5.0).all(), "column outside the head slice was written"
+    assert_close(got[:, 1:], out_ref[:, 1:], "out")
+    assert_close(gw, w_ref, "weights")
+    if mask is not None:
+        assert (got[0, 1:] == 0).all() and (gw[0] == 0).all()
+
+
+def test_additive_mask_values(oracle, dev):
+    """A dense mask is additive: finite biases shift the scores, +inf / nan entries drop the key."""
+    lib = api.load()
+    rs = np.random.RandomState(7)
+    nq, nk, hd = 37, 70, 32
+    q, k, v = (rs.randn(n, hd).astype(np.float32) for n in (nq, nk, nk))
+    mask = (rs.randn(nq, nk) * 2).astype(np.float32)
+    mask[rs.rand(nq, nk) < 0.2] = -np.inf
+    mask[2, 3] = np.inf
+    mask[4, 5] = np.nan
+    scale = 0.25
+    out_ref = np.zeros((nq, hd), dtype=np.float32)
+    w_ref = np.zeros((nq, nk), dtype=np.float32)
+    a = binding.head_args(q.reshape(-1), k.reshape(-1), v.reshape(-1), out_ref.reshape(-1), nq, nk, hd, scale, hd, hd,
+                          hd, hd, 0, weights=w_ref.reshape(-1), mask=mask.reshape(-1))
+    assert oracle.orc_attention_head_core(C.byref(a)) == 0
+    got, gw = _run_single(lib, q.reshape(-1), k.reshape(-1), v.reshape(-1), nq, nk, hd, scale, hd, hd, hd, hd, 0,
+                          mask=mask.reshape(-1))
+    assert_close(got, out_ref, "out")
+    assert_close(gw, w_ref, "weights")
+    assert gw[2, 3] == 0 and gw[4, 5] == 0
+
+
+# ---------------------------------------------------------------------------
+# dense mask builders on the device: bit-exact
+# ---------------------------------------------------------------------------
+def _variants():
+    sq, skv = 19, 23
+    docs = [7, 15, 15]
+    qg = [i % 3 for i in range(sq)]
+    kg = [j % 3 for j in range(skv)]
+    # the variant matrix of tests/parity/parity_cuda_composites.c:66-105
+    table = [(True, 0, False, False, False), (False, 5, False, False, False), (True, 4, True, False, False),
+             (False, 0, True, False, False), (True, 0, False, True, True), (True, 0, False, True, False),
+             (True, 6, True, True, True)]
+    for causal, window, use_docs, use_groups, bidir in table:
+        yield sq, skv, causal, window, docs if use_docs else None, (qg, kg) if use_groups else None, bidir, 0
+    # sizes past one block, causal offsets, sorted groups (cross-attention)
+    yield 300, 517, True, 0, None, None, False, 217
+    yield 300, 517, True, 64, None, None, False, 217
+    yield 128, 512, False, 0, None, ([p for p in range(128)], [j // 4 for j in range(512)]), True, 0
+
+
+@pytest.mark.parametrize("case", list(_variants()), ids=lambda c: "q%d_k%d_c%d_w%d_d%d_g%d_b%d_o%d" % (
+    c[0], c[1], c[2], c[3], c[4] is not None, c[5] is not None, c[6], c[7]))
+def test_attention_mask_bit_exact(case, oracle, dev):
+    sq, skv, causal, window, docs, groups, bidir, off = case
+    lib = api.load()
+    cfg = abi.BltMaskConfig()
+    cfg.seq_len_q, cfg.seq_len_kv = sq, skv
+    cfg.is_causal, cfg.sliding_window, cfg.causal_offset = causal, window, off
+    keep = []
+    if docs is not None:
+        arr = abi.size_array(docs)
+        keep.append(arr)
+        cfg.doc_boundaries, cfg.num_docs = arr, len(docs) + 1
+    if groups is not None:
+        qa, ka = abi.size_array(groups[0]), abi.size_array(groups[1])
+        keep += [qa, ka]
+        cfg.query_group_ids, cfg.kv_group_ids = qa, ka
+        cfg.bidirectional_within_group = bidir
+    want = np.empty(sq * skv, dtype=np.float32)
+    assert oracle.orc_build_attention_mask(C.byref(cfg), binding.fptr(want)) == 0
+    arena = lib.blt_arena_create(8 << 20, abi.BLT_BACKEND_HIP)
+    t = abi.BltTensor()
+    lib.blt_build_attention_mask(C.byref(cfg), C.byref(t), arena)  # public dispatcher -> HIP twin
+    assert t.backend == abi.BLT_BACKEND_HIP and t.shape[0] == sq and t.shape[1] == skv and t.numel == sq * skv
+    got = np.empty(sq * skv, dtype=np.float32)
+    lib.blt_tensor_download(C.byref(t), got.ctypes.data, got.nbytes)
+    lib.blt_arena_destroy(arena)
+    assert got.tobytes() == want.tobytes()
+    # the row-range reduction describes the same visibility whenever it claims to
+    lo = (C.c_uint32 * sq)()
+    hi = (C.c_uint32 * sq)()
+    if lib.blt_mask_config_row_ranges(C.byref(cfg), lo, hi):
+        allowed = want.reshape(sq, skv) == 0
+        for i in range(sq):
+            row = np.zeros(skv, dtype=bool)
+            row[lo[i]:hi[i]] = True
+            assert (row == allowed[i]).all(), i
+    else:
+        assert groups is not None  # only unsorted group ids are not interval-shaped
+
+
+@pytest.mark.parametrize("mode,S,N,B,starts", [
+    (abi.BLT_BDM_TRAIN, 14, 6, 4, [2, 4]),
+    (abi.BLT_BDM_INFER, 7, 3, 0, None),
+    (abi.BLT_BDM_TRAIN, 24, 12, 2, [0, 4, 1, 7, 3, 11]),
+    (abi.BLT_BDM_INFER, 24, 12, 2, None),
+    (abi.BLT_BDM_INFER, 524, 508, 16, None),
+    (abi.BLT_BDM_TRAIN, 9 + 3 * 4, 9, 3, [1, 3, 5, 8]),
+])
+def test_block_diffusion_mask_bit_exact(mode, S, N, B, starts, oracle, dev):
+    lib = api.load()
+    cfg = abi.BltBlockDiffusionConfig()
+    cfg.mode, cfg.seq_len, cfg.num_clean, cfg.block_size = mode, S, N, B
+    keep = None
+    if starts is not None:
+        keep = abi.size_array(starts)
+        cfg.block_starts, cfg.num_blocks = keep, len(starts)
+    want = np.empty(S * S, dtype=np.float32)
+    assert oracle.orc_build_block_diffusion_mask(C.byref(cfg), binding.fptr(want)) == 0
+    arena = lib.blt_arena_create(8 << 20, abi.BLT_BACKEND_HIP)
+    t = abi.BltTensor()
+    lib.blt_build_block_diffusion_mask(C.byref(cfg), C.byref(t), arena)
+    got = np.empty(S * S, dtype=np.float32)
+    lib.blt_tensor_download(C.byref(t), got.ctypes.data, got.nbytes)
+    lib.blt_arena_destroy(arena)
+    assert got.tobytes() == want.tobytes()
+
+
+# ---------------------------------------------------------------------------
+# KV-cache step (config 4) and block verify (config 5)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("batch,steps,H,hd,len_hi", [(3, 5, 4, 32, 70), (64, 6, 4, 32, 512), (5, 4, 2, 64, 100),
+                                                     (4, 3, 8, 16, 40), (2, 40, 4, 32, 3)])
+def test_kv_decode_steps(batch, steps, H, hd, len_hi, oracle, dev):
+    kw = workloads.config4(batch=batch, steps=steps, H=H, hd=hd, len_hi=len_hi)
+    ref_out, ref_k, ref_v = orunner.run_kv(kw, lib=oracle)
+    d = dev.DeviceKvWorkload(kw)
+    d.run()
+    out, ck, cv, lens = d.results()
+    assert (lens == kw.lens.astype(np.int64) + steps).all()          # slot bookkeeping: exact
+    assert ck.tobytes() == ref_k.tobytes() and cv.tobytes() == ref_v.tobytes()  # write-through: bit-exact rows
+    assert_close(out, ref_out, "kv decode")
+
+
+def test_kv_decode_window(oracle, dev):
+    kw = workloads.config4(batch=6, steps=4, H=4, hd=32, len_hi=200)
+    kw.window = 48
+    ref_out, ref_k, ref_v = orunner.run_kv(kw, lib=oracle)
+    d = dev.DeviceKvWorkload(kw)
+    d.run()
+    out, ck, cv, lens = d.results()
+    assert ck.tobytes() == ref_k.tobytes()
+    assert_close(out, ref_out, "kv decode window")
+
+
+@pytest.mark.parametrize("n", [2, 3, 8, 20])
+def test_kv_prefill_chunk(n, oracle, dev):
+    """n > 1 rows per step, chunk-causal (kv_cache.c:229-236): same kernel, causal kind."""
+    kw = workloads.config4(batch=5, steps=3, H=4, hd=32, len_hi=90)
+    rs = np.random.RandomState(n)
+    kw.n = n
+    kw.q_new, kw.k_new, kw.v_new = (rs.randn(kw.steps, kw.batch * n, kw.E).astype(np.float32) for _ in range(3))
+    ref_out, ref_k, ref_v = orunner.run_kv(kw, lib=oracle)
+    d = dev.DeviceKvWorkload(kw)
+    d.run()
+    out, ck, cv, lens = d.results()
+    assert (lens == kw.lens.astype(np.int64) + n * kw.steps).all()
+    assert ck.tobytes() == ref_k.tobytes() and cv.tobytes() == ref_v.tobytes()
+    assert_close(out, ref_out, "kv chunk n=%d" % n)
+
+
+@pytest.mark.parametrize("B", [4, 8, 16, 32])
+@pytest.mark.parametrize("batch", [3, 64])
+def test_block_verify(B, batch, oracle, dev):
+    kw = workloads.config5(batch=batch, B=B)
+    ref_out, ref_k, ref_v = orunner.run_kv(kw, lib=oracle)
+    d = dev.DeviceKvWorkload(kw)
+    d.run()
+    out, ck, cv, lens = d.results()
+    assert (lens == kw.lens).all()   # verify does not commit
+    assert ck.tobytes() == ref_k.tobytes() and cv.tobytes() == ref_v.tobytes()
+    assert_close(out, ref_out, "block verify B=%d" % B)
+
+
+# ---------------------------------------------------------------------------
+# small device utilities
+# ---------------------------------------------------------------------------
+def test_strided_copy_softmax_dot(oracle, dev):
+    import torch
+    lib = api.load()
+    rs = np.random.RandomState(3)
+    src = rs.randn(9, 24).astype(np.float32)
+    tsrc = torch.from_numpy(src).cuda()
+    for cols, off in [(8, 4), (5, 3)]:
+        dst = torch.zeros((9, 16), dtype=torch.float32, device="cuda")
+        lib.blt_strided_copy(abi.BLT_BACKEND_HIP, dst.data_ptr() + 4 * 2, 16, tsrc.data_ptr() + 4 * off, 24, 9, cols)
+        lib.blt_backend_pass_sync(abi.BLT_BACKEND_HIP)
+        want = np.zeros((9, 16), dtype=np.float32)
+        want[:, 2:2 + cols] = src[:, off:off + cols]
+        assert (dst.cpu().numpy() == want).all()
+    for n, causal, use_mask in [(1, False, False), (300, True, False), (1000, False, True)]:
+        row = rs.randn(n).astype(np.float32) * 3
+        mask = np.where(rs.rand(n) < 0.3, -np.inf, 0).astype(np.float32) if use_mask else None
+        ref = row.copy()
+        oracle.orc_softmax_masked_row_inplace(binding.fptr(ref), n, n // 2, causal, binding.fptr(mask), 0.5)
+        t = torch.from_numpy(row).cuda()
+        tm = torch.from_numpy(mask).cuda() if use_mask else None
+        lib.blt_softmax_masked_row_inplace(abi.BLT_BACKEND_HIP, t.data_ptr(), n, n // 2, causal,
+                                           tm.data_ptr() if use_mask else None, 0.5)
+        lib.blt_backend_pass_sync(abi.BLT_BACKEND_HIP)
+        assert_close(t.cpu().numpy(), ref, "softmax row")
+    a, b = rs.randn(777).astype(np.float32), rs.randn(777).astype(np.float32)
+    ta, tb = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    got = lib.blt_vec_dot(abi.BLT_BACKEND_HIP, ta.data_ptr(), tb.data_ptr(), 777)
+    assert abs(got - float(np.dot(a.astype(np.float64), b.astype(np.float64)))) < 1e-3
