@@ -352,7 +352,7 @@ def test_kv_decode_window(oracle, dev):
 @pytest.mark.parametrize("n", [2, 3, 8, 20])
 def test_kv_prefill_chunk(n, oracle, dev):
     """n > 1 rows per step, chunk-causal (kv_cache.c:229-236): same kernel, causal kind."""
-    kw = workloads.config4(batch=5, steps=3, H=4, hd=32, len_hi=90)
+    kw = workloads.config4(batch=5, steps=3, H=4, hd=32, len_hi=90, max_seq_len=90 + 3 * n)
     rs = np.random.RandomState(n)
     kw.n = n
     kw.q_new, kw.k_new, kw.v_new = (rs.randn(kw.steps, kw.batch * n, kw.E).astype(np.float32) for _ in range(3))
