@@ -1,0 +1,251 @@
+#!/usr/bin/env python3
+"""Attention hot-path benchmark on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only c2]
+
+A "step" is one pass of the headline workload -- the patch-transformer
+block-causal attention (batch 16, 128 patches, 8 heads of 64, fp32) -- through
+the HIP library: one resident plan, one kernel launch per step, inputs already
+in HBM.  The single JSON line on stdout carries the whole-job throughput of
+that workload, the roofline figures of its kernel (duration from HIP events
+attached to every launch of the timed region), the CPU baseline (the checker
+under oracle/, one host core, bounded sample) and, under "workloads", the same
+figures for the other four attention shapes of the path.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
+
+# HBM bytes per launch from `rocprofv3 --pmc` (FETCH_SIZE, WRITE_SIZE; see the
+# summaries under profiles/), None where not measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def roofline(bound, work, avg_s, traffic=None):
+    """work = algorithmic bytes (hbm) or flops (mfma) per launch."""
+    if bound == "hbm":
+        achieved, peak, unit = work / avg_s / 1e9, HBM_PEAK_GBS, "GB/s"
+    else:
+        achieved, peak, unit = work / avg_s / 1e12, FP32_MFMA_PEAK_TFLOPS, "TFLOP/s"
+    return {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
+            "traffic": traffic}
+
+
+def time_plan(lib, api, plan, steps, warmup):
+    """(wall seconds for `steps` launches, {tag: (launches, total_ms, min, max)})."""
+    for _ in range(warmup):
+        lib.blt_attention_plan_run_hip(plan)
+    lib.blt_backend_pass_sync_hip()
+    lib.blt_hip_profile_begin()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        lib.blt_attention_plan_run_hip(plan)
+    lib.blt_backend_pass_sync_hip()
+    wall = time.perf_counter() - t0
+    return wall, api.profile_end()
+
+
+def bench_dense(make, steps, warmup, bound, mask_mode="descriptor"):
+    from fblt_amd import api, runner
+    lib = api.load()
+    w = make()
+    d = runner.DeviceWorkload(w)
+    plan = d.make_plan(mask_mode)
+    kernel = lib.blt_attention_plan_kernel_hip(plan).decode()
+    wall, prof = time_plan(lib, api, plan, steps, warmup)
+    # the same launches without events attached: the whole-job rate
+    lib.blt_backend_pass_sync_hip()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        lib.blt_attention_plan_run_hip(plan)
+    lib.blt_backend_pass_sync_hip()
+    wall_plain = time.perf_counter() - t0
+    lib.blt_attention_plan_destroy_hip(plan)
+    d.close()
+    launches = sum(v[0] for v in prof.values())
+    kern_ms = sum(v[1] for v in prof.values())
+    avg_s = kern_ms / 1e3 / steps       # device time of one step (all its launches)
+    res = {
+        "workload": w.name, "kernel": kernel, "launches_per_step": launches / steps,
+        "tokens_per_step": w.tokens, "ms_per_step": wall_plain / steps * 1e3,
+        "ms_per_step_with_events": wall / steps * 1e3,
+        "kernel_us_avg": avg_s * 1e6, "kernel_us_min": min(v[2] for v in prof.values()) * 1e3,
+        "tokens_per_s": w.tokens * steps / wall_plain,
+        "tokens_per_s_kernel": w.tokens / avg_s,
+        "flops": w.flops, "bytes": w.bytes,
+        "roofline_hbm": roofline("hbm", w.bytes, avg_s, MEASURED_TRAFFIC_BYTES.get(w.name)),
+        "roofline_mfma": roofline("mfma", w.flops, avg_s),
+    }
+    res["roofline"] = res["roofline_" + bound]
+    return res, w
+
+
+def bench_kv(kw, steps, warmup):
+    """KV-cache workloads: `steps` consecutive step calls after `warmup` calls.  A
+    committing workload (decode) appends one row per call and needs kw.steps >=
+    warmup + steps; a non-committing one (verify) repeats its single step."""
+    from fblt_amd import api, runner
+    lib = api.load()
+    d = runner.DeviceKvWorkload(kw)
+    idx = (lambda s: s) if kw.commit else (lambda s: 0)
+
+    def one_pass(profiled):
+        d.reset()
+        for s in range(warmup):
+            d.step(idx(s))
+        lib.blt_backend_pass_sync_hip()
+        if profiled:
+            lib.blt_hip_profile_begin()
+        t0 = time.perf_counter()
+        for s in range(warmup, warmup + steps):
+            d.step(idx(s))
+        lib.blt_backend_pass_sync_hip()
+        wall = time.perf_counter() - t0
+        return wall, (api.profile_end() if profiled else None)
+
+    wall, prof = one_pass(True)
+    wall_plain, _ = one_pass(False)
+    kern_ms = sum(v[1] for v in prof.values())
+    launches = sum(v[0] for v in prof.values())
+    avg_s = kern_ms / 1e3 / steps
+    # algorithmic work of an average timed step: lengths grow by n per committed step
+    E, n = kw.E, kw.n
+    base = float(kw.lens.astype("int64").sum())
+    grown = kw.batch * n * (warmup + (steps - 1) / 2.0) if kw.commit else 0.0
+    mean_keys = base + grown + kw.batch * n            # sum over sequences of keys attended
+    rows = kw.batch * n
+    # K and V of every attended key, plus Q in / O out per row, plus the appended K/V rows (decode)
+    bytes_step = 4.0 * (2 * E * mean_keys + rows * 2 * E + (rows * 2 * E if kw.commit else 0))
+    flops_step = 4.0 * kw.hd * kw.H * n * mean_keys
+    res = {
+        "workload": kw.name, "kernel": "kv_step", "launches_per_step": launches / steps,
+        "tokens_per_step": kw.tokens, "us_per_step": wall_plain / steps * 1e6,
+        "us_per_step_with_events": wall / steps * 1e6, "kernel_us_avg": avg_s * 1e6,
+        "kernel_us_min": min(v[2] for v in prof.values()) * 1e3,
+        "tokens_per_s": kw.tokens * steps / wall_plain, "tokens_per_s_kernel": kw.tokens / avg_s,
+        "flops": flops_step, "bytes": bytes_step,
+        "roofline_hbm": roofline("hbm", bytes_step, avg_s, MEASURED_TRAFFIC_BYTES.get(kw.name)),
+        "roofline_mfma": roofline("mfma", flops_step, avg_s),
+    }
+    res["roofline"] = res["roofline_hbm"]
+    return res, kw
+
+
+def cpu_dense(w, budget_s):
+    """Checker on one host core over the same workload; repeated whole passes up to the budget."""
+    from oracle import binding, runner as orunner
+    lib = binding.load_oracle()
+    passes, spent = 0, 0.0
+    while passes < 1 or (spent < budget_s and passes < 200):
+        spent += orunner.run(w, lib=lib, timed=True)
+        passes += 1
+    return {"value": w.tokens * passes / spent, "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": "%d full passes of %s, %.1f s, dense mask passed in, one core call per (sequence, head)"
+                      % (passes, w.name, spent), "ms_per_pass": spent / passes * 1e3}
+
+
+def cpu_kv(kw, budget_s, max_steps):
+    from oracle import binding, runner as orunner
+    lib = binding.load_oracle()
+    steps = 1
+    out = orunner.run_kv(kw, lib=lib, steps=1, timed=True)
+    per = out[3]
+    steps = int(max(1, min(max_steps, budget_s / max(per, 1e-6))))
+    out = orunner.run_kv(kw, lib=lib, steps=steps, timed=True)
+    spent = out[3]
+    return {"value": kw.tokens * steps / spent, "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": "first %d steps of %s, %.1f s, write-through then one core call per (sequence, head)"
+                      % (steps, kw.name, spent), "us_per_step": spent / steps * 1e6}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--only", default="", help="comma list of c1,c2,c3,c4,c5 (c2 always runs)")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU budget of the headline workload")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the workload shards by sequence "
+                 "with no exchange step; run one process per GPU on its own sequences). Use --gpus 1.")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU: the HIP attention backend has no CPU path")
+    from fblt_amd import workloads
+
+    only = set(x for x in args.only.split(",") if x)
+    want = lambda c: not only or c in only
+    K, W = args.steps, args.warmup
+
+    head, w2 = bench_dense(workloads.config2, K, W, "hbm")
+    log("c2", json.dumps(head))
+    others = {}
+    cpu = {}
+    if want("c1"):
+        others["c1"], w1 = bench_dense(workloads.config1, K, W, "mfma")
+        log("c1", json.dumps(others["c1"]))
+    if want("c3"):
+        others["c3"], w3 = bench_dense(workloads.config3, K, W, "hbm")
+        log("c3", json.dumps(others["c3"]))
+    if want("c4"):
+        others["c4"], k4 = bench_kv(workloads.config4(steps=W + 256, max_seq_len=512 + W + 256), 256, W)
+        log("c4", json.dumps(others["c4"]))
+    if want("c5"):
+        for B in (4, 8, 16):
+            others["c5_B%d" % B], k5 = bench_kv(workloads.config5(B=B), K, W)
+            log("c5_B%d" % B, json.dumps(others["c5_B%d" % B]))
+    # batch-swept prefill: the same kernels away from the launch floor
+    if want("sweep"):
+        for name, make in (("c1_x64", lambda: workloads.config1(batch=64)),
+                           ("c2_x8", lambda: workloads.config2(batch=128))):
+            others[name], _ = bench_dense(make, max(10, K // 10), 3, "mfma")
+            log(name, json.dumps(others[name]))
+
+    cpu_head = None
+    if not args.no_cpu:
+        cpu_head = cpu_dense(w2, args.cpu_seconds)
+        log("cpu c2", json.dumps(cpu_head))
+        if want("c1"):
+            others["c1"]["cpu_baseline"] = cpu_dense(w1, 2.0)
+        if want("c3"):
+            others["c3"]["cpu_baseline"] = cpu_dense(w3, 2.0)
+        if want("c4"):
+            others["c4"]["cpu_baseline"] = cpu_kv(workloads.config4(steps=64), 3.0, 64)
+        if want("c5"):
+            for B in (4, 8, 16):
+                others["c5_B%d" % B]["cpu_baseline"] = cpu_kv(workloads.config5(B=B, steps=1), 1.0, 1)
+
+    line = {
+        "metric": "attn_tokens_per_s", "value": head["tokens_per_s"], "unit": "tokens/s",
+        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "patch-transformer block-causal attention: batch 16, P=128 patches, 8 heads, "
+                               "head_dim 64, fp32, seeded N(0,1) (BASELINE configs[1])",
+                   "entry": "blt_attention_plan_run_hip, causal descriptor, one launch per step",
+                   "kernel": head["kernel"], "tokens_per_step": head["tokens_per_step"]},
+        "kernel_us_avg": head["kernel_us_avg"],
+        "roofline": head["roofline"],
+        "roofline_mfma": head["roofline_mfma"],
+        "cpu_baseline": cpu_head,
+        "workloads": others,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -45,6 +45,11 @@ class BltKvAttnCache(C.Structure):
     ]
 
 
+class BltHipKernelTime(C.Structure):
+    _fields_ = [("name", C.c_char * 48), ("launches", C.c_uint64), ("total_ms", C.c_double),
+                ("min_ms", C.c_double), ("max_ms", C.c_double)]
+
+
 # name -> (restype, argtypes); every symbol include/blt_hip.h declares
 SYMBOLS = {
     "blt_attention_head_core_hip": (None, [C.c_int, C.POINTER(abi.BltAttentionHeadArgs)]),
@@ -96,6 +101,8 @@ SYMBOLS = {
     "blt_kv_attend_step_hip": (None, [C.POINTER(BltKvAttnCache), C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t,
                                       C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t, C.c_int, C.c_int,
                                       C.c_size_t]),
+    "blt_hip_profile_begin": (None, []),
+    "blt_hip_profile_end": (C.c_size_t, [C.POINTER(BltHipKernelTime), C.c_size_t]),
     "blt_hip_build_info": (C.c_char_p, []),
 }
 
@@ -152,3 +159,11 @@ def problem_array(problems):
     for i, p in enumerate(problems):
         arr[i] = p
     return arr
+
+
+def profile_end():
+    """Close the open profile: {kernel tag: (launches, total_ms, min_ms, max_ms)}."""
+    rows = (BltHipKernelTime * 16)()
+    n = load().blt_hip_profile_end(rows, 16)
+    return {rows[i].name.decode(): (int(rows[i].launches), rows[i].total_ms, rows[i].min_ms, rows[i].max_ms)
+            for i in range(min(n, 16))}

@@ -24,6 +24,7 @@
 #include "blt_fatal.h"
 #include "hip_check.h"
 #include "attn_device.h"
+#include "launch.h"
 
 #include <algorithm>
 
@@ -250,7 +251,7 @@ template <int G, int NQ>
 void launch_step(const StepArgs &a, uint32_t batch, hipStream_t s) {
     const uint32_t hpb = std::min<uint32_t>(a.num_heads, 4u);
     dim3 grid(a.chunks, batch, (a.num_heads + hpb - 1) / hpb);
-    hipLaunchKernelGGL((kv_step_kernel<G, NQ>), grid, dim3(64 * hpb), 0, s, a);
+    blt_launch("kv_step", kv_step_kernel<G, NQ>, grid, dim3(64 * hpb), 0, s, a);
 }
 
 template <int G>

@@ -36,6 +36,7 @@
 #include "attn_device.h"
 #include "attn_launch.h"
 #include "hip_check.h"
+#include "launch.h"
 
 #include <algorithm>
 
@@ -297,11 +298,11 @@ template <int HD>
 void launch_mfma(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t ntiles, const AttnProb *single,
                  hipStream_t s) {
     if (single) {
-        hipLaunchKernelGGL((attn_mfma_kernel<HD, true>), dim3(ntiles), dim3(256), 0, s, dprobs, dtiles, *single);
+        blt_launch("attn_mfma", attn_mfma_kernel<HD, true>, dim3(ntiles), dim3(256), 0, s, dprobs, dtiles, *single);
     } else {
         AttnProb none;
         __builtin_memset(&none, 0, sizeof(none));
-        hipLaunchKernelGGL((attn_mfma_kernel<HD, false>), dim3(ntiles), dim3(256), 0, s, dprobs, dtiles, none);
+        blt_launch("attn_mfma", attn_mfma_kernel<HD, false>, dim3(ntiles), dim3(256), 0, s, dprobs, dtiles, none);
     }
 }
 

@@ -13,6 +13,7 @@
  */
 #include "attn_device.h"
 #include "attn_launch.h"
+#include "launch.h"
 
 namespace {
 
@@ -165,11 +166,11 @@ void launch_rows(const AttnProb *dprobs, uint32_t base, uint32_t count, uint32_t
     constexpr int ROWS_PER_BLOCK = 4 * (64 / G);
     dim3 grid((max_nq + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK, count, 1);
     if (single) {
-        hipLaunchKernelGGL((attn_rows_kernel<G, T, true>), grid, dim3(256), 0, s, dprobs, base, *single);
+        blt_launch("attn_rows", attn_rows_kernel<G, T, true>, grid, dim3(256), 0, s, dprobs, base, *single);
     } else {
         AttnProb none;
         __builtin_memset(&none, 0, sizeof(none));
-        hipLaunchKernelGGL((attn_rows_kernel<G, T, false>), grid, dim3(256), 0, s, dprobs, base, none);
+        blt_launch("attn_rows", attn_rows_kernel<G, T, false>, grid, dim3(256), 0, s, dprobs, base, none);
     }
 }
 

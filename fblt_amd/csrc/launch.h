@@ -1,0 +1,31 @@
+/*
+ * Kernel launches of the library go through blt_launch(): a plain
+ * hipLaunchKernelGGL normally; while a profile is open, the same launch with
+ * a start and a stop event attached to the dispatch, so that the kernel's own
+ * begin/end timestamps can be read back per launch and summed per kernel tag.
+ */
+#ifndef FBLT_AMD_LAUNCH_H
+#define FBLT_AMD_LAUNCH_H
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
+
+#include "hip_check.h"
+
+bool blt_profile_is_open();
+/* A fresh (start, stop) event pair owned by the open profile, booked under `tag`. */
+void blt_profile_book(const char *tag, hipEvent_t *start, hipEvent_t *stop);
+
+template <typename Kernel, typename... Args>
+inline void blt_launch(const char *tag, Kernel kernel, dim3 grid, dim3 block, size_t lds_bytes, hipStream_t stream,
+                       Args... args) {
+    if (blt_profile_is_open()) {
+        hipEvent_t e0, e1;
+        blt_profile_book(tag, &e0, &e1);
+        hipExtLaunchKernelGGL(kernel, grid, block, (unsigned)lds_bytes, stream, e0, e1, 0, args...);
+    } else {
+        hipLaunchKernelGGL(kernel, grid, block, (unsigned)lds_bytes, stream, args...);
+    }
+}
+
+#endif

@@ -193,6 +193,20 @@ void blt_kv_attend_step_hip(const blt_kv_attn_cache *cache, const float *q_rows,
                             float *combined, size_t combined_stride, size_t n, int step_kind, int commit,
                             size_t max_len_hint);
 
+/* Per-kernel device time of every launch the library issues between begin and
+ * end, from HIP events attached to each dispatch (the kernel's own begin/end
+ * timestamps, without launch gaps).  `end` synchronises the device, fills up to
+ * `capacity` rows (one per kernel tag) and returns the number of tags seen. */
+typedef struct {
+    char name[48];
+    uint64_t launches;
+    double total_ms;
+    double min_ms;
+    double max_ms;
+} blt_hip_kernel_time;
+void blt_hip_profile_begin(void);
+size_t blt_hip_profile_end(blt_hip_kernel_time *out, size_t capacity);
+
 /* Library build tag and the architecture its kernels were compiled for. */
 const char *blt_hip_build_info(void);
 

@@ -1,0 +1,170 @@
+"""CPU-only checks of the shipped library: it loads, exports every symbol the
+public header declares, its host-side integer code agrees with the checker,
+and it fails loudly (never falls back) when asked for CPU compute."""
+import ctypes as C
+import os
+import re
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from fblt_amd import abi, api
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "blt_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = re.findall(r"\b(blt_[a-z0-9_]+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = C.CDLL(api.LIB_PATH)
+    names = declared_functions()
+    assert len(names) >= 35
+    for n in names:
+        assert hasattr(lib, n), "include/blt_hip.h declares %s but the library does not export it" % n
+    assert set(names) == set(api.SYMBOLS), set(names) ^ set(api.SYMBOLS)
+    assert b"gfx950" in api.load().blt_hip_build_info()
+
+
+def test_header_layout_assertions_compile():
+    """include/blt_abi.h carries its own static assertions; compile it as C99 and C++17."""
+    for cc, std, lang in (("gcc", "-std=c99", "c"), ("g++", "-std=c++17", "c++")):
+        src = '#include "blt_abi.h"\n#include "blt_hip.h"\nint main(void){return 0;}\n'
+        p = subprocess.run([cc, std, "-x", lang, "-fsyntax-only", "-I", os.path.join(ROOT, "include"), "-"],
+                           input=src, text=True, capture_output=True)
+        assert p.returncode == 0, p.stderr
+
+
+def test_patch_helpers_match_checker(oracle):
+    lib = api.load()
+    rs = np.random.RandomState(21)
+    for _ in range(80):
+        P = rs.randint(1, 14)
+        lens = rs.randint(1, 17, size=P)
+        starts = np.concatenate(([0], np.cumsum(lens)[:-1]))
+        if rs.randint(4) == 0:
+            starts = starts + rs.randint(1, 5)
+        p = abi.patch_array(starts, lens)
+        T = int(starts[-1] + lens[-1])
+        for pos in range(T + 4):
+            assert lib.blt_patch_decoder_latent_at(p, P, pos) == oracle.orc_patch_decoder_latent_at(p, P, pos)
+        if starts[0] == 0:
+            q1, k1, q2, k2 = (abi.size_array([7] * max(P, T)) for _ in range(4))
+            lib.blt_patch_build_group_ids(p, P, T, q1, k1)
+            assert oracle.orc_patch_build_group_ids(p, P, T, q2, k2) == 0
+            assert list(q1)[:P] == list(q2)[:P] and list(k1)[:T] == list(k2)[:T]
+            k = rs.randint(1, 4)
+            e1, e2 = abi.size_array([0] * (T * k)), abi.size_array([0] * (T * k))
+            lib.blt_patch_expand_group_ids(k1, T, k, e1)
+            oracle.orc_patch_expand_group_ids(k2, T, k, e2)
+            assert list(e1) == list(e2)
+    # the reference's vectors (tests/unit/models/unit_local_decoder.c:94-113)
+    p = abi.patch_array([0, 3, 7, 8, 15], [3, 4, 1, 7, 1])
+    assert [lib.blt_patch_decoder_latent_at(p, 5, i) for i in range(16)] == [0, 0, 0, 0, 0, 0, 1, 2, 2, 2, 2, 2, 2,
+                                                                            2, 3, 3]
+    assert lib.blt_patch_decoder_latent_at(p, 5, 100) == 4
+
+
+def test_row_ranges_describe_the_dense_mask(oracle):
+    from oracle import binding
+    lib = api.load()
+    rs = np.random.RandomState(22)
+    claimed = 0
+    for trial in range(300):
+        nq, nk = rs.randint(1, 30), rs.randint(1, 30)
+        cfg = abi.BltMaskConfig()
+        cfg.seq_len_q, cfg.seq_len_kv = nq, nk
+        cfg.is_causal = bool(rs.randint(2))
+        cfg.sliding_window = int(rs.choice([0, 0, 1, 4]))
+        cfg.causal_offset = int(rs.choice([0, 0, 2, 11]))
+        keep = []
+        if rs.randint(2):
+            b = abi.size_array(sorted(rs.randint(0, 32, size=rs.randint(1, 4)).tolist()))
+            keep.append(b)
+            cfg.doc_boundaries, cfg.num_docs = b, len(b) + 1
+        sorted_groups = True
+        if rs.randint(2):
+            sorted_groups = bool(rs.randint(2))
+            qa = abi.size_array(rs.randint(0, 4, nq))
+            ka = abi.size_array(np.sort(rs.randint(0, 4, nk)) if sorted_groups else rs.randint(0, 4, nk))
+            keep += [qa, ka]
+            cfg.query_group_ids, cfg.kv_group_ids = qa, ka
+            cfg.bidirectional_within_group = bool(rs.randint(2))
+        dense = np.empty(nq * nk, dtype=np.float32)
+        rc = oracle.orc_build_attention_mask(C.byref(cfg), binding.fptr(dense))
+        lo, hi = (C.c_uint32 * nq)(), (C.c_uint32 * nq)()
+        ok = lib.blt_mask_config_row_ranges(C.byref(cfg), lo, hi)
+        if sorted_groups:
+            assert ok == 1
+        if not ok:
+            continue
+        claimed += 1
+        allowed = dense.reshape(nq, nk) == 0
+        for i in range(nq):
+            row = np.zeros(nk, dtype=bool)
+            row[lo[i]:hi[i]] = True
+            if rc == 4 and not allowed[i].any():
+                assert lo[i] == hi[i]
+                break          # the dense builder stops at the first dead row
+            assert (row == allowed[i]).all(), (trial, i)
+    assert claimed > 150
+
+
+def test_host_arena_and_tensor():
+    lib = api.load()
+    arena = lib.blt_arena_create(4096, abi.BLT_BACKEND_CPU)
+    assert arena.contents.capacity == 4096 and arena.contents.offset == 0
+    p1 = lib.blt_arena_alloc(arena, 10, 1)
+    p2 = lib.blt_arena_alloc(arena, 4, 64)
+    assert p2 % 64 == 0 and p2 > p1 and arena.contents.offset == (p2 - arena.contents.buffer) + 4
+    shape = (C.c_size_t * 2)(3, 5)
+    t = lib.blt_tensor_create(arena, shape, 2, abi.BLT_DTYPE_FP32)
+    assert t.numel == 15 and t.strides[0] == 5 and t.strides[1] == 1 and t.data % 64 == 0
+    assert t.backend == abi.BLT_BACKEND_CPU and not t.is_view
+    vals = np.arange(15, dtype=np.float32)
+    lib.blt_tensor_upload(C.byref(t), vals.ctypes.data, vals.nbytes)
+    back = np.zeros(15, dtype=np.float32)
+    lib.blt_tensor_download(C.byref(t), back.ctypes.data, back.nbytes)
+    assert (back == vals).all()
+    lib.blt_arena_reset(arena)
+    assert arena.contents.offset == 0
+    lib.blt_arena_destroy(arena)
+
+
+FATAL_SNIPPETS = {
+    "cpu_backend_attention": """
+a = abi.BltAttentionHeadArgs()
+lib.blt_attention_head_core(abi.BLT_BACKEND_CPU, C.byref(a))
+""",
+    "cpu_arena_mask": """
+arena = lib.blt_arena_create(1 << 16, abi.BLT_BACKEND_CPU)
+cfg = abi.BltMaskConfig(); cfg.seq_len_q = cfg.seq_len_kv = 4
+t = abi.BltTensor()
+lib.blt_build_attention_mask(C.byref(cfg), C.byref(t), arena)
+""",
+    "arena_overflow": """
+arena = lib.blt_arena_create(64, abi.BLT_BACKEND_CPU)
+lib.blt_arena_alloc(arena, 65, 1)
+""",
+    "bad_patch_tiling": """
+p = abi.patch_array([0, 4], [3, 2])
+q, k = abi.size_array([0] * 8), abi.size_array([0] * 8)
+lib.blt_patch_build_group_ids(p, 2, 6, q, k)
+""",
+}
+
+
+@pytest.mark.parametrize("name", list(FATAL_SNIPPETS))
+def test_fatal_errors_exit_like_the_reference(name):
+    """csrc/core/backend.h:13-31: message on stderr, exit(EXIT_FAILURE); never a silent fallback."""
+    code = "import ctypes as C, sys\nsys.path.insert(0, %r)\nfrom fblt_amd import abi, api\nlib = api.load()\n" % ROOT
+    code += FATAL_SNIPPETS[name] + "\nprint('SURVIVED')\n"
+    p = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert p.returncode == 1, (p.returncode, p.stdout, p.stderr)
+    assert "BLT Fatal Error [" in p.stderr and "SURVIVED" not in p.stdout

@@ -1,0 +1,307 @@
+"""Pins the CPU checker WITHOUT the reference build: reference-held vectors,
+closed forms, float64 brute force and structural invariants, each chosen so
+that a plausible slip (dropped scale, wrong sign, transposed operand, off-by-one
+in a mask) fails at least one of them."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from fblt_amd import abi
+from oracle import binding
+
+
+def core(orc, q, k, v, scale, mask=None, causal=False, hd=None, nq=None, nk=None):
+    nq = nq or q.shape[0]
+    nk = nk or k.shape[0]
+    hd = hd or q.shape[1]
+    out = np.full((nq, hd), 3.0, dtype=np.float32)
+    w = np.full((nq, nk), 3.0, dtype=np.float32)
+    a = binding.head_args(q.reshape(-1), k.reshape(-1), v.reshape(-1), out.reshape(-1), nq, nk, hd, scale,
+                          q.shape[1], k.shape[1], v.shape[1], hd, 0, weights=w.reshape(-1),
+                          mask=None if mask is None else mask.reshape(-1), causal=causal)
+    assert orc.orc_attention_head_core(C.byref(a)) == 0
+    return out, w
+
+
+def test_reference_inline_vector(oracle):
+    # tests/unit/models/unit_attention.c:24-88 (identity projections => Q=K=V=input slices)
+    x = np.array([[1, 0], [0, 1]], dtype=np.float32)
+    scale = float(np.float32(1.0) / np.sqrt(np.float32(2.0)))
+    out, w = core(oracle, x, x, x, scale)
+    assert np.allclose(out, [[0.6697615, 0.3302385], [0.3302385, 0.6697615]], atol=1e-7)
+    # causal variants, unit_attention.c:160-184: row 0 is one-hot; mask form == flag form
+    out_c, w_c = core(oracle, x, x, x, scale, causal=True)
+    assert np.allclose(out_c, [[1, 0], [0.3302385, 0.6697615]], atol=1e-7)
+    m = np.array([[0, -np.inf], [0, 0]], dtype=np.float32)
+    out_m, w_m = core(oracle, x, x, x, scale, mask=m)
+    assert np.array_equal(out_m, out_c) and np.array_equal(w_m, w_c)
+
+
+def test_two_key_softmax_is_a_sigmoid(oracle):
+    rs = np.random.RandomState(0)
+    for _ in range(50):
+        hd = rs.randint(1, 40)
+        q = rs.randn(1, hd).astype(np.float32)
+        k = rs.randn(2, hd).astype(np.float32)
+        v = np.array([[1.0], [0.0]], dtype=np.float32)
+        vv = np.zeros((2, hd), dtype=np.float32)
+        vv[:, :1] = v
+        scale = float(rs.rand() + 0.1)
+        out, w = core(oracle, q, k, vv, scale)
+        d = (q.astype(np.float64) @ (k[0] - k[1]).astype(np.float64))[0] * scale
+        sig = 1.0 / (1.0 + np.exp(-d))
+        assert abs(w[0, 0] - sig) < 2e-6 and abs(out[0, 0] - sig) < 2e-6   # wrong sign => 1 - sig
+        assert abs(w.sum() - 1) < 1e-6
+
+
+def test_uniform_and_single_key_and_dead_rows(oracle):
+    rs = np.random.RandomState(1)
+    nq, nk, hd = 6, 9, 5
+    k = rs.randn(nk, hd).astype(np.float32)
+    v = rs.randn(nk, hd).astype(np.float32)
+    zero_q = np.zeros((nq, hd), dtype=np.float32)
+    out, w = core(oracle, zero_q, k, v, 0.7, causal=True)
+    for i in range(nq):  # equal scores: mean of the visible V rows, keys j <= i only
+        assert np.allclose(out[i], v[:i + 1].astype(np.float64).mean(0), atol=1e-6)
+        assert np.allclose(w[i, :i + 1], 1.0 / (i + 1), atol=1e-7) and (w[i, i + 1:] == 0).all()
+    q = rs.randn(nq, hd).astype(np.float32)
+    mask = np.full((nq, nk), -np.inf, dtype=np.float32)
+    for i in range(nq - 1):
+        mask[i, (3 * i) % nk] = 0.0           # exactly one visible key
+    out, w = core(oracle, q, k, v, 0.3, mask=mask)
+    for i in range(nq - 1):
+        assert np.array_equal(out[i], v[(3 * i) % nk])      # weight exactly 1.0 => exact copy
+    assert (out[nq - 1] == 0).all() and (w[nq - 1] == 0).all()   # all-masked row: zeros
+
+
+def test_float64_brute_force(oracle):
+    rs = np.random.RandomState(2)
+    for trial in range(30):
+        nq, nk, hd = rs.randint(1, 9), rs.randint(1, 12), rs.randint(1, 10)
+        qs, ks, vs = hd + rs.randint(0, 3), hd + rs.randint(0, 3), hd + rs.randint(0, 3)
+        q = rs.randn(nq, qs).astype(np.float32)
+        k = rs.randn(nk, ks).astype(np.float32)
+        v = rs.randn(nk, vs).astype(np.float32)
+        scale = float(rs.rand() * 2)
+        mask = np.where(rs.rand(nq, nk) < 0.3, -np.inf, rs.randn(nq, nk)).astype(np.float32)
+        out, w = core(oracle, q, k, v, scale, mask=mask, hd=hd)
+        s = q[:, :hd].astype(np.float64) @ k[:, :hd].astype(np.float64).T * scale + mask
+        for i in range(nq):
+            fin = np.isfinite(s[i])
+            ref = np.zeros(nk)
+            if fin.any():
+                e = np.exp(s[i, fin] - s[i, fin].max())
+                ref[fin] = e / e.sum()
+            assert np.allclose(w[i], ref, atol=2e-6)
+            assert np.allclose(out[i], ref @ v[:, :hd].astype(np.float64), atol=5e-6)
+
+
+def test_nonfinite_scores_are_dropped(oracle):
+    # csrc/ops/vecmath_cpu.c:33-46: only finite entries enter the max and the sum
+    q = np.array([[1.0, 0.0]], dtype=np.float32)
+    k = np.array([[np.inf, 0.0], [1.0, 0.0], [2.0, 0.0]], dtype=np.float32)
+    v = np.eye(3, 2, dtype=np.float32)
+    out, w = core(oracle, q, k, v, 1.0)
+    assert w[0, 0] == 0.0 and abs(w[0, 1] + w[0, 2] - 1) < 1e-6 and w[0, 2] > w[0, 1]
+
+
+def mask_of(orc, **kw):
+    cfg = abi.BltMaskConfig()
+    keep = []
+    for name, val in kw.items():
+        if name in ("doc_boundaries", "query_group_ids", "kv_group_ids"):
+            arr = abi.size_array(val)
+            keep.append(arr)
+            setattr(cfg, name, arr)
+        else:
+            setattr(cfg, name, val)
+    out = np.empty(cfg.seq_len_q * cfg.seq_len_kv, dtype=np.float32)
+    rc = orc.orc_build_attention_mask(C.byref(cfg), binding.fptr(out))
+    return rc, out.reshape(cfg.seq_len_q, cfg.seq_len_kv) == 0.0, out
+
+
+def test_mask_builder_reference_cases(oracle):
+    # tests/unit/backend/unit_mask.c:14-192
+    rc, ok, raw = mask_of(oracle, seq_len_q=4, seq_len_kv=4, is_causal=True)
+    assert rc == 0 and (ok == np.tril(np.ones((4, 4), bool))).all()
+    assert set(np.unique(raw)) == {0.0, -np.inf}
+    rc, ok, _ = mask_of(oracle, seq_len_q=6, seq_len_kv=6, is_causal=True, sliding_window=3)
+    assert list(ok[5]) == [False, False, False, True, True, True]
+    rc, ok, _ = mask_of(oracle, seq_len_q=6, seq_len_kv=6, doc_boundaries=[3], num_docs=2)
+    assert ok[1, 2] and ok[4, 5] and not ok[2, 3] and not ok[5, 0]
+    rc, ok, _ = mask_of(oracle, seq_len_q=4, seq_len_kv=4, query_group_ids=[0, 0, 1, 1], kv_group_ids=[0, 0, 1, 1])
+    assert not ok[0, 2] and not ok[3, 1] and ok[1, 0] and not ok[0, 1]
+    # a row without any key is the reference's abort (mask_builder_cpu.c:93)
+    rc, _, _ = mask_of(oracle, seq_len_q=2, seq_len_kv=2, query_group_ids=[0, 5], kv_group_ids=[0, 0],
+                       bidirectional_within_group=True)
+    assert rc == 4
+
+
+def test_mask_builder_randomised_predicate(oracle):
+    # independent statement of the rule (tests/unit/models/unit_global_transformer.c:121+ style fuzz)
+    rs = np.random.RandomState(3)
+    for _ in range(60):
+        nq, nk = rs.randint(1, 20), rs.randint(1, 20)
+        causal, W, off = bool(rs.randint(2)), int(rs.choice([0, 0, 1, 3, 7])), int(rs.choice([0, 0, 2, 5]))
+        bounds = sorted(rs.randint(0, max(nq, nk) + 1, size=rs.randint(0, 4)).tolist())
+        use_g, bidir = bool(rs.randint(2)), bool(rs.randint(2))
+        qg, kg = rs.randint(0, 3, nq).tolist(), rs.randint(0, 3, nk).tolist()
+        kw = dict(seq_len_q=nq, seq_len_kv=nk, is_causal=causal, sliding_window=W, causal_offset=off)
+        if bounds:
+            kw.update(doc_boundaries=bounds, num_docs=len(bounds) + 1)
+        if use_g:
+            kw.update(query_group_ids=qg, kv_group_ids=kg, bidirectional_within_group=bidir)
+        rc, ok, _ = mask_of(oracle, **kw)
+        doc = lambda p: sum(1 for b in bounds if p >= b)
+        dead = False
+        for i in range(nq):
+            row_any = False
+            for j in range(nk):
+                want = True
+                if causal and j > i + off:
+                    want = False
+                if W > 0 and abs((i + off if causal else i) - j) >= W:
+                    want = False
+                if bounds and doc(i) != doc(j):
+                    want = False
+                if use_g and (qg[i] != kg[j] or (not bidir and j > i)):
+                    want = False
+                assert ok[i, j] == want, (kw, i, j)
+                row_any |= want
+            if not row_any:
+                dead = True
+                break          # rows after the first dead one are unspecified
+        assert (rc == 4) == dead
+
+
+def test_block_diffusion_fixture(oracle):
+    # tests/unit/models/unit_block_diffusion.c:115-172
+    want = ["10000000000000", "11000000000000", "11100000000000", "11110000000000", "11111000000000",
+            "11111100000000", "11000011110000", "11000011110000", "11000011110000", "11000011110000",
+            "11110000001111", "11110000001111", "11110000001111", "11110000001111"]
+    cfg = abi.BltBlockDiffusionConfig()
+    starts = abi.size_array([2, 4])
+    cfg.mode, cfg.seq_len, cfg.num_clean, cfg.block_size = abi.BLT_BDM_TRAIN, 14, 6, 4
+    cfg.block_starts, cfg.num_blocks = starts, 2
+    out = np.empty(14 * 14, dtype=np.float32)
+    assert oracle.orc_build_block_diffusion_mask(C.byref(cfg), binding.fptr(out)) == 0
+    got = ["".join("1" if x == 0 else "0" for x in row) for row in out.reshape(14, 14)]
+    assert got == want
+    assert np.isneginf(out[out != 0]).all()
+    cfg = abi.BltBlockDiffusionConfig()
+    cfg.mode, cfg.seq_len, cfg.num_clean = abi.BLT_BDM_INFER, 7, 3
+    out = np.empty(49, dtype=np.float32)
+    assert oracle.orc_build_block_diffusion_mask(C.byref(cfg), binding.fptr(out)) == 0
+    ok = out.reshape(7, 7) == 0
+    for i in range(7):
+        for j in range(7):
+            assert ok[i, j] == ((j <= i) if i < 3 else True)
+    # bad configurations are the reference's aborts (mask_builder_cpu.c:103-119)
+    cfg.num_clean = 0
+    assert oracle.orc_build_block_diffusion_mask(C.byref(cfg), binding.fptr(out)) == 5
+
+
+def test_block_diffusion_no_leak(oracle):
+    # tests/unit/models/unit_block_diffusion.c:186-238
+    N, B, starts = 9, 3, [1, 3, 5, 8]
+    S = N + B * len(starts)
+    cfg = abi.BltBlockDiffusionConfig()
+    arr = abi.size_array(starts)
+    cfg.mode, cfg.seq_len, cfg.num_clean, cfg.block_size = abi.BLT_BDM_TRAIN, S, N, B
+    cfg.block_starts, cfg.num_blocks = arr, len(starts)
+    out = np.empty(S * S, dtype=np.float32)
+    assert oracle.orc_build_block_diffusion_mask(C.byref(cfg), binding.fptr(out)) == 0
+    ok = out.reshape(S, S) == 0
+    for i in range(S):
+        for j in range(S):
+            if i < N:
+                assert ok[i, j] == (j < N and j <= i)
+            else:
+                blk = (i - N) // B
+                own = j >= N and (j - N) // B == blk
+                assert ok[i, j] == (j < starts[blk] or own)
+
+
+def test_patch_index_reference_vectors(oracle):
+    # tests/unit/models/unit_local_decoder.c:94-113
+    p = abi.patch_array([0, 3, 7, 8, 15], [3, 4, 1, 7, 1])
+    got = [oracle.orc_patch_decoder_latent_at(p, 5, pos) for pos in range(16)]
+    assert got == [0, 0, 0, 0, 0, 0, 1, 2, 2, 2, 2, 2, 2, 2, 3, 3]
+    assert oracle.orc_patch_decoder_latent_at(p, 5, 16) == 4 and oracle.orc_patch_decoder_latent_at(p, 5, 100) == 4
+    # tests/unit/backend/unit_mask.c:116-127
+    src, dst = abi.size_array([0, 1]), abi.size_array([9] * 6)
+    oracle.orc_patch_expand_group_ids(src, 2, 3, dst)
+    assert list(dst) == [0, 0, 0, 1, 1, 1]
+    # group ids: patch p is query group p, its bytes carry p; bad tilings are rejected
+    q, kv = abi.size_array([9] * 5), abi.size_array([9] * 16)
+    assert oracle.orc_patch_build_group_ids(p, 5, 16, q, kv) == 0
+    assert list(q) == [0, 1, 2, 3, 4]
+    assert list(kv) == [0] * 3 + [1] * 4 + [2] + [3] * 7 + [4]
+    assert oracle.orc_patch_build_group_ids(p, 5, 17, q, kv) == 6
+    gap = abi.patch_array([0, 4], [3, 2])
+    assert oracle.orc_patch_build_group_ids(gap, 2, 6, q, kv) == 6
+    # one-hot cross mask rows (unit_local_decoder.c:34-87)
+    rc, ok, _ = mask_of(oracle, seq_len_q=16, seq_len_kv=5, query_group_ids=list(kv), kv_group_ids=list(q),
+                        bidirectional_within_group=True)
+    assert rc == 0 and (ok.sum(1) == 1).all() and (ok.argmax(1) == np.array(list(kv))).all()
+
+
+def test_kv_slab_indexing(oracle):
+    # [batch*max_seq_len, E] row-major, row == absolute position (kv_cache.c:56-60, kv_cache.h:17-18)
+    assert oracle.orc_kv_row(0, 0, 768) == 0 and oracle.orc_kv_row(3, 5, 768) == 3 * 768 + 5
+    assert oracle.orc_kv_slot(2, 7, 3, 9, 768, 128, 32) == ((2 * 768 + 7) * 128 + 3 * 32 + 9)
+    m = np.empty(3 * 8, dtype=np.float32)
+    oracle.orc_kv_self_mask(binding.fptr(m), 3, 5, 0)
+    ok = m.reshape(3, 8) == 0
+    for r in range(3):
+        assert list(ok[r]) == [j <= 5 + r for j in range(8)]
+    oracle.orc_kv_self_mask(binding.fptr(m), 3, 5, 4)
+    ok = m.reshape(3, 8) == 0
+    for r in range(3):
+        assert list(ok[r]) == [j <= 5 + r and 5 + r - j < 4 for j in range(8)]
+
+
+@pytest.mark.parametrize("chunks", [[1] * 12, [5, 1, 1, 5], [12], [3, 4, 5]])
+@pytest.mark.parametrize("window", [0, 5])
+def test_kv_cached_equals_dense(chunks, window, oracle):
+    """The reference's invariant (tests/unit/infer/unit_kv_cache.c:136-151): stepping through the
+    cache in any chunking gives bit-identical rows to one dense causal pass."""
+    rs = np.random.RandomState(11)
+    T, H, hd = sum(chunks), 2, 6
+    E = H * hd
+    q, k, v = (rs.randn(T, E).astype(np.float32) for _ in range(3))
+    # dense: one causal(+window) pass over all T rows
+    cfg = abi.BltMaskConfig()
+    cfg.seq_len_q = cfg.seq_len_kv = T
+    cfg.is_causal, cfg.sliding_window = True, window
+    mask = np.empty(T * T, dtype=np.float32)
+    assert oracle.orc_build_attention_mask(C.byref(cfg), binding.fptr(mask)) == 0
+    dense = np.zeros((T, E), dtype=np.float32)
+    scratch = np.empty(T * T, dtype=np.float32)
+    for h in range(H):
+        a = binding.head_args(q.reshape(-1), k.reshape(-1), v.reshape(-1), dense.reshape(-1), T, T, hd,
+                              float(np.float32(1) / np.sqrt(np.float32(hd))), E, E, E, E, h * hd, q_off=h * hd,
+                              k_off=h * hd, v_off=h * hd, scratch=scratch, mask=mask)
+        assert oracle.orc_attention_head_core(C.byref(a)) == 0
+    # cached: sequence 1 of a 2-sequence slab, chunk by chunk
+    max_len = T + 3
+    ck = np.full((2 * max_len, E), 99.0, dtype=np.float32)
+    cv = np.full((2 * max_len, E), 99.0, dtype=np.float32)
+    got = np.zeros((T, E), dtype=np.float32)
+    base = 0
+    for n in chunks:
+        rows = slice(base, base + n)
+        comb = np.zeros((n, E), dtype=np.float32)
+        rc = oracle.orc_kv_attend_step(binding.fptr(ck.reshape(-1)), binding.fptr(cv.reshape(-1)), max_len, E, H, 1,
+                                       base, n, window, binding.fptr(np.ascontiguousarray(q[rows])),
+                                       binding.fptr(np.ascontiguousarray(k[rows])),
+                                       binding.fptr(np.ascontiguousarray(v[rows])), binding.fptr(comb.reshape(-1)))
+        assert rc == 0
+        got[rows] = comb
+        base += n
+    assert got.tobytes() == dense.tobytes()
+    assert (ck[:max_len] == 99.0).all() and np.array_equal(ck[max_len:max_len + T], k)  # only slab 1 rows touched
+    assert oracle.orc_kv_attend_step(binding.fptr(ck.reshape(-1)), binding.fptr(cv.reshape(-1)), max_len, E, H, 1,
+                                     T, 4, 0, binding.fptr(q), binding.fptr(k), binding.fptr(v),
+                                     binding.fptr(got.reshape(-1))) == 7   # over capacity

@@ -1,0 +1,191 @@
+"""Bit-for-bit comparison of the CPU checker with the reference's own CPU ops
+(oracle/_ref/libblt_ref.so, compiled from the reference's sources by
+`make -C oracle ref`).  Skipped on machines without that build; the committed
+fixtures under tests/golden/ carry the same evidence there."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from fblt_amd import abi
+from oracle import binding
+
+CPU = abi.BLT_BACKEND_CPU
+
+
+def _both_core(orc, ref, q, k, v, nq, nk, hd, scale, qs, ks, vs, mask, causal, use_weights):
+    res = []
+    for lib in (orc, ref):
+        out = np.full((nq, hd + 2), 4.0, dtype=np.float32)
+        w = np.full(nq * nk, 4.0, dtype=np.float32)
+        a = binding.head_args(q, k, v, out.reshape(-1), nq, nk, hd, scale, qs, ks, vs, hd + 2, 1,
+                              weights=w if use_weights else None, scratch=None if use_weights else w, mask=mask,
+                              causal=causal)
+        if lib is orc:
+            assert lib.orc_attention_head_core(C.byref(a)) == 0
+        else:
+            lib.blt_attention_head_core(CPU, C.byref(a))
+        res.append((out, w))
+    return res
+
+
+def test_attention_core_bit_exact(oracle, ref):
+    rs = np.random.RandomState(5)
+    for trial in range(120):
+        nq, nk, hd = rs.randint(1, 40), rs.randint(1, 60), int(rs.choice([1, 2, 7, 16, 32, 64]))
+        qs, ks, vs = hd + rs.randint(0, 5), hd + rs.randint(0, 5), hd + rs.randint(0, 5)
+        q = (rs.randn(nq * qs) * rs.choice([0.1, 1, 5])).astype(np.float32)
+        k = rs.randn(nk * ks).astype(np.float32)
+        v = rs.randn(nk * vs).astype(np.float32)
+        kind = trial % 4
+        mask, causal = None, False
+        if kind == 1:
+            causal = True
+        elif kind == 2:
+            mask = np.where(rs.rand(nq * nk) < 0.5, -np.inf, 0.0).astype(np.float32)
+        elif kind == 3:
+            mask = (rs.randn(nq * nk) * 3).astype(np.float32)
+            mask[rs.rand(nq * nk) < 0.1] = np.inf
+        scale = float(np.float32(1) / np.sqrt(np.float32(hd)))
+        (o1, w1), (o2, w2) = _both_core(oracle, ref, q, k, v, nq, nk, hd, scale, qs, ks, vs, mask, causal,
+                                        trial % 2 == 0)
+        assert o1.tobytes() == o2.tobytes(), trial
+        assert w1.tobytes() == w2.tobytes(), trial
+
+
+def test_softmax_dot_copy_bit_exact(oracle, ref):
+    rs = np.random.RandomState(6)
+    for trial in range(60):
+        n = rs.randint(1, 200)
+        row = (rs.randn(n) * 4).astype(np.float32)
+        if trial % 5 == 0:
+            row[rs.randint(n)] = np.inf
+        mask = np.where(rs.rand(n) < 0.4, -np.inf, 0).astype(np.float32) if trial % 3 == 0 else None
+        a, b = row.copy(), row.copy()
+        idx, causal, scale = rs.randint(n), trial % 2 == 1, float(rs.rand() + 0.05)
+        oracle.orc_softmax_masked_row_inplace(binding.fptr(a), n, idx, causal, binding.fptr(mask), scale)
+        ref.blt_softmax_masked_row_inplace(CPU, binding.fptr(b), n, idx, causal, binding.fptr(mask), scale)
+        assert a.tobytes() == b.tobytes()
+        x, y = rs.randn(n).astype(np.float32), rs.randn(n).astype(np.float32)
+        d1 = oracle.orc_vec_dot(binding.fptr(x), binding.fptr(y), n)
+        d2 = ref.blt_vec_dot(CPU, binding.fptr(x), binding.fptr(y), n)
+        assert np.float32(d1).tobytes() == np.float32(d2).tobytes()
+    src = rs.randn(7, 20).astype(np.float32)
+    d1, d2 = np.zeros((7, 11), np.float32), np.zeros((7, 11), np.float32)
+    oracle.orc_strided_copy(binding.fptr(d1.reshape(-1)), 11, binding.fptr(src.reshape(-1)), 20, 7, 9)
+    ref.blt_strided_copy(CPU, binding.fptr(d2.reshape(-1)), 11, binding.fptr(src.reshape(-1)), 20, 7, 9)
+    assert d1.tobytes() == d2.tobytes()
+
+
+def _ref_mask(ref, cfg, builder):
+    arena = ref.blt_arena_create(16 << 20, CPU)
+    t = abi.BltTensor()
+    getattr(ref, builder)(C.byref(cfg), C.byref(t), arena)
+    n = t.numel
+    out = np.ctypeslib.as_array(C.cast(t.data, C.POINTER(C.c_float)), shape=(n,)).copy()
+    ref.blt_arena_destroy(arena)
+    return out, tuple(t.shape[:2])
+
+
+def test_mask_builders_bit_exact(oracle, ref):
+    rs = np.random.RandomState(8)
+    done = 0
+    for trial in range(400):
+        nq, nk = rs.randint(1, 40), rs.randint(1, 40)
+        cfg = abi.BltMaskConfig()
+        cfg.seq_len_q, cfg.seq_len_kv = nq, nk
+        cfg.is_causal = bool(rs.randint(2))
+        cfg.sliding_window = int(rs.choice([0, 0, 2, 9]))
+        cfg.causal_offset = int(rs.choice([0, 0, 3, 17]))
+        keep = []
+        if rs.randint(2):
+            b = sorted(rs.randint(0, 45, size=rs.randint(1, 4)).tolist())
+            arr = abi.size_array(b)
+            keep.append(arr)
+            cfg.doc_boundaries, cfg.num_docs = arr, len(b) + 1
+        if rs.randint(2):
+            qa = abi.size_array(np.sort(rs.randint(0, 4, nq)) if rs.randint(2) else rs.randint(0, 3, nq))
+            ka = abi.size_array(np.sort(rs.randint(0, 4, nk)) if rs.randint(2) else rs.randint(0, 3, nk))
+            keep += [qa, ka]
+            cfg.query_group_ids, cfg.kv_group_ids = qa, ka
+            cfg.bidirectional_within_group = bool(rs.randint(2))
+        mine = np.empty(nq * nk, dtype=np.float32)
+        rc = oracle.orc_build_attention_mask(C.byref(cfg), binding.fptr(mine))
+        if rc != 0:
+            continue  # the reference would exit the process on this recipe
+        theirs, shape = _ref_mask(ref, cfg, "blt_build_attention_mask")
+        assert shape == (nq, nk) and mine.tobytes() == theirs.tobytes(), trial
+        done += 1
+    assert done > 100
+    for trial in range(40):
+        N, B, NB = rs.randint(1, 20), rs.randint(1, 5), rs.randint(0, 5)
+        cfg = abi.BltBlockDiffusionConfig()
+        train = trial % 2 == 0
+        starts = abi.size_array(rs.randint(0, N, size=max(NB, 1)))
+        cfg.mode = abi.BLT_BDM_TRAIN if train else abi.BLT_BDM_INFER
+        cfg.seq_len, cfg.num_clean, cfg.block_size = N + B * NB, N, B
+        cfg.block_starts, cfg.num_blocks = starts, NB
+        S = N + B * NB
+        mine = np.empty(S * S, dtype=np.float32)
+        assert oracle.orc_build_block_diffusion_mask(C.byref(cfg), binding.fptr(mine)) == 0
+        theirs, _ = _ref_mask(ref, cfg, "blt_build_block_diffusion_mask")
+        assert mine.tobytes() == theirs.tobytes()
+
+
+def test_patch_helpers_equal(oracle, ref):
+    rs = np.random.RandomState(9)
+    for _ in range(50):
+        P = rs.randint(1, 12)
+        lens = rs.randint(1, 9, size=P)
+        starts = np.concatenate(([0], np.cumsum(lens)[:-1]))
+        if rs.randint(3) == 0:
+            starts = starts + rs.randint(1, 4)  # uncovered head: latent rule still defined
+        p = abi.patch_array(starts, lens)
+        T = int(starts[-1] + lens[-1])
+        for pos in range(T + 3):
+            assert oracle.orc_patch_decoder_latent_at(p, P, pos) == ref.blt_patch_decoder_latent_at(p, P, pos)
+        if starts[0] == 0:
+            q1, k1, q2, k2 = (abi.size_array([0] * max(P, T)) for _ in range(4))
+            assert oracle.orc_patch_build_group_ids(p, P, T, q1, k1) == 0
+            ref.blt_patch_build_group_ids(p, P, T, q2, k2)
+            assert list(q1)[:P] == list(q2)[:P] and list(k1)[:T] == list(k2)[:T]
+
+
+def test_kv_step_against_reference_op_sequence(oracle, ref):
+    """orc_kv_attend_step against the reference's ops issued in the order of
+    csrc/infer/kv_cache.c:363-390 (strided copies into the slab, then one core
+    call per head with the dense step mask and a scratch score buffer)."""
+    rs = np.random.RandomState(10)
+    H, hd, max_len, batch = 4, 8, 40, 3
+    E = H * hd
+    ck1 = rs.randn(batch * max_len, E).astype(np.float32)
+    cv1 = rs.randn(batch * max_len, E).astype(np.float32)
+    ck2, cv2 = ck1.copy(), cv1.copy()
+    for b, base, n, window in [(0, 0, 1, 0), (1, 5, 1, 0), (2, 7, 6, 0), (1, 6, 3, 4), (0, 1, 30, 9)]:
+        q, k, v = (rs.randn(n, E).astype(np.float32) for _ in range(3))
+        mine = np.zeros((n, E), dtype=np.float32)
+        assert oracle.orc_kv_attend_step(binding.fptr(ck1.reshape(-1)), binding.fptr(cv1.reshape(-1)), max_len, E, H,
+                                         b, base, n, window, binding.fptr(q), binding.fptr(k), binding.fptr(v),
+                                         binding.fptr(mine.reshape(-1))) == 0
+        total = base + n
+        kd, vd = ck2.reshape(-1), cv2.reshape(-1)
+        slab = b * max_len * E
+        for h in range(H):
+            for dst, src in ((kd, k), (vd, v)):
+                ref.blt_strided_copy(CPU, C.cast(dst.ctypes.data + 4 * (slab + base * E + h * hd), C.POINTER(C.c_float)),
+                                     E, C.cast(src.ctypes.data + 4 * h * hd, C.POINTER(C.c_float)), E, n, hd)
+        mask = np.empty(n * total, dtype=np.float32)   # kv_cache.c:229-236, restated in numpy
+        for r in range(n):
+            p = base + r
+            for j in range(total):
+                ok = j <= p and not (window > 0 and p - j >= window)
+                mask[r * total + j] = 0.0 if ok else -np.inf
+        theirs = np.zeros((n, E), dtype=np.float32)
+        scratch = np.empty(n * total, dtype=np.float32)
+        for h in range(H):
+            a = binding.head_args(q.reshape(-1), kd, vd, theirs.reshape(-1), n, total, hd,
+                                  float(np.float32(1) / np.sqrt(np.float32(hd))), E, E, E, E, h * hd, q_off=h * hd,
+                                  k_off=slab + h * hd, v_off=slab + h * hd, scratch=scratch, mask=mask)
+            ref.blt_attention_head_core(CPU, C.byref(a))
+        assert mine.tobytes() == theirs.tobytes()
+        assert ck1.tobytes() == ck2.tobytes() and cv1.tobytes() == cv2.tobytes()
