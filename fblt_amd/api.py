@@ -116,6 +116,14 @@ def load():
         return _lib
     if not os.path.exists(LIB_PATH):
         raise RuntimeError("%s is missing: run `python -m fblt_amd.build` (there is no fallback path)" % LIB_PATH)
+    # One HIP runtime per process: PyTorch-ROCm ships its own libamdhip64 with the
+    # same SONAME the library needs.  Whoever is loaded first wins, and a process
+    # that ends up with two runtimes loses its device.  The Python callers here use
+    # torch for device memory, so let torch bring in its runtime first.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = C.CDLL(LIB_PATH)
     for name, (restype, argtypes) in SYMBOLS.items():
         fn = getattr(lib, name)  # AttributeError if the symbol is not exported
