@@ -5,20 +5,22 @@
  * new rows (reference order of operations: csrc/infer/kv_cache.c:343-390).
  *
  * Memory-bound split-KV design, no matrix cores:
- *   - a workgroup owns 32 consecutive cache rows (keys) of one sequence; its
- *     wavefronts are the heads, so together they read whole 4*E-byte rows;
+ *   - the keys of a sequence are cut into `splits` contiguous spans, one
+ *     workgroup each, so that batch x splits workgroups fill the chip;
+ *   - a workgroup has one wavefront per (head, slice): the waves of one slice
+ *     are the heads and read whole 4*E-byte cache rows between them, the
+ *     slices take the span's 32-key sub-chunks round-robin;
  *   - inside a wave, groups of G = head_dim/4 lanes own one key each per
  *     16-byte load: one load instruction of the wave covers 64/G consecutive
- *     keys, every byte of the fetched lines is used;
- *   - all K and V loads of the chunk are issued before any arithmetic, so a
- *     wave has its whole 32-key chunk in flight at once;
- *   - dot products are reduced across the G lanes with wavefront shuffles,
- *     the per-group partial softmax states (max, sum, output) are merged
- *     across the wave with shuffles too, and one partial per (sequence,
- *     chunk, head, query) goes to a scratch buffer;
- *   - the last workgroup of a sequence to finish (device-scope ticket) merges
- *     that sequence's partials, writes the output rows, and advances the
- *     sequence's length when the step commits.
+ *     keys and every byte of the fetched lines is used; the next sub-chunk is
+ *     requested before the current one is consumed;
+ *   - dot products are reduced across the G lanes with wavefront shuffles;
+ *     each lane group keeps an online-softmax state (max, sum, output) over
+ *     its keys, the groups of a wave merge with shuffles once at the end;
+ *   - slices merge through LDS; with more than one split the per-split
+ *     states go to a small scratch buffer and the last workgroup of the
+ *     sequence to finish (device-scope ticket) merges them, writes the output
+ *     rows and advances the sequence's length when the step commits.
  */
 #include "blt_hip.h"
 #include "blt_fatal.h"
@@ -27,11 +29,12 @@
 #include "launch.h"
 
 #include <algorithm>
+#include <cstdlib>
 
 namespace {
 
-/* keys per workgroup: 32, or one full load instruction of the wave if that is more */
-constexpr int chunk_keys(int G) { return 64 / G > 32 ? 64 / G : 32; }
+constexpr int SUB = 32;        /* keys per sub-chunk (one wave, one head)       */
+constexpr int MAX_SPLITS = 16; /* workgroups per sequence                        */
 
 struct StepArgs {
     float *cache_k;
@@ -41,14 +44,17 @@ struct StepArgs {
     const float *k_rows;
     const float *v_rows;
     float *combined;
-    float *partial;    /* [batch][chunks][heads][NQ][hd + 2] */
+    float *partial;    /* [batch][splits][heads][NQ][hd + 2] */
     uint32_t *tickets; /* [batch] */
     uint32_t q_stride, k_stride, v_stride, out_stride;
-    uint32_t max_seq_len, embed_dim, num_heads, head_dim;
+    uint32_t max_seq_len, embed_dim, num_heads;
     uint32_t window;
     uint32_t n;        /* new rows per sequence */
     uint32_t q0;       /* first query row this launch handles */
-    uint32_t chunks;   /* gridDim.x */
+    uint32_t splits;   /* gridDim.x */
+    uint32_t span;     /* keys per split, a multiple of SUB */
+    uint32_t hpb;      /* heads per workgroup */
+    uint32_t slices;   /* waves per head in a workgroup */
     float scale;
     int block_kind;    /* every new row sees all keys */
     int write_through; /* this launch stores the new rows into the cache */
@@ -64,49 +70,57 @@ __device__ __forceinline__ float group_sum(float x) {
 
 __device__ __forceinline__ float dot4(float4 a, float4 b) { return a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w; }
 
-/* merge softmax state (m2, l2, o2) into (m, l, o) */
-__device__ __forceinline__ void merge_state(float &m, float &l, float4 &o, float m2, float l2, float4 o2) {
-    const float mn = fmaxf(m, m2);
-    const float a = m == neg_inf() ? 0.f : softmax_exp(m - mn);
-    const float b = m2 == neg_inf() ? 0.f : softmax_exp(m2 - mn);
-    l = l * a + l2 * b;
-    o.x = o.x * a + o2.x * b;
-    o.y = o.y * a + o2.y * b;
-    o.z = o.z * a + o2.z * b;
-    o.w = o.w * a + o2.w * b;
-    m = mn;
+/* Device-scope store / load of data another workgroup (possibly on another
+ * die of the package) reads within the same launch. */
+__device__ __forceinline__ void publish(float *p, float x) {
+    __hip_atomic_store(p, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float observe(const float *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-/* G lanes per key (head_dim = 4*G), NQ query rows per sequence in this launch,
- * blockDim.x = 64 * heads-per-block, head = blockIdx.z * (blockDim.x/64) + wave. */
-template <int G, int NQ>
-__global__ __launch_bounds__(256) void kv_step_kernel(StepArgs a) {
-    constexpr int KPL = 64 / G;          /* keys per load instruction of a wave */
-    constexpr int CHUNK = chunk_keys(G);
-    constexpr int LOADS = CHUNK / KPL;   /* loads per lane for K (and for V)   */
+/* G lanes per key (head_dim = 4*G), NQ query rows per launch, at most WAVES
+ * waves per workgroup. */
+template <int G, int NQ, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void kv_step_kernel(StepArgs a) {
+    constexpr int KPL = 64 / G;                    /* keys per load instruction of a wave */
+    /* loads per lane and sub-chunk: at most four 16-byte loads each for K and V */
+    constexpr int LOADS = SUB / KPL < 1 ? 1 : (SUB / KPL > 4 ? 4 : SUB / KPL);
+    constexpr int STEP = LOADS * KPL;              /* keys a wave consumes per sub-chunk  */
     constexpr int HD = 4 * G;
-    constexpr int DPL = (HD + 63) / 64;  /* output columns per lane in the final merge */
 
+    extern __shared__ float sm[];                  /* [waves][NQ][HD + 2] */
     __shared__ uint32_t sm_ticket;
 
     const uint32_t b = blockIdx.y;
-    const uint32_t chunk = blockIdx.x;
+    const uint32_t split = blockIdx.x;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
-    const uint32_t head = blockIdx.z * (blockDim.x >> 6) + wave;
+    const uint32_t slice = wave / a.hpb;
+    const uint32_t head = blockIdx.z * a.hpb + wave % a.hpb;
     const uint32_t g = lane % G;
     const uint32_t grp = lane / G;
     const bool head_ok = head < a.num_heads;
 
     const uint32_t len = a.self_len[b];
     const uint32_t nk = len + a.n;
-    const uint32_t c0 = chunk * CHUNK;
     const size_t slab = (size_t)b * a.max_seq_len;
-    const uint32_t col = head * HD + 4u * g;
+    const uint32_t col = (head_ok ? head : 0u) * HD + 4u * g;
+    const uint32_t k_begin = split * a.span;
+    const uint32_t k_end = min(k_begin + a.span, nk);
 
-    if (c0 < nk && head_ok) {
-        /* ---- issue every load of the chunk ---- */
-        float4 kf[LOADS], vf[LOADS];
+    float4 q[NQ], o[NQ];
+    float m[NQ], l[NQ];
+#pragma unroll
+    for (int r = 0; r < NQ; r++) {
+        const uint32_t qi = min(a.q0 + r, a.n - 1u);
+        q[r] = *reinterpret_cast<const float4 *>(a.q_rows + ((size_t)b * a.n + qi) * a.q_stride + col);
+        o[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+        m[r] = neg_inf();
+        l[r] = 0.f;
+    }
+
+    auto fetch = [&](uint32_t c0, float4 (&kf)[LOADS], float4 (&vf)[LOADS]) {
 #pragma unroll
         for (int t = 0; t < LOADS; t++) {
             const uint32_t j = min(c0 + grp + KPL * t, nk - 1u);
@@ -119,122 +133,194 @@ __global__ __launch_bounds__(256) void kv_step_kernel(StepArgs a) {
                 vf[t] = *reinterpret_cast<const float4 *>(a.v_rows + r * a.v_stride + col);
             }
         }
-        float4 q[NQ];
-#pragma unroll
-        for (int r = 0; r < NQ; r++) {
-            const uint32_t qi = min(a.q0 + r, a.n - 1u);
-            q[r] = *reinterpret_cast<const float4 *>(a.q_rows + ((size_t)b * a.n + qi) * a.q_stride + col);
-        }
+    };
 
-        /* ---- write-through of the new rows this chunk holds ---- */
-        if (a.write_through) {
+    const uint32_t stride = a.slices * STEP;
+    uint32_t c0 = k_begin + slice * STEP;
+    float4 kf[LOADS], vf[LOADS];
+    if (c0 < k_end) fetch(c0, kf, vf);
+    while (c0 < k_end) {
+        const uint32_t cn = c0 + stride;
+        float4 kn[LOADS], vn[LOADS];
+        if (cn < k_end) fetch(cn, kn, vn);
+
+        /* write-through of the new rows this sub-chunk holds */
+        if (a.write_through && head_ok) {
 #pragma unroll
             for (int t = 0; t < LOADS; t++) {
                 const uint32_t j = c0 + grp + KPL * t;
-                if (j >= len && j < nk) {
+                if (j >= len && j < k_end) {
                     *reinterpret_cast<float4 *>(a.cache_k + (slab + j) * a.embed_dim + col) = kf[t];
                     *reinterpret_cast<float4 *>(a.cache_v + (slab + j) * a.embed_dim + col) = vf[t];
                 }
             }
         }
 
-        /* ---- scores, chunk-local softmax, PV, merge across the wave ---- */
 #pragma unroll
         for (int r = 0; r < NQ; r++) {
             const uint32_t qi = a.q0 + r;
             const uint32_t p = len + qi; /* absolute position of the query */
             float x[LOADS];
-            float m = neg_inf();
+            float mt = neg_inf();
 #pragma unroll
             for (int t = 0; t < LOADS; t++) {
                 const uint32_t j = c0 + grp + KPL * t;
                 const float s = group_sum<G>(dot4(q[r], kf[t])) * a.scale;
-                bool vis = j < nk && qi < a.n;
+                bool vis = j < k_end && qi < a.n;
                 if (!a.block_kind) vis = vis && j <= p && (a.window == 0u || p - j < a.window);
                 vis = vis && isfinite(s);
                 x[t] = vis ? s : neg_inf();
-                m = fmaxf(m, x[t]);
+                mt = fmaxf(mt, x[t]);
             }
-            float l = 0.f;
-            float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+            const float mn = fmaxf(m[r], mt);
+            const float alpha = m[r] == neg_inf() ? 0.f : softmax_exp(m[r] - mn);
+            float ls = 0.f;
+            float4 acc = make_float4(o[r].x * alpha, o[r].y * alpha, o[r].z * alpha, o[r].w * alpha);
 #pragma unroll
             for (int t = 0; t < LOADS; t++) {
-                const float w = x[t] == neg_inf() ? 0.f : softmax_exp(x[t] - m);
-                l += w;
-                o.x += w * vf[t].x;
-                o.y += w * vf[t].y;
-                o.z += w * vf[t].z;
-                o.w += w * vf[t].w;
+                const float w = x[t] == neg_inf() ? 0.f : softmax_exp(x[t] - mn);
+                ls += w;
+                acc.x += w * vf[t].x;
+                acc.y += w * vf[t].y;
+                acc.z += w * vf[t].z;
+                acc.w += w * vf[t].w;
             }
+            o[r] = acc;
+            l[r] = l[r] * alpha + ls;
+            m[r] = mn;
+        }
+
 #pragma unroll
-            for (int off = G; off < 64; off <<= 1) {
-                const float m2 = __shfl_xor(m, off, 64);
-                const float l2 = __shfl_xor(l, off, 64);
-                float4 o2;
-                o2.x = __shfl_xor(o.x, off, 64);
-                o2.y = __shfl_xor(o.y, off, 64);
-                o2.z = __shfl_xor(o.z, off, 64);
-                o2.w = __shfl_xor(o.w, off, 64);
-                merge_state(m, l, o, m2, l2, o2);
+        for (int t = 0; t < LOADS; t++) {
+            kf[t] = kn[t];
+            vf[t] = vn[t];
+        }
+        c0 = cn;
+    }
+
+    /* ---- merge the lane groups of the wave, park the wave's state in LDS ---- */
+    float *mine = sm + (size_t)wave * NQ * (HD + 2);
+#pragma unroll
+    for (int r = 0; r < NQ; r++) {
+#pragma unroll
+        for (int off = G; off < 64; off <<= 1) {
+            const float m2 = __shfl_xor(m[r], off, 64);
+            const float l2 = __shfl_xor(l[r], off, 64);
+            float4 o2;
+            o2.x = __shfl_xor(o[r].x, off, 64);
+            o2.y = __shfl_xor(o[r].y, off, 64);
+            o2.z = __shfl_xor(o[r].z, off, 64);
+            o2.w = __shfl_xor(o[r].w, off, 64);
+            const float mn = fmaxf(m[r], m2);
+            const float fa = m[r] == neg_inf() ? 0.f : softmax_exp(m[r] - mn);
+            const float fb = m2 == neg_inf() ? 0.f : softmax_exp(m2 - mn);
+            l[r] = l[r] * fa + l2 * fb;
+            o[r].x = o[r].x * fa + o2.x * fb;
+            o[r].y = o[r].y * fa + o2.y * fb;
+            o[r].z = o[r].z * fa + o2.z * fb;
+            o[r].w = o[r].w * fa + o2.w * fb;
+            m[r] = mn;
+        }
+        if (grp == 0) {
+            float *dst = mine + r * (HD + 2) + 4u * g;
+            dst[0] = o[r].x;
+            dst[1] = o[r].y;
+            dst[2] = o[r].z;
+            dst[3] = o[r].w;
+            if (g == 0) {
+                mine[r * (HD + 2) + HD + 0] = m[r];
+                mine[r * (HD + 2) + HD + 1] = l[r];
             }
-            if (grp == 0) {
-                float *dst = a.partial +
-                             ((((size_t)b * a.chunks + chunk) * a.num_heads + head) * NQ + r) * (HD + 2);
-                *reinterpret_cast<float4 *>(dst + 4u * g) = o;
-                if (g == 0) {
-                    dst[HD + 0] = m;
-                    dst[HD + 1] = l;
-                }
+        }
+    }
+    __syncthreads();
+
+    /* ---- merge the slices: thread t owns (local head, query, column) ---- */
+    const uint32_t cells = a.hpb * NQ * HD;
+    for (uint32_t t = threadIdx.x; t < cells; t += blockDim.x) {
+        const uint32_t d = t % HD;
+        const uint32_t r = (t / HD) % NQ;
+        const uint32_t hl = t / (HD * NQ);
+        const uint32_t hh = blockIdx.z * a.hpb + hl;
+        const uint32_t qi = a.q0 + r;
+        if (hh >= a.num_heads || qi >= a.n) continue;
+        float M = neg_inf();
+        for (uint32_t s = 0; s < a.slices; s++)
+            M = fmaxf(M, sm[((size_t)(s * a.hpb + hl) * NQ + r) * (HD + 2) + HD]);
+        float L = 0.f, acc = 0.f;
+        for (uint32_t s = 0; s < a.slices; s++) {
+            const float *ps = sm + ((size_t)(s * a.hpb + hl) * NQ + r) * (HD + 2);
+            const float f = ps[HD] == neg_inf() ? 0.f : softmax_exp(ps[HD] - M);
+            L += ps[HD + 1] * f;
+            acc += ps[d] * f;
+        }
+        if (a.splits == 1u) {
+            a.combined[((size_t)b * a.n + qi) * a.out_stride + hh * HD + d] = L > 0.f ? acc / L : 0.f;
+        } else {
+            float *dst = a.partial + ((((size_t)b * a.splits + split) * a.num_heads + hh) * NQ + r) * (HD + 2);
+            publish(dst + d, acc);
+            if (d == 0) {
+                publish(dst + HD + 0, M);
+                publish(dst + HD + 1, L);
             }
         }
     }
 
-    /* ---- ticket: the last workgroup of the sequence merges ---- */
-    __threadfence();
+    if (a.splits == 1u && gridDim.z == 1u) {
+        if (a.commit && threadIdx.x == 0) a.self_len[b] = nk;
+        return;
+    }
+
+    /* ---- ticket: the last workgroup of the sequence merges the splits ----
+     * The per-split states were stored with device-scope write-through stores
+     * and are read back with device-scope loads, so they never sit dirty or
+     * stale in one die's L2 and no cache write-back or invalidate is needed;
+     * the barrier's wait on outstanding memory operations orders the stores
+     * before this workgroup's ticket. */
     __syncthreads();
-    if (threadIdx.x == 0) sm_ticket = atomicAdd(&a.tickets[b], 1u);
+    if (threadIdx.x == 0) sm_ticket = __hip_atomic_fetch_add(&a.tickets[b], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (sm_ticket != gridDim.x * gridDim.z - 1u) return;
-    __threadfence();
 
-    const uint32_t used = (nk + CHUNK - 1) / CHUNK;
-    const uint32_t heads_per_block = blockDim.x >> 6;
-    /* this block's waves sweep all heads (other z-blocks have finished) */
-    for (uint32_t hh = wave; hh < a.num_heads; hh += heads_per_block) {
-        for (uint32_t r = 0; r < (uint32_t)NQ; r++) {
+    if (a.splits > 1u) {
+        const uint32_t all = a.num_heads * NQ * HD;
+        const size_t sstride = (size_t)a.num_heads * NQ * (HD + 2);
+        for (uint32_t t = threadIdx.x; t < all; t += blockDim.x) {
+            const uint32_t d = t % HD;
+            const uint32_t r = (t / HD) % NQ;
+            const uint32_t hh = t / (HD * NQ);
             const uint32_t qi = a.q0 + r;
-            if (qi >= a.n) break;
-            const float *base = a.partial + (((size_t)b * a.chunks * a.num_heads + hh) * NQ + r) * (HD + 2);
-            const size_t cstride = (size_t)a.num_heads * NQ * (HD + 2);
-            float M = neg_inf();
-            for (uint32_t c = 0; c < used; c++) M = fmaxf(M, base[c * cstride + HD]);
-            float L = 0.f, acc[DPL];
+            if (qi >= a.n) continue;
+            const float *base = a.partial + (((size_t)b * a.splits * a.num_heads + hh) * NQ + r) * (HD + 2);
+            float pm[MAX_SPLITS], pl[MAX_SPLITS], po[MAX_SPLITS];
 #pragma unroll
-            for (int e = 0; e < DPL; e++) acc[e] = 0.f;
-            for (uint32_t c = 0; c < used; c++) {
-                const float *pc = base + c * cstride;
-                const float mc = pc[HD];
-                const float f = mc == neg_inf() ? 0.f : softmax_exp(mc - M);
-                L += pc[HD + 1] * f;
-#pragma unroll
-                for (int e = 0; e < DPL; e++)
-                    if (lane + 64u * e < (uint32_t)HD) acc[e] += pc[lane + 64u * e] * f;
+            for (int s = 0; s < MAX_SPLITS; s++) {
+                const bool on = (uint32_t)s < a.splits;
+                const float *ps = base + (on ? s : 0) * sstride;
+                pm[s] = on ? observe(ps + HD) : neg_inf();
+                pl[s] = on ? observe(ps + HD + 1) : 0.f;
+                po[s] = on ? observe(ps + d) : 0.f;
             }
+            float M = neg_inf();
 #pragma unroll
-            for (int e = 0; e < DPL; e++)
-                if (lane + 64u * e < (uint32_t)HD)
-                    a.combined[((size_t)b * a.n + qi) * a.out_stride + hh * HD + lane + 64u * e] =
-                        L > 0.f ? acc[e] / L : 0.f;
+            for (int s = 0; s < MAX_SPLITS; s++) M = fmaxf(M, pm[s]);
+            float L = 0.f, acc = 0.f;
+#pragma unroll
+            for (int s = 0; s < MAX_SPLITS; s++) {
+                const float f = pm[s] == neg_inf() ? 0.f : softmax_exp(pm[s] - M);
+                L += pl[s] * f;
+                acc += po[s] * f;
+            }
+            a.combined[((size_t)b * a.n + qi) * a.out_stride + hh * HD + d] = L > 0.f ? acc / L : 0.f;
         }
     }
-    __syncthreads();
     if (threadIdx.x == 0) {
         a.tickets[b] = 0u;
         if (a.commit) a.self_len[b] = nk;
     }
 }
 
-/* scratch the family owns: partial softmax states and per-sequence tickets */
+/* scratch the family owns: per-split softmax states and per-sequence tickets */
 struct Scratch {
     float *partial = nullptr;
     size_t partial_floats = 0;
@@ -247,20 +333,38 @@ Scratch &scratch() {
     return s;
 }
 
-template <int G, int NQ>
-void launch_step(const StepArgs &a, uint32_t batch, hipStream_t s) {
-    const uint32_t hpb = std::min<uint32_t>(a.num_heads, 4u);
-    dim3 grid(a.chunks, batch, (a.num_heads + hpb - 1) / hpb);
-    blt_launch("kv_step", kv_step_kernel<G, NQ>, grid, dim3(64 * hpb), 0, s, a);
+template <int G, int NQ, int WAVES>
+void launch_step(StepArgs a, uint32_t batch, hipStream_t s) {
+    constexpr int HD = 4 * G;
+    a.hpb = std::min<uint32_t>(a.num_heads, (uint32_t)WAVES);
+    a.slices = std::max<uint32_t>(1u, (uint32_t)WAVES / a.hpb);
+    /* no more slices than a span has sub-chunks */
+    const uint32_t subs = (a.span + SUB - 1) / SUB;
+    a.slices = std::min(a.slices, std::max(1u, subs));
+    const uint32_t waves = a.hpb * a.slices;
+    dim3 grid(a.splits, batch, (a.num_heads + a.hpb - 1) / a.hpb);
+    const size_t lds = (size_t)waves * NQ * (HD + 2) * sizeof(float);
+    blt_launch("kv_step", kv_step_kernel<G, NQ, WAVES>, grid, dim3(64 * waves), lds, s, a);
+}
+
+/* tuning hooks: BLT_HIP_DECODE_WAVES = 4|8|16 waves per workgroup (decode
+ * rows only), BLT_HIP_DECODE_SPAN = sub-chunks of 32 keys per split */
+int env_int(const char *name, int fallback) {
+    const char *e = getenv(name);
+    return e && *e ? atoi(e) : fallback;
 }
 
 template <int G>
 void dispatch_nq(const StepArgs &a, uint32_t nq, uint32_t batch, hipStream_t s) {
-    if (nq <= 1) launch_step<G, 1>(a, batch, s);
-    else if (nq <= 2) launch_step<G, 2>(a, batch, s);
-    else if (nq <= 4) launch_step<G, 4>(a, batch, s);
-    else if (nq <= 8) launch_step<G, 8>(a, batch, s);
-    else launch_step<G, 16>(a, batch, s);
+    static const int waves = env_int("BLT_HIP_DECODE_WAVES", 4);
+    if (nq <= 1) {
+        if (waves >= 16) launch_step<G, 1, 16>(a, batch, s);
+        else if (waves >= 8) launch_step<G, 1, 8>(a, batch, s);
+        else launch_step<G, 1, 4>(a, batch, s);
+    } else if (nq <= 2) launch_step<G, 2, 8>(a, batch, s);
+    else if (nq <= 4) launch_step<G, 4, 4>(a, batch, s);
+    else if (nq <= 8) launch_step<G, 8, 4>(a, batch, s);
+    else launch_step<G, 16, 4>(a, batch, s);
 }
 
 } // namespace
@@ -281,8 +385,8 @@ extern "C" void blt_kv_attend_step_hip(const blt_kv_attn_cache *cache, const flo
     const size_t E = cache->embed_dim, H = cache->num_heads;
     BLT_REQUIRE(H >= 1 && E % H == 0, "blt_kv_attend_step: embed_dim must be divisible by num_heads");
     const size_t hd = E / H;
-    BLT_REQUIRE(hd == 4 || hd == 8 || hd == 16 || hd == 32 || hd == 64 || hd == 128 || hd == 256,
-                "blt_kv_attend_step: head_dim must be a power of two in [4, 256]");
+    BLT_REQUIRE(hd == 4 || hd == 8 || hd == 16 || hd == 32 || hd == 64 || hd == 128,
+                "blt_kv_attend_step: head_dim must be a power of two in [4, 128]");
     BLT_REQUIRE(max_len_hint >= n && max_len_hint <= cache->max_seq_len, "blt_kv_attend_step: exceeds cache capacity");
     BLT_REQUIRE(cache->batch >= 1 && cache->batch <= 65535, "blt_kv_attend_step: batch must be in [1, 65535]");
     BLT_REQUIRE(q_stride % 4 == 0 && k_stride % 4 == 0 && v_stride % 4 == 0 && combined_stride >= E &&
@@ -308,16 +412,28 @@ extern "C" void blt_kv_attend_step_hip(const blt_kv_attn_cache *cache, const flo
     a.max_seq_len = (uint32_t)cache->max_seq_len;
     a.embed_dim = (uint32_t)E;
     a.num_heads = (uint32_t)H;
-    a.head_dim = (uint32_t)hd;
     a.window = (uint32_t)cache->window;
     a.n = (uint32_t)n;
-    const size_t chunk = (size_t)chunk_keys((int)(hd / 4));
-    a.chunks = (uint32_t)((max_len_hint + chunk - 1) / chunk);
     a.scale = 1.0f / sqrtf((float)hd);
     a.block_kind = step_kind == BLT_KV_STEP_BLOCK;
+    a.hpb = a.slices = 1;
+
+    /* enough workgroups to fill 256 compute units a few times over (sequences
+     * shorter than the hint leave theirs idle), but no span shorter than two
+     * sub-chunks */
+    static const int span_env = env_int("BLT_HIP_DECODE_SPAN", 0);
+    const size_t subs = (max_len_hint + SUB - 1) / SUB;
+    size_t splits = (1024 + cache->batch - 1) / cache->batch;
+    splits = std::min<size_t>(splits, (subs + 1) / 2);
+    if (span_env > 0) splits = (subs + span_env - 1) / span_env;
+    splits = std::max<size_t>(1, std::min<size_t>(splits, MAX_SPLITS));
+    const size_t span_subs = (subs + splits - 1) / splits;
+    splits = (subs + span_subs - 1) / span_subs;
+    a.splits = (uint32_t)splits;
+    a.span = (uint32_t)(span_subs * SUB);
 
     Scratch &sc = scratch();
-    const size_t need = cache->batch * (size_t)a.chunks * H * 16u * (hd + 2);
+    const size_t need = cache->batch * (size_t)MAX_SPLITS * H * 16u * (hd + 2);
     if (need > sc.partial_floats) {
         if (sc.partial) {
             HIP_CHECK(hipDeviceSynchronize());
@@ -352,8 +468,7 @@ extern "C" void blt_kv_attend_step_hip(const blt_kv_attn_cache *cache, const flo
         case 16: dispatch_nq<4>(a, nq, (uint32_t)cache->batch, 0); break;
         case 32: dispatch_nq<8>(a, nq, (uint32_t)cache->batch, 0); break;
         case 64: dispatch_nq<16>(a, nq, (uint32_t)cache->batch, 0); break;
-        case 128: dispatch_nq<32>(a, nq, (uint32_t)cache->batch, 0); break;
-        default: dispatch_nq<64>(a, nq, (uint32_t)cache->batch, 0); break;
+        default: dispatch_nq<32>(a, nq, (uint32_t)cache->batch, 0); break;
         }
     }
     HIP_CHECK_LAUNCH("blt_kv_attend_step");
