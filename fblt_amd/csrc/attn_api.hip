@@ -22,6 +22,10 @@ enum Family : uint32_t { FAM_ROWS = 0, FAM_MFMA = 1, FAM_COUNT = 2 };
 struct Bucket {
     Family fam;
     uint32_t hd;      /* head_dim shared by the bucket */
+    bool vec4;        /* every problem has ATTN_FLAG_VEC4 */
+    bool dense;       /* every problem reads a dense mask */
+    bool affine;      /* mfma: problems are one strided batch, see `aff` */
+    AttnAffine aff;
     uint32_t base;    /* first descriptor in the sorted array */
     uint32_t count;
     uint32_t max_nq;
@@ -119,6 +123,78 @@ Family choose_family(const AttnProb &d) {
     return FAM_ROWS;
 }
 
+/* Element distance between two float pointers (either both NULL or both set). */
+bool elem_delta(const void *a, const void *b, int64_t &out) {
+    if ((a == nullptr) != (b == nullptr)) return false;
+    const int64_t bytes = (int64_t)(reinterpret_cast<intptr_t>(b) - reinterpret_cast<intptr_t>(a));
+    if (bytes % 4 != 0) return false;
+    out = bytes / 4;
+    return true;
+}
+
+bool same_shape(const AttnProb &a, const AttnProb &b) {
+    return a.q_stride == b.q_stride && a.k_stride == b.k_stride && a.v_stride == b.v_stride &&
+           a.out_stride == b.out_stride && a.nq == b.nq && a.nk == b.nk && a.hd == b.hd && a.vis == b.vis &&
+           a.causal_off == b.causal_off && a.window == b.window && a.scale == b.scale && a.flags == b.flags;
+}
+
+/* The nine pointers of a problem, in a fixed order. */
+void pointers_of(const AttnProb &d, const void *(&out)[9]) {
+    out[0] = d.q, out[1] = d.k, out[2] = d.v, out[3] = d.out, out[4] = d.weights, out[5] = d.lse, out[6] = d.mask;
+    out[7] = d.row_lo, out[8] = d.row_hi;
+}
+
+/* Are problems p[0..n) one strided batch: p[i] = p[0] + (i / H) * seq + (i % H) * head
+ * for every pointer, with a common shape?  Fills `out` for the first H that fits. */
+bool detect_affine(const AttnProb *p, uint32_t n, AttnAffine &out) {
+    if (n < 2) return false;
+    for (uint32_t i = 1; i < n; i++)
+        if (!same_shape(p[0], p[i])) return false;
+    for (uint32_t H = 1; H <= n; H++) {
+        if (n % H != 0) continue;
+        int64_t head[9], seq[9];
+        const void *p0[9], *pi[9];
+        pointers_of(p[0], p0);
+        bool ok = true;
+        for (int f = 0; f < 9 && ok; f++) {
+            head[f] = seq[f] = 0;
+            if (H > 1) {
+                pointers_of(p[1], pi);
+                ok = elem_delta(p0[f], pi[f], head[f]);
+            }
+            if (ok && n > H) {
+                pointers_of(p[H], pi);
+                ok = elem_delta(p0[f], pi[f], seq[f]);
+            }
+        }
+        for (uint32_t i = 0; i < n && ok; i++) {
+            pointers_of(p[i], pi);
+            for (int f = 0; f < 9 && ok; f++) {
+                int64_t d;
+                ok = elem_delta(p0[f], pi[f], d) &&
+                     (p0[f] == nullptr || d == (int64_t)(i / H) * seq[f] + (int64_t)(i % H) * head[f]);
+            }
+        }
+        if (!ok) continue;
+        if (seq[7] != seq[8] || head[7] != head[8]) continue; /* row_lo and row_hi move together */
+        std::memset(&out, 0, sizeof(out));
+        out.first = p[0];
+        out.q_seq = seq[0], out.q_head = head[0];
+        out.k_seq = seq[1], out.k_head = head[1];
+        out.v_seq = seq[2], out.v_head = head[2];
+        out.o_seq = seq[3], out.o_head = head[3];
+        out.w_seq = seq[4], out.w_head = head[4];
+        out.lse_seq = seq[5], out.lse_head = head[5];
+        out.mask_seq = seq[6], out.mask_head = head[6];
+        out.range_seq = seq[7], out.range_head = head[7];
+        out.count = n;
+        out.heads = H;
+        out.nqt = (p[0].nq + 31u) / 32u;
+        return true;
+    }
+    return false;
+}
+
 } // namespace
 
 struct blt_attention_plan {
@@ -144,7 +220,8 @@ void plan_build(blt_attention_plan &pl, const blt_attention_problem *problems, s
         AttnProb d = translate(problems[t], need_score_buffer, what);
         if (d.nq == 0) continue; /* nothing to write */
         const Family f = choose_family(d);
-        keyed.emplace_back(((uint64_t)f << 32) | d.hd, d);
+        const uint64_t vec4 = (d.flags & ATTN_FLAG_VEC4) ? 1u : 0u, dense = d.vis == ATTN_VIS_DENSE ? 1u : 0u;
+        keyed.emplace_back(((uint64_t)f << 40) | ((uint64_t)d.hd << 8) | (vec4 << 1) | dense, d);
     }
     std::stable_sort(keyed.begin(), keyed.end(),
                      [](const std::pair<uint64_t, AttnProb> &x, const std::pair<uint64_t, AttnProb> &y) {
@@ -152,11 +229,14 @@ void plan_build(blt_attention_plan &pl, const blt_attention_problem *problems, s
                      });
     for (size_t t = 0; t < keyed.size(); t++) {
         const AttnProb &d = keyed[t].second;
-        const Family f = (Family)(keyed[t].first >> 32);
-        if (pl.buckets.empty() || pl.buckets.back().fam != f || pl.buckets.back().hd != d.hd) {
+        const Family f = (Family)(keyed[t].first >> 40);
+        if (t == 0 || keyed[t].first != keyed[t - 1].first) {
             Bucket b;
+            std::memset(&b, 0, sizeof(b));
             b.fam = f;
             b.hd = d.hd;
+            b.vec4 = (d.flags & ATTN_FLAG_VEC4) != 0;
+            b.dense = d.vis == ATTN_VIS_DENSE;
             b.base = (uint32_t)t;
             b.count = 0;
             b.max_nq = 0;
@@ -171,6 +251,8 @@ void plan_build(blt_attention_plan &pl, const blt_attention_problem *problems, s
     }
     for (Bucket &b : pl.buckets) {
         if (b.fam != FAM_MFMA) continue;
+        b.affine = detect_affine(pl.host.data() + b.base, b.count, b.aff);
+        if (b.affine) continue; /* no descriptor or tile memory needed */
         b.tile_base = (uint32_t)pl.tiles.size();
         attn_mfma_make_tiles(pl.host.data(), b.base, b.count, pl.tiles);
         b.tiles = (uint32_t)pl.tiles.size() - b.tile_base;
@@ -182,8 +264,10 @@ void plan_build(blt_attention_plan &pl, const blt_attention_problem *problems, s
 
 void plan_launch(const blt_attention_plan &pl, const AttnProb *dev, const AttnTile *dev_tiles) {
     for (const Bucket &b : pl.buckets) {
-        if (b.fam == FAM_MFMA)
-            attn_mfma_launch(dev, dev_tiles + b.tile_base, b.tiles, b.hd, 0);
+        if (b.fam == FAM_MFMA && b.affine)
+            attn_mfma_launch_affine(b.aff, 0);
+        else if (b.fam == FAM_MFMA)
+            attn_mfma_launch(dev, dev_tiles + b.tile_base, b.tiles, b.hd, b.vec4, b.dense, 0);
         else
             attn_rows_launch(dev, b.base, b.count, b.hd, b.max_nq, 0);
     }

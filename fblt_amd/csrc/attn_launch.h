@@ -15,6 +15,19 @@ struct AttnTile {
     uint32_t qtile; /* rows [32*qtile, 32*qtile+32)            */
 };
 
+/* A batch whose problems differ from the first one only by (sequence, head)
+ * strides: problem i = seq * heads + head.  Travels in the kernel arguments,
+ * so a launch needs no descriptor memory at all.  Strides are in elements. */
+struct AttnAffine {
+    AttnProb first;
+    int64_t q_seq, q_head, k_seq, k_head, v_seq, v_head, o_seq, o_head;
+    int64_t w_seq, w_head, lse_seq, lse_head, mask_seq, mask_head, range_seq, range_head;
+    uint32_t count; /* problems                       */
+    uint32_t heads; /* problems per sequence          */
+    uint32_t nqt;   /* 32-row query tiles per problem */
+    uint32_t reserved;
+};
+
 /* rows family: problems [base, base+count) of a device array share head_dim hd */
 void attn_rows_launch(const AttnProb *dprobs, uint32_t base, uint32_t count, uint32_t hd, uint32_t max_nq,
                       hipStream_t s);
@@ -25,7 +38,9 @@ void attn_rows_launch_single(const AttnProb &single, hipStream_t s);
 bool attn_mfma_can(const AttnProb &d);
 bool attn_mfma_takes(const AttnProb &d);
 void attn_mfma_make_tiles(const AttnProb *host, uint32_t base, uint32_t count, std::vector<AttnTile> &tiles);
-void attn_mfma_launch(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t ntiles, uint32_t hd, hipStream_t s);
+void attn_mfma_launch(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t ntiles, uint32_t hd, bool vec4,
+                      bool dense, hipStream_t s);
 void attn_mfma_launch_single(const AttnProb &single, hipStream_t s);
+void attn_mfma_launch_affine(const AttnAffine &aff, hipStream_t s);
 
 #endif

@@ -47,10 +47,21 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 /* key (within a 32-key tile) that accumulator register r of lane half h holds */
 __device__ __forceinline__ constexpr uint32_t acc_key(uint32_t r, uint32_t h) { return 8u * (r >> 2) + 4u * h + (r & 3u); }
 
-template <int HALF> /* HALF = HD/2 floats of one row, starting at element d0 */
+/* HALF = HD/2 floats of one row starting at element d0.  EXACT: 16-byte
+ * aligned rows and head_dim == HD, so no element needs a guard. */
+template <int HALF, bool EXACT>
 __device__ __forceinline__ void load_half_row(float (&dst)[HALF], const float *row, uint32_t d0, uint32_t hd,
                                               bool vec4) {
-    if (vec4) {
+    if (EXACT) {
+#pragma unroll
+        for (int s = 0; s < HALF; s += 4) {
+            const float4 t = *reinterpret_cast<const float4 *>(row + d0 + s);
+            dst[s + 0] = t.x;
+            dst[s + 1] = t.y;
+            dst[s + 2] = t.z;
+            dst[s + 3] = t.w;
+        }
+    } else if (vec4) {
 #pragma unroll
         for (int s = 0; s < HALF; s += 4) {
             float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -66,26 +77,147 @@ __device__ __forceinline__ void load_half_row(float (&dst)[HALF], const float *r
     }
 }
 
-template <int HD, bool SINGLE>
+/* where a workgroup finds its problem */
+enum : int {
+    SRC_TILES = 0,  /* device arrays: tiles[blockIdx.x] -> probs[tile.prob]           */
+    SRC_SINGLE = 1, /* one problem in the kernel arguments                            */
+    SRC_AFFINE = 2  /* kernel arguments: first problem + (sequence, head) strides     */
+};
+
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+
+/* 2^x on the transcendental unit; 2^(-inf) = 0 */
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+/* ---- operand movement helpers (register arrays by reference so they stay in registers) ---- */
+
+/* 32 rows x HD floats, rows [row0, row0+32) clamped to nrows-1: consecutive
+ * lanes take consecutive 16-byte pieces of a row; one wave moves the tile. */
+template <int HD>
+__device__ __forceinline__ void tile_to_regs(float (&kg)[HD / 2], const float *base, uint32_t stride,
+                                             uint32_t row0, uint32_t nrows, uint32_t lane) {
+    constexpr int LPR = HD / 4;
+#pragma unroll
+    for (int t = 0; t < HD / 8; t++) {
+        const uint32_t r = t * (64 / LPR) + lane / LPR;
+        const uint32_t j = min(row0 + r, nrows - 1u);
+        const float4 x = *reinterpret_cast<const float4 *>(base + (size_t)j * stride + 4u * (lane % LPR));
+        kg[4 * t + 0] = x.x;
+        kg[4 * t + 1] = x.y;
+        kg[4 * t + 2] = x.z;
+        kg[4 * t + 3] = x.w;
+    }
+}
+
+template <int HD>
+__device__ __forceinline__ void regs_to_lds(const float (&kg)[HD / 2], float *dst, uint32_t lane) {
+    constexpr int LPR = HD / 4;
+    constexpr int ROW = HD + 4;
+#pragma unroll
+    for (int t = 0; t < HD / 8; t++) {
+        const uint32_t r = t * (64 / LPR) + lane / LPR;
+        *reinterpret_cast<float4 *>(dst + r * ROW + 4u * (lane % LPR)) =
+            make_float4(kg[4 * t + 0], kg[4 * t + 1], kg[4 * t + 2], kg[4 * t + 3]);
+    }
+}
+
+/* generic tile move (unaligned rows or head_dim < HD): element by element */
+template <int HD>
+__device__ __forceinline__ void tile_to_lds_slow(float *dst, const float *base, uint32_t stride, uint32_t row0,
+                                                 uint32_t nrows, uint32_t hd, uint32_t first, uint32_t step) {
+    constexpr int ROW = HD + 4;
+    for (uint32_t e = first; e < 32u * HD; e += step) {
+        const uint32_t r = e / HD, d = e % HD;
+        const uint32_t j = min(row0 + r, nrows - 1u);
+        dst[r * ROW + d] = d < hd ? base[(size_t)j * stride + d] : 0.f;
+    }
+}
+
+/* MFMA fragment of lane (h, c): row c, floats [h*HD/2, (h+1)*HD/2) */
+template <int HD>
+__device__ __forceinline__ void frag_from_lds(float (&dst)[HD / 2], const float *src, uint32_t h, uint32_t c) {
+    constexpr int ROW = HD + 4;
+    constexpr int HALF = HD / 2;
+#pragma unroll
+    for (int s4 = 0; s4 < HALF; s4 += 4) {
+        const float4 t = *reinterpret_cast<const float4 *>(src + c * ROW + h * HALF + s4);
+        dst[s4 + 0] = t.x;
+        dst[s4 + 1] = t.y;
+        dst[s4 + 2] = t.z;
+        dst[s4 + 3] = t.w;
+    }
+}
+
+/* LDS of one workgroup.  Q tile and per-wave K tiles are row-major with a
+ * 4-float pad per row: a lane's 16-byte fragment reads (row = lane % 32) then
+ * fall on distinct banks for every 16 lanes.  The output merge reuses the K
+ * area once the key loop is over. */
+template <int HD, bool STAGE>
+struct MfmaLds {
+    static constexpr int ROW = HD + 4;
+    static constexpr int Q_FLOATS = STAGE ? 32 * ROW : 0;
+    static constexpr int K_FLOATS = STAGE ? 4 * 32 * ROW : 0;
+    static constexpr int MERGE_FLOATS = 3 * HD * 33;
+    static constexpr int BODY_FLOATS = K_FLOATS > MERGE_FLOATS ? K_FLOATS : MERGE_FLOATS;
+};
+
+template <int HD, int SRC, bool EXACT, bool DENSE>
 __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnProb *__restrict__ probs,
-                                                        const AttnTile *__restrict__ tiles, AttnProb single) {
+                                                        const AttnTile *__restrict__ tiles, AttnAffine aff) {
     constexpr int HALF = HD / 2;
     constexpr int DB = HD / 32; /* 32-wide blocks of the head dim */
+    /* K and Q tiles go through LDS (coalesced global reads, transposing LDS
+     * reads) whenever they fit the 64 KB a workgroup may declare statically */
+    constexpr bool STAGE = HD <= 64;
+    using Lds = MfmaLds<HD, STAGE>;
+    constexpr int ROW = Lds::ROW;
 
     __shared__ float sm_m[4][32];
     __shared__ float sm_l[4][32];
-    __shared__ float sm_o[3][HD][33];
+    __shared__ __attribute__((aligned(16))) float sm_q[Lds::Q_FLOATS > 0 ? Lds::Q_FLOATS : 4];
+    __shared__ __attribute__((aligned(16))) float sm_body[Lds::BODY_FLOATS];
+    float(*sm_o)[HD][33] = reinterpret_cast<float(*)[HD][33]>(sm_body);
 
-    /* SINGLE: the one problem arrives as a kernel argument and block b takes
-     * query tile (last - b): later tiles of a causal problem are the long ones */
-    const uint32_t qtile = SINGLE ? gridDim.x - 1u - blockIdx.x : tiles[blockIdx.x].qtile;
-    const AttnProb p = SINGLE ? single : probs[tiles[blockIdx.x].prob];
+    uint32_t qtile;
+    AttnProb p;
+    if (SRC == SRC_TILES) {
+        qtile = tiles[blockIdx.x].qtile;
+        p = probs[tiles[blockIdx.x].prob];
+    } else if (SRC == SRC_SINGLE) {
+        /* block b takes query tile (last - b): later tiles of a causal problem are the long ones */
+        qtile = gridDim.x - 1u - blockIdx.x;
+        p = aff.first;
+    } else {
+        /* consecutive blocks are different problems of the same query tile,
+         * longest tiles first; all tiles of a problem sit at blockIdx = prob
+         * (mod count), i.e. on one die when count is a multiple of the die count */
+        const uint32_t prob = blockIdx.x % aff.count;
+        qtile = aff.nqt - 1u - blockIdx.x / aff.count;
+        const int64_t sq = prob / aff.heads, hh = prob % aff.heads;
+        /* field by field: a whole-struct copy that is then edited ends up in scratch memory */
+        const AttnProb &f = aff.first;
+        p.q = f.q + (sq * aff.q_seq + hh * aff.q_head);
+        p.k = f.k + (sq * aff.k_seq + hh * aff.k_head);
+        p.v = f.v + (sq * aff.v_seq + hh * aff.v_head);
+        p.out = f.out + (sq * aff.o_seq + hh * aff.o_head);
+        p.weights = f.weights ? f.weights + (sq * aff.w_seq + hh * aff.w_head) : nullptr;
+        p.lse = f.lse ? f.lse + (sq * aff.lse_seq + hh * aff.lse_head) : nullptr;
+        p.mask = DENSE ? f.mask + (sq * aff.mask_seq + hh * aff.mask_head) : nullptr;
+        const bool ranged = f.vis == ATTN_VIS_RANGE;
+        p.row_lo = ranged ? f.row_lo + (sq * aff.range_seq + hh * aff.range_head) : nullptr;
+        p.row_hi = ranged ? f.row_hi + (sq * aff.range_seq + hh * aff.range_head) : nullptr;
+        p.q_stride = f.q_stride, p.k_stride = f.k_stride, p.v_stride = f.v_stride, p.out_stride = f.out_stride;
+        p.nq = f.nq, p.nk = f.nk, p.hd = f.hd, p.vis = f.vis;
+        p.causal_off = f.causal_off, p.window = f.window, p.scale = f.scale, p.flags = f.flags;
+        p.reserved0 = p.reserved1 = 0;
+    }
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
     const uint32_t h = lane >> 5;
     const uint32_t c = lane & 31u;
-    const bool vec4 = (p.flags & ATTN_FLAG_VEC4) != 0;
+    const bool vec4 = EXACT || (p.flags & ATTN_FLAG_VEC4) != 0;
 
     const uint32_t q0 = qtile * 32u;
     const uint32_t row = q0 + c;
@@ -96,20 +228,35 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnProb *__restri
     row_key_range(p, i, lo, hi);
     if (!live) hi = lo;
 
-    /* key tiles any row of this query tile can see */
-    uint32_t tlo = hi > lo ? lo : 0xFFFFFFFFu, thi = hi > lo ? hi : 0u;
+    /* key tiles any row of this query tile can see [tlo, thi), and the keys
+     * every row sees [flo, fhi): closed form unless rows carry their own ranges */
+    uint32_t tlo, thi, flo, fhi;
+    if (p.vis == ATTN_VIS_RANGE) {
+        tlo = hi > lo ? lo : 0xFFFFFFFFu, thi = hi > lo ? hi : 0u;
+        flo = lo, fhi = hi;
 #pragma unroll
-    for (int off = 1; off < 32; off <<= 1) {
-        tlo = min(tlo, (uint32_t)__shfl_xor((int)tlo, off, 64));
-        thi = max(thi, (uint32_t)__shfl_xor((int)thi, off, 64));
+        for (int off = 1; off < 32; off <<= 1) {
+            tlo = min(tlo, (uint32_t)__shfl_xor((int)tlo, off, 64));
+            thi = max(thi, (uint32_t)__shfl_xor((int)thi, off, 64));
+            flo = max(flo, (uint32_t)__shfl_xor((int)flo, off, 64));
+            fhi = min(fhi, (uint32_t)__shfl_xor((int)fhi, off, 64));
+        }
+    } else {
+        /* ranges are monotone in the row index: first and last row bound the tile */
+        const uint32_t last = min(q0 + 31u, p.nq - 1u);
+        uint32_t lo_a, hi_a, lo_b, hi_b;
+        row_key_range(p, q0, lo_a, hi_a);
+        row_key_range(p, last, lo_b, hi_b);
+        tlo = hi_a > lo_a ? lo_a : (hi_b > lo_b ? lo_b : 0xFFFFFFFFu);
+        thi = hi_b > lo_b ? hi_b : hi_a;
+        if (!(thi > tlo)) tlo = 0xFFFFFFFFu, thi = 0u;
+        flo = lo_b, fhi = hi_a;
     }
     const uint32_t kt_lo = thi > tlo ? tlo / 32u : 0u;
     const uint32_t kt_hi = thi > tlo ? (thi + 31u) / 32u : 0u;
 
-    float qf[HALF];
-    load_half_row<HALF>(qf, p.q + (size_t)i * p.q_stride, h * HALF, p.hd, vec4);
-
-    const float *mrow = p.vis == ATTN_VIS_DENSE ? p.mask + (size_t)i * p.nk : nullptr;
+    const float *mrow = DENSE ? p.mask + (size_t)i * p.nk : nullptr;
+    const float scale2 = p.scale * LOG2E; /* scores are kept in log2 units: weights are 2^(x - m) */
 
     floatx16 oacc[DB];
 #pragma unroll
@@ -118,21 +265,88 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnProb *__restri
         for (int r = 0; r < 16; r++) oacc[b][r] = 0.f;
     float m = neg_inf(), l = 0.f;
 
-    for (uint32_t kt = kt_lo + wave; kt < kt_hi; kt += 4u) {
-        const uint32_t k0 = kt * 32u;
-        /* ---- fetch ---- */
-        float kf[HALF];
-        {
-            const uint32_t j = min(k0 + c, p.nk - 1u);
-            load_half_row<HALF>(kf, p.k + (size_t)j * p.k_stride, h * HALF, p.hd, vec4);
+    /* ---- operand movement ----
+     * STAGE: a tile (32 rows x HD floats) is read from global memory with
+     * consecutive lanes on consecutive 16-byte pieces of a row (a few cache
+     * lines per load instruction instead of one per lane), parked in LDS and
+     * read back as MFMA fragments (lane = row).  !STAGE: fragments are read
+     * straight from global memory. */
+    constexpr int LPR = HD / 4;          /* lanes per row, 16-byte pieces           */
+    float kg[HD / 2]; /* one 32-row tile spread over the wave, 16 bytes per lane and step */
+    float *my_k = sm_body + (STAGE ? wave * 32 * ROW : 0);
+
+    float qf[HALF];
+    float kf[HALF];
+    float vf[DB][16];
+
+    if (STAGE) {
+        /* the query tile is shared by the four waves: each brings a quarter */
+        if (EXACT) {
+            constexpr int QPT = 32 * LPR / 256 > 0 ? 32 * LPR / 256 : 1; /* float4 per thread */
+#pragma unroll
+            for (int t = 0; t < QPT; t++) {
+                const uint32_t e = threadIdx.x + 256u * t;
+                if (e < 32u * LPR) {
+                    const uint32_t r = e / LPR, f4 = e % LPR;
+                    const uint32_t qi = min(q0 + r, p.nq - 1u);
+                    *reinterpret_cast<float4 *>(sm_q + r * ROW + 4u * f4) =
+                        *reinterpret_cast<const float4 *>(p.q + (size_t)qi * p.q_stride + 4u * f4);
+                }
+            }
+        } else {
+            tile_to_lds_slow<HD>(sm_q, p.q, p.q_stride, q0, p.nq, p.hd, threadIdx.x, 256u);
         }
-        float vf[DB][16];
+    } else {
+        load_half_row<HALF, EXACT>(qf, p.q + (size_t)i * p.q_stride, h * HALF, p.hd, vec4);
+    }
+
+    /* K tile kt: global -> (registers ->) this wave's LDS area, in two steps
+     * so the global reads can be in flight while other work runs */
+#define K_REQUEST(kt_)                                                                                             \
+    do {                                                                                                           \
+        if (STAGE) {                                                                                               \
+            if (EXACT) tile_to_regs<HD>(kg, p.k, p.k_stride, (kt_) * 32u, p.nk, lane);                             \
+        } else {                                                                                                   \
+            const uint32_t j_ = min((kt_) * 32u + c, p.nk - 1u);                                                   \
+            load_half_row<HALF, EXACT>(kf, p.k + (size_t)j_ * p.k_stride, h * HALF, p.hd, vec4);                   \
+        }                                                                                                          \
+    } while (0)
+#define K_PARK(kt_)                                                                                                \
+    do {                                                                                                           \
+        if (STAGE) {                                                                                               \
+            if (EXACT) regs_to_lds<HD>(kg, my_k, lane);                                                            \
+            else tile_to_lds_slow<HD>(my_k, p.k, p.k_stride, (kt_) * 32u, p.nk, p.hd, lane, 64u);                  \
+        }                                                                                                          \
+    } while (0)
+
+    auto fetch_v = [&](uint32_t kt) __attribute__((always_inline)) {
 #pragma unroll
         for (int s = 0; s < 16; s++) {
-            const uint32_t j = min(k0 + acc_key(s, h), p.nk - 1u);
+            const uint32_t j = min(kt * 32u + acc_key(s, h), p.nk - 1u);
             const float *vrow = p.v + (size_t)j * p.v_stride;
 #pragma unroll
-            for (int b = 0; b < DB; b++) vf[b][s] = (b * 32u + c) < p.hd ? vrow[b * 32 + c] : 0.f;
+            for (int b = 0; b < DB; b++) vf[b][s] = (EXACT || (b * 32u + c) < p.hd) ? vrow[b * 32 + c] : 0.f;
+        }
+    };
+
+    uint32_t kt = kt_lo + wave;
+    if (kt < kt_hi) {
+        K_REQUEST(kt);
+        fetch_v(kt);
+    }
+    if (STAGE) {
+        __syncthreads(); /* query tile complete */
+        frag_from_lds<HD>(qf, sm_q, h, c);
+        if (kt < kt_hi) K_PARK(kt);
+    }
+    while (kt < kt_hi) {
+        const uint32_t k0 = kt * 32u;
+        const uint32_t ktn = kt + 4u;
+
+        if (STAGE) {
+            frag_from_lds<HD>(kf, my_k, h, c);
+            /* the next tile's K rows travel while this tile is worked on */
+            if (ktn < kt_hi) K_REQUEST(ktn);
         }
 
         /* ---- S^T = K Q^T ---- */
@@ -141,26 +355,31 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnProb *__restri
         for (int r = 0; r < 16; r++) sacc[r] = 0.f;
 #pragma unroll
         for (int s = 0; s < HALF; s++) sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[s], qf[s], sacc, 0, 0, 0);
+        if (!STAGE && ktn < kt_hi) K_REQUEST(ktn);
 
         /* ---- scale, mask, tile maximum ---- */
         float x[16];
         float mt = neg_inf();
+        const bool all_seen = !DENSE && k0 >= flo && k0 + 32u <= fhi; /* uniform: no row masks any key */
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const uint32_t j = k0 + acc_key(r, h);
-            float t = sacc[r] * p.scale;
-            if (mrow) t += mrow[min(j, p.nk - 1u)];
-            const bool vis = j >= lo && j < hi && isfinite(t);
+            float t;
+            if (DENSE) t = (sacc[r] * p.scale + mrow[min(j, p.nk - 1u)]) * LOG2E;
+            else t = sacc[r] * scale2;
+            bool vis = isfinite(t);
+            if (!all_seen) vis = vis && j >= lo && j < hi;
             x[r] = vis ? t : neg_inf();
             mt = fmaxf(mt, x[r]);
         }
         mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
         const float mn = fmaxf(m, mt);
-        const float alpha = m == neg_inf() ? 0.f : softmax_exp(m - mn);
+        const float ms = mn == neg_inf() ? 0.f : mn; /* nothing seen yet: keep the differences finite */
+        const float alpha = fast_exp2(m - ms);
         float ps = 0.f;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            x[r] = x[r] == neg_inf() ? 0.f : softmax_exp(x[r] - mn);
+            x[r] = fast_exp2(x[r] - ms);
             ps += x[r];
         }
         l = l * alpha + ps;
@@ -175,12 +394,18 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnProb *__restri
             for (int s = 0; s < 16; s++)
                 oacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf[b][s], x[s], oacc[b], 0, 0, 0);
         }
+        if (ktn < kt_hi) {
+            fetch_v(ktn);
+            K_PARK(ktn);
+        }
+        kt = ktn;
     }
 
     /* both halves of a column carry the same m, their sums add */
     l += __shfl_xor(l, 32, 64);
 
-    /* ---- merge the four waves ---- */
+    /* ---- merge the four waves (the merge area overlays the K tiles) ---- */
+    if (STAGE) __syncthreads();
     if (h == 0) {
         sm_m[wave][c] = m;
         sm_l[wave][c] = l;
@@ -197,11 +422,11 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnProb *__restri
     if (wave == 0) {
 #pragma unroll
         for (int w = 0; w < 4; w++) M = fmaxf(M, sm_m[w][c]);
+        const float Ms = M == neg_inf() ? 0.f : M;
         float f[4];
 #pragma unroll
         for (int w = 0; w < 4; w++) {
-            const float mw = sm_m[w][c];
-            f[w] = mw == neg_inf() ? 0.f : softmax_exp(mw - M);
+            f[w] = fast_exp2(sm_m[w][c] - Ms);
             L += sm_l[w][c] * f[w];
         }
         const float inv = L > 0.f ? 1.0f / L : 0.f;
@@ -221,7 +446,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnProb *__restri
                 for (int g = 0; g < 4; g++) {
                     const uint32_t d0 = b * 32 + 8 * g + 4 * h;
                     if (vec4) {
-                        if (d0 < p.hd)
+                        if (EXACT || d0 < p.hd)
                             *reinterpret_cast<float4 *>(orow + d0) =
                                 make_float4(oacc[b][4 * g + 0], oacc[b][4 * g + 1], oacc[b][4 * g + 2], oacc[b][4 * g + 3]);
                     } else {
@@ -233,7 +458,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnProb *__restri
             }
         }
         if (live && h == 0 && p.lse) {
-            p.lse[2 * (size_t)i + 0] = M;
+            p.lse[2 * (size_t)i + 0] = M * LN2; /* back to natural units */
             p.lse[2 * (size_t)i + 1] = L;
         }
     }
@@ -253,15 +478,17 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnProb *__restri
     float *wrow = p.weights + (size_t)i * p.nk;
     const bool wvec = (p.nk % 4u == 0u) && ((reinterpret_cast<uintptr_t>(p.weights) & 15u) == 0u);
     const uint32_t nkt = (p.nk + 31u) / 32u;
-    for (uint32_t kt = wave; kt < nkt; kt += 4u) {
-        const uint32_t k0 = kt * 32u;
+    for (uint32_t wt = wave; wt < nkt; wt += 4u) {
+        const uint32_t k0 = wt * 32u;
         float w[16];
 #pragma unroll
         for (int r = 0; r < 16; r++) w[r] = 0.f;
-        if (kt >= kt_lo && kt < kt_hi) {
-            float kf[HALF];
-            const uint32_t jr = min(k0 + c, p.nk - 1u);
-            load_half_row<HALF>(kf, p.k + (size_t)jr * p.k_stride, h * HALF, p.hd, vec4);
+        if (wt >= kt_lo && wt < kt_hi) {
+            K_REQUEST(wt);
+            if (STAGE) {
+                K_PARK(wt);
+                frag_from_lds<HD>(kf, my_k, h, c);
+            }
             floatx16 sacc;
 #pragma unroll
             for (int r = 0; r < 16; r++) sacc[r] = 0.f;
@@ -270,10 +497,11 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnProb *__restri
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const uint32_t j = k0 + acc_key(r, h);
-                float t = sacc[r] * p.scale;
-                if (mrow) t += mrow[min(j, p.nk - 1u)];
+                float t;
+                if (DENSE) t = (sacc[r] * p.scale + mrow[min(j, p.nk - 1u)]) * LOG2E;
+                else t = sacc[r] * scale2;
                 const bool vis = j >= lo && j < hi && isfinite(t);
-                w[r] = vis ? softmax_exp(t - M) * invL : 0.f;
+                w[r] = vis ? fast_exp2(t - M) * invL : 0.f;
             }
         }
         if (live) {
@@ -294,16 +522,29 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnProb *__restri
     }
 }
 
-template <int HD>
-void launch_mfma(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t ntiles, const AttnProb *single,
-                 hipStream_t s) {
-    if (single) {
-        blt_launch("attn_mfma", attn_mfma_kernel<HD, true>, dim3(ntiles), dim3(256), 0, s, dprobs, dtiles, *single);
-    } else {
-        AttnProb none;
-        __builtin_memset(&none, 0, sizeof(none));
-        blt_launch("attn_mfma", attn_mfma_kernel<HD, false>, dim3(ntiles), dim3(256), 0, s, dprobs, dtiles, none);
-    }
+#undef K_REQUEST
+#undef K_PARK
+
+template <int HD, int SRC>
+void launch_variant(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t nblocks, const AttnAffine &aff,
+                    bool exact, bool dense, hipStream_t s) {
+    const dim3 grid(nblocks), block(256);
+    if (exact && dense)
+        blt_launch("attn_mfma", attn_mfma_kernel<HD, SRC, true, true>, grid, block, 0, s, dprobs, dtiles, aff);
+    else if (exact)
+        blt_launch("attn_mfma", attn_mfma_kernel<HD, SRC, true, false>, grid, block, 0, s, dprobs, dtiles, aff);
+    else if (dense)
+        blt_launch("attn_mfma", attn_mfma_kernel<HD, SRC, false, true>, grid, block, 0, s, dprobs, dtiles, aff);
+    else
+        blt_launch("attn_mfma", attn_mfma_kernel<HD, SRC, false, false>, grid, block, 0, s, dprobs, dtiles, aff);
+}
+
+template <int SRC>
+void launch_hd(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t nblocks, const AttnAffine &aff, uint32_t hd,
+               bool vec4, bool dense, hipStream_t s) {
+    if (hd <= 32u) launch_variant<32, SRC>(dprobs, dtiles, nblocks, aff, vec4 && hd == 32u, dense, s);
+    else if (hd <= 64u) launch_variant<64, SRC>(dprobs, dtiles, nblocks, aff, vec4 && hd == 64u, dense, s);
+    else launch_variant<128, SRC>(dprobs, dtiles, nblocks, aff, vec4 && hd == 128u, dense, s);
 }
 
 } // namespace
@@ -349,17 +590,29 @@ void attn_mfma_make_tiles(const AttnProb *host, uint32_t base, uint32_t count, s
     for (const Item &it : items) tiles.push_back(it.t);
 }
 
-void attn_mfma_launch(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t ntiles, uint32_t hd, hipStream_t s) {
+/* Tile-list launch: every problem of the list has head_dim hd; `vec4` and
+ * `dense` must hold for all of them (the caller buckets by these). */
+void attn_mfma_launch(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t ntiles, uint32_t hd, bool vec4,
+                      bool dense, hipStream_t s) {
     if (ntiles == 0) return;
-    if (hd <= 32u) launch_mfma<32>(dprobs, dtiles, ntiles, nullptr, s);
-    else if (hd <= 64u) launch_mfma<64>(dprobs, dtiles, ntiles, nullptr, s);
-    else launch_mfma<128>(dprobs, dtiles, ntiles, nullptr, s);
+    AttnAffine none;
+    __builtin_memset(&none, 0, sizeof(none));
+    launch_hd<SRC_TILES>(dprobs, dtiles, ntiles, none, hd, vec4, dense, s);
 }
 
 void attn_mfma_launch_single(const AttnProb &single, hipStream_t s) {
     const uint32_t ntiles = (single.nq + 31u) / 32u;
     if (ntiles == 0) return;
-    if (single.hd <= 32u) launch_mfma<32>(nullptr, nullptr, ntiles, &single, s);
-    else if (single.hd <= 64u) launch_mfma<64>(nullptr, nullptr, ntiles, &single, s);
-    else launch_mfma<128>(nullptr, nullptr, ntiles, &single, s);
+    AttnAffine a;
+    __builtin_memset(&a, 0, sizeof(a));
+    a.first = single;
+    launch_hd<SRC_SINGLE>(nullptr, nullptr, ntiles, a, single.hd, (single.flags & ATTN_FLAG_VEC4) != 0,
+                          single.vis == ATTN_VIS_DENSE, s);
+}
+
+void attn_mfma_launch_affine(const AttnAffine &aff, hipStream_t s) {
+    const uint32_t blocks = aff.count * aff.nqt;
+    if (blocks == 0) return;
+    launch_hd<SRC_AFFINE>(nullptr, nullptr, blocks, aff, aff.first.hd, (aff.first.flags & ATTN_FLAG_VEC4) != 0,
+                          aff.first.vis == ATTN_VIS_DENSE, s);
 }

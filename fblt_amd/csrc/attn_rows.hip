@@ -81,45 +81,68 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const AttnProb *__restri
         o[t] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
 
-    /* the wave walks the union of its rows' ranges; each group ignores keys
-     * outside its own range */
-    uint32_t wlo = lo, whi = hi;
-    if (lo == hi) {
-        wlo = 0xFFFFFFFFu;
-        whi = 0;
-    }
+    /* every group walks its own range, U keys per trip with all 2*U*T loads
+     * of the trip issued before any arithmetic; the wave makes as many trips
+     * as its longest row needs */
+    constexpr int U = T > 2 ? 1 : 4; /* very wide heads keep one key in flight: registers */
+    uint32_t trips = (hi - lo + U - 1) / U;
 #pragma unroll
-    for (int off = G; off < 64; off <<= 1) {
-        wlo = min(wlo, (uint32_t)__shfl_xor((int)wlo, off, 64));
-        whi = max(whi, (uint32_t)__shfl_xor((int)whi, off, 64));
-    }
+    for (int off = G; off < 64; off <<= 1) trips = max(trips, (uint32_t)__shfl_xor((int)trips, off, 64));
 
     float m = neg_inf(), l = 0.f;
     const float *mrow = p.vis == ATTN_VIS_DENSE ? p.mask + (size_t)i * p.nk : nullptr;
+    const uint32_t last = hi > lo ? hi - 1u : 0u; /* a readable key of this row (row 0 when it has none) */
 
-    for (uint32_t j = wlo; j < whi; j++) {
-        const bool mine = j >= lo && j < hi;
-        const uint32_t jj = mine ? j : lo; /* lo < nk whenever the row has keys; else unused */
-        const float *krow = p.k + (size_t)(hi > lo ? jj : 0) * p.k_stride;
-        float part = 0.f;
+    for (uint32_t trip = 0; trip < trips; trip++) {
+        float4 kk[U][T], vv[U][T];
+        float bias[U];
+        uint32_t jj[U];
 #pragma unroll
-        for (int t = 0; t < T; t++) part += dot4(q[t], load4(krow, 4u * (g + G * t), p.hd, vec4));
-        float x = group_sum<G>(part) * p.scale;
-        if (mrow) x += mrow[hi > lo ? jj : 0];
-        const bool take = mine && isfinite(x);
-        if (take) {
-            const float mn = fmaxf(m, x);
-            const float a = softmax_exp(m - mn);
-            const float w = softmax_exp(x - mn);
-            l = l * a + w;
-            const float *vrow = p.v + (size_t)jj * p.v_stride;
+        for (int u = 0; u < U; u++) {
+            jj[u] = lo + trip * U + u;
+            const uint32_t jr = p.nk ? min(min(jj[u], last), p.nk - 1u) : 0u;
+            const float *krow = p.k + (size_t)jr * p.k_stride;
+            const float *vrow = p.v + (size_t)jr * p.v_stride;
 #pragma unroll
             for (int t = 0; t < T; t++) {
-                const float4 v = load4(vrow, 4u * (g + G * t), p.hd, vec4);
-                o[t].x = o[t].x * a + w * v.x;
-                o[t].y = o[t].y * a + w * v.y;
-                o[t].z = o[t].z * a + w * v.z;
-                o[t].w = o[t].w * a + w * v.w;
+                kk[u][t] = load4(krow, 4u * (g + G * t), p.hd, vec4);
+                vv[u][t] = load4(vrow, 4u * (g + G * t), p.hd, vec4);
+            }
+            bias[u] = mrow ? mrow[jr] : 0.f;
+        }
+        float x[U];
+        float mt = neg_inf();
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            float part = 0.f;
+#pragma unroll
+            for (int t = 0; t < T; t++) part += dot4(q[t], kk[u][t]);
+            const float sc = group_sum<G>(part) * p.scale + bias[u];
+            x[u] = (jj[u] < hi && isfinite(sc)) ? sc : neg_inf();
+            mt = fmaxf(mt, x[u]);
+        }
+        if (mt != neg_inf()) { /* uniform per group */
+            const float mn = fmaxf(m, mt);
+            const float a = softmax_exp(m - mn);
+            l *= a;
+#pragma unroll
+            for (int t = 0; t < T; t++) {
+                o[t].x *= a;
+                o[t].y *= a;
+                o[t].z *= a;
+                o[t].w *= a;
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const float w = softmax_exp(x[u] - mn); /* exp(-inf) = 0 for keys not taken */
+                l += w;
+#pragma unroll
+                for (int t = 0; t < T; t++) {
+                    o[t].x += w * vv[u][t].x;
+                    o[t].y += w * vv[u][t].y;
+                    o[t].z += w * vv[u][t].z;
+                    o[t].w += w * vv[u][t].w;
+                }
             }
             m = mn;
         }
