@@ -26,40 +26,14 @@
 #include "blt_fatal.h"
 #include "hip_check.h"
 #include "attn_device.h"
+#include "kv_step.h"
 #include "launch.h"
 
 #include <algorithm>
 #include <cstdlib>
+#include <cstring>
 
 namespace {
-
-constexpr int SUB = 32;        /* keys per sub-chunk (one wave, one head)       */
-constexpr int MAX_SPLITS = 16; /* workgroups per sequence                        */
-
-struct StepArgs {
-    float *cache_k;
-    float *cache_v;
-    uint32_t *self_len;
-    const float *q_rows;
-    const float *k_rows;
-    const float *v_rows;
-    float *combined;
-    float *partial;    /* [batch][splits][heads][NQ][hd + 2] */
-    uint32_t *tickets; /* [batch] */
-    uint32_t q_stride, k_stride, v_stride, out_stride;
-    uint32_t max_seq_len, embed_dim, num_heads;
-    uint32_t window;
-    uint32_t n;        /* new rows per sequence */
-    uint32_t q0;       /* first query row this launch handles */
-    uint32_t splits;   /* gridDim.x */
-    uint32_t span;     /* keys per split, a multiple of SUB */
-    uint32_t hpb;      /* heads per workgroup */
-    uint32_t slices;   /* waves per head in a workgroup */
-    float scale;
-    int block_kind;    /* every new row sees all keys */
-    int write_through; /* this launch stores the new rows into the cache */
-    int commit;        /* advance self_len when the sequence is done */
-};
 
 template <int G>
 __device__ __forceinline__ float group_sum(float x) {
@@ -69,15 +43,6 @@ __device__ __forceinline__ float group_sum(float x) {
 }
 
 __device__ __forceinline__ float dot4(float4 a, float4 b) { return a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w; }
-
-/* Device-scope store / load of data another workgroup (possibly on another
- * die of the package) reads within the same launch. */
-__device__ __forceinline__ void publish(float *p, float x) {
-    __hip_atomic_store(p, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ float observe(const float *p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 
 /* G lanes per key (head_dim = 4*G), NQ query rows per launch, at most WAVES
  * waves per workgroup. */
@@ -266,58 +231,7 @@ __global__ __launch_bounds__(64 * WAVES) void kv_step_kernel(StepArgs a) {
         }
     }
 
-    if (a.splits == 1u && gridDim.z == 1u) {
-        if (a.commit && threadIdx.x == 0) a.self_len[b] = nk;
-        return;
-    }
-
-    /* ---- ticket: the last workgroup of the sequence merges the splits ----
-     * The per-split states were stored with device-scope write-through stores
-     * and are read back with device-scope loads, so they never sit dirty or
-     * stale in one die's L2 and no cache write-back or invalidate is needed;
-     * the barrier's wait on outstanding memory operations orders the stores
-     * before this workgroup's ticket. */
-    __syncthreads();
-    if (threadIdx.x == 0) sm_ticket = __hip_atomic_fetch_add(&a.tickets[b], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    if (sm_ticket != gridDim.x * gridDim.z - 1u) return;
-
-    if (a.splits > 1u) {
-        const uint32_t all = a.num_heads * NQ * HD;
-        const size_t sstride = (size_t)a.num_heads * NQ * (HD + 2);
-        for (uint32_t t = threadIdx.x; t < all; t += blockDim.x) {
-            const uint32_t d = t % HD;
-            const uint32_t r = (t / HD) % NQ;
-            const uint32_t hh = t / (HD * NQ);
-            const uint32_t qi = a.q0 + r;
-            if (qi >= a.n) continue;
-            const float *base = a.partial + (((size_t)b * a.splits * a.num_heads + hh) * NQ + r) * (HD + 2);
-            float pm[MAX_SPLITS], pl[MAX_SPLITS], po[MAX_SPLITS];
-#pragma unroll
-            for (int s = 0; s < MAX_SPLITS; s++) {
-                const bool on = (uint32_t)s < a.splits;
-                const float *ps = base + (on ? s : 0) * sstride;
-                pm[s] = on ? observe(ps + HD) : neg_inf();
-                pl[s] = on ? observe(ps + HD + 1) : 0.f;
-                po[s] = on ? observe(ps + d) : 0.f;
-            }
-            float M = neg_inf();
-#pragma unroll
-            for (int s = 0; s < MAX_SPLITS; s++) M = fmaxf(M, pm[s]);
-            float L = 0.f, acc = 0.f;
-#pragma unroll
-            for (int s = 0; s < MAX_SPLITS; s++) {
-                const float f = pm[s] == neg_inf() ? 0.f : softmax_exp(pm[s] - M);
-                L += pl[s] * f;
-                acc += po[s] * f;
-            }
-            a.combined[((size_t)b * a.n + qi) * a.out_stride + hh * HD + d] = L > 0.f ? acc / L : 0.f;
-        }
-    }
-    if (threadIdx.x == 0) {
-        a.tickets[b] = 0u;
-        if (a.commit) a.self_len[b] = nk;
-    }
+    kv_finish_sequence<HD>(a, (uint32_t)NQ, b, nk, &sm_ticket);
 }
 
 /* scratch the family owns: per-split softmax states and per-sequence tickets */
@@ -433,7 +347,7 @@ extern "C" void blt_kv_attend_step_hip(const blt_kv_attn_cache *cache, const flo
     a.span = (uint32_t)(span_subs * SUB);
 
     Scratch &sc = scratch();
-    const size_t need = cache->batch * (size_t)MAX_SPLITS * H * 16u * (hd + 2);
+    const size_t need = cache->batch * (size_t)MAX_SPLITS * H * 32u * (hd + 2); /* 32 = widest query block */
     if (need > sc.partial_floats) {
         if (sc.partial) {
             HIP_CHECK(hipDeviceSynchronize());
@@ -454,9 +368,34 @@ extern "C" void blt_kv_attend_step_hip(const blt_kv_attn_cache *cache, const flo
     a.partial = sc.partial;
     a.tickets = sc.tickets;
 
-    /* query rows go in slices of at most 16; every slice reads the new rows
-     * from the inputs, so only the first one stores them and only the last
-     * one may advance the lengths */
+    /* Blocks of five or more rows go to the matrix-core kernel (one launch for
+     * up to 32 rows; its cost does not depend on the row count) where it takes
+     * the head_dim; shorter blocks, single rows and the shapes it does not
+     * take go to the VALU kernel in slices of at most 16 rows.
+     * Every launch reads the new rows from the inputs, so only the first one
+     * stores them and only the last one may advance the lengths.
+     * BLT_HIP_BLOCK_KERNEL=valu|mfma pins the choice (tuning and test hook). */
+    static const int pinned = [] {
+        const char *e = getenv("BLT_HIP_BLOCK_KERNEL");
+        return e && strcmp(e, "valu") == 0 ? 1 : e && strcmp(e, "mfma") == 0 ? 2 : 0;
+    }();
+    const bool want_mfma = pinned == 2 || (pinned == 0 && a.n >= 5u);
+    if (want_mfma && (hd == 32 || hd == 64)) {
+        /* the block kernel merges slices inside the workgroup, so it wants few,
+         * long spans: just enough workgroups to cover the compute units */
+        const size_t zblocks = (H + 1) / 2;
+        size_t bs = span_env > 0 ? (subs + span_env - 1) / span_env : (256 + cache->batch * zblocks - 1) / (cache->batch * zblocks);
+        bs = std::max<size_t>(1, std::min<size_t>(std::min<size_t>(bs, MAX_SPLITS), (subs + 3) / 4));
+        const size_t bspan = (subs + bs - 1) / bs;
+        a.splits = (uint32_t)((subs + bspan - 1) / bspan);
+        a.span = (uint32_t)(bspan * SUB);
+        a.q0 = 0;
+        a.write_through = 1;
+        a.commit = commit;
+        kv_block_mfma_launch(a, (uint32_t)cache->batch, (uint32_t)hd, 0);
+        HIP_CHECK_LAUNCH("blt_kv_attend_step");
+        return;
+    }
     for (uint32_t q0 = 0; q0 < a.n; q0 += 16u) {
         const uint32_t nq = std::min<uint32_t>(16u, a.n - q0);
         a.q0 = q0;

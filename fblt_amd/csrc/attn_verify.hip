@@ -1,0 +1,304 @@
+/*
+ * Block kernel of the KV-cache step: a block of n query rows per sequence
+ * (BLT-D/DV draft and verify blocks, chunked prefill) against the cached
+ * prefix plus the n new rows, on the fp32 matrix cores.
+ *
+ * Same split-KV frame as the decode kernel (a workgroup owns one contiguous
+ * span of a sequence's keys, its waves are the heads, per-split softmax states
+ * are merged by the last workgroup of the sequence), but the inner product of
+ * a 32-key sub-chunk with all query rows of the block is one transposed MFMA
+ * tile, exactly as in the prefill kernel:
+ *
+ *   S^T[key, query] = K Q^T      (32 x 32 x head_dim,  v_mfma_f32_32x32x2_f32)
+ *   O^T[d,   query] += V^T P^T   (head_dim x 32 x 32)
+ *
+ * The block's query rows (at most 32) are the N dimension of both products,
+ * so K and V stream through once for the whole block; rows beyond n are
+ * padding and never stored.  K rows are read coalesced and turned into MFMA
+ * fragments through a per-wave LDS tile; V rows are read one dword per lane
+ * (32 lanes = one 128-byte row segment).  The kernel is HBM-bound: ~8*head_dim
+ * bytes of K/V per 2*head_dim MFMAs of a sub-chunk.
+ */
+#include "blt_hip.h"
+#include "blt_fatal.h"
+#include "hip_check.h"
+#include "attn_device.h"
+#include "kv_step.h"
+#include "launch.h"
+
+#include <algorithm>
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int SLOTS = 32; /* query capacity of a launch = MFMA tile width */
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+
+__device__ __forceinline__ constexpr uint32_t acc_key(uint32_t r, uint32_t h) { return 8u * (r >> 2) + 4u * h + (r & 3u); }
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+/* One wavefront per (head, slice): blockDim.x = 64 * hpb * slices, head =
+ * blockIdx.z * hpb + wave % hpb, slice = wave / hpb.  The slices of a head
+ * take the span's 32-key sub-chunks round-robin and merge through LDS. */
+template <int HD, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void kv_block_mfma_kernel(StepArgs a) {
+    constexpr int HALF = HD / 2;
+    constexpr int DB = HD / 32;
+    constexpr int ROW = HD + 4;
+    constexpr int PR = HD + 2;  /* a parked result row: HD columns, max, sum; 32 * PR fits a K tile */
+    constexpr int LPR = HD / 4; /* lanes per row when a wave moves a K tile, 16 bytes each */
+
+    __shared__ __attribute__((aligned(16))) float sm_k[WAVES][32 * ROW];
+    __shared__ uint32_t sm_ticket;
+
+    const uint32_t b = blockIdx.y;
+    const uint32_t split = blockIdx.x;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t slice = wave / a.hpb;
+    const uint32_t head = blockIdx.z * a.hpb + wave % a.hpb;
+    const bool head_ok = head < a.num_heads;
+    const uint32_t hsafe = head_ok ? head : 0u;
+    const uint32_t h = lane >> 5;
+    const uint32_t c = lane & 31u;
+
+    const uint32_t len = a.self_len[b];
+    const uint32_t nk = len + a.n;
+    const size_t slab = (size_t)b * a.max_seq_len;
+    const uint32_t k_begin = split * a.span;
+    const uint32_t k_end = min(k_begin + a.span, nk);
+    const size_t newrow0 = (size_t)b * a.n;
+
+    /* query fragment: row c of the block (clamped), floats [h*HALF, (h+1)*HALF) of the head */
+    const uint32_t qi = a.q0 + c;
+    const bool q_ok = qi < a.n;
+    float qf[HALF];
+    {
+        const float *qrow = a.q_rows + (newrow0 + min(qi, a.n - 1u)) * a.q_stride + hsafe * HD + h * HALF;
+#pragma unroll
+        for (int s = 0; s < HALF; s += 4) {
+            const float4 t = *reinterpret_cast<const float4 *>(qrow + s);
+            qf[s + 0] = t.x, qf[s + 1] = t.y, qf[s + 2] = t.z, qf[s + 3] = t.w;
+        }
+    }
+    /* keys this lane's query sees within the span, as [vis_lo, vis_lo + vis_len):
+     * causal rows see keys up to their own position (kv_cache.c:229-236, with
+     * the local window cut), block rows see everything; padding rows nothing */
+    uint32_t vis_lo = 0, vis_hi = k_end;
+    if (!a.block_kind) {
+        const uint32_t qpos = len + qi; /* absolute position of this lane's query */
+        vis_hi = min(vis_hi, qpos + 1u);
+        if (a.window > 0u && qpos + 1u > a.window) vis_lo = qpos + 1u - a.window;
+    }
+    if (!q_ok) vis_hi = 0;
+    const uint32_t vis_len = vis_hi > vis_lo ? vis_hi - vis_lo : 0u;
+    const float scale2 = a.scale * LOG2E;
+
+    floatx16 oacc[DB];
+#pragma unroll
+    for (int d = 0; d < DB; d++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) oacc[d][r] = 0.f;
+    float m = neg_inf(), l = 0.f;
+
+    float *my_k = sm_k[wave];
+    float kg[HALF]; /* K tile in flight: HD/8 pieces of 16 bytes per lane */
+    float vf[DB][16];
+
+    /* row j of the sequence: cached rows come from the slab, new rows from the step's inputs */
+    auto k_row = [&](uint32_t j) __attribute__((always_inline)) -> const float * {
+        return j < len ? a.cache_k + (slab + j) * a.embed_dim : a.k_rows + (newrow0 + (j - len)) * a.k_stride;
+    };
+    auto v_row = [&](uint32_t j) __attribute__((always_inline)) -> const float * {
+        return j < len ? a.cache_v + (slab + j) * a.embed_dim : a.v_rows + (newrow0 + (j - len)) * a.v_stride;
+    };
+
+    /* A sub-chunk that lies entirely in the cached prefix (the common case) is
+     * addressed from one per-lane base with compile-time row steps; one that
+     * touches the new rows or the end of the sequence selects row by row. */
+#define REQUEST_K(c0_)                                                                                             \
+    do {                                                                                                           \
+        if ((c0_) + 32u <= len) {                                                                                  \
+            const float *kb_ = a.cache_k + (slab + (c0_) + lane / LPR) * a.embed_dim + hsafe * HD +                \
+                               4u * (lane % LPR);                                                                  \
+            _Pragma("unroll") for (int t = 0; t < HD / 8; t++) {                                                   \
+                const float4 x_ = *reinterpret_cast<const float4 *>(kb_ + (size_t)(t * (64 / LPR)) * a.embed_dim); \
+                kg[4 * t + 0] = x_.x, kg[4 * t + 1] = x_.y, kg[4 * t + 2] = x_.z, kg[4 * t + 3] = x_.w;            \
+            }                                                                                                      \
+        } else {                                                                                                   \
+            _Pragma("unroll") for (int t = 0; t < HD / 8; t++) {                                                   \
+                const uint32_t r_ = t * (64 / LPR) + lane / LPR;                                                   \
+                const uint32_t j_ = min((c0_) + r_, nk - 1u);                                                      \
+                const float4 x_ = *reinterpret_cast<const float4 *>(k_row(j_) + hsafe * HD + 4u * (lane % LPR));   \
+                kg[4 * t + 0] = x_.x, kg[4 * t + 1] = x_.y, kg[4 * t + 2] = x_.z, kg[4 * t + 3] = x_.w;            \
+            }                                                                                                      \
+        }                                                                                                          \
+    } while (0)
+#define REQUEST_V(c0_)                                                                                             \
+    do {                                                                                                           \
+        if ((c0_) + 32u <= len) {                                                                                  \
+            const float *vb_ = a.cache_v + (slab + (c0_) + 4u * h) * a.embed_dim + hsafe * HD + c;                 \
+            _Pragma("unroll") for (int s = 0; s < 16; s++) {                                                       \
+                const float *vr_ = vb_ + (size_t)(8 * (s >> 2) + (s & 3)) * a.embed_dim;                           \
+                _Pragma("unroll") for (int d = 0; d < DB; d++) vf[d][s] = vr_[32 * d];                             \
+            }                                                                                                      \
+        } else {                                                                                                   \
+            _Pragma("unroll") for (int s = 0; s < 16; s++) {                                                       \
+                const uint32_t j_ = min((c0_) + acc_key(s, h), nk - 1u);                                           \
+                const float *vr_ = v_row(j_) + hsafe * HD + c;                                                     \
+                _Pragma("unroll") for (int d = 0; d < DB; d++) vf[d][s] = vr_[32 * d];                             \
+            }                                                                                                      \
+        }                                                                                                          \
+    } while (0)
+
+    const uint32_t step = a.slices * 32u;
+    uint32_t c0 = k_begin + slice * 32u;
+    if (c0 < k_end) {
+        REQUEST_K(c0);
+        REQUEST_V(c0);
+    }
+    while (c0 < k_end) {
+        const uint32_t cn = c0 + step;
+
+        /* K tile: write-through of new rows, then LDS -> fragment (lane = key row) */
+#pragma unroll
+        for (int t = 0; t < HD / 8; t++) {
+            const uint32_t r = t * (64 / LPR) + lane / LPR;
+            const float4 piece = make_float4(kg[4 * t + 0], kg[4 * t + 1], kg[4 * t + 2], kg[4 * t + 3]);
+            const uint32_t j = c0 + r;
+            if (a.write_through && head_ok && c0 + 32u > len && j >= len && j < k_end)
+                *reinterpret_cast<float4 *>(a.cache_k + (slab + j) * a.embed_dim + head * HD + 4u * (lane % LPR)) = piece;
+            *reinterpret_cast<float4 *>(my_k + r * ROW + 4u * (lane % LPR)) = piece;
+        }
+        float kf[HALF];
+#pragma unroll
+        for (int s = 0; s < HALF; s += 4) {
+            const float4 t = *reinterpret_cast<const float4 *>(my_k + c * ROW + h * HALF + s);
+            kf[s + 0] = t.x, kf[s + 1] = t.y, kf[s + 2] = t.z, kf[s + 3] = t.w;
+        }
+        /* the next sub-chunk's K rows travel while this one is worked on */
+        if (cn < k_end) REQUEST_K(cn);
+
+        floatx16 sacc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) sacc[r] = 0.f;
+#pragma unroll
+        for (int s = 0; s < HALF; s++) sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[s], qf[s], sacc, 0, 0, 0);
+
+        float x[16];
+        float mt = neg_inf();
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const float t = sacc[r] * scale2;
+            /* one unsigned compare: vis_lo <= j < vis_lo + vis_len */
+            const bool vis = (c0 + acc_key(r, h) - vis_lo) < vis_len && isfinite(t);
+            x[r] = vis ? t : neg_inf();
+            mt = fmaxf(mt, x[r]);
+        }
+        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+        const float mn = fmaxf(m, mt);
+        const float ms = mn == neg_inf() ? 0.f : mn;
+        const float alpha = fast_exp2(m - ms);
+        float ps = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            x[r] = fast_exp2(x[r] - ms);
+            ps += x[r];
+        }
+        l = l * alpha + ps;
+        m = mn;
+#pragma unroll
+        for (int d = 0; d < DB; d++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[d][r] *= alpha;
+#pragma unroll
+            for (int s = 0; s < 16; s++) oacc[d] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf[d][s], x[s], oacc[d], 0, 0, 0);
+        }
+
+        /* V: write-through of new rows from the values just used, then the next sub-chunk's rows */
+        if (a.write_through && head_ok && c0 + 32u > len) {
+#pragma unroll
+            for (int s = 0; s < 16; s++) {
+                const uint32_t j = c0 + acc_key(s, h);
+                if (j >= len && j < k_end) {
+#pragma unroll
+                    for (int d = 0; d < DB; d++) a.cache_v[(slab + j) * a.embed_dim + head * HD + 32 * d + c] = vf[d][s];
+                }
+            }
+        }
+        if (cn < k_end) REQUEST_V(cn);
+        c0 = cn;
+    }
+#undef REQUEST_K
+#undef REQUEST_V
+
+    l += __shfl_xor(l, 32, 64);
+
+    /* lane (h, c) holds O^T[d = 32*db + acc_key(r, h)][query c].  The wave
+     * turns that into rows [query][HD columns, max, sum] in its LDS tile; then
+     * the workgroup merges the slices of each head with consecutive threads
+     * on consecutive floats of a row, which is also the order of the output
+     * rows and of the per-split records in the partial buffer. */
+#pragma unroll
+    for (int d = 0; d < DB; d++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) my_k[c * PR + 32 * d + acc_key(r, h)] = oacc[d][r];
+    if (h == 0) {
+        my_k[c * PR + HD + 0] = m * LN2; /* merges work in natural units */
+        my_k[c * PR + HD + 1] = l;
+    }
+    __syncthreads();
+
+    const uint32_t rows = a.n - a.q0 < (uint32_t)SLOTS ? a.n - a.q0 : (uint32_t)SLOTS;
+    const uint32_t cells = a.hpb * rows * PR;
+    for (uint32_t t = threadIdx.x; t < cells; t += blockDim.x) {
+        const uint32_t col = t % PR;
+        const uint32_t r = (t / PR) % rows;
+        const uint32_t hl = t / (PR * rows);
+        const uint32_t hh = blockIdx.z * a.hpb + hl;
+        if (hh >= a.num_heads) continue;
+        float M = neg_inf();
+        for (uint32_t s = 0; s < a.slices; s++) M = fmaxf(M, sm_k[s * a.hpb + hl][r * PR + HD]);
+        float L = 0.f, acc = 0.f;
+        for (uint32_t s = 0; s < a.slices; s++) {
+            const float *ps = sm_k[s * a.hpb + hl] + r * PR;
+            const float f = ps[HD] == neg_inf() ? 0.f : softmax_exp(ps[HD] - M);
+            L += ps[HD + 1] * f;
+            if (col < (uint32_t)HD) acc += ps[col] * f;
+        }
+        if (a.splits == 1u) {
+            if (col < (uint32_t)HD)
+                a.combined[(newrow0 + a.q0 + r) * a.out_stride + hh * HD + col] = L > 0.f ? acc / L : 0.f;
+        } else {
+            float *dst = a.partial + ((((size_t)b * a.splits + split) * a.num_heads + hh) * SLOTS + r) * PR;
+            publish(dst + col, col < (uint32_t)HD ? acc : (col == (uint32_t)HD ? M : L));
+        }
+    }
+
+    kv_finish_sequence<HD>(a, (uint32_t)SLOTS, b, nk, &sm_ticket);
+}
+
+template <int HD, int WAVES>
+void launch_block(StepArgs a, uint32_t batch, hipStream_t s) {
+    /* two heads per workgroup when there are several: the other waves are slices */
+    a.hpb = std::min<uint32_t>(a.num_heads, WAVES >= 4 ? 2u : 1u);
+    const uint32_t subs = (a.span + 31u) / 32u;
+    a.slices = std::max(1u, std::min<uint32_t>((uint32_t)WAVES / a.hpb, subs));
+    dim3 grid(a.splits, batch, (a.num_heads + a.hpb - 1) / a.hpb);
+    blt_launch("kv_block_mfma", kv_block_mfma_kernel<HD, WAVES>, grid, dim3(64 * a.hpb * a.slices), 0, s, a);
+}
+
+} // namespace
+
+/* Takes head_dim 32 and 64 (the K tiles of four waves fit the static LDS
+ * budget); the caller falls back to the VALU kernel otherwise.  Handles up to
+ * 32 query rows per launch: a.q0 .. a.q0 + 31. */
+bool kv_block_mfma_launch(const StepArgs &a, uint32_t batch, uint32_t head_dim, hipStream_t s) {
+    /* the per-wave K tiles bound the workgroup: 8 waves of 4.6 KB or 4 of 8.7 KB */
+    if (head_dim == 32u) launch_block<32, 8>(a, batch, s);
+    else if (head_dim == 64u) launch_block<64, 4>(a, batch, s);
+    else return false;
+    return true;
+}

@@ -1,0 +1,116 @@
+/*
+ * Shared by the two kernels behind blt_kv_attend_step_hip (the VALU decode
+ * kernel and the MFMA block kernel): the launch arguments, the device-scope
+ * publish/observe accessors for data that crosses workgroups inside one
+ * launch, and the ticket + merge that finishes a sequence.
+ */
+#ifndef FBLT_AMD_KV_STEP_H
+#define FBLT_AMD_KV_STEP_H
+
+#include "attn_device.h"
+
+constexpr int SUB = 32;        /* keys per sub-chunk (one wave, one head)       */
+constexpr int MAX_SPLITS = 16; /* workgroups per sequence                        */
+
+struct StepArgs {
+    float *cache_k;
+    float *cache_v;
+    uint32_t *self_len;
+    const float *q_rows;
+    const float *k_rows;
+    const float *v_rows;
+    float *combined;
+    float *partial;    /* [batch][splits][heads][NQ][hd + 2] */
+    uint32_t *tickets; /* [batch] */
+    uint32_t q_stride, k_stride, v_stride, out_stride;
+    uint32_t max_seq_len, embed_dim, num_heads;
+    uint32_t window;
+    uint32_t n;        /* new rows per sequence */
+    uint32_t q0;       /* first query row this launch handles */
+    uint32_t splits;   /* gridDim.x */
+    uint32_t span;     /* keys per split, a multiple of SUB */
+    uint32_t hpb;      /* heads per workgroup */
+    uint32_t slices;   /* waves per head in a workgroup */
+    float scale;
+    int block_kind;    /* every new row sees all keys */
+    int write_through; /* this launch stores the new rows into the cache */
+    int commit;        /* advance self_len when the sequence is done */
+};
+
+
+/* Device-scope store / load of data another workgroup (possibly on another
+ * die of the package) reads within the same launch. */
+__device__ __forceinline__ void publish(float *p, float x) {
+    __hip_atomic_store(p, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float observe(const float *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+/* Called by every thread of every workgroup of sequence b once its per-split
+ * state is published (splits > 1) or its output rows are written (splits ==
+ * 1).  The last workgroup of the sequence to arrive merges the splits into
+ * the output rows, re-arms the ticket and advances the sequence's length when
+ * the step commits.  `slots` is the query capacity of the partial layout
+ * [batch][splits][heads][slots][HD + 2] (max, sum in the two extra floats).
+ *
+ * The per-split states were stored with device-scope write-through stores and
+ * are read back with device-scope loads, so they never sit dirty or stale in
+ * one die's L2 and no cache write-back or invalidate is needed; the barrier's
+ * wait on outstanding memory operations orders the stores before this
+ * workgroup's ticket. */
+template <int HD>
+__device__ __forceinline__ void kv_finish_sequence(const StepArgs &a, uint32_t slots, uint32_t b, uint32_t nk,
+                                                   uint32_t *sm_ticket) {
+    if (a.splits == 1u && gridDim.z == 1u) {
+        if (a.commit && threadIdx.x == 0) a.self_len[b] = nk;
+        return;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0)
+        *sm_ticket = __hip_atomic_fetch_add(&a.tickets[b], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (*sm_ticket != gridDim.x * gridDim.z - 1u) return;
+
+    if (a.splits > 1u) {
+        const uint32_t all = a.num_heads * slots * HD;
+        const size_t sstride = (size_t)a.num_heads * slots * (HD + 2);
+        for (uint32_t t = threadIdx.x; t < all; t += blockDim.x) {
+            const uint32_t d = t % HD;
+            const uint32_t r = (t / HD) % slots;
+            const uint32_t hh = t / (HD * slots);
+            const uint32_t qi = a.q0 + r;
+            if (qi >= a.n) continue;
+            const float *base = a.partial + (((size_t)b * a.splits * a.num_heads + hh) * slots + r) * (HD + 2);
+            float pm[MAX_SPLITS], pl[MAX_SPLITS], po[MAX_SPLITS];
+#pragma unroll
+            for (int s = 0; s < MAX_SPLITS; s++) {
+                const bool on = (uint32_t)s < a.splits;
+                const float *ps = base + (on ? s : 0) * sstride;
+                pm[s] = on ? observe(ps + HD) : neg_inf();
+                pl[s] = on ? observe(ps + HD + 1) : 0.f;
+                po[s] = on ? observe(ps + d) : 0.f;
+            }
+            float M = neg_inf();
+#pragma unroll
+            for (int s = 0; s < MAX_SPLITS; s++) M = fmaxf(M, pm[s]);
+            float L = 0.f, acc = 0.f;
+#pragma unroll
+            for (int s = 0; s < MAX_SPLITS; s++) {
+                const float f = pm[s] == neg_inf() ? 0.f : softmax_exp(pm[s] - M);
+                L += pl[s] * f;
+                acc += po[s] * f;
+            }
+            a.combined[((size_t)b * a.n + qi) * a.out_stride + hh * HD + d] = L > 0.f ? acc / L : 0.f;
+        }
+    }
+    if (threadIdx.x == 0) {
+        a.tickets[b] = 0u;
+        if (a.commit) a.self_len[b] = nk;
+    }
+}
+
+/* launch of the MFMA block kernel (attn_verify.hip); false when it does not take the shape */
+bool kv_block_mfma_launch(const StepArgs &a, uint32_t batch, uint32_t head_dim, hipStream_t s);
+
+#endif

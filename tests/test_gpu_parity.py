@@ -409,3 +409,40 @@ def test_strided_copy_softmax_dot(oracle, dev):
     ta, tb = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
     got = lib.blt_vec_dot(abi.BLT_BACKEND_HIP, ta.data_ptr(), tb.data_ptr(), 777)
     assert abs(got - float(np.dot(a.astype(np.float64), b.astype(np.float64)))) < 1e-3
+
+
+@pytest.mark.parametrize("kernel", ["valu", "mfma"])
+@pytest.mark.parametrize("kind,n", [("block", 4), ("block", 16), ("causal", 3), ("causal", 12), ("block", 32)])
+def test_kv_step_kernel_families_agree(kernel, kind, n, oracle):
+    """Both kernels behind blt_kv_attend_step_hip (VALU and matrix-core) on the same step,
+    pinned through BLT_HIP_BLOCK_KERNEL in a fresh process (the hook is read once)."""
+    import subprocess
+    import sys
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = """
+import sys
+sys.path.insert(0, %r)
+import numpy as np
+from fblt_amd import workloads, runner
+from oracle import runner as orunner
+kind, n = %r, %d
+if kind == "block":
+    kw = workloads.config5(batch=9, B=n)
+else:
+    kw = workloads.config4(batch=9, steps=2, len_hi=150, max_seq_len=150 + 2 * n)
+    rs = np.random.RandomState(n)
+    kw.n = n
+    kw.q_new, kw.k_new, kw.v_new = (rs.randn(kw.steps, kw.batch * n, kw.E).astype(np.float32) for _ in range(3))
+ref_out, ref_k, ref_v = orunner.run_kv(kw)
+d = runner.DeviceKvWorkload(kw)
+d.run()
+out, ck, cv, lens = d.results()
+assert ck.tobytes() == ref_k.tobytes() and cv.tobytes() == ref_v.tobytes()
+err = np.abs(out.astype(np.float64) - ref_out)
+assert (err <= 1e-5 + 1e-4 * np.abs(ref_out)).all(), float(err.max())
+print("OK", float(err.max()))
+""" % (root, kind, n)
+    env = dict(os.environ, BLT_HIP_BLOCK_KERNEL=kernel)
+    p = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300, env=env)
+    assert p.returncode == 0 and "OK" in p.stdout, p.stdout + p.stderr
