@@ -24,9 +24,19 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 
-# HBM bytes per launch from `rocprofv3 --pmc` (FETCH_SIZE, WRITE_SIZE; see the
-# summaries under profiles/), None where not measured.
-MEASURED_TRAFFIC_BYTES = {}
+# HBM bytes per launch from two `rocprofv3 --pmc` runs (FETCH_SIZE, then
+# WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for
+# the plain 64 MiB streaming copy (--probe-copy-mib 64): x1.999 for FETCH_SIZE,
+# x1.000 for WRITE_SIZE.  The summaries under profiles/ hold the readings.
+MEASURED_TRAFFIC_BYTES = {
+    "c2_patch_block_causal": (6250.1 * 1.999 + 4096.0) * 1024,
+    "c1_local_decoder_causal": (715.0 * 1.999 + 256.0) * 1024,
+    "c3_encoder_cross": (4699.1 * 1.999 + 1024.0) * 1024,
+    "c4_kv_decode": (12157.2 * 1.999 + 664.4) * 1024,
+    "c5_block_verify_B4": (10250.3 * 1.999 + 2064.5) * 1024,
+    "c5_block_verify_B8": (10278.5 * 1.999 + 1977.3) * 1024,   # B = 8 and 16 were collected together
+    "c5_block_verify_B16": (10278.5 * 1.999 + 1977.3) * 1024,
+}
 
 
 def log(*a):
@@ -178,6 +188,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--only", default="", help="comma list of c1,c2,c3,c4,c5 (c2 always runs)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU budget of the headline workload")
+    ap.add_argument("--probe-copy-mib", type=int, default=0,
+                    help="only run the plain streaming copy of this many MiB --steps times (counter yardstick)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the workload shards by sequence "
@@ -187,6 +199,22 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU: the HIP attention backend has no CPU path")
     from fblt_amd import workloads
+
+    if args.probe_copy_mib:
+        from fblt_amd import api
+        lib = api.load()
+        nbytes = args.probe_copy_mib << 20
+        src = torch.ones(nbytes // 4, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            lib.blt_hip_stream_copy_probe(dst.data_ptr(), src.data_ptr(), nbytes)
+        lib.blt_backend_pass_sync_hip()
+        dt = time.perf_counter() - t0
+        print(json.dumps({"probe": "stream_copy", "bytes_in": nbytes, "bytes_out": nbytes, "launches": args.steps,
+                          "GBps_read_plus_write": 2.0 * nbytes * args.steps / dt / 1e9}), flush=True)
+        return
 
     only = set(x for x in args.only.split(",") if x)
     want = lambda c: not only or c in only

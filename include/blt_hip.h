@@ -207,6 +207,11 @@ typedef struct {
 void blt_hip_profile_begin(void);
 size_t blt_hip_profile_end(blt_hip_kernel_time *out, size_t capacity);
 
+/* Measurement yardstick: a plain device-to-device streaming copy of `bytes`
+ * (a multiple of 16) on the default stream.  Hardware-counter readings of the
+ * attention kernels are scaled by what the same counters read for this copy. */
+void blt_hip_stream_copy_probe(void *dst, const void *src, size_t bytes);
+
 /* Library build tag and the architecture its kernels were compiled for. */
 const char *blt_hip_build_info(void);
 
