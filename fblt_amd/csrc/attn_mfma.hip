@@ -177,8 +177,6 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnProb *__restri
     __shared__ float sm_l[4][32];
     __shared__ __attribute__((aligned(16))) float sm_q[Lds::Q_FLOATS > 0 ? Lds::Q_FLOATS : 4];
     __shared__ __attribute__((aligned(16))) float sm_body[Lds::BODY_FLOATS];
-    float(*sm_o)[HD][33] = reinterpret_cast<float(*)[HD][33]>(sm_body);
-
     uint32_t qtile;
     AttnProb p;
     if (SRC == SRC_TILES) {
@@ -404,22 +402,29 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnProb *__restri
     /* both halves of a column carry the same m, their sums add */
     l += __shfl_xor(l, 32, 64);
 
-    /* ---- merge the four waves (the merge area overlays the K tiles) ---- */
+    /* ---- merge the four waves (the merge area overlays the K tiles) ----
+     * QUARTER (head dims whose four partial outputs fit the LDS body): every
+     * wave parks its partial O^T and merges a quarter of the columns for all
+     * 32 rows, reading the four partials from LDS in its own fragment layout.
+     * Otherwise wave 0 merges the other three into its registers. */
+    constexpr bool QUARTER = 4 * HD * 33 <= Lds::BODY_FLOATS;
+    float(*sm_o)[HD][33] = reinterpret_cast<float(*)[HD][33]>(sm_body);
     if (STAGE) __syncthreads();
     if (h == 0) {
         sm_m[wave][c] = m;
         sm_l[wave][c] = l;
     }
-    if (wave > 0) {
+    if (QUARTER || wave > 0) {
+        const uint32_t slot = QUARTER ? wave : wave - 1u;
 #pragma unroll
         for (int b = 0; b < DB; b++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) sm_o[wave - 1][b * 32 + acc_key(r, h)][c] = oacc[b][r];
+            for (int r = 0; r < 16; r++) sm_o[slot][b * 32 + acc_key(r, h)][c] = oacc[b][r];
     }
     __syncthreads();
 
     float M = neg_inf(), L = 0.f;
-    if (wave == 0) {
+    if (QUARTER || wave == 0) {
 #pragma unroll
         for (int w = 0; w < 4; w++) M = fmaxf(M, sm_m[w][c]);
         const float Ms = M == neg_inf() ? 0.f : M;
@@ -431,33 +436,60 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnProb *__restri
         }
         const float inv = L > 0.f ? 1.0f / L : 0.f;
         float *orow = p.out + (size_t)i * p.out_stride;
+        if (QUARTER) {
+            /* DB * 4 groups of four consecutive columns; this wave takes DB of them */
 #pragma unroll
-        for (int b = 0; b < DB; b++) {
+            for (int k = 0; k < DB; k++) {
+                const uint32_t gid = wave * DB + k;
+                const uint32_t d0 = (gid >> 2) * 32u + 8u * (gid & 3u) + 4u * h;
+                float o4[4];
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const uint32_t d = b * 32 + acc_key(r, h);
-                float acc = oacc[b][r] * f[0];
+                for (int e = 0; e < 4; e++) {
+                    float acc = 0.f;
 #pragma unroll
-                for (int w = 1; w < 4; w++) acc += sm_o[w - 1][d][c] * f[w];
-                oacc[b][r] = acc * inv;
-            }
-            if (live) {
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const uint32_t d0 = b * 32 + 8 * g + 4 * h;
+                    for (int w = 0; w < 4; w++) acc += sm_o[w][d0 + e][c] * f[w];
+                    o4[e] = acc * inv;
+                }
+                if (live) {
                     if (vec4) {
                         if (EXACT || d0 < p.hd)
-                            *reinterpret_cast<float4 *>(orow + d0) =
-                                make_float4(oacc[b][4 * g + 0], oacc[b][4 * g + 1], oacc[b][4 * g + 2], oacc[b][4 * g + 3]);
+                            *reinterpret_cast<float4 *>(orow + d0) = make_float4(o4[0], o4[1], o4[2], o4[3]);
                     } else {
 #pragma unroll
                         for (int e = 0; e < 4; e++)
-                            if (d0 + e < p.hd) orow[d0 + e] = oacc[b][4 * g + e];
+                            if (d0 + e < p.hd) orow[d0 + e] = o4[e];
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int b = 0; b < DB; b++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const uint32_t d = b * 32 + acc_key(r, h);
+                    float acc = oacc[b][r] * f[0];
+#pragma unroll
+                    for (int w = 1; w < 4; w++) acc += sm_o[w - 1][d][c] * f[w];
+                    oacc[b][r] = acc * inv;
+                }
+                if (live) {
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const uint32_t d0 = b * 32 + 8 * g + 4 * h;
+                        if (vec4) {
+                            if (EXACT || d0 < p.hd)
+                                *reinterpret_cast<float4 *>(orow + d0) = make_float4(
+                                    oacc[b][4 * g + 0], oacc[b][4 * g + 1], oacc[b][4 * g + 2], oacc[b][4 * g + 3]);
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                if (d0 + e < p.hd) orow[d0 + e] = oacc[b][4 * g + e];
+                        }
                     }
                 }
             }
         }
-        if (live && h == 0 && p.lse) {
+        if (wave == 0 && live && h == 0 && p.lse) {
             p.lse[2 * (size_t)i + 0] = M * LN2; /* back to natural units */
             p.lse[2 * (size_t)i + 1] = L;
         }
