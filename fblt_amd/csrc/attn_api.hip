@@ -2,7 +2,7 @@
  * Entry points of the attention forward path: the per-head device twin the
  * reference's dispatcher binds, the whole-batch launch and the resident plan.
  * Host code only (argument checks, descriptor translation, kernel choice);
- * the kernels live in attn_rows.hip and attn_mfma.hip.
+ * the kernels live in attn_rows.hip, attn_mfma.hip and attn_wide.hip.
  */
 #include "blt_hip.h"
 #include "blt_fatal.h"
@@ -17,7 +17,7 @@
 namespace {
 
 /* Kernel family a problem is routed to. */
-enum Family : uint32_t { FAM_ROWS = 0, FAM_MFMA = 1, FAM_COUNT = 2 };
+enum Family : uint32_t { FAM_ROWS = 0, FAM_MFMA = 1, FAM_WIDE = 2 };
 
 struct Bucket {
     Family fam;
@@ -103,13 +103,14 @@ AttnProb translate(const blt_attention_problem &pr, bool need_score_buffer, cons
     return d;
 }
 
-/* BLT_HIP_ATTN_FAMILY=rows|mfma pins the kernel family wherever the shape
- * allows it (tuning and test hook); unset or anything else = automatic. */
+/* BLT_HIP_ATTN_FAMILY=rows|mfma|wide pins the kernel family wherever the
+ * shape allows it (tuning and test hook); unset or anything else = automatic. */
 int family_override() {
     static const int cached = [] {
         const char *e = getenv("BLT_HIP_ATTN_FAMILY");
         if (e && std::strcmp(e, "rows") == 0) return 1;
         if (e && std::strcmp(e, "mfma") == 0) return 2;
+        if (e && std::strcmp(e, "wide") == 0) return 3;
         return 0;
     }();
     return cached;
@@ -118,9 +119,34 @@ int family_override() {
 Family choose_family(const AttnProb &d) {
     const int forced = family_override();
     if (forced == 1) return FAM_ROWS;
-    if (forced == 2 && attn_mfma_can(d)) return FAM_MFMA;
+    if (forced >= 2 && attn_mfma_can(d)) return FAM_MFMA;
     if (attn_mfma_takes(d)) return FAM_MFMA;
     return FAM_ROWS;
+}
+
+/* The wide kernel pays off once its 128-row work items fill the chip a few
+ * times over; below that the latency-oriented mfma kernel, which splits the
+ * keys of a 32-row tile over four waves, finishes first.
+ * BLT_HIP_WIDE_MIN_GROUPS overrides the threshold. */
+uint32_t wide_min_groups() {
+    static const uint32_t cached = [] {
+        const char *e = getenv("BLT_HIP_WIDE_MIN_GROUPS");
+        const long v = e ? std::atol(e) : 0;
+        return v > 0 ? (uint32_t)v : 1024u;
+    }();
+    return cached;
+}
+
+/* Do problems p[0..n), all routed to the mfma family, go to the wide kernel instead? */
+bool choose_wide(const AttnProb *p, uint32_t n) {
+    const int forced = family_override();
+    if (forced == 1 || forced == 2) return false;
+    uint64_t groups = 0;
+    for (uint32_t i = 0; i < n; i++) {
+        if (!attn_wide_can(p[i])) return false;
+        groups += attn_wide_groups(p[i]);
+    }
+    return forced == 3 || groups >= wide_min_groups();
 }
 
 /* Element distance between two float pointers (either both NULL or both set). */
@@ -251,20 +277,32 @@ void plan_build(blt_attention_plan &pl, const blt_attention_problem *problems, s
     }
     for (Bucket &b : pl.buckets) {
         if (b.fam != FAM_MFMA) continue;
+        if (choose_wide(pl.host.data() + b.base, b.count)) b.fam = FAM_WIDE;
         b.affine = detect_affine(pl.host.data() + b.base, b.count, b.aff);
-        if (b.affine) continue; /* no descriptor or tile memory needed */
+        if (b.affine) {
+            /* no descriptor or tile memory needed */
+            if (b.fam == FAM_WIDE) b.aff.nqt = attn_wide_groups(b.aff.first);
+            continue;
+        }
         b.tile_base = (uint32_t)pl.tiles.size();
-        attn_mfma_make_tiles(pl.host.data(), b.base, b.count, pl.tiles);
+        if (b.fam == FAM_WIDE) attn_wide_make_tiles(pl.host.data(), b.base, b.count, pl.tiles);
+        else attn_mfma_make_tiles(pl.host.data(), b.base, b.count, pl.tiles);
         b.tiles = (uint32_t)pl.tiles.size() - b.tile_base;
     }
-    bool any_mfma = false, any_rows = false;
-    for (const Bucket &b : pl.buckets) (b.fam == FAM_MFMA ? any_mfma : any_rows) = true;
-    pl.kernel = any_mfma && any_rows ? "mfma+rows" : any_mfma ? "mfma" : any_rows ? "rows" : "none";
+    bool any[3] = {false, false, false};
+    for (const Bucket &b : pl.buckets) any[b.fam] = true;
+    static const char *const names[8] = {"none",      "rows",      "mfma",      "mfma+rows",
+                                         "wide",      "wide+rows", "wide+mfma", "wide+mfma+rows"};
+    pl.kernel = names[(any[FAM_ROWS] ? 1 : 0) | (any[FAM_MFMA] ? 2 : 0) | (any[FAM_WIDE] ? 4 : 0)];
 }
 
 void plan_launch(const blt_attention_plan &pl, const AttnProb *dev, const AttnTile *dev_tiles) {
     for (const Bucket &b : pl.buckets) {
-        if (b.fam == FAM_MFMA && b.affine)
+        if (b.fam == FAM_WIDE && b.affine)
+            attn_wide_launch_affine(b.aff, 0);
+        else if (b.fam == FAM_WIDE)
+            attn_wide_launch(dev, dev_tiles + b.tile_base, b.tiles, b.hd, b.dense, 0);
+        else if (b.fam == FAM_MFMA && b.affine)
             attn_mfma_launch_affine(b.aff, 0);
         else if (b.fam == FAM_MFMA)
             attn_mfma_launch(dev, dev_tiles + b.tile_base, b.tiles, b.hd, b.vec4, b.dense, 0);
@@ -334,7 +372,9 @@ extern "C" void blt_attention_head_core_hip(blt_backend backend, const blt_atten
     /* one problem: the descriptor travels as a kernel argument, nothing is staged */
     const AttnProb d = translate(pr, true, "blt_attention_head_core");
     if (d.nq == 0) return;
-    if (choose_family(d) == FAM_MFMA) attn_mfma_launch_single(d, 0);
+    const Family f = choose_family(d);
+    if (f == FAM_MFMA && choose_wide(&d, 1)) attn_wide_launch_single(d, 0);
+    else if (f == FAM_MFMA) attn_mfma_launch_single(d, 0);
     else attn_rows_launch_single(d, 0);
     HIP_CHECK_LAUNCH("blt_attention_head_core");
 }

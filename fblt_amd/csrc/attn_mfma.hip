@@ -35,17 +35,13 @@
  */
 #include "attn_device.h"
 #include "attn_launch.h"
+#include "attn_tile.h"
 #include "hip_check.h"
 #include "launch.h"
 
 #include <algorithm>
 
 namespace {
-
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-
-/* key (within a 32-key tile) that accumulator register r of lane half h holds */
-__device__ __forceinline__ constexpr uint32_t acc_key(uint32_t r, uint32_t h) { return 8u * (r >> 2) + 4u * h + (r & 3u); }
 
 /* HALF = HD/2 floats of one row starting at element d0.  EXACT: 16-byte
  * aligned rows and head_dim == HD, so no element needs a guard. */
@@ -76,19 +72,6 @@ __device__ __forceinline__ void load_half_row(float (&dst)[HALF], const float *r
         for (int s = 0; s < HALF; s++) dst[s] = d0 + s < hd ? row[d0 + s] : 0.f;
     }
 }
-
-/* where a workgroup finds its problem */
-enum : int {
-    SRC_TILES = 0,  /* device arrays: tiles[blockIdx.x] -> probs[tile.prob]           */
-    SRC_SINGLE = 1, /* one problem in the kernel arguments                            */
-    SRC_AFFINE = 2  /* kernel arguments: first problem + (sequence, head) strides     */
-};
-
-constexpr float LOG2E = 1.4426950408889634f;
-constexpr float LN2 = 0.6931471805599453f;
-
-/* 2^x on the transcendental unit; 2^(-inf) = 0 */
-__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 /* ---- operand movement helpers (register arrays by reference so they stay in registers) ---- */
 
@@ -192,23 +175,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnProb *__restri
          * (mod count), i.e. on one die when count is a multiple of the die count */
         const uint32_t prob = blockIdx.x % aff.count;
         qtile = aff.nqt - 1u - blockIdx.x / aff.count;
-        const int64_t sq = prob / aff.heads, hh = prob % aff.heads;
-        /* field by field: a whole-struct copy that is then edited ends up in scratch memory */
-        const AttnProb &f = aff.first;
-        p.q = f.q + (sq * aff.q_seq + hh * aff.q_head);
-        p.k = f.k + (sq * aff.k_seq + hh * aff.k_head);
-        p.v = f.v + (sq * aff.v_seq + hh * aff.v_head);
-        p.out = f.out + (sq * aff.o_seq + hh * aff.o_head);
-        p.weights = f.weights ? f.weights + (sq * aff.w_seq + hh * aff.w_head) : nullptr;
-        p.lse = f.lse ? f.lse + (sq * aff.lse_seq + hh * aff.lse_head) : nullptr;
-        p.mask = DENSE ? f.mask + (sq * aff.mask_seq + hh * aff.mask_head) : nullptr;
-        const bool ranged = f.vis == ATTN_VIS_RANGE;
-        p.row_lo = ranged ? f.row_lo + (sq * aff.range_seq + hh * aff.range_head) : nullptr;
-        p.row_hi = ranged ? f.row_hi + (sq * aff.range_seq + hh * aff.range_head) : nullptr;
-        p.q_stride = f.q_stride, p.k_stride = f.k_stride, p.v_stride = f.v_stride, p.out_stride = f.out_stride;
-        p.nq = f.nq, p.nk = f.nk, p.hd = f.hd, p.vis = f.vis;
-        p.causal_off = f.causal_off, p.window = f.window, p.scale = f.scale, p.flags = f.flags;
-        p.reserved0 = p.reserved1 = 0;
+        affine_problem(p, aff, prob, DENSE);
     }
 
     const uint32_t lane = threadIdx.x & 63u;
@@ -240,15 +207,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnProb *__restri
             fhi = min(fhi, (uint32_t)__shfl_xor((int)fhi, off, 64));
         }
     } else {
-        /* ranges are monotone in the row index: first and last row bound the tile */
-        const uint32_t last = min(q0 + 31u, p.nq - 1u);
-        uint32_t lo_a, hi_a, lo_b, hi_b;
-        row_key_range(p, q0, lo_a, hi_a);
-        row_key_range(p, last, lo_b, hi_b);
-        tlo = hi_a > lo_a ? lo_a : (hi_b > lo_b ? lo_b : 0xFFFFFFFFu);
-        thi = hi_b > lo_b ? hi_b : hi_a;
-        if (!(thi > tlo)) tlo = 0xFFFFFFFFu, thi = 0u;
-        flo = lo_b, fhi = hi_a;
+        span_key_bounds(p, q0, min(q0 + 31u, p.nq - 1u), tlo, thi, flo, fhi);
     }
     const uint32_t kt_lo = thi > tlo ? tlo / 32u : 0u;
     const uint32_t kt_hi = thi > tlo ? (thi + 31u) / 32u : 0u;

@@ -88,6 +88,37 @@ def config2(batch=16, P=128, H=8, hd=64, T_bytes=512):
     return w
 
 
+def offset_causal(batch=2, nq=100, nk=228, H=2, hd=32, causal_offset=None, window=0, seed_cfg=6):
+    """Causal attention of nq new rows over nk keys (query i sees keys up to
+    i + causal_offset, optionally only the last `window` of them): the shape of
+    chunked prefill and sliding-window layers.  Separate Q / K / V buffers."""
+    if causal_offset is None:
+        causal_offset = nk - nq
+    E = H * hd
+    q = synth.normal(synth.seed_for(seed_cfg, synth.S_Q), (batch, nq, E))
+    k = synth.normal(synth.seed_for(seed_cfg, synth.S_K), (batch, nk, E))
+    v = synth.normal(synth.seed_for(seed_cfg, synth.S_V), (batch, nk, E))
+    out = np.zeros((batch, nq, E), dtype=np.float32)
+    scale = float(np.float32(1.0) / np.sqrt(np.float32(hd)))
+    heads = []
+    pairs = 0
+    for b in range(batch):
+        for h in range(H):
+            heads.append(Head(q=("q", b * nq * E + h * hd, E), k=("k", b * nk * E + h * hd, E),
+                              v=("v", b * nk * E + h * hd, E), out=("out", b * nq * E, E, h * hd),
+                              nq=nq, nk=nk, hd=hd, scale=scale, mask="causal", causal_offset=causal_offset,
+                              window=window, seq=b))
+    for i in range(nq):
+        hi = min(nk, i + causal_offset + 1)
+        lo = max(0, i + causal_offset + 1 - window) if window else 0
+        pairs += max(0, hi - lo)
+    pairs *= batch * H
+    return Workload(name="offset_causal", buffers={"q": q.reshape(-1), "k": k.reshape(-1), "v": v.reshape(-1),
+                                                   "out": out.reshape(-1)}, heads=heads, tokens=batch * nq,
+                    flops=4.0 * hd * pairs, bytes=4.0 * (q.size + k.size + v.size + out.size),
+                    meta=dict(batch=batch, nq=nq, nk=nk, H=H, hd=hd, E=E))
+
+
 def config3(batch=16, T=512, P=128, H=4, hd=32):
     """Local-encoder cross-attention: patch queries over the bytes of their own patch."""
     E = H * hd

@@ -1,0 +1,86 @@
+"""Runs a fixed list of attention cases through libfblt_hip.so and checks each
+against the CPU checker.  Not collected by pytest: test_gpu_parity.py starts it
+in a fresh process per kernel family, because the library reads the
+BLT_HIP_ATTN_FAMILY hook once per process.
+
+Tolerance: |got - ref| <= 1e-5 + 1e-4 * |ref| element-wise.
+"""
+import os
+import sys
+
+import numpy as np
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+
+from fblt_amd import runner, workloads  # noqa: E402
+from oracle import binding, runner as orunner  # noqa: E402
+
+CASES = {
+    "c1_small": lambda: workloads.config1(batch=1, T=96, H=2, hd=32),
+    "c1_ragged": lambda: workloads.config1(batch=2, T=77, H=2, hd=32),
+    "c1_300": lambda: workloads.config1(batch=2, T=300, H=2, hd=64),
+    "c1_129": lambda: workloads.config1(batch=3, T=129, H=1, hd=32),
+    "c2_small": lambda: workloads.config2(batch=2, P=48, H=2, hd=64, T_bytes=192),
+    "chunk_prefill": lambda: workloads.offset_causal(batch=2, nq=100, nk=228, H=2, hd=32),
+    "window": lambda: workloads.offset_causal(batch=2, nq=200, nk=200, H=2, hd=64, window=40),
+    "window_offset": lambda: workloads.offset_causal(batch=1, nq=150, nk=400, H=2, hd=32, window=70),
+    "c1_full": lambda: workloads.config1(),
+    "c2_full": lambda: workloads.config2(),
+}
+ENTRIES = ("batch_descriptor", "batch_dense", "per_head_flag", "plan_lse")
+
+
+def check(name, entry, got, ref):
+    err = np.abs(got.astype(np.float64) - ref.astype(np.float64))
+    bad = err > 1e-5 + 1e-4 * np.abs(ref)
+    if bad.any():
+        print("FAIL %s/%s: %d out of tolerance, max %.3e" % (name, entry, int(bad.sum()), float(err.max())))
+        sys.exit(1)
+    return float(err.max())
+
+
+def main():
+    import torch
+    orc = binding.load_oracle()
+    kernels = set()
+    for name, make in CASES.items():
+        w = make()
+        orunner.run(w, lib=orc)
+        ref = w.buffers["out"].copy()
+        w.buffers["out"][:] = 0
+        d = runner.DeviceWorkload(w)
+        try:
+            for entry in ENTRIES:
+                h0 = w.heads[0]
+                if entry == "per_head_flag" and (h0.causal_offset != 0 or h0.window != 0):
+                    continue  # the flag only describes plain causal problems
+                if entry == "batch_dense" and name.endswith("_full"):
+                    continue
+                print("case %s/%s" % (name, entry), flush=True)
+                d.zero_outputs()
+                if entry == "batch_descriptor":
+                    d.run_batch("descriptor")
+                elif entry == "batch_dense":
+                    d.run_batch("dense")
+                elif entry == "per_head_flag":
+                    d.run_per_head("flag", with_weights=False)
+                else:
+                    lse = [torch.full((h.nq * 2,), 7.0, dtype=torch.float32, device="cuda") for h in w.heads]
+                    arr = d.problems("descriptor", None, [t.data_ptr() for t in lse])
+                    plan = d.lib.blt_attention_plan_create_hip(arr, len(w.heads))
+                    kernels.add(d.lib.blt_attention_plan_kernel_hip(plan).decode())
+                    d.lib.blt_attention_plan_run_hip(plan)
+                    d.lib.blt_backend_pass_sync_hip()
+                    d.lib.blt_attention_plan_destroy_hip(plan)
+                    for t in lse:
+                        x = t.cpu().numpy().reshape(-1, 2)
+                        assert np.isfinite(x).all() and (x[:, 1] >= 1.0 - 1e-4).all(), "lse"
+                check(name, entry, d.output("out"), ref)
+        finally:
+            d.close()
+    print("KERNELS", ",".join(sorted(kernels)))
+    print("OK")
+
+
+if __name__ == "__main__":
+    main()

@@ -446,3 +446,19 @@ print("OK", float(err.max()))
     env = dict(os.environ, BLT_HIP_BLOCK_KERNEL=kernel)
     p = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300, env=env)
     assert p.returncode == 0 and "OK" in p.stdout, p.stdout + p.stderr
+
+
+@pytest.mark.parametrize("family", ["rows", "mfma", "wide"])
+def test_attention_kernel_families(family):
+    """Every attention kernel family on the same cases (causal, chunked prefill, sliding window,
+    dense masks, lse output), pinned through BLT_HIP_ATTN_FAMILY in a fresh process."""
+    import subprocess
+    import sys
+    import os
+    here = os.path.dirname(os.path.abspath(__file__))
+    env = dict(os.environ, BLT_HIP_ATTN_FAMILY=family)
+    p = subprocess.run([sys.executable, "-u", os.path.join(here, "family_cases.py")], capture_output=True, text=True,
+                       timeout=600, env=env)
+    assert p.returncode == 0 and "OK" in p.stdout, p.stdout[-2000:] + p.stderr[-2000:]
+    kernels = [ln for ln in p.stdout.splitlines() if ln.startswith("KERNELS")][0].split()[1]
+    assert kernels == family, kernels
