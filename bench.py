@@ -240,7 +240,9 @@ def main():
     # batch-swept prefill: the same kernels away from the launch floor
     if want("sweep"):
         for name, make in (("c1_x64", lambda: workloads.config1(batch=64)),
-                           ("c2_x8", lambda: workloads.config2(batch=128))):
+                           ("c2_x8", lambda: workloads.config2(batch=128)),
+                           ("c1_T4096", lambda: workloads.config1(batch=8, T=4096)),
+                           ("c2_P2048", lambda: workloads.config2(batch=8, P=2048, T_bytes=8192))):
             others[name], _ = bench_dense(make, max(10, K // 10), 3, "mfma")
             log(name, json.dumps(others[name]))
 

@@ -42,7 +42,7 @@
 namespace {
 
 template <int HD, int SRC, bool DENSE>
-__global__ __launch_bounds__(256) void attn_wide_kernel(const AttnProb *__restrict__ probs,
+__global__ __launch_bounds__(256, 2) void attn_wide_kernel(const AttnProb *__restrict__ probs,
                                                         const AttnTile *__restrict__ tiles, AttnAffine aff) {
     constexpr int HALF = HD / 2;
     constexpr int DB = HD / 32;
@@ -77,7 +77,10 @@ __global__ __launch_bounds__(256) void attn_wide_kernel(const AttnProb *__restri
     const uint32_t c = lane & 31u;
 
     const uint32_t g0 = group * 128u;       /* first row of the workgroup */
-    const uint32_t q0 = g0 + wave * 32u;    /* first row of this wave     */
+    /* which of the four query tiles a wave owns rotates with the group index:
+     * under a causal mask the later tiles are longer, and waves with the same
+     * index tend to share a SIMD across resident workgroups */
+    const uint32_t q0 = g0 + ((wave + group) & 3u) * 32u; /* first row of this wave */
     const uint32_t row = q0 + c;
     const bool live = row < p.nq;
     const uint32_t i = live ? row : p.nq - 1u;
@@ -194,19 +197,30 @@ __global__ __launch_bounds__(256) void attn_wide_kernel(const AttnProb *__restri
                 sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(t.w, qf[s4 + 3], sacc, 0, 0, 0);
             }
 
-            /* ---- mask, tile maximum ---- */
+            /* ---- mask, tile maximum ----
+             * Interior tiles (no row masks any key) only drop non-finite
+             * scores; edge tiles compare the key's offset into the row's
+             * range with one unsigned test.  No per-element branches. */
             float x[16];
             float mt = neg_inf();
-            const bool all_seen = !DENSE && k0 >= flo && k0 + 32u <= fhi; /* uniform: no row masks any key */
+            const bool all_seen = !DENSE && k0 >= flo && k0 + 32u <= fhi; /* wave-uniform */
+            if (all_seen) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const uint32_t j = k0 + acc_key(r, h);
-                float t = sacc[r];
-                if (DENSE) t += mk[r] * LOG2E;
-                bool vis = isfinite(t);
-                if (!all_seen) vis = vis && (j - lo) < (hi - lo);
-                x[r] = vis ? t : neg_inf();
-                mt = fmaxf(mt, x[r]);
+                for (int r = 0; r < 16; r++) {
+                    const float t = sacc[r];
+                    x[r] = isfinite(t) ? t : neg_inf();
+                    mt = fmaxf(mt, x[r]);
+                }
+            } else {
+                const uint32_t rel = k0 + 4u * h - lo, len = hi - lo;
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    float t = sacc[r];
+                    if (DENSE) t += mk[r] * LOG2E;
+                    const bool vis = (rel + (8u * (r >> 2) + (r & 3u)) < len) & isfinite(t);
+                    x[r] = vis ? t : neg_inf();
+                    mt = fmaxf(mt, x[r]);
+                }
             }
             mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
             const float mn = fmaxf(m, mt);
