@@ -279,11 +279,7 @@ void plan_build(blt_attention_plan &pl, const blt_attention_problem *problems, s
         if (b.fam != FAM_MFMA) continue;
         if (choose_wide(pl.host.data() + b.base, b.count)) b.fam = FAM_WIDE;
         b.affine = detect_affine(pl.host.data() + b.base, b.count, b.aff);
-        if (b.affine) {
-            /* no descriptor or tile memory needed */
-            if (b.fam == FAM_WIDE) b.aff.nqt = attn_wide_groups(b.aff.first);
-            continue;
-        }
+        if (b.affine) continue; /* no descriptor or tile memory needed */
         b.tile_base = (uint32_t)pl.tiles.size();
         if (b.fam == FAM_WIDE) attn_wide_make_tiles(pl.host.data(), b.base, b.count, pl.tiles);
         else attn_mfma_make_tiles(pl.host.data(), b.base, b.count, pl.tiles);

@@ -43,8 +43,8 @@ void attn_mfma_launch(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t n
 void attn_mfma_launch_single(const AttnProb &single, hipStream_t s);
 void attn_mfma_launch_affine(const AttnAffine &aff, hipStream_t s);
 
-/* wide family: work items are 128-row groups (AttnTile.qtile = group index,
- * AttnAffine.nqt = groups per problem) */
+/* wide family: work items are 128-row groups or pairs of them (AttnTile.qtile
+ * = two 16-bit group indices) */
 bool attn_wide_can(const AttnProb &d);
 uint32_t attn_wide_groups(const AttnProb &d);
 void attn_wide_make_tiles(const AttnProb *host, uint32_t base, uint32_t count, std::vector<AttnTile> &tiles);

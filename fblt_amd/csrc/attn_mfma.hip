@@ -146,7 +146,7 @@ struct MfmaLds {
 };
 
 template <int HD, int SRC, bool EXACT, bool DENSE>
-__global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnProb *__restrict__ probs,
+__global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_mfma_kernel(const AttnProb *__restrict__ probs,
                                                         const AttnTile *__restrict__ tiles, AttnAffine aff) {
     constexpr int HALF = HD / 2;
     constexpr int DB = HD / 32; /* 32-wide blocks of the head dim */

@@ -43,7 +43,7 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
  * blockIdx.z * hpb + wave % hpb, slice = wave / hpb.  The slices of a head
  * take the span's 32-key sub-chunks round-robin and merge through LDS. */
 template <int HD, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void kv_block_mfma_kernel(StepArgs a) {
+__global__ __launch_bounds__(64 * WAVES, 2) void kv_block_mfma_kernel(StepArgs a) {
     constexpr int HALF = HD / 2;
     constexpr int DB = HD / 32;
     constexpr int ROW = HD + 4;

@@ -24,7 +24,16 @@
  *
  * Causal problems: the workgroup walks the union of its four tiles' key
  * ranges; a wave skips the arithmetic (not the loads or barriers) of key
- * tiles outside its own range.
+ * tiles outside its own range.  Because later groups of a causal problem see
+ * more keys, a work item is a PAIR of groups (g, G-1-g) run back to back, so
+ * every workgroup of a problem does the same amount of work.
+ *
+ * Non-finite scores (the reference drops such keys) are handled
+ * optimistically: the key loop runs without per-element finiteness tests --
+ * on gfx950 the fp32 matrix instructions and the vector ALU share issue
+ * cycles, so every VALU instruction saved is matrix time gained -- and a NaN
+ * or +inf score necessarily leaves a non-finite row sum behind; a workgroup
+ * that finds one re-runs its group with the tests compiled in.
  *
  * Shapes: head_dim 32 or 64 exactly, 16-byte aligned rows, no weights
  * output, any visibility except per-row ranges.  Bound: MFMA (HD MFMAs of 64
@@ -41,35 +50,18 @@
 
 namespace {
 
-template <int HD, int SRC, bool DENSE>
-__global__ __launch_bounds__(256, 2) void attn_wide_kernel(const AttnProb *__restrict__ probs,
-                                                        const AttnTile *__restrict__ tiles, AttnAffine aff) {
+/* One 128-row group of problem p.  CHECK: test every score for finiteness.
+ * Returns (to every thread of the workgroup that asks) whether this lane's
+ * row ended with a non-finite sum, which only happens when !CHECK let a
+ * non-finite score through; nothing is stored in that case. */
+template <int HD, bool DENSE, bool CHECK>
+__device__ __forceinline__ bool wide_group(const AttnProb &p, uint32_t group, float (&sm_k)[2][32 * (HD + 4)],
+                                           float (&sm_v)[2][32 * (HD + 4)]) {
     constexpr int HALF = HD / 2;
     constexpr int DB = HD / 32;
-    constexpr int ROW = HD + 4;         /* LDS row pitch in floats: 16-byte fragment reads of 32 rows spread over all banks */
-    constexpr int TILE = 32 * ROW;
-    constexpr int LPR = HD / 4;         /* 16-byte pieces per row                 */
-    constexpr int PIECES = 32 * LPR / 256; /* pieces of one tile per thread       */
-
-    __shared__ __attribute__((aligned(16))) float sm_k[2][TILE];
-    __shared__ __attribute__((aligned(16))) float sm_v[2][TILE];
-
-    uint32_t group;
-    AttnProb p;
-    if (SRC == SRC_TILES) {
-        group = tiles[blockIdx.x].qtile;
-        p = probs[tiles[blockIdx.x].prob];
-    } else if (SRC == SRC_SINGLE) {
-        group = gridDim.x - 1u - blockIdx.x; /* causal: the long groups start first */
-        p = aff.first;
-    } else {
-        /* consecutive blocks are different problems of the same group index,
-         * so all groups of one problem land on one die (shared L2) whenever
-         * the problem count is a multiple of the die count */
-        const uint32_t prob = blockIdx.x % aff.count;
-        group = aff.nqt - 1u - blockIdx.x / aff.count;
-        affine_problem(p, aff, prob, DENSE);
-    }
+    constexpr int ROW = HD + 4;
+    constexpr int LPR = HD / 4;            /* 16-byte pieces per row               */
+    constexpr int PIECES = 32 * LPR / 256; /* pieces of one tile per thread        */
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
@@ -198,9 +190,9 @@ __global__ __launch_bounds__(256, 2) void attn_wide_kernel(const AttnProb *__res
             }
 
             /* ---- mask, tile maximum ----
-             * Interior tiles (no row masks any key) only drop non-finite
-             * scores; edge tiles compare the key's offset into the row's
-             * range with one unsigned test.  No per-element branches. */
+             * Interior tiles (no row masks any key) take the scores as they
+             * are; edge tiles compare the key's offset into the row's range
+             * with one unsigned test.  No per-element branches. */
             float x[16];
             float mt = neg_inf();
             const bool all_seen = !DENSE && k0 >= flo && k0 + 32u <= fhi; /* wave-uniform */
@@ -208,7 +200,7 @@ __global__ __launch_bounds__(256, 2) void attn_wide_kernel(const AttnProb *__res
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const float t = sacc[r];
-                    x[r] = isfinite(t) ? t : neg_inf();
+                    x[r] = (!CHECK || isfinite(t)) ? t : neg_inf();
                     mt = fmaxf(mt, x[r]);
                 }
             } else {
@@ -217,7 +209,7 @@ __global__ __launch_bounds__(256, 2) void attn_wide_kernel(const AttnProb *__res
                 for (int r = 0; r < 16; r++) {
                     float t = sacc[r];
                     if (DENSE) t += mk[r] * LOG2E;
-                    const bool vis = (rel + (8u * (r >> 2) + (r & 3u)) < len) & isfinite(t);
+                    const bool vis = (rel + (8u * (r >> 2) + (r & 3u)) < len) & (!CHECK || isfinite(t));
                     x[r] = vis ? t : neg_inf();
                     mt = fmaxf(mt, x[r]);
                 }
@@ -258,7 +250,8 @@ __global__ __launch_bounds__(256, 2) void attn_wide_kernel(const AttnProb *__res
 
     /* both halves of a column carry the same m, their sums add */
     l += __shfl_xor(l, 32, 64);
-    if (!live) return;
+    if (!CHECK && !isfinite(l)) return true;
+    if (!live) return false;
 
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     float *orow = p.out + (size_t)i * p.out_stride;
@@ -272,6 +265,52 @@ __global__ __launch_bounds__(256, 2) void attn_wide_kernel(const AttnProb *__res
     if (h == 0 && p.lse) {
         p.lse[2 * (size_t)i + 0] = m * LN2; /* back to natural units */
         p.lse[2 * (size_t)i + 1] = l;
+    }
+    return false;
+}
+
+/* Work item encoding shared by the three sources: two group indices, the
+ * second one WIDE_NO_GROUP when the item is a single group. */
+constexpr uint32_t WIDE_NO_GROUP = 0xFFFFu;
+
+/* item t of a problem with G groups, paired: (G-1-t, t), the middle one alone */
+__device__ __forceinline__ void wide_pair(uint32_t t, uint32_t G, uint32_t &ga, uint32_t &gb) {
+    ga = G - 1u - t;
+    gb = t < ga ? t : WIDE_NO_GROUP;
+}
+
+template <int HD, int SRC, bool DENSE>
+__global__ __launch_bounds__(256, 2) void attn_wide_kernel(const AttnProb *__restrict__ probs,
+                                                           const AttnTile *__restrict__ tiles, AttnAffine aff) {
+    constexpr int TILE = 32 * (HD + 4);
+    __shared__ __attribute__((aligned(16))) float sm_k[2][TILE];
+    __shared__ __attribute__((aligned(16))) float sm_v[2][TILE];
+
+    uint32_t ga, gb = WIDE_NO_GROUP;
+    AttnProb p;
+    if (SRC == SRC_TILES) {
+        const uint32_t code = tiles[blockIdx.x].qtile;
+        ga = code & 0xFFFFu, gb = code >> 16;
+        p = probs[tiles[blockIdx.x].prob];
+    } else if (SRC == SRC_SINGLE) {
+        p = aff.first;
+        if (aff.reserved) wide_pair(blockIdx.x, aff.nqt, ga, gb);
+        else ga = aff.nqt - 1u - blockIdx.x; /* causal with a window: the long groups start first */
+    } else {
+        /* consecutive blocks are different problems of the same item index,
+         * so all groups of one problem land on one die (shared L2) whenever
+         * the problem count is a multiple of the die count */
+        const uint32_t prob = blockIdx.x % aff.count;
+        if (aff.reserved) wide_pair(blockIdx.x / aff.count, aff.nqt, ga, gb);
+        else ga = aff.nqt - 1u - blockIdx.x / aff.count;
+        affine_problem(p, aff, prob, DENSE);
+    }
+
+    for (int pass = 0; pass < 2; pass++) {
+        const uint32_t group = pass == 0 ? ga : gb;
+        if (group == WIDE_NO_GROUP) break;
+        const bool bad = wide_group<HD, DENSE, false>(p, group, sm_k, sm_v);
+        if (__syncthreads_or(bad)) wide_group<HD, DENSE, true>(p, group, sm_k, sm_v);
     }
 }
 
@@ -294,35 +333,56 @@ void launch_wide(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t nblock
 /* shapes the kernel is able to run */
 bool attn_wide_can(const AttnProb &d) {
     return (d.hd == 32u || d.hd == 64u) && (d.flags & ATTN_FLAG_VEC4) != 0 && d.weights == nullptr &&
-           d.vis != ATTN_VIS_RANGE && d.nk >= 1u && d.nq >= 1u;
+           d.vis != ATTN_VIS_RANGE && d.nk >= 1u && d.nq >= 1u && d.nq <= 0xFFFEu * 128u; /* group indices travel in 16 bits */
 }
 
 uint32_t attn_wide_groups(const AttnProb &d) { return (d.nq + 127u) / 128u; }
 
-/* Work items (128-row groups) for problems [base, base+count), longest first. */
+/* Causal problems without a window: group g sees ~g+1 times the keys of group
+ * 0, so groups are run in pairs (g, G-1-g) of equal total work.  Short
+ * problems keep single groups: their imbalance is bounded by a few tiles and
+ * twice the workgroups hide more latency. */
+bool attn_wide_pairs(const AttnProb &d) {
+    return d.vis == ATTN_VIS_CAUSAL && d.window == 0u && attn_wide_groups(d) >= 8u;
+}
+
+/* work items of one problem */
+uint32_t attn_wide_items(const AttnProb &d) {
+    const uint32_t G = attn_wide_groups(d);
+    return attn_wide_pairs(d) ? (G + 1u) / 2u : G;
+}
+
+/* Work items for problems [base, base+count), longest first. */
 void attn_wide_make_tiles(const AttnProb *host, uint32_t base, uint32_t count, std::vector<AttnTile> &tiles) {
     struct Item {
         AttnTile t;
         uint32_t work;
     };
+    auto key_tiles = [](const AttnProb &d, uint32_t g) -> uint32_t {
+        uint64_t hi = d.nk, lo = 0;
+        if (d.vis == ATTN_VIS_CAUSAL) {
+            const uint64_t last = std::min<uint64_t>((uint64_t)g * 128u + 127u, d.nq - 1u) + d.causal_off;
+            hi = std::min<uint64_t>(hi, last + 1u);
+            if (d.window > 0) {
+                const uint64_t first = (uint64_t)g * 128u + d.causal_off;
+                lo = first + 1u > d.window ? first + 1u - d.window : 0u;
+            }
+        }
+        return hi > lo ? (uint32_t)((hi - lo + 31u) / 32u) : 0u;
+    };
     std::vector<Item> items;
     for (uint32_t n = 0; n < count; n++) {
         const AttnProb &d = host[base + n];
-        const uint32_t ng = attn_wide_groups(d);
-        for (uint32_t t = 0; t < ng; t++) {
-            uint64_t hi = d.nk, lo = 0;
-            if (d.vis == ATTN_VIS_CAUSAL) {
-                const uint64_t last = std::min<uint64_t>((uint64_t)t * 128u + 127u, d.nq - 1u) + d.causal_off;
-                hi = std::min<uint64_t>(hi, last + 1u);
-                if (d.window > 0) {
-                    const uint64_t first = (uint64_t)t * 128u + d.causal_off;
-                    lo = first + 1u > d.window ? first + 1u - d.window : 0u;
-                }
-            }
+        const uint32_t G = attn_wide_groups(d);
+        const bool pairs = attn_wide_pairs(d);
+        const uint32_t n_items = attn_wide_items(d);
+        for (uint32_t t = 0; t < n_items; t++) {
+            const uint32_t ga = pairs ? G - 1u - t : t;
+            const uint32_t gb = pairs && t < ga ? t : 0xFFFFu;
             Item it;
             it.t.prob = base + n;
-            it.t.qtile = t;
-            it.work = hi > lo ? (uint32_t)((hi - lo + 31u) / 32u) : 0u;
+            it.t.qtile = ga | (gb << 16);
+            it.work = key_tiles(d, ga) + (gb != 0xFFFFu ? key_tiles(d, gb) : 0u);
             items.push_back(it);
         }
     }
@@ -342,12 +402,18 @@ void attn_wide_launch_single(const AttnProb &single, hipStream_t s) {
     AttnAffine a;
     __builtin_memset(&a, 0, sizeof(a));
     a.first = single;
-    launch_wide<SRC_SINGLE>(nullptr, nullptr, attn_wide_groups(single), a, single.hd, single.vis == ATTN_VIS_DENSE, s);
+    a.nqt = attn_wide_groups(single);
+    a.reserved = attn_wide_pairs(single) ? 1u : 0u;
+    launch_wide<SRC_SINGLE>(nullptr, nullptr, attn_wide_items(single), a, single.hd, single.vis == ATTN_VIS_DENSE, s);
 }
 
-/* `aff.nqt` counts 128-row groups here */
-void attn_wide_launch_affine(const AttnAffine &aff, hipStream_t s) {
-    const uint32_t blocks = aff.count * aff.nqt;
+/* The batch descriptor of the mfma family, re-read for this kernel: `nqt`
+ * counts 128-row groups and `reserved` says whether groups run in pairs. */
+void attn_wide_launch_affine(const AttnAffine &aff_in, hipStream_t s) {
+    AttnAffine aff = aff_in;
+    aff.nqt = attn_wide_groups(aff.first);
+    aff.reserved = attn_wide_pairs(aff.first) ? 1u : 0u;
+    const uint32_t blocks = aff.count * attn_wide_items(aff.first);
     if (blocks == 0) return;
     launch_wide<SRC_AFFINE>(nullptr, nullptr, blocks, aff, aff.first.hd, aff.first.vis == ATTN_VIS_DENSE, s);
 }

@@ -15,7 +15,20 @@ sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 from fblt_amd import runner, workloads  # noqa: E402
 from oracle import binding, runner as orunner  # noqa: E402
 
+def _nonfinite_keys():
+    """Causal self-attention whose K holds a NaN, a +inf and a -inf: the scores against those
+    keys are not finite and the reference drops such keys from the softmax."""
+    w = workloads.config1(batch=1, T=160, H=2, hd=32)
+    E = w.meta["E"]
+    qkv = w.buffers["qkv"].reshape(160, 3 * E)
+    qkv[5, E + 3] = np.nan
+    qkv[70, E + 32] = np.inf
+    qkv[100, E + 7] = -np.inf
+    return w
+
+
 CASES = {
+    "nonfinite_keys": _nonfinite_keys,
     "c1_small": lambda: workloads.config1(batch=1, T=96, H=2, hd=32),
     "c1_ragged": lambda: workloads.config1(batch=2, T=77, H=2, hd=32),
     "c1_300": lambda: workloads.config1(batch=2, T=300, H=2, hd=64),
