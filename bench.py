@@ -246,6 +246,15 @@ def main():
             others[name], _ = bench_dense(make, max(10, K // 10), 3, "mfma")
             log(name, json.dumps(others[name]))
 
+        # decode and block verify with enough cached keys to leave the launch floor
+        big = workloads.config4(batch=128, steps=3 + 20, len_lo=1024, len_hi=2048, max_seq_len=2048 + 32,
+                               cache_period=8)
+        others["c4_b128_L2048"], _ = bench_kv(big, 20, 3)
+        log("c4_b128_L2048", json.dumps(others["c4_b128_L2048"]))
+        bigv = workloads.config5(batch=128, B=16, len_lo=1024, len_hi=2032, max_seq_len=2048, cache_period=8)
+        others["c5_B16_b128_L2048"], _ = bench_kv(bigv, 20, 3)
+        log("c5_B16_b128_L2048", json.dumps(others["c5_B16_b128_L2048"]))
+
     cpu_head = None
     if not args.no_cpu:
         cpu_head = cpu_dense(w2, args.cpu_seconds)

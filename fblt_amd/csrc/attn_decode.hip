@@ -71,8 +71,9 @@ __global__ __launch_bounds__(64 * WAVES) void kv_step_kernel(StepArgs a) {
     const uint32_t nk = len + a.n;
     const size_t slab = (size_t)b * a.max_seq_len;
     const uint32_t col = (head_ok ? head : 0u) * HD + 4u * g;
-    const uint32_t k_begin = split * a.span;
-    const uint32_t k_end = min(k_begin + a.span, nk);
+    const uint32_t span = kv_span_of(a, nk);
+    const uint32_t k_begin = split * span;
+    const uint32_t k_end = min(k_begin + span, nk);
 
     float4 q[NQ], o[NQ];
     float m[NQ], l[NQ];

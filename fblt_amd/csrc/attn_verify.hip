@@ -67,8 +67,9 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block_mfma_kernel(StepArgs a
     const uint32_t len = a.self_len[b];
     const uint32_t nk = len + a.n;
     const size_t slab = (size_t)b * a.max_seq_len;
-    const uint32_t k_begin = split * a.span;
-    const uint32_t k_end = min(k_begin + a.span, nk);
+    const uint32_t span = kv_span_of(a, nk);
+    const uint32_t k_begin = split * span;
+    const uint32_t k_end = min(k_begin + span, nk);
     const size_t newrow0 = (size_t)b * a.n;
 
     /* query fragment: row c of the block (clamped), floats [h*HALF, (h+1)*HALF) of the head */

@@ -38,6 +38,15 @@ struct StepArgs {
 };
 
 
+/* Keys per split for a sequence that attends nk keys: the sequence's own
+ * sub-chunks divided evenly over the launch's splits, so that every workgroup
+ * of a sequence gets the same share whatever the sequence's length (a.span,
+ * sized for the longest sequence, is the upper bound). */
+__device__ __forceinline__ uint32_t kv_span_of(const StepArgs &a, uint32_t nk) {
+    const uint32_t subs = (nk + SUB - 1u) / SUB;
+    return min(a.span, ((subs + a.splits - 1u) / a.splits) * SUB);
+}
+
 /* Device-scope store / load of data another workgroup (possibly on another
  * die of the package) reads within the same launch. */
 __device__ __forceinline__ void publish(float *p, float x) {

@@ -178,9 +178,16 @@ class KvWorkload:
         return self.H * self.hd
 
 
-def _fill_cache(cfg_id, batch, max_seq_len, E, lens):
-    k = synth.normal(synth.seed_for(cfg_id, synth.S_K), (batch, max_seq_len, E))
-    v = synth.normal(synth.seed_for(cfg_id, synth.S_V), (batch, max_seq_len, E))
+def _fill_cache(cfg_id, batch, max_seq_len, E, lens, period=None):
+    """`period`: generate that many sequences and repeat them over the batch (large
+    bandwidth workloads, where drawing every value would dominate the run time)."""
+    gen = batch if not period else min(batch, period)
+    k = synth.normal(synth.seed_for(cfg_id, synth.S_K), (gen, max_seq_len, E))
+    v = synth.normal(synth.seed_for(cfg_id, synth.S_V), (gen, max_seq_len, E))
+    if gen < batch:
+        reps = (batch + gen - 1) // gen
+        k = np.tile(k, (reps, 1, 1))[:batch].copy()
+        v = np.tile(v, (reps, 1, 1))[:batch].copy()
     # rows past the valid length hold stale data in the reference too; keep them
     # finite but recognisable so that a kernel reading them would be caught
     for b in range(batch):
@@ -189,13 +196,13 @@ def _fill_cache(cfg_id, batch, max_seq_len, E, lens):
     return k.reshape(batch * max_seq_len, E), v.reshape(batch * max_seq_len, E)
 
 
-def config4(batch=64, steps=256, H=4, hd=32, len_lo=1, len_hi=512, max_seq_len=None):
+def config4(batch=64, steps=256, H=4, hd=32, len_lo=1, len_hi=512, max_seq_len=None, cache_period=None):
     """KV-cache decode: one new byte per sequence and step, appended before attending."""
     E = H * hd
     if max_seq_len is None:
         max_seq_len = len_hi + steps
     lens = synth.integers(synth.seed_for(4, synth.S_LEN), batch, len_lo, len_hi).astype(np.uint32)
-    ck, cv = _fill_cache(4, batch, max_seq_len, E, lens)
+    ck, cv = _fill_cache(4, batch, max_seq_len, E, lens, cache_period)
     q_new = synth.normal(synth.seed_for(4, synth.S_NEWQ), (steps, batch, E))
     k_new = synth.normal(synth.seed_for(4, synth.S_NEWK), (steps, batch, E))
     v_new = synth.normal(synth.seed_for(4, synth.S_NEWV), (steps, batch, E))
@@ -206,14 +213,14 @@ def config4(batch=64, steps=256, H=4, hd=32, len_lo=1, len_hi=512, max_seq_len=N
                       bytes=4.0 * (2 * E * float(nk0.sum()) + batch * (E + E + 2 * E)))
 
 
-def config5(batch=64, B=4, H=4, hd=32, len_lo=64, len_hi=508, max_seq_len=None, steps=1):
+def config5(batch=64, B=4, H=4, hd=32, len_lo=64, len_hi=508, max_seq_len=None, steps=1, cache_period=None):
     """BLT-D/DV block verify: B query rows per sequence see the cached prefix and the whole block."""
     E = H * hd
     if max_seq_len is None:
         max_seq_len = 768
     assert len_hi + B <= max_seq_len
     lens = synth.integers(synth.seed_for(5, synth.S_LEN), batch, len_lo, len_hi).astype(np.uint32)
-    ck, cv = _fill_cache(5, batch, max_seq_len, E, lens)
+    ck, cv = _fill_cache(5, batch, max_seq_len, E, lens, cache_period)
     q_new = synth.normal(synth.seed_for(5, synth.S_NEWQ), (steps, batch * B, E))
     k_new = synth.normal(synth.seed_for(5, synth.S_NEWK), (steps, batch * B, E))
     v_new = synth.normal(synth.seed_for(5, synth.S_NEWV), (steps, batch * B, E))
