@@ -271,7 +271,10 @@ int env_int(const char *name, int fallback) {
 
 template <int G>
 void dispatch_nq(const StepArgs &a, uint32_t nq, uint32_t batch, hipStream_t s) {
-    static const int waves = env_int("BLT_HIP_DECODE_WAVES", 4);
+    /* single rows: one wave per head, and a second slice of waves once a split
+     * holds enough keys to keep both busy */
+    static const int pinned_waves = env_int("BLT_HIP_DECODE_WAVES", 0);
+    const int waves = pinned_waves > 0 ? pinned_waves : (a.span >= 256u ? 8 : 4);
     if (nq <= 1) {
         if (waves >= 16) launch_step<G, 1, 16>(a, batch, s);
         else if (waves >= 8) launch_step<G, 1, 8>(a, batch, s);

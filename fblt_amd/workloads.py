@@ -119,6 +119,33 @@ def offset_causal(batch=2, nq=100, nk=228, H=2, hd=32, causal_offset=None, windo
                     meta=dict(batch=batch, nq=nq, nk=nk, H=H, hd=hd, E=E))
 
 
+def merged(name, parts):
+    """One workload holding the heads of several (buffers renamed "<k>.<name>"): a
+    batch whose problems differ in shape, as a caller that flattens layers produces."""
+    import dataclasses
+    buffers, ranges, heads, outputs = {}, {}, [], []
+    tokens, flops, nbytes = 0, 0.0, 0.0
+    for k, w in enumerate(parts):
+        pre = "%d." % k
+        buffers.update({pre + n: a for n, a in w.buffers.items()})
+        ranges.update({pre + n: a for n, a in w.ranges.items()})
+        outputs += [pre + n for n in w.outputs]
+        for h in w.heads:
+            ref = h.mask_ref
+            if h.mask == "range":
+                ref = (pre + ref[0], pre + ref[1], ref[2])
+            elif h.mask == "dense":
+                ref = (pre + ref[0], ref[1])
+            heads.append(dataclasses.replace(h, q=(pre + h.q[0],) + tuple(h.q[1:]), k=(pre + h.k[0],) + tuple(h.k[1:]),
+                                             v=(pre + h.v[0],) + tuple(h.v[1:]),
+                                             out=(pre + h.out[0],) + tuple(h.out[1:]), mask_ref=ref))
+        tokens += w.tokens
+        flops += w.flops
+        nbytes += w.bytes
+    return Workload(name=name, buffers=buffers, ranges=ranges, heads=heads, outputs=tuple(outputs), tokens=tokens,
+                    flops=flops, bytes=nbytes)
+
+
 def config3(batch=16, T=512, P=128, H=4, hd=32):
     """Local-encoder cross-attention: patch queries over the bytes of their own patch."""
     E = H * hd

@@ -37,6 +37,9 @@ CASES = {
     "chunk_prefill": lambda: workloads.offset_causal(batch=2, nq=100, nk=228, H=2, hd=32),
     "window": lambda: workloads.offset_causal(batch=2, nq=200, nk=200, H=2, hd=64, window=40),
     "window_offset": lambda: workloads.offset_causal(batch=1, nq=150, nk=400, H=2, hd=32, window=70),
+    "mixed_shapes": lambda: workloads.merged("mixed", [workloads.config1(batch=1, T=96, H=2, hd=32),
+                                                       workloads.config1(batch=2, T=300, H=1, hd=32),
+                                                       workloads.offset_causal(batch=1, nq=70, nk=200, H=3, hd=32)]),
     "c1_full": lambda: workloads.config1(),
     "c2_full": lambda: workloads.config2(),
 }
@@ -59,13 +62,13 @@ def main():
     for name, make in CASES.items():
         w = make()
         orunner.run(w, lib=orc)
-        ref = w.buffers["out"].copy()
-        w.buffers["out"][:] = 0
+        ref = {n: w.buffers[n].copy() for n in w.outputs}
+        for n in w.outputs:
+            w.buffers[n][:] = 0
         d = runner.DeviceWorkload(w)
         try:
             for entry in ENTRIES:
-                h0 = w.heads[0]
-                if entry == "per_head_flag" and (h0.causal_offset != 0 or h0.window != 0):
+                if entry == "per_head_flag" and any(h.causal_offset != 0 or h.window != 0 for h in w.heads):
                     continue  # the flag only describes plain causal problems
                 if entry == "batch_dense" and name.endswith("_full"):
                     continue
@@ -88,7 +91,8 @@ def main():
                     for t in lse:
                         x = t.cpu().numpy().reshape(-1, 2)
                         assert np.isfinite(x).all() and (x[:, 1] >= 1.0 - 1e-4).all(), "lse"
-                check(name, entry, d.output("out"), ref)
+                for n in w.outputs:
+                    check(name, entry + ":" + n, d.output(n), ref[n])
         finally:
             d.close()
     print("KERNELS", ",".join(sorted(kernels)))
