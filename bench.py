@@ -233,6 +233,11 @@ def main():
     if want("c4"):
         others["c4"], k4 = bench_kv(workloads.config4(steps=W + 256, max_seq_len=512 + W + 256), 256, W)
         log("c4", json.dumps(others["c4"]))
+        # the same steps with the rotation of the new Q/K rows fused in (un-rotated inputs + tables)
+        others["c4_rope"], _ = bench_kv(workloads.config4(steps=W + 256, max_seq_len=512 + W + 256, rope=True), 256,
+                                        W)
+        others["c4_rope"]["workload"] = "c4_kv_decode + fused RoPE of new rows"
+        log("c4_rope", json.dumps(others["c4_rope"]))
     if want("c5"):
         for B in (4, 8, 16):
             others["c5_B%d" % B], k5 = bench_kv(workloads.config5(B=B), K, W)

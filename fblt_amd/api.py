@@ -101,6 +101,9 @@ SYMBOLS = {
     "blt_kv_attend_step_hip": (None, [C.POINTER(BltKvAttnCache), C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t,
                                       C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t, C.c_int, C.c_int,
                                       C.c_size_t]),
+    "blt_kv_rope_attend_step_hip": (None, [C.POINTER(BltKvAttnCache), C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t,
+                                           C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p,
+                                           C.c_size_t, C.c_size_t, C.c_int, C.c_int, C.c_size_t]),
     "blt_hip_profile_begin": (None, []),
     "blt_hip_profile_end": (C.c_size_t, [C.POINTER(BltHipKernelTime), C.c_size_t]),
     "blt_hip_stream_copy_probe": (None, [C.c_void_p, C.c_void_p, C.c_size_t]),

@@ -81,6 +81,10 @@ __global__ __launch_bounds__(64 * WAVES) void kv_step_kernel(StepArgs a) {
     for (int r = 0; r < NQ; r++) {
         const uint32_t qi = min(a.q0 + r, a.n - 1u);
         q[r] = *reinterpret_cast<const float4 *>(a.q_rows + ((size_t)b * a.n + qi) * a.q_stride + col);
+        if (a.rope_cos) { /* the query sits at position len + qi */
+            const size_t at = (size_t)(len + qi) * (HD / 2) + 2u * g;
+            q[r] = rope_rotate4(q[r], a.rope_cos + at, a.rope_sin + at);
+        }
         o[r] = make_float4(0.f, 0.f, 0.f, 0.f);
         m[r] = neg_inf();
         l[r] = 0.f;
@@ -97,6 +101,10 @@ __global__ __launch_bounds__(64 * WAVES) void kv_step_kernel(StepArgs a) {
                 const size_t r = (size_t)b * a.n + (j - len);
                 kf[t] = *reinterpret_cast<const float4 *>(a.k_rows + r * a.k_stride + col);
                 vf[t] = *reinterpret_cast<const float4 *>(a.v_rows + r * a.v_stride + col);
+                if (a.rope_cos) { /* a new key row is rotated at its own position j */
+                    const size_t at = (size_t)j * (HD / 2) + 2u * g;
+                    kf[t] = rope_rotate4(kf[t], a.rope_cos + at, a.rope_sin + at);
+                }
             }
         }
     };
@@ -287,10 +295,11 @@ void dispatch_nq(const StepArgs &a, uint32_t nq, uint32_t batch, hipStream_t s) 
 
 } // namespace
 
-extern "C" void blt_kv_attend_step_hip(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride,
-                                       const float *k_rows, size_t k_stride, const float *v_rows, size_t v_stride,
-                                       float *combined, size_t combined_stride, size_t n, int step_kind, int commit,
-                                       size_t max_len_hint) {
+namespace {
+
+void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride, const float *k_rows,
+                 size_t k_stride, const float *v_rows, size_t v_stride, const float *rope_cos, const float *rope_sin,
+                 float *combined, size_t combined_stride, size_t n, int step_kind, int commit, size_t max_len_hint) {
     BLT_REQUIRE(cache != NULL && cache->self_k != NULL && cache->self_v != NULL && cache->self_len != NULL,
                 "blt_kv_attend_step: cache buffers must not be NULL");
     BLT_REQUIRE(q_rows != NULL && k_rows != NULL && v_rows != NULL && combined != NULL,
@@ -323,6 +332,8 @@ extern "C" void blt_kv_attend_step_hip(const blt_kv_attn_cache *cache, const flo
     a.k_rows = k_rows;
     a.v_rows = v_rows;
     a.combined = combined;
+    a.rope_cos = rope_cos;
+    a.rope_sin = rope_sin;
     a.q_stride = (uint32_t)q_stride;
     a.k_stride = (uint32_t)k_stride;
     a.v_stride = (uint32_t)v_stride;
@@ -415,4 +426,29 @@ extern "C" void blt_kv_attend_step_hip(const blt_kv_attn_cache *cache, const flo
         }
     }
     HIP_CHECK_LAUNCH("blt_kv_attend_step");
+}
+
+} // namespace
+
+extern "C" void blt_kv_attend_step_hip(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride,
+                                       const float *k_rows, size_t k_stride, const float *v_rows, size_t v_stride,
+                                       float *combined, size_t combined_stride, size_t n, int step_kind, int commit,
+                                       size_t max_len_hint) {
+    kv_step_run(cache, q_rows, q_stride, k_rows, k_stride, v_rows, v_stride, nullptr, nullptr, combined,
+                combined_stride, n, step_kind, commit, max_len_hint);
+}
+
+extern "C" void blt_kv_rope_attend_step_hip(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride,
+                                            const float *k_rows, size_t k_stride, const float *v_rows,
+                                            size_t v_stride, const float *rope_cos, const float *rope_sin,
+                                            size_t rope_positions, float *combined, size_t combined_stride, size_t n,
+                                            int step_kind, int commit, size_t max_len_hint) {
+    BLT_REQUIRE(rope_cos != NULL && rope_sin != NULL, "blt_kv_rope_attend_step: rotation tables must not be NULL");
+    BLT_REQUIRE(((reinterpret_cast<uintptr_t>(rope_cos) | reinterpret_cast<uintptr_t>(rope_sin)) & 7u) == 0,
+                "blt_kv_rope_attend_step: rotation tables must be 8-byte aligned");
+    BLT_REQUIRE(max_len_hint <= rope_positions,
+                "blt_kv_rope_attend_step: positions up to %zu exceed the rotation tables (%zu rows)", max_len_hint,
+                rope_positions);
+    kv_step_run(cache, q_rows, q_stride, k_rows, k_stride, v_rows, v_stride, rope_cos, rope_sin, combined,
+                combined_stride, n, step_kind, commit, max_len_hint);
 }

@@ -80,7 +80,11 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block_mfma_kernel(StepArgs a
         const float *qrow = a.q_rows + (newrow0 + min(qi, a.n - 1u)) * a.q_stride + hsafe * HD + h * HALF;
 #pragma unroll
         for (int s = 0; s < HALF; s += 4) {
-            const float4 t = *reinterpret_cast<const float4 *>(qrow + s);
+            float4 t = *reinterpret_cast<const float4 *>(qrow + s);
+            if (a.rope_cos) { /* the query sits at position len + qi */
+                const size_t at = (size_t)(len + min(qi, a.n - 1u)) * HALF + (h * HALF + s) / 2;
+                t = rope_rotate4(t, a.rope_cos + at, a.rope_sin + at);
+            }
             qf[s + 0] = t.x, qf[s + 1] = t.y, qf[s + 2] = t.z, qf[s + 3] = t.w;
         }
     }
@@ -167,8 +171,12 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block_mfma_kernel(StepArgs a
 #pragma unroll
         for (int t = 0; t < HD / 8; t++) {
             const uint32_t r = t * (64 / LPR) + lane / LPR;
-            const float4 piece = make_float4(kg[4 * t + 0], kg[4 * t + 1], kg[4 * t + 2], kg[4 * t + 3]);
+            float4 piece = make_float4(kg[4 * t + 0], kg[4 * t + 1], kg[4 * t + 2], kg[4 * t + 3]);
             const uint32_t j = c0 + r;
+            if (a.rope_cos && c0 + 32u > len && j >= len && j < nk) { /* a new key row is rotated at its position j */
+                const size_t at = (size_t)j * HALF + 2u * (lane % LPR);
+                piece = rope_rotate4(piece, a.rope_cos + at, a.rope_sin + at);
+            }
             if (a.write_through && head_ok && c0 + 32u > len && j >= len && j < k_end)
                 *reinterpret_cast<float4 *>(a.cache_k + (slab + j) * a.embed_dim + head * HD + 4u * (lane % LPR)) = piece;
             *reinterpret_cast<float4 *>(my_k + r * ROW + 4u * (lane % LPR)) = piece;

@@ -151,7 +151,8 @@ class DeviceWorkload:
 
 
 class DeviceKvWorkload:
-    """Device-resident KV-cache workload driving blt_kv_attend_step_hip."""
+    """Device-resident KV-cache workload driving blt_kv_attend_step_hip, or
+    blt_kv_rope_attend_step_hip when the workload carries rotation tables."""
 
     def __init__(self, kw):
         torch = _torch()
@@ -164,6 +165,9 @@ class DeviceKvWorkload:
         self.q_new = torch.from_numpy(kw.q_new).cuda()
         self.k_new = torch.from_numpy(kw.k_new).cuda()
         self.v_new = torch.from_numpy(kw.v_new).cuda()
+        self.rope = None
+        if kw.rope_cos is not None:
+            self.rope = (torch.from_numpy(kw.rope_cos).cuda(), torch.from_numpy(kw.rope_sin).cuda())
         self.out = torch.zeros((kw.steps, kw.batch * kw.n, kw.E), dtype=torch.float32, device="cuda")
         self.host_max_len = int(kw.lens.max())
         self.c = api.BltKvAttnCache()
@@ -184,9 +188,16 @@ class DeviceKvWorkload:
         kw = self.kw
         E = kw.E
         hint = self.host_max_len + kw.n
-        self.lib.blt_kv_attend_step_hip(C.byref(self.c), self.q_new[s].data_ptr(), E, self.k_new[s].data_ptr(), E,
-                                        self.v_new[s].data_ptr(), E, self.out[s].data_ptr(), E, kw.n, self.kind,
-                                        1 if kw.commit else 0, hint)
+        if self.rope is not None:
+            self.lib.blt_kv_rope_attend_step_hip(C.byref(self.c), self.q_new[s].data_ptr(), E,
+                                                 self.k_new[s].data_ptr(), E, self.v_new[s].data_ptr(), E,
+                                                 self.rope[0].data_ptr(), self.rope[1].data_ptr(),
+                                                 self.rope[0].shape[0], self.out[s].data_ptr(), E, kw.n, self.kind,
+                                                 1 if kw.commit else 0, hint)
+        else:
+            self.lib.blt_kv_attend_step_hip(C.byref(self.c), self.q_new[s].data_ptr(), E, self.k_new[s].data_ptr(),
+                                            E, self.v_new[s].data_ptr(), E, self.out[s].data_ptr(), E, kw.n,
+                                            self.kind, 1 if kw.commit else 0, hint)
         if kw.commit:
             self.host_max_len += kw.n
 

@@ -196,6 +196,8 @@ class KvWorkload:
     H: int
     hd: int
     window: int = 0
+    rope_cos: np.ndarray = None   # [max_seq_len, hd/2] rotation tables: q_new / k_new are un-rotated
+    rope_sin: np.ndarray = None
     tokens: int = 0          # query rows per step
     flops: float = 0.0       # per step (first step)
     bytes: float = 0.0
@@ -203,6 +205,16 @@ class KvWorkload:
     @property
     def E(self):
         return self.H * self.hd
+
+
+def rope_tables(positions, hd, theta=500000.0):
+    """cos / sin of pos / theta^(2i/hd), [positions, hd/2] fp32 (the quantities
+    blt_rope_precompute tabulates; computed in float64 here and rounded once, so
+    the values are inputs of a workload, not a restatement of that function)."""
+    i = np.arange(hd // 2, dtype=np.float64)
+    freq = 1.0 / np.power(np.float64(theta), 2.0 * i / hd)
+    angle = np.arange(positions, dtype=np.float64)[:, None] * freq[None, :]
+    return np.cos(angle).astype(np.float32), np.sin(angle).astype(np.float32)
 
 
 def _fill_cache(cfg_id, batch, max_seq_len, E, lens, period=None):
@@ -223,7 +235,8 @@ def _fill_cache(cfg_id, batch, max_seq_len, E, lens, period=None):
     return k.reshape(batch * max_seq_len, E), v.reshape(batch * max_seq_len, E)
 
 
-def config4(batch=64, steps=256, H=4, hd=32, len_lo=1, len_hi=512, max_seq_len=None, cache_period=None):
+def config4(batch=64, steps=256, H=4, hd=32, len_lo=1, len_hi=512, max_seq_len=None, cache_period=None,
+            rope=False):
     """KV-cache decode: one new byte per sequence and step, appended before attending."""
     E = H * hd
     if max_seq_len is None:
@@ -234,13 +247,15 @@ def config4(batch=64, steps=256, H=4, hd=32, len_lo=1, len_hi=512, max_seq_len=N
     k_new = synth.normal(synth.seed_for(4, synth.S_NEWK), (steps, batch, E))
     v_new = synth.normal(synth.seed_for(4, synth.S_NEWV), (steps, batch, E))
     nk0 = lens.astype(np.int64) + 1
+    rc, rs = rope_tables(max_seq_len, hd) if rope else (None, None)
     return KvWorkload(name="c4_kv_decode", cache_k=ck, cache_v=cv, lens=lens, q_new=q_new, k_new=k_new, v_new=v_new,
                       n=1, steps=steps, kind="causal", commit=True, batch=batch, max_seq_len=max_seq_len, H=H, hd=hd,
-                      tokens=batch, flops=4.0 * hd * H * float(nk0.sum()),
+                      rope_cos=rc, rope_sin=rs, tokens=batch, flops=4.0 * hd * H * float(nk0.sum()),
                       bytes=4.0 * (2 * E * float(nk0.sum()) + batch * (E + E + 2 * E)))
 
 
-def config5(batch=64, B=4, H=4, hd=32, len_lo=64, len_hi=508, max_seq_len=None, steps=1, cache_period=None):
+def config5(batch=64, B=4, H=4, hd=32, len_lo=64, len_hi=508, max_seq_len=None, steps=1, cache_period=None,
+            rope=False):
     """BLT-D/DV block verify: B query rows per sequence see the cached prefix and the whole block."""
     E = H * hd
     if max_seq_len is None:
@@ -252,8 +267,9 @@ def config5(batch=64, B=4, H=4, hd=32, len_lo=64, len_hi=508, max_seq_len=None, 
     k_new = synth.normal(synth.seed_for(5, synth.S_NEWK), (steps, batch * B, E))
     v_new = synth.normal(synth.seed_for(5, synth.S_NEWV), (steps, batch * B, E))
     nk = lens.astype(np.int64) + B
+    rc, rs = rope_tables(max_seq_len, hd) if rope else (None, None)
     return KvWorkload(name="c5_block_verify_B%d" % B, cache_k=ck, cache_v=cv, lens=lens, q_new=q_new, k_new=k_new,
                       v_new=v_new, n=B, steps=steps, kind="block", commit=False, batch=batch,
-                      max_seq_len=max_seq_len, H=H, hd=hd, tokens=batch * B,
+                      max_seq_len=max_seq_len, H=H, hd=hd, rope_cos=rc, rope_sin=rs, tokens=batch * B,
                       flops=4.0 * hd * H * B * float(nk.sum()),
                       bytes=4.0 * (2 * E * float(nk.sum()) + batch * B * 2 * E))

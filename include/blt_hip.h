@@ -193,6 +193,26 @@ void blt_kv_attend_step_hip(const blt_kv_attn_cache *cache, const float *q_rows,
                             float *combined, size_t combined_stride, size_t n, int step_kind, int commit,
                             size_t max_len_hint);
 
+/* blt_kv_attend_step_hip with the rotation of the new rows fused in: the step
+ * of blt_kv_decode_step from the QKV projection's output to `combined`
+ * (csrc/infer/kv_cache.c:262-271 position gather, 343-366 per-head copy-out,
+ * blt_rope_apply of Q and K, copy-back and write-through, 368-390 attention).
+ * q_rows / k_rows / v_rows are the UN-rotated new rows, typically the three
+ * column blocks of the packed [batch*n, 3E] projection output (stride 3E).
+ * Row r of sequence b sits at position self_len[b] + r; Q and K pairs
+ * (2i, 2i+1) of every head are rotated by rope_cos / rope_sin
+ * [rope_positions, head_dim/2] (DEVICE copies of the tables
+ * blt_rope_precompute fills, csrc/ops/reductions_cpu.c:179-197) exactly as
+ * blt_rope_apply_cpu does (reductions_cpu.c:199-229), so the K rows stored in
+ * the cache are bit-identical to the reference's.  Requires max_len_hint <=
+ * rope_positions.  One launch replaces the reference's 6 strided copies + 2
+ * rotations + 1 attention call per head. */
+void blt_kv_rope_attend_step_hip(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride,
+                                 const float *k_rows, size_t k_stride, const float *v_rows, size_t v_stride,
+                                 const float *rope_cos, const float *rope_sin, size_t rope_positions,
+                                 float *combined, size_t combined_stride, size_t n, int step_kind, int commit,
+                                 size_t max_len_hint);
+
 /* Per-kernel device time of every launch the library issues between begin and
  * end, from HIP events attached to each dispatch (the kernel's own begin/end
  * timestamps, without launch gaps).  `end` synchronises the device, fills up to

@@ -10,6 +10,8 @@ import ctypes as C
 import os
 import subprocess
 
+import numpy as np
+
 from fblt_amd import abi
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -66,7 +68,37 @@ def load_oracle():
     lib.orc_kv_attend_step.restype = C.c_int
     lib.orc_kv_attend_step.argtypes = [_fp, _fp, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t,
                                        C.c_size_t, C.c_size_t, _fp, _fp, _fp, _fp]
+    lib.orc_rope_precompute.restype = C.c_int
+    lib.orc_rope_precompute.argtypes = [C.c_size_t, C.c_float, C.c_size_t, _fp, _fp]
+    lib.orc_rope_apply.restype = None
+    lib.orc_rope_apply.argtypes = [_fp, C.c_size_t, C.c_size_t, C.c_size_t, _fp, _fp, _fp]
+    lib.orc_rope_position_gather.restype = C.c_int
+    lib.orc_rope_position_gather.argtypes = [_fp, _fp, C.c_size_t, C.c_size_t, _sp, C.c_size_t, _fp, _fp]
+    lib.orc_kv_rope_attend_step.restype = C.c_int
+    lib.orc_kv_rope_attend_step.argtypes = [_fp, _fp] + [C.c_size_t] * 7 + [_fp, C.c_size_t, _fp, C.c_size_t, _fp,
+                                                                           C.c_size_t, _fp, _fp, C.c_size_t, _fp]
     return lib
+
+
+class BltRopeConfig(C.Structure):
+    """blt_rope_config, csrc/ops/rope.h:10-13"""
+    _fields_ = [("theta", C.c_float), ("head_dim", C.c_size_t)]
+
+
+def ref_rope_apply(ref, x, cos_rows, sin_rows):
+    """x [rows, heads, hd] through the reference's blt_rope_apply with cos/sin rows [rows, hd/2]."""
+    rows, heads, hd = x.shape
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    cos_rows = np.ascontiguousarray(cos_rows, dtype=np.float32)
+    sin_rows = np.ascontiguousarray(sin_rows, dtype=np.float32)
+    out = np.empty_like(x)
+    tx, tc, ts, to = abi.BltTensor(), abi.BltTensor(), abi.BltTensor(), abi.BltTensor()
+    ref.blt_tensor_view_3d(C.byref(tx), x.ctypes.data, rows, heads, hd, abi.BLT_BACKEND_CPU)
+    ref.blt_tensor_view_3d(C.byref(to), out.ctypes.data, rows, heads, hd, abi.BLT_BACKEND_CPU)
+    ref.blt_tensor_view_2d(C.byref(tc), cos_rows.ctypes.data, rows, hd // 2, abi.BLT_BACKEND_CPU)
+    ref.blt_tensor_view_2d(C.byref(ts), sin_rows.ctypes.data, rows, hd // 2, abi.BLT_BACKEND_CPU)
+    ref.blt_rope_apply(C.byref(tx), C.byref(tc), C.byref(ts), C.byref(to))
+    return out
 
 
 def load_ref():
@@ -90,6 +122,15 @@ def load_ref():
     lib.blt_build_attention_mask.restype = None
     lib.blt_build_attention_mask.argtypes = [C.POINTER(abi.BltMaskConfig), C.POINTER(abi.BltTensor),
                                              C.POINTER(abi.BltArena)]
+    T = C.POINTER(abi.BltTensor)
+    lib.blt_tensor_view_2d.restype = None
+    lib.blt_tensor_view_2d.argtypes = [T, C.c_void_p, C.c_size_t, C.c_size_t, C.c_int]
+    lib.blt_tensor_view_3d.restype = None
+    lib.blt_tensor_view_3d.argtypes = [T, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int]
+    lib.blt_rope_precompute.restype = None
+    lib.blt_rope_precompute.argtypes = [C.c_size_t, C.POINTER(BltRopeConfig), T, T]
+    lib.blt_rope_apply.restype = None
+    lib.blt_rope_apply.argtypes = [T, T, T, T]
     lib.blt_build_block_diffusion_mask.restype = None
     lib.blt_build_block_diffusion_mask.argtypes = [C.POINTER(abi.BltBlockDiffusionConfig),
                                                    C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)]

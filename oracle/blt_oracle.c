@@ -320,3 +320,90 @@ int orc_kv_attend_step(float *self_k, float *self_v, size_t max_seq_len, size_t 
     free(scratch);
     return rc;
 }
+
+/* csrc/ops/reductions_cpu.c:179-197: angle = pos / theta^(2i/head_dim), in float */
+int orc_rope_precompute(size_t max_seq_len, float theta, size_t head_dim, float *cos_out, float *sin_out) {
+    if (head_dim % 2 != 0) return ORC_ERR_ARG;
+    const size_t half = head_dim / 2;
+    for (size_t pos = 0; pos < max_seq_len; pos++) {
+        for (size_t i = 0; i < half; i++) {
+            float freq = 1.0f / powf(theta, (float)(2 * i) / (float)head_dim);
+            float angle = (float)pos * freq;
+            cos_out[pos * half + i] = cosf(angle);
+            sin_out[pos * half + i] = sinf(angle);
+        }
+    }
+    return ORC_OK;
+}
+
+/* csrc/ops/reductions_cpu.c:199-229: x, out are [seq_len, num_heads, head_dim]; row t uses cos/sin row t */
+void orc_rope_apply(const float *x, size_t seq_len, size_t num_heads, size_t head_dim, const float *cos_rows,
+                    const float *sin_rows, float *out) {
+    const size_t half = head_dim / 2;
+    for (size_t t = 0; t < seq_len; t++) {
+        for (size_t h = 0; h < num_heads; h++) {
+            const float *xv = x + (t * num_heads + h) * head_dim;
+            float *ov = out + (t * num_heads + h) * head_dim;
+            const float *c = cos_rows + t * half;
+            const float *s = sin_rows + t * half;
+            for (size_t i = 0; i < half; i++) {
+                float x0 = xv[2 * i];
+                float x1 = xv[2 * i + 1];
+                ov[2 * i] = x0 * c[i] - x1 * s[i];
+                ov[2 * i + 1] = x1 * c[i] + x0 * s[i];
+            }
+        }
+    }
+}
+
+/* csrc/infer/rope_gather.c:5-35: out row i = cache row positions[i] */
+int orc_rope_position_gather(const float *cos_cache, const float *sin_cache, size_t cache_rows, size_t half,
+                             const size_t *positions, size_t n, float *cos_out, float *sin_out) {
+    for (size_t i = 0; i < n; i++)
+        if (positions[i] >= cache_rows) return ORC_ERR_ARG;
+    for (size_t i = 0; i < n; i++) {
+        memcpy(cos_out + i * half, cos_cache + positions[i] * half, half * sizeof(float));
+        memcpy(sin_out + i * half, sin_cache + positions[i] * half, half * sizeof(float));
+    }
+    return ORC_OK;
+}
+
+/* csrc/infer/kv_cache.c:262-271 and 343-390: the new rows arrive un-rotated
+ * (q/k/v rows with their own strides, as slices of the packed QKV rows); per
+ * head Q and K are copied out, rotated at positions base..base+n-1, Q is
+ * collected, rotated K and plain V are written through, then the heads attend. */
+int orc_kv_rope_attend_step(float *self_k, float *self_v, size_t max_seq_len, size_t E, size_t H, size_t b,
+                            size_t base, size_t n, size_t window, const float *q_rows, size_t q_stride,
+                            const float *k_rows, size_t k_stride, const float *v_rows, size_t v_stride,
+                            const float *cos_cache, const float *sin_cache, size_t cache_rows, float *combined) {
+    if (base + n > max_seq_len) return ORC_ERR_CAPACITY;
+    const size_t hd = E / H, half = hd / 2;
+    size_t *positions = (size_t *)malloc(n * sizeof(size_t));
+    float *rc = (float *)malloc(n * half * sizeof(float));
+    float *rs = (float *)malloc(n * half * sizeof(float));
+    float *q_head = (float *)malloc(n * hd * sizeof(float));
+    float *k_head = (float *)malloc(n * hd * sizeof(float));
+    float *q_rot = (float *)malloc(n * hd * sizeof(float));
+    float *k_rot = (float *)malloc(n * hd * sizeof(float));
+    float *q_full = (float *)malloc(n * E * sizeof(float));
+    float *k_full = (float *)malloc(n * E * sizeof(float));
+    float *v_full = (float *)malloc(n * E * sizeof(float));
+    for (size_t r = 0; r < n; r++) positions[r] = base + r;
+    int rcode = orc_rope_position_gather(cos_cache, sin_cache, cache_rows, half, positions, n, rc, rs);
+    if (rcode == ORC_OK) {
+        for (size_t h = 0; h < H; h++) {
+            orc_strided_copy(q_head, hd, q_rows + h * hd, q_stride, n, hd);
+            orc_strided_copy(k_head, hd, k_rows + h * hd, k_stride, n, hd);
+            orc_rope_apply(q_head, n, 1, hd, rc, rs, q_rot);
+            orc_rope_apply(k_head, n, 1, hd, rc, rs, k_rot);
+            orc_strided_copy(q_full + h * hd, E, q_rot, hd, n, hd);
+            orc_strided_copy(k_full + h * hd, E, k_rot, hd, n, hd);
+            orc_strided_copy(v_full + h * hd, E, v_rows + h * hd, v_stride, n, hd);
+        }
+        rcode = orc_kv_attend_step(self_k, self_v, max_seq_len, E, H, b, base, n, window, q_full, k_full, v_full,
+                                   combined);
+    }
+    free(positions), free(rc), free(rs), free(q_head), free(k_head), free(q_rot), free(k_rot);
+    free(q_full), free(k_full), free(v_full);
+    return rcode;
+}

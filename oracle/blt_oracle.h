@@ -33,6 +33,16 @@
  *       csrc/infer/kv_cache.c:343-390, and against the dense causal attention
  *       over the same rows (the reference's cached == dense invariant,
  *       tests/unit/infer/unit_kv_cache.c:136-151).
+ *   orc_rope_precompute, orc_rope_apply, orc_rope_position_gather,
+ *   orc_kv_rope_attend_step
+ *       bit-for-bit against oracle/_ref (blt_rope_precompute_cpu,
+ *       blt_rope_apply_cpu over the same rows); closed forms: position 0 is
+ *       the identity, (cos, sin) = (0, 1) maps (x0, x1) to (-x1, x0) -- the
+ *       forward twin of the reference's backward vector
+ *       (tests/unit/backend/unit_reductions_cpu.c:133-157) --, pair norms are
+ *       preserved, q.k after rotation depends only on the position
+ *       difference; the step against rotating by hand and calling
+ *       orc_kv_attend_step.
  */
 #ifndef FBLT_AMD_ORACLE_H
 #define FBLT_AMD_ORACLE_H
@@ -53,7 +63,8 @@ enum {
     ORC_ERR_ROW_WITHOUT_KEY = 4, /* mask_builder_cpu.c:93, 152 */
     ORC_ERR_BAD_BLOCK_CONFIG = 5,/* mask_builder_cpu.c:105-119 */
     ORC_ERR_PATCH_TILING = 6,    /* patch_pool_cpu.c:107-111 */
-    ORC_ERR_CAPACITY = 7         /* kv_cache.c:191 */
+    ORC_ERR_CAPACITY = 7,        /* kv_cache.c:191 */
+    ORC_ERR_ARG = 8              /* reductions_cpu.c:181, rope_gather.c:21-25 */
 };
 
 /* csrc/ops/vecmath_cpu.c:6-14 */
@@ -125,6 +136,28 @@ void orc_kv_cross_mask(float *out, const size_t *q_group_ids, size_t n, const si
 int orc_kv_attend_step(float *self_k, float *self_v, size_t max_seq_len, size_t embed_dim, size_t num_heads,
                        size_t b, size_t base, size_t n, size_t window, const float *q_rows,
                        const float *k_rows, const float *v_rows, float *combined);
+
+/* RoPE tables, reductions_cpu.c:179-197: cos_out / sin_out are [max_seq_len, head_dim/2]. */
+int orc_rope_precompute(size_t max_seq_len, float theta, size_t head_dim, float *cos_out, float *sin_out);
+
+/* reductions_cpu.c:199-229: rotate pairs (2i, 2i+1) of every head of row t by
+ * the angle in cos/sin row t.  x and out are [seq_len, num_heads, head_dim]. */
+void orc_rope_apply(const float *x, size_t seq_len, size_t num_heads, size_t head_dim, const float *cos_rows,
+                    const float *sin_rows, float *out);
+
+/* rope_gather.c:5-35: out row i = cache row positions[i]; ORC_ERR_ARG when a position is past the cache. */
+int orc_rope_position_gather(const float *cos_cache, const float *sin_cache, size_t cache_rows, size_t half,
+                             const size_t *positions, size_t n, float *cos_out, float *sin_out);
+
+/* One decode step for one sequence including the rotation, kv_cache.c:262-271
+ * and 343-390: the n new Q/K/V rows arrive un-rotated with their own row
+ * strides (slices of the packed QKV rows); Q and K are rotated per head at
+ * positions base..base+n-1, rotated K and V are written through, then the
+ * heads attend as in orc_kv_attend_step. */
+int orc_kv_rope_attend_step(float *self_k, float *self_v, size_t max_seq_len, size_t embed_dim, size_t num_heads,
+                            size_t b, size_t base, size_t n, size_t window, const float *q_rows, size_t q_stride,
+                            const float *k_rows, size_t k_stride, const float *v_rows, size_t v_stride,
+                            const float *cos_cache, const float *sin_cache, size_t cache_rows, float *combined);
 
 #ifdef __cplusplus
 }

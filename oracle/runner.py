@@ -118,6 +118,17 @@ def run_kv(kw, lib=None, steps=None, timed=False):
             v = np.ascontiguousarray(kw.v_new[s, rows])
             comb = out[s, rows]
             base = int(lens[b])
+            if kw.rope_cos is not None and kw.kind == "causal":
+                rc = lib.orc_kv_rope_attend_step(binding.fptr(ck.reshape(-1)), binding.fptr(cv.reshape(-1)),
+                                                 kw.max_seq_len, E, H, b, base, n, kw.window, binding.fptr(q), E,
+                                                 binding.fptr(k), E, binding.fptr(v), E,
+                                                 binding.fptr(kw.rope_cos.reshape(-1)),
+                                                 binding.fptr(kw.rope_sin.reshape(-1)), kw.rope_cos.shape[0],
+                                                 binding.fptr(comb.reshape(-1)))
+                assert rc == 0, rc
+                continue
+            if kw.rope_cos is not None:
+                q, k = _rotate_rows(lib, kw, base, q), _rotate_rows(lib, kw, base, k)
             if kw.kind == "causal":
                 rc = lib.orc_kv_attend_step(binding.fptr(ck.reshape(-1)), binding.fptr(cv.reshape(-1)),
                                             kw.max_seq_len, E, H, b, base, n, kw.window, binding.fptr(q),
@@ -129,6 +140,21 @@ def run_kv(kw, lib=None, steps=None, timed=False):
         if kw.commit:
             lens += n
     return (out, ck, cv, elapsed) if timed else (out, ck, cv)
+
+
+def _rotate_rows(lib, kw, base, x):
+    """Rows [n, E] at positions base..base+n-1 rotated head by head
+    (csrc/infer/kv_cache.c:262-271, 349-358; block rows: models/block_diffusion.c:264-277)."""
+    n, H, hd = x.shape[0], kw.H, kw.hd
+    half = hd // 2
+    pos = abi.size_array(range(base, base + n))
+    rc, rs = np.empty(n * half, dtype=np.float32), np.empty(n * half, dtype=np.float32)
+    assert lib.orc_rope_position_gather(binding.fptr(kw.rope_cos.reshape(-1)), binding.fptr(kw.rope_sin.reshape(-1)),
+                                        kw.rope_cos.shape[0], half, pos, n, binding.fptr(rc), binding.fptr(rs)) == 0
+    out = np.empty_like(x)
+    lib.orc_rope_apply(binding.fptr(np.ascontiguousarray(x).reshape(-1)), n, H, hd, binding.fptr(rc), binding.fptr(rs),
+                       binding.fptr(out.reshape(-1)))
+    return out
 
 
 def _block_rows(lib, kw, ck, cv, b, base, q, k, v, comb):

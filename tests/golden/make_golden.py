@@ -42,6 +42,8 @@ KV_CASES = {
     "c5_B4": lambda: workloads.config5(B=4),
     "c5_B8": lambda: workloads.config5(B=8),
     "c5_B16": lambda: workloads.config5(B=16),
+    "c4_rope_small": lambda: workloads.config4(batch=5, steps=6, len_hi=90, rope=True),
+    "c5_B8_rope_small": lambda: workloads.config5(batch=4, B=8, len_hi=120, max_seq_len=160, rope=True),
 }
 
 
@@ -100,6 +102,12 @@ def run_kv(ref, kw):
             q = np.ascontiguousarray(kw.q_new[s, b * n:(b + 1) * n])
             k = np.ascontiguousarray(kw.k_new[s, b * n:(b + 1) * n])
             v = np.ascontiguousarray(kw.v_new[s, b * n:(b + 1) * n])
+            if kw.rope_cos is not None:
+                # kv_cache.c:262-271, 349-358: rows of the tables at positions base..base+n-1 (the position
+                # gather is a row copy), then the reference's blt_rope_apply on Q and K
+                rc, rs = kw.rope_cos[base:base + n], kw.rope_sin[base:base + n]
+                q = binding.ref_rope_apply(ref, q.reshape(n, H, hd), rc, rs).reshape(n, E)
+                k = binding.ref_rope_apply(ref, k.reshape(n, H, hd), rc, rs).reshape(n, E)
             for h in range(H):   # write-through first (kv_cache.c:363-365)
                 for dst, src in ((kd, k), (vd, v)):
                     ref.blt_strided_copy(CPU, C.cast(dst.ctypes.data + 4 * (slab + base * E + h * hd), _fp), E,

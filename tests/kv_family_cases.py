@@ -1,0 +1,67 @@
+"""Runs a fixed list of KV-cache step cases through blt_kv_attend_step_hip /
+blt_kv_rope_attend_step_hip and checks each against the CPU checker.  Not
+collected by pytest: test_gpu_parity.py starts it in a fresh process per
+kernel (VALU or matrix-core), because the library reads BLT_HIP_BLOCK_KERNEL
+once per process.
+
+Outputs: |got - ref| <= 1e-5 + 1e-4 * |ref|; cache contents bit for bit.
+"""
+import os
+import sys
+
+import numpy as np
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+
+from fblt_amd import runner, workloads  # noqa: E402
+from oracle import binding, runner as orunner  # noqa: E402
+
+
+def chunked(n, rope, hd=32, window=0):
+    """n new rows per sequence and step, causal within the chunk (prefill chunks)."""
+    kw = workloads.config4(batch=9, steps=2, H=4 if hd == 32 else 2, hd=hd, len_hi=150, max_seq_len=150 + 2 * n,
+                           rope=rope)
+    rs = np.random.RandomState(n)
+    kw.n = n
+    kw.window = window
+    kw.q_new, kw.k_new, kw.v_new = (rs.randn(kw.steps, kw.batch * n, kw.E).astype(np.float32) for _ in range(3))
+    return kw
+
+
+CASES = {
+    "block4": lambda: workloads.config5(batch=9, B=4),
+    "block16": lambda: workloads.config5(batch=9, B=16),
+    "block32": lambda: workloads.config5(batch=9, B=32),
+    "chunk3": lambda: chunked(3, False),
+    "chunk12": lambda: chunked(12, False),
+    "decode_rope": lambda: workloads.config4(batch=7, steps=4, len_hi=200, rope=True),
+    "chunk3_rope": lambda: chunked(3, True),
+    "chunk12_rope": lambda: chunked(12, True),
+    "chunk20_rope_hd64": lambda: chunked(20, True, hd=64),
+    "chunk6_rope_window": lambda: chunked(6, True, window=40),
+    "block8_rope": lambda: workloads.config5(batch=9, B=8, rope=True),
+    "block16_rope_hd64": lambda: workloads.config5(batch=5, B=16, H=2, hd=64, rope=True),
+}
+
+
+def main():
+    orc = binding.load_oracle()
+    for name, make in CASES.items():
+        print("case", name, flush=True)
+        kw = make()
+        ref_out, ref_k, ref_v = orunner.run_kv(kw, lib=orc)
+        d = runner.DeviceKvWorkload(kw)
+        d.run()
+        out, ck, cv, lens = d.results()
+        if ck.tobytes() != ref_k.tobytes() or cv.tobytes() != ref_v.tobytes():
+            print("FAIL %s: cache contents differ" % name)
+            sys.exit(1)
+        err = np.abs(out.astype(np.float64) - ref_out)
+        if not (err <= 1e-5 + 1e-4 * np.abs(ref_out)).all():
+            print("FAIL %s: max err %.3e" % (name, float(err.max())))
+            sys.exit(1)
+    print("OK")
+
+
+if __name__ == "__main__":
+    main()

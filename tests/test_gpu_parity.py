@@ -412,40 +412,18 @@ def test_strided_copy_softmax_dot(oracle, dev):
 
 
 @pytest.mark.parametrize("kernel", ["valu", "mfma"])
-@pytest.mark.parametrize("kind,n", [("block", 4), ("block", 16), ("causal", 3), ("causal", 12), ("block", 32)])
-def test_kv_step_kernel_families_agree(kernel, kind, n, oracle):
-    """Both kernels behind blt_kv_attend_step_hip (VALU and matrix-core) on the same step,
-    pinned through BLT_HIP_BLOCK_KERNEL in a fresh process (the hook is read once)."""
+def test_kv_step_kernel_families_agree(kernel):
+    """Both kernels behind the KV step entry points (VALU and matrix-core) on the same cases -- block
+    rows, prefill chunks, rotation fused in or not -- pinned through BLT_HIP_BLOCK_KERNEL in a fresh
+    process (the hook is read once)."""
     import subprocess
     import sys
     import os
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    code = """
-import sys
-sys.path.insert(0, %r)
-import numpy as np
-from fblt_amd import workloads, runner
-from oracle import runner as orunner
-kind, n = %r, %d
-if kind == "block":
-    kw = workloads.config5(batch=9, B=n)
-else:
-    kw = workloads.config4(batch=9, steps=2, len_hi=150, max_seq_len=150 + 2 * n)
-    rs = np.random.RandomState(n)
-    kw.n = n
-    kw.q_new, kw.k_new, kw.v_new = (rs.randn(kw.steps, kw.batch * n, kw.E).astype(np.float32) for _ in range(3))
-ref_out, ref_k, ref_v = orunner.run_kv(kw)
-d = runner.DeviceKvWorkload(kw)
-d.run()
-out, ck, cv, lens = d.results()
-assert ck.tobytes() == ref_k.tobytes() and cv.tobytes() == ref_v.tobytes()
-err = np.abs(out.astype(np.float64) - ref_out)
-assert (err <= 1e-5 + 1e-4 * np.abs(ref_out)).all(), float(err.max())
-print("OK", float(err.max()))
-""" % (root, kind, n)
+    here = os.path.dirname(os.path.abspath(__file__))
     env = dict(os.environ, BLT_HIP_BLOCK_KERNEL=kernel)
-    p = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300, env=env)
-    assert p.returncode == 0 and "OK" in p.stdout, p.stdout + p.stderr
+    p = subprocess.run([sys.executable, "-u", os.path.join(here, "kv_family_cases.py")], capture_output=True,
+                       text=True, timeout=600, env=env)
+    assert p.returncode == 0 and "OK" in p.stdout, p.stdout[-2000:] + p.stderr[-2000:]
 
 
 @pytest.mark.parametrize("family", ["rows", "mfma", "wide"])
@@ -462,3 +440,39 @@ def test_attention_kernel_families(family):
     assert p.returncode == 0 and "OK" in p.stdout, p.stdout[-2000:] + p.stderr[-2000:]
     kernels = [ln for ln in p.stdout.splitlines() if ln.startswith("KERNELS")][0].split()[1]
     assert kernels == family, kernels
+
+
+@pytest.mark.parametrize("case", ["decode", "chunk5", "block16", "packed"])
+def test_kv_rope_step(case, oracle, dev):
+    """blt_kv_rope_attend_step_hip: rotation of the new Q/K rows fused into the step.  Rotated K rows
+    land in the cache bit for bit as the reference's blt_rope_apply writes them."""
+    import torch
+    if case == "decode":
+        kw = workloads.config4(batch=11, steps=6, len_hi=300, rope=True)
+    elif case == "chunk5":
+        kw = workloads.config4(batch=6, steps=3, len_hi=100, max_seq_len=100 + 15, rope=True)
+        rs = np.random.RandomState(5)
+        kw.n = 5
+        kw.q_new, kw.k_new, kw.v_new = (rs.randn(kw.steps, kw.batch * 5, kw.E).astype(np.float32) for _ in range(3))
+    elif case == "block16":
+        kw = workloads.config5(batch=8, B=16, rope=True)
+    else:
+        kw = workloads.config4(batch=4, steps=1, len_hi=60, rope=True)
+    ref_out, ref_k, ref_v = orunner.run_kv(kw, lib=oracle)
+    d = dev.DeviceKvWorkload(kw)
+    if case == "packed":
+        # the three column blocks of one packed [batch*n, 3E] buffer, row stride 3E
+        E = kw.E
+        qkv = torch.from_numpy(np.concatenate([kw.q_new[0], kw.k_new[0], kw.v_new[0]], axis=1)).cuda()
+        d.lib.blt_kv_rope_attend_step_hip(C.byref(d.c), qkv.data_ptr(), 3 * E, qkv.data_ptr() + 4 * E, 3 * E,
+                                          qkv.data_ptr() + 8 * E, 3 * E, d.rope[0].data_ptr(), d.rope[1].data_ptr(),
+                                          d.rope[0].shape[0], d.out[0].data_ptr(), E, kw.n, d.kind, 1,
+                                          d.host_max_len + kw.n)
+        d.lib.blt_backend_pass_sync_hip()
+    else:
+        d.run()
+    out, ck, cv, lens = d.results()
+    assert ck.tobytes() == ref_k.tobytes() and cv.tobytes() == ref_v.tobytes()
+    assert_close(out, ref_out, "rope " + case)
+    if kw.commit:
+        assert (lens == kw.lens + kw.n * kw.steps).all()

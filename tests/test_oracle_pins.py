@@ -305,3 +305,116 @@ def test_kv_cached_equals_dense(chunks, window, oracle):
     assert oracle.orc_kv_attend_step(binding.fptr(ck.reshape(-1)), binding.fptr(cv.reshape(-1)), max_len, E, H, 1,
                                      T, 4, 0, binding.fptr(q), binding.fptr(k), binding.fptr(v),
                                      binding.fptr(got.reshape(-1))) == 7   # over capacity
+
+
+# ---------------------------------------------------------------------------
+# RoPE (csrc/ops/reductions_cpu.c:179-229, csrc/infer/rope_gather.c)
+# ---------------------------------------------------------------------------
+def _rope_apply(oracle, x, c, s):
+    rows, heads, hd = x.shape
+    out = np.empty_like(x)
+    oracle.orc_rope_apply(binding.fptr(x.reshape(-1)), rows, heads, hd, binding.fptr(c.reshape(-1)),
+                          binding.fptr(s.reshape(-1)), binding.fptr(out.reshape(-1)))
+    return out
+
+
+def test_rope_tables_against_float64(oracle):
+    """angle = pos / theta^(2i/hd): position 0 is (1, 0), band 0 turns by one radian per position,
+    every entry within float rounding of the float64 value."""
+    for hd, theta, n in ((32, 500000.0, 300), (64, 10000.0, 50), (2, 500000.0, 9)):
+        half = hd // 2
+        c, s = np.empty(n * half, dtype=np.float32), np.empty(n * half, dtype=np.float32)
+        assert oracle.orc_rope_precompute(n, theta, hd, binding.fptr(c), binding.fptr(s)) == 0
+        c, s = c.reshape(n, half), s.reshape(n, half)
+        assert (c[0] == 1.0).all() and (s[0] == 0.0).all()
+        assert abs(c[1, 0] - np.cos(1.0)) < 1e-7 and abs(s[1, 0] - np.sin(1.0)) < 1e-7
+        i = np.arange(half, dtype=np.float64)
+        ang = np.arange(n, dtype=np.float64)[:, None] / np.power(theta, 2.0 * i / hd)[None, :]
+        # the float angle carries a relative error of ~2^-23, i.e. up to pos * 2^-23 absolute
+        tol = 4e-7 + np.arange(n)[:, None] * 3e-7
+        assert (np.abs(c - np.cos(ang)) < tol).all() and (np.abs(s - np.sin(ang)) < tol).all()
+    assert oracle.orc_rope_precompute(4, 500000.0, 3, binding.fptr(c.reshape(-1)), binding.fptr(s.reshape(-1))) != 0
+
+
+def test_rope_apply_closed_forms(oracle):
+    rs = np.random.RandomState(3)
+    x = rs.randn(5, 3, 8).astype(np.float32)
+    one, zero = np.ones((5, 4), dtype=np.float32), np.zeros((5, 4), dtype=np.float32)
+    # angle 0: identity, bit for bit
+    assert _rope_apply(oracle, x, one, zero).tobytes() == x.tobytes()
+    # quarter turn (cos, sin) = (0, 1): (x0, x1) -> (-x1, x0); the forward twin of the reference's
+    # backward vector (tests/unit/backend/unit_reductions_cpu.c:133-157: grad (1, 0) -> (0, -1))
+    q = _rope_apply(oracle, x, zero, one)
+    assert (q[..., 0::2] == -x[..., 1::2]).all() and (q[..., 1::2] == x[..., 0::2]).all()
+    back = _rope_apply(oracle, np.array([[[0.0, -1.0]]], dtype=np.float32), zero[:1, :1], one[:1, :1])
+    assert back.reshape(-1).tolist() == [1.0, 0.0]
+    # general angle against float64, pair norms preserved, rows use their own table row
+    ang = rs.rand(5, 4) * 6.0
+    c, s = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    y = _rope_apply(oracle, x, c, s).astype(np.float64)
+    x64, c64, s64 = x.astype(np.float64), c.astype(np.float64)[:, None, :], s.astype(np.float64)[:, None, :]
+    want0 = x64[..., 0::2] * c64 - x64[..., 1::2] * s64
+    want1 = x64[..., 1::2] * c64 + x64[..., 0::2] * s64
+    assert np.abs(y[..., 0::2] - want0).max() < 1e-6 and np.abs(y[..., 1::2] - want1).max() < 1e-6
+    n_in = x64[..., 0::2] ** 2 + x64[..., 1::2] ** 2
+    n_out = y[..., 0::2] ** 2 + y[..., 1::2] ** 2
+    assert np.abs(n_in - n_out).max() < 1e-5
+
+
+def test_rope_scores_depend_on_position_difference(oracle):
+    """q.k after rotating q at position p+d and k at position p equals the same for (d, 0)."""
+    hd, n = 16, 64
+    half = hd // 2
+    c, s = np.empty(n * half, dtype=np.float32), np.empty(n * half, dtype=np.float32)
+    oracle.orc_rope_precompute(n, 100.0, hd, binding.fptr(c), binding.fptr(s))
+    c, s = c.reshape(n, half), s.reshape(n, half)
+    rs = np.random.RandomState(4)
+    q, k = rs.randn(1, 1, hd).astype(np.float32), rs.randn(1, 1, hd).astype(np.float32)
+    def score(pq, pk):
+        a = _rope_apply(oracle, q, c[pq:pq + 1], s[pq:pq + 1]).astype(np.float64)
+        b = _rope_apply(oracle, k, c[pk:pk + 1], s[pk:pk + 1]).astype(np.float64)
+        return float((a * b).sum())
+    for d in (0, 1, 7):
+        base = score(d, 0)
+        for p in (3, 20, 50):
+            assert abs(score(p + d, p) - base) < 2e-4, (d, p)
+
+
+def test_rope_gather_and_step_composition(oracle):
+    """The gather copies table rows; the rotating step equals rotating by hand and calling the plain step."""
+    rs = np.random.RandomState(6)
+    H, hd, max_len, batch = 2, 8, 30, 2
+    E, half = H * hd, hd // 2
+    c, s = np.empty(max_len * half, dtype=np.float32), np.empty(max_len * half, dtype=np.float32)
+    oracle.orc_rope_precompute(max_len, 500000.0, hd, binding.fptr(c), binding.fptr(s))
+    pos = abi.size_array([7, 0, 29])
+    gc, gs = np.empty(3 * half, dtype=np.float32), np.empty(3 * half, dtype=np.float32)
+    assert oracle.orc_rope_position_gather(binding.fptr(c), binding.fptr(s), max_len, half, pos, 3, binding.fptr(gc),
+                                           binding.fptr(gs)) == 0
+    assert (gc.reshape(3, half) == c.reshape(max_len, half)[[7, 0, 29]]).all()
+    assert (gs.reshape(3, half) == s.reshape(max_len, half)[[7, 0, 29]]).all()
+    assert oracle.orc_rope_position_gather(binding.fptr(c), binding.fptr(s), max_len, half, abi.size_array([30]), 1,
+                                           binding.fptr(gc), binding.fptr(gs)) != 0
+    ck1 = rs.randn(batch * max_len, E).astype(np.float32)
+    cv1 = rs.randn(batch * max_len, E).astype(np.float32)
+    ck2, cv2 = ck1.copy(), cv1.copy()
+    for b, base, n, window in ((0, 4, 1, 0), (1, 9, 5, 0), (0, 5, 3, 4)):
+        qkv = rs.randn(n, 3 * E).astype(np.float32)   # packed rows: strides 3E
+        mine = np.zeros((n, E), dtype=np.float32)
+        f = qkv.reshape(-1)
+        rc = oracle.orc_kv_rope_attend_step(
+            binding.fptr(ck1.reshape(-1)), binding.fptr(cv1.reshape(-1)), max_len, E, H, b, base, n, window,
+            binding.fptr(f), 3 * E, C.cast(f.ctypes.data + 4 * E, binding._fp), 3 * E,
+            C.cast(f.ctypes.data + 8 * E, binding._fp), 3 * E, binding.fptr(c), binding.fptr(s), max_len,
+            binding.fptr(mine.reshape(-1)))
+        assert rc == 0
+        tc, ts = c.reshape(max_len, half)[base:base + n].copy(), s.reshape(max_len, half)[base:base + n].copy()
+        q = _rope_apply(oracle, np.ascontiguousarray(qkv[:, :E]).reshape(n, H, hd), tc, ts).reshape(n, E)
+        k = _rope_apply(oracle, np.ascontiguousarray(qkv[:, E:2 * E]).reshape(n, H, hd), tc, ts).reshape(n, E)
+        v = np.ascontiguousarray(qkv[:, 2 * E:])
+        theirs = np.zeros((n, E), dtype=np.float32)
+        assert oracle.orc_kv_attend_step(binding.fptr(ck2.reshape(-1)), binding.fptr(cv2.reshape(-1)), max_len, E, H,
+                                         b, base, n, window, binding.fptr(q), binding.fptr(k), binding.fptr(v),
+                                         binding.fptr(theirs.reshape(-1))) == 0
+        assert mine.tobytes() == theirs.tobytes()
+        assert ck1.tobytes() == ck2.tobytes() and cv1.tobytes() == cv2.tobytes()

@@ -189,3 +189,79 @@ def test_kv_step_against_reference_op_sequence(oracle, ref):
             ref.blt_attention_head_core(CPU, C.byref(a))
         assert mine.tobytes() == theirs.tobytes()
         assert ck1.tobytes() == ck2.tobytes() and cv1.tobytes() == cv2.tobytes()
+
+
+def test_rope_bit_exact(oracle, ref):
+    """orc_rope_precompute / orc_rope_apply against blt_rope_precompute / blt_rope_apply of the
+    reference (csrc/ops/reductions_cpu.c:179-229)."""
+    for hd, theta, n in ((32, 500000.0, 700), (64, 500000.0, 300), (8, 10000.0, 40)):
+        half = hd // 2
+        c1, s1 = np.empty(n * half, dtype=np.float32), np.empty(n * half, dtype=np.float32)
+        assert oracle.orc_rope_precompute(n, theta, hd, binding.fptr(c1), binding.fptr(s1)) == 0
+        c2, s2 = np.empty(n * half, dtype=np.float32), np.empty(n * half, dtype=np.float32)
+        tc, ts = abi.BltTensor(), abi.BltTensor()
+        ref.blt_tensor_view_2d(C.byref(tc), c2.ctypes.data, n, half, CPU)
+        ref.blt_tensor_view_2d(C.byref(ts), s2.ctypes.data, n, half, CPU)
+        cfg = binding.BltRopeConfig(theta, hd)
+        ref.blt_rope_precompute(n, C.byref(cfg), C.byref(tc), C.byref(ts))
+        assert c1.tobytes() == c2.tobytes() and s1.tobytes() == s2.tobytes()
+        rs = np.random.RandomState(hd)
+        x = rs.randn(n, 3, hd).astype(np.float32)
+        mine = np.empty_like(x)
+        oracle.orc_rope_apply(binding.fptr(x.reshape(-1)), n, 3, hd, binding.fptr(c1), binding.fptr(s1),
+                              binding.fptr(mine.reshape(-1)))
+        theirs = binding.ref_rope_apply(ref, x, c2.reshape(n, half), s2.reshape(n, half))
+        assert mine.tobytes() == theirs.tobytes()
+
+
+def test_kv_rope_step_against_reference_op_sequence(oracle, ref):
+    """orc_kv_rope_attend_step against the reference's ops in the order of kv_cache.c:343-366:
+    per head copy Q and K out of the packed rows, blt_rope_apply both at positions base..base+n-1,
+    copy rotated Q into q_full and rotated K / plain V into the slab; then the (separately pinned)
+    attention of the plain step."""
+    rs = np.random.RandomState(12)
+    H, hd, max_len, batch = 4, 8, 40, 2
+    E, half = H * hd, hd // 2
+    cos, sin = np.empty(max_len * half, dtype=np.float32), np.empty(max_len * half, dtype=np.float32)
+    oracle.orc_rope_precompute(max_len, 500000.0, hd, binding.fptr(cos), binding.fptr(sin))
+    ck1 = rs.randn(batch * max_len, E).astype(np.float32)
+    cv1 = rs.randn(batch * max_len, E).astype(np.float32)
+    ck2, cv2 = ck1.copy(), cv1.copy()
+    fp = C.POINTER(C.c_float)
+    for b, base, n, window in [(0, 0, 1, 0), (1, 5, 1, 0), (0, 7, 6, 0), (1, 6, 3, 4)]:
+        qkv = rs.randn(n, 3 * E).astype(np.float32)
+        f = qkv.reshape(-1)
+        mine = np.zeros((n, E), dtype=np.float32)
+        assert oracle.orc_kv_rope_attend_step(
+            binding.fptr(ck1.reshape(-1)), binding.fptr(cv1.reshape(-1)), max_len, E, H, b, base, n, window,
+            binding.fptr(f), 3 * E, C.cast(f.ctypes.data + 4 * E, fp), 3 * E, C.cast(f.ctypes.data + 8 * E, fp), 3 * E,
+            binding.fptr(cos), binding.fptr(sin), max_len, binding.fptr(mine.reshape(-1))) == 0
+        rc = cos.reshape(max_len, half)[base:base + n].copy()
+        rsn = sin.reshape(max_len, half)[base:base + n].copy()
+        q_full = np.zeros((n, E), dtype=np.float32)
+        kd, vd = ck2.reshape(-1), cv2.reshape(-1)
+        slab = b * max_len * E
+        for h in range(H):
+            q_head, k_head = np.empty((n, hd), dtype=np.float32), np.empty((n, hd), dtype=np.float32)
+            ref.blt_strided_copy(CPU, binding.fptr(q_head.reshape(-1)), hd, C.cast(f.ctypes.data + 4 * h * hd, fp),
+                                 3 * E, n, hd)
+            ref.blt_strided_copy(CPU, binding.fptr(k_head.reshape(-1)), hd,
+                                 C.cast(f.ctypes.data + 4 * (E + h * hd), fp), 3 * E, n, hd)
+            q_rot = binding.ref_rope_apply(ref, q_head.reshape(n, 1, hd), rc, rsn).reshape(n, hd)
+            k_rot = binding.ref_rope_apply(ref, k_head.reshape(n, 1, hd), rc, rsn).reshape(n, hd)
+            ref.blt_strided_copy(CPU, C.cast(q_full.ctypes.data + 4 * h * hd, fp), E, binding.fptr(q_rot.reshape(-1)),
+                                 hd, n, hd)
+            ref.blt_strided_copy(CPU, C.cast(kd.ctypes.data + 4 * (slab + base * E + h * hd), fp), E,
+                                 binding.fptr(k_rot.reshape(-1)), hd, n, hd)
+            ref.blt_strided_copy(CPU, C.cast(vd.ctypes.data + 4 * (slab + base * E + h * hd), fp), E,
+                                 C.cast(f.ctypes.data + 4 * (2 * E + h * hd), fp), 3 * E, n, hd)
+        assert ck1.tobytes() == ck2.tobytes() and cv1.tobytes() == cv2.tobytes()
+        # attention over the slab with the rotated Q: rows already in place, so re-writing them is a no-op
+        k_rows = np.ascontiguousarray(ck2.reshape(batch, max_len, E)[b, base:base + n])
+        v_rows = np.ascontiguousarray(cv2.reshape(batch, max_len, E)[b, base:base + n])
+        theirs = np.zeros((n, E), dtype=np.float32)
+        assert oracle.orc_kv_attend_step(binding.fptr(ck2.reshape(-1)), binding.fptr(cv2.reshape(-1)), max_len, E, H,
+                                         b, base, n, window, binding.fptr(q_full.reshape(-1)),
+                                         binding.fptr(k_rows.reshape(-1)), binding.fptr(v_rows.reshape(-1)),
+                                         binding.fptr(theirs.reshape(-1))) == 0
+        assert mine.tobytes() == theirs.tobytes()
