@@ -91,6 +91,24 @@ class BltBlockDiffusionConfig(C.Structure):
     ]
 
 
+class BltRopeConfig(C.Structure):
+    _fields_ = [("theta", C.c_float), ("head_dim", C.c_size_t)]
+
+
+class BltAttentionConfig(C.Structure):
+    _fields_ = [
+        ("embed_dim", C.c_size_t),
+        ("num_heads", C.c_size_t),
+        ("head_dim", C.c_size_t),
+        ("is_causal", C.c_bool),
+        ("use_rope", C.c_bool),
+        ("rope_theta", C.c_float),
+        ("rope_cos_cache", C.POINTER(BltTensor)),
+        ("rope_sin_cache", C.POINTER(BltTensor)),
+        ("mask_config", C.POINTER(BltMaskConfig)),
+    ]
+
+
 class BltPatchInfo(C.Structure):
     _fields_ = [
         ("start_idx", C.c_size_t),
@@ -110,6 +128,24 @@ def check_layout():
     assert BltMaskConfig.causal_offset.offset == 64
     assert C.sizeof(BltBlockDiffusionConfig) == 48
     assert C.sizeof(BltPatchInfo) == 24
+    assert C.sizeof(BltRopeConfig) == 16 and BltRopeConfig.head_dim.offset == 8
+    assert C.sizeof(BltAttentionConfig) == 56 and BltAttentionConfig.rope_theta.offset == 28
+    assert BltAttentionConfig.mask_config.offset == 48
+
+
+def tensor_view(ptr, shape, backend, dtype=BLT_DTYPE_FP32):
+    """A row-major blt_tensor view of existing memory (csrc/core/tensor.c:48-75)."""
+    t = BltTensor()
+    t.data = ptr
+    numel, stride = 1, 1
+    for d in range(len(shape)):
+        t.shape[d] = shape[d]
+        numel *= shape[d]
+    for d in reversed(range(len(shape))):
+        t.strides[d] = stride
+        stride *= shape[d]
+    t.ndim, t.numel, t.dtype, t.backend, t.is_view = len(shape), numel, dtype, backend, True
+    return t
 
 
 check_layout()

@@ -104,6 +104,20 @@ SYMBOLS = {
     "blt_kv_rope_attend_step_hip": (None, [C.POINTER(BltKvAttnCache), C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t,
                                            C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p,
                                            C.c_size_t, C.c_size_t, C.c_int, C.c_int, C.c_size_t]),
+    "blt_matmul_hip": (None, [C.POINTER(abi.BltTensor)] * 3),
+    "blt_matmul": (None, [C.POINTER(abi.BltTensor)] * 3),
+    "blt_rope_apply_hip": (None, [C.POINTER(abi.BltTensor)] * 4),
+    "blt_rope_apply": (None, [C.POINTER(abi.BltTensor)] * 4),
+    "blt_rope_apply_packed_hip": (None, [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p,
+                                         C.c_void_p]),
+    "blt_rope_apply_packed": (None, [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p,
+                                     C.c_void_p, C.c_int]),
+    "blt_rope_precompute": (None, [C.c_size_t, C.POINTER(abi.BltRopeConfig), C.POINTER(abi.BltTensor),
+                                   C.POINTER(abi.BltTensor)]),
+    "blt_multihead_attention_hip": (None, [C.POINTER(abi.BltTensor)] * 4 + [C.POINTER(abi.BltAttentionConfig),
+                                                                           C.POINTER(abi.BltArena)]),
+    "blt_multihead_attention": (None, [C.POINTER(abi.BltTensor)] * 4 + [C.POINTER(abi.BltAttentionConfig),
+                                                                       C.POINTER(abi.BltArena)]),
     "blt_hip_profile_begin": (None, []),
     "blt_hip_profile_end": (C.c_size_t, [C.POINTER(BltHipKernelTime), C.c_size_t]),
     "blt_hip_stream_copy_probe": (None, [C.c_void_p, C.c_void_p, C.c_size_t]),

@@ -9,6 +9,7 @@
 #include "blt_hip.h"
 #include "blt_fatal.h"
 
+#include <math.h>
 #include <stdlib.h>
 #include <string.h>
 
@@ -156,6 +157,62 @@ void blt_softmax_masked_row_inplace(blt_backend backend, float *row, size_t row_
                                     const float *mask_row, float scale) {
     BLT_DEVICE_ONLY(backend, "blt_softmax_masked_row_inplace");
     blt_softmax_masked_row_inplace_hip(backend, row, row_len, row_idx, is_causal, mask_row, scale);
+}
+
+void blt_matmul(const blt_tensor *a, const blt_tensor *b, blt_tensor *out) {
+    BLT_REQUIRE(a != NULL, "matmul: inputs must not be NULL");
+    BLT_DEVICE_ONLY(a->backend, "blt_matmul");
+    blt_matmul_hip(a, b, out);
+}
+
+void blt_rope_precompute(size_t max_seq_len, const blt_rope_config *config, blt_tensor *cos_out, blt_tensor *sin_out) {
+    BLT_REQUIRE(config != NULL && cos_out != NULL && sin_out != NULL, "rope: arguments must not be NULL");
+    BLT_DEVICE_ONLY(cos_out->backend, "blt_rope_precompute");
+    BLT_REQUIRE(config->head_dim % 2 == 0, "rope: head_dim must be even");
+    const size_t half = config->head_dim / 2;
+    BLT_REQUIRE(cos_out->ndim == 2 && cos_out->dtype == BLT_DTYPE_FP32 && cos_out->shape[0] == max_seq_len &&
+                    cos_out->shape[1] == half,
+                "rope cos_out");
+    BLT_REQUIRE(sin_out->ndim == 2 && sin_out->dtype == BLT_DTYPE_FP32 && sin_out->shape[0] == max_seq_len &&
+                    sin_out->shape[1] == half && sin_out->backend == cos_out->backend,
+                "rope sin_out");
+    if (max_seq_len * half == 0) return;
+    float *c = (float *)malloc(max_seq_len * half * sizeof(float));
+    float *s = (float *)malloc(max_seq_len * half * sizeof(float));
+    BLT_REQUIRE(c != NULL && s != NULL, "rope: failed to allocate host staging");
+    /* the reference's formula and libm calls, csrc/ops/reductions_cpu.c:188-196 */
+    for (size_t pos = 0; pos < max_seq_len; pos++) {
+        for (size_t i = 0; i < half; i++) {
+            float freq = 1.0f / powf(config->theta, (float)(2 * i) / (float)config->head_dim);
+            float angle = (float)pos * freq;
+            c[pos * half + i] = cosf(angle);
+            s[pos * half + i] = sinf(angle);
+        }
+    }
+    blt_hip_memcpy_h2d(cos_out->data, c, max_seq_len * half * sizeof(float));
+    blt_hip_memcpy_h2d(sin_out->data, s, max_seq_len * half * sizeof(float));
+    blt_backend_pass_sync_hip(); /* the staging buffers are freed next */
+    free(c);
+    free(s);
+}
+
+void blt_rope_apply(const blt_tensor *x, const blt_tensor *cos, const blt_tensor *sin, blt_tensor *out) {
+    BLT_REQUIRE(x != NULL, "rope: x must be 3D FP32");
+    BLT_DEVICE_ONLY(x->backend, "blt_rope_apply");
+    blt_rope_apply_hip(x, cos, sin, out);
+}
+
+void blt_rope_apply_packed(float *qkv_data, size_t qkv_stride, size_t head_offset, size_t seq_len, size_t head_dim,
+                           const float *cos, const float *sin, blt_backend backend) {
+    BLT_DEVICE_ONLY(backend, "blt_rope_apply_packed");
+    blt_rope_apply_packed_hip(qkv_data, qkv_stride, head_offset, seq_len, head_dim, cos, sin);
+}
+
+void blt_multihead_attention(const blt_tensor *input, const blt_tensor *weight_qkv, const blt_tensor *weight_proj,
+                             blt_tensor *output, const blt_attention_config *config, blt_arena *arena) {
+    BLT_REQUIRE(input != NULL, "blt_multihead_attention: input must be [seq_len, embed_dim] FP32");
+    BLT_DEVICE_ONLY(input->backend, "blt_multihead_attention");
+    blt_multihead_attention_hip(input, weight_qkv, weight_proj, output, config, arena);
 }
 
 float blt_vec_dot(blt_backend backend, const float *a, const float *b, size_t n) {

@@ -8,6 +8,7 @@
 #define FBLT_AMD_KV_STEP_H
 
 #include "attn_device.h"
+#include "rope_device.h"
 
 constexpr int SUB = 32;        /* keys per sub-chunk (one wave, one head)       */
 constexpr int MAX_SPLITS = 16; /* workgroups per sequence                        */
@@ -47,24 +48,6 @@ struct StepArgs {
 __device__ __forceinline__ uint32_t kv_span_of(const StepArgs &a, uint32_t nk) {
     const uint32_t subs = (nk + SUB - 1u) / SUB;
     return min(a.span, ((subs + a.splits - 1u) / a.splits) * SUB);
-}
-
-/* Rotary position embedding of four consecutive elements (two pairs) of a
- * row at one position: (x0, x1) -> (x0*c - x1*s, x1*c + x0*s) with separately
- * rounded products (csrc/ops/reductions_cpu.c:219-226; the reference is built
- * without fused multiply-add, and the rotated K rows are stored in the cache,
- * where they must match it bit for bit).  cs / sn point at the tables' entries
- * for the first of the two pairs. */
-__device__ __forceinline__ float4 rope_rotate4(float4 x, const float *cs, const float *sn) {
-#pragma clang fp contract(off) /* no fused multiply-add in this block, also after inlining */
-    const float2 c = *reinterpret_cast<const float2 *>(cs);
-    const float2 s = *reinterpret_cast<const float2 *>(sn);
-    float4 r;
-    r.x = x.x * c.x - x.y * s.x;
-    r.y = x.y * c.x + x.x * s.x;
-    r.z = x.z * c.y - x.w * s.y;
-    r.w = x.w * c.y + x.z * s.y;
-    return r;
 }
 
 /* Device-scope store / load of data another workgroup (possibly on another

@@ -130,6 +130,25 @@ typedef struct {
     float peak_entropy;
 } blt_patch_info;
 
+/* ---- rotary embedding recipe (16 bytes), csrc/ops/rope.h:10-13 ---------- */
+typedef struct {
+    float theta;     /* 500000.0f in BLT */
+    size_t head_dim; /* even */
+} blt_rope_config;
+
+/* ---- multi-head attention block (56 bytes), csrc/models/attention.h:12-22 */
+typedef struct {
+    size_t embed_dim;
+    size_t num_heads;
+    size_t head_dim; /* 0 = embed_dim / num_heads */
+    bool is_causal;
+    bool use_rope;
+    float rope_theta;
+    const blt_tensor *rope_cos_cache;   /* optional [seq_len, head_dim/2] */
+    const blt_tensor *rope_sin_cache;
+    const blt_mask_config *mask_config; /* overrides is_causal when non-NULL */
+} blt_attention_config;
+
 #ifdef __cplusplus
 }
 #define BLT_ABI_ASSERT(c, m) static_assert(c, m)
@@ -147,6 +166,10 @@ BLT_ABI_ASSERT(offsetof(blt_attention_head_args, is_causal) == 128 &&
                    offsetof(blt_attention_head_args, scale) == 132,
                "blt_attention_head_args tail");
 BLT_ABI_ASSERT(sizeof(blt_mask_config) == 72, "blt_mask_config layout");
+BLT_ABI_ASSERT(sizeof(blt_rope_config) == 16 && offsetof(blt_rope_config, head_dim) == 8, "blt_rope_config layout");
+BLT_ABI_ASSERT(sizeof(blt_attention_config) == 56 && offsetof(blt_attention_config, rope_theta) == 28 &&
+                   offsetof(blt_attention_config, mask_config) == 48,
+               "blt_attention_config layout");
 BLT_ABI_ASSERT(offsetof(blt_mask_config, bidirectional_within_group) == 56 &&
                    offsetof(blt_mask_config, is_causal) == 57 && offsetof(blt_mask_config, causal_offset) == 64,
                "blt_mask_config tail");

@@ -62,6 +62,32 @@ void blt_softmax_masked_row_inplace_hip(blt_backend backend, float *row, size_t 
  * result returned to the host (blocking). */
 float blt_vec_dot_hip(blt_backend backend, const float *a, const float *b, size_t n);
 
+/* Replaces blt_matmul_cuda (csrc/ops/linalg.cu:48-134): out[M,N] = a[M,K] *
+ * b[K,N], row-major fp32 device tensors.  Up to 32 rows the result is
+ * bit-identical to blt_matmul_cpu (csrc/ops/linalg_cpu.c:8-18); above that it
+ * is accumulated on the matrix cores in another order.  BF16 operands, which
+ * the reference converts first, are rejected. */
+void blt_matmul_hip(const blt_tensor *a, const blt_tensor *b, blt_tensor *out);
+
+/* Replaces blt_rope_apply_cuda (csrc/ops/reductions.cu:253-319): x, out are
+ * [seq_len, num_heads, head_dim], cos / sin [seq_len, head_dim/2]; row t is
+ * rotated by table row t.  Bit-identical to blt_rope_apply_cpu. */
+void blt_rope_apply_hip(const blt_tensor *x, const blt_tensor *cos, const blt_tensor *sin, blt_tensor *out);
+
+/* Replaces blt_rope_apply_packed_cuda (csrc/ops/reductions.cu:321-340): the
+ * same rotation in place on one head's column block of packed rows. */
+void blt_rope_apply_packed_hip(float *qkv_data, size_t qkv_stride, size_t head_offset, size_t seq_len,
+                               size_t head_dim, const float *cos, const float *sin);
+
+/* blt_multihead_attention for device tensors (csrc/models/attention.c:
+ * 130-207): QKV projection (+ rotation), all heads in one attention launch,
+ * output projection.  Work buffers come from `arena` (a device arena); when
+ * use_rope is set without caches the tables are computed on the host by
+ * blt_rope_precompute and uploaded. */
+void blt_multihead_attention_hip(const blt_tensor *input, const blt_tensor *weight_qkv,
+                                 const blt_tensor *weight_proj, blt_tensor *output,
+                                 const blt_attention_config *config, blt_arena *arena);
+
 /* ===================================================================== */
 /* Part 2 -- device memory shim (csrc/core/cuda_shim.h:18-31,             */
 /*           csrc/ops/memory.cu:19-77)                                    */
@@ -103,6 +129,20 @@ void blt_strided_copy(blt_backend backend, float *dst, size_t dst_stride, const 
 void blt_softmax_masked_row_inplace(blt_backend backend, float *row, size_t row_len, size_t row_idx,
                                     bool is_causal, const float *mask_row, float scale);
 float blt_vec_dot(blt_backend backend, const float *a, const float *b, size_t n);
+/* csrc/core/backend.c:397-399, 307-345; csrc/models/attention.h:24-26.  The
+ * backend comes from the first tensor (matmul, rope_apply), the output
+ * tensors (precompute), the explicit argument (packed) or the input tensor
+ * (attention block). */
+void blt_matmul(const blt_tensor *a, const blt_tensor *b, blt_tensor *out);
+/* Tables for device tensors are computed on the host with the reference's
+ * own formula and libm calls (csrc/ops/reductions_cpu.c:179-197), so they are
+ * bit-identical to the CPU reference, then uploaded (blocking). */
+void blt_rope_precompute(size_t max_seq_len, const blt_rope_config *config, blt_tensor *cos_out, blt_tensor *sin_out);
+void blt_rope_apply(const blt_tensor *x, const blt_tensor *cos, const blt_tensor *sin, blt_tensor *out);
+void blt_rope_apply_packed(float *qkv_data, size_t qkv_stride, size_t head_offset, size_t seq_len, size_t head_dim,
+                           const float *cos, const float *sin, blt_backend backend);
+void blt_multihead_attention(const blt_tensor *input, const blt_tensor *weight_qkv, const blt_tensor *weight_proj,
+                             blt_tensor *output, const blt_attention_config *config, blt_arena *arena);
 
 /* Byte<->patch index helpers; host integer code in the reference as well
  * (csrc/ops/patch_pool.h:29-41, patch_pool_cpu.c:98-142). */

@@ -74,6 +74,13 @@ def load_oracle():
     lib.orc_rope_apply.argtypes = [_fp, C.c_size_t, C.c_size_t, C.c_size_t, _fp, _fp, _fp]
     lib.orc_rope_position_gather.restype = C.c_int
     lib.orc_rope_position_gather.argtypes = [_fp, _fp, C.c_size_t, C.c_size_t, _sp, C.c_size_t, _fp, _fp]
+    lib.orc_matmul.restype = None
+    lib.orc_matmul.argtypes = [_fp, _fp, _fp, C.c_size_t, C.c_size_t, C.c_size_t]
+    lib.orc_rope_apply_packed.restype = None
+    lib.orc_rope_apply_packed.argtypes = [_fp, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, _fp, _fp]
+    lib.orc_multihead_attention.restype = C.c_int
+    lib.orc_multihead_attention.argtypes = [_fp, _fp, _fp, _fp, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int, C.c_int,
+                                            C.c_float, _fp, _fp, C.POINTER(abi.BltMaskConfig)]
     lib.orc_kv_rope_attend_step.restype = C.c_int
     lib.orc_kv_rope_attend_step.argtypes = [_fp, _fp] + [C.c_size_t] * 7 + [_fp, C.c_size_t, _fp, C.c_size_t, _fp,
                                                                            C.c_size_t, _fp, _fp, C.c_size_t, _fp]
@@ -131,6 +138,12 @@ def load_ref():
     lib.blt_rope_precompute.argtypes = [C.c_size_t, C.POINTER(BltRopeConfig), T, T]
     lib.blt_rope_apply.restype = None
     lib.blt_rope_apply.argtypes = [T, T, T, T]
+    lib.blt_matmul.restype = None
+    lib.blt_matmul.argtypes = [T, T, T]
+    lib.blt_rope_apply_packed.restype = None
+    lib.blt_rope_apply_packed.argtypes = [_fp, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, _fp, _fp, C.c_int]
+    lib.blt_multihead_attention.restype = None
+    lib.blt_multihead_attention.argtypes = [T, T, T, T, C.POINTER(abi.BltAttentionConfig), C.POINTER(abi.BltArena)]
     lib.blt_build_block_diffusion_mask.restype = None
     lib.blt_build_block_diffusion_mask.argtypes = [C.POINTER(abi.BltBlockDiffusionConfig),
                                                    C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)]

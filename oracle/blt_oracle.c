@@ -407,3 +407,91 @@ int orc_kv_rope_attend_step(float *self_k, float *self_v, size_t max_seq_len, si
     free(q_full), free(k_full), free(v_full);
     return rcode;
 }
+
+/* csrc/ops/linalg_cpu.c:8-18 */
+void orc_matmul(const float *a, const float *b, float *out, size_t m, size_t k, size_t n) {
+    for (size_t row = 0; row < m; ++row) {
+        for (size_t col = 0; col < n; ++col) {
+            float sum = 0.0f;
+            for (size_t inner = 0; inner < k; ++inner) sum += a[row * k + inner] * b[inner * n + col];
+            out[row * n + col] = sum;
+        }
+    }
+}
+
+/* csrc/core/backend.c:331-344: in-place rotation of one head's column block of packed rows */
+void orc_rope_apply_packed(float *qkv, size_t qkv_stride, size_t head_offset, size_t seq_len, size_t head_dim,
+                           const float *cos_rows, const float *sin_rows) {
+    const size_t half = head_dim / 2;
+    for (size_t t = 0; t < seq_len; t++) {
+        float *base = qkv + t * qkv_stride + head_offset;
+        const float *c = cos_rows + t * half;
+        const float *s = sin_rows + t * half;
+        for (size_t i = 0; i < half; i++) {
+            float x0 = base[2 * i];
+            float x1 = base[2 * i + 1];
+            base[2 * i] = x0 * c[i] - x1 * s[i];
+            base[2 * i + 1] = x1 * c[i] + x0 * s[i];
+        }
+    }
+}
+
+/* csrc/models/attention.c:130-207 (BLT_FLASH_ATTN unset): packed projection,
+ * rotation of the Q and K blocks head by head (76-90), dense mask from the
+ * mask configuration when there is one (58-74), one core call per head with
+ * weights_out (92-128), output projection. */
+int orc_multihead_attention(const float *input, const float *weight_qkv, const float *weight_proj, float *output,
+                            size_t seq_len, size_t embed_dim, size_t num_heads, int is_causal, int use_rope,
+                            float rope_theta, const float *rope_cos_cache, const float *rope_sin_cache,
+                            const blt_mask_config *mask_config) {
+    if (num_heads == 0 || embed_dim % num_heads != 0) return ORC_ERR_ARG;
+    const size_t hd = embed_dim / num_heads, half = hd / 2, E = embed_dim;
+    if (use_rope && (hd % 2 != 0 || !(rope_theta > 0.0f))) return ORC_ERR_ARG;
+    float *qkv = (float *)malloc(seq_len * 3 * E * sizeof(float));
+    float *combined = (float *)calloc(seq_len * E, sizeof(float));
+    float *scores = (float *)malloc(seq_len * seq_len * sizeof(float));
+    float *mask = NULL, *cs = NULL, *sn = NULL;
+    int rc = ORC_OK;
+    orc_matmul(input, weight_qkv, qkv, seq_len, E, 3 * E);
+    if (use_rope) {
+        const float *c = rope_cos_cache, *s = rope_sin_cache;
+        if (!(c && s)) {
+            cs = (float *)malloc(seq_len * half * sizeof(float));
+            sn = (float *)malloc(seq_len * half * sizeof(float));
+            rc = orc_rope_precompute(seq_len, rope_theta, hd, cs, sn);
+            c = cs, s = sn;
+        }
+        for (size_t h = 0; h < num_heads && rc == ORC_OK; h++) {
+            orc_rope_apply_packed(qkv, 3 * E, h * hd, seq_len, hd, c, s);
+            orc_rope_apply_packed(qkv, 3 * E, E + h * hd, seq_len, hd, c, s);
+        }
+    }
+    if (rc == ORC_OK && mask_config != NULL) {
+        if (mask_config->seq_len_q != seq_len || mask_config->seq_len_kv != seq_len) rc = ORC_ERR_ARG;
+        else {
+            mask = (float *)malloc(seq_len * seq_len * sizeof(float));
+            rc = orc_build_attention_mask(mask_config, mask);
+        }
+    }
+    for (size_t h = 0; h < num_heads && rc == ORC_OK; h++) {
+        blt_attention_head_args a;
+        memset(&a, 0, sizeof(a));
+        a.q = qkv + h * hd;
+        a.k = qkv + E + h * hd;
+        a.v = qkv + 2 * E + h * hd;
+        a.q_stride = a.k_stride = a.v_stride = 3 * E;
+        a.combined = combined;
+        a.combined_stride = E;
+        a.combined_col_offset = h * hd;
+        a.weights_out = scores;
+        a.mask = mask;
+        a.nq = a.nk = seq_len;
+        a.head_dim = hd;
+        a.is_causal = is_causal != 0;
+        a.scale = 1.0f / sqrtf((float)hd);
+        rc = orc_attention_head_core(&a);
+    }
+    if (rc == ORC_OK) orc_matmul(combined, weight_proj, output, seq_len, E, E);
+    free(qkv), free(combined), free(scores), free(mask), free(cs), free(sn);
+    return rc;
+}

@@ -43,6 +43,14 @@
  *       preserved, q.k after rotation depends only on the position
  *       difference; the step against rotating by hand and calling
  *       orc_kv_attend_step.
+ *   orc_matmul, orc_rope_apply_packed, orc_multihead_attention
+ *       bit-for-bit against oracle/_ref (blt_matmul, blt_rope_apply_packed,
+ *       blt_multihead_attention compiled from csrc/models/attention.c); the
+ *       reference's vectors: [[1,2],[3,4]] x [[5,6],[7,8]] = [[19,22],[43,50]]
+ *       (tests/unit/backend/unit_linalg_cpu.c:10-48) and the identity-weight
+ *       two-token block -> {0.6697615, 0.3302385, ...}, causal row 0 one-hot
+ *       (tests/unit/models/unit_attention.c:82-88, 160-171); a float64 numpy
+ *       product; the block against its parts called by hand.
  */
 #ifndef FBLT_AMD_ORACLE_H
 #define FBLT_AMD_ORACLE_H
@@ -158,6 +166,22 @@ int orc_kv_rope_attend_step(float *self_k, float *self_v, size_t max_seq_len, si
                             size_t b, size_t base, size_t n, size_t window, const float *q_rows, size_t q_stride,
                             const float *k_rows, size_t k_stride, const float *v_rows, size_t v_stride,
                             const float *cos_cache, const float *sin_cache, size_t cache_rows, float *combined);
+
+/* linalg_cpu.c:8-18: out[m,n] = a[m,k] * b[k,n], k ascending, product and sum rounded separately. */
+void orc_matmul(const float *a, const float *b, float *out, size_t m, size_t k, size_t n);
+
+/* backend.c:331-344: rotation in place of one head's column block of packed rows. */
+void orc_rope_apply_packed(float *qkv, size_t qkv_stride, size_t head_offset, size_t seq_len, size_t head_dim,
+                           const float *cos_rows, const float *sin_rows);
+
+/* models/attention.c:130-207 with host buffers: input [T,E], weight_qkv
+ * [E,3E], weight_proj [E,E], output [T,E].  Tables are computed inside when
+ * use_rope is set and no caches are given.  mask_config (or NULL) as in
+ * blt_attention_config. */
+int orc_multihead_attention(const float *input, const float *weight_qkv, const float *weight_proj, float *output,
+                            size_t seq_len, size_t embed_dim, size_t num_heads, int is_causal, int use_rope,
+                            float rope_theta, const float *rope_cos_cache, const float *rope_sin_cache,
+                            const blt_mask_config *mask_config);
 
 #ifdef __cplusplus
 }

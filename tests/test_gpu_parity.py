@@ -476,3 +476,140 @@ def test_kv_rope_step(case, oracle, dev):
     assert_close(out, ref_out, "rope " + case)
     if kw.commit:
         assert (lens == kw.lens + kw.n * kw.steps).all()
+
+
+# ---------------------------------------------------------------------------
+# projections, rotation and the attention block
+# ---------------------------------------------------------------------------
+def _dev_tensor(t, shape=None):
+    return abi.tensor_view(t.data_ptr(), tuple(t.shape) if shape is None else shape, abi.BLT_BACKEND_HIP)
+
+
+@pytest.mark.parametrize("m,k,n,exact", [(1, 128, 384, True), (5, 33, 17, True), (32, 512, 512, True),
+                                          (16, 128, 512, True), (33, 64, 64, False), (64, 128, 384, False),
+                                          (512, 128, 384, False), (100, 70, 50, False), (513, 129, 130, False),
+                                          (2048, 512, 1536, False)])
+def test_matmul(m, k, n, exact, oracle, dev):
+    """blt_matmul: up to 32 rows bit-identical to the reference loop, above that fp32 tolerance."""
+    import torch
+    lib = api.load()
+    rs = np.random.RandomState(m + k + n)
+    a = rs.randn(m, k).astype(np.float32)
+    b = (rs.randn(k, n) / np.sqrt(k)).astype(np.float32)
+    ref = np.zeros((m, n), dtype=np.float32)
+    oracle.orc_matmul(binding.fptr(a.reshape(-1)), binding.fptr(b.reshape(-1)), binding.fptr(ref.reshape(-1)), m, k, n)
+    ta, tb = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    to = torch.full((m, n), 7.0, dtype=torch.float32, device="cuda")
+    va, vb, vo = _dev_tensor(ta), _dev_tensor(tb), _dev_tensor(to)
+    lib.blt_matmul(C.byref(va), C.byref(vb), C.byref(vo))
+    lib.blt_backend_pass_sync_hip()
+    got = to.cpu().numpy()
+    if exact:
+        assert got.tobytes() == ref.tobytes()
+    else:
+        assert_close(got, ref, "matmul %dx%dx%d" % (m, k, n))
+
+
+def test_rope_apply_bit_exact(oracle, dev):
+    import torch
+    lib = api.load()
+    rs = np.random.RandomState(77)
+    T, H, hd = 45, 3, 32
+    half = hd // 2
+    x = rs.randn(T, H, hd).astype(np.float32)
+    cos, sin = np.empty(T * half, dtype=np.float32), np.empty(T * half, dtype=np.float32)
+    assert oracle.orc_rope_precompute(T, 500000.0, hd, binding.fptr(cos), binding.fptr(sin)) == 0
+    # tables: the device dispatcher computes them on the host with the same formula
+    tc = torch.zeros((T, half), dtype=torch.float32, device="cuda")
+    ts = torch.zeros((T, half), dtype=torch.float32, device="cuda")
+    vc, vs = _dev_tensor(tc), _dev_tensor(ts)
+    cfg = abi.BltRopeConfig(500000.0, hd)
+    lib.blt_rope_precompute(T, C.byref(cfg), C.byref(vc), C.byref(vs))
+    assert tc.cpu().numpy().tobytes() == cos.tobytes() and ts.cpu().numpy().tobytes() == sin.tobytes()
+    ref = np.empty_like(x)
+    oracle.orc_rope_apply(binding.fptr(x.reshape(-1)), T, H, hd, binding.fptr(cos), binding.fptr(sin),
+                          binding.fptr(ref.reshape(-1)))
+    tx = torch.from_numpy(x).cuda()
+    to = torch.zeros_like(tx)
+    vx, vo = _dev_tensor(tx), _dev_tensor(to)
+    lib.blt_rope_apply(C.byref(vx), C.byref(vc), C.byref(vs), C.byref(vo))
+    lib.blt_backend_pass_sync_hip()
+    assert to.cpu().numpy().tobytes() == ref.tobytes()
+    # packed, in place, one head block of [T, 3E] rows
+    E = H * hd
+    qkv = rs.randn(T, 3 * E).astype(np.float32)
+    want = qkv.copy()
+    oracle.orc_rope_apply_packed(binding.fptr(want.reshape(-1)), 3 * E, E + hd, T, hd, binding.fptr(cos),
+                                 binding.fptr(sin))
+    tq = torch.from_numpy(qkv).cuda()
+    lib.blt_rope_apply_packed(tq.data_ptr(), 3 * E, E + hd, T, hd, tc.data_ptr(), ts.data_ptr(), abi.BLT_BACKEND_HIP)
+    lib.blt_backend_pass_sync_hip()
+    assert tq.cpu().numpy().tobytes() == want.tobytes()
+
+
+@pytest.mark.parametrize("T,E,H,causal,rope,mask,cached", [
+    (2, 4, 2, False, False, None, False),          # the reference's identity-weight block
+    (20, 32, 4, True, True, None, False),          # few rows: exact products, separate rotation pass
+    (96, 64, 2, True, True, None, True),
+    (512, 128, 4, False, True, "causal_cfg", True),  # the local decoder's call at C1 size
+    (300, 128, 4, False, True, "window", False),
+    (70, 48, 3, False, False, "docs", False),        # dense mask from the device builder
+    (128, 512, 8, False, False, "causal_cfg", False),  # the patch transformer's call at C2 size
+])
+def test_multihead_attention_block(T, E, H, causal, rope, mask, cached, oracle, dev):
+    """blt_multihead_attention on device tensors against the restated block."""
+    import torch
+    lib = api.load()
+    rs = np.random.RandomState(T + E)
+    hd, half = E // H, E // H // 2
+    if (T, E, H) == (2, 4, 2):
+        x = np.array([[1, 0, 1, 0], [0, 1, 0, 1]], dtype=np.float32)
+        wqkv = np.zeros((4, 12), dtype=np.float32)
+        for i in range(4):
+            wqkv[i, i] = wqkv[i, 4 + i] = wqkv[i, 8 + i] = 1.0
+        wproj = np.eye(4, dtype=np.float32)
+    else:
+        x = rs.randn(T, E).astype(np.float32)
+        wqkv = (rs.randn(E, 3 * E) / np.sqrt(E)).astype(np.float32)
+        wproj = (rs.randn(E, E) / np.sqrt(E)).astype(np.float32)
+    cfg, keep = None, None
+    if mask is not None:
+        cfg = abi.BltMaskConfig()
+        cfg.seq_len_q = cfg.seq_len_kv = T
+        if mask == "window":
+            cfg.is_causal, cfg.sliding_window = True, 40
+        elif mask == "docs":
+            keep = abi.size_array([21, 50])
+            cfg.doc_boundaries, cfg.num_docs = keep, 3
+        else:
+            cfg.is_causal = True
+    ref = np.zeros((T, E), dtype=np.float32)
+    assert oracle.orc_multihead_attention(
+        binding.fptr(x.reshape(-1)), binding.fptr(wqkv.reshape(-1)), binding.fptr(wproj.reshape(-1)),
+        binding.fptr(ref.reshape(-1)), T, E, H, int(causal), int(rope), 500000.0, None, None,
+        C.byref(cfg) if cfg is not None else None) == 0
+    if (T, E, H) == (2, 4, 2):   # tests/unit/models/unit_attention.c:82-88
+        assert abs(ref[0, 0] - 0.6697615) < 1e-6 and abs(ref[0, 1] - 0.3302385) < 1e-6
+    tx, tq, tp = (torch.from_numpy(v).cuda() for v in (x, wqkv, wproj))
+    to = torch.full((T, E), 7.0, dtype=torch.float32, device="cuda")
+    ac = abi.BltAttentionConfig()
+    ac.embed_dim, ac.num_heads, ac.head_dim = E, H, hd
+    ac.is_causal, ac.use_rope, ac.rope_theta = causal, rope, 500000.0
+    if cfg is not None:
+        ac.mask_config = C.pointer(cfg)
+    tables = None
+    if rope and cached:
+        cos, sin = np.empty(T * half, dtype=np.float32), np.empty(T * half, dtype=np.float32)
+        oracle.orc_rope_precompute(T, 500000.0, hd, binding.fptr(cos), binding.fptr(sin))
+        tables = (torch.from_numpy(cos.reshape(T, half)).cuda(), torch.from_numpy(sin.reshape(T, half)).cuda())
+        vc, vs = _dev_tensor(tables[0]), _dev_tensor(tables[1])
+        ac.rope_cos_cache, ac.rope_sin_cache = C.pointer(vc), C.pointer(vs)
+    arena = lib.blt_arena_create(64 << 20, abi.BLT_BACKEND_HIP)
+    try:
+        vx, vq, vp, vo = _dev_tensor(tx), _dev_tensor(tq), _dev_tensor(tp), _dev_tensor(to)
+        lib.blt_multihead_attention(C.byref(vx), C.byref(vq), C.byref(vp), C.byref(vo), C.byref(ac), arena)
+        lib.blt_backend_pass_sync_hip()
+        got = to.cpu().numpy()
+    finally:
+        lib.blt_arena_destroy(arena)
+    assert_close(got, ref, "attention block T=%d E=%d H=%d" % (T, E, H))

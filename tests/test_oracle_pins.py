@@ -418,3 +418,112 @@ def test_rope_gather_and_step_composition(oracle):
                                          binding.fptr(theirs.reshape(-1))) == 0
         assert mine.tobytes() == theirs.tobytes()
         assert ck1.tobytes() == ck2.tobytes() and cv1.tobytes() == cv2.tobytes()
+
+
+# ---------------------------------------------------------------------------
+# projections and the attention block (csrc/ops/linalg_cpu.c:8-18, csrc/models/attention.c:130-207)
+# ---------------------------------------------------------------------------
+def test_matmul_reference_vector_and_float64(oracle):
+    a = np.array([1, 2, 3, 4], dtype=np.float32)
+    b = np.array([5, 6, 7, 8], dtype=np.float32)
+    out = np.zeros(4, dtype=np.float32)
+    oracle.orc_matmul(binding.fptr(a), binding.fptr(b), binding.fptr(out), 2, 2, 2)
+    assert out.tolist() == [19.0, 22.0, 43.0, 50.0]   # tests/unit/backend/unit_linalg_cpu.c:10-48
+    rs = np.random.RandomState(8)
+    for m, k, n in ((1, 7, 5), (9, 33, 17), (40, 128, 24)):
+        a, b = rs.randn(m, k).astype(np.float32), rs.randn(k, n).astype(np.float32)
+        out = np.zeros((m, n), dtype=np.float32)
+        oracle.orc_matmul(binding.fptr(a.reshape(-1)), binding.fptr(b.reshape(-1)), binding.fptr(out.reshape(-1)), m,
+                          k, n)
+        want = a.astype(np.float64) @ b.astype(np.float64)
+        assert np.abs(out - want).max() < 2e-5
+        # not a transposed operand: a non-square case fails if either were
+        assert np.abs(out - (b.T.astype(np.float64) @ a.T.astype(np.float64)).T).max() < 2e-5
+    # the sum runs over k in ascending order with separate rounding: a case where the order shows
+    a = np.array([[1e8, 1.0, -1e8]], dtype=np.float32)
+    b = np.ones((3, 1), dtype=np.float32)
+    out = np.zeros((1, 1), dtype=np.float32)
+    oracle.orc_matmul(binding.fptr(a.reshape(-1)), binding.fptr(b.reshape(-1)), binding.fptr(out.reshape(-1)), 1, 3, 1)
+    assert out[0, 0] == 0.0   # (1e8 + 1) rounds to 1e8, then - 1e8
+
+
+def _mha(oracle, x, wqkv, wproj, H, causal=False, rope=False, theta=10000.0, mask_cfg=None, caches=None):
+    T, E = x.shape
+    out = np.full((T, E), 3.0, dtype=np.float32)
+    c = binding.fptr(caches[0].reshape(-1)) if caches else None
+    s = binding.fptr(caches[1].reshape(-1)) if caches else None
+    rc = oracle.orc_multihead_attention(binding.fptr(x.reshape(-1)), binding.fptr(wqkv.reshape(-1)),
+                                        binding.fptr(wproj.reshape(-1)), binding.fptr(out.reshape(-1)), T, E, H,
+                                        int(causal), int(rope), theta, c, s,
+                                        C.byref(mask_cfg) if mask_cfg is not None else None)
+    assert rc == 0, rc
+    return out
+
+
+def _identity_block():
+    x = np.array([[1, 0, 1, 0], [0, 1, 0, 1]], dtype=np.float32)
+    wqkv = np.zeros((4, 12), dtype=np.float32)
+    for i in range(4):
+        wqkv[i, i] = wqkv[i, 4 + i] = wqkv[i, 8 + i] = 1.0
+    return x, wqkv, np.eye(4, dtype=np.float32)
+
+
+def test_attention_block_reference_vectors(oracle):
+    """tests/unit/models/unit_attention.c:30-88 (identity weights, two tokens, two heads) and
+    160-171 (causal: row 0 sees only itself)."""
+    x, wqkv, wproj = _identity_block()
+    out = _mha(oracle, x, wqkv, wproj, 2)
+    want = np.array([[0.6697615, 0.3302385, 0.6697615, 0.3302385], [0.3302385, 0.6697615, 0.3302385, 0.6697615]])
+    assert np.abs(out - want).max() < 1e-6
+    out_c = _mha(oracle, x, wqkv, wproj, 2, causal=True)
+    assert np.abs(out_c[0] - np.array([1, 0, 1, 0])).max() < 1e-6
+    assert np.abs(out_c[1] - want[1]).max() < 1e-6
+    # mask_config causal == is_causal (unit_attention.c:184)
+    cfg = abi.BltMaskConfig()
+    cfg.seq_len_q = cfg.seq_len_kv = 2
+    cfg.is_causal = True
+    assert _mha(oracle, x, wqkv, wproj, 2, mask_cfg=cfg).tobytes() == out_c.tobytes()
+    # with rotation: position 0 is not rotated, and running it twice gives the same bits (unit_attention.c:66-79)
+    r1 = _mha(oracle, x, wqkv, wproj, 2, rope=True)
+    r2 = _mha(oracle, x, wqkv, wproj, 2, rope=True)
+    assert r1.tobytes() == r2.tobytes() and np.isfinite(r1).all()
+
+
+def test_attention_block_equals_its_parts(oracle):
+    rs = np.random.RandomState(21)
+    T, E, H = 19, 24, 3
+    hd, half = E // H, E // H // 2
+    x = rs.randn(T, E).astype(np.float32)
+    wqkv = (rs.randn(E, 3 * E) / np.sqrt(E)).astype(np.float32)
+    wproj = (rs.randn(E, E) / np.sqrt(E)).astype(np.float32)
+    cos, sin = np.empty(T * half, dtype=np.float32), np.empty(T * half, dtype=np.float32)
+    assert oracle.orc_rope_precompute(T, 500000.0, hd, binding.fptr(cos), binding.fptr(sin)) == 0
+    got = _mha(oracle, x, wqkv, wproj, H, causal=True, rope=True, theta=500000.0)
+    got_cached = _mha(oracle, x, wqkv, wproj, H, causal=True, rope=True, theta=1.0, caches=(cos, sin))
+    assert got.tobytes() == got_cached.tobytes()   # caches win over theta
+    qkv = np.zeros((T, 3 * E), dtype=np.float32)
+    oracle.orc_matmul(binding.fptr(x.reshape(-1)), binding.fptr(wqkv.reshape(-1)), binding.fptr(qkv.reshape(-1)), T, E,
+                      3 * E)
+    # packed rotation == copy out, orc_rope_apply, copy back
+    q_heads = np.ascontiguousarray(qkv[:, :E]).reshape(T, H, hd)
+    rot = np.empty_like(q_heads)
+    oracle.orc_rope_apply(binding.fptr(q_heads.reshape(-1)), T, H, hd, binding.fptr(cos), binding.fptr(sin),
+                          binding.fptr(rot.reshape(-1)))
+    for h in range(H):
+        oracle.orc_rope_apply_packed(binding.fptr(qkv.reshape(-1)), 3 * E, h * hd, T, hd, binding.fptr(cos),
+                                     binding.fptr(sin))
+        oracle.orc_rope_apply_packed(binding.fptr(qkv.reshape(-1)), 3 * E, E + h * hd, T, hd, binding.fptr(cos),
+                                     binding.fptr(sin))
+    assert qkv[:, :E].reshape(T, H, hd).tobytes() == rot.tobytes()
+    comb = np.zeros((T, E), dtype=np.float32)
+    w = np.zeros(T * T, dtype=np.float32)
+    flat = qkv.reshape(-1)
+    for h in range(H):
+        a = binding.head_args(flat, flat, flat, comb.reshape(-1), T, T, hd, float(np.float32(1) / np.sqrt(np.float32(hd))),
+                              3 * E, 3 * E, 3 * E, E, h * hd, q_off=h * hd, k_off=E + h * hd, v_off=2 * E + h * hd,
+                              weights=w, causal=True)
+        assert oracle.orc_attention_head_core(C.byref(a)) == 0
+    want = np.zeros((T, E), dtype=np.float32)
+    oracle.orc_matmul(binding.fptr(comb.reshape(-1)), binding.fptr(wproj.reshape(-1)), binding.fptr(want.reshape(-1)), T,
+                      E, E)
+    assert got.tobytes() == want.tobytes()

@@ -265,3 +265,53 @@ def test_kv_rope_step_against_reference_op_sequence(oracle, ref):
                                          binding.fptr(k_rows.reshape(-1)), binding.fptr(v_rows.reshape(-1)),
                                          binding.fptr(theirs.reshape(-1))) == 0
         assert mine.tobytes() == theirs.tobytes()
+
+
+def test_matmul_and_attention_block_bit_exact(oracle, ref):
+    """orc_matmul and orc_multihead_attention against blt_matmul / blt_multihead_attention compiled
+    from the reference (csrc/ops/linalg_cpu.c, csrc/models/attention.c:130-207)."""
+    rs = np.random.RandomState(31)
+    for m, k, n in ((1, 16, 48), (7, 33, 5), (64, 128, 96)):
+        a, b = rs.randn(m, k).astype(np.float32), rs.randn(k, n).astype(np.float32)
+        mine, theirs = np.zeros((m, n), dtype=np.float32), np.zeros((m, n), dtype=np.float32)
+        oracle.orc_matmul(binding.fptr(a.reshape(-1)), binding.fptr(b.reshape(-1)), binding.fptr(mine.reshape(-1)), m,
+                          k, n)
+        ta, tb, to = (abi.tensor_view(x.ctypes.data, x.shape, CPU) for x in (a, b, theirs))
+        ref.blt_matmul(C.byref(ta), C.byref(tb), C.byref(to))
+        assert mine.tobytes() == theirs.tobytes()
+    arena = ref.blt_arena_create(32 << 20, CPU)
+    try:
+        for T, E, H, causal, rope, mask in ((2, 4, 2, False, False, None), (37, 32, 4, True, True, None),
+                                            (50, 64, 2, False, True, "window"), (33, 24, 3, False, False, "docs"),
+                                            (40, 32, 2, True, True, "causal_cfg")):
+            x = rs.randn(T, E).astype(np.float32)
+            wqkv = (rs.randn(E, 3 * E) / np.sqrt(E)).astype(np.float32)
+            wproj = (rs.randn(E, E) / np.sqrt(E)).astype(np.float32)
+            cfg, keep = None, None
+            if mask is not None:
+                cfg = abi.BltMaskConfig()
+                cfg.seq_len_q = cfg.seq_len_kv = T
+                if mask == "window":
+                    cfg.is_causal, cfg.sliding_window = True, 9
+                elif mask == "docs":
+                    keep = abi.size_array([11, 20])
+                    cfg.doc_boundaries, cfg.num_docs = keep, 3
+                else:
+                    cfg.is_causal = True
+            mine = np.zeros((T, E), dtype=np.float32)
+            assert oracle.orc_multihead_attention(
+                binding.fptr(x.reshape(-1)), binding.fptr(wqkv.reshape(-1)), binding.fptr(wproj.reshape(-1)),
+                binding.fptr(mine.reshape(-1)), T, E, H, int(causal), int(rope), 500000.0, None, None,
+                C.byref(cfg) if cfg is not None else None) == 0
+            theirs = np.zeros((T, E), dtype=np.float32)
+            ac = abi.BltAttentionConfig()
+            ac.embed_dim, ac.num_heads, ac.head_dim = E, H, E // H
+            ac.is_causal, ac.use_rope, ac.rope_theta = causal, rope, 500000.0
+            if cfg is not None:
+                ac.mask_config = C.pointer(cfg)
+            tx, tq, tp, to = (abi.tensor_view(v.ctypes.data, v.shape, CPU) for v in (x, wqkv, wproj, theirs))
+            arena.contents.offset = 0
+            ref.blt_multihead_attention(C.byref(tx), C.byref(tq), C.byref(tp), C.byref(to), C.byref(ac), arena)
+            assert mine.tobytes() == theirs.tobytes(), (T, E, H, causal, rope, mask)
+    finally:
+        ref.blt_arena_destroy(arena)
