@@ -153,6 +153,80 @@ def bench_kv(kw, steps, warmup):
     return res, kw
 
 
+def bench_block(name, T, E, H, steps, warmup, gemm_only=None):
+    """blt_multihead_attention (projection, rotation, all heads, projection) on random
+    device tensors, or with gemm_only=(m, k, n) one blt_matmul of that shape."""
+    import ctypes as C
+    import numpy as np
+    import torch
+    from fblt_amd import abi, api
+    lib = api.load()
+    view = lambda t: abi.tensor_view(t.data_ptr(), tuple(t.shape), abi.BLT_BACKEND_HIP)
+    g = torch.Generator(device="cpu").manual_seed(1234)
+    rnd = lambda *shape: torch.randn(*shape, generator=g, dtype=torch.float32)
+    keep = []
+    if gemm_only:
+        m, k, n = gemm_only
+        a, b, o = rnd(m, k).cuda(), (rnd(k, n) / k ** 0.5).cuda(), torch.zeros((m, n), device="cuda")
+        va, vb, vo = view(a), view(b), view(o)
+        run = lambda: lib.blt_matmul(C.byref(va), C.byref(vb), C.byref(vo))
+        flops, nbytes, tokens = 2.0 * m * k * n, 4.0 * (m * k + k * n + m * n), m
+    else:
+        hd = E // H
+        x, wq, wp = rnd(T, E).cuda(), (rnd(E, 3 * E) / E ** 0.5).cuda(), (rnd(E, E) / E ** 0.5).cuda()
+        o = torch.zeros((T, E), device="cuda")
+        arena = lib.blt_arena_create(256 << 20, abi.BLT_BACKEND_HIP)
+        cos = torch.zeros((T, hd // 2), device="cuda")
+        sin = torch.zeros((T, hd // 2), device="cuda")
+        vc, vs = view(cos), view(sin)
+        rcfg = abi.BltRopeConfig(500000.0, hd)
+        lib.blt_rope_precompute(T, C.byref(rcfg), C.byref(vc), C.byref(vs))
+        mc = abi.BltMaskConfig()
+        mc.seq_len_q = mc.seq_len_kv = T
+        mc.is_causal = True
+        ac = abi.BltAttentionConfig()
+        ac.embed_dim, ac.num_heads, ac.head_dim = E, H, hd
+        ac.use_rope, ac.rope_theta = True, 500000.0
+        ac.rope_cos_cache, ac.rope_sin_cache, ac.mask_config = C.pointer(vc), C.pointer(vs), C.pointer(mc)
+        vx, vq, vp, vo = view(x), view(wq), view(wp), view(o)
+        keep += [cos, sin, vc, vs, mc]
+
+        def run():
+            arena.contents.offset = 0
+            lib.blt_multihead_attention(C.byref(vx), C.byref(vq), C.byref(vp), C.byref(vo), C.byref(ac), arena)
+        pairs = H * (T * (T + 1) // 2)
+        flops = 2.0 * T * E * 3 * E + 4.0 * hd * pairs + 2.0 * T * E * E
+        nbytes = 4.0 * (T * E + 3 * E * E + E * E + T * E)
+        tokens = T
+    for _ in range(warmup):
+        run()
+    lib.blt_backend_pass_sync_hip()
+    lib.blt_hip_profile_begin()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        run()
+    lib.blt_backend_pass_sync_hip()
+    wall = time.perf_counter() - t0
+    prof = api.profile_end()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        run()
+    lib.blt_backend_pass_sync_hip()
+    wall_plain = time.perf_counter() - t0
+    if not gemm_only:
+        lib.blt_arena_destroy(arena)
+    avg_s = sum(v[1] for v in prof.values()) / 1e3 / steps
+    res = {"workload": name, "kernel": "+".join(sorted(prof)), "launches_per_step": sum(v[0] for v in prof.values()) / steps,
+           "tokens_per_step": tokens, "ms_per_step": wall_plain / steps * 1e3,
+           "ms_per_step_with_events": wall / steps * 1e3, "kernel_us_avg": avg_s * 1e6,
+           "kernel_us_min": min(v[2] for v in prof.values()) * 1e3,
+           "per_kernel_us": {k: v[1] * 1e3 / steps for k, v in prof.items()},
+           "tokens_per_s": tokens * steps / wall_plain, "tokens_per_s_kernel": tokens / avg_s, "flops": flops,
+           "bytes": nbytes, "roofline_hbm": roofline("hbm", nbytes, avg_s), "roofline_mfma": roofline("mfma", flops, avg_s)}
+    res["roofline"] = res["roofline_mfma"]
+    return res
+
+
 def cpu_dense(w, budget_s):
     """Checker on one host core over the same workload; repeated whole passes up to the budget."""
     from oracle import binding, runner as orunner
@@ -259,6 +333,16 @@ def main():
         bigv = workloads.config5(batch=128, B=16, len_lo=1024, len_hi=2032, max_seq_len=2048, cache_period=8)
         others["c5_B16_b128_L2048"], _ = bench_kv(bigv, 20, 3)
         log("c5_B16_b128_L2048", json.dumps(others["c5_B16_b128_L2048"]))
+
+    # the callers either side of the core: the whole attention block and its projection
+    if want("block"):
+        others["mha_c1"] = bench_block("blt_multihead_attention T=512 E=128 H=4 rope causal", 512, 128, 4, K, W)
+        log("mha_c1", json.dumps(others["mha_c1"]))
+        others["mha_c2"] = bench_block("blt_multihead_attention T=128 E=512 H=8 rope causal", 128, 512, 8, K, W)
+        log("mha_c2", json.dumps(others["mha_c2"]))
+        others["matmul_8192x512x1536"] = bench_block("blt_matmul 8192x512x1536", 0, 0, 0, max(10, K // 10), 3,
+                                                     gemm_only=(8192, 512, 1536))
+        log("matmul", json.dumps(others["matmul_8192x512x1536"]))
 
     cpu_head = None
     if not args.no_cpu:

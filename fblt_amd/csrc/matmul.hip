@@ -4,7 +4,7 @@
  * csrc/ops/matmul.h, CPU loop csrc/ops/linalg_cpu.c:8-18, device twin
  * csrc/ops/linalg.cu:48-134).
  *
- * Two kernels:
+ * Three kernels:
  *
  *  - "skinny" (M <= 32: the n new rows of a decode / verify step): one thread
  *    per output column, the column of b read coalesced across the wave, the
@@ -22,6 +22,14 @@
  *    embedding of the Q and K blocks of a packed QKV projection
  *    (csrc/models/attention.c:76-90) -- without a second pass over the
  *    result.  Summation order differs from the reference's (fp32 tolerance).
+ *
+ *  - "splitk" (outputs too small to give every compute unit a 64x64 tile,
+ *    e.g. 512x128 * 128x384): one 32x32 output tile per workgroup, its four
+ *    wavefronts take the 32-wide K chunks round-robin straight from global
+ *    memory (no LDS staging, no barrier in the loop) and add their partial
+ *    tiles through LDS at the end.  Same accumulator layout and epilogue as
+ *    the mfma kernel; the serial MFMA chain per wave is a quarter as long and
+ *    there are four times as many workgroups.
  */
 #include "blt_hip.h"
 #include "blt_fatal.h"
@@ -148,6 +156,81 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_kernel(MatmulArgs g) {
     }
 }
 
+/* 32x32 output tile per workgroup, K split over the four waves. */
+template <bool VEC, bool ROPE>
+__global__ __launch_bounds__(256, 2) void matmul_splitk_kernel(MatmulArgs g) {
+    __shared__ float part[4][16][64];
+
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t h = lane >> 5, c = lane & 31u;
+    const uint32_t row = blockIdx.y * 32u + c, col = blockIdx.x * 32u + c;
+    const float *arow = g.a + (size_t)min(row, g.m - 1u) * g.lda;
+    const float *bcol = g.b + min(col, g.n - 1u);
+
+    /* fragments of one 32-wide K chunk: lane (h, c) holds a[row][k0 + 16h + t] and b[k0 + 16h + t][col] */
+    auto fetch = [&](uint32_t k0, float (&fa)[16], float (&fb)[16]) __attribute__((always_inline)) {
+        const uint32_t kb = k0 + 16u * h;
+        if (VEC) {
+#pragma unroll
+            for (int t = 0; t < 16; t += 4) {
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (kb + t < g.k) v = *reinterpret_cast<const float4 *>(arow + kb + t);
+                fa[t + 0] = v.x, fa[t + 1] = v.y, fa[t + 2] = v.z, fa[t + 3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 16; t++) fa[t] = kb + t < g.k ? arow[kb + t] : 0.f;
+        }
+#pragma unroll
+        for (int t = 0; t < 16; t++) fb[t] = kb + t < g.k ? bcol[(size_t)(kb + t) * g.ldb] : 0.f;
+    };
+
+    floatx16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    const uint32_t chunks = (g.k + 31u) / 32u;
+    float fa[16], fb[16];
+    uint32_t ch = wave;
+    if (ch < chunks) fetch(ch * 32u, fa, fb);
+    while (ch < chunks) {
+        const uint32_t nx = ch + 4u;
+        float na[16], nb[16];
+        if (nx < chunks) fetch(nx * 32u, na, nb);
+#pragma unroll
+        for (int t = 0; t < 16; t++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[t], fa[t], acc, 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < 16; t++) fa[t] = na[t], fb[t] = nb[t];
+        ch = nx;
+    }
+
+#pragma unroll
+    for (int r = 0; r < 16; r++) part[wave][r][lane] = acc[r];
+    __syncthreads();
+    /* wave w finishes register group w: out[row][col0 + 8w + 4h + 0..3] */
+    float v4[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        v4[i] = (part[0][4 * wave + i][lane] + part[1][4 * wave + i][lane]) +
+                (part[2][4 * wave + i][lane] + part[3][4 * wave + i][lane]);
+    if (row >= g.m) return;
+    const uint32_t oc = blockIdx.x * 32u + 8u * wave + 4u * h;
+    float4 v = make_float4(v4[0], v4[1], v4[2], v4[3]);
+    if (ROPE && oc < g.rope_cols) {
+        const size_t at = (size_t)row * (g.head_dim / 2u) + (oc % g.head_dim) / 2u;
+        v = rope_rotate4(v, g.rope_cos + at, g.rope_sin + at);
+    }
+    float *orow = g.out + (size_t)row * g.ldo;
+    if (VEC && (g.ldo % 4u == 0u) && ((reinterpret_cast<uintptr_t>(g.out) & 15u) == 0u)) {
+        if (oc < g.n) *reinterpret_cast<float4 *>(orow + oc) = v;
+    } else {
+        if (oc + 0 < g.n) orow[oc + 0] = v.x;
+        if (oc + 1 < g.n) orow[oc + 1] = v.y;
+        if (oc + 2 < g.n) orow[oc + 2] = v.z;
+        if (oc + 3 < g.n) orow[oc + 3] = v.w;
+    }
+}
+
 /* R rows of a per thread, one output column per thread. */
 template <int R>
 __global__ __launch_bounds__(256) void matmul_skinny_kernel(MatmulArgs g) {
@@ -191,6 +274,18 @@ void matmul_f32_launch(const MatmulArgs &g, hipStream_t s) {
     const dim3 grid((g.n + TN - 1) / TN, (g.m + TM - 1) / TM), block(256);
     const bool vec = aligned16(g.a) && aligned16(g.b) && g.lda % 4u == 0 && g.ldb % 4u == 0 && g.k % 4u == 0 &&
                      g.n % 4u == 0;
+    if ((uint64_t)grid.x * grid.y < 128u) {
+        /* fewer 64x64 tiles than half the compute units: quarter tiles, K split over the waves */
+        const dim3 sgrid((g.n + 31u) / 32u, (g.m + 31u) / 32u);
+        if (rope) {
+            if (vec) blt_launch("matmul_splitk", matmul_splitk_kernel<true, true>, sgrid, block, 0, s, g);
+            else blt_launch("matmul_splitk", matmul_splitk_kernel<false, true>, sgrid, block, 0, s, g);
+        } else {
+            if (vec) blt_launch("matmul_splitk", matmul_splitk_kernel<true, false>, sgrid, block, 0, s, g);
+            else blt_launch("matmul_splitk", matmul_splitk_kernel<false, false>, sgrid, block, 0, s, g);
+        }
+        return;
+    }
     if (rope) {
         if (vec) blt_launch("matmul_mfma", matmul_mfma_kernel<true, true>, grid, block, 0, s, g);
         else blt_launch("matmul_mfma", matmul_mfma_kernel<false, true>, grid, block, 0, s, g);
