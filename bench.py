@@ -29,13 +29,13 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 # the plain 64 MiB streaming copy (--probe-copy-mib 64): x1.999 for FETCH_SIZE,
 # x1.000 for WRITE_SIZE.  The summaries under profiles/ hold the readings.
 MEASURED_TRAFFIC_BYTES = {
-    "c2_patch_block_causal": (6250.1 * 1.999 + 4096.0) * 1024,
-    "c1_local_decoder_causal": (715.0 * 1.999 + 256.0) * 1024,
+    "c2_patch_block_causal": (6243.1 * 1.999 + 4096.0) * 1024,
+    "c1_local_decoder_causal": (708.6 * 1.999 + 256.0) * 1024,
     "c3_encoder_cross": (4699.1 * 1.999 + 1024.0) * 1024,
-    "c4_kv_decode": (12157.2 * 1.999 + 664.4) * 1024,
-    "c5_block_verify_B4": (10250.3 * 1.999 + 2064.5) * 1024,
-    "c5_block_verify_B8": (10278.5 * 1.999 + 1977.3) * 1024,   # B = 8 and 16 were collected together
-    "c5_block_verify_B16": (10278.5 * 1.999 + 1977.3) * 1024,
+    "c4_kv_decode": (12198.8 * 1.999 + 664.9) * 1024,           # mean over the 256 growing steps
+    "c5_block_verify_B4": (10268.6 * 1.999 + 2065.2) * 1024,
+    "c5_block_verify_B8": (10263.3 * 1.999 + 1977.0) * 1024,   # B = 8 and 16 run the same kernel and were
+    "c5_block_verify_B16": (10263.3 * 1.999 + 1977.0) * 1024,  # collected together
 }
 
 
