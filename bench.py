@@ -264,6 +264,10 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU budget of the headline workload")
     ap.add_argument("--probe-copy-mib", type=int, default=0,
                     help="only run the plain streaming copy of this many MiB --steps times (counter yardstick)")
+    ap.add_argument("--probe-read-mib", default="",
+                    help="only run the plain streaming read over buffers of these sizes (comma list of MiB)")
+    ap.add_argument("--probe-issue", action="store_true",
+                    help="only run the matrix / vector issue probe (do fp32 MFMA and VALU overlap on a SIMD?)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the workload shards by sequence "
@@ -288,6 +292,30 @@ def main():
         dt = time.perf_counter() - t0
         print(json.dumps({"probe": "stream_copy", "bytes_in": nbytes, "bytes_out": nbytes, "launches": args.steps,
                           "GBps_read_plus_write": 2.0 * nbytes * args.steps / dt / 1e9}), flush=True)
+        return
+
+    if args.probe_read_mib:
+        from fblt_amd import api
+        lib = api.load()
+        sizes = [int(x) for x in args.probe_read_mib.split(",") if x]
+        buf = torch.ones((max(sizes) << 20) // 4, dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()
+        out = []
+        for mib in sizes:
+            ms = lib.blt_hip_stream_read_probe(buf.data_ptr(), mib << 20, 10)
+            out.append({"MiB": mib, "us_per_launch": ms * 1e3, "GBps": (mib << 20) / ms / 1e6,
+                        "frac_of_hbm_peak": (mib << 20) / ms / 1e6 / HBM_PEAK_GBS})
+        print(json.dumps({"probe": "stream_read", "results": out}), flush=True)
+        return
+    if args.probe_issue:
+        from fblt_amd import api
+        lib = api.load()
+        groups = 4000
+        ms = {m: min(lib.blt_hip_issue_probe(m, groups) for _ in range(3)) for m in (1, 2, 3)}
+        tflops = 256 * 4 * groups * 8 * 4096 / (ms[1] * 1e-3) / 1e12   # one matrix wave per SIMD
+        print(json.dumps({"probe": "issue", "groups": groups, "ms_matrix_only": ms[1], "ms_vector_only": ms[2],
+                          "ms_both": ms[3], "both_over_sum": ms[3] / (ms[1] + ms[2]),
+                          "both_over_max": ms[3] / max(ms[1], ms[2]), "matrix_only_TFLOPs": tflops}), flush=True)
         return
 
     only = set(x for x in args.only.split(",") if x)
