@@ -383,7 +383,7 @@ void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_s
     a.partial = sc.partial;
     a.tickets = sc.tickets;
 
-    /* Blocks of five or more rows go to the matrix-core kernel (one launch for
+    /* Blocks of four or more rows go to the matrix-core kernel (one launch for
      * up to 32 rows; its cost does not depend on the row count) where it takes
      * the head_dim; shorter blocks, single rows and the shapes it does not
      * take go to the VALU kernel in slices of at most 16 rows.
@@ -394,11 +394,12 @@ void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_s
         const char *e = getenv("BLT_HIP_BLOCK_KERNEL");
         return e && strcmp(e, "valu") == 0 ? 1 : e && strcmp(e, "mfma") == 0 ? 2 : 0;
     }();
-    const bool want_mfma = pinned == 2 || (pinned == 0 && a.n >= 5u);
+    const bool want_mfma = pinned == 2 || (pinned == 0 && a.n >= 4u);
     if (want_mfma && (hd == 32 || hd == 64)) {
         /* the block kernel merges slices inside the workgroup, so it wants few,
          * long spans: just enough workgroups to cover the compute units */
-        const size_t zblocks = (H + 1) / 2;
+        a.hpb = kv_block_heads_per_group((uint32_t)cache->batch, (uint32_t)subs, (uint32_t)H);
+        const size_t zblocks = (H + a.hpb - 1) / a.hpb;
         size_t bs = span_env > 0 ? (subs + span_env - 1) / span_env : (256 + cache->batch * zblocks - 1) / (cache->batch * zblocks);
         bs = std::max<size_t>(1, std::min<size_t>(std::min<size_t>(bs, MAX_SPLITS), (subs + 3) / 4));
         const size_t bspan = (subs + bs - 1) / bs;

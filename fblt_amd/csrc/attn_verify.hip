@@ -291,8 +291,8 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block_mfma_kernel(StepArgs a
 
 template <int HD, int WAVES>
 void launch_block(StepArgs a, uint32_t batch, hipStream_t s) {
-    /* two heads per workgroup when there are several: the other waves are slices */
-    a.hpb = std::min<uint32_t>(a.num_heads, WAVES >= 4 ? 2u : 1u);
+    /* a.hpb heads per workgroup (the caller's choice, see kv_block_heads_per_group); the other waves are slices */
+    a.hpb = std::max(1u, std::min<uint32_t>(std::min<uint32_t>(a.hpb, a.num_heads), (uint32_t)WAVES));
     const uint32_t subs = (a.span + 31u) / 32u;
     a.slices = std::max(1u, std::min<uint32_t>((uint32_t)WAVES / a.hpb, subs));
     dim3 grid(a.splits, batch, (a.num_heads + a.hpb - 1) / a.hpb);
@@ -300,6 +300,16 @@ void launch_block(StepArgs a, uint32_t batch, hipStream_t s) {
 }
 
 } // namespace
+
+/* Heads per workgroup for `batch` sequences of `subs` 32-key sub-chunks: one
+ * head (all waves are slices of it, which keeps short launches free of the
+ * cross-workgroup merge) when there are enough sub-chunks to occupy the
+ * slices and one workgroup per (sequence, head) does not exceed what the
+ * chip holds at once (one 8-wave workgroup per compute unit); else two. */
+uint32_t kv_block_heads_per_group(uint32_t batch, uint32_t subs, uint32_t num_heads) {
+    if (num_heads == 1u) return 1u;
+    return subs >= 4u && (uint64_t)batch * num_heads <= 256u ? 1u : 2u;
+}
 
 /* Takes head_dim 32 and 64 (the K tiles of four waves fit the static LDS
  * budget); the caller falls back to the VALU kernel otherwise.  Handles up to

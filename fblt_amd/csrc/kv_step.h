@@ -74,7 +74,9 @@ __device__ __forceinline__ float observe(const float *p) {
 template <int HD>
 __device__ __forceinline__ void kv_finish_sequence(const StepArgs &a, uint32_t slots, uint32_t b, uint32_t nk,
                                                    uint32_t *sm_ticket) {
-    if (a.splits == 1u && gridDim.z == 1u) {
+    if (a.splits == 1u && (gridDim.z == 1u || !a.commit)) {
+        /* the output rows are written; the ticket is only needed to tell when the
+         * last workgroup of the sequence has read the old length */
         if (a.commit && threadIdx.x == 0) a.self_len[b] = nk;
         return;
     }
@@ -122,6 +124,8 @@ __device__ __forceinline__ void kv_finish_sequence(const StepArgs &a, uint32_t s
     }
 }
 
+/* heads per workgroup the MFMA block kernel should be launched with (set StepArgs.hpb to it) */
+uint32_t kv_block_heads_per_group(uint32_t batch, uint32_t subs, uint32_t num_heads);
 /* launch of the MFMA block kernel (attn_verify.hip); false when it does not take the shape */
 bool kv_block_mfma_launch(const StepArgs &a, uint32_t batch, uint32_t head_dim, hipStream_t s);
 
