@@ -259,7 +259,8 @@ Scratch &scratch() {
 template <int G, int NQ, int WAVES>
 void launch_step(StepArgs a, uint32_t batch, hipStream_t s) {
     constexpr int HD = 4 * G;
-    a.hpb = std::min<uint32_t>(a.num_heads, (uint32_t)WAVES);
+    /* a.hpb == 0: as many heads per workgroup as there are waves */
+    a.hpb = std::min<uint32_t>(a.num_heads, a.hpb ? std::min<uint32_t>(a.hpb, (uint32_t)WAVES) : (uint32_t)WAVES);
     a.slices = std::max<uint32_t>(1u, (uint32_t)WAVES / a.hpb);
     /* no more slices than a span has sub-chunks */
     const uint32_t subs = (a.span + SUB - 1) / SUB;
@@ -282,7 +283,7 @@ void dispatch_nq(const StepArgs &a, uint32_t nq, uint32_t batch, hipStream_t s) 
     /* single rows: one wave per head, and a second slice of waves once a split
      * holds enough keys to keep both busy */
     static const int pinned_waves = env_int("BLT_HIP_DECODE_WAVES", 0);
-    const int waves = pinned_waves > 0 ? pinned_waves : (a.span >= 256u ? 8 : 4);
+    const int waves = pinned_waves > 0 ? pinned_waves : (a.hpb == 1u ? 16 : a.span >= 256u ? 8 : 4);
     if (nq <= 1) {
         if (waves >= 16) launch_step<G, 1, 16>(a, batch, s);
         else if (waves >= 8) launch_step<G, 1, 8>(a, batch, s);
@@ -345,7 +346,7 @@ void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_s
     a.n = (uint32_t)n;
     a.scale = 1.0f / sqrtf((float)hd);
     a.block_kind = step_kind == BLT_KV_STEP_BLOCK;
-    a.hpb = a.slices = 1;
+    a.hpb = 0, a.slices = 1;
 
     /* enough workgroups to fill 256 compute units a few times over (sequences
      * shorter than the hint leave theirs idle), but no span shorter than two
@@ -360,6 +361,18 @@ void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_s
     splits = (subs + span_subs - 1) / span_subs;
     a.splits = (uint32_t)splits;
     a.span = (uint32_t)(span_subs * SUB);
+    a.hpb = 0;
+    /* Single rows of a batch that one workgroup per (sequence, head) already
+     * spreads over the chip: all 16 waves of a workgroup slice one head's keys
+     * and merge through LDS, so nothing crosses workgroups but the ticket.
+     * BLT_HIP_DECODE_HPB=0 keeps the split layout (tuning hook). */
+    static const int hpb_env = env_int("BLT_HIP_DECODE_HPB", 1);
+    if (hpb_env == 1 && a.n == 1u && span_env == 0 && subs >= 4 && subs <= 64 && cache->batch * H >= 128 &&
+        cache->batch * H <= 512) {
+        a.hpb = 1;
+        a.splits = 1;
+        a.span = (uint32_t)(subs * SUB);
+    }
 
     Scratch &sc = scratch();
     const size_t need = cache->batch * (size_t)MAX_SPLITS * H * 32u * (hd + 2); /* 32 = widest query block */
