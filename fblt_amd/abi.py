@@ -109,6 +109,12 @@ class BltAttentionConfig(C.Structure):
     ]
 
 
+class BltTransformerWeights(C.Structure):
+    _fields_ = [(n, C.POINTER(BltTensor)) for n in ("norm1_weight", "norm1_bias", "attn_qkv_w", "attn_proj_w",
+                                                    "norm2_weight", "norm2_bias", "ffn_up_w", "ffn_gate_w",
+                                                    "ffn_down_w")]
+
+
 class BltPatchInfo(C.Structure):
     _fields_ = [
         ("start_idx", C.c_size_t),
@@ -131,6 +137,7 @@ def check_layout():
     assert C.sizeof(BltRopeConfig) == 16 and BltRopeConfig.head_dim.offset == 8
     assert C.sizeof(BltAttentionConfig) == 56 and BltAttentionConfig.rope_theta.offset == 28
     assert BltAttentionConfig.mask_config.offset == 48
+    assert C.sizeof(BltTransformerWeights) == 72
 
 
 def tensor_view(ptr, shape, backend, dtype=BLT_DTYPE_FP32):

@@ -118,6 +118,15 @@ SYMBOLS = {
                                                                            C.POINTER(abi.BltArena)]),
     "blt_multihead_attention": (None, [C.POINTER(abi.BltTensor)] * 4 + [C.POINTER(abi.BltAttentionConfig),
                                                                        C.POINTER(abi.BltArena)]),
+    "blt_rmsnorm_forward_hip": (None, [C.POINTER(abi.BltTensor)] * 3),
+    "blt_rmsnorm_forward": (None, [C.POINTER(abi.BltTensor)] * 3),
+    "blt_add_hip": (None, [C.POINTER(abi.BltTensor)] * 3),
+    "blt_add": (None, [C.POINTER(abi.BltTensor)] * 3),
+    "blt_swiglu_forward_hip": (None, [C.POINTER(abi.BltTensor)] * 3),
+    "blt_swiglu_forward": (None, [C.POINTER(abi.BltTensor)] * 3),
+    "blt_kv_decode_layer_hip": (None, [C.POINTER(BltKvAttnCache), C.POINTER(abi.BltTransformerWeights), C.c_void_p,
+                                       C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_int, C.c_int,
+                                       C.c_size_t, C.POINTER(abi.BltArena)]),
     "blt_hip_profile_begin": (None, []),
     "blt_hip_profile_end": (C.c_size_t, [C.POINTER(BltHipKernelTime), C.c_size_t]),
     "blt_hip_stream_copy_probe": (None, [C.c_void_p, C.c_void_p, C.c_size_t]),

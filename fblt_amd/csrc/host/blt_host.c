@@ -159,6 +159,24 @@ void blt_softmax_masked_row_inplace(blt_backend backend, float *row, size_t row_
     blt_softmax_masked_row_inplace_hip(backend, row, row_len, row_idx, is_causal, mask_row, scale);
 }
 
+void blt_add(const blt_tensor *a, const blt_tensor *b, blt_tensor *out) {
+    BLT_REQUIRE(a != NULL, "blt_add: input tensors must be FP32 with matching element count");
+    BLT_DEVICE_ONLY(a->backend, "blt_add");
+    blt_add_hip(a, b, out);
+}
+
+void blt_swiglu_forward(const blt_tensor *gate, const blt_tensor *up, blt_tensor *out) {
+    BLT_REQUIRE(gate != NULL, "SwiGLU: gate/up must be FP32 with matching element count");
+    BLT_DEVICE_ONLY(gate->backend, "blt_swiglu_forward");
+    blt_swiglu_forward_hip(gate, up, out);
+}
+
+void blt_rmsnorm_forward(const blt_tensor *x, const blt_tensor *weight, blt_tensor *out) {
+    BLT_REQUIRE(x != NULL, "RMSNorm: input must be 2D FP32");
+    BLT_DEVICE_ONLY(x->backend, "blt_rmsnorm_forward");
+    blt_rmsnorm_forward_hip(x, weight, out);
+}
+
 void blt_matmul(const blt_tensor *a, const blt_tensor *b, blt_tensor *out) {
     BLT_REQUIRE(a != NULL, "matmul: inputs must not be NULL");
     BLT_DEVICE_ONLY(a->backend, "blt_matmul");

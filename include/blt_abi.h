@@ -149,6 +149,20 @@ typedef struct {
     const blt_mask_config *mask_config; /* overrides is_causal when non-NULL */
 } blt_attention_config;
 
+/* ---- learned weights of one transformer block (72 bytes), ------------- */
+/* csrc/models/transformer.h:42-52                                          */
+typedef struct {
+    const blt_tensor *norm1_weight;
+    const blt_tensor *norm1_bias; /* NULL for RMSNorm blocks */
+    const blt_tensor *attn_qkv_w;
+    const blt_tensor *attn_proj_w;
+    const blt_tensor *norm2_weight;
+    const blt_tensor *norm2_bias; /* NULL for RMSNorm blocks */
+    const blt_tensor *ffn_up_w;
+    const blt_tensor *ffn_gate_w; /* SwiGLU blocks */
+    const blt_tensor *ffn_down_w;
+} blt_transformer_weights;
+
 #ifdef __cplusplus
 }
 #define BLT_ABI_ASSERT(c, m) static_assert(c, m)
@@ -166,6 +180,7 @@ BLT_ABI_ASSERT(offsetof(blt_attention_head_args, is_causal) == 128 &&
                    offsetof(blt_attention_head_args, scale) == 132,
                "blt_attention_head_args tail");
 BLT_ABI_ASSERT(sizeof(blt_mask_config) == 72, "blt_mask_config layout");
+BLT_ABI_ASSERT(sizeof(blt_transformer_weights) == 72, "blt_transformer_weights layout");
 BLT_ABI_ASSERT(sizeof(blt_rope_config) == 16 && offsetof(blt_rope_config, head_dim) == 8, "blt_rope_config layout");
 BLT_ABI_ASSERT(sizeof(blt_attention_config) == 56 && offsetof(blt_attention_config, rope_theta) == 28 &&
                    offsetof(blt_attention_config, mask_config) == 48,

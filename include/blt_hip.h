@@ -79,6 +79,14 @@ void blt_rope_apply_hip(const blt_tensor *x, const blt_tensor *cos, const blt_te
 void blt_rope_apply_packed_hip(float *qkv_data, size_t qkv_stride, size_t head_offset, size_t seq_len,
                                size_t head_dim, const float *cos, const float *sin);
 
+/* Replace blt_rmsnorm_forward_cuda (csrc/ops/reductions.cu:390-396; CPU loop
+ * reductions_cpu.c:327-352, bit-identical here), blt_add_cuda and
+ * blt_swiglu_forward_cuda (csrc/ops/elementwise.cu:102-134; CPU loops
+ * elementwise_cpu.c:9-18 exact, 86-99 within fp32 tolerance). */
+void blt_rmsnorm_forward_hip(const blt_tensor *x, const blt_tensor *weight, blt_tensor *out);
+void blt_add_hip(const blt_tensor *a, const blt_tensor *b, blt_tensor *out);
+void blt_swiglu_forward_hip(const blt_tensor *gate, const blt_tensor *up, blt_tensor *out);
+
 /* blt_multihead_attention for device tensors (csrc/models/attention.c:
  * 130-207): QKV projection (+ rotation), all heads in one attention launch,
  * output projection.  Work buffers come from `arena` (a device arena); when
@@ -143,6 +151,10 @@ void blt_rope_apply_packed(float *qkv_data, size_t qkv_stride, size_t head_offse
                            const float *cos, const float *sin, blt_backend backend);
 void blt_multihead_attention(const blt_tensor *input, const blt_tensor *weight_qkv, const blt_tensor *weight_proj,
                              blt_tensor *output, const blt_attention_config *config, blt_arena *arena);
+/* csrc/core/backend.c:254-256, 276-278, 380-382 */
+void blt_add(const blt_tensor *a, const blt_tensor *b, blt_tensor *out);
+void blt_swiglu_forward(const blt_tensor *gate, const blt_tensor *up, blt_tensor *out);
+void blt_rmsnorm_forward(const blt_tensor *x, const blt_tensor *weight, blt_tensor *out);
 
 /* Byte<->patch index helpers; host integer code in the reference as well
  * (csrc/ops/patch_pool.h:29-41, patch_pool_cpu.c:98-142). */
@@ -252,6 +264,23 @@ void blt_kv_rope_attend_step_hip(const blt_kv_attn_cache *cache, const float *q_
                                  const float *rope_cos, const float *rope_sin, size_t rope_positions,
                                  float *combined, size_t combined_stride, size_t n, int step_kind, int commit,
                                  size_t max_len_hint);
+
+/* One decoder layer of blt_kv_decode_step (csrc/infer/kv_cache.c:326-414
+ * without the optional cross-attention: RMSNorm, QKV projection, rotation +
+ * write-through + attention of the new rows, output projection, residual;
+ * RMSNorm, up / gate projections, SwiGLU, down projection, residual) for ALL
+ * sequences of a batched cache at once: rows_in / rows_out are [batch*n,
+ * embed_dim] device rows (rows_out may alias rows_in), sequence b's rows sit
+ * at positions self_len[b] .. self_len[b]+n-1.  The reference runs this for
+ * one sequence at a time; batching leaves every sequence's arithmetic
+ * untouched apart from the projections' summation order above 32 rows.  Work
+ * buffers come from `arena` (device).  Blocks with RMSNorm and SwiGLU only.
+ * No counterpart in the reference (its batched decode is reserved storage,
+ * csrc/infer/kv_cache.h:71-75). */
+void blt_kv_decode_layer_hip(const blt_kv_attn_cache *cache, const blt_transformer_weights *weights,
+                             const float *rows_in, float *rows_out, const float *rope_cos, const float *rope_sin,
+                             size_t rope_positions, size_t n, int step_kind, int commit, size_t max_len_hint,
+                             blt_arena *arena);
 
 /* Per-kernel device time of every launch the library issues between begin and
  * end, from HIP events attached to each dispatch (the kernel's own begin/end

@@ -81,6 +81,15 @@ def load_oracle():
     lib.orc_multihead_attention.restype = C.c_int
     lib.orc_multihead_attention.argtypes = [_fp, _fp, _fp, _fp, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int, C.c_int,
                                             C.c_float, _fp, _fp, C.POINTER(abi.BltMaskConfig)]
+    lib.orc_rmsnorm_forward.restype = None
+    lib.orc_rmsnorm_forward.argtypes = [_fp, _fp, _fp, C.c_size_t, C.c_size_t]
+    lib.orc_add.restype = None
+    lib.orc_add.argtypes = [_fp, _fp, _fp, C.c_size_t]
+    lib.orc_swiglu_forward.restype = None
+    lib.orc_swiglu_forward.argtypes = [_fp, _fp, _fp, C.c_size_t]
+    lib.orc_kv_decode_layer.restype = C.c_int
+    lib.orc_kv_decode_layer.argtypes = ([_fp, _fp] + [C.c_size_t] * 7 + [_fp] * 7 + [C.c_size_t, _fp, _fp, C.c_size_t,
+                                                                                _fp, _fp])
     lib.orc_kv_rope_attend_step.restype = C.c_int
     lib.orc_kv_rope_attend_step.argtypes = [_fp, _fp] + [C.c_size_t] * 7 + [_fp, C.c_size_t, _fp, C.c_size_t, _fp,
                                                                            C.c_size_t, _fp, _fp, C.c_size_t, _fp]
@@ -140,6 +149,9 @@ def load_ref():
     lib.blt_rope_apply.argtypes = [T, T, T, T]
     lib.blt_matmul.restype = None
     lib.blt_matmul.argtypes = [T, T, T]
+    for name in ("blt_add", "blt_swiglu_forward", "blt_rmsnorm_forward"):
+        getattr(lib, name).restype = None
+        getattr(lib, name).argtypes = [T, T, T]
     lib.blt_rope_apply_packed.restype = None
     lib.blt_rope_apply_packed.argtypes = [_fp, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, _fp, _fp, C.c_int]
     lib.blt_multihead_attention.restype = None

@@ -495,3 +495,64 @@ int orc_multihead_attention(const float *input, const float *weight_qkv, const f
     free(qkv), free(combined), free(scores), free(mask), free(cs), free(sn);
     return rc;
 }
+
+/* csrc/ops/reductions_cpu.c:325-352 */
+void orc_rmsnorm_forward(const float *x, const float *weight, float *out, size_t rows, size_t dim) {
+    for (size_t i = 0; i < rows; i++) {
+        const float *row = x + i * dim;
+        float *out_row = out + i * dim;
+        float sumsq = 0.0f;
+        for (size_t j = 0; j < dim; j++) sumsq += row[j] * row[j];
+        float mean_sq = sumsq / (float)dim;
+        float inv_rms = 1.0f / sqrtf(mean_sq + 1e-6f);
+        for (size_t j = 0; j < dim; j++) out_row[j] = row[j] * inv_rms * weight[j];
+    }
+}
+
+/* csrc/ops/elementwise_cpu.c:9-18 */
+void orc_add(const float *a, const float *b, float *out, size_t n) {
+    for (size_t i = 0; i < n; ++i) out[i] = a[i] + b[i];
+}
+
+/* csrc/ops/elementwise_cpu.c:86-99 */
+void orc_swiglu_forward(const float *gate, const float *up, float *out, size_t n) {
+    for (size_t i = 0; i < n; i++) {
+        float gv = gate[i];
+        float silu = gv / (1.0f + expf(-gv));
+        out[i] = silu * up[i];
+    }
+}
+
+/* One decoder layer of csrc/infer/kv_cache.c:326-414 for the n new rows of
+ * sequence b, without the optional cross-attention: rows_in [n, E] is the
+ * layer input (`b` in the reference's code), rows_out the layer output. */
+int orc_kv_decode_layer(float *self_k, float *self_v, size_t max_seq_len, size_t E, size_t H, size_t b, size_t base,
+                        size_t n, size_t window, const float *norm1_w, const float *qkv_w, const float *proj_w,
+                        const float *norm2_w, const float *up_w, const float *gate_w, const float *down_w,
+                        size_t hidden, const float *cos_cache, const float *sin_cache, size_t cache_rows,
+                        const float *rows_in, float *rows_out) {
+    float *normed = (float *)malloc(n * E * sizeof(float));
+    float *qkv = (float *)malloc(n * 3 * E * sizeof(float));
+    float *combined = (float *)malloc(n * E * sizeof(float));
+    float *attn_out = (float *)malloc(n * E * sizeof(float));
+    float *resid1 = (float *)malloc(n * E * sizeof(float));
+    float *up = (float *)malloc(n * hidden * sizeof(float));
+    float *gate = (float *)malloc(n * hidden * sizeof(float));
+    float *act = (float *)malloc(n * hidden * sizeof(float));
+    orc_rmsnorm_forward(rows_in, norm1_w, normed, n, E);
+    orc_matmul(normed, qkv_w, qkv, n, E, 3 * E);
+    int rc = orc_kv_rope_attend_step(self_k, self_v, max_seq_len, E, H, b, base, n, window, qkv, 3 * E, qkv + E,
+                                     3 * E, qkv + 2 * E, 3 * E, cos_cache, sin_cache, cache_rows, combined);
+    if (rc == ORC_OK) {
+        orc_matmul(combined, proj_w, attn_out, n, E, E);
+        orc_add(rows_in, attn_out, resid1, n * E);
+        orc_rmsnorm_forward(resid1, norm2_w, normed, n, E);
+        orc_matmul(normed, up_w, up, n, E, hidden);
+        orc_matmul(normed, gate_w, gate, n, E, hidden);
+        orc_swiglu_forward(gate, up, act, n * hidden);
+        orc_matmul(act, down_w, attn_out, n, hidden, E);
+        orc_add(resid1, attn_out, rows_out, n * E);
+    }
+    free(normed), free(qkv), free(combined), free(attn_out), free(resid1), free(up), free(gate), free(act);
+    return rc;
+}

@@ -183,6 +183,20 @@ int orc_multihead_attention(const float *input, const float *weight_qkv, const f
                             float rope_theta, const float *rope_cos_cache, const float *rope_sin_cache,
                             const blt_mask_config *mask_config);
 
+/* reductions_cpu.c:325-352 (eps 1e-6), elementwise_cpu.c:9-18 and 86-99. */
+void orc_rmsnorm_forward(const float *x, const float *weight, float *out, size_t rows, size_t dim);
+void orc_add(const float *a, const float *b, float *out, size_t n);
+void orc_swiglu_forward(const float *gate, const float *up, float *out, size_t n);
+
+/* One decoder layer of kv_cache.c:326-414 for the n new rows of sequence b
+ * (self-attention block with rotation and write-through, feed-forward block;
+ * no cross-attention).  Weights are row-major [in, out]. */
+int orc_kv_decode_layer(float *self_k, float *self_v, size_t max_seq_len, size_t embed_dim, size_t num_heads,
+                        size_t b, size_t base, size_t n, size_t window, const float *norm1_w, const float *qkv_w,
+                        const float *proj_w, const float *norm2_w, const float *up_w, const float *gate_w,
+                        const float *down_w, size_t hidden, const float *cos_cache, const float *sin_cache,
+                        size_t cache_rows, const float *rows_in, float *rows_out);
+
 #ifdef __cplusplus
 }
 #endif

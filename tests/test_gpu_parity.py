@@ -613,3 +613,115 @@ def test_multihead_attention_block(T, E, H, causal, rope, mask, cached, oracle, 
     finally:
         lib.blt_arena_destroy(arena)
     assert_close(got, ref, "attention block T=%d E=%d H=%d" % (T, E, H))
+
+
+def test_row_ops(oracle, dev):
+    """blt_rmsnorm_forward and blt_add bit-identical to the reference loops, blt_swiglu_forward in tolerance."""
+    import torch
+    lib = api.load()
+    rs = np.random.RandomState(61)
+    for rows, dim in ((1, 128), (64, 128), (100, 512), (7, 33), (2048, 128), (3, 1000)):
+        x = (rs.randn(rows, dim) * 2).astype(np.float32)
+        w = rs.randn(dim).astype(np.float32)
+        y = rs.randn(rows, dim).astype(np.float32)
+        ref = np.zeros_like(x)
+        oracle.orc_rmsnorm_forward(binding.fptr(x.reshape(-1)), binding.fptr(w), binding.fptr(ref.reshape(-1)), rows, dim)
+        tx, tw, ty = torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda(), torch.from_numpy(y).cuda()
+        to = torch.zeros_like(tx)
+        vx, vw, vy, vo = _dev_tensor(tx), _dev_tensor(tw), _dev_tensor(ty), _dev_tensor(to)
+        lib.blt_rmsnorm_forward(C.byref(vx), C.byref(vw), C.byref(vo))
+        lib.blt_backend_pass_sync_hip()
+        assert to.cpu().numpy().tobytes() == ref.tobytes(), (rows, dim)
+        oracle.orc_add(binding.fptr(x.reshape(-1)), binding.fptr(y.reshape(-1)), binding.fptr(ref.reshape(-1)), rows * dim)
+        lib.blt_add(C.byref(vx), C.byref(vy), C.byref(vo))
+        lib.blt_backend_pass_sync_hip()
+        assert to.cpu().numpy().tobytes() == ref.tobytes()
+        oracle.orc_swiglu_forward(binding.fptr(x.reshape(-1)), binding.fptr(y.reshape(-1)), binding.fptr(ref.reshape(-1)),
+                                  rows * dim)
+        lib.blt_swiglu_forward(C.byref(vx), C.byref(vy), C.byref(vo))
+        lib.blt_backend_pass_sync_hip()
+        assert_close(to.cpu().numpy(), ref, "swiglu")
+
+
+@pytest.mark.parametrize("batch,n,H,hd,hidden,kind", [(3, 1, 2, 32, 96, "causal"), (64, 1, 4, 32, 256, "causal"),
+                                                      (5, 6, 2, 64, 200, "causal"), (9, 16, 4, 32, 128, "block")])
+def test_kv_decode_layer(batch, n, H, hd, hidden, kind, oracle, dev):
+    """blt_kv_decode_layer_hip for all sequences at once against the restated layer run per sequence."""
+    import torch
+    lib = api.load()
+    rs = np.random.RandomState(batch * 7 + n)
+    E, half = H * hd, hd // 2
+    max_len = 80 + 2 * n
+    lens = rs.randint(1, 70, size=batch).astype(np.uint32)
+    ck = rs.randn(batch * max_len, E).astype(np.float32)
+    cv = rs.randn(batch * max_len, E).astype(np.float32)
+    W = {k: (rs.randn(*shape) / np.sqrt(shape[0])).astype(np.float32)
+         for k, shape in dict(qkv=(E, 3 * E), proj=(E, E), up=(E, hidden), gate=(E, hidden), down=(hidden, E)).items()}
+    n1, n2 = (1.0 + 0.1 * rs.randn(E)).astype(np.float32), (1.0 + 0.1 * rs.randn(E)).astype(np.float32)
+    cos, sin = np.empty(max_len * half, dtype=np.float32), np.empty(max_len * half, dtype=np.float32)
+    oracle.orc_rope_precompute(max_len, 500000.0, hd, binding.fptr(cos), binding.fptr(sin))
+    x = rs.randn(batch * n, E).astype(np.float32)
+    fp = lambda a: binding.fptr(a.reshape(-1))
+    # reference: one sequence at a time (block rows: the verify step attends the whole block; the
+    # restated layer is causal, so block kind is checked through the device's own causal/block split below)
+    ref_k, ref_v = ck.copy(), cv.copy()
+    ref_out = np.zeros((batch * n, E), dtype=np.float32)
+    if kind == "causal":
+        for b in range(batch):
+            xb = np.ascontiguousarray(x[b * n:(b + 1) * n])
+            ob = np.zeros((n, E), dtype=np.float32)
+            assert oracle.orc_kv_decode_layer(fp(ref_k), fp(ref_v), max_len, E, H, b, int(lens[b]), n, 0, fp(n1),
+                                              fp(W["qkv"]), fp(W["proj"]), fp(n2), fp(W["up"]), fp(W["gate"]),
+                                              fp(W["down"]), hidden, fp(cos), fp(sin), max_len, fp(xb), fp(ob)) == 0
+            ref_out[b * n:(b + 1) * n] = ob
+    t = {k: torch.from_numpy(v).cuda() for k, v in W.items()}
+    tn1, tn2 = torch.from_numpy(n1).cuda(), torch.from_numpy(n2).cuda()
+    tck, tcv = torch.from_numpy(ck).cuda(), torch.from_numpy(cv).cuda()
+    tlens = torch.from_numpy(lens.astype(np.int32)).cuda()
+    tcos, tsin = torch.from_numpy(cos.reshape(max_len, half)).cuda(), torch.from_numpy(sin.reshape(max_len, half)).cuda()
+    tx = torch.from_numpy(x).cuda()
+    to = torch.zeros_like(tx)
+    views = {k: _dev_tensor(v) for k, v in t.items()}
+    vn1, vn2 = _dev_tensor(tn1), _dev_tensor(tn2)
+    w = abi.BltTransformerWeights()
+    w.norm1_weight, w.norm2_weight = C.pointer(vn1), C.pointer(vn2)
+    w.attn_qkv_w, w.attn_proj_w = C.pointer(views["qkv"]), C.pointer(views["proj"])
+    w.ffn_up_w, w.ffn_gate_w, w.ffn_down_w = C.pointer(views["up"]), C.pointer(views["gate"]), C.pointer(views["down"])
+    c = api.BltKvAttnCache()
+    c.self_k, c.self_v, c.self_len = tck.data_ptr(), tcv.data_ptr(), tlens.data_ptr()
+    c.batch, c.max_seq_len, c.embed_dim, c.num_heads, c.window = batch, max_len, E, H, 0
+    arena = lib.blt_arena_create(64 << 20, abi.BLT_BACKEND_HIP)
+    try:
+        step_kind = api.BLT_KV_STEP_CAUSAL if kind == "causal" else api.BLT_KV_STEP_BLOCK
+        lib.blt_kv_decode_layer_hip(C.byref(c), C.byref(w), tx.data_ptr(), to.data_ptr(), tcos.data_ptr(),
+                                    tsin.data_ptr(), max_len, n, step_kind, 1 if kind == "causal" else 0,
+                                    int(lens.max()) + n, arena)
+        lib.blt_backend_pass_sync_hip()
+        got = to.cpu().numpy()
+        got_k, got_v, got_len = tck.cpu().numpy(), tcv.cpu().numpy(), tlens.cpu().numpy()
+    finally:
+        lib.blt_arena_destroy(arena)
+    if kind == "causal":
+        assert (got_len == lens + n).all()
+        assert_close(got, ref_out, "decode layer")
+        # rows of a batch above 32 come from the matrix-core projection: cache rows in tolerance, not bitwise
+        assert_close(got_k, ref_k, "cache k")
+        assert_close(got_v, ref_v, "cache v")
+    else:
+        # block rows: same layer with the block step; check against the device's own pieces
+        assert (got_len == lens).all() and np.isfinite(got).all()
+        tx2 = torch.from_numpy(x).cuda()
+        normed = torch.zeros_like(tx2)
+        vx, vnm = _dev_tensor(tx2), _dev_tensor(normed)
+        lib.blt_rmsnorm_forward(C.byref(vx), C.byref(vn1), C.byref(vnm))
+        qkv = torch.zeros((batch * n, 3 * E), dtype=torch.float32, device="cuda")
+        vq = _dev_tensor(qkv)
+        lib.blt_matmul(C.byref(vnm), C.byref(views["qkv"]), C.byref(vq))
+        tck2, tcv2 = torch.from_numpy(ck).cuda(), torch.from_numpy(cv).cuda()
+        c.self_k, c.self_v = tck2.data_ptr(), tcv2.data_ptr()
+        comb = torch.zeros_like(tx2)
+        lib.blt_kv_rope_attend_step_hip(C.byref(c), qkv.data_ptr(), 3 * E, qkv.data_ptr() + 4 * E, 3 * E,
+                                        qkv.data_ptr() + 8 * E, 3 * E, tcos.data_ptr(), tsin.data_ptr(), max_len,
+                                        comb.data_ptr(), E, n, step_kind, 0, int(lens.max()) + n)
+        lib.blt_backend_pass_sync_hip()
+        assert tck2.cpu().numpy().tobytes() == got_k.tobytes()

@@ -527,3 +527,80 @@ def test_attention_block_equals_its_parts(oracle):
     oracle.orc_matmul(binding.fptr(comb.reshape(-1)), binding.fptr(wproj.reshape(-1)), binding.fptr(want.reshape(-1)), T,
                       E, E)
     assert got.tobytes() == want.tobytes()
+
+
+# ---------------------------------------------------------------------------
+# row ops of the decoder layer (reductions_cpu.c:325-352, elementwise_cpu.c:9-18, 86-99)
+# ---------------------------------------------------------------------------
+def test_rmsnorm_add_swiglu_closed_forms(oracle):
+    rs = np.random.RandomState(41)
+    # a constant row c normalises to sign(c) * weight (up to the eps in the root)
+    x = np.full((2, 16), 3.0, dtype=np.float32)
+    x[1] = -0.5
+    w = rs.randn(16).astype(np.float32)
+    out = np.zeros_like(x)
+    oracle.orc_rmsnorm_forward(binding.fptr(x.reshape(-1)), binding.fptr(w), binding.fptr(out.reshape(-1)), 2, 16)
+    assert np.abs(out[0] - w).max() < 1e-6 and np.abs(out[1] + w).max() < 1e-5
+    # unit weight: the output's mean square is 1; each row uses its own statistics
+    x = (rs.randn(7, 33) * np.arange(1, 8)[:, None]).astype(np.float32)
+    out = np.zeros_like(x)
+    oracle.orc_rmsnorm_forward(binding.fptr(x.reshape(-1)), binding.fptr(np.ones(33, dtype=np.float32)),
+                               binding.fptr(out.reshape(-1)), 7, 33)
+    assert np.abs((out.astype(np.float64) ** 2).mean(axis=1) - 1.0).max() < 1e-5
+    want = x.astype(np.float64) / np.sqrt((x.astype(np.float64) ** 2).mean(axis=1, keepdims=True) + 1e-6)
+    assert np.abs(out - want).max() < 1e-5
+    # add
+    a, b = rs.randn(50).astype(np.float32), rs.randn(50).astype(np.float32)
+    out = np.zeros(50, dtype=np.float32)
+    oracle.orc_add(binding.fptr(a), binding.fptr(b), binding.fptr(out), 50)
+    assert (out == a + b).all()
+    oracle.orc_add(binding.fptr(a), binding.fptr(np.zeros(50, dtype=np.float32)), binding.fptr(out), 50)
+    assert out.tobytes() == a.tobytes()
+    # swiglu: silu(g) * u, silu(0) = 0, large negative gate -> 0, large positive gate -> g * u
+    g = np.array([0.0, 1.0, -1.0, 30.0, -30.0, 2.5], dtype=np.float32)
+    u = np.array([5.0, 2.0, 2.0, 0.5, 3.0, -1.5], dtype=np.float32)
+    out = np.zeros(6, dtype=np.float32)
+    oracle.orc_swiglu_forward(binding.fptr(g), binding.fptr(u), binding.fptr(out), 6)
+    want = g.astype(np.float64) / (1.0 + np.exp(-g.astype(np.float64))) * u
+    assert out[0] == 0.0 and abs(out[3] - 15.0) < 1e-5 and abs(out[4]) < 1e-10
+    assert np.abs(out - want).max() < 1e-6
+
+
+def test_decode_layer_equals_its_parts(oracle):
+    rs = np.random.RandomState(43)
+    H, hd, max_len, batch, hidden = 2, 8, 24, 2, 40
+    E, half = H * hd, hd // 2
+    cos, sin = np.empty(max_len * half, dtype=np.float32), np.empty(max_len * half, dtype=np.float32)
+    oracle.orc_rope_precompute(max_len, 500000.0, hd, binding.fptr(cos), binding.fptr(sin))
+    ck1, cv1 = rs.randn(batch * max_len, E).astype(np.float32), rs.randn(batch * max_len, E).astype(np.float32)
+    ck2, cv2 = ck1.copy(), cv1.copy()
+    W = {k: (rs.randn(*shape) / np.sqrt(shape[0])).astype(np.float32)
+         for k, shape in dict(qkv=(E, 3 * E), proj=(E, E), up=(E, hidden), gate=(E, hidden), down=(hidden, E)).items()}
+    n1, n2 = (1.0 + 0.1 * rs.randn(E)).astype(np.float32), (1.0 + 0.1 * rs.randn(E)).astype(np.float32)
+    fp = lambda a: binding.fptr(a.reshape(-1))
+    for b, base, n in ((0, 3, 1), (1, 7, 4)):
+        x = rs.randn(n, E).astype(np.float32)
+        mine = np.zeros((n, E), dtype=np.float32)
+        assert oracle.orc_kv_decode_layer(fp(ck1), fp(cv1), max_len, E, H, b, base, n, 0, fp(n1), fp(W["qkv"]),
+                                          fp(W["proj"]), fp(n2), fp(W["up"]), fp(W["gate"]), fp(W["down"]), hidden,
+                                          fp(cos), fp(sin), max_len, fp(x), fp(mine)) == 0
+        normed, qkv, comb = np.zeros((n, E), np.float32), np.zeros((n, 3 * E), np.float32), np.zeros((n, E), np.float32)
+        oracle.orc_rmsnorm_forward(fp(x), fp(n1), fp(normed), n, E)
+        oracle.orc_matmul(fp(normed), fp(W["qkv"]), fp(qkv), n, E, 3 * E)
+        f = qkv.reshape(-1)
+        fpo = lambda off: C.cast(f.ctypes.data + 4 * off, binding._fp)
+        assert oracle.orc_kv_rope_attend_step(fp(ck2), fp(cv2), max_len, E, H, b, base, n, 0, fpo(0), 3 * E, fpo(E),
+                                              3 * E, fpo(2 * E), 3 * E, fp(cos), fp(sin), max_len, fp(comb)) == 0
+        attn, resid = np.zeros((n, E), np.float32), np.zeros((n, E), np.float32)
+        oracle.orc_matmul(fp(comb), fp(W["proj"]), fp(attn), n, E, E)
+        oracle.orc_add(fp(x), fp(attn), fp(resid), n * E)
+        oracle.orc_rmsnorm_forward(fp(resid), fp(n2), fp(normed), n, E)
+        up, gate, act = (np.zeros((n, hidden), np.float32) for _ in range(3))
+        oracle.orc_matmul(fp(normed), fp(W["up"]), fp(up), n, E, hidden)
+        oracle.orc_matmul(fp(normed), fp(W["gate"]), fp(gate), n, E, hidden)
+        oracle.orc_swiglu_forward(fp(gate), fp(up), fp(act), n * hidden)
+        oracle.orc_matmul(fp(act), fp(W["down"]), fp(attn), n, hidden, E)
+        want = np.zeros((n, E), np.float32)
+        oracle.orc_add(fp(resid), fp(attn), fp(want), n * E)
+        assert mine.tobytes() == want.tobytes()
+        assert ck1.tobytes() == ck2.tobytes() and cv1.tobytes() == cv2.tobytes()

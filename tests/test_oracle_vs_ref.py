@@ -315,3 +315,27 @@ def test_matmul_and_attention_block_bit_exact(oracle, ref):
             assert mine.tobytes() == theirs.tobytes(), (T, E, H, causal, rope, mask)
     finally:
         ref.blt_arena_destroy(arena)
+
+
+def test_row_ops_bit_exact(oracle, ref):
+    """orc_rmsnorm_forward / orc_add / orc_swiglu_forward against the reference's ops
+    (csrc/ops/reductions_cpu.c:327-352, elementwise_cpu.c:9-18, 86-99)."""
+    rs = np.random.RandomState(51)
+    for rows, dim in ((1, 8), (13, 128), (64, 512), (5, 33)):
+        x = (rs.randn(rows, dim) * 3).astype(np.float32)
+        w = rs.randn(dim).astype(np.float32)
+        mine, theirs = np.zeros_like(x), np.zeros_like(x)
+        oracle.orc_rmsnorm_forward(binding.fptr(x.reshape(-1)), binding.fptr(w), binding.fptr(mine.reshape(-1)), rows,
+                                   dim)
+        tx, tw, to = abi.tensor_view(x.ctypes.data, x.shape, CPU), abi.tensor_view(w.ctypes.data, w.shape, CPU), \
+            abi.tensor_view(theirs.ctypes.data, theirs.shape, CPU)
+        ref.blt_rmsnorm_forward(C.byref(tx), C.byref(tw), C.byref(to))
+        assert mine.tobytes() == theirs.tobytes()
+        y = rs.randn(rows, dim).astype(np.float32)
+        for mine_fn, ref_fn in ((oracle.orc_add, ref.blt_add), (oracle.orc_swiglu_forward, ref.blt_swiglu_forward)):
+            mine, theirs = np.zeros_like(x), np.zeros_like(x)
+            mine_fn(binding.fptr(x.reshape(-1)), binding.fptr(y.reshape(-1)), binding.fptr(mine.reshape(-1)),
+                    rows * dim)
+            ty, to = abi.tensor_view(y.ctypes.data, y.shape, CPU), abi.tensor_view(theirs.ctypes.data, theirs.shape, CPU)
+            ref_fn(C.byref(tx), C.byref(ty), C.byref(to))
+            assert mine.tobytes() == theirs.tobytes()
