@@ -227,6 +227,83 @@ def bench_block(name, T, E, H, steps, warmup, gemm_only=None):
     return res
 
 
+def bench_decode_layer(steps, warmup, batch=64, H=4, hd=32, hidden=512, len_hi=512):
+    """blt_kv_decode_layer_hip: one decoder layer (self-attention block with fused RoPE and
+    write-through, feed-forward block) for `batch` sequences, one new row each, per step."""
+    import ctypes as C
+    import numpy as np
+    import torch
+    from fblt_amd import abi, api, synth
+    lib = api.load()
+    E, half = H * hd, hd // 2
+    total = warmup + steps
+    max_len = len_hi + 2 * total + 2
+    lens = synth.integers(synth.seed_for(4, synth.S_LEN), batch, 1, len_hi).astype(np.int32)
+    g = torch.Generator(device="cpu").manual_seed(99)
+    rnd = lambda *shape: torch.randn(*shape, generator=g, dtype=torch.float32)
+    ck, cv = rnd(batch * max_len, E).cuda(), rnd(batch * max_len, E).cuda()
+    Wt = {k: (rnd(*shape) / shape[0] ** 0.5).cuda() for k, shape in
+          dict(qkv=(E, 3 * E), proj=(E, E), up=(E, hidden), gate=(E, hidden), down=(hidden, E)).items()}
+    n1, n2 = torch.ones(E, device="cuda"), torch.ones(E, device="cuda")
+    view = lambda t: abi.tensor_view(t.data_ptr(), tuple(t.shape), abi.BLT_BACKEND_HIP)
+    views = {k: view(v) for k, v in Wt.items()}
+    vn1, vn2 = view(n1), view(n2)
+    w = abi.BltTransformerWeights()
+    w.norm1_weight, w.norm2_weight = C.pointer(vn1), C.pointer(vn2)
+    w.attn_qkv_w, w.attn_proj_w = C.pointer(views["qkv"]), C.pointer(views["proj"])
+    w.ffn_up_w, w.ffn_gate_w, w.ffn_down_w = C.pointer(views["up"]), C.pointer(views["gate"]), C.pointer(views["down"])
+    cos, sin = torch.zeros((max_len, half), device="cuda"), torch.zeros((max_len, half), device="cuda")
+    vc, vs = view(cos), view(sin)
+    rcfg = abi.BltRopeConfig(500000.0, hd)
+    lib.blt_rope_precompute(max_len, C.byref(rcfg), C.byref(vc), C.byref(vs))
+    tl0 = torch.from_numpy(lens).cuda()
+    tl = tl0.clone()
+    c = api.BltKvAttnCache()
+    c.self_k, c.self_v, c.self_len = ck.data_ptr(), cv.data_ptr(), tl.data_ptr()
+    c.batch, c.max_seq_len, c.embed_dim, c.num_heads, c.window = batch, max_len, E, H, 0
+    x, o = rnd(batch, E).cuda(), torch.zeros((batch, E), device="cuda")
+    arena = lib.blt_arena_create(64 << 20, abi.BLT_BACKEND_HIP)
+    hint0 = int(lens.max())
+
+    def run(count, first):
+        for s in range(count):
+            arena.contents.offset = 0
+            lib.blt_kv_decode_layer_hip(C.byref(c), C.byref(w), x.data_ptr(), o.data_ptr(), cos.data_ptr(),
+                                        sin.data_ptr(), max_len, 1, api.BLT_KV_STEP_CAUSAL, 1, hint0 + first + s + 1,
+                                        arena)
+    run(warmup, 0)
+    lib.blt_backend_pass_sync_hip()
+    lib.blt_hip_profile_begin()
+    t0 = time.perf_counter()
+    run(steps, warmup)
+    lib.blt_backend_pass_sync_hip()
+    wall = time.perf_counter() - t0
+    prof = api.profile_end()
+    tl.copy_(tl0)
+    torch.cuda.synchronize()
+    run(warmup, 0)
+    lib.blt_backend_pass_sync_hip()
+    t0 = time.perf_counter()
+    run(steps, warmup)
+    lib.blt_backend_pass_sync_hip()
+    wall_plain = time.perf_counter() - t0
+    lib.blt_arena_destroy(arena)
+    avg_s = sum(v[1] for v in prof.values()) / 1e3 / steps
+    mean_keys = float(lens.astype("int64").sum()) + batch * (warmup + (steps - 1) / 2.0) + batch
+    flops = batch * 2.0 * (E * 3 * E + E * E + 3 * E * hidden) + 4.0 * hd * H * mean_keys
+    nbytes = 4.0 * (2 * E * mean_keys + 3 * E * E + E * E + 3 * E * hidden)
+    res = {"workload": "decoder layer step: %d sequences, E=%d, H=%d, hidden=%d, cached 1..%d" % (batch, E, H, hidden, len_hi),
+           "kernel": "+".join(sorted(prof)), "launches_per_step": sum(v[0] for v in prof.values()) / steps,
+           "tokens_per_step": batch, "us_per_step": wall_plain / steps * 1e6,
+           "us_per_step_with_events": wall / steps * 1e6, "kernel_us_avg": avg_s * 1e6,
+           "kernel_us_min": min(v[2] for v in prof.values()) * 1e3,
+           "per_kernel_us": {k: v[1] * 1e3 / steps for k, v in prof.items()},
+           "tokens_per_s": batch * steps / wall_plain, "tokens_per_s_kernel": batch / avg_s, "flops": flops,
+           "bytes": nbytes, "roofline_hbm": roofline("hbm", nbytes, avg_s), "roofline_mfma": roofline("mfma", flops, avg_s)}
+    res["roofline"] = res["roofline_hbm"]
+    return res
+
+
 def cpu_dense(w, budget_s):
     """Checker on one host core over the same workload; repeated whole passes up to the budget."""
     from oracle import binding, runner as orunner
@@ -371,6 +448,8 @@ def main():
         others["matmul_8192x512x1536"] = bench_block("blt_matmul 8192x512x1536", 0, 0, 0, max(10, K // 10), 3,
                                                      gemm_only=(8192, 512, 1536))
         log("matmul", json.dumps(others["matmul_8192x512x1536"]))
+        others["decode_layer"] = bench_decode_layer(K, W)
+        log("decode_layer", json.dumps(others["decode_layer"]))
 
     cpu_head = None
     if not args.no_cpu:

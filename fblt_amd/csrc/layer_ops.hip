@@ -31,8 +31,8 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const float *__restri
                                                            float *__restrict__ out, uint32_t rows, uint32_t dim,
                                                            uint32_t parts) {
 #pragma clang fp contract(off) /* products and sums rounded separately, as the reference's loop */
-    extern __shared__ float stage[]; /* [256 / parts rows][dim + 1] */
-    const uint32_t pitch = dim + 1u;
+    extern __shared__ __attribute__((aligned(16))) float stage[]; /* [256 / parts rows][pitch] */
+    const uint32_t pitch = ((dim + 3u) & ~3u) + 4u; /* rows start 16-byte aligned, 4 banks apart */
     const uint32_t r_local = threadIdx.x / parts, part = threadIdx.x % parts;
     const uint32_t row = blockIdx.x * (256u / parts) + r_local;
     const bool ok = row < rows;
@@ -42,10 +42,19 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const float *__restri
     float inv_rms = 0.f;
     if (part == 0) {
         float sumsq = 0.0f;
-        for (uint32_t j = 0; j < dim; j++) {
-            const float v = stage[r_local * pitch + j];
-            sumsq = sumsq + v * v;
+        const float *mine = stage + r_local * pitch;
+        uint32_t j = 0;
+        for (; j + 16u <= dim; j += 16u) { /* loads in bulk, then the sums in element order */
+            float v[16];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float4 t = *reinterpret_cast<const float4 *>(mine + j + 4 * q);
+                v[4 * q + 0] = t.x, v[4 * q + 1] = t.y, v[4 * q + 2] = t.z, v[4 * q + 3] = t.w;
+            }
+#pragma unroll
+            for (int q = 0; q < 16; q++) sumsq = sumsq + v[q] * v[q];
         }
+        for (; j < dim; j++) sumsq = sumsq + mine[j] * mine[j];
         const float mean_sq = sumsq / (float)dim;
         inv_rms = 1.0f / sqrtf(mean_sq + RMSNORM_EPS);
     }
@@ -75,10 +84,11 @@ uint32_t blocks_for(uint64_t n) { return (uint32_t)((n + 255u) / 256u < 2048u ? 
 void rmsnorm_launch(const float *x, const float *w, float *out, size_t rows, size_t dim) {
     if (rows == 0 || dim == 0) return;
     uint32_t parts = 8u; /* 32 rows per workgroup while they fit 48 KB of LDS, fewer for wide rows */
-    while (parts < 64u && (256u / parts) * (dim + 1u) * sizeof(float) > 48u * 1024u) parts *= 2u;
+    const size_t pitch = ((dim + 3u) & ~(size_t)3u) + 4u;
+    while (parts < 64u && (256u / parts) * pitch * sizeof(float) > 48u * 1024u) parts *= 2u;
     const uint32_t rpw = 256u / parts;
-    const size_t lds = rpw * (dim + 1u) * sizeof(float);
-    BLT_REQUIRE(lds <= 64u * 1024u, "RMSNorm: embed_dim up to 4095 is supported by the HIP backend (got %zu)", dim);
+    const size_t lds = rpw * pitch * sizeof(float);
+    BLT_REQUIRE(lds <= 64u * 1024u, "RMSNorm: embed_dim up to 4088 is supported by the HIP backend (got %zu)", dim);
     blt_launch("rmsnorm_rows", rmsnorm_rows_kernel, dim3((uint32_t)((rows + rpw - 1u) / rpw)), dim3(256), lds, 0, x, w,
                out, (uint32_t)rows, (uint32_t)dim, parts);
 }
@@ -100,10 +110,13 @@ void check_weight(const blt_tensor *t, size_t rows, size_t cols, const char *wha
                 "%s (the HIP backend takes FP32 device weights only)", what);
 }
 
-void gemm(const float *a, const float *b, float *out, size_t m, size_t k, size_t n) {
+/* out = a * b (+ residual), or silu(a * gate_w) .* (a * b) with gate_w set */
+void gemm(const float *a, const float *b, float *out, size_t m, size_t k, size_t n, const float *residual = nullptr,
+          const float *gate_w = nullptr, const float *norm_w = nullptr) {
     MatmulArgs g;
     std::memset(&g, 0, sizeof(g));
     g.a = a, g.b = b, g.out = out;
+    g.residual = residual, g.b2 = gate_w, g.norm_w = norm_w;
     g.m = (uint32_t)m, g.k = (uint32_t)k, g.n = (uint32_t)n;
     g.lda = (uint32_t)k, g.ldb = (uint32_t)n, g.ldo = (uint32_t)n;
     matmul_f32_launch(g, 0);
@@ -173,24 +186,37 @@ extern "C" void blt_kv_decode_layer_hip(const blt_kv_attn_cache *cache, const bl
     float *normed = (float *)blt_arena_alloc(arena, rows * E * sizeof(float), 64);
     float *qkv = (float *)blt_arena_alloc(arena, rows * 3 * E * sizeof(float), 64);
     float *combined = (float *)blt_arena_alloc(arena, rows * E * sizeof(float), 64);
-    float *attn_out = (float *)blt_arena_alloc(arena, rows * E * sizeof(float), 64);
     float *resid1 = (float *)blt_arena_alloc(arena, rows * E * sizeof(float), 64);
     float *up = (float *)blt_arena_alloc(arena, rows * Hd * sizeof(float), 64);
     float *gate = (float *)blt_arena_alloc(arena, rows * Hd * sizeof(float), 64);
 
+    MatmulArgs probe;
+    std::memset(&probe, 0, sizeof(probe));
+    probe.m = (uint32_t)rows, probe.k = (uint32_t)E;
     /* self-attention block, kv_cache.c:326-394 */
-    rmsnorm_launch(rows_in, f32(w->norm1_weight), normed, rows, E);
-    gemm(normed, f32(w->attn_qkv_w), qkv, rows, E, 3 * E);
+    probe.n = (uint32_t)(3 * E);
+    if (matmul_takes_norm(probe)) {
+        gemm(rows_in, f32(w->attn_qkv_w), qkv, rows, E, 3 * E, nullptr, nullptr, f32(w->norm1_weight));
+    } else {
+        rmsnorm_launch(rows_in, f32(w->norm1_weight), normed, rows, E);
+        gemm(normed, f32(w->attn_qkv_w), qkv, rows, E, 3 * E);
+    }
     blt_kv_rope_attend_step_hip(cache, qkv, 3 * E, qkv + E, 3 * E, qkv + 2 * E, 3 * E, rope_cos, rope_sin,
                                 rope_positions, combined, E, n, step_kind, commit, max_len_hint);
-    gemm(combined, f32(w->attn_proj_w), attn_out, rows, E, E);
-    add_launch(rows_in, attn_out, resid1, rows * E);
+    gemm(combined, f32(w->attn_proj_w), resid1, rows, E, E, rows_in); /* projection + residual in one pass */
     /* feed-forward block, kv_cache.c:396-414 */
-    rmsnorm_launch(resid1, f32(w->norm2_weight), normed, rows, E);
-    gemm(normed, f32(w->ffn_up_w), up, rows, E, Hd);
-    gemm(normed, f32(w->ffn_gate_w), gate, rows, E, Hd);
-    swiglu_launch(gate, up, gate, rows * Hd);
-    gemm(gate, f32(w->ffn_down_w), attn_out, rows, Hd, E);
-    add_launch(resid1, attn_out, rows_out, rows * E);
+    probe.n = (uint32_t)Hd;
+    if (matmul_takes_norm(probe)) { /* RMSNorm, up, gate and SwiGLU in one pass */
+        gemm(resid1, f32(w->ffn_up_w), gate, rows, E, Hd, nullptr, f32(w->ffn_gate_w), f32(w->norm2_weight));
+    } else if (matmul_takes_gated(probe)) {
+        rmsnorm_launch(resid1, f32(w->norm2_weight), normed, rows, E);
+        gemm(normed, f32(w->ffn_up_w), gate, rows, E, Hd, nullptr, f32(w->ffn_gate_w)); /* up, gate, SwiGLU */
+    } else {
+        rmsnorm_launch(resid1, f32(w->norm2_weight), normed, rows, E);
+        gemm(normed, f32(w->ffn_up_w), up, rows, E, Hd);
+        gemm(normed, f32(w->ffn_gate_w), gate, rows, E, Hd);
+        swiglu_launch(gate, up, gate, rows * Hd);
+    }
+    gemm(gate, f32(w->ffn_down_w), rows_out, rows, Hd, E, resid1); /* projection + residual */
     HIP_CHECK_LAUNCH("blt_kv_decode_layer");
 }

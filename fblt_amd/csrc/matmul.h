@@ -15,6 +15,13 @@
 struct MatmulArgs {
     const float *a;
     const float *b;
+    const float *b2;       /* optional second weight matrix [k, n] (same ldb): out = silu(a*b2) .* (a*b), the gated
+                              feed-forward activation (csrc/ops/elementwise_cpu.c:86-99) in one pass          */
+    const float *residual; /* optional [m, n] (leading dimension ldo) added to the result                     */
+    const float *norm_w;   /* optional [k]: the rows of a are RMS-normalised with this weight first, i.e. the
+                              product is taken of blt_rmsnorm_forward(a, norm_w) (csrc/ops/reductions_cpu.c:
+                              327-352) without materialising it; the row statistic is accumulated from the
+                              same loads (fp32 tolerance: the scale is applied after the product)              */
     float *out;
     const float *rope_cos;
     const float *rope_sin;
@@ -24,5 +31,9 @@ struct MatmulArgs {
 };
 
 void matmul_f32_launch(const MatmulArgs &g, hipStream_t s);
+/* b2 is only implemented by the kernels for small outputs; false = run the two products and the activation apart */
+bool matmul_takes_gated(const MatmulArgs &g);
+/* norm_w likewise */
+bool matmul_takes_norm(const MatmulArgs &g);
 
 #endif

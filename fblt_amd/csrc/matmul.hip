@@ -47,6 +47,38 @@ constexpr int TM = 64, TN = 64, TK = 32;
 constexpr int A_PITCH = TK + 4; /* floats per LDS row of the a tile: 16-byte fragment reads of 32 rows hit all banks */
 constexpr int B_PITCH = TN + 4;
 
+__device__ __forceinline__ float silu_times(float gate, float up) {
+    const float silu = gate / (1.0f + expf(-gate));
+    return silu * up;
+}
+
+/* Four consecutive results of output row `row` starting at column `col`:
+ * optional rotation, optional residual, store with bounds. */
+template <bool ROPE>
+__device__ __forceinline__ void store4(const MatmulArgs &g, uint32_t row, uint32_t col, float4 v, bool vec_ok) {
+    if (ROPE && col < g.rope_cols) {
+        /* columns col..col+3 are pairs (col % head_dim)/2 and the next one of the row's position */
+        const size_t at = (size_t)row * (g.head_dim / 2u) + (col % g.head_dim) / 2u;
+        v = rope_rotate4(v, g.rope_cos + at, g.rope_sin + at);
+    }
+    float *orow = g.out + (size_t)row * g.ldo;
+    const float *rrow = g.residual ? g.residual + (size_t)row * g.ldo : nullptr;
+    if (vec_ok) {
+        if (col < g.n) {
+            if (rrow) {
+                const float4 r = *reinterpret_cast<const float4 *>(rrow + col);
+                v.x = r.x + v.x, v.y = r.y + v.y, v.z = r.z + v.z, v.w = r.w + v.w;
+            }
+            *reinterpret_cast<float4 *>(orow + col) = v;
+        }
+    } else {
+        const float e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (col + i < g.n) orow[col + i] = rrow ? rrow[col + i] + e[i] : e[i];
+    }
+}
+
 /* VEC: a, b 16-byte aligned with lda, ldb, K, N multiples of 4, so a 16-byte
  * piece is either entirely inside or entirely outside the matrices.
  * ROPE: rotate pairs of the first g.rope_cols columns in the epilogue. */
@@ -134,32 +166,19 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_kernel(MatmulArgs g) {
     /* lane (h, c) holds out[row0 + 32*wr + c][col0 + 32*wc + 8*q + 4*h + 0..3] in acc[4q..4q+3] */
     const uint32_t row = row0 + wr * 32u + c;
     if (row >= g.m) return;
-    float *orow = g.out + (size_t)row * g.ldo;
-    const bool vst = VEC && (g.ldo % 4u == 0u) && ((reinterpret_cast<uintptr_t>(g.out) & 15u) == 0u);
+    const bool vst = VEC && (g.ldo % 4u == 0u) && ((reinterpret_cast<uintptr_t>(g.out) & 15u) == 0u) &&
+                     ((reinterpret_cast<uintptr_t>(g.residual) & 15u) == 0u);
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const uint32_t col = col0 + wc * 32u + 8u * q + 4u * h;
-        float4 v = make_float4(acc[4 * q + 0], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
-        if (ROPE && col < g.rope_cols) {
-            /* columns col..col+3 are pairs (col % head_dim)/2 and the next one of the row's position */
-            const size_t at = (size_t)row * (g.head_dim / 2u) + (col % g.head_dim) / 2u;
-            v = rope_rotate4(v, g.rope_cos + at, g.rope_sin + at);
-        }
-        if (vst) {
-            if (col < g.n) *reinterpret_cast<float4 *>(orow + col) = v;
-        } else {
-            if (col + 0 < g.n) orow[col + 0] = v.x;
-            if (col + 1 < g.n) orow[col + 1] = v.y;
-            if (col + 2 < g.n) orow[col + 2] = v.z;
-            if (col + 3 < g.n) orow[col + 3] = v.w;
-        }
-    }
+    for (int q = 0; q < 4; q++)
+        store4<ROPE>(g, row, col0 + wc * 32u + 8u * q + 4u * h,
+                     make_float4(acc[4 * q + 0], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]), vst);
 }
 
 /* 32x32 output tile per workgroup, K split over the four waves. */
-template <bool VEC, bool ROPE>
+template <bool VEC, bool ROPE, bool GATED>
 __global__ __launch_bounds__(256, 2) void matmul_splitk_kernel(MatmulArgs g) {
-    __shared__ float part[4][16][64];
+    __shared__ float part[GATED ? 8 : 4][16][64];
+    __shared__ float part_ss[4][32];
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
@@ -167,9 +186,11 @@ __global__ __launch_bounds__(256, 2) void matmul_splitk_kernel(MatmulArgs g) {
     const uint32_t row = blockIdx.y * 32u + c, col = blockIdx.x * 32u + c;
     const float *arow = g.a + (size_t)min(row, g.m - 1u) * g.lda;
     const float *bcol = g.b + min(col, g.n - 1u);
+    const float *b2col = GATED ? g.b2 + min(col, g.n - 1u) : nullptr;
 
+    float ss = 0.f; /* this lane's share of sum_k a[row][k]^2 (norm_w only) */
     /* fragments of one 32-wide K chunk: lane (h, c) holds a[row][k0 + 16h + t] and b[k0 + 16h + t][col] */
-    auto fetch = [&](uint32_t k0, float (&fa)[16], float (&fb)[16]) __attribute__((always_inline)) {
+    auto fetch = [&](uint32_t k0, float (&fa)[16], float (&fb)[16], float (&fg)[16]) __attribute__((always_inline)) {
         const uint32_t kb = k0 + 16u * h;
         if (VEC) {
 #pragma unroll
@@ -182,110 +203,175 @@ __global__ __launch_bounds__(256, 2) void matmul_splitk_kernel(MatmulArgs g) {
 #pragma unroll
             for (int t = 0; t < 16; t++) fa[t] = kb + t < g.k ? arow[kb + t] : 0.f;
         }
+        if (g.norm_w) { /* uniform: sum of squares of the raw row, then the norm weight folded into a */
+#pragma unroll
+            for (int t = 0; t < 16; t++) {
+                ss += fa[t] * fa[t];
+                fa[t] *= kb + t < g.k ? g.norm_w[kb + t] : 0.f;
+            }
+        }
 #pragma unroll
         for (int t = 0; t < 16; t++) fb[t] = kb + t < g.k ? bcol[(size_t)(kb + t) * g.ldb] : 0.f;
+        if (GATED) {
+#pragma unroll
+            for (int t = 0; t < 16; t++) fg[t] = kb + t < g.k ? b2col[(size_t)(kb + t) * g.ldb] : 0.f;
+        }
     };
 
-    floatx16 acc;
+    floatx16 acc, acc2;
 #pragma unroll
-    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    for (int r = 0; r < 16; r++) acc[r] = 0.f, acc2[r] = 0.f;
     const uint32_t chunks = (g.k + 31u) / 32u;
-    float fa[16], fb[16];
+    float fa[16], fb[16], fg[GATED ? 16 : 1];
+    float dummy[GATED ? 1 : 16]; /* stands in for the gate fragment when there is none */
+    (void)dummy;
     uint32_t ch = wave;
-    if (ch < chunks) fetch(ch * 32u, fa, fb);
+    if (ch < chunks) {
+        if constexpr (GATED) fetch(ch * 32u, fa, fb, fg);
+        else fetch(ch * 32u, fa, fb, dummy);
+    }
     while (ch < chunks) {
         const uint32_t nx = ch + 4u;
-        float na[16], nb[16];
-        if (nx < chunks) fetch(nx * 32u, na, nb);
+        float na[16], nb[16], ng[GATED ? 16 : 1];
+        if (nx < chunks) {
+            if constexpr (GATED) fetch(nx * 32u, na, nb, ng);
+            else fetch(nx * 32u, na, nb, dummy);
+        }
 #pragma unroll
-        for (int t = 0; t < 16; t++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[t], fa[t], acc, 0, 0, 0);
+        for (int t = 0; t < 16; t++) {
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[t], fa[t], acc, 0, 0, 0);
+            if (GATED) acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(fg[t], fa[t], acc2, 0, 0, 0);
+        }
 #pragma unroll
-        for (int t = 0; t < 16; t++) fa[t] = na[t], fb[t] = nb[t];
+        for (int t = 0; t < 16; t++) {
+            fa[t] = na[t], fb[t] = nb[t];
+            if (GATED) fg[t] = ng[t];
+        }
         ch = nx;
     }
 
 #pragma unroll
-    for (int r = 0; r < 16; r++) part[wave][r][lane] = acc[r];
+    for (int r = 0; r < 16; r++) {
+        part[wave][r][lane] = acc[r];
+        if (GATED) part[4 + wave][r][lane] = acc2[r];
+    }
+    if (g.norm_w) {
+        ss += __shfl_xor(ss, 32, 64);
+        if (h == 0) part_ss[wave][c] = ss;
+    }
     __syncthreads();
+    float row_scale = 1.0f;
+    if (g.norm_w) {
+        const float tot = (part_ss[0][c] + part_ss[1][c]) + (part_ss[2][c] + part_ss[3][c]);
+        row_scale = 1.0f / sqrtf(tot / (float)g.k + 1e-6f); /* reductions_cpu.c:345-346 */
+    }
     /* wave w finishes register group w: out[row][col0 + 8w + 4h + 0..3] */
     float v4[4];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
-        v4[i] = (part[0][4 * wave + i][lane] + part[1][4 * wave + i][lane]) +
-                (part[2][4 * wave + i][lane] + part[3][4 * wave + i][lane]);
+    for (int i = 0; i < 4; i++) {
+        v4[i] = ((part[0][4 * wave + i][lane] + part[1][4 * wave + i][lane]) +
+                 (part[2][4 * wave + i][lane] + part[3][4 * wave + i][lane])) * row_scale;
+        if (GATED) {
+            const float gate = ((part[4][4 * wave + i][lane] + part[5][4 * wave + i][lane]) +
+                                (part[6][4 * wave + i][lane] + part[7][4 * wave + i][lane])) * row_scale;
+            v4[i] = silu_times(gate, v4[i]);
+        }
+    }
     if (row >= g.m) return;
-    const uint32_t oc = blockIdx.x * 32u + 8u * wave + 4u * h;
-    float4 v = make_float4(v4[0], v4[1], v4[2], v4[3]);
-    if (ROPE && oc < g.rope_cols) {
-        const size_t at = (size_t)row * (g.head_dim / 2u) + (oc % g.head_dim) / 2u;
-        v = rope_rotate4(v, g.rope_cos + at, g.rope_sin + at);
-    }
-    float *orow = g.out + (size_t)row * g.ldo;
-    if (VEC && (g.ldo % 4u == 0u) && ((reinterpret_cast<uintptr_t>(g.out) & 15u) == 0u)) {
-        if (oc < g.n) *reinterpret_cast<float4 *>(orow + oc) = v;
-    } else {
-        if (oc + 0 < g.n) orow[oc + 0] = v.x;
-        if (oc + 1 < g.n) orow[oc + 1] = v.y;
-        if (oc + 2 < g.n) orow[oc + 2] = v.z;
-        if (oc + 3 < g.n) orow[oc + 3] = v.w;
-    }
+    const bool vst = VEC && (g.ldo % 4u == 0u) && ((reinterpret_cast<uintptr_t>(g.out) & 15u) == 0u) &&
+                     ((reinterpret_cast<uintptr_t>(g.residual) & 15u) == 0u);
+    store4<ROPE>(g, row, blockIdx.x * 32u + 8u * wave + 4u * h, make_float4(v4[0], v4[1], v4[2], v4[3]), vst);
 }
 
 /* R rows of a per thread, one output column per thread. */
-template <int R>
+template <int R, bool GATED>
 __global__ __launch_bounds__(256) void matmul_skinny_kernel(MatmulArgs g) {
 #pragma clang fp contract(off) /* product and sum rounded separately, as the reference's loop */
     const uint32_t j = blockIdx.x * 256u + threadIdx.x;
     const uint32_t r0 = blockIdx.y * R;
     if (j >= g.n) return;
-    float acc[R];
+    float acc[R], acc2[R];
 #pragma unroll
-    for (int r = 0; r < R; r++) acc[r] = 0.0f;
+    for (int r = 0; r < R; r++) acc[r] = 0.0f, acc2[r] = 0.0f;
     for (uint32_t k = 0; k < g.k; k++) {
         const float bj = g.b[(size_t)k * g.ldb + j];
+        const float gj = GATED ? g.b2[(size_t)k * g.ldb + j] : 0.0f;
 #pragma unroll
         for (int r = 0; r < R; r++) {
             const uint32_t row = min(r0 + r, g.m - 1u);
-            acc[r] = acc[r] + g.a[(size_t)row * g.lda + k] * bj;
+            const float av = g.a[(size_t)row * g.lda + k];
+            acc[r] = acc[r] + av * bj;
+            if (GATED) acc2[r] = acc2[r] + av * gj;
         }
     }
 #pragma unroll
-    for (int r = 0; r < R; r++)
-        if (r0 + r < g.m) g.out[(size_t)(r0 + r) * g.ldo + j] = acc[r];
+    for (int r = 0; r < R; r++) {
+        if (r0 + r >= g.m) continue;
+        float v = GATED ? silu_times(acc2[r], acc[r]) : acc[r];
+        if (g.residual) v = g.residual[(size_t)(r0 + r) * g.ldo + j] + v;
+        g.out[(size_t)(r0 + r) * g.ldo + j] = v;
+    }
 }
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 } // namespace
 
+namespace {
+
+enum Path { PATH_SKINNY, PATH_SPLITK, PATH_MFMA };
+
+Path choose_path(const MatmulArgs &g) {
+    const bool rope = g.rope_cos != nullptr && g.rope_cols > 0;
+    if (g.m <= 32u && !rope) return PATH_SKINNY;
+    /* fewer 64x64 tiles than half the compute units: quarter tiles, K split over the waves */
+    if ((uint64_t)((g.n + TN - 1) / TN) * ((g.m + TM - 1) / TM) < 128u) return PATH_SPLITK;
+    return PATH_MFMA;
+}
+
+template <bool VEC, bool ROPE>
+void launch_splitk(const MatmulArgs &g, dim3 grid, hipStream_t s) {
+    if (g.b2) blt_launch("matmul_splitk", matmul_splitk_kernel<VEC, ROPE, true>, grid, dim3(256), 0, s, g);
+    else blt_launch("matmul_splitk", matmul_splitk_kernel<VEC, ROPE, false>, grid, dim3(256), 0, s, g);
+}
+
+} // namespace
+
+bool matmul_takes_gated(const MatmulArgs &g) { return choose_path(g) != PATH_MFMA; }
+bool matmul_takes_norm(const MatmulArgs &g) { return choose_path(g) == PATH_SPLITK; }
+
 void matmul_f32_launch(const MatmulArgs &g, hipStream_t s) {
     if (g.m == 0 || g.n == 0) return;
     const bool rope = g.rope_cos != nullptr && g.rope_cols > 0;
-    if (g.m <= 32u && !rope) {
-        const dim3 block(256);
+    const Path path = choose_path(g);
+    BLT_REQUIRE(g.b2 == nullptr || path != PATH_MFMA, "matmul: the gated product is not available for this shape");
+    BLT_REQUIRE(g.norm_w == nullptr || path == PATH_SPLITK, "matmul: the fused row norm is not available for this shape");
+    const dim3 block(256);
+    if (path == PATH_SKINNY) {
+        const dim3 g4((g.n + 255u) / 256u, 1), g8((g.n + 255u) / 256u, (g.m + 7u) / 8u);
         if (g.m <= 4u) {
-            blt_launch("matmul_skinny", matmul_skinny_kernel<4>, dim3((g.n + 255u) / 256u, 1), block, 0, s, g);
+            if (g.b2) blt_launch("matmul_skinny", matmul_skinny_kernel<4, true>, g4, block, 0, s, g);
+            else blt_launch("matmul_skinny", matmul_skinny_kernel<4, false>, g4, block, 0, s, g);
         } else {
-            blt_launch("matmul_skinny", matmul_skinny_kernel<8>, dim3((g.n + 255u) / 256u, (g.m + 7u) / 8u), block, 0,
-                       s, g);
+            if (g.b2) blt_launch("matmul_skinny", matmul_skinny_kernel<8, true>, g8, block, 0, s, g);
+            else blt_launch("matmul_skinny", matmul_skinny_kernel<8, false>, g8, block, 0, s, g);
         }
         return;
     }
-    const dim3 grid((g.n + TN - 1) / TN, (g.m + TM - 1) / TM), block(256);
     const bool vec = aligned16(g.a) && aligned16(g.b) && g.lda % 4u == 0 && g.ldb % 4u == 0 && g.k % 4u == 0 &&
                      g.n % 4u == 0;
-    if ((uint64_t)grid.x * grid.y < 128u) {
-        /* fewer 64x64 tiles than half the compute units: quarter tiles, K split over the waves */
+    if (path == PATH_SPLITK) {
         const dim3 sgrid((g.n + 31u) / 32u, (g.m + 31u) / 32u);
         if (rope) {
-            if (vec) blt_launch("matmul_splitk", matmul_splitk_kernel<true, true>, sgrid, block, 0, s, g);
-            else blt_launch("matmul_splitk", matmul_splitk_kernel<false, true>, sgrid, block, 0, s, g);
+            if (vec) launch_splitk<true, true>(g, sgrid, s);
+            else launch_splitk<false, true>(g, sgrid, s);
         } else {
-            if (vec) blt_launch("matmul_splitk", matmul_splitk_kernel<true, false>, sgrid, block, 0, s, g);
-            else blt_launch("matmul_splitk", matmul_splitk_kernel<false, false>, sgrid, block, 0, s, g);
+            if (vec) launch_splitk<true, false>(g, sgrid, s);
+            else launch_splitk<false, false>(g, sgrid, s);
         }
         return;
     }
+    const dim3 grid((g.n + TN - 1) / TN, (g.m + TM - 1) / TM);
     if (rope) {
         if (vec) blt_launch("matmul_mfma", matmul_mfma_kernel<true, true>, grid, block, 0, s, g);
         else blt_launch("matmul_mfma", matmul_mfma_kernel<false, true>, grid, block, 0, s, g);

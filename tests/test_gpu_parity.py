@@ -724,4 +724,5 @@ def test_kv_decode_layer(batch, n, H, hd, hidden, kind, oracle, dev):
                                         qkv.data_ptr() + 8 * E, 3 * E, tcos.data_ptr(), tsin.data_ptr(), max_len,
                                         comb.data_ptr(), E, n, step_kind, 0, int(lens.max()) + n)
         lib.blt_backend_pass_sync_hip()
-        assert tck2.cpu().numpy().tobytes() == got_k.tobytes()
+        # the layer folds the norm into the projection (scale applied after the product): tolerance, not bits
+        assert_close(got_k, tck2.cpu().numpy(), "cache k (block)")
