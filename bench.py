@@ -304,6 +304,39 @@ def bench_decode_layer(steps, warmup, batch=64, H=4, hd=32, hidden=512, len_hi=5
     return res
 
 
+def cpu_decode_layer(budget_s, batch=64, H=4, hd=32, hidden=512, len_hi=512):
+    """The restated decoder layer on one host core, one sequence at a time as the reference runs it."""
+    import numpy as np
+    from fblt_amd import synth
+    from oracle import binding
+    lib = binding.load_oracle()
+    E, half = H * hd, hd // 2
+    max_len = len_hi + 64
+    rs = np.random.RandomState(5)
+    lens = synth.integers(synth.seed_for(4, synth.S_LEN), batch, 1, len_hi)
+    ck, cv = rs.randn(batch * max_len, E).astype(np.float32), rs.randn(batch * max_len, E).astype(np.float32)
+    W = {k: (rs.randn(*shape) / np.sqrt(shape[0])).astype(np.float32) for k, shape in
+         dict(qkv=(E, 3 * E), proj=(E, E), up=(E, hidden), gate=(E, hidden), down=(hidden, E)).items()}
+    ones = np.ones(E, dtype=np.float32)
+    cos, sin = np.empty(max_len * half, dtype=np.float32), np.empty(max_len * half, dtype=np.float32)
+    lib.orc_rope_precompute(max_len, 500000.0, hd, binding.fptr(cos), binding.fptr(sin))
+    x, o = rs.randn(batch, E).astype(np.float32), np.zeros((batch, E), dtype=np.float32)
+    fp = lambda a: binding.fptr(a.reshape(-1))
+    steps, spent = 0, 0.0
+    while steps < 1 or (spent < budget_s and steps < 32):
+        t0 = time.perf_counter()
+        for b in range(batch):
+            rc = lib.orc_kv_decode_layer(fp(ck), fp(cv), max_len, E, H, b, int(lens[b]) + steps, 1, 0, fp(ones),
+                                         fp(W["qkv"]), fp(W["proj"]), fp(ones), fp(W["up"]), fp(W["gate"]),
+                                         fp(W["down"]), hidden, fp(cos), fp(sin), max_len, fp(x[b:b + 1]),
+                                         fp(o[b:b + 1]))
+            assert rc == 0
+        spent += time.perf_counter() - t0
+        steps += 1
+    return {"value": spent / steps * 1e6, "unit": "us/step", "cores": 1, "kind": "port",
+            "sample": "%d layer steps of %d sequences, %.1f s" % (steps, batch, spent)}
+
+
 def cpu_dense(w, budget_s):
     """Checker on one host core over the same workload; repeated whole passes up to the budget."""
     from oracle import binding, runner as orunner
@@ -449,6 +482,8 @@ def main():
                                                      gemm_only=(8192, 512, 1536))
         log("matmul", json.dumps(others["matmul_8192x512x1536"]))
         others["decode_layer"] = bench_decode_layer(K, W)
+        if not args.no_cpu:
+            others["decode_layer"]["cpu_baseline"] = cpu_decode_layer(2.0)
         log("decode_layer", json.dumps(others["decode_layer"]))
 
     cpu_head = None

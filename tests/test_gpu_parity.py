@@ -644,7 +644,8 @@ def test_row_ops(oracle, dev):
 
 
 @pytest.mark.parametrize("batch,n,H,hd,hidden,kind", [(3, 1, 2, 32, 96, "causal"), (64, 1, 4, 32, 256, "causal"),
-                                                      (5, 6, 2, 64, 200, "causal"), (9, 16, 4, 32, 128, "block")])
+                                                      (5, 6, 2, 64, 200, "causal"), (9, 16, 4, 32, 128, "block"),
+                                                      (128, 16, 4, 32, 512, "causal")])
 def test_kv_decode_layer(batch, n, H, hd, hidden, kind, oracle, dev):
     """blt_kv_decode_layer_hip for all sequences at once against the restated layer run per sequence."""
     import torch
