@@ -265,12 +265,12 @@ def bench_decode_layer(steps, warmup, batch=64, H=4, hd=32, hidden=512, len_hi=5
     arena = lib.blt_arena_create(64 << 20, abi.BLT_BACKEND_HIP)
     hint0 = int(lens.max())
 
-    def run(count, first):
+    def run(count, first, commit=1):
         for s in range(count):
             arena.contents.offset = 0
             lib.blt_kv_decode_layer_hip(C.byref(c), C.byref(w), x.data_ptr(), o.data_ptr(), cos.data_ptr(),
-                                        sin.data_ptr(), max_len, 1, api.BLT_KV_STEP_CAUSAL, 1, hint0 + first + s + 1,
-                                        arena)
+                                        sin.data_ptr(), max_len, 1, api.BLT_KV_STEP_CAUSAL, commit,
+                                        hint0 + first + s + 1, arena)
     run(warmup, 0)
     lib.blt_backend_pass_sync_hip()
     lib.blt_hip_profile_begin()
@@ -287,6 +287,28 @@ def bench_decode_layer(steps, warmup, batch=64, H=4, hd=32, hidden=512, len_hi=5
     run(steps, warmup)
     lib.blt_backend_pass_sync_hip()
     wall_plain = time.perf_counter() - t0
+    # the same layer step recorded once into a HIP graph (no commit: a replay repeats the step at
+    # the lengths reached above) against the same step issued eagerly
+    lib.blt_backend_pass_sync_hip()
+    t0 = time.perf_counter()
+    run(steps, warmup + steps - 1, commit=0)
+    lib.blt_backend_pass_sync_hip()
+    wall_eager_fixed = time.perf_counter() - t0
+    per_graph = 6   # as many layer steps per graph as a 6-layer decoder issues per token
+    lib.blt_hip_capture_begin()
+    for _ in range(per_graph):
+        run(1, warmup + steps - 1, commit=0)
+    graph = lib.blt_hip_capture_end()
+    for _ in range(warmup):
+        lib.blt_hip_graph_launch(graph)
+    lib.blt_backend_pass_sync_hip()
+    replays = max(1, steps // per_graph)
+    t0 = time.perf_counter()
+    for _ in range(replays):
+        lib.blt_hip_graph_launch(graph)
+    lib.blt_backend_pass_sync_hip()
+    wall_graph = (time.perf_counter() - t0) * steps / (replays * per_graph)
+    lib.blt_hip_graph_destroy(graph)
     lib.blt_arena_destroy(arena)
     avg_s = sum(v[1] for v in prof.values()) / 1e3 / steps
     mean_keys = float(lens.astype("int64").sum()) + batch * (warmup + (steps - 1) / 2.0) + batch
@@ -295,6 +317,8 @@ def bench_decode_layer(steps, warmup, batch=64, H=4, hd=32, hidden=512, len_hi=5
     res = {"workload": "decoder layer step: %d sequences, E=%d, H=%d, hidden=%d, cached 1..%d" % (batch, E, H, hidden, len_hi),
            "kernel": "+".join(sorted(prof)), "launches_per_step": sum(v[0] for v in prof.values()) / steps,
            "tokens_per_step": batch, "us_per_step": wall_plain / steps * 1e6,
+           "us_per_step_fixed_length_eager": wall_eager_fixed / steps * 1e6,
+           "us_per_step_fixed_length_graph_replay": wall_graph / steps * 1e6,   # 6 layer steps (30 kernels) per graph
            "us_per_step_with_events": wall / steps * 1e6, "kernel_us_avg": avg_s * 1e6,
            "kernel_us_min": min(v[2] for v in prof.values()) * 1e3,
            "per_kernel_us": {k: v[1] * 1e3 / steps for k, v in prof.items()},

@@ -127,6 +127,12 @@ SYMBOLS = {
     "blt_kv_decode_layer_hip": (None, [C.POINTER(BltKvAttnCache), C.POINTER(abi.BltTransformerWeights), C.c_void_p,
                                        C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_int, C.c_int,
                                        C.c_size_t, C.POINTER(abi.BltArena)]),
+    "blt_hip_set_stream": (None, [C.c_void_p]),
+    "blt_hip_get_stream": (C.c_void_p, []),
+    "blt_hip_capture_begin": (None, []),
+    "blt_hip_capture_end": (C.c_void_p, []),
+    "blt_hip_graph_launch": (None, [C.c_void_p]),
+    "blt_hip_graph_destroy": (None, [C.c_void_p]),
     "blt_hip_profile_begin": (None, []),
     "blt_hip_profile_end": (C.c_size_t, [C.POINTER(BltHipKernelTime), C.c_size_t]),
     "blt_hip_stream_copy_probe": (None, [C.c_void_p, C.c_void_p, C.c_size_t]),

@@ -16,7 +16,7 @@ LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(LIBDIR, "obj")
 LIB = os.path.join(LIBDIR, "libfblt_hip.so")
 
-HIP_SOURCES = ["memory.hip", "mask_builder.hip", "vecmath.hip", "attn_rows.hip", "attn_mfma.hip", "attn_wide.hip", "matmul.hip", "rope.hip", "mha.hip", "layer_ops.hip", "probes.hip",
+HIP_SOURCES = ["memory.hip", "mask_builder.hip", "vecmath.hip", "attn_rows.hip", "attn_mfma.hip", "attn_wide.hip", "matmul.hip", "rope.hip", "mha.hip", "layer_ops.hip", "probes.hip", "stream.hip",
                "attn_decode.hip", "attn_verify.hip", "attn_api.hip", "profile.hip"]
 C_SOURCES = ["host/blt_host.c"]
 

@@ -8,6 +8,7 @@
 #include "blt_fatal.h"
 #include "hip_check.h"
 #include "attn_launch.h"
+#include "launch.h"
 
 #include <algorithm>
 #include <cstdlib>
@@ -326,6 +327,9 @@ struct Staging {
         const size_t tbytes = plan.tiles.size() * sizeof(AttnTile);
         const size_t need = pbytes + tbytes;
         if (need == 0) return;
+        BLT_REQUIRE(!blt_stream_capturing(),
+                    "blt_attention_batch: this batch stages its descriptors through host memory, which a graph "
+                    "cannot replay; use a resident plan (blt_attention_plan_*) or a strided batch under capture");
         if (!copied) HIP_CHECK(hipEventCreateWithFlags(&copied, hipEventDisableTiming));
         if (in_flight) {
             HIP_CHECK(hipEventSynchronize(copied));
@@ -343,8 +347,8 @@ struct Staging {
         }
         std::memcpy(pinned, plan.host.data(), pbytes);
         if (tbytes) std::memcpy(static_cast<char *>(pinned) + pbytes, plan.tiles.data(), tbytes);
-        HIP_CHECK(hipMemcpyAsync(device, pinned, need, hipMemcpyHostToDevice, 0));
-        HIP_CHECK(hipEventRecord(copied, 0));
+        HIP_CHECK(hipMemcpyAsync(device, pinned, need, hipMemcpyHostToDevice, blt_stream()));
+        HIP_CHECK(hipEventRecord(copied, blt_stream()));
         in_flight = true;
         plan_launch(plan, static_cast<const AttnProb *>(device),
                     reinterpret_cast<const AttnTile *>(static_cast<const char *>(device) + pbytes));

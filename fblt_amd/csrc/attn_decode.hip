@@ -376,6 +376,9 @@ void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_s
 
     Scratch &sc = scratch();
     const size_t need = cache->batch * (size_t)MAX_SPLITS * H * 32u * (hd + 2); /* 32 = widest query block */
+    BLT_REQUIRE(!blt_stream_capturing() || (need <= sc.partial_floats && cache->batch <= sc.ticket_count),
+                "blt_kv_attend_step: the step would allocate its scratch while a graph capture is open; run it once "
+                "eagerly with this batch size first");
     if (need > sc.partial_floats) {
         if (sc.partial) {
             HIP_CHECK(hipDeviceSynchronize());
@@ -391,7 +394,7 @@ void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_s
         }
         sc.ticket_count = std::max<size_t>(cache->batch, 1024);
         HIP_CHECK(hipMalloc((void **)&sc.tickets, sc.ticket_count * sizeof(uint32_t)));
-        HIP_CHECK(hipMemsetAsync(sc.tickets, 0, sc.ticket_count * sizeof(uint32_t), 0));
+        HIP_CHECK(hipMemsetAsync(sc.tickets, 0, sc.ticket_count * sizeof(uint32_t), blt_stream()));
     }
     a.partial = sc.partial;
     a.tickets = sc.tickets;

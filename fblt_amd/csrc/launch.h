@@ -3,6 +3,7 @@
  * hipLaunchKernelGGL normally; while a profile is open, the same launch with
  * a start and a stop event attached to the dispatch, so that the kernel's own
  * begin/end timestamps can be read back per launch and summed per kernel tag.
+ * A stream argument of 0 means the calling thread's current stream.
  */
 #ifndef FBLT_AMD_LAUNCH_H
 #define FBLT_AMD_LAUNCH_H
@@ -13,12 +14,17 @@
 #include "hip_check.h"
 
 bool blt_profile_is_open();
+/* The calling thread's current stream (null stream by default) and whether a
+ * graph capture is open on it (stream.hip). */
+hipStream_t blt_stream();
+bool blt_stream_capturing();
 /* A fresh (start, stop) event pair owned by the open profile, booked under `tag`. */
 void blt_profile_book(const char *tag, hipEvent_t *start, hipEvent_t *stop);
 
 template <typename Kernel, typename... Args>
 inline void blt_launch(const char *tag, Kernel kernel, dim3 grid, dim3 block, size_t lds_bytes, hipStream_t stream,
                        Args... args) {
+    if (!stream) stream = blt_stream(); /* callers pass 0 for "the library's current stream" */
     if (blt_profile_is_open()) {
         hipEvent_t e0, e1;
         blt_profile_book(tag, &e0, &e1);

@@ -11,6 +11,7 @@
 #include "blt_hip.h"
 #include "blt_fatal.h"
 #include "hip_check.h"
+#include "launch.h"
 
 #include <stdint.h>
 #include <stdlib.h>
@@ -160,11 +161,11 @@ extern "C" void blt_build_attention_mask_hip(const blt_mask_config *config, blt_
     uint32_t *dead = row_ok + nq;
     blt_hip_memset(row_ok, 0, (nq + 1) * sizeof(uint32_t));
 
-    hipLaunchKernelGGL(attention_mask_kernel, mask_grid(nq, nk), dim3(256), 0, 0,
+    hipLaunchKernelGGL(attention_mask_kernel, mask_grid(nq, nk), dim3(256), 0, blt_stream(),
                        static_cast<float *>(out_mask->data), r, row_ok);
     HIP_CHECK_LAUNCH("blt_build_attention_mask");
     const unsigned cblocks = (unsigned)((nq + 255u) / 256u < 1024u ? (nq + 255u) / 256u : 1024u);
-    hipLaunchKernelGGL(count_dead_rows_kernel, dim3(cblocks), dim3(256), 0, 0, row_ok, (uint64_t)nq, dead);
+    hipLaunchKernelGGL(count_dead_rows_kernel, dim3(cblocks), dim3(256), 0, blt_stream(), row_ok, (uint64_t)nq, dead);
     HIP_CHECK_LAUNCH("blt_build_attention_mask row check");
 
     /* The staged id vectors (dq, dk) must outlive the asynchronous copies:
@@ -205,7 +206,7 @@ extern "C" void blt_build_block_diffusion_mask_hip(const blt_block_diffusion_con
     r.infer = train ? 0 : 1;
     r.starts = train ? stage_u64(config->block_starts, config->num_blocks, arena) : nullptr;
 
-    hipLaunchKernelGGL(block_diffusion_mask_kernel, mask_grid(S, S), dim3(256), 0, 0,
+    hipLaunchKernelGGL(block_diffusion_mask_kernel, mask_grid(S, S), dim3(256), 0, blt_stream(),
                        static_cast<float *>(out_mask->data), r);
     HIP_CHECK_LAUNCH("blt_build_block_diffusion_mask");
     /* Row i always sees column min(i, N-1) or itself, so no row can be empty

@@ -2,11 +2,13 @@
  * Device-memory shim of the HIP backend: the functions the reference's core
  * calls for device arenas and tensor transfers (reference contract:
  * csrc/core/cuda_shim.h:18-31; behaviour: csrc/ops/memory.cu:37-77).  Memset
- * and host-to-device copies are asynchronous on the null stream; the
+ * and host-to-device copies are asynchronous on the library's current stream
+ * (the null stream unless blt_hip_set_stream chose another); the
  * device-to-host copy blocks and is the implicit synchronisation point.
  */
 #include "blt_hip.h"
 #include "hip_check.h"
+#include "launch.h"
 
 extern "C" void *blt_hip_malloc(size_t bytes) {
     void *p = nullptr;
@@ -22,17 +24,19 @@ extern "C" void blt_hip_free(void *ptr) {
 
 extern "C" void blt_hip_memset(void *dst, int value, size_t bytes) {
     if (bytes == 0) return;
-    HIP_CHECK(hipMemsetAsync(dst, value, bytes, 0));
+    HIP_CHECK(hipMemsetAsync(dst, value, bytes, blt_stream()));
 }
 
 extern "C" void blt_hip_memcpy_h2d(void *dst, const void *src, size_t bytes) {
     if (bytes == 0) return;
-    HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, 0));
+    HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, blt_stream()));
 }
 
 extern "C" void blt_hip_memcpy_d2h(void *dst, const void *src, size_t bytes) {
     if (bytes == 0) return;
-    HIP_CHECK(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+    /* the copy waits for the library's current stream, whichever it is */
+    HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, blt_stream()));
+    HIP_CHECK(hipStreamSynchronize(blt_stream()));
 }
 
 extern "C" void blt_backend_pass_sync_hip(void) {
@@ -52,7 +56,7 @@ __global__ __launch_bounds__(256) void stream_copy_kernel(float4 *__restrict__ d
 extern "C" void blt_hip_stream_copy_probe(void *dst, const void *src, size_t bytes) {
     BLT_REQUIRE(dst != NULL && src != NULL && bytes % 16 == 0, "blt_hip_stream_copy_probe: need 16-byte multiples");
     if (bytes == 0) return;
-    hipLaunchKernelGGL(stream_copy_kernel, dim3(2048), dim3(256), 0, 0, static_cast<float4 *>(dst),
+    hipLaunchKernelGGL(stream_copy_kernel, dim3(2048), dim3(256), 0, blt_stream(), static_cast<float4 *>(dst),
                        static_cast<const float4 *>(src), bytes / 16);
     HIP_CHECK_LAUNCH("blt_hip_stream_copy_probe");
 }

@@ -6,6 +6,7 @@
 #include "blt_hip.h"
 #include "blt_fatal.h"
 #include "hip_check.h"
+#include "launch.h"
 
 #include <stdint.h>
 
@@ -102,10 +103,10 @@ extern "C" void blt_strided_copy_hip(blt_backend backend, float *dst, size_t dst
     const uint64_t work = rows * (vec ? cols / 4 : cols);
     const unsigned blocks = (unsigned)((work + 255u) / 256u < 4096u ? (work + 255u) / 256u : 4096u);
     if (vec)
-        hipLaunchKernelGGL(strided_copy_kernel<true>, dim3(blocks), dim3(256), 0, 0, dst, (uint64_t)dst_stride, src,
+        hipLaunchKernelGGL(strided_copy_kernel<true>, dim3(blocks), dim3(256), 0, blt_stream(), dst, (uint64_t)dst_stride, src,
                            (uint64_t)src_stride, (uint64_t)rows, (uint64_t)cols);
     else
-        hipLaunchKernelGGL(strided_copy_kernel<false>, dim3(blocks), dim3(256), 0, 0, dst, (uint64_t)dst_stride, src,
+        hipLaunchKernelGGL(strided_copy_kernel<false>, dim3(blocks), dim3(256), 0, blt_stream(), dst, (uint64_t)dst_stride, src,
                            (uint64_t)src_stride, (uint64_t)rows, (uint64_t)cols);
     HIP_CHECK_LAUNCH("blt_strided_copy");
 }
@@ -116,7 +117,7 @@ extern "C" void blt_softmax_masked_row_inplace_hip(blt_backend backend, float *r
                 "blt_softmax_masked_row_inplace: HIP implementation called with non-HIP backend");
     if (row_len == 0) return;
     BLT_REQUIRE(row != NULL, "blt_softmax_masked_row_inplace: row must not be NULL");
-    hipLaunchKernelGGL(softmax_row_kernel, dim3(1), dim3(256), 0, 0, row, (uint64_t)row_len, (uint64_t)row_idx,
+    hipLaunchKernelGGL(softmax_row_kernel, dim3(1), dim3(256), 0, blt_stream(), row, (uint64_t)row_len, (uint64_t)row_idx,
                        is_causal ? 1 : 0, mask_row, scale);
     HIP_CHECK_LAUNCH("blt_softmax_masked_row_inplace");
 }
@@ -127,9 +128,10 @@ extern "C" float blt_vec_dot_hip(blt_backend backend, const float *a, const floa
     BLT_REQUIRE(a != NULL && b != NULL, "blt_vec_dot: buffers must not be NULL");
     static thread_local float *slot = nullptr;
     if (!slot) HIP_CHECK(hipMalloc((void **)&slot, sizeof(float)));
-    hipLaunchKernelGGL(dot_kernel, dim3(1), dim3(256), 0, 0, a, b, (uint64_t)n, slot);
+    hipLaunchKernelGGL(dot_kernel, dim3(1), dim3(256), 0, blt_stream(), a, b, (uint64_t)n, slot);
     HIP_CHECK_LAUNCH("blt_vec_dot");
     float r = 0.f;
-    HIP_CHECK(hipMemcpy(&r, slot, sizeof(float), hipMemcpyDeviceToHost));
+    HIP_CHECK(hipMemcpyAsync(&r, slot, sizeof(float), hipMemcpyDeviceToHost, blt_stream()));
+    HIP_CHECK(hipStreamSynchronize(blt_stream()));
     return r;
 }

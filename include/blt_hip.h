@@ -282,6 +282,27 @@ void blt_kv_decode_layer_hip(const blt_kv_attn_cache *cache, const blt_transform
                              size_t rope_positions, size_t n, int step_kind, int commit, size_t max_len_hint,
                              blt_arena *arena);
 
+/* The stream every launch, asynchronous copy and memset of the library goes
+ * to, per calling thread: the null stream (the reference's behaviour) unless
+ * set otherwise.  `stream` is a hipStream_t. */
+void blt_hip_set_stream(void *stream);
+void *blt_hip_get_stream(void);
+
+/* Record the library calls issued between begin and end into a HIP graph
+ * instead of running them (the calls go to a library-owned stream under
+ * hipStreamBeginCapture), and replay them with one graph launch on the
+ * current stream: for launch-bound loops such as a decode step of several
+ * small kernels.  Calls that would allocate device memory or stage
+ * descriptors through host memory during a capture end with a message: run
+ * each call once eagerly first; use resident plans or strided batches for
+ * attention.  A replay repeats the recorded launches with the recorded
+ * arguments (pointers, lengths hints); data behind the pointers is read anew. */
+typedef struct blt_hip_graph blt_hip_graph;
+void blt_hip_capture_begin(void);
+blt_hip_graph *blt_hip_capture_end(void);
+void blt_hip_graph_launch(const blt_hip_graph *graph);
+void blt_hip_graph_destroy(blt_hip_graph *graph);
+
 /* Per-kernel device time of every launch the library issues between begin and
  * end, from HIP events attached to each dispatch (the kernel's own begin/end
  * timestamps, without launch gaps).  `end` synchronises the device, fills up to
