@@ -53,6 +53,21 @@ def roofline(bound, work, avg_s, traffic=None):
             "traffic": traffic}
 
 
+def step_percentiles(lib, api, one_step, count):
+    """Device time of `count` further steps, one profile per step (kernel durations of the
+    step's launches summed; each step ends with a device sync): mean / p50 / p90 / p99 in us."""
+    import numpy as np
+    samples = []
+    for s in range(count):
+        lib.blt_hip_profile_begin()
+        one_step(s)
+        samples.append(sum(v[1] for v in api.profile_end().values()) * 1e3)
+    a = np.sort(np.array(samples))
+    pick = lambda q: float(a[min(len(a) - 1, int(q * len(a)))])
+    return {"n": len(a), "mean": float(a.mean()), "p50": pick(0.50), "p90": pick(0.90), "p99": pick(0.99),
+            "min": float(a[0]), "max": float(a[-1])}
+
+
 def time_plan(lib, api, plan, steps, warmup):
     """(wall seconds for `steps` launches, {tag: (launches, total_ms, min, max)})."""
     for _ in range(warmup):
@@ -82,6 +97,7 @@ def bench_dense(make, steps, warmup, bound, mask_mode="descriptor"):
         lib.blt_attention_plan_run_hip(plan)
     lib.blt_backend_pass_sync_hip()
     wall_plain = time.perf_counter() - t0
+    pct = step_percentiles(lib, api, lambda s_: lib.blt_attention_plan_run_hip(plan), min(steps, 256))
     lib.blt_attention_plan_destroy_hip(plan)
     d.close()
     launches = sum(v[0] for v in prof.values())
@@ -92,6 +108,7 @@ def bench_dense(make, steps, warmup, bound, mask_mode="descriptor"):
         "tokens_per_step": w.tokens, "ms_per_step": wall_plain / steps * 1e3,
         "ms_per_step_with_events": wall / steps * 1e3,
         "kernel_us_avg": avg_s * 1e6, "kernel_us_min": min(v[2] for v in prof.values()) * 1e3,
+        "kernel_us_percentiles": pct,
         "tokens_per_s": w.tokens * steps / wall_plain,
         "tokens_per_s_kernel": w.tokens / avg_s,
         "flops": w.flops, "bytes": w.bytes,
@@ -127,6 +144,11 @@ def bench_kv(kw, steps, warmup):
 
     wall, prof = one_pass(True)
     wall_plain, _ = one_pass(False)
+    d.reset()
+    for s in range(warmup):
+        d.step(idx(s))
+    lib.blt_backend_pass_sync_hip()
+    pct = step_percentiles(lib, api, lambda s_: d.step(idx(warmup + s_)), min(steps, 256))
     kern_ms = sum(v[1] for v in prof.values())
     launches = sum(v[0] for v in prof.values())
     avg_s = kern_ms / 1e3 / steps
@@ -143,7 +165,7 @@ def bench_kv(kw, steps, warmup):
         "workload": kw.name, "kernel": "kv_step", "launches_per_step": launches / steps,
         "tokens_per_step": kw.tokens, "us_per_step": wall_plain / steps * 1e6,
         "us_per_step_with_events": wall / steps * 1e6, "kernel_us_avg": avg_s * 1e6,
-        "kernel_us_min": min(v[2] for v in prof.values()) * 1e3,
+        "kernel_us_min": min(v[2] for v in prof.values()) * 1e3, "kernel_us_percentiles": pct,
         "tokens_per_s": kw.tokens * steps / wall_plain, "tokens_per_s_kernel": kw.tokens / avg_s,
         "flops": flops_step, "bytes": bytes_step,
         "roofline_hbm": roofline("hbm", bytes_step, avg_s, MEASURED_TRAFFIC_BYTES.get(kw.name)),
@@ -533,6 +555,7 @@ def main():
                    "entry": "blt_attention_plan_run_hip, causal descriptor, one launch per step",
                    "kernel": head["kernel"], "tokens_per_step": head["tokens_per_step"]},
         "kernel_us_avg": head["kernel_us_avg"],
+        "kernel_us_percentiles": head["kernel_us_percentiles"],
         "roofline": head["roofline"],
         "roofline_mfma": head["roofline_mfma"],
         "cpu_baseline": cpu_head,
