@@ -3,10 +3,11 @@
  * cores of gfx950 (v_mfma_f32_32x32x2_f32), for prefill and block shapes.
  *
  * Work item = one tile of 32 query rows of one (sequence, head) problem, run
- * by a workgroup of four wavefronts.  The four waves split the tile's key
- * tiles (32 keys each) round-robin, each keeps its own running (max, sum,
- * output) and they merge once through LDS at the end, so the serial chain per
- * wave is a quarter of the row's key tiles.
+ * by a workgroup of four wavefronts (eight when the launch has fewer
+ * workgroups than half the compute units and the head dim is 32).  The waves
+ * split the tile's key tiles (32 keys each) round-robin, each keeps its own
+ * running (max, sum, output) and they merge once through LDS at the end, so
+ * the serial chain per wave is a quarter (an eighth) of the row's key tiles.
  *
  * Both contractions are computed TRANSPOSED so that no operand ever has to be
  * re-laid-out between them:
@@ -136,28 +137,32 @@ __device__ __forceinline__ void frag_from_lds(float (&dst)[HD / 2], const float 
  * 4-float pad per row: a lane's 16-byte fragment reads (row = lane % 32) then
  * fall on distinct banks for every 16 lanes.  The output merge reuses the K
  * area once the key loop is over. */
-template <int HD, bool STAGE>
+template <int HD, bool STAGE, int NW>
 struct MfmaLds {
     static constexpr int ROW = HD + 4;
     static constexpr int Q_FLOATS = STAGE ? 32 * ROW : 0;
-    static constexpr int K_FLOATS = STAGE ? 4 * 32 * ROW : 0;
+    static constexpr int K_FLOATS = STAGE ? NW * 32 * ROW : 0;
     static constexpr int MERGE_FLOATS = 3 * HD * 33;
     static constexpr int BODY_FLOATS = K_FLOATS > MERGE_FLOATS ? K_FLOATS : MERGE_FLOATS;
 };
 
-template <int HD, int SRC, bool EXACT, bool DENSE>
-__global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_mfma_kernel(const AttnProb *__restrict__ probs,
-                                                        const AttnTile *__restrict__ tiles, AttnAffine aff) {
+/* NW = wavefronts per workgroup: 4, or 8 for launches with too few workgroups
+ * to occupy the chip (each wave's serial chain of key tiles halves). */
+template <int HD, int SRC, bool EXACT, bool DENSE, int NW>
+__global__ __launch_bounds__(64 * NW, HD <= 64 ? 2 : 1) void attn_mfma_kernel(const AttnProb *__restrict__ probs,
+                                                                            const AttnTile *__restrict__ tiles,
+                                                                            AttnAffine aff) {
+    constexpr uint32_t NT = 64u * NW; /* threads */
     constexpr int HALF = HD / 2;
     constexpr int DB = HD / 32; /* 32-wide blocks of the head dim */
     /* K and Q tiles go through LDS (coalesced global reads, transposing LDS
      * reads) whenever they fit the 64 KB a workgroup may declare statically */
     constexpr bool STAGE = HD <= 64;
-    using Lds = MfmaLds<HD, STAGE>;
+    using Lds = MfmaLds<HD, STAGE, NW>;
     constexpr int ROW = Lds::ROW;
 
-    __shared__ float sm_m[4][32];
-    __shared__ float sm_l[4][32];
+    __shared__ float sm_m[NW][32];
+    __shared__ float sm_l[NW][32];
     __shared__ __attribute__((aligned(16))) float sm_q[Lds::Q_FLOATS > 0 ? Lds::Q_FLOATS : 4];
     __shared__ __attribute__((aligned(16))) float sm_body[Lds::BODY_FLOATS];
     uint32_t qtile;
@@ -237,12 +242,12 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_mfma_kernel(const 
     float vf[DB][16];
 
     if (STAGE) {
-        /* the query tile is shared by the four waves: each brings a quarter */
+        /* the query tile is shared by the waves: each brings its share */
         if (EXACT) {
-            constexpr int QPT = 32 * LPR / 256 > 0 ? 32 * LPR / 256 : 1; /* float4 per thread */
+            constexpr int QPT = 32 * LPR / NT > 0 ? 32 * LPR / NT : 1; /* float4 per thread */
 #pragma unroll
             for (int t = 0; t < QPT; t++) {
-                const uint32_t e = threadIdx.x + 256u * t;
+                const uint32_t e = threadIdx.x + NT * t;
                 if (e < 32u * LPR) {
                     const uint32_t r = e / LPR, f4 = e % LPR;
                     const uint32_t qi = min(q0 + r, p.nq - 1u);
@@ -251,7 +256,7 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_mfma_kernel(const 
                 }
             }
         } else {
-            tile_to_lds_slow<HD>(sm_q, p.q, p.q_stride, q0, p.nq, p.hd, threadIdx.x, 256u);
+            tile_to_lds_slow<HD>(sm_q, p.q, p.q_stride, q0, p.nq, p.hd, threadIdx.x, NT);
         }
     } else {
         load_half_row<HALF, EXACT>(qf, p.q + (size_t)i * p.q_stride, h * HALF, p.hd, vec4);
@@ -298,7 +303,7 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_mfma_kernel(const 
     }
     while (kt < kt_hi) {
         const uint32_t k0 = kt * 32u;
-        const uint32_t ktn = kt + 4u;
+        const uint32_t ktn = kt + NW;
 
         if (STAGE) {
             frag_from_lds<HD>(kf, my_k, h, c);
@@ -366,7 +371,8 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_mfma_kernel(const 
      * wave parks its partial O^T and merges a quarter of the columns for all
      * 32 rows, reading the four partials from LDS in its own fragment layout.
      * Otherwise wave 0 merges the other three into its registers. */
-    constexpr bool QUARTER = 4 * HD * 33 <= Lds::BODY_FLOATS;
+    constexpr bool QUARTER = NW * HD * 33 <= Lds::BODY_FLOATS;
+    static_assert(QUARTER || NW == 4, "the single-merger path is written for four waves");
     float(*sm_o)[HD][33] = reinterpret_cast<float(*)[HD][33]>(sm_body);
     if (STAGE) __syncthreads();
     if (h == 0) {
@@ -385,28 +391,30 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_mfma_kernel(const 
     float M = neg_inf(), L = 0.f;
     if (QUARTER || wave == 0) {
 #pragma unroll
-        for (int w = 0; w < 4; w++) M = fmaxf(M, sm_m[w][c]);
+        for (int w = 0; w < NW; w++) M = fmaxf(M, sm_m[w][c]);
         const float Ms = M == neg_inf() ? 0.f : M;
-        float f[4];
+        float f[NW];
 #pragma unroll
-        for (int w = 0; w < 4; w++) {
+        for (int w = 0; w < NW; w++) {
             f[w] = fast_exp2(sm_m[w][c] - Ms);
             L += sm_l[w][c] * f[w];
         }
         const float inv = L > 0.f ? 1.0f / L : 0.f;
         float *orow = p.out + (size_t)i * p.out_stride;
         if (QUARTER) {
-            /* DB * 4 groups of four consecutive columns; this wave takes DB of them */
+            /* DB * 4 groups of four consecutive columns, shared out over the waves */
+            constexpr int GPW = DB * 4 / NW > 0 ? DB * 4 / NW : 1;
 #pragma unroll
-            for (int k = 0; k < DB; k++) {
-                const uint32_t gid = wave * DB + k;
+            for (int k = 0; k < GPW; k++) {
+                const uint32_t gid = wave * GPW + k;
+                if (gid >= (uint32_t)(DB * 4)) break; /* more waves than groups */
                 const uint32_t d0 = (gid >> 2) * 32u + 8u * (gid & 3u) + 4u * h;
                 float o4[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     float acc = 0.f;
 #pragma unroll
-                    for (int w = 0; w < 4; w++) acc += sm_o[w][d0 + e][c] * f[w];
+                    for (int w = 0; w < NW; w++) acc += sm_o[w][d0 + e][c] * f[w];
                     o4[e] = acc * inv;
                 }
                 if (live) {
@@ -469,7 +477,7 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_mfma_kernel(const 
     float *wrow = p.weights + (size_t)i * p.nk;
     const bool wvec = (p.nk % 4u == 0u) && ((reinterpret_cast<uintptr_t>(p.weights) & 15u) == 0u);
     const uint32_t nkt = (p.nk + 31u) / 32u;
-    for (uint32_t wt = wave; wt < nkt; wt += 4u) {
+    for (uint32_t wt = wave; wt < nkt; wt += NW) {
         const uint32_t k0 = wt * 32u;
         float w[16];
 #pragma unroll
@@ -519,15 +527,28 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_mfma_kernel(const 
 template <int HD, int SRC>
 void launch_variant(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t nblocks, const AttnAffine &aff,
                     bool exact, bool dense, hipStream_t s) {
-    const dim3 grid(nblocks), block(256);
+    const dim3 grid(nblocks);
+    if constexpr (HD == 32) {
+        /* fewer workgroups than half the compute units: eight waves each (their K tiles fit LDS at this head dim) */
+        if (exact && nblocks < 128u) {
+            if (dense)
+                blt_launch("attn_mfma", attn_mfma_kernel<HD, SRC, true, true, 8>, grid, dim3(512), 0, s, dprobs, dtiles,
+                           aff);
+            else
+                blt_launch("attn_mfma", attn_mfma_kernel<HD, SRC, true, false, 8>, grid, dim3(512), 0, s, dprobs,
+                           dtiles, aff);
+            return;
+        }
+    }
+    const dim3 block(256);
     if (exact && dense)
-        blt_launch("attn_mfma", attn_mfma_kernel<HD, SRC, true, true>, grid, block, 0, s, dprobs, dtiles, aff);
+        blt_launch("attn_mfma", attn_mfma_kernel<HD, SRC, true, true, 4>, grid, block, 0, s, dprobs, dtiles, aff);
     else if (exact)
-        blt_launch("attn_mfma", attn_mfma_kernel<HD, SRC, true, false>, grid, block, 0, s, dprobs, dtiles, aff);
+        blt_launch("attn_mfma", attn_mfma_kernel<HD, SRC, true, false, 4>, grid, block, 0, s, dprobs, dtiles, aff);
     else if (dense)
-        blt_launch("attn_mfma", attn_mfma_kernel<HD, SRC, false, true>, grid, block, 0, s, dprobs, dtiles, aff);
+        blt_launch("attn_mfma", attn_mfma_kernel<HD, SRC, false, true, 4>, grid, block, 0, s, dprobs, dtiles, aff);
     else
-        blt_launch("attn_mfma", attn_mfma_kernel<HD, SRC, false, false>, grid, block, 0, s, dprobs, dtiles, aff);
+        blt_launch("attn_mfma", attn_mfma_kernel<HD, SRC, false, false, 4>, grid, block, 0, s, dprobs, dtiles, aff);
 }
 
 template <int SRC>
