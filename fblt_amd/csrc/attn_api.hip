@@ -125,17 +125,20 @@ Family choose_family(const AttnProb &d) {
     return FAM_ROWS;
 }
 
-/* The wide kernel pays off once its 128-row work items fill the chip a few
- * times over; below that the latency-oriented mfma kernel, which splits the
- * keys of a 32-row tile over four waves, finishes first.
+/* The wide kernel pays off once its 128-row work items give every compute
+ * unit one (short rows: few key tiles per item) or two (long rows: the
+ * latency-oriented mfma kernel, which splits the keys of a 32-row tile over
+ * its waves, keeps the shorter serial chain for longer) -- measured
+ * crossovers: 128..256 items at 128 keys, 256..512 items at 512 keys.
  * BLT_HIP_WIDE_MIN_GROUPS overrides the threshold. */
-uint32_t wide_min_groups() {
-    static const uint32_t cached = [] {
+uint32_t wide_min_groups(uint32_t max_nk) {
+    static const uint32_t pinned = [] {
         const char *e = getenv("BLT_HIP_WIDE_MIN_GROUPS");
         const long v = e ? std::atol(e) : 0;
-        return v > 0 ? (uint32_t)v : 1024u;
+        return v > 0 ? (uint32_t)v : 0u;
     }();
-    return cached;
+    if (pinned) return pinned;
+    return max_nk <= 256u ? 256u : 512u;
 }
 
 /* Do problems p[0..n), all routed to the mfma family, go to the wide kernel instead? */
@@ -143,11 +146,13 @@ bool choose_wide(const AttnProb *p, uint32_t n) {
     const int forced = family_override();
     if (forced == 1 || forced == 2) return false;
     uint64_t groups = 0;
+    uint32_t max_nk = 0;
     for (uint32_t i = 0; i < n; i++) {
         if (!attn_wide_can(p[i])) return false;
         groups += attn_wide_groups(p[i]);
+        max_nk = std::max(max_nk, p[i].nk);
     }
-    return forced == 3 || groups >= wide_min_groups();
+    return forced == 3 || groups >= wide_min_groups(max_nk);
 }
 
 /* Element distance between two float pointers (either both NULL or both set). */
