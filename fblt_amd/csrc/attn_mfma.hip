@@ -3,8 +3,8 @@
  * cores of gfx950 (v_mfma_f32_32x32x2_f32), for prefill and block shapes.
  *
  * Work item = one tile of 32 query rows of one (sequence, head) problem, run
- * by a workgroup of four wavefronts (eight when the launch has fewer
- * workgroups than half the compute units and the head dim is 32).  The waves
+ * by a workgroup of four wavefronts (eight when the launch has about as
+ * many workgroups as compute units or fewer, and the head dim is 32).  The waves
  * split the tile's key tiles (32 keys each) round-robin, each keeps its own
  * running (max, sum, output) and they merge once through LDS at the end, so
  * the serial chain per wave is a quarter (an eighth) of the row's key tiles.
@@ -41,6 +41,7 @@
 #include "launch.h"
 
 #include <algorithm>
+#include <cstdlib>
 
 namespace {
 
@@ -529,8 +530,13 @@ void launch_variant(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t nbl
                     bool exact, bool dense, hipStream_t s) {
     const dim3 grid(nblocks);
     if constexpr (HD == 32) {
-        /* fewer workgroups than half the compute units: eight waves each (their K tiles fit LDS at this head dim) */
-        if (exact && nblocks < 128u) {
+        /* fewer workgroups than the compute units can spread: eight waves each (their K tiles fit
+         * LDS at this head dim).  BLT_HIP_MFMA_WAVES8_BELOW overrides the workgroup count (tuning hook). */
+        static const uint32_t below = [] {
+            const char *e = getenv("BLT_HIP_MFMA_WAVES8_BELOW");
+            return e && *e ? (uint32_t)atoi(e) : 320u; /* measured: ahead up to 256 workgroups, level at 512 */
+        }();
+        if (exact && nblocks < below) {
             if (dense)
                 blt_launch("attn_mfma", attn_mfma_kernel<HD, SRC, true, true, 8>, grid, dim3(512), 0, s, dprobs, dtiles,
                            aff);
