@@ -175,9 +175,10 @@ def bench_kv(kw, steps, warmup):
     return res, kw
 
 
-def bench_block(name, T, E, H, steps, warmup, gemm_only=None):
+def bench_block(name, T, E, H, steps, warmup, gemm_only=None, cross=None):
     """blt_multihead_attention (projection, rotation, all heads, projection) on random
-    device tensors, or with gemm_only=(m, k, n) one blt_matmul of that shape."""
+    device tensors; with gemm_only=(m, k, n) one blt_matmul of that shape; with cross=P
+    blt_cross_attention_forward of P patches over T bytes (T / P bytes per patch)."""
     import ctypes as C
     import numpy as np
     import torch
@@ -193,6 +194,28 @@ def bench_block(name, T, E, H, steps, warmup, gemm_only=None):
         va, vb, vo = view(a), view(b), view(o)
         run = lambda: lib.blt_matmul(C.byref(va), C.byref(vb), C.byref(vo))
         flops, nbytes, tokens = 2.0 * m * k * n, 4.0 * (m * k + k * n + m * n), m
+    elif cross:
+        P = cross
+        xq, xkv, o = rnd(P, E).cuda(), rnd(T, E).cuda(), torch.zeros((P, E), device="cuda")
+        ws = [(rnd(E, E) / E ** 0.5).cuda() for _ in range(4)]
+        arena = lib.blt_arena_create(256 << 20, abi.BLT_BACKEND_HIP)
+        mc = abi.BltMaskConfig()
+        mc.seq_len_q, mc.seq_len_kv = P, T
+        qg, kg = abi.size_array(list(range(P))), abi.size_array([i // (T // P) for i in range(T)])
+        mc.query_group_ids, mc.kv_group_ids, mc.bidirectional_within_group = qg, kg, True
+        vws = [view(w) for w in ws]
+        wts = abi.BltCrossAttentionWeights(*(C.pointer(v) for v in vws))
+        cc = abi.BltCrossAttentionConfig()
+        cc.embed_dim, cc.num_heads, cc.head_dim, cc.mask_config = E, H, E // H, C.pointer(mc)
+        vq, vkv, vo = view(xq), view(xkv), view(o)
+        keep += [mc, qg, kg, vws, wts, ws]
+
+        def run():
+            arena.contents.offset = 0
+            lib.blt_cross_attention_forward(C.byref(vq), C.byref(vkv), C.byref(wts), C.byref(vo), C.byref(cc), arena)
+        flops = 2.0 * E * E * (2 * P + 2 * T) + 4.0 * (E // H) * H * T
+        nbytes = 4.0 * (P * E + T * E + 4 * E * E + P * E)
+        tokens = T
     else:
         hd = E // H
         x, wq, wp = rnd(T, E).cuda(), (rnd(E, 3 * E) / E ** 0.5).cuda(), (rnd(E, E) / E ** 0.5).cuda()
@@ -522,6 +545,9 @@ def main():
     if want("block"):
         others["mha_c1"] = bench_block("blt_multihead_attention T=512 E=128 H=4 rope causal", 512, 128, 4, K, W)
         log("mha_c1", json.dumps(others["mha_c1"]))
+        others["xattn_c3"] = bench_block("blt_cross_attention_forward P=128 T=512 E=128 H=4 patch mask", 512, 128, 4,
+                                         K, W, cross=128)
+        log("xattn_c3", json.dumps(others["xattn_c3"]))
         others["mha_c2"] = bench_block("blt_multihead_attention T=128 E=512 H=8 rope causal", 128, 512, 8, K, W)
         log("mha_c2", json.dumps(others["mha_c2"]))
         others["matmul_8192x512x1536"] = bench_block("blt_matmul 8192x512x1536", 0, 0, 0, max(10, K // 10), 3,

@@ -109,6 +109,22 @@ class BltAttentionConfig(C.Structure):
     ]
 
 
+class BltCrossAttentionConfig(C.Structure):
+    """csrc/models/cross_attention.h:27-34"""
+    _fields_ = [
+        ("embed_dim", C.c_size_t),
+        ("patch_dim", C.c_size_t),
+        ("split_mode", C.c_int),
+        ("num_heads", C.c_size_t),
+        ("head_dim", C.c_size_t),
+        ("mask_config", C.POINTER(BltMaskConfig)),
+    ]
+
+
+class BltCrossAttentionWeights(C.Structure):
+    _fields_ = [(n, C.POINTER(BltTensor)) for n in ("weight_q", "weight_k", "weight_v", "weight_proj")]
+
+
 class BltTransformerWeights(C.Structure):
     _fields_ = [(n, C.POINTER(BltTensor)) for n in ("norm1_weight", "norm1_bias", "attn_qkv_w", "attn_proj_w",
                                                     "norm2_weight", "norm2_bias", "ffn_up_w", "ffn_gate_w",
@@ -138,6 +154,8 @@ def check_layout():
     assert C.sizeof(BltAttentionConfig) == 56 and BltAttentionConfig.rope_theta.offset == 28
     assert BltAttentionConfig.mask_config.offset == 48
     assert C.sizeof(BltTransformerWeights) == 72
+    assert C.sizeof(BltCrossAttentionConfig) == 48 and BltCrossAttentionConfig.num_heads.offset == 24
+    assert C.sizeof(BltCrossAttentionWeights) == 32
 
 
 def tensor_view(ptr, shape, backend, dtype=BLT_DTYPE_FP32):

@@ -127,6 +127,12 @@ SYMBOLS = {
     "blt_kv_decode_layer_hip": (None, [C.POINTER(BltKvAttnCache), C.POINTER(abi.BltTransformerWeights), C.c_void_p,
                                        C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_int, C.c_int,
                                        C.c_size_t, C.POINTER(abi.BltArena)]),
+    "blt_cross_attention_forward_hip": (None, [C.POINTER(abi.BltTensor), C.POINTER(abi.BltTensor),
+                                               C.POINTER(abi.BltCrossAttentionWeights), C.POINTER(abi.BltTensor),
+                                               C.POINTER(abi.BltCrossAttentionConfig), C.POINTER(abi.BltArena)]),
+    "blt_cross_attention_forward": (None, [C.POINTER(abi.BltTensor), C.POINTER(abi.BltTensor),
+                                           C.POINTER(abi.BltCrossAttentionWeights), C.POINTER(abi.BltTensor),
+                                           C.POINTER(abi.BltCrossAttentionConfig), C.POINTER(abi.BltArena)]),
     "blt_hip_set_stream": (None, [C.c_void_p]),
     "blt_hip_get_stream": (C.c_void_p, []),
     "blt_hip_capture_begin": (None, []),

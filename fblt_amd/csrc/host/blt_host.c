@@ -159,6 +159,14 @@ void blt_softmax_masked_row_inplace(blt_backend backend, float *row, size_t row_
     blt_softmax_masked_row_inplace_hip(backend, row, row_len, row_idx, is_causal, mask_row, scale);
 }
 
+void blt_cross_attention_forward(const blt_tensor *query_in, const blt_tensor *kv_in,
+                                 const blt_cross_attention_weights *weights, blt_tensor *output,
+                                 const blt_cross_attention_config *config, blt_arena *arena) {
+    BLT_REQUIRE(query_in != NULL, "blt_cross_attention: query_in must be [num_patches, embed_dim] FP32");
+    BLT_DEVICE_ONLY(query_in->backend, "blt_cross_attention_forward");
+    blt_cross_attention_forward_hip(query_in, kv_in, weights, output, config, arena);
+}
+
 void blt_add(const blt_tensor *a, const blt_tensor *b, blt_tensor *out) {
     BLT_REQUIRE(a != NULL, "blt_add: input tensors must be FP32 with matching element count");
     BLT_DEVICE_ONLY(a->backend, "blt_add");

@@ -18,6 +18,10 @@ bool blt_profile_is_open();
  * graph capture is open on it (stream.hip). */
 hipStream_t blt_stream();
 bool blt_stream_capturing();
+/* Host-to-device copy that returns at once and lets the caller reuse `src`
+ * right away: the bytes go through a small ring of pinned buffers owned by
+ * the calling thread (memory.hip).  Not usable while a graph is captured. */
+void blt_upload_staged(void *dst, const void *src, size_t bytes);
 /* A fresh (start, stop) event pair owned by the open profile, booked under `tag`. */
 void blt_profile_book(const char *tag, hipEvent_t *start, hipEvent_t *stop);
 

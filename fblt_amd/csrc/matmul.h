@@ -17,6 +17,7 @@ struct MatmulArgs {
     const float *b;
     const float *b2;       /* optional second weight matrix [k, n] (same ldb): out = silu(a*b2) .* (a*b), the gated
                               feed-forward activation (csrc/ops/elementwise_cpu.c:86-99) in one pass          */
+    float *out2;           /* with b2: store a*b2 here (same ldo) instead of gating the first product with it  */
     const float *residual; /* optional [m, n] (leading dimension ldo) added to the result                     */
     const float *norm_w;   /* optional [k]: the rows of a are RMS-normalised with this weight first, i.e. the
                               product is taken of blt_rmsnorm_forward(a, norm_w) (csrc/ops/reductions_cpu.c:
@@ -31,6 +32,9 @@ struct MatmulArgs {
 };
 
 void matmul_f32_launch(const MatmulArgs &g, hipStream_t s);
+/* g0 (plain) and g1 (two weight matrices, two outputs) in one launch; only when matmul_pair_ok says so */
+bool matmul_pair_ok(const MatmulArgs &g0, const MatmulArgs &g1);
+void matmul_f32_launch_pair(const MatmulArgs &g0, const MatmulArgs &g1, hipStream_t s);
 /* b2 is only implemented by the kernels for small outputs; false = run the two products and the activation apart */
 bool matmul_takes_gated(const MatmulArgs &g);
 /* norm_w likewise */

@@ -174,16 +174,14 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_kernel(MatmulArgs g) {
                      make_float4(acc[4 * q + 0], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]), vst);
 }
 
-/* 32x32 output tile per workgroup, K split over the four waves. */
+/* 32x32 output tile (bx, by) per workgroup, K split over the four waves. */
 template <bool VEC, bool ROPE, bool GATED>
-__global__ __launch_bounds__(256, 2) void matmul_splitk_kernel(MatmulArgs g) {
-    __shared__ float part[GATED ? 8 : 4][16][64];
-    __shared__ float part_ss[4][32];
-
+__device__ __forceinline__ void splitk_tile(const MatmulArgs &g, const uint32_t bx, const uint32_t by,
+                                            float (*part)[16][64], float (*part_ss)[32]) {
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
     const uint32_t h = lane >> 5, c = lane & 31u;
-    const uint32_t row = blockIdx.y * 32u + c, col = blockIdx.x * 32u + c;
+    const uint32_t row = by * 32u + c, col = bx * 32u + c;
     const float *arow = g.a + (size_t)min(row, g.m - 1u) * g.lda;
     const float *bcol = g.b + min(col, g.n - 1u);
     const float *b2col = GATED ? g.b2 + min(col, g.n - 1u) : nullptr;
@@ -266,7 +264,7 @@ __global__ __launch_bounds__(256, 2) void matmul_splitk_kernel(MatmulArgs g) {
         row_scale = 1.0f / sqrtf(tot / (float)g.k + 1e-6f); /* reductions_cpu.c:345-346 */
     }
     /* wave w finishes register group w: out[row][col0 + 8w + 4h + 0..3] */
-    float v4[4];
+    float v4[4], second[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         v4[i] = ((part[0][4 * wave + i][lane] + part[1][4 * wave + i][lane]) +
@@ -274,13 +272,46 @@ __global__ __launch_bounds__(256, 2) void matmul_splitk_kernel(MatmulArgs g) {
         if (GATED) {
             const float gate = ((part[4][4 * wave + i][lane] + part[5][4 * wave + i][lane]) +
                                 (part[6][4 * wave + i][lane] + part[7][4 * wave + i][lane])) * row_scale;
-            v4[i] = silu_times(gate, v4[i]);
+            if (g.out2) second[i] = gate; /* two products, two outputs */
+            else v4[i] = silu_times(gate, v4[i]);
         }
     }
     if (row >= g.m) return;
     const bool vst = VEC && (g.ldo % 4u == 0u) && ((reinterpret_cast<uintptr_t>(g.out) & 15u) == 0u) &&
-                     ((reinterpret_cast<uintptr_t>(g.residual) & 15u) == 0u);
-    store4<ROPE>(g, row, blockIdx.x * 32u + 8u * wave + 4u * h, make_float4(v4[0], v4[1], v4[2], v4[3]), vst);
+                     ((reinterpret_cast<uintptr_t>(g.residual) & 15u) == 0u) &&
+                     ((reinterpret_cast<uintptr_t>(g.out2) & 15u) == 0u);
+    const uint32_t oc = bx * 32u + 8u * wave + 4u * h;
+    store4<ROPE>(g, row, oc, make_float4(v4[0], v4[1], v4[2], v4[3]), vst);
+    if (GATED && g.out2) {
+        MatmulArgs g2 = g;
+        g2.out = g.out2;
+        g2.residual = nullptr;
+        store4<false>(g2, row, oc, make_float4(second[0], second[1], second[2], second[3]), vst);
+    }
+}
+
+template <bool VEC, bool ROPE, bool GATED>
+__global__ __launch_bounds__(256, 2) void matmul_splitk_kernel(MatmulArgs g) {
+    __shared__ float part[GATED ? 8 : 4][16][64];
+    __shared__ float part_ss[4][32];
+    splitk_tile<VEC, ROPE, GATED>(g, blockIdx.x, blockIdx.y, part, part_ss);
+}
+
+/* Two independent products in one launch: the tile rows of the second are
+ * stacked under those of the first (rows0 tile rows); the second may carry a
+ * second weight matrix.  For pairs of small products whose launches would
+ * otherwise each pay the fixed launch cost. */
+template <bool VEC>
+__global__ __launch_bounds__(256, 2) void matmul_splitk_pair_kernel(MatmulArgs g0, MatmulArgs g1, uint32_t rows0) {
+    __shared__ float part[8][16][64];
+    __shared__ float part_ss[4][32];
+    if (blockIdx.y < rows0) { /* uniform per workgroup */
+        if (blockIdx.x * 32u >= g0.n) return;
+        splitk_tile<VEC, false, false>(g0, blockIdx.x, blockIdx.y, part, part_ss);
+    } else {
+        if (blockIdx.x * 32u >= g1.n) return;
+        splitk_tile<VEC, false, true>(g1, blockIdx.x, blockIdx.y - rows0, part, part_ss);
+    }
 }
 
 /* R rows of a per thread, one output column per thread. */
@@ -307,9 +338,10 @@ __global__ __launch_bounds__(256) void matmul_skinny_kernel(MatmulArgs g) {
 #pragma unroll
     for (int r = 0; r < R; r++) {
         if (r0 + r >= g.m) continue;
-        float v = GATED ? silu_times(acc2[r], acc[r]) : acc[r];
+        float v = (GATED && !g.out2) ? silu_times(acc2[r], acc[r]) : acc[r];
         if (g.residual) v = g.residual[(size_t)(r0 + r) * g.ldo + j] + v;
         g.out[(size_t)(r0 + r) * g.ldo + j] = v;
+        if (GATED && g.out2) g.out2[(size_t)(r0 + r) * g.ldo + j] = acc2[r];
     }
 }
 
@@ -340,6 +372,30 @@ void launch_splitk(const MatmulArgs &g, dim3 grid, hipStream_t s) {
 bool matmul_takes_gated(const MatmulArgs &g) { return choose_path(g) != PATH_MFMA; }
 bool matmul_takes_norm(const MatmulArgs &g) { return choose_path(g) == PATH_SPLITK; }
 
+namespace {
+bool vec_ok(const MatmulArgs &g) {
+    return aligned16(g.a) && aligned16(g.b) && g.lda % 4u == 0 && g.ldb % 4u == 0 && g.k % 4u == 0 && g.n % 4u == 0;
+}
+} // namespace
+
+bool matmul_pair_ok(const MatmulArgs &g0, const MatmulArgs &g1) {
+    const auto plain = [](const MatmulArgs &g) {
+        return g.m != 0 && g.n != 0 && g.k != 0 && g.m > 32u && choose_path(g) == PATH_SPLITK && !g.residual &&
+               !g.norm_w && !(g.rope_cos != nullptr && g.rope_cols > 0);
+    };
+    return plain(g0) && plain(g1) && g0.b2 == nullptr && g1.b2 != nullptr && g1.out2 != nullptr;
+}
+
+void matmul_f32_launch_pair(const MatmulArgs &g0, const MatmulArgs &g1, hipStream_t s) {
+    BLT_REQUIRE(matmul_pair_ok(g0, g1), "matmul: this pair of products cannot share a launch");
+    const uint32_t rows0 = (g0.m + 31u) / 32u, rows1 = (g1.m + 31u) / 32u;
+    const uint32_t cols = (std::max(g0.n, g1.n) + 31u) / 32u;
+    const dim3 grid(cols, rows0 + rows1);
+    if (vec_ok(g0) && vec_ok(g1))
+        blt_launch("matmul_splitk", matmul_splitk_pair_kernel<true>, grid, dim3(256), 0, s, g0, g1, rows0);
+    else blt_launch("matmul_splitk", matmul_splitk_pair_kernel<false>, grid, dim3(256), 0, s, g0, g1, rows0);
+}
+
 void matmul_f32_launch(const MatmulArgs &g, hipStream_t s) {
     if (g.m == 0 || g.n == 0) return;
     const bool rope = g.rope_cos != nullptr && g.rope_cols > 0;
@@ -358,8 +414,7 @@ void matmul_f32_launch(const MatmulArgs &g, hipStream_t s) {
         }
         return;
     }
-    const bool vec = aligned16(g.a) && aligned16(g.b) && g.lda % 4u == 0 && g.ldb % 4u == 0 && g.k % 4u == 0 &&
-                     g.n % 4u == 0;
+    const bool vec = vec_ok(g);
     if (path == PATH_SPLITK) {
         const dim3 sgrid((g.n + 31u) / 32u, (g.m + 31u) / 32u);
         if (rope) {

@@ -7,6 +7,7 @@
  * device-to-host copy blocks and is the implicit synchronisation point.
  */
 #include "blt_hip.h"
+#include "blt_fatal.h"
 #include "hip_check.h"
 #include "launch.h"
 
@@ -30,6 +31,45 @@ extern "C" void blt_hip_memset(void *dst, int value, size_t bytes) {
 extern "C" void blt_hip_memcpy_h2d(void *dst, const void *src, size_t bytes) {
     if (bytes == 0) return;
     HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, blt_stream()));
+}
+
+namespace {
+
+/* Ring of pinned buffers, one event each: a slot is reused only after the copy
+ * that read it has finished. */
+struct PinnedRing {
+    static constexpr int SLOTS = 8;
+    struct Slot {
+        void *host = nullptr;
+        size_t capacity = 0;
+        hipEvent_t copied = nullptr;
+        bool in_flight = false;
+    } slot[SLOTS];
+    int next = 0;
+};
+
+} // namespace
+
+void blt_upload_staged(void *dst, const void *src, size_t bytes) {
+    if (bytes == 0) return;
+    BLT_REQUIRE(!blt_stream_capturing(), "host data cannot be staged to the device while a graph is captured");
+    static thread_local PinnedRing ring;
+    PinnedRing::Slot &s = ring.slot[ring.next];
+    ring.next = (ring.next + 1) % PinnedRing::SLOTS;
+    if (!s.copied) HIP_CHECK(hipEventCreateWithFlags(&s.copied, hipEventDisableTiming));
+    if (s.in_flight) {
+        HIP_CHECK(hipEventSynchronize(s.copied));
+        s.in_flight = false;
+    }
+    if (bytes > s.capacity) {
+        if (s.host) HIP_CHECK(hipHostFree(s.host));
+        s.capacity = bytes < 4096 ? 4096 : 2 * bytes;
+        HIP_CHECK(hipHostMalloc(&s.host, s.capacity, hipHostMallocDefault));
+    }
+    __builtin_memcpy(s.host, src, bytes);
+    HIP_CHECK(hipMemcpyAsync(dst, s.host, bytes, hipMemcpyHostToDevice, blt_stream()));
+    HIP_CHECK(hipEventRecord(s.copied, blt_stream()));
+    s.in_flight = true;
 }
 
 extern "C" void blt_hip_memcpy_d2h(void *dst, const void *src, size_t bytes) {

@@ -149,6 +149,29 @@ typedef struct {
     const blt_mask_config *mask_config; /* overrides is_causal when non-NULL */
 } blt_attention_config;
 
+/* ---- cross-attention block (48 + 32 bytes), csrc/models/cross_attention.h:21-41 */
+typedef enum {
+    BLT_CROSS_ATTN_NO_SPLIT = 0,
+    BLT_CROSS_ATTN_SPLIT_QUERY,
+    BLT_CROSS_ATTN_SPLIT_KV
+} blt_cross_attention_split_mode;
+
+typedef struct {
+    size_t embed_dim;
+    size_t patch_dim;                          /* carried for the callers; the forward pass does not read it */
+    blt_cross_attention_split_mode split_mode; /* likewise */
+    size_t num_heads;
+    size_t head_dim;                           /* 0 = embed_dim / num_heads */
+    const blt_mask_config *mask_config;        /* required: block-diagonal patch mask */
+} blt_cross_attention_config;
+
+typedef struct {
+    const blt_tensor *weight_q;    /* [embed_dim, embed_dim] each */
+    const blt_tensor *weight_k;
+    const blt_tensor *weight_v;
+    const blt_tensor *weight_proj;
+} blt_cross_attention_weights;
+
 /* ---- learned weights of one transformer block (72 bytes), ------------- */
 /* csrc/models/transformer.h:42-52                                          */
 typedef struct {
@@ -181,6 +204,9 @@ BLT_ABI_ASSERT(offsetof(blt_attention_head_args, is_causal) == 128 &&
                "blt_attention_head_args tail");
 BLT_ABI_ASSERT(sizeof(blt_mask_config) == 72, "blt_mask_config layout");
 BLT_ABI_ASSERT(sizeof(blt_transformer_weights) == 72, "blt_transformer_weights layout");
+BLT_ABI_ASSERT(sizeof(blt_cross_attention_config) == 48 && offsetof(blt_cross_attention_config, num_heads) == 24,
+               "blt_cross_attention_config layout");
+BLT_ABI_ASSERT(sizeof(blt_cross_attention_weights) == 32, "blt_cross_attention_weights layout");
 BLT_ABI_ASSERT(sizeof(blt_rope_config) == 16 && offsetof(blt_rope_config, head_dim) == 8, "blt_rope_config layout");
 BLT_ABI_ASSERT(sizeof(blt_attention_config) == 56 && offsetof(blt_attention_config, rope_theta) == 28 &&
                    offsetof(blt_attention_config, mask_config) == 48,

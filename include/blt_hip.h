@@ -79,6 +79,16 @@ void blt_rope_apply_hip(const blt_tensor *x, const blt_tensor *cos, const blt_te
 void blt_rope_apply_packed_hip(float *qkv_data, size_t qkv_stride, size_t head_offset, size_t seq_len,
                                size_t head_dim, const float *cos, const float *sin);
 
+/* blt_cross_attention_forward for device tensors (csrc/models/
+ * cross_attention.c:101-157): Q projection, K and V projections in one launch
+ * (they share the input), all heads in one attention launch with the patch
+ * mask reduced to per-row key ranges on the host (blt_mask_config_row_ranges;
+ * dense device-built mask when a configuration does not reduce), output
+ * projection.  No positional embedding, no residual, as in the reference. */
+void blt_cross_attention_forward_hip(const blt_tensor *query_in, const blt_tensor *kv_in,
+                                     const blt_cross_attention_weights *weights, blt_tensor *output,
+                                     const blt_cross_attention_config *config, blt_arena *arena);
+
 /* Replace blt_rmsnorm_forward_cuda (csrc/ops/reductions.cu:390-396; CPU loop
  * reductions_cpu.c:327-352, bit-identical here), blt_add_cuda and
  * blt_swiglu_forward_cuda (csrc/ops/elementwise.cu:102-134; CPU loops
@@ -151,6 +161,10 @@ void blt_rope_apply_packed(float *qkv_data, size_t qkv_stride, size_t head_offse
                            const float *cos, const float *sin, blt_backend backend);
 void blt_multihead_attention(const blt_tensor *input, const blt_tensor *weight_qkv, const blt_tensor *weight_proj,
                              blt_tensor *output, const blt_attention_config *config, blt_arena *arena);
+/* csrc/models/cross_attention.h:49-51 */
+void blt_cross_attention_forward(const blt_tensor *query_in, const blt_tensor *kv_in,
+                                 const blt_cross_attention_weights *weights, blt_tensor *output,
+                                 const blt_cross_attention_config *config, blt_arena *arena);
 /* csrc/core/backend.c:254-256, 276-278, 380-382 */
 void blt_add(const blt_tensor *a, const blt_tensor *b, blt_tensor *out);
 void blt_swiglu_forward(const blt_tensor *gate, const blt_tensor *up, blt_tensor *out);

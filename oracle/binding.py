@@ -90,6 +90,8 @@ def load_oracle():
     lib.orc_kv_decode_layer.restype = C.c_int
     lib.orc_kv_decode_layer.argtypes = ([_fp, _fp] + [C.c_size_t] * 7 + [_fp] * 7 + [C.c_size_t, _fp, _fp, C.c_size_t,
                                                                                 _fp, _fp])
+    lib.orc_cross_attention_forward.restype = C.c_int
+    lib.orc_cross_attention_forward.argtypes = [_fp] * 7 + [C.c_size_t] * 4 + [C.POINTER(abi.BltMaskConfig)]
     lib.orc_kv_rope_attend_step.restype = C.c_int
     lib.orc_kv_rope_attend_step.argtypes = [_fp, _fp] + [C.c_size_t] * 7 + [_fp, C.c_size_t, _fp, C.c_size_t, _fp,
                                                                            C.c_size_t, _fp, _fp, C.c_size_t, _fp]
@@ -156,6 +158,9 @@ def load_ref():
     lib.blt_rope_apply_packed.argtypes = [_fp, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, _fp, _fp, C.c_int]
     lib.blt_multihead_attention.restype = None
     lib.blt_multihead_attention.argtypes = [T, T, T, T, C.POINTER(abi.BltAttentionConfig), C.POINTER(abi.BltArena)]
+    lib.blt_cross_attention_forward.restype = None
+    lib.blt_cross_attention_forward.argtypes = [T, T, C.POINTER(abi.BltCrossAttentionWeights), T,
+                                                C.POINTER(abi.BltCrossAttentionConfig), C.POINTER(abi.BltArena)]
     lib.blt_build_block_diffusion_mask.restype = None
     lib.blt_build_block_diffusion_mask.argtypes = [C.POINTER(abi.BltBlockDiffusionConfig),
                                                    C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)]

@@ -556,3 +556,45 @@ int orc_kv_decode_layer(float *self_k, float *self_v, size_t max_seq_len, size_t
     free(normed), free(qkv), free(combined), free(attn_out), free(resid1), free(up), free(gate), free(act);
     return rc;
 }
+
+/* csrc/models/cross_attention.c:101-157: Q from query_in, K and V from kv_in,
+ * dense mask from the (required) mask configuration, one core call per head
+ * with weights_out, output projection; no positional embedding, no residual. */
+int orc_cross_attention_forward(const float *query_in, const float *kv_in, const float *wq, const float *wk,
+                                const float *wv, const float *wproj, float *output, size_t num_patches,
+                                size_t seq_len, size_t embed_dim, size_t num_heads,
+                                const blt_mask_config *mask_config) {
+    if (mask_config == NULL || num_heads == 0 || embed_dim % num_heads != 0) return ORC_ERR_ARG;
+    if (mask_config->seq_len_q != num_patches || mask_config->seq_len_kv != seq_len) return ORC_ERR_ARG;
+    const size_t E = embed_dim, hd = E / num_heads;
+    float *q = (float *)malloc(num_patches * E * sizeof(float));
+    float *k = (float *)malloc(seq_len * E * sizeof(float));
+    float *v = (float *)malloc(seq_len * E * sizeof(float));
+    float *combined = (float *)calloc(num_patches * E, sizeof(float));
+    float *scores = (float *)malloc(num_patches * seq_len * sizeof(float));
+    float *mask = (float *)malloc(num_patches * seq_len * sizeof(float));
+    orc_matmul(query_in, wq, q, num_patches, E, E);
+    orc_matmul(kv_in, wk, k, seq_len, E, E);
+    orc_matmul(kv_in, wv, v, seq_len, E, E);
+    int rc = orc_build_attention_mask(mask_config, mask);
+    for (size_t h = 0; h < num_heads && rc == ORC_OK; h++) {
+        blt_attention_head_args a;
+        memset(&a, 0, sizeof(a));
+        a.q = q + h * hd, a.k = k + h * hd, a.v = v + h * hd;
+        a.q_stride = a.k_stride = a.v_stride = E;
+        a.combined = combined;
+        a.combined_stride = E;
+        a.combined_col_offset = h * hd;
+        a.weights_out = scores;
+        a.mask = mask;
+        a.nq = num_patches;
+        a.nk = seq_len;
+        a.head_dim = hd;
+        a.is_causal = false;
+        a.scale = 1.0f / sqrtf((float)hd);
+        rc = orc_attention_head_core(&a);
+    }
+    if (rc == ORC_OK) orc_matmul(combined, wproj, output, num_patches, E, E);
+    free(q), free(k), free(v), free(combined), free(scores), free(mask);
+    return rc;
+}

@@ -43,9 +43,13 @@
  *       preserved, q.k after rotation depends only on the position
  *       difference; the step against rotating by hand and calling
  *       orc_kv_attend_step.
- *   orc_matmul, orc_rope_apply_packed, orc_multihead_attention
+ *   orc_matmul, orc_rope_apply_packed, orc_multihead_attention,
+ *   orc_cross_attention_forward
  *       bit-for-bit against oracle/_ref (blt_matmul, blt_rope_apply_packed,
- *       blt_multihead_attention compiled from csrc/models/attention.c); the
+ *       blt_multihead_attention and blt_cross_attention_forward compiled from
+ *       csrc/models/attention.c and cross_attention.c; the cross block also
+ *       against the numbers and the group isolation of
+ *       tests/unit/models/unit_cross_attention.c:111-117, 229-246); the
  *       reference's vectors: [[1,2],[3,4]] x [[5,6],[7,8]] = [[19,22],[43,50]]
  *       (tests/unit/backend/unit_linalg_cpu.c:10-48) and the identity-weight
  *       two-token block -> {0.6697615, 0.3302385, ...}, causal row 0 one-hot
@@ -182,6 +186,13 @@ int orc_multihead_attention(const float *input, const float *weight_qkv, const f
                             size_t seq_len, size_t embed_dim, size_t num_heads, int is_causal, int use_rope,
                             float rope_theta, const float *rope_cos_cache, const float *rope_sin_cache,
                             const blt_mask_config *mask_config);
+
+/* models/cross_attention.c:101-157 with host buffers: query_in [P,E], kv_in
+ * [T,E], four [E,E] weights, output [P,E]; mask_config is required. */
+int orc_cross_attention_forward(const float *query_in, const float *kv_in, const float *wq, const float *wk,
+                                const float *wv, const float *wproj, float *output, size_t num_patches,
+                                size_t seq_len, size_t embed_dim, size_t num_heads,
+                                const blt_mask_config *mask_config);
 
 /* reductions_cpu.c:325-352 (eps 1e-6), elementwise_cpu.c:9-18 and 86-99. */
 void orc_rmsnorm_forward(const float *x, const float *weight, float *out, size_t rows, size_t dim);

@@ -615,6 +615,68 @@ def test_multihead_attention_block(T, E, H, causal, rope, mask, cached, oracle, 
     assert_close(got, ref, "attention block T=%d E=%d H=%d" % (T, E, H))
 
 
+@pytest.mark.parametrize("P,T,E,H,kind", [
+    (2, 4, 4, 2, "identity"),          # tests/unit/models/unit_cross_attention.c:24-117
+    (9, 70, 32, 4, "groups"),          # few rows: exact products
+    (128, 512, 128, 4, "groups"),      # the encoder's call at C3 size: split-K products, two outputs in one pass
+    (128, 512, 128, 4, "even"),        # 4 bytes per patch, the shape the bench uses
+    (40, 4099, 128, 2, "groups"),      # long, ragged groups; K and V through the 64x64 product kernel
+    (33, 100, 48, 3, "interleaved"),   # groups not contiguous: dense mask from the device builder
+    (64, 200, 64, 2, "window"),        # no groups: window-only visibility
+])
+def test_cross_attention_block(P, T, E, H, kind, oracle, dev):
+    """blt_cross_attention_forward on device tensors against the restated block."""
+    import torch
+    lib = api.load()
+    rs = np.random.RandomState(P + T + E)
+    if kind == "identity":
+        xq = np.array([[1, 0, 1, 0], [0, 1, 0, 1]], dtype=np.float32)
+        xkv = np.array([[1, 0, 1, 0], [0, 1, 0, 1], [1, 0, 1, 0], [0, 1, 0, 1]], dtype=np.float32)
+        ws = [np.eye(4, dtype=np.float32) for _ in range(4)]
+    else:
+        xq, xkv = rs.randn(P, E).astype(np.float32), rs.randn(T, E).astype(np.float32)
+        ws = [(rs.randn(E, E) / np.sqrt(E)).astype(np.float32) for _ in range(4)]
+    cfg = abi.BltMaskConfig()
+    cfg.seq_len_q, cfg.seq_len_kv = P, T
+    keep = None
+    if kind == "window":
+        cfg.sliding_window = 90
+    else:
+        if kind == "identity":
+            groups = np.array([0, 0, 1, 1])
+        elif kind == "even":
+            groups = np.arange(T) // (T // P)
+        else:
+            groups = np.sort(np.concatenate([np.arange(P), rs.randint(0, P, size=T - P)]))
+            if kind == "interleaved":
+                groups = rs.permutation(groups)
+        keep = (abi.size_array(list(range(P))), abi.size_array(groups.tolist()))
+        cfg.query_group_ids, cfg.kv_group_ids = keep
+        cfg.bidirectional_within_group = True
+    ref = np.zeros((P, E), dtype=np.float32)
+    assert oracle.orc_cross_attention_forward(*(binding.fptr(a.reshape(-1)) for a in (xq, xkv, *ws, ref)), P, T, E, H,
+                                              C.byref(cfg)) == 0
+    if kind == "identity":
+        assert abs(ref[0, 0] - 0.6697615) < 1e-6 and abs(ref[1, 0] - 0.3302385) < 1e-6
+    dev_in = [torch.from_numpy(a).cuda() for a in (xq, xkv, *ws)]
+    to = torch.full((P, E), 7.0, dtype=torch.float32, device="cuda")
+    views = [_dev_tensor(t) for t in dev_in]
+    vo = _dev_tensor(to)
+    wts = abi.BltCrossAttentionWeights(*(C.pointer(v) for v in views[2:]))
+    cc = abi.BltCrossAttentionConfig()
+    cc.embed_dim, cc.num_heads, cc.head_dim = E, H, 0   # 0 = embed_dim / num_heads
+    cc.mask_config = C.pointer(cfg)
+    arena = lib.blt_arena_create(64 << 20, abi.BLT_BACKEND_HIP)
+    try:
+        lib.blt_cross_attention_forward(C.byref(views[0]), C.byref(views[1]), C.byref(wts), C.byref(vo), C.byref(cc),
+                                        arena)
+        lib.blt_backend_pass_sync_hip()
+        got = to.cpu().numpy()
+    finally:
+        lib.blt_arena_destroy(arena)
+    assert_close(got, ref, "cross attention P=%d T=%d E=%d H=%d %s" % (P, T, E, H, kind))
+
+
 def test_row_ops(oracle, dev):
     """blt_rmsnorm_forward and blt_add bit-identical to the reference loops, blt_swiglu_forward in tolerance."""
     import torch

@@ -529,6 +529,90 @@ def test_attention_block_equals_its_parts(oracle):
     assert got.tobytes() == want.tobytes()
 
 
+def _group_cfg(P, T, q_groups, kv_groups):
+    cfg = abi.BltMaskConfig()
+    cfg.seq_len_q, cfg.seq_len_kv = P, T
+    keep = (abi.size_array(q_groups), abi.size_array(kv_groups))
+    cfg.query_group_ids, cfg.kv_group_ids = keep
+    cfg.bidirectional_within_group = True
+    return cfg, keep
+
+
+def _xattn(oracle, xq, xkv, wq, wk, wv, wp, H, cfg):
+    P, E = xq.shape
+    out = np.full((P, E), 3.0, dtype=np.float32)
+    rc = oracle.orc_cross_attention_forward(*(binding.fptr(a.reshape(-1)) for a in (xq, xkv, wq, wk, wv, wp, out)), P,
+                                            xkv.shape[0], E, H, C.byref(cfg) if cfg is not None else None)
+    return rc, out
+
+
+def test_cross_attention_reference_vectors(oracle):
+    """tests/unit/models/unit_cross_attention.c:24-117 (identity weights, two patches over two bytes
+    each) and 124-246 (bytes of patch 1 never reach patch 0)."""
+    xq = np.array([[1, 0, 1, 0], [0, 1, 0, 1]], dtype=np.float32)
+    xkv = np.array([[1, 0, 1, 0], [0, 1, 0, 1], [1, 0, 1, 0], [0, 1, 0, 1]], dtype=np.float32)
+    eye = np.eye(4, dtype=np.float32)
+    cfg, _keep = _group_cfg(2, 4, [0, 1], [0, 0, 1, 1])
+    rc, out = _xattn(oracle, xq, xkv, eye, eye, eye, eye, 2, cfg)
+    want = np.array([[0.6697615, 0.3302385, 0.6697615, 0.3302385], [0.3302385, 0.6697615, 0.3302385, 0.6697615]])
+    assert rc == 0 and np.abs(out - want).max() < 1e-6
+    xkv_b = xkv.copy()
+    xkv_b[2] = [500, -500, 250, -250]
+    xkv_b[3] = [-500, 500, -250, 250]
+    rc, out_b = _xattn(oracle, xq, xkv_b, eye, eye, eye, eye, 2, cfg)
+    assert rc == 0 and out_b[0].tobytes() == out[0].tobytes() and np.abs(out_b[1] - out[1]).max() > 1e-3
+    # the mask is required, and its lengths must be the call's (cross_attention.c:23-24, 58-60)
+    assert _xattn(oracle, xq, xkv, eye, eye, eye, eye, 2, None)[0] == 8
+    bad, _k2 = _group_cfg(2, 3, [0, 1], [0, 0, 1])
+    assert _xattn(oracle, xq, xkv, eye, eye, eye, eye, 2, bad)[0] == 8
+
+
+def test_cross_attention_equals_its_parts_and_float64(oracle):
+    rs = np.random.RandomState(77)
+    P, T, E, H = 5, 23, 24, 3
+    hd = E // H
+    xq, xkv = rs.randn(P, E).astype(np.float32), rs.randn(T, E).astype(np.float32)
+    wq, wk, wv, wp = ((rs.randn(E, E) / np.sqrt(E)).astype(np.float32) for _ in range(4))
+    kv_groups = np.sort(np.concatenate([np.arange(P), rs.randint(0, P, size=T - P)]))
+    cfg, _keep = _group_cfg(P, T, list(range(P)), kv_groups.tolist())
+    rc, got = _xattn(oracle, xq, xkv, wq, wk, wv, wp, H, cfg)
+    assert rc == 0
+    # a patch that owns no byte is refused by the mask builder (mask_builder_cpu.c:93)
+    holed = kv_groups.copy()
+    holed[holed == 2] = 3
+    cfg_h, _keep_h = _group_cfg(P, T, list(range(P)), holed.tolist())
+    assert _xattn(oracle, xq, xkv, wq, wk, wv, wp, H, cfg_h)[0] == 4
+    # composition of the pinned parts, bit for bit
+    def mm(a, b):
+        o = np.zeros((a.shape[0], b.shape[1]), dtype=np.float32)
+        oracle.orc_matmul(binding.fptr(a.reshape(-1)), binding.fptr(b.reshape(-1)), binding.fptr(o.reshape(-1)),
+                          a.shape[0], a.shape[1], b.shape[1])
+        return o
+    q, k, v = mm(xq, wq), mm(xkv, wk), mm(xkv, wv)
+    mask = np.empty(P * T, dtype=np.float32)
+    assert oracle.orc_build_attention_mask(C.byref(cfg), binding.fptr(mask)) == 0
+    comb = np.zeros((P, E), dtype=np.float32)
+    w = np.zeros(P * T, dtype=np.float32)
+    for h in range(H):
+        a = binding.head_args(q.reshape(-1), k.reshape(-1), v.reshape(-1), comb.reshape(-1), P, T, hd,
+                              float(np.float32(1) / np.sqrt(np.float32(hd))), E, E, E, E, h * hd, q_off=h * hd,
+                              k_off=h * hd, v_off=h * hd, weights=w, mask=mask)
+        assert oracle.orc_attention_head_core(C.byref(a)) == 0
+    assert got.tobytes() == mm(comb, wp).tobytes()
+    # float64 restatement from the definition (different operand for K/V than for Q shows a swapped input)
+    q64, k64, v64 = xq.astype(np.float64) @ wq, xkv.astype(np.float64) @ wk, xkv.astype(np.float64) @ wv
+    comb64 = np.zeros((P, E))
+    for h in range(H):
+        sl = slice(h * hd, (h + 1) * hd)
+        sc = q64[:, sl] @ k64[:, sl].T / np.sqrt(hd)
+        for i in range(P):
+            keys = np.nonzero(kv_groups == i)[0]
+            e = np.exp(sc[i, keys] - sc[i, keys].max())
+            comb64[i, sl] = (e / e.sum()) @ v64[keys, sl]
+    want = comb64 @ wp.astype(np.float64)
+    assert np.abs(got - want).max() < 2e-5
+
+
 # ---------------------------------------------------------------------------
 # row ops of the decoder layer (reductions_cpu.c:325-352, elementwise_cpu.c:9-18, 86-99)
 # ---------------------------------------------------------------------------

@@ -317,6 +317,45 @@ def test_matmul_and_attention_block_bit_exact(oracle, ref):
         ref.blt_arena_destroy(arena)
 
 
+def test_cross_attention_block_bit_exact(oracle, ref):
+    """orc_cross_attention_forward against blt_cross_attention_forward compiled from the reference
+    (csrc/models/cross_attention.c:101-157)."""
+    rs = np.random.RandomState(53)
+    arena = ref.blt_arena_create(32 << 20, CPU)
+    try:
+        for P, T, E, H, kind in ((2, 4, 4, 2, "groups"), (9, 70, 32, 4, "groups"), (16, 64, 64, 2, "uneven"),
+                                 (12, 40, 24, 3, "window")):
+            xq, xkv = rs.randn(P, E).astype(np.float32), rs.randn(T, E).astype(np.float32)
+            ws = [(rs.randn(E, E) / np.sqrt(E)).astype(np.float32) for _ in range(4)]
+            cfg = abi.BltMaskConfig()
+            cfg.seq_len_q, cfg.seq_len_kv = P, T
+            keep = None
+            if kind == "window":
+                cfg.sliding_window = 7
+            else:
+                # every patch owns at least one byte (a patch without one is fatal: mask_builder_cpu.c:93)
+                extra = rs.randint(0, P, size=T - P) if kind == "groups" else rs.randint(0, 3, size=T - P)
+                groups = np.sort(np.concatenate([np.arange(P), extra]))
+                keep = (abi.size_array(list(range(P))), abi.size_array(groups.tolist()))
+                cfg.query_group_ids, cfg.kv_group_ids = keep
+                cfg.bidirectional_within_group = True
+            mine = np.zeros((P, E), dtype=np.float32)
+            assert oracle.orc_cross_attention_forward(
+                *(binding.fptr(a.reshape(-1)) for a in (xq, xkv, *ws, mine)), P, T, E, H, C.byref(cfg)) == 0
+            theirs = np.zeros((P, E), dtype=np.float32)
+            tq, tkv, tw0, tw1, tw2, tw3, to = (abi.tensor_view(a.ctypes.data, a.shape, CPU)
+                                               for a in (xq, xkv, *ws, theirs))
+            wts = abi.BltCrossAttentionWeights(C.pointer(tw0), C.pointer(tw1), C.pointer(tw2), C.pointer(tw3))
+            cc = abi.BltCrossAttentionConfig()
+            cc.embed_dim, cc.num_heads, cc.head_dim = E, H, E // H
+            cc.mask_config = C.pointer(cfg)
+            arena.contents.offset = 0
+            ref.blt_cross_attention_forward(C.byref(tq), C.byref(tkv), C.byref(wts), C.byref(to), C.byref(cc), arena)
+            assert mine.tobytes() == theirs.tobytes(), (P, T, E, H, kind)
+    finally:
+        ref.blt_arena_destroy(arena)
+
+
 def test_row_ops_bit_exact(oracle, ref):
     """orc_rmsnorm_forward / orc_add / orc_swiglu_forward against the reference's ops
     (csrc/ops/reductions_cpu.c:327-352, elementwise_cpu.c:9-18, 86-99)."""
