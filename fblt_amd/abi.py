@@ -139,6 +139,66 @@ class BltPatchInfo(C.Structure):
     ]
 
 
+class BltLocalLayerStorage(C.Structure):
+    """csrc/models/local_common.h:21-35"""
+    _fields_ = [(n, BltTensor) for n in (
+        "norm1_weight", "attn_qkv_w", "attn_proj_w", "norm2_weight", "ffn_up_w", "ffn_gate_w", "ffn_down_w",
+        "cross_norm_weight", "cross_weight_q", "cross_weight_k", "cross_weight_v", "cross_weight_proj")]
+
+
+class BltLocalDecoderConfig(C.Structure):
+    """csrc/models/local_decoder.h:17-30"""
+    _fields_ = [
+        ("embed_dim", C.c_size_t),
+        ("patch_dim", C.c_size_t),
+        ("num_layers", C.c_size_t),
+        ("hidden_dim", C.c_size_t),
+        ("num_heads", C.c_size_t),
+        ("cross_attn_heads", C.c_size_t),
+        ("local_window", C.c_size_t),
+        ("cross_attn_all_layers", C.c_bool),
+        ("cross_attn_placement", C.c_int),
+        ("rope_theta", C.c_float),
+        ("max_seq_len", C.c_size_t),
+        ("vocab_size", C.c_size_t),
+    ]
+
+
+class BltLocalDecoder(C.Structure):
+    """csrc/models/local_decoder.h:60-72"""
+    _fields_ = [
+        ("config", BltLocalDecoderConfig),
+        ("rope_cos_cache", BltTensor),
+        ("rope_sin_cache", BltTensor),
+        ("layers", C.POINTER(BltLocalLayerStorage)),
+        ("lm_head_weight", BltTensor),
+        ("d0_embed_weight", BltTensor),
+    ]
+
+
+class BltKvCache(C.Structure):
+    """csrc/infer/kv_cache.h:45-65"""
+    _fields_ = [
+        ("decoder", C.POINTER(BltLocalDecoder)),
+        ("max_seq_len", C.c_size_t),
+        ("batch_size", C.c_size_t),
+        ("max_subtokens", C.c_size_t),
+        ("embed_dim", C.c_size_t),
+        ("k", C.c_size_t),
+        ("patch_dim", C.c_size_t),
+        ("self_k", C.POINTER(BltTensor)),
+        ("self_v", C.POINTER(BltTensor)),
+        ("self_len", C.c_size_t),
+        ("cross_k", C.POINTER(BltTensor)),
+        ("cross_v", C.POINTER(BltTensor)),
+        ("cross_num_patches", C.c_size_t),
+        ("cached_patches", C.POINTER(BltPatchInfo)),
+    ]
+
+
+BLT_XATTN_DEFAULT, BLT_XATTN_NONE, BLT_XATTN_LAST, BLT_XATTN_ALL, BLT_XATTN_FIRST = range(5)
+
+
 def check_layout():
     assert C.sizeof(BltTensor) == 104
     assert C.sizeof(BltArena) == 32
@@ -156,6 +216,9 @@ def check_layout():
     assert C.sizeof(BltTransformerWeights) == 72
     assert C.sizeof(BltCrossAttentionConfig) == 48 and BltCrossAttentionConfig.num_heads.offset == 24
     assert C.sizeof(BltCrossAttentionWeights) == 32
+    assert C.sizeof(BltLocalLayerStorage) == 1248 and C.sizeof(BltLocalDecoderConfig) == 88
+    assert C.sizeof(BltLocalDecoder) == 512 and BltLocalDecoder.layers.offset == 296
+    assert C.sizeof(BltKvCache) == 112 and BltKvCache.cached_patches.offset == 104
 
 
 def tensor_view(ptr, shape, backend, dtype=BLT_DTYPE_FP32):

@@ -50,6 +50,11 @@ class BltHipKernelTime(C.Structure):
                 ("min_ms", C.c_double), ("max_ms", C.c_double)]
 
 
+KV_REFRESH_ARGS = [C.POINTER(abi.BltKvCache), C.POINTER(abi.BltTensor), C.POINTER(abi.BltPatchInfo), C.c_size_t,
+                   C.c_size_t, C.POINTER(abi.BltArena)]
+KV_STEP_ARGS = [C.POINTER(abi.BltKvCache), C.POINTER(abi.BltTensor), C.POINTER(abi.BltPatchInfo), C.c_size_t,
+                C.POINTER(abi.BltTensor), C.c_int, C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)]
+
 # name -> (restype, argtypes); every symbol include/blt_hip.h declares
 SYMBOLS = {
     "blt_attention_head_core_hip": (None, [C.c_int, C.POINTER(abi.BltAttentionHeadArgs)]),
@@ -133,6 +138,25 @@ SYMBOLS = {
     "blt_cross_attention_forward": (None, [C.POINTER(abi.BltTensor), C.POINTER(abi.BltTensor),
                                            C.POINTER(abi.BltCrossAttentionWeights), C.POINTER(abi.BltTensor),
                                            C.POINTER(abi.BltCrossAttentionConfig), C.POINTER(abi.BltArena)]),
+    "blt_kv_cache_create": (C.POINTER(abi.BltKvCache), [C.POINTER(abi.BltArena), C.POINTER(abi.BltLocalDecoder),
+                                                        C.c_size_t]),
+    "blt_kv_cache_create_batched": (C.POINTER(abi.BltKvCache), [C.POINTER(abi.BltArena),
+                                                                C.POINTER(abi.BltLocalDecoder), C.c_size_t,
+                                                                C.c_size_t]),
+    "blt_kv_cache_destroy": (None, [C.POINTER(abi.BltKvCache)]),
+    "blt_kv_cache_reset": (None, [C.POINTER(abi.BltKvCache)]),
+    "blt_kv_cache_truncate": (None, [C.POINTER(abi.BltKvCache), C.c_size_t, C.c_size_t]),
+    "blt_kv_cache_common_patches": (C.c_size_t, [C.POINTER(abi.BltKvCache), C.POINTER(abi.BltPatchInfo), C.c_size_t]),
+    "blt_local_cross_attn_fires": (C.c_bool, [C.c_int, C.c_bool, C.c_size_t, C.c_size_t]),
+    "blt_kv_cache_refresh_cross": (None, KV_REFRESH_ARGS),
+    "blt_kv_cache_refresh_cross_hip": (None, KV_REFRESH_ARGS),
+    "blt_kv_cache_refresh_cross_seq_hip": (None, [KV_REFRESH_ARGS[0], C.c_size_t] + KV_REFRESH_ARGS[1:]),
+    "blt_kv_decode_step": (None, KV_STEP_ARGS),
+    "blt_kv_decode_step_hip": (None, KV_STEP_ARGS),
+    "blt_kv_decode_step_batched_hip": (None, [C.POINTER(abi.BltKvCache), abi.c_size_p,
+                                              C.POINTER(C.POINTER(abi.BltPatchInfo)), abi.c_size_p,
+                                              C.POINTER(C.c_int), C.POINTER(abi.BltTensor), C.POINTER(abi.BltTensor),
+                                              C.POINTER(abi.BltArena)]),
     "blt_hip_set_stream": (None, [C.c_void_p]),
     "blt_hip_get_stream": (C.c_void_p, []),
     "blt_hip_capture_begin": (None, []),

@@ -167,6 +167,110 @@ void blt_cross_attention_forward(const blt_tensor *query_in, const blt_tensor *k
     blt_cross_attention_forward_hip(query_in, kv_in, weights, output, config, arena);
 }
 
+/* ------------------------------------------------------------------ */
+/* two-tier KV cache container (csrc/infer/kv_cache.c:27-110)          */
+/* ------------------------------------------------------------------ */
+blt_kv_cache *blt_kv_cache_create_batched(blt_arena *arena, const blt_local_decoder *decoder, size_t max_seq_len,
+                                          size_t batch_size) {
+    if (batch_size == 0) batch_size = 1;
+    BLT_REQUIRE(arena != NULL && decoder != NULL, "blt_kv_cache_create: arena and decoder cannot be NULL");
+    BLT_REQUIRE(max_seq_len >= 2 && max_seq_len <= decoder->config.max_seq_len,
+                "blt_kv_cache_create: max_seq_len must be in [2, decoder max_seq_len]");
+    const size_t E = decoder->config.embed_dim;
+    const size_t patch_dim = decoder->config.patch_dim ? decoder->config.patch_dim : E;
+    BLT_REQUIRE(E != 0 && patch_dim % E == 0, "blt_kv_cache_create: patch_dim must be a multiple of embed_dim");
+    const size_t L = decoder->config.num_layers;
+    blt_kv_cache *c = (blt_kv_cache *)calloc(1, sizeof(*c));
+    BLT_REQUIRE(c != NULL, "blt_kv_cache_create: failed to allocate cache container");
+    c->decoder = decoder;
+    c->max_seq_len = max_seq_len;
+    c->batch_size = batch_size;
+    c->max_subtokens = max_seq_len; /* a patch holds at least one byte */
+    c->embed_dim = E;
+    c->patch_dim = patch_dim;
+    c->k = patch_dim / E;
+    /* four separate heap arrays, as the reference's destroy frees them one by one (kv_cache.c:77-87) */
+    c->self_k = (blt_tensor *)calloc(L ? L : 1, sizeof(blt_tensor));
+    c->self_v = (blt_tensor *)calloc(L ? L : 1, sizeof(blt_tensor));
+    c->cross_k = (blt_tensor *)calloc(L ? L : 1, sizeof(blt_tensor));
+    c->cross_v = (blt_tensor *)calloc(L ? L : 1, sizeof(blt_tensor));
+    BLT_REQUIRE(c->self_k && c->self_v && c->cross_k && c->cross_v,
+                "blt_kv_cache_create: failed to allocate layer handle arrays");
+    const size_t self_shape[2] = {batch_size * max_seq_len, E};
+    const size_t cross_shape[2] = {batch_size * c->max_subtokens, E};
+    for (size_t l = 0; l < L; l++) {
+        c->self_k[l] = blt_tensor_create(arena, self_shape, 2, BLT_DTYPE_FP32);
+        c->self_v[l] = blt_tensor_create(arena, self_shape, 2, BLT_DTYPE_FP32);
+        c->cross_k[l] = blt_tensor_create(arena, cross_shape, 2, BLT_DTYPE_FP32);
+        c->cross_v[l] = blt_tensor_create(arena, cross_shape, 2, BLT_DTYPE_FP32);
+    }
+    c->cached_patches = (blt_patch_info *)calloc(batch_size * max_seq_len, sizeof(blt_patch_info));
+    BLT_REQUIRE(c->cached_patches != NULL, "blt_kv_cache_create: failed to allocate patch table");
+    return c;
+}
+
+blt_kv_cache *blt_kv_cache_create(blt_arena *arena, const blt_local_decoder *decoder, size_t max_seq_len) {
+    return blt_kv_cache_create_batched(arena, decoder, max_seq_len, 1);
+}
+
+void blt_kv_cache_destroy(blt_kv_cache *cache) {
+    if (!cache) return;
+    free(cache->self_k);
+    free(cache->self_v);
+    free(cache->cross_k);
+    free(cache->cross_v);
+    free(cache->cached_patches);
+    free(cache);
+}
+
+void blt_kv_cache_reset(blt_kv_cache *cache) {
+    cache->self_len = 0;
+    cache->cross_num_patches = 0;
+}
+
+void blt_kv_cache_truncate(blt_kv_cache *cache, size_t self_len, size_t num_patches) {
+    BLT_REQUIRE(self_len <= cache->max_seq_len, "blt_kv_cache_truncate: self_len out of range");
+    BLT_REQUIRE(num_patches <= cache->max_subtokens, "blt_kv_cache_truncate: num_patches out of range");
+    cache->self_len = self_len;
+    cache->cross_num_patches = num_patches;
+}
+
+size_t blt_kv_cache_common_patches(const blt_kv_cache *cache, const blt_patch_info *patches, size_t num_patches) {
+    size_t same = 0;
+    while (same < cache->cross_num_patches && same < num_patches &&
+           cache->cached_patches[same].start_idx == patches[same].start_idx &&
+           cache->cached_patches[same].length == patches[same].length)
+        same++;
+    return same;
+}
+
+bool blt_local_cross_attn_fires(blt_xattn_placement placement, bool cross_attn_all_layers, size_t num_layers,
+                                size_t layer) {
+    switch (placement) {
+    case BLT_XATTN_NONE: return false;
+    case BLT_XATTN_LAST: return layer + 1 == num_layers;
+    case BLT_XATTN_ALL: return true;
+    case BLT_XATTN_FIRST: return layer == 0;
+    case BLT_XATTN_DEFAULT:
+    default: return cross_attn_all_layers || layer + 1 == num_layers;
+    }
+}
+
+void blt_kv_cache_refresh_cross(blt_kv_cache *cache, const blt_tensor *patch_in, const blt_patch_info *patches,
+                                size_t num_patches, size_t from_patch, blt_arena *arena) {
+    BLT_REQUIRE(patch_in != NULL, "blt_kv_cache_refresh_cross: arguments cannot be NULL");
+    BLT_DEVICE_ONLY(patch_in->backend, "blt_kv_cache_refresh_cross");
+    blt_kv_cache_refresh_cross_hip(cache, patch_in, patches, num_patches, from_patch, arena);
+}
+
+void blt_kv_decode_step(blt_kv_cache *cache, const blt_tensor *patch_in, const blt_patch_info *patches,
+                        size_t num_patches, const blt_tensor *d0_rows, int trailing_closed, blt_tensor *logits_out,
+                        blt_arena *arena) {
+    BLT_REQUIRE(d0_rows != NULL, "blt_kv_decode_step: arguments cannot be NULL");
+    BLT_DEVICE_ONLY(d0_rows->backend, "blt_kv_decode_step");
+    blt_kv_decode_step_hip(cache, patch_in, patches, num_patches, d0_rows, trailing_closed, logits_out, arena);
+}
+
 void blt_add(const blt_tensor *a, const blt_tensor *b, blt_tensor *out) {
     BLT_REQUIRE(a != NULL, "blt_add: input tensors must be FP32 with matching element count");
     BLT_DEVICE_ONLY(a->backend, "blt_add");

@@ -17,8 +17,10 @@
 #include "launch.h"
 #include "matmul.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <vector>
 
 namespace {
 
@@ -219,4 +221,335 @@ extern "C" void blt_kv_decode_layer_hip(const blt_kv_attn_cache *cache, const bl
     }
     gemm(gate, f32(w->ffn_down_w), rows_out, rows, Hd, E, resid1); /* projection + residual */
     HIP_CHECK_LAUNCH("blt_kv_decode_layer");
+}
+
+/* ===================================================================== */
+/* The whole incremental decoder step (csrc/infer/kv_cache.c:112-416)     */
+/* ===================================================================== */
+namespace {
+
+struct CrossRowsArgs {
+    const float *q;     /* [rows, E] projected queries                               */
+    const float *k;     /* tier-2 slabs [batch*slab_rows, E]                         */
+    const float *v;
+    float *out;         /* [rows, E] combined                                        */
+    const uint32_t *lo; /* [rows] first visible sub-token of the row's own slab      */
+    const uint32_t *hi; /* [rows] one past the last                                  */
+    uint32_t n;         /* new rows per sequence: row R belongs to sequence R / n    */
+    uint32_t E, xhd;
+    uint64_t slab_rows;
+    float scale;
+};
+
+/* One wave per (new row, head): the row sees the few sub-tokens of its latent
+ * patch (kv_cache.c:240-251), so the keys are walked one after the other,
+ * lanes over the head's columns.  Softmax as blt_softmax_masked_row_inplace:
+ * maximum over finite scores, non-finite scores weigh nothing, an empty or
+ * all-dead row gives zeros. */
+__global__ __launch_bounds__(64) void kv_cross_rows_kernel(CrossRowsArgs a) {
+    const uint32_t R = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    const uint32_t seq = R / a.n;
+    const uint32_t lo = a.lo[R], hi = a.hi[R];
+    const float *q = a.q + (size_t)R * a.E + head * a.xhd;
+    const float *kb = a.k + (size_t)seq * a.slab_rows * a.E + head * a.xhd;
+    const float *vb = a.v + (size_t)seq * a.slab_rows * a.E + head * a.xhd;
+    auto score = [&](uint32_t j) {
+        float p = 0.f;
+        for (uint32_t d = lane; d < a.xhd; d += 64u) p += q[d] * kb[(size_t)j * a.E + d];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) p += __shfl_xor(p, off, 64);
+        return p * a.scale;
+    };
+    float mx = -INFINITY;
+    for (uint32_t j = lo; j < hi; j++) {
+        const float s = score(j);
+        if (isfinite(s)) mx = fmaxf(mx, s);
+    }
+    float sum = 0.f;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f}; /* head widths up to 256 columns */
+    for (uint32_t j = lo; j < hi; j++) {
+        const float s = score(j);
+        const float e = isfinite(s) ? expf(s - mx) : 0.f;
+        if (e == 0.f) continue;
+        sum += e;
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const uint32_t d = lane + 64u * t;
+            if (d < a.xhd) acc[t] += e * vb[(size_t)j * a.E + d];
+        }
+    }
+    const float inv = sum > 0.f ? 1.0f / sum : 0.f;
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const uint32_t d = lane + 64u * t;
+        if (d < a.xhd) a.out[(size_t)R * a.E + head * a.xhd + d] = acc[t] * inv;
+    }
+}
+
+bool cross_fires(const blt_local_decoder_config *c, size_t layer) {
+    switch (c->cross_attn_placement) { /* csrc/models/local_common.c:49-64 */
+    case BLT_XATTN_NONE: return false;
+    case BLT_XATTN_LAST: return layer + 1 == c->num_layers;
+    case BLT_XATTN_ALL: return true;
+    case BLT_XATTN_FIRST: return layer == 0;
+    default: return c->cross_attn_all_layers || layer + 1 == c->num_layers;
+    }
+}
+
+void check_vec(const blt_tensor &t, size_t dim, const char *what) {
+    BLT_REQUIRE(t.data != NULL && t.ndim == 1 && t.shape[0] == dim && t.dtype == BLT_DTYPE_FP32 &&
+                    t.backend == BLT_BACKEND_HIP,
+                "%s", what);
+}
+
+/* The step for `batch` sequences with n new rows each: base[b] is sequence b's
+ * valid length, group[b*n + r] the latent patch of its row r.  Lengths and
+ * group ranges travel to the device in one staged copy. */
+void decode_step_run(const blt_kv_cache *cache, size_t batch, size_t n, const size_t *base, const size_t *group,
+                     const float *d0_rows, float *logits, blt_arena *arena) {
+    const blt_local_decoder *dec = cache->decoder;
+    const blt_local_decoder_config *cfg = &dec->config;
+    const size_t E = cache->embed_dim, L = cfg->num_layers, H = cfg->num_heads, XH = cfg->cross_attn_heads;
+    const size_t V = cfg->vocab_size, rows = batch * n, hd = E / H, xhd = E / XH;
+    BLT_REQUIRE(xhd <= 256, "blt_kv_decode_step: cross-attention heads wider than 256 columns are not supported");
+    check_weight(&dec->lm_head_weight, E, V, "blt_kv_decode_step: lm_head_weight must be [embed_dim, vocab_size]");
+    check_weight(&dec->rope_cos_cache, cfg->max_seq_len, hd / 2,
+                 "blt_kv_decode_step: rope_cos_cache must be [max_seq_len, head_dim/2]");
+    check_weight(&dec->rope_sin_cache, cfg->max_seq_len, hd / 2,
+                 "blt_kv_decode_step: rope_sin_cache must be [max_seq_len, head_dim/2]");
+
+    /* lengths, then lo / hi of every row's sub-token range, in one upload */
+    std::vector<uint32_t> host(batch + 2 * rows);
+    size_t max_total = 0;
+    for (size_t b = 0; b < batch; b++) {
+        host[b] = (uint32_t)base[b];
+        max_total = std::max(max_total, base[b] + n);
+        for (size_t r = 0; r < n; r++) {
+            host[batch + b * n + r] = (uint32_t)(group[b * n + r] * cache->k);
+            host[batch + rows + b * n + r] = (uint32_t)((group[b * n + r] + 1) * cache->k);
+        }
+    }
+    uint32_t *dev = (uint32_t *)blt_arena_alloc(arena, host.size() * sizeof(uint32_t), 64);
+    blt_upload_staged(dev, host.data(), host.size() * sizeof(uint32_t));
+
+    float *ping = (float *)blt_arena_alloc(arena, rows * E * sizeof(float), 64);
+    float *pong = (float *)blt_arena_alloc(arena, rows * E * sizeof(float), 64);
+    float *mid = (float *)blt_arena_alloc(arena, rows * E * sizeof(float), 64);
+    float *xq = (float *)blt_arena_alloc(arena, rows * E * sizeof(float), 64);
+    float *xnorm = (float *)blt_arena_alloc(arena, rows * E * sizeof(float), 64);
+    float *xcomb = (float *)blt_arena_alloc(arena, rows * E * sizeof(float), 64);
+    const size_t arena_mark = arena->offset;
+
+    const float *cur = d0_rows;
+    for (size_t l = 0; l < L; l++) {
+        const blt_local_layer_storage *s = &dec->layers[l];
+        const float *in = cur;
+        if (cross_fires(cfg, l)) { /* kv_cache.c:303-341 */
+            check_vec(s->cross_norm_weight, E, "blt_kv_decode_step: cross_norm_weight must be [embed_dim] FP32");
+            check_weight(&s->cross_weight_q, E, E, "blt_kv_decode_step: cross_weight_q must be [embed_dim, embed_dim]");
+            check_weight(&s->cross_weight_proj, E, E,
+                         "blt_kv_decode_step: cross_weight_proj must be [embed_dim, embed_dim]");
+            MatmulArgs probe;
+            std::memset(&probe, 0, sizeof(probe));
+            probe.m = (uint32_t)rows, probe.k = (uint32_t)E, probe.n = (uint32_t)E;
+            if (matmul_takes_norm(probe)) {
+                gemm(cur, (const float *)s->cross_weight_q.data, xq, rows, E, E, nullptr, nullptr,
+                     (const float *)s->cross_norm_weight.data);
+            } else {
+                rmsnorm_launch(cur, (const float *)s->cross_norm_weight.data, xnorm, rows, E);
+                gemm(xnorm, (const float *)s->cross_weight_q.data, xq, rows, E, E);
+            }
+            CrossRowsArgs c;
+            c.q = xq;
+            c.k = (const float *)cache->cross_k[l].data;
+            c.v = (const float *)cache->cross_v[l].data;
+            c.out = xcomb;
+            c.lo = dev + batch, c.hi = dev + batch + rows;
+            c.n = (uint32_t)n, c.E = (uint32_t)E, c.xhd = (uint32_t)xhd;
+            c.slab_rows = cache->max_subtokens;
+            c.scale = 1.0f / sqrtf((float)xhd);
+            blt_launch("kv_cross_rows", kv_cross_rows_kernel, dim3((unsigned)rows, (unsigned)XH), dim3(64), 0, 0, c);
+            gemm(xcomb, (const float *)s->cross_weight_proj.data, mid, rows, E, E, cur); /* + residual */
+            in = mid;
+        }
+        blt_kv_attn_cache view;
+        view.self_k = (float *)cache->self_k[l].data;
+        view.self_v = (float *)cache->self_v[l].data;
+        view.self_len = dev;
+        view.batch = batch;
+        view.max_seq_len = cache->max_seq_len;
+        view.embed_dim = E;
+        view.num_heads = H;
+        view.window = cfg->local_window;
+        blt_transformer_weights w;
+        std::memset(&w, 0, sizeof(w));
+        w.norm1_weight = &s->norm1_weight, w.attn_qkv_w = &s->attn_qkv_w, w.attn_proj_w = &s->attn_proj_w;
+        w.norm2_weight = &s->norm2_weight, w.ffn_up_w = &s->ffn_up_w, w.ffn_gate_w = &s->ffn_gate_w;
+        w.ffn_down_w = &s->ffn_down_w;
+        float *next = (cur == ping) ? pong : ping;
+        arena->offset = arena_mark; /* the layer's work buffers are reused by the next layer */
+        blt_kv_decode_layer_hip(&view, &w, in, next, (const float *)dec->rope_cos_cache.data,
+                                (const float *)dec->rope_sin_cache.data, cfg->max_seq_len, n, BLT_KV_STEP_CAUSAL, 0,
+                                max_total, arena);
+        cur = next;
+    }
+    gemm(cur, (const float *)dec->lm_head_weight.data, logits, rows, E, V); /* kv_cache.c:416 */
+    HIP_CHECK_LAUNCH("blt_kv_decode_step");
+}
+
+void check_cache(const blt_kv_cache *cache, const char *fn) {
+    BLT_REQUIRE(cache != NULL && cache->decoder != NULL, "%s: cache cannot be NULL", fn);
+    const blt_local_decoder_config *cfg = &cache->decoder->config;
+    BLT_REQUIRE(cfg->num_heads != 0 && cfg->cross_attn_heads != 0 && cache->embed_dim == cfg->embed_dim &&
+                    cfg->embed_dim % cfg->num_heads == 0 && cfg->embed_dim % cfg->cross_attn_heads == 0,
+                "%s: decoder configuration is inconsistent", fn);
+    BLT_REQUIRE(cache->self_k != NULL && cache->self_v != NULL && cache->cross_k != NULL && cache->cross_v != NULL,
+                "%s: cache tiers are missing", fn);
+    for (size_t l = 0; l < cfg->num_layers; l++)
+        BLT_REQUIRE(cache->self_k[l].backend == BLT_BACKEND_HIP && cache->cross_k[l].backend == BLT_BACKEND_HIP,
+                    "%s: HIP implementation called with a cache that is not in device memory", fn);
+}
+
+void refresh_cross_seq(blt_kv_cache *cache, size_t seq, const blt_tensor *patch_in, const blt_patch_info *patches,
+                       size_t num_patches, size_t from_patch) {
+    const blt_local_decoder *dec = cache->decoder;
+    const size_t E = cache->embed_dim, L = dec->config.num_layers;
+    const size_t first = from_patch * cache->k, count = (num_patches - from_patch) * cache->k;
+    for (size_t l = 0; l < L; l++) {
+        if (!cross_fires(&dec->config, l)) continue;
+        const blt_local_layer_storage *s = &dec->layers[l];
+        check_weight(&s->cross_weight_k, E, E, "blt_kv_cache_refresh_cross: cross_weight_k must be [embed_dim, embed_dim]");
+        check_weight(&s->cross_weight_v, E, E, "blt_kv_cache_refresh_cross: cross_weight_v must be [embed_dim, embed_dim]");
+        const size_t row0 = seq * cache->max_subtokens + first;
+        MatmulArgs g;
+        std::memset(&g, 0, sizeof(g));
+        g.a = (const float *)patch_in->data + first * E;
+        g.b = (const float *)s->cross_weight_k.data;
+        g.out = (float *)cache->cross_k[l].data + row0 * E;
+        g.m = (uint32_t)count, g.k = (uint32_t)E, g.n = (uint32_t)E;
+        g.lda = g.ldb = g.ldo = (uint32_t)E;
+        g.b2 = (const float *)s->cross_weight_v.data;
+        g.out2 = (float *)cache->cross_v[l].data + row0 * E;
+        if (matmul_takes_gated(g)) { /* K and V in one pass over the patch rows */
+            matmul_f32_launch(g, 0);
+        } else {
+            g.b2 = nullptr, g.out2 = nullptr;
+            matmul_f32_launch(g, 0);
+            g.b = (const float *)s->cross_weight_v.data;
+            g.out = (float *)cache->cross_v[l].data + row0 * E;
+            matmul_f32_launch(g, 0);
+        }
+    }
+    std::memcpy(&cache->cached_patches[seq * cache->max_seq_len + from_patch], &patches[from_patch],
+                (num_patches - from_patch) * sizeof(blt_patch_info)); /* kv_cache.c:154-157 */
+    HIP_CHECK_LAUNCH("blt_kv_cache_refresh_cross");
+}
+
+void check_refresh_args(const blt_kv_cache *cache, const blt_tensor *patch_in, const blt_patch_info *patches,
+                        size_t num_patches, size_t from_patch, const blt_arena *arena) {
+    BLT_REQUIRE(patch_in != NULL && patches != NULL && arena != NULL,
+                "blt_kv_cache_refresh_cross: arguments cannot be NULL");
+    BLT_REQUIRE(num_patches >= 1 && from_patch < num_patches,
+                "blt_kv_cache_refresh_cross: need from_patch < num_patches");
+    BLT_REQUIRE(patch_in->data != NULL && patch_in->ndim == 2 && patch_in->shape[0] == num_patches &&
+                    patch_in->shape[1] == cache->patch_dim && patch_in->dtype == BLT_DTYPE_FP32,
+                "blt_kv_cache_refresh_cross: patch_in must be [num_patches, patch_dim] FP32");
+    BLT_REQUIRE(patch_in->backend == BLT_BACKEND_HIP,
+                "blt_kv_cache_refresh_cross: HIP implementation called with a non-HIP tensor");
+    BLT_REQUIRE(num_patches * cache->k <= cache->max_subtokens,
+                "blt_kv_cache_refresh_cross: sub-token count exceeds cache capacity");
+}
+
+} // namespace
+
+extern "C" void blt_kv_cache_refresh_cross_hip(blt_kv_cache *cache, const blt_tensor *patch_in,
+                                               const blt_patch_info *patches, size_t num_patches, size_t from_patch,
+                                               blt_arena *arena) {
+    check_cache(cache, "blt_kv_cache_refresh_cross");
+    check_refresh_args(cache, patch_in, patches, num_patches, from_patch, arena);
+    BLT_REQUIRE(from_patch <= cache->cross_num_patches,
+                "blt_kv_cache_refresh_cross: from_patch must not skip uncached patches "
+                "(truncate to the LCP first)");
+    refresh_cross_seq(cache, 0, patch_in, patches, num_patches, from_patch);
+    cache->cross_num_patches = num_patches;
+}
+
+extern "C" void blt_kv_cache_refresh_cross_seq_hip(blt_kv_cache *cache, size_t seq, const blt_tensor *patch_in,
+                                                   const blt_patch_info *patches, size_t num_patches,
+                                                   size_t from_patch, blt_arena *arena) {
+    check_cache(cache, "blt_kv_cache_refresh_cross");
+    BLT_REQUIRE(seq < cache->batch_size, "blt_kv_cache_refresh_cross: sequence index out of range");
+    check_refresh_args(cache, patch_in, patches, num_patches, from_patch, arena);
+    refresh_cross_seq(cache, seq, patch_in, patches, num_patches, from_patch);
+}
+
+extern "C" void blt_kv_decode_step_hip(blt_kv_cache *cache, const blt_tensor *patch_in, const blt_patch_info *patches,
+                                       size_t num_patches, const blt_tensor *d0_rows, int trailing_closed,
+                                       blt_tensor *logits_out, blt_arena *arena) {
+    check_cache(cache, "blt_kv_decode_step");
+    const blt_local_decoder_config *cfg = &cache->decoder->config;
+    const size_t E = cache->embed_dim, V = cfg->vocab_size, hd = E / cfg->num_heads;
+    BLT_REQUIRE(hd > 0 && hd % 2 == 0, "blt_kv_decode_step: RoPE requires an even head_dim");
+    BLT_REQUIRE(patch_in != NULL && patches != NULL && d0_rows != NULL && logits_out != NULL && arena != NULL,
+                "blt_kv_decode_step: arguments cannot be NULL");
+    BLT_REQUIRE(arena->backend == BLT_BACKEND_HIP, "blt_kv_decode_step: HIP implementation needs a device arena");
+    BLT_REQUIRE(num_patches >= 1 && num_patches == cache->cross_num_patches,
+                "blt_kv_decode_step: tier-2 cache must cover all patches (refresh first)");
+    BLT_REQUIRE(d0_rows->data != NULL && d0_rows->ndim == 2 && d0_rows->shape[1] == E &&
+                    d0_rows->dtype == BLT_DTYPE_FP32,
+                "blt_kv_decode_step: d0_rows must be [n, embed_dim] FP32");
+    BLT_REQUIRE(d0_rows->backend == BLT_BACKEND_HIP, "blt_kv_decode_step: HIP implementation called with a non-HIP tensor");
+    const size_t n = d0_rows->shape[0];
+    BLT_REQUIRE(n >= 1, "blt_kv_decode_step: need at least one row");
+    const size_t base = cache->self_len, total = base + n;
+    BLT_REQUIRE(total <= cache->max_seq_len, "blt_kv_decode_step: exceeds cache capacity");
+    BLT_REQUIRE(logits_out->data != NULL && logits_out->ndim == 2 && logits_out->shape[0] == n &&
+                    logits_out->shape[1] == V && logits_out->dtype == BLT_DTYPE_FP32 &&
+                    logits_out->backend == BLT_BACKEND_HIP,
+                "blt_kv_decode_step: logits_out must be [n, vocab_size] FP32");
+    BLT_REQUIRE(num_patches * cache->k <= cache->max_subtokens,
+                "blt_kv_decode_step: sub-token count exceeds cache capacity");
+    std::vector<size_t> group(n); /* kv_cache.c:199-213 */
+    for (size_t r = 0; r < n; r++) group[r] = blt_patch_decoder_latent_at(patches, num_patches, base + r);
+    if (trailing_closed) group[n - 1] = num_patches - 1;
+    decode_step_run(cache, 1, n, &base, group.data(), (const float *)d0_rows->data, (float *)logits_out->data, arena);
+    cache->self_len = total;
+}
+
+extern "C" void blt_kv_decode_step_batched_hip(blt_kv_cache *cache, size_t *self_len,
+                                               const blt_patch_info *const *patches, const size_t *num_patches,
+                                               const int *trailing_closed, const blt_tensor *d0_rows,
+                                               blt_tensor *logits_out, blt_arena *arena) {
+    check_cache(cache, "blt_kv_decode_step_batched");
+    const blt_local_decoder_config *cfg = &cache->decoder->config;
+    const size_t E = cache->embed_dim, V = cfg->vocab_size, hd = E / cfg->num_heads, batch = cache->batch_size;
+    BLT_REQUIRE(hd > 0 && hd % 2 == 0, "blt_kv_decode_step_batched: RoPE requires an even head_dim");
+    BLT_REQUIRE(self_len != NULL && patches != NULL && num_patches != NULL && d0_rows != NULL && logits_out != NULL &&
+                    arena != NULL,
+                "blt_kv_decode_step_batched: arguments cannot be NULL");
+    BLT_REQUIRE(arena->backend == BLT_BACKEND_HIP, "blt_kv_decode_step_batched: HIP implementation needs a device arena");
+    BLT_REQUIRE(d0_rows->data != NULL && d0_rows->ndim == 2 && d0_rows->shape[1] == E &&
+                    d0_rows->dtype == BLT_DTYPE_FP32 && d0_rows->backend == BLT_BACKEND_HIP,
+                "blt_kv_decode_step_batched: d0_rows must be [batch*n, embed_dim] FP32 in device memory");
+    BLT_REQUIRE(batch >= 1 && d0_rows->shape[0] >= batch && d0_rows->shape[0] % batch == 0,
+                "blt_kv_decode_step_batched: d0_rows must hold the same number n >= 1 of rows for every sequence");
+    const size_t n = d0_rows->shape[0] / batch;
+    BLT_REQUIRE(logits_out->data != NULL && logits_out->ndim == 2 && logits_out->shape[0] == batch * n &&
+                    logits_out->shape[1] == V && logits_out->dtype == BLT_DTYPE_FP32 &&
+                    logits_out->backend == BLT_BACKEND_HIP,
+                "blt_kv_decode_step_batched: logits_out must be [batch*n, vocab_size] FP32 in device memory");
+    std::vector<size_t> group(batch * n);
+    for (size_t b = 0; b < batch; b++) {
+        BLT_REQUIRE(patches[b] != NULL && num_patches[b] >= 1,
+                    "blt_kv_decode_step_batched: every sequence needs at least one patch");
+        BLT_REQUIRE(self_len[b] + n <= cache->max_seq_len, "blt_kv_decode_step_batched: exceeds cache capacity");
+        BLT_REQUIRE(num_patches[b] * cache->k <= cache->max_subtokens,
+                    "blt_kv_decode_step_batched: sub-token count exceeds cache capacity");
+        for (size_t r = 0; r < n; r++)
+            group[b * n + r] = blt_patch_decoder_latent_at(patches[b], num_patches[b], self_len[b] + r);
+        if (trailing_closed != NULL && trailing_closed[b]) group[b * n + n - 1] = num_patches[b] - 1;
+    }
+    decode_step_run(cache, batch, n, self_len, group.data(), (const float *)d0_rows->data,
+                    (float *)logits_out->data, arena);
+    for (size_t b = 0; b < batch; b++) self_len[b] += n;
 }

@@ -186,6 +186,73 @@ typedef struct {
     const blt_tensor *ffn_down_w;
 } blt_transformer_weights;
 
+/* ---- local decoder and its two-tier KV cache ---------------------------- */
+/* csrc/models/local_common.h:21-35, 58-64; csrc/models/local_decoder.h:17-30,
+ * 60-72; csrc/infer/kv_cache.h:45-65.  Only the inference-side members are
+ * listed by name in comments; the layouts are complete.                     */
+typedef enum {
+    BLT_XATTN_DEFAULT = 0, /* cross_attn_all_layers decides: all layers, or the last one only */
+    BLT_XATTN_NONE,
+    BLT_XATTN_LAST,
+    BLT_XATTN_ALL,
+    BLT_XATTN_FIRST
+} blt_xattn_placement;
+
+typedef struct {
+    blt_tensor norm1_weight;      /* [E]        */
+    blt_tensor attn_qkv_w;        /* [E, 3E]    */
+    blt_tensor attn_proj_w;       /* [E, E]     */
+    blt_tensor norm2_weight;      /* [E]        */
+    blt_tensor ffn_up_w;          /* [E, hidden]*/
+    blt_tensor ffn_gate_w;        /* [E, hidden]*/
+    blt_tensor ffn_down_w;        /* [hidden, E]*/
+    blt_tensor cross_norm_weight; /* [E]; the cross block comes first in a decoder layer */
+    blt_tensor cross_weight_q;    /* [E, E]     */
+    blt_tensor cross_weight_k;
+    blt_tensor cross_weight_v;
+    blt_tensor cross_weight_proj;
+} blt_local_layer_storage;
+
+typedef struct {
+    size_t embed_dim;
+    size_t patch_dim; /* 0 = embed_dim; a multiple k of embed_dim splits every patch into k sub-tokens */
+    size_t num_layers;
+    size_t hidden_dim;
+    size_t num_heads;
+    size_t cross_attn_heads;
+    size_t local_window; /* 0 = full causal */
+    bool cross_attn_all_layers;
+    blt_xattn_placement cross_attn_placement;
+    float rope_theta;
+    size_t max_seq_len;
+    size_t vocab_size;
+} blt_local_decoder_config;
+
+typedef struct {
+    blt_local_decoder_config config;
+    blt_tensor rope_cos_cache, rope_sin_cache; /* [max_seq_len, head_dim/2] */
+    blt_local_layer_storage *layers;           /* [num_layers] */
+    blt_tensor lm_head_weight;                 /* [embed_dim, vocab_size] */
+    blt_tensor d0_embed_weight;                /* [257, embed_dim]; not read by the decode step */
+} blt_local_decoder;
+
+typedef struct {
+    const blt_local_decoder *decoder;
+    size_t max_seq_len;
+    size_t batch_size;
+    size_t max_subtokens; /* = max_seq_len */
+    size_t embed_dim;
+    size_t k;             /* patch_dim / embed_dim */
+    size_t patch_dim;
+    blt_tensor *self_k;   /* [num_layers] x [batch_size*max_seq_len, embed_dim]: row b*max_seq_len + pos */
+    blt_tensor *self_v;
+    size_t self_len;      /* valid byte positions of the single-sequence cache */
+    blt_tensor *cross_k;  /* [num_layers] x [batch_size*max_subtokens, embed_dim] */
+    blt_tensor *cross_v;
+    size_t cross_num_patches;
+    blt_patch_info *cached_patches; /* [batch_size*max_seq_len] boundary snapshot */
+} blt_kv_cache;
+
 #ifdef __cplusplus
 }
 #define BLT_ABI_ASSERT(c, m) static_assert(c, m)
@@ -216,5 +283,16 @@ BLT_ABI_ASSERT(offsetof(blt_mask_config, bidirectional_within_group) == 56 &&
                "blt_mask_config tail");
 BLT_ABI_ASSERT(sizeof(blt_block_diffusion_config) == 48, "blt_block_diffusion_config layout");
 BLT_ABI_ASSERT(sizeof(blt_patch_info) == 24, "blt_patch_info layout");
+BLT_ABI_ASSERT(sizeof(blt_local_layer_storage) == 12 * 104, "blt_local_layer_storage layout");
+BLT_ABI_ASSERT(sizeof(blt_local_decoder_config) == 88 && offsetof(blt_local_decoder_config, cross_attn_placement) == 60 &&
+                   offsetof(blt_local_decoder_config, rope_theta) == 64 &&
+                   offsetof(blt_local_decoder_config, max_seq_len) == 72,
+               "blt_local_decoder_config layout");
+BLT_ABI_ASSERT(sizeof(blt_local_decoder) == 512 && offsetof(blt_local_decoder, layers) == 296 &&
+                   offsetof(blt_local_decoder, lm_head_weight) == 304,
+               "blt_local_decoder layout");
+BLT_ABI_ASSERT(sizeof(blt_kv_cache) == 112 && offsetof(blt_kv_cache, self_len) == 72 &&
+                   offsetof(blt_kv_cache, cached_patches) == 104,
+               "blt_kv_cache layout");
 
 #endif /* FBLT_AMD_BLT_ABI_H */

@@ -89,6 +89,23 @@ void blt_cross_attention_forward_hip(const blt_tensor *query_in, const blt_tenso
                                      const blt_cross_attention_weights *weights, blt_tensor *output,
                                      const blt_cross_attention_config *config, blt_arena *arena);
 
+/* Device twins of the cache-aware decoder step (csrc/infer/kv_cache.c:
+ * 112-159 and 161-416) with the reference's signatures, for a cache, decoder
+ * weights and rows that live in device memory.  refresh_cross: one launch per
+ * firing layer computes K and V of the new sub-tokens straight into the
+ * tier-2 slabs.  decode_step: per layer the cross block (RMSNorm + Q
+ * projection, the rows' few sub-tokens, projection + residual: 3 launches)
+ * and the self-attention / feed-forward layer (5 launches), then the LM
+ * head; the dense masks, strided copies and per-head calls of the reference
+ * are gone, the row groups follow the same latent rule (kv_cache.c:199-213).
+ * Up to 32 new rows every projection is bit-identical to the CPU reference;
+ * attention is within fp32 tolerance. */
+void blt_kv_cache_refresh_cross_hip(blt_kv_cache *cache, const blt_tensor *patch_in, const blt_patch_info *patches,
+                                    size_t num_patches, size_t from_patch, blt_arena *arena);
+void blt_kv_decode_step_hip(blt_kv_cache *cache, const blt_tensor *patch_in, const blt_patch_info *patches,
+                            size_t num_patches, const blt_tensor *d0_rows, int trailing_closed,
+                            blt_tensor *logits_out, blt_arena *arena);
+
 /* Replace blt_rmsnorm_forward_cuda (csrc/ops/reductions.cu:390-396; CPU loop
  * reductions_cpu.c:327-352, bit-identical here), blt_add_cuda and
  * blt_swiglu_forward_cuda (csrc/ops/elementwise.cu:102-134; CPU loops
@@ -169,6 +186,25 @@ void blt_cross_attention_forward(const blt_tensor *query_in, const blt_tensor *k
 void blt_add(const blt_tensor *a, const blt_tensor *b, blt_tensor *out);
 void blt_swiglu_forward(const blt_tensor *gate, const blt_tensor *up, blt_tensor *out);
 void blt_rmsnorm_forward(const blt_tensor *x, const blt_tensor *weight, blt_tensor *out);
+
+/* csrc/infer/kv_cache.h:70-117 and csrc/models/local_common.h:68-69.  The
+ * cache container and its handle arrays live on the host heap, the K/V
+ * payloads come zero-filled from `arena` (kv_cache.c:27-75); reset, truncate
+ * and common_patches are host bookkeeping (kv_cache.c:77-110). */
+blt_kv_cache *blt_kv_cache_create(blt_arena *arena, const blt_local_decoder *decoder, size_t max_seq_len);
+blt_kv_cache *blt_kv_cache_create_batched(blt_arena *arena, const blt_local_decoder *decoder, size_t max_seq_len,
+                                          size_t batch_size);
+void blt_kv_cache_destroy(blt_kv_cache *cache);
+void blt_kv_cache_reset(blt_kv_cache *cache);
+void blt_kv_cache_truncate(blt_kv_cache *cache, size_t self_len, size_t num_patches);
+size_t blt_kv_cache_common_patches(const blt_kv_cache *cache, const blt_patch_info *patches, size_t num_patches);
+void blt_kv_cache_refresh_cross(blt_kv_cache *cache, const blt_tensor *patch_in, const blt_patch_info *patches,
+                                size_t num_patches, size_t from_patch, blt_arena *arena);
+void blt_kv_decode_step(blt_kv_cache *cache, const blt_tensor *patch_in, const blt_patch_info *patches,
+                        size_t num_patches, const blt_tensor *d0_rows, int trailing_closed, blt_tensor *logits_out,
+                        blt_arena *arena);
+bool blt_local_cross_attn_fires(blt_xattn_placement placement, bool cross_attn_all_layers, size_t num_layers,
+                                size_t layer);
 
 /* Byte<->patch index helpers; host integer code in the reference as well
  * (csrc/ops/patch_pool.h:29-41, patch_pool_cpu.c:98-142). */
@@ -295,6 +331,25 @@ void blt_kv_decode_layer_hip(const blt_kv_attn_cache *cache, const blt_transform
                              const float *rows_in, float *rows_out, const float *rope_cos, const float *rope_sin,
                              size_t rope_positions, size_t n, int step_kind, int commit, size_t max_len_hint,
                              blt_arena *arena);
+
+/* The decoder step for every sequence of a batched cache at once -- the
+ * decode indexing the reference reserves storage for but does not implement
+ * (csrc/infer/kv_cache.h:71-75).  Sequence b has self_len[b] valid byte rows
+ * (HOST array [batch_size], advanced by n on return; the cache's own scalar
+ * self_len / cross_num_patches are not used), its own patch table patches[b]
+ * of num_patches[b] entries whose sub-tokens refresh_cross_seq has written,
+ * and n = d0_rows->shape[0] / batch_size new rows at d0_rows[b*n .. b*n+n);
+ * trailing_closed may be NULL (all 0).  logits_out is [batch_size*n,
+ * vocab_size].  Every sequence's arithmetic is that of blt_kv_decode_step_hip
+ * on that sequence alone, apart from the projections' summation order once
+ * batch_size*n exceeds 32 rows.  Lengths and row groups are staged through
+ * host memory: not capturable into a graph. */
+void blt_kv_cache_refresh_cross_seq_hip(blt_kv_cache *cache, size_t seq, const blt_tensor *patch_in,
+                                        const blt_patch_info *patches, size_t num_patches, size_t from_patch,
+                                        blt_arena *arena);
+void blt_kv_decode_step_batched_hip(blt_kv_cache *cache, size_t *self_len, const blt_patch_info *const *patches,
+                                    const size_t *num_patches, const int *trailing_closed, const blt_tensor *d0_rows,
+                                    blt_tensor *logits_out, blt_arena *arena);
 
 /* The stream every launch, asynchronous copy and memset of the library goes
  * to, per calling thread: the null stream (the reference's behaviour) unless

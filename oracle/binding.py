@@ -92,6 +92,15 @@ def load_oracle():
                                                                                 _fp, _fp])
     lib.orc_cross_attention_forward.restype = C.c_int
     lib.orc_cross_attention_forward.argtypes = [_fp] * 7 + [C.c_size_t] * 4 + [C.POINTER(abi.BltMaskConfig)]
+    lib.orc_local_cross_attn_fires.restype = C.c_int
+    lib.orc_local_cross_attn_fires.argtypes = [C.c_int, C.c_int, C.c_size_t, C.c_size_t]
+    lib.orc_kv_cache_refresh_cross.restype = C.c_int
+    lib.orc_kv_cache_refresh_cross.argtypes = [C.POINTER(abi.BltKvCache), C.c_size_t, _fp, C.c_size_t, C.c_size_t]
+    lib.orc_kv_cross_block.restype = C.c_int
+    lib.orc_kv_cross_block.argtypes = [_fp, _fp] + [C.c_size_t] * 6 + [abi.c_size_p, C.c_size_t] + [_fp] * 5
+    lib.orc_kv_decode_step.restype = C.c_int
+    lib.orc_kv_decode_step.argtypes = [C.POINTER(abi.BltKvCache), C.c_size_t, C.c_size_t,
+                                       C.POINTER(abi.BltPatchInfo), C.c_size_t, _fp, C.c_size_t, C.c_int, _fp]
     lib.orc_kv_rope_attend_step.restype = C.c_int
     lib.orc_kv_rope_attend_step.argtypes = [_fp, _fp] + [C.c_size_t] * 7 + [_fp, C.c_size_t, _fp, C.c_size_t, _fp,
                                                                            C.c_size_t, _fp, _fp, C.c_size_t, _fp]
@@ -161,6 +170,29 @@ def load_ref():
     lib.blt_cross_attention_forward.restype = None
     lib.blt_cross_attention_forward.argtypes = [T, T, C.POINTER(abi.BltCrossAttentionWeights), T,
                                                 C.POINTER(abi.BltCrossAttentionConfig), C.POINTER(abi.BltArena)]
+    lib.blt_kv_cache_create_batched.restype = C.POINTER(abi.BltKvCache)
+    lib.blt_kv_cache_create_batched.argtypes = [C.POINTER(abi.BltArena), C.POINTER(abi.BltLocalDecoder), C.c_size_t,
+                                                C.c_size_t]
+    lib.blt_kv_cache_destroy.restype = None
+    lib.blt_kv_cache_destroy.argtypes = [C.POINTER(abi.BltKvCache)]
+    lib.blt_kv_cache_truncate.restype = None
+    lib.blt_kv_cache_truncate.argtypes = [C.POINTER(abi.BltKvCache), C.c_size_t, C.c_size_t]
+    lib.blt_kv_cache_common_patches.restype = C.c_size_t
+    lib.blt_kv_cache_common_patches.argtypes = [C.POINTER(abi.BltKvCache), C.POINTER(abi.BltPatchInfo), C.c_size_t]
+    lib.blt_kv_cache_refresh_cross.restype = None
+    lib.blt_kv_cache_refresh_cross.argtypes = [C.POINTER(abi.BltKvCache), T, C.POINTER(abi.BltPatchInfo), C.c_size_t,
+                                               C.c_size_t, C.POINTER(abi.BltArena)]
+    lib.blt_kv_decode_step.restype = None
+    lib.blt_kv_decode_step.argtypes = [C.POINTER(abi.BltKvCache), T, C.POINTER(abi.BltPatchInfo), C.c_size_t, T,
+                                       C.c_int, T, C.POINTER(abi.BltArena)]
+    lib.blt_local_cross_attn_fires.restype = C.c_bool
+    lib.blt_local_cross_attn_fires.argtypes = [C.c_int, C.c_bool, C.c_size_t, C.c_size_t]
+    # blt_local_decoder_forward_ext(model, byte_hidden_in, patch_in, patches, num_patches, bytes_in, targets,
+    #                               doc_boundaries, num_docs, d0_opts, trailing_closed, logits_out, loss_out, arena)
+    lib.blt_local_decoder_forward_ext.restype = None
+    lib.blt_local_decoder_forward_ext.argtypes = [C.POINTER(abi.BltLocalDecoder), T, T, C.POINTER(abi.BltPatchInfo),
+                                                  C.c_size_t, T, T, abi.c_size_p, C.c_size_t, C.c_void_p, C.c_int, T,
+                                                  T, C.POINTER(abi.BltArena)]
     lib.blt_build_block_diffusion_mask.restype = None
     lib.blt_build_block_diffusion_mask.argtypes = [C.POINTER(abi.BltBlockDiffusionConfig),
                                                    C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)]

@@ -598,3 +598,127 @@ int orc_cross_attention_forward(const float *query_in, const float *kv_in, const
     free(q), free(k), free(v), free(combined), free(scores), free(mask);
     return rc;
 }
+
+/* csrc/models/local_common.c:49-64 */
+int orc_local_cross_attn_fires(int placement, int cross_attn_all_layers, size_t num_layers, size_t layer) {
+    switch (placement) {
+    case BLT_XATTN_NONE: return 0;
+    case BLT_XATTN_LAST: return layer + 1 == num_layers;
+    case BLT_XATTN_ALL: return 1;
+    case BLT_XATTN_FIRST: return layer == 0;
+    default: return cross_attn_all_layers || layer + 1 == num_layers;
+    }
+}
+
+/* csrc/infer/kv_cache.c:112-159: K and V of the sub-tokens of patches
+ * [from_patch, num_patches) of sequence `b`, for every layer whose cross block
+ * fires, written in place into the tier-2 slabs. */
+int orc_kv_cache_refresh_cross(blt_kv_cache *cache, size_t b, const float *patch_in, size_t num_patches,
+                               size_t from_patch) {
+    const blt_local_decoder *dec = cache->decoder;
+    const size_t E = cache->embed_dim, L = dec->config.num_layers;
+    if (num_patches < 1 || from_patch >= num_patches || num_patches * cache->k > cache->max_subtokens)
+        return ORC_ERR_ARG;
+    const size_t first = from_patch * cache->k, count = (num_patches - from_patch) * cache->k;
+    for (size_t l = 0; l < L; l++) {
+        if (!orc_local_cross_attn_fires(dec->config.cross_attn_placement, dec->config.cross_attn_all_layers, L, l))
+            continue;
+        const blt_local_layer_storage *s = &dec->layers[l];
+        const size_t row0 = b * cache->max_subtokens + first;
+        orc_matmul(patch_in + first * E, (const float *)s->cross_weight_k.data,
+                   (float *)cache->cross_k[l].data + row0 * E, count, E, E);
+        orc_matmul(patch_in + first * E, (const float *)s->cross_weight_v.data,
+                   (float *)cache->cross_v[l].data + row0 * E, count, E, E);
+    }
+    return ORC_OK;
+}
+
+/* csrc/infer/kv_cache.c:303-341: the cross block in front of a decoder layer
+ * for the n new rows of sequence b: RMSNorm, Q projection, every head over
+ * the total_sub cached sub-tokens under the one-hot group mask
+ * (kv_cache.c:240-251), output projection, residual. */
+int orc_kv_cross_block(const float *cross_k, const float *cross_v, size_t max_subtokens, size_t E, size_t heads,
+                       size_t b, size_t total_sub, size_t k_split, const size_t *q_group, size_t n,
+                       const float *norm_w, const float *wq, const float *wproj, const float *rows_in,
+                       float *rows_out) {
+    const size_t xhd = E / heads;
+    float *normed = (float *)malloc(n * E * sizeof(float));
+    float *q = (float *)malloc(n * E * sizeof(float));
+    float *combined = (float *)calloc(n * E, sizeof(float));
+    float *out = (float *)malloc(n * E * sizeof(float));
+    float *mask = (float *)malloc(n * total_sub * sizeof(float));
+    float *scratch = (float *)malloc(n * total_sub * sizeof(float));
+    for (size_t r = 0; r < n; r++)
+        for (size_t j = 0; j < total_sub; j++) mask[r * total_sub + j] = (j / k_split == q_group[r]) ? 0.0f : -INFINITY;
+    orc_rmsnorm_forward(rows_in, norm_w, normed, n, E);
+    orc_matmul(normed, wq, q, n, E, E);
+    int rc = ORC_OK;
+    for (size_t h = 0; h < heads && rc == ORC_OK; h++) {
+        blt_attention_head_args a;
+        memset(&a, 0, sizeof(a));
+        a.q = q + h * xhd;
+        a.k = cross_k + b * max_subtokens * E + h * xhd;
+        a.v = cross_v + b * max_subtokens * E + h * xhd;
+        a.q_stride = a.k_stride = a.v_stride = E;
+        a.combined = combined;
+        a.combined_stride = E;
+        a.combined_col_offset = h * xhd;
+        a.scores_scratch = scratch;
+        a.mask = mask;
+        a.nq = n;
+        a.nk = total_sub;
+        a.head_dim = xhd;
+        a.scale = 1.0f / sqrtf((float)xhd);
+        rc = orc_attention_head_core(&a);
+    }
+    if (rc == ORC_OK) {
+        orc_matmul(combined, wproj, out, n, E, E);
+        orc_add(rows_in, out, rows_out, n * E);
+    }
+    free(normed), free(q), free(combined), free(out), free(mask), free(scratch);
+    return rc;
+}
+
+/* csrc/infer/kv_cache.c:161-416 for sequence `b` of a (possibly batched)
+ * cache whose valid length is `base`: group of every new row by the decoder
+ * latent rule (199-213), then per layer the cross block where it fires and the
+ * self-attention / feed-forward layer, then the LM head.  The caller advances
+ * the sequence's length. */
+int orc_kv_decode_step(blt_kv_cache *cache, size_t b, size_t base, const blt_patch_info *patches,
+                       size_t num_patches, const float *d0_rows, size_t n, int trailing_closed,
+                       float *logits_out) {
+    const blt_local_decoder *dec = cache->decoder;
+    const blt_local_decoder_config *cfg = &dec->config;
+    const size_t E = cache->embed_dim, L = cfg->num_layers, H = cfg->num_heads, XH = cfg->cross_attn_heads;
+    if (n < 1 || num_patches < 1) return ORC_ERR_ARG;
+    if (base + n > cache->max_seq_len || num_patches * cache->k > cache->max_subtokens) return ORC_ERR_CAPACITY;
+    size_t *q_group = (size_t *)malloc(n * sizeof(size_t));
+    for (size_t r = 0; r < n; r++) q_group[r] = orc_patch_decoder_latent_at(patches, num_patches, base + r);
+    if (trailing_closed) q_group[n - 1] = num_patches - 1;
+    float *cur = (float *)malloc(n * E * sizeof(float));
+    float *mid = (float *)malloc(n * E * sizeof(float));
+    memcpy(cur, d0_rows, n * E * sizeof(float));
+    int rc = ORC_OK;
+    for (size_t l = 0; l < L && rc == ORC_OK; l++) {
+        const blt_local_layer_storage *s = &dec->layers[l];
+        const float *in = cur;
+        if (orc_local_cross_attn_fires(cfg->cross_attn_placement, cfg->cross_attn_all_layers, L, l)) {
+            rc = orc_kv_cross_block((const float *)cache->cross_k[l].data, (const float *)cache->cross_v[l].data,
+                                    cache->max_subtokens, E, XH, b, num_patches * cache->k, cache->k, q_group, n,
+                                    (const float *)s->cross_norm_weight.data, (const float *)s->cross_weight_q.data,
+                                    (const float *)s->cross_weight_proj.data, cur, mid);
+            in = mid;
+        }
+        if (rc != ORC_OK) break;
+        rc = orc_kv_decode_layer((float *)cache->self_k[l].data, (float *)cache->self_v[l].data, cache->max_seq_len,
+                                 E, H, b, base, n, cfg->local_window, (const float *)s->norm1_weight.data,
+                                 (const float *)s->attn_qkv_w.data, (const float *)s->attn_proj_w.data,
+                                 (const float *)s->norm2_weight.data, (const float *)s->ffn_up_w.data,
+                                 (const float *)s->ffn_gate_w.data, (const float *)s->ffn_down_w.data,
+                                 s->ffn_up_w.shape[1], (const float *)dec->rope_cos_cache.data,
+                                 (const float *)dec->rope_sin_cache.data, dec->rope_cos_cache.shape[0], in, cur);
+    }
+    if (rc == ORC_OK) orc_matmul(cur, (const float *)dec->lm_head_weight.data, logits_out, n, E, cfg->vocab_size);
+    free(q_group), free(cur), free(mid);
+    return rc;
+}

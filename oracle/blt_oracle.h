@@ -43,6 +43,14 @@
  *       preserved, q.k after rotation depends only on the position
  *       difference; the step against rotating by hand and calling
  *       orc_kv_attend_step.
+ *   orc_kv_cache_refresh_cross, orc_kv_cross_block, orc_kv_decode_step
+ *       bit-for-bit (logits and all four cache tiers) against oracle/_ref's
+ *       blt_kv_cache_refresh_cross and blt_kv_decode_step (csrc/infer/
+ *       kv_cache.c) over prefill chunks and single-row steps, with and
+ *       without window, sub-token split and trailing_closed; and through the
+ *       reference's own invariant that the cached steps reproduce the dense
+ *       decoder forward (tests/unit/infer/unit_kv_cache.c:136-151), here
+ *       blt_local_decoder_forward of oracle/_ref.
  *   orc_matmul, orc_rope_apply_packed, orc_multihead_attention,
  *   orc_cross_attention_forward
  *       bit-for-bit against oracle/_ref (blt_matmul, blt_rope_apply_packed,
@@ -207,6 +215,30 @@ int orc_kv_decode_layer(float *self_k, float *self_v, size_t max_seq_len, size_t
                         const float *proj_w, const float *norm2_w, const float *up_w, const float *gate_w,
                         const float *down_w, size_t hidden, const float *cos_cache, const float *sin_cache,
                         size_t cache_rows, const float *rows_in, float *rows_out);
+
+/* models/local_common.c:49-64 */
+int orc_local_cross_attn_fires(int placement, int cross_attn_all_layers, size_t num_layers, size_t layer);
+
+/* infer/kv_cache.c:112-159 for sequence b of a host cache: K / V of the
+ * sub-tokens of patches [from_patch, num_patches) into the tier-2 slabs of
+ * every layer whose cross block fires.  patch_in is [num_patches*k, E]. */
+int orc_kv_cache_refresh_cross(blt_kv_cache *cache, size_t b, const float *patch_in, size_t num_patches,
+                               size_t from_patch);
+
+/* infer/kv_cache.c:303-341 (mask 240-251): the cross block of a decoder layer
+ * for the n new rows of sequence b; q_group[r] is the latent patch of row r,
+ * sub-token j belongs to patch j / k_split. */
+int orc_kv_cross_block(const float *cross_k, const float *cross_v, size_t max_subtokens, size_t E, size_t heads,
+                       size_t b, size_t total_sub, size_t k_split, const size_t *q_group, size_t n,
+                       const float *norm_w, const float *wq, const float *wproj, const float *rows_in,
+                       float *rows_out);
+
+/* infer/kv_cache.c:161-416: the whole incremental decoder step for the n new
+ * rows of sequence b (valid length `base`) of a host cache, LM head included.
+ * Does not advance any length. */
+int orc_kv_decode_step(blt_kv_cache *cache, size_t b, size_t base, const blt_patch_info *patches,
+                       size_t num_patches, const float *d0_rows, size_t n, int trailing_closed,
+                       float *logits_out);
 
 #ifdef __cplusplus
 }

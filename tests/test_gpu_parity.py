@@ -794,6 +794,168 @@ def test_kv_decode_layer(batch, n, H, hd, hidden, kind, oracle, dev):
 # ---------------------------------------------------------------------------
 # streams and graphs
 # ---------------------------------------------------------------------------
+# ---------------------------------------------------------------------------
+# the whole incremental decoder step on the device (csrc/infer/kv_cache.c:112-416)
+# ---------------------------------------------------------------------------
+STEP_CASES = [
+    dict(E=16, H=2, XH=2, L=2, hidden=24, V=19, max_len=40, k=1, window=0, all_layers=True, placement=0),
+    dict(E=24, H=3, XH=2, L=3, hidden=40, V=256, max_len=48, k=2, window=7, all_layers=False, placement=0),
+    dict(E=128, H=4, XH=4, L=2, hidden=512, V=256, max_len=64, k=1, window=0, all_layers=True, placement=0),
+    dict(E=64, H=2, XH=4, L=2, hidden=96, V=50, max_len=32, k=3, window=5, all_layers=False, placement=4),
+]
+
+
+def _decoders(oracle, c, seed):
+    """The same seeded decoder twice: over numpy arrays for the checker, over device copies for the library."""
+    from fblt_amd import decoder
+    hd, half = c["E"] // c["H"], c["E"] // c["H"] // 2
+    cos, sin = (np.empty(c["max_len"] * half, dtype=np.float32) for _ in range(2))
+    assert oracle.orc_rope_precompute(c["max_len"], 500000.0, hd, binding.fptr(cos), binding.fptr(sin)) == 0
+    w = decoder.random_weights(c["E"], c["hidden"], c["L"], c["V"], seed)
+    args = (c["E"], c["H"], c["XH"], c["hidden"], c["V"], c["max_len"])
+    kw = dict(patch_dim=c["k"] * c["E"], window=c["window"], all_layers=c["all_layers"], placement=c["placement"])
+    tables = (cos.reshape(c["max_len"], half), sin.reshape(c["max_len"], half))
+    host = decoder.bind(w, *tables, abi.BLT_BACKEND_CPU, decoder.host_place, *args, **kw)
+    device = decoder.bind(w, *tables, abi.BLT_BACKEND_HIP, decoder.device_place, *args, **kw)
+    return host, device
+
+
+def _tier(lib, cache, name, layer, rows, E):
+    out = np.empty((rows, E), dtype=np.float32)
+    lib.blt_hip_memcpy_d2h(out.ctypes.data, getattr(cache.contents, name)[layer].data, out.nbytes)
+    return out
+
+
+@pytest.mark.parametrize("case", range(len(STEP_CASES)))
+def test_kv_decode_step_single_sequence(case, oracle, dev):
+    """blt_kv_cache_refresh_cross + blt_kv_decode_step on device memory against the restated step:
+    prefill chunk, single rows, re-segmentation; logits and all four cache tiers after every call."""
+    import torch
+    from fblt_amd import decoder
+    lib = api.load()
+    c = STEP_CASES[case]
+    E, V, k, L = c["E"], c["V"], c["k"], c["L"]
+    rs = np.random.RandomState(300 + case)
+    host, device = _decoders(oracle, c, 400 + case)
+    mine = decoder.HostCache(host, c["max_len"])
+    arena = lib.blt_arena_create(64 << 20, abi.BLT_BACKEND_HIP)
+    try:
+        cache = lib.blt_kv_cache_create(arena, device.ptr, c["max_len"])
+        assert cache.contents.k == k and cache.contents.max_subtokens == c["max_len"]
+        mark = arena.contents.offset
+        d0_all = rs.randn(21, E).astype(np.float32)
+        script = [([3, 4], 0, 7, 0), ([3, 4, 1], 2, 1, 0), ([3, 4, 2], 2, 1, 1), ([3, 4, 2, 5], 3, 5, 0),
+                  ([3, 4, 2, 5, 1], 4, 1, 0), ([3, 4, 2, 5, 4], 4, 3, 1), ([3, 4, 2, 5, 4, 3], 5, 3, 0)]
+        done, prev = 0, None
+        for lengths, from_patch, n, closed in script:
+            P = len(lengths)
+            patches = decoder.patch_table(lengths)
+            patch_in = rs.randn(P, k * E).astype(np.float32)
+            if from_patch:
+                patch_in[:from_patch] = prev[:from_patch]
+            prev = patch_in
+            same = lib.blt_kv_cache_common_patches(cache, patches, P)
+            assert same == from_patch
+            lib.blt_kv_cache_truncate(cache, cache.contents.self_len, min(from_patch, cache.contents.cross_num_patches))
+            tp = torch.from_numpy(patch_in).cuda()
+            vp = _dev_tensor(tp)
+            arena.contents.offset = mark
+            lib.blt_kv_cache_refresh_cross(cache, C.byref(vp), patches, P, from_patch, arena)
+            assert cache.contents.cross_num_patches == P
+            assert oracle.orc_kv_cache_refresh_cross(mine.ptr, 0, binding.fptr(patch_in.reshape(-1)), P, from_patch) == 0
+            rows = np.ascontiguousarray(d0_all[done:done + n])
+            ref = np.zeros((n, V), dtype=np.float32)
+            assert oracle.orc_kv_decode_step(mine.ptr, 0, done, patches, P, binding.fptr(rows.reshape(-1)), n, closed,
+                                             binding.fptr(ref.reshape(-1))) == 0
+            td = torch.from_numpy(rows).cuda()
+            tl = torch.full((n, V), 7.0, dtype=torch.float32, device="cuda")
+            vd, vl = _dev_tensor(td), _dev_tensor(tl)
+            lib.blt_kv_decode_step(cache, C.byref(vp), patches, P, C.byref(vd), closed, C.byref(vl), arena)
+            lib.blt_backend_pass_sync_hip()
+            done += n
+            assert cache.contents.self_len == done
+            assert_close(tl.cpu().numpy(), ref, "decode step logits case %d %s" % (case, lengths))
+            for name in ("self_k", "self_v", "cross_k", "cross_v"):
+                for l in range(L):
+                    assert_close(_tier(lib, cache, name, l, c["max_len"], E), mine.tiers[name][l],
+                                 "%s[%d] case %d %s" % (name, l, case, lengths))
+        lib.blt_kv_cache_reset(cache)
+        assert cache.contents.self_len == 0 and cache.contents.cross_num_patches == 0
+        lib.blt_kv_cache_destroy(cache)
+    finally:
+        lib.blt_arena_destroy(arena)
+
+
+@pytest.mark.parametrize("batch,n,case", [(8, 1, 0), (64, 1, 2), (16, 4, 1), (5, 3, 3), (64, 8, 2)])
+def test_kv_decode_step_batched(batch, n, case, oracle, dev):
+    """blt_kv_decode_step_batched_hip: every sequence of a batched cache in one pass, against the
+    restated step run sequence by sequence; two steps in a row."""
+    import torch
+    from fblt_amd import decoder
+    lib = api.load()
+    c = STEP_CASES[case]
+    E, V, k, L, max_len = c["E"], c["V"], c["k"], c["L"], c["max_len"]
+    rs = np.random.RandomState(500 + batch + n)
+    host, device = _decoders(oracle, c, 600 + case)
+    mine = decoder.HostCache(host, max_len, batch)
+    arena = lib.blt_arena_create(256 << 20, abi.BLT_BACKEND_HIP)
+    try:
+        cache = lib.blt_kv_cache_create_batched(arena, device.ptr, max_len, batch)
+        mark = arena.contents.offset
+        lens = rs.randint(1, max_len - 2 * n, size=batch)
+        tables, counts, keep_in = [], [], []
+        for b in range(batch):
+            # patches tile the decoded bytes plus the rows of both steps
+            total = int(lens[b]) + 2 * n
+            cuts = np.sort(rs.choice(np.arange(1, total), size=min(total - 1, rs.randint(1, 6)), replace=False))
+            lengths = np.diff(np.concatenate([[0], cuts, [total]])).tolist()
+            tables.append(decoder.patch_table(lengths))
+            counts.append(len(lengths))
+            patch_in = rs.randn(len(lengths), k * E).astype(np.float32)
+            tp = torch.from_numpy(patch_in).cuda()
+            vp = _dev_tensor(tp)
+            keep_in.append(tp)
+            lib.blt_kv_cache_refresh_cross_seq_hip(cache, b, C.byref(vp), tables[b], counts[b], 0, arena)
+            assert oracle.orc_kv_cache_refresh_cross(mine.ptr, b, binding.fptr(patch_in.reshape(-1)), counts[b], 0) == 0
+        # valid tier-1 rows: the same random content on both sides
+        for name in ("self_k", "self_v"):
+            for l in range(L):
+                slab = mine.tiers[name][l]
+                for b in range(batch):
+                    slab[b * max_len:b * max_len + lens[b]] = rs.randn(int(lens[b]), E).astype(np.float32)
+                lib.blt_hip_memcpy_h2d(getattr(cache.contents, name)[l].data, slab.ctypes.data, slab.nbytes)
+        lib.blt_backend_pass_sync_hip()
+        self_len = abi.size_array(lens.tolist())
+        table_ptrs = (C.POINTER(abi.BltPatchInfo) * batch)(*(C.cast(t, C.POINTER(abi.BltPatchInfo)) for t in tables))
+        num = abi.size_array(counts)
+        for step in range(2):
+            closed = (C.c_int * batch)(*([0] * batch if step == 0 else rs.randint(0, 2, size=batch).tolist()))
+            rows = rs.randn(batch * n, E).astype(np.float32)
+            ref = np.zeros((batch * n, V), dtype=np.float32)
+            for b in range(batch):
+                r = np.ascontiguousarray(rows[b * n:(b + 1) * n])
+                out = np.zeros((n, V), dtype=np.float32)
+                assert oracle.orc_kv_decode_step(mine.ptr, b, int(lens[b]) + step * n, tables[b], counts[b],
+                                                 binding.fptr(r.reshape(-1)), n, closed[b],
+                                                 binding.fptr(out.reshape(-1))) == 0
+                ref[b * n:(b + 1) * n] = out
+            td = torch.from_numpy(rows).cuda()
+            tl = torch.full((batch * n, V), 7.0, dtype=torch.float32, device="cuda")
+            vd, vl = _dev_tensor(td), _dev_tensor(tl)
+            arena.contents.offset = mark
+            lib.blt_kv_decode_step_batched_hip(cache, self_len, table_ptrs, num, closed, C.byref(vd), C.byref(vl), arena)
+            lib.blt_backend_pass_sync_hip()
+            assert [self_len[b] for b in range(batch)] == (lens + (step + 1) * n).tolist()
+            assert_close(tl.cpu().numpy(), ref, "batched step %d logits" % step)
+            for name in ("self_k", "self_v", "cross_k", "cross_v"):
+                for l in range(L):
+                    assert_close(_tier(lib, cache, name, l, batch * max_len, E), mine.tiers[name][l],
+                                 "%s[%d] batched step %d" % (name, l, step))
+        lib.blt_kv_cache_destroy(cache)
+    finally:
+        lib.blt_arena_destroy(arena)
+
+
 def test_graph_replay_of_a_plan_and_a_decode_layer(oracle, dev):
     """Library launches recorded into a HIP graph: every replay, with eager work and
     synchronisations in between, gives the eager result."""

@@ -41,6 +41,61 @@ def test_header_layout_assertions_compile():
         assert p.returncode == 0, p.stderr
 
 
+LAYOUT_PROBE = r"""
+#include <stdio.h>
+#include <stddef.h>
+%s
+#define S(t) printf(#t " %%zu\n", sizeof(t))
+#define O(t, f) printf(#t "." #f " %%zu\n", offsetof(t, f))
+int main(void) {
+    S(blt_tensor); O(blt_tensor, strides); O(blt_tensor, dtype); O(blt_tensor, is_view); S(blt_arena);
+    S(blt_attention_head_args); O(blt_attention_head_args, combined_col_offset); O(blt_attention_head_args, lse_out);
+    O(blt_attention_head_args, mask); O(blt_attention_head_args, is_causal); O(blt_attention_head_args, scale);
+    S(blt_mask_config); O(blt_mask_config, doc_boundaries); O(blt_mask_config, kv_group_ids);
+    O(blt_mask_config, is_causal); O(blt_mask_config, causal_offset);
+    S(blt_block_diffusion_config); S(blt_patch_info); O(blt_patch_info, peak_entropy);
+    S(blt_rope_config); S(blt_attention_config); O(blt_attention_config, use_rope); O(blt_attention_config, rope_theta);
+    O(blt_attention_config, mask_config);
+    S(blt_cross_attention_config); O(blt_cross_attention_config, split_mode); O(blt_cross_attention_config, num_heads);
+    O(blt_cross_attention_config, mask_config); S(blt_cross_attention_weights); O(blt_cross_attention_weights, weight_proj);
+    S(blt_transformer_weights); O(blt_transformer_weights, ffn_gate_w);
+    S(blt_local_layer_storage); O(blt_local_layer_storage, cross_norm_weight); O(blt_local_layer_storage, cross_weight_proj);
+    S(blt_local_decoder_config); O(blt_local_decoder_config, cross_attn_all_layers);
+    O(blt_local_decoder_config, cross_attn_placement); O(blt_local_decoder_config, rope_theta);
+    O(blt_local_decoder_config, max_seq_len); O(blt_local_decoder_config, vocab_size);
+    S(blt_local_decoder); O(blt_local_decoder, rope_sin_cache); O(blt_local_decoder, layers);
+    O(blt_local_decoder, lm_head_weight); O(blt_local_decoder, d0_embed_weight);
+    S(blt_kv_cache); O(blt_kv_cache, k); O(blt_kv_cache, self_k); O(blt_kv_cache, self_len); O(blt_kv_cache, cross_k);
+    O(blt_kv_cache, cross_num_patches); O(blt_kv_cache, cached_patches);
+    printf("enum %%d %%d %%d %%d\n", (int)BLT_XATTN_FIRST, (int)BLT_DTYPE_FP32, (int)BLT_BACKEND_CPU,
+           (int)BLT_CROSS_ATTN_SPLIT_KV);
+    return 0;
+}
+"""
+
+REF_ROOT = "/root/reference/csrc"
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_ROOT), reason="the reference headers are not on this machine")
+def test_layout_matches_reference_headers(tmp_path):
+    """Sizes and member offsets of every mirrored struct, printed once by a program compiled against
+    the reference's own headers and once against include/blt_abi.h, must read the same."""
+    ref_inc = "\n".join('#include "%s"' % h for h in (
+        "core/tensor.h", "core/allocator.h", "ops/attn_core.h", "ops/mask_builder.h", "ops/rope.h",
+        "models/attention.h", "models/cross_attention.h", "models/transformer.h", "models/patcher.h",
+        "models/local_decoder.h", "infer/kv_cache.h"))
+    outs = []
+    for tag, inc_dir, inc in (("ref", REF_ROOT, ref_inc), ("own", os.path.join(ROOT, "include"), '#include "blt_abi.h"')):
+        src = tmp_path / (tag + ".c")
+        src.write_text(LAYOUT_PROBE % inc)
+        exe = str(tmp_path / tag)
+        p = subprocess.run(["gcc", "-std=c99", "-D_POSIX_C_SOURCE=200809L", "-I", inc_dir, str(src), "-o", exe],
+                           capture_output=True, text=True)
+        assert p.returncode == 0, p.stderr
+        outs.append(subprocess.run([exe], capture_output=True, text=True, check=True).stdout)
+    assert outs[0] == outs[1] and outs[0].count("\n") > 50
+
+
 def test_patch_helpers_match_checker(oracle):
     lib = api.load()
     rs = np.random.RandomState(21)

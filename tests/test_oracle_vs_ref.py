@@ -378,3 +378,114 @@ def test_row_ops_bit_exact(oracle, ref):
             ty, to = abi.tensor_view(y.ctypes.data, y.shape, CPU), abi.tensor_view(theirs.ctypes.data, theirs.shape, CPU)
             ref_fn(C.byref(tx), C.byref(ty), C.byref(to))
             assert mine.tobytes() == theirs.tobytes()
+
+
+# ---------------------------------------------------------------------------
+# the whole incremental decoder step (csrc/infer/kv_cache.c:112-416)
+# ---------------------------------------------------------------------------
+DECODER_CASES = [
+    # E, H, XH, L, hidden, V, max_len, k_split, window, all_layers, placement
+    dict(E=16, H=2, XH=2, L=2, hidden=24, V=19, max_len=40, k=1, window=0, all_layers=True, placement=0),
+    dict(E=24, H=3, XH=2, L=3, hidden=40, V=256, max_len=48, k=2, window=7, all_layers=False, placement=0),
+    dict(E=16, H=4, XH=1, L=2, hidden=16, V=11, max_len=32, k=1, window=0, all_layers=False, placement=4),  # FIRST
+    dict(E=16, H=2, XH=4, L=2, hidden=16, V=11, max_len=32, k=3, window=5, all_layers=True, placement=1),   # NONE
+]
+
+
+def _host_decoder(oracle, c, seed):
+    from fblt_amd import decoder
+    hd, half = c["E"] // c["H"], c["E"] // c["H"] // 2
+    cos, sin = (np.empty(c["max_len"] * half, dtype=np.float32) for _ in range(2))
+    assert oracle.orc_rope_precompute(c["max_len"], 500000.0, hd, binding.fptr(cos), binding.fptr(sin)) == 0
+    w = decoder.random_weights(c["E"], c["hidden"], c["L"], c["V"], seed)
+    bound = decoder.bind(w, cos.reshape(c["max_len"], half), sin.reshape(c["max_len"], half), CPU, decoder.host_place,
+                         c["E"], c["H"], c["XH"], c["hidden"], c["V"], c["max_len"], patch_dim=c["k"] * c["E"],
+                         window=c["window"], all_layers=c["all_layers"], placement=c["placement"])
+    return bound
+
+
+@pytest.mark.parametrize("case", range(len(DECODER_CASES)))
+def test_kv_decode_step_bit_exact(case, oracle, ref):
+    """orc_kv_cache_refresh_cross + orc_kv_decode_step against blt_kv_cache_refresh_cross +
+    blt_kv_decode_step compiled from the reference, over a prefill chunk, single-row steps and a
+    re-segmentation (truncate to the common patches, refresh, decode again): logits and all four
+    cache tiers bit for bit; then the reference's own invariant -- the cached steps give the dense
+    decoder forward's logits (tests/unit/infer/unit_kv_cache.c:136-151)."""
+    from fblt_amd import decoder
+    c = DECODER_CASES[case]
+    E, V, k = c["E"], c["V"], c["k"]
+    rs = np.random.RandomState(100 + case)
+    bound = _host_decoder(oracle, c, 200 + case)
+    assert all(bool(ref.blt_local_cross_attn_fires(c["placement"], c["all_layers"], c["L"], l)) ==
+               bool(oracle.orc_local_cross_attn_fires(c["placement"], int(c["all_layers"]), c["L"], l))
+               for l in range(c["L"]))
+    mine = decoder.HostCache(bound, c["max_len"])
+    arena = ref.blt_arena_create(64 << 20, CPU)
+    try:
+        theirs = ref.blt_kv_cache_create_batched(arena, bound.ptr, c["max_len"], 1)
+        mark = arena.contents.offset
+        total_bytes = 21
+        d0_all = rs.randn(total_bytes, E).astype(np.float32)
+        # (patch lengths so far, from_patch for the refresh, rows to decode, trailing_closed)
+        script = [([3, 4], 0, 7, 0), ([3, 4, 1], 2, 1, 0), ([3, 4, 2], 2, 1, 1), ([3, 4, 2, 5], 3, 5, 0),
+                  ([3, 4, 2, 5, 1], 4, 1, 0), ([3, 4, 2, 5, 4], 4, 3, 1), ([3, 4, 2, 5, 4, 3], 5, 3, 0)]
+        done = 0
+        all_logits = []
+        for lengths, from_patch, n, closed in script:
+            P = len(lengths)
+            patches = decoder.patch_table(lengths)
+            patch_in = rs.randn(P, k * E).astype(np.float32)
+            if from_patch:   # rows of completed patches do not change (append-only tier 2)
+                patch_in[:from_patch] = prev_patch_in[:from_patch]
+            prev_patch_in = patch_in
+            tp = abi.tensor_view(patch_in.ctypes.data, patch_in.shape, CPU)
+            same = ref.blt_kv_cache_common_patches(theirs, patches, P)
+            assert same >= min(from_patch, theirs.contents.cross_num_patches)
+            ref.blt_kv_cache_truncate(theirs, theirs.contents.self_len, min(from_patch, theirs.contents.cross_num_patches))
+            ref.blt_kv_cache_refresh_cross(theirs, C.byref(tp), patches, P, from_patch, arena)
+            assert oracle.orc_kv_cache_refresh_cross(mine.ptr, 0, binding.fptr(patch_in.reshape(-1)), P,
+                                                     from_patch) == 0
+            rows = np.ascontiguousarray(d0_all[done:done + n])
+            got, want = np.zeros((n, V), dtype=np.float32), np.zeros((n, V), dtype=np.float32)
+            td, tl = abi.tensor_view(rows.ctypes.data, rows.shape, CPU), abi.tensor_view(want.ctypes.data, want.shape, CPU)
+            arena.contents.offset = mark
+            ref.blt_kv_decode_step(theirs, C.byref(tp), patches, P, C.byref(td), closed, C.byref(tl), arena)
+            assert oracle.orc_kv_decode_step(mine.ptr, 0, done, patches, P, binding.fptr(rows.reshape(-1)), n, closed,
+                                             binding.fptr(got.reshape(-1))) == 0
+            assert got.tobytes() == want.tobytes(), (case, lengths, n)
+            done += n
+            assert theirs.contents.self_len == done
+            for name in ("self_k", "self_v", "cross_k", "cross_v"):
+                for l in range(c["L"]):
+                    t = getattr(theirs.contents, name)[l]
+                    view = np.ctypeslib.as_array(C.cast(t.data, C.POINTER(C.c_float)), shape=(c["max_len"], E))
+                    assert view.tobytes() == mine.tiers[name][l].tobytes(), (name, l, lengths)
+            all_logits.append((done - n, closed, got))
+        assert done == total_bytes
+        ref.blt_kv_cache_destroy(theirs)
+        # the reference's invariant: with the segmentation known up front, decoding in chunks gives
+        # the dense forward's logits bit for bit, whatever the chunking
+        lengths = script[-1][0]
+        P = len(lengths)
+        patches = decoder.patch_table(lengths)
+        th = abi.tensor_view(d0_all.ctypes.data, d0_all.shape, CPU)
+        tp = abi.tensor_view(prev_patch_in.ctypes.data, prev_patch_in.shape, CPU)
+        for closed, chunks in ((0, (4, 1, 1, 6, 9)), (1, (21,)), (1, (1,) * 21), (0, (10, 11))):
+            dense = np.zeros((total_bytes, V), dtype=np.float32)
+            tl = abi.tensor_view(dense.ctypes.data, dense.shape, CPU)
+            arena.contents.offset = mark
+            ref.blt_local_decoder_forward_ext(bound.ptr, C.byref(th), C.byref(tp), patches, P, None, None, None, 0,
+                                              None, closed, C.byref(tl), None, arena)
+            fresh = decoder.HostCache(bound, c["max_len"])
+            assert oracle.orc_kv_cache_refresh_cross(fresh.ptr, 0, binding.fptr(prev_patch_in.reshape(-1)), P, 0) == 0
+            at = 0
+            for n in chunks:
+                rows = np.ascontiguousarray(d0_all[at:at + n])
+                got = np.zeros((n, V), dtype=np.float32)
+                last = at + n == total_bytes
+                assert oracle.orc_kv_decode_step(fresh.ptr, 0, at, patches, P, binding.fptr(rows.reshape(-1)), n,
+                                                 closed if last else 0, binding.fptr(got.reshape(-1))) == 0
+                assert got.tobytes() == dense[at:at + n].tobytes(), (case, closed, chunks, at)
+                at += n
+    finally:
+        ref.blt_arena_destroy(arena)
