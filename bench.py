@@ -406,6 +406,132 @@ def cpu_decode_layer(budget_s, batch=64, H=4, hd=32, hidden=512, len_hi=512):
             "sample": "%d layer steps of %d sequences, %.1f s" % (steps, batch, spent)}
 
 
+def _decode_step_setup(batch, L, E, H, hidden, V, len_hi, total_steps, seed=17):
+    """Seeded decoder weights, per-sequence lengths and patch tables (4 bytes per patch) of the
+    batched decoder-step workload."""
+    import numpy as np
+    from fblt_amd import decoder, synth
+    max_len = len_hi + total_steps + 8
+    max_len += (-max_len) % 4
+    lens = synth.integers(synth.seed_for(4, synth.S_LEN), batch, 1, len_hi).astype(np.int64)
+    weights = decoder.random_weights(E, hidden, L, V, seed)
+    tables = [decoder.patch_table([4] * (max_len // 4)) for _ in range(batch)]
+    return max_len, lens, weights, tables
+
+
+def bench_decode_step(steps, warmup, batch=64, L=2, E=128, H=4, hidden=512, V=256, len_hi=512):
+    """blt_kv_decode_step_batched_hip: the whole incremental decoder step (per layer the cross block
+    over the tier-2 cache and the self-attention / feed-forward layer, then the LM head) for `batch`
+    sequences, one new row each, per step."""
+    import ctypes as C
+    import numpy as np
+    import torch
+    from fblt_amd import abi, api, decoder
+    lib = api.load()
+    hd, half = E // H, E // H // 2
+    max_len, lens, weights, tables = _decode_step_setup(batch, L, E, H, hidden, V, len_hi, 2 * (warmup + steps))
+    view = lambda t: abi.tensor_view(t.data_ptr(), tuple(t.shape), abi.BLT_BACKEND_HIP)
+    cos, sin = torch.zeros((max_len, half), device="cuda"), torch.zeros((max_len, half), device="cuda")
+    vc, vs = view(cos), view(sin)
+    rcfg = abi.BltRopeConfig(500000.0, hd)
+    lib.blt_rope_precompute(max_len, C.byref(rcfg), C.byref(vc), C.byref(vs))
+    bound = decoder.bind(weights, cos.cpu().numpy(), sin.cpu().numpy(), abi.BLT_BACKEND_HIP, decoder.device_place,
+                         E, H, H, hidden, V, max_len)
+    arena = lib.blt_arena_create(1 << 30, abi.BLT_BACKEND_HIP)
+    cache = lib.blt_kv_cache_create_batched(arena, bound.ptr, max_len, batch)
+    g = torch.Generator(device="cpu").manual_seed(7)
+    P = max_len // 4
+    for l in range(L):   # cached rows: random content, as after a prefill
+        for name in ("self_k", "self_v"):
+            t = torch.randn(batch * max_len, E, generator=g, dtype=torch.float32)
+            lib.blt_hip_memcpy_h2d(getattr(cache.contents, name)[l].data, t.data_ptr(), t.numel() * 4)
+            lib.blt_backend_pass_sync_hip()
+    for b in range(batch):
+        pin = torch.randn(P, E, generator=g, dtype=torch.float32).cuda()
+        vp = view(pin)
+        lib.blt_kv_cache_refresh_cross_seq_hip(cache, b, C.byref(vp), tables[b], P, 0, arena)
+    lib.blt_backend_pass_sync_hip()
+    mark = arena.contents.offset
+    table_ptrs = (C.POINTER(abi.BltPatchInfo) * batch)(*(C.cast(t, C.POINTER(abi.BltPatchInfo)) for t in tables))
+    num = abi.size_array([P] * batch)
+    x = torch.randn(batch, E, generator=g, dtype=torch.float32).cuda()
+    logits = torch.zeros((batch, V), device="cuda")
+    vx, vl = view(x), view(logits)
+    self_len = abi.size_array(lens.tolist())
+
+    def run(count):
+        for _ in range(count):
+            arena.contents.offset = mark
+            lib.blt_kv_decode_step_batched_hip(cache, self_len, table_ptrs, num, None, C.byref(vx), C.byref(vl), arena)
+    run(warmup)
+    lib.blt_backend_pass_sync_hip()
+    lib.blt_hip_profile_begin()
+    t0 = time.perf_counter()
+    run(steps)
+    lib.blt_backend_pass_sync_hip()
+    wall = time.perf_counter() - t0
+    prof = api.profile_end()
+    run(warmup)
+    lib.blt_backend_pass_sync_hip()
+    t0 = time.perf_counter()
+    run(steps)
+    lib.blt_backend_pass_sync_hip()
+    wall_plain = time.perf_counter() - t0
+    lib.blt_kv_cache_destroy(cache)
+    lib.blt_arena_destroy(arena)
+    avg_s = sum(v[1] for v in prof.values()) / 1e3 / steps
+    mean_keys = float(lens.sum()) + batch * (warmup + (steps - 1) / 2.0) + batch
+    per_layer_w = E * E * 2 + E * 3 * E + E * E + 3 * E * hidden   # cross q / proj, qkv, proj, up / gate / down
+    flops = L * (batch * 2.0 * per_layer_w + 4.0 * hd * H * mean_keys + 4.0 * E * batch) + batch * 2.0 * E * V
+    nbytes = 4.0 * (L * (2 * E * mean_keys + per_layer_w + 2 * E * batch) + E * V)
+    res = {"workload": "decoder step: %d sequences, %d layers (cross block in each), E=%d, H=%d, hidden=%d, V=%d, "
+                       "cached 1..%d" % (batch, L, E, H, hidden, V, len_hi),
+           "kernel": "+".join(sorted(prof)), "launches_per_step": sum(v[0] for v in prof.values()) / steps,
+           "tokens_per_step": batch, "us_per_step": wall_plain / steps * 1e6,
+           "us_per_step_with_events": wall / steps * 1e6, "kernel_us_avg": avg_s * 1e6,
+           "kernel_us_min": min(v[2] for v in prof.values()) * 1e3,
+           "per_kernel_us": {k: v[1] * 1e3 / steps for k, v in prof.items()},
+           "tokens_per_s": batch * steps / wall_plain, "tokens_per_s_kernel": batch / avg_s, "flops": flops,
+           "bytes": nbytes, "roofline_hbm": roofline("hbm", nbytes, avg_s), "roofline_mfma": roofline("mfma", flops, avg_s)}
+    res["roofline"] = res["roofline_hbm"]
+    return res
+
+
+def cpu_decode_step(budget_s, batch=64, L=2, E=128, H=4, hidden=512, V=256, len_hi=512):
+    """The restated decoder step on one host core, one sequence at a time as the reference runs it."""
+    import numpy as np
+    from fblt_amd import abi, decoder
+    from oracle import binding
+    lib = binding.load_oracle()
+    hd, half = E // H, E // H // 2
+    max_len, lens, weights, tables = _decode_step_setup(batch, L, E, H, hidden, V, len_hi, 40)
+    cos, sin = np.empty(max_len * half, dtype=np.float32), np.empty(max_len * half, dtype=np.float32)
+    lib.orc_rope_precompute(max_len, 500000.0, hd, binding.fptr(cos), binding.fptr(sin))
+    bound = decoder.bind(weights, cos.reshape(max_len, half), sin.reshape(max_len, half), abi.BLT_BACKEND_CPU,
+                         decoder.host_place, E, H, H, hidden, V, max_len)
+    cache = decoder.HostCache(bound, max_len, batch)
+    rs = np.random.RandomState(3)
+    P = max_len // 4
+    for name in ("self_k", "self_v"):
+        for l in range(L):
+            cache.tiers[name][l][:] = rs.randn(batch * max_len, E).astype(np.float32)
+    for b in range(batch):
+        pin = rs.randn(P, E).astype(np.float32)
+        assert lib.orc_kv_cache_refresh_cross(cache.ptr, b, binding.fptr(pin.reshape(-1)), P, 0) == 0
+    x, o = rs.randn(batch, E).astype(np.float32), np.zeros((batch, V), dtype=np.float32)
+    fp = lambda a: binding.fptr(a.reshape(-1))
+    steps, spent = 0, 0.0
+    while steps < 1 or (spent < budget_s and steps < 16):
+        t0 = time.perf_counter()
+        for b in range(batch):
+            assert lib.orc_kv_decode_step(cache.ptr, b, int(lens[b]) + steps, tables[b], P, fp(x[b:b + 1]), 1, 0,
+                                          fp(o[b:b + 1])) == 0
+        spent += time.perf_counter() - t0
+        steps += 1
+    return {"value": spent / steps * 1e6, "unit": "us/step", "cores": 1, "kind": "port",
+            "sample": "%d decoder steps of %d sequences, %.1f s" % (steps, batch, spent)}
+
+
 def cpu_dense(w, budget_s):
     """Checker on one host core over the same workload; repeated whole passes up to the budget."""
     from oracle import binding, runner as orunner
@@ -557,6 +683,10 @@ def main():
         if not args.no_cpu:
             others["decode_layer"]["cpu_baseline"] = cpu_decode_layer(2.0)
         log("decode_layer", json.dumps(others["decode_layer"]))
+        others["decode_step"] = bench_decode_step(K, W)
+        if not args.no_cpu:
+            others["decode_step"]["cpu_baseline"] = cpu_decode_step(2.0)
+        log("decode_step", json.dumps(others["decode_step"]))
 
     cpu_head = None
     if not args.no_cpu:
