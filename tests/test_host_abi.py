@@ -96,6 +96,43 @@ def test_layout_matches_reference_headers(tmp_path):
     assert outs[0] == outs[1] and outs[0].count("\n") > 50
 
 
+def test_kv_cache_container_bookkeeping():
+    """Host side of csrc/infer/kv_cache.c:27-110 on a host arena: shapes, zero fill, truncate,
+    common patches, reset, and the placement rule of csrc/models/local_common.c:49-64."""
+    lib = api.load()
+    dec = abi.BltLocalDecoder()
+    dec.config.embed_dim, dec.config.patch_dim, dec.config.max_seq_len, dec.config.num_layers = 8, 24, 32, 3
+    arena = lib.blt_arena_create(1 << 20, abi.BLT_BACKEND_CPU)
+    cache = lib.blt_kv_cache_create_batched(arena, C.byref(dec), 20, 5)
+    c = cache.contents
+    assert (c.max_seq_len, c.batch_size, c.max_subtokens, c.embed_dim, c.k, c.patch_dim) == (20, 5, 20, 8, 3, 24)
+    for l in range(3):
+        for tier in (c.self_k, c.self_v, c.cross_k, c.cross_v):
+            assert tuple(tier[l].shape[:2]) == (100, 8) and tier[l].numel == 800
+            assert not np.ctypeslib.as_array(C.cast(tier[l].data, C.POINTER(C.c_float)), shape=(800,)).any()
+    assert c.self_len == 0 and c.cross_num_patches == 0
+    new = abi.patch_array([0, 3, 7], [3, 4, 2])
+    assert lib.blt_kv_cache_common_patches(cache, new, 3) == 0      # nothing cached yet
+    for i, (s0, ln) in enumerate(((0, 3), (3, 4), (7, 5))):
+        c.cached_patches[i].start_idx, c.cached_patches[i].length = s0, ln
+    lib.blt_kv_cache_truncate(cache, 12, 3)
+    assert (c.self_len, c.cross_num_patches) == (12, 3)
+    assert lib.blt_kv_cache_common_patches(cache, new, 3) == 2      # the third patch changed its length
+    assert lib.blt_kv_cache_common_patches(cache, new, 1) == 1
+    lib.blt_kv_cache_reset(cache)
+    assert (c.self_len, c.cross_num_patches) == (0, 0)
+    lib.blt_kv_cache_destroy(cache)
+    lib.blt_arena_destroy(arena)
+    fires = lambda placement, all_layers, L: [bool(lib.blt_local_cross_attn_fires(placement, all_layers, L, l))
+                                              for l in range(L)]
+    assert fires(abi.BLT_XATTN_DEFAULT, True, 3) == [True, True, True]
+    assert fires(abi.BLT_XATTN_DEFAULT, False, 3) == [False, False, True]
+    assert fires(abi.BLT_XATTN_NONE, True, 3) == [False, False, False]
+    assert fires(abi.BLT_XATTN_LAST, True, 3) == [False, False, True]
+    assert fires(abi.BLT_XATTN_ALL, False, 3) == [True, True, True]
+    assert fires(abi.BLT_XATTN_FIRST, True, 3) == [True, False, False]
+
+
 def test_patch_helpers_match_checker(oracle):
     lib = api.load()
     rs = np.random.RandomState(21)
@@ -206,6 +243,38 @@ lib.blt_build_attention_mask(C.byref(cfg), C.byref(t), arena)
     "arena_overflow": """
 arena = lib.blt_arena_create(64, abi.BLT_BACKEND_CPU)
 lib.blt_arena_alloc(arena, 65, 1)
+""",
+    "cpu_cross_attention": """
+import numpy as np
+x = np.zeros((2, 4), dtype=np.float32)
+t = abi.tensor_view(x.ctypes.data, x.shape, abi.BLT_BACKEND_CPU)
+w = abi.BltCrossAttentionWeights(C.pointer(t), C.pointer(t), C.pointer(t), C.pointer(t))
+m = abi.BltMaskConfig(); m.seq_len_q = m.seq_len_kv = 2
+c = abi.BltCrossAttentionConfig(); c.embed_dim, c.num_heads, c.mask_config = 4, 2, C.pointer(m)
+arena = lib.blt_arena_create(1 << 16, abi.BLT_BACKEND_CPU)
+lib.blt_cross_attention_forward(C.byref(t), C.byref(t), C.byref(w), C.byref(t), C.byref(c), arena)
+""",
+    "kv_cache_longer_than_decoder": """
+dec = abi.BltLocalDecoder(); dec.config.embed_dim, dec.config.max_seq_len, dec.config.num_layers = 8, 16, 1
+arena = lib.blt_arena_create(1 << 20, abi.BLT_BACKEND_CPU)
+lib.blt_kv_cache_create(arena, C.byref(dec), 17)
+""",
+    "kv_cache_truncate_past_capacity": """
+dec = abi.BltLocalDecoder(); dec.config.embed_dim, dec.config.max_seq_len, dec.config.num_layers = 8, 16, 1
+arena = lib.blt_arena_create(1 << 20, abi.BLT_BACKEND_CPU)
+cache = lib.blt_kv_cache_create(arena, C.byref(dec), 16)
+assert cache.contents.max_subtokens == 16 and cache.contents.k == 1
+lib.blt_kv_cache_truncate(cache, 17, 0)
+""",
+    "cpu_decode_step": """
+import numpy as np
+dec = abi.BltLocalDecoder(); dec.config.embed_dim, dec.config.max_seq_len, dec.config.num_layers = 8, 16, 1
+arena = lib.blt_arena_create(1 << 20, abi.BLT_BACKEND_CPU)
+cache = lib.blt_kv_cache_create(arena, C.byref(dec), 16)
+x = np.zeros((1, 8), dtype=np.float32)
+t = abi.tensor_view(x.ctypes.data, x.shape, abi.BLT_BACKEND_CPU)
+p = abi.patch_array([0], [1])
+lib.blt_kv_decode_step(cache, C.byref(t), p, 1, C.byref(t), 0, C.byref(t), arena)
 """,
     "bad_patch_tiling": """
 p = abi.patch_array([0, 4], [3, 2])
