@@ -109,27 +109,19 @@ __global__ __launch_bounds__(64 * WAVES) void kv_step_kernel(StepArgs a) {
         }
     };
 
-    const uint32_t stride = a.slices * STEP;
-    uint32_t c0 = k_begin + slice * STEP;
-    float4 kf[LOADS], vf[LOADS];
-    if (c0 < k_end) fetch(c0, kf, vf);
-    while (c0 < k_end) {
-        const uint32_t cn = c0 + stride;
-        float4 kn[LOADS], vn[LOADS];
-        if (cn < k_end) fetch(cn, kn, vn);
-
-        /* write-through of the new rows this sub-chunk holds */
-        if (a.write_through && head_ok) {
+    /* the same for a sub-chunk that lies entirely in the cached prefix: no branch, one address form */
+    auto fetch_cached = [&](uint32_t c0, float4 (&kf)[LOADS], float4 (&vf)[LOADS]) __attribute__((always_inline)) {
+        const float *kb = a.cache_k + (slab + c0 + grp) * a.embed_dim + col;
+        const float *vb = a.cache_v + (slab + c0 + grp) * a.embed_dim + col;
 #pragma unroll
-            for (int t = 0; t < LOADS; t++) {
-                const uint32_t j = c0 + grp + KPL * t;
-                if (j >= len && j < k_end) {
-                    *reinterpret_cast<float4 *>(a.cache_k + (slab + j) * a.embed_dim + col) = kf[t];
-                    *reinterpret_cast<float4 *>(a.cache_v + (slab + j) * a.embed_dim + col) = vf[t];
-                }
-            }
+        for (int t = 0; t < LOADS; t++) {
+            kf[t] = *reinterpret_cast<const float4 *>(kb + (size_t)(KPL * t) * a.embed_dim);
+            vf[t] = *reinterpret_cast<const float4 *>(vb + (size_t)(KPL * t) * a.embed_dim);
         }
+    };
 
+    /* scores, online softmax and weighted sum of one sub-chunk for every query row of the launch */
+    auto attend = [&](uint32_t c0, const float4 (&kf)[LOADS], const float4 (&vf)[LOADS]) __attribute__((always_inline)) {
 #pragma unroll
         for (int r = 0; r < NQ; r++) {
             const uint32_t qi = a.q0 + r;
@@ -163,7 +155,47 @@ __global__ __launch_bounds__(64 * WAVES) void kv_step_kernel(StepArgs a) {
             l[r] = l[r] * alpha + ls;
             m[r] = mn;
         }
+    };
 
+    const uint32_t stride = a.slices * STEP;
+    uint32_t c0 = k_begin + slice * STEP;
+    float4 kf[LOADS], vf[LOADS];
+    if (c0 < k_end) fetch(c0, kf, vf);
+    /* Cached sub-chunks first, in a loop whose body has no branch around a
+     * load or a store: the rows of the next sub-chunk are requested, then
+     * this one is worked on, and the wait before the work counts exactly the
+     * requests issued after its own rows.  (With branches around the loads
+     * the wait falls back to "everything", next sub-chunk included.) */
+    while (c0 + stride + STEP <= len && c0 + stride < k_end) {
+        float4 kn[LOADS], vn[LOADS];
+        fetch_cached(c0 + stride, kn, vn);
+        __builtin_amdgcn_sched_barrier(0); /* requests stay ahead of the work */
+        attend(c0, kf, vf);
+#pragma unroll
+        for (int t = 0; t < LOADS; t++) {
+            kf[t] = kn[t];
+            vf[t] = vn[t];
+        }
+        c0 += stride;
+    }
+    /* the last sub-chunks of the slice: may hold the new rows (rotation, write-through) */
+    while (c0 < k_end) {
+        const uint32_t cn = c0 + stride;
+        float4 kn[LOADS], vn[LOADS];
+        if (cn < k_end) fetch(cn, kn, vn);
+
+        /* write-through of the new rows this sub-chunk holds */
+        if (a.write_through && head_ok) {
+#pragma unroll
+            for (int t = 0; t < LOADS; t++) {
+                const uint32_t j = c0 + grp + KPL * t;
+                if (j >= len && j < k_end) {
+                    *reinterpret_cast<float4 *>(a.cache_k + (slab + j) * a.embed_dim + col) = kf[t];
+                    *reinterpret_cast<float4 *>(a.cache_v + (slab + j) * a.embed_dim + col) = vf[t];
+                }
+            }
+        }
+        attend(c0, kf, vf);
 #pragma unroll
         for (int t = 0; t < LOADS; t++) {
             kf[t] = kn[t];

@@ -27,6 +27,7 @@
 #include "launch.h"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace {
 
@@ -109,76 +110,92 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block_mfma_kernel(StepArgs a
     float m = neg_inf(), l = 0.f;
 
     float *my_k = sm_k[wave];
-    float kg[HALF]; /* K tile in flight: HD/8 pieces of 16 bytes per lane */
-    float vf[DB][16];
 
-    /* row j of the sequence: cached rows come from the slab, new rows from the step's inputs */
+    /* row j of the sequence: cached rows come from the slab, new rows from the step's inputs.
+     * (Argument fields are copied out first: a select between two fields read in place becomes a
+     * per-lane load of the argument block itself.) */
+    const float *const cache_k = a.cache_k, *const cache_v = a.cache_v;
+    const float *const new_k = a.k_rows, *const new_v = a.v_rows;
+    const size_t embed_dim = a.embed_dim, k_stride = a.k_stride, v_stride = a.v_stride;
     auto k_row = [&](uint32_t j) __attribute__((always_inline)) -> const float * {
-        return j < len ? a.cache_k + (slab + j) * a.embed_dim : a.k_rows + (newrow0 + (j - len)) * a.k_stride;
+        const size_t at = j < len ? (slab + j) * embed_dim : (newrow0 + (j - len)) * k_stride;
+        return (j < len ? cache_k : new_k) + at;
     };
     auto v_row = [&](uint32_t j) __attribute__((always_inline)) -> const float * {
-        return j < len ? a.cache_v + (slab + j) * a.embed_dim : a.v_rows + (newrow0 + (j - len)) * a.v_stride;
+        const size_t at = j < len ? (slab + j) * embed_dim : (newrow0 + (j - len)) * v_stride;
+        return (j < len ? cache_v : new_v) + at;
     };
 
-    /* A sub-chunk that lies entirely in the cached prefix (the common case) is
-     * addressed from one per-lane base with compile-time row steps; one that
-     * touches the new rows or the end of the sequence selects row by row. */
-#define REQUEST_K(c0_)                                                                                             \
-    do {                                                                                                           \
-        if ((c0_) + 32u <= len) {                                                                                  \
-            const float *kb_ = a.cache_k + (slab + (c0_) + lane / LPR) * a.embed_dim + hsafe * HD +                \
-                               4u * (lane % LPR);                                                                  \
-            _Pragma("unroll") for (int t = 0; t < HD / 8; t++) {                                                   \
-                const float4 x_ = *reinterpret_cast<const float4 *>(kb_ + (size_t)(t * (64 / LPR)) * a.embed_dim); \
-                kg[4 * t + 0] = x_.x, kg[4 * t + 1] = x_.y, kg[4 * t + 2] = x_.z, kg[4 * t + 3] = x_.w;            \
-            }                                                                                                      \
-        } else {                                                                                                   \
-            _Pragma("unroll") for (int t = 0; t < HD / 8; t++) {                                                   \
-                const uint32_t r_ = t * (64 / LPR) + lane / LPR;                                                   \
-                const uint32_t j_ = min((c0_) + r_, nk - 1u);                                                      \
-                const float4 x_ = *reinterpret_cast<const float4 *>(k_row(j_) + hsafe * HD + 4u * (lane % LPR));   \
-                kg[4 * t + 0] = x_.x, kg[4 * t + 1] = x_.y, kg[4 * t + 2] = x_.z, kg[4 * t + 3] = x_.w;            \
-            }                                                                                                      \
-        }                                                                                                          \
-    } while (0)
-#define REQUEST_V(c0_)                                                                                             \
-    do {                                                                                                           \
-        if ((c0_) + 32u <= len) {                                                                                  \
-            const float *vb_ = a.cache_v + (slab + (c0_) + 4u * h) * a.embed_dim + hsafe * HD + c;                 \
-            _Pragma("unroll") for (int s = 0; s < 16; s++) {                                                       \
-                const float *vr_ = vb_ + (size_t)(8 * (s >> 2) + (s & 3)) * a.embed_dim;                           \
-                _Pragma("unroll") for (int d = 0; d < DB; d++) vf[d][s] = vr_[32 * d];                             \
-            }                                                                                                      \
-        } else {                                                                                                   \
-            _Pragma("unroll") for (int s = 0; s < 16; s++) {                                                       \
-                const uint32_t j_ = min((c0_) + acc_key(s, h), nk - 1u);                                           \
-                const float *vr_ = v_row(j_) + hsafe * HD + c;                                                     \
-                _Pragma("unroll") for (int d = 0; d < DB; d++) vf[d][s] = vr_[32 * d];                             \
-            }                                                                                                      \
-        }                                                                                                          \
-    } while (0)
+    /* Requests for the K tile (HD/8 pieces of 16 bytes per lane) and the V
+     * fragment of the sub-chunk at key cs.  A sub-chunk that lies entirely in
+     * the cached prefix (the common case) is addressed from one per-lane base
+     * with compile-time row steps; one that touches the new rows or the end
+     * of the sequence selects row by row. */
+    auto request_k = [&](auto cached_only, float (&kg)[HALF], uint32_t cs) __attribute__((always_inline)) {
+        if (decltype(cached_only)::value || cs + 32u <= len) {
+            const float *kb = cache_k + (slab + cs + lane / LPR) * embed_dim + hsafe * HD + 4u * (lane % LPR);
+#pragma unroll
+            for (int t = 0; t < HD / 8; t++) {
+                const float4 x = *reinterpret_cast<const float4 *>(kb + (size_t)(t * (64 / LPR)) * embed_dim);
+                kg[4 * t + 0] = x.x, kg[4 * t + 1] = x.y, kg[4 * t + 2] = x.z, kg[4 * t + 3] = x.w;
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < HD / 8; t++) {
+                const uint32_t r = t * (64 / LPR) + lane / LPR;
+                const uint32_t j = min(cs + r, nk - 1u);
+                const float4 x = *reinterpret_cast<const float4 *>(k_row(j) + hsafe * HD + 4u * (lane % LPR));
+                kg[4 * t + 0] = x.x, kg[4 * t + 1] = x.y, kg[4 * t + 2] = x.z, kg[4 * t + 3] = x.w;
+            }
+        }
+    };
+    auto request_v = [&](auto cached_only, float (&vf)[DB][16], uint32_t cs) __attribute__((always_inline)) {
+        if (decltype(cached_only)::value || cs + 32u <= len) {
+            const float *vb = cache_v + (slab + cs + 4u * h) * embed_dim + hsafe * HD + c;
+#pragma unroll
+            for (int s = 0; s < 16; s++) {
+                const float *vr = vb + (size_t)(8 * (s >> 2) + (s & 3)) * embed_dim;
+#pragma unroll
+                for (int d = 0; d < DB; d++) vf[d][s] = vr[32 * d];
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < 16; s++) {
+                const uint32_t j = min(cs + acc_key(s, h), nk - 1u);
+                const float *vr = v_row(j) + hsafe * HD + c;
+#pragma unroll
+                for (int d = 0; d < DB; d++) vf[d][s] = vr[32 * d];
+            }
+        }
+    };
 
-    const uint32_t step = a.slices * 32u;
-    uint32_t c0 = k_begin + slice * 32u;
-    if (c0 < k_end) {
-        REQUEST_K(c0);
-        REQUEST_V(c0);
-    }
-    while (c0 < k_end) {
-        const uint32_t cn = c0 + step;
-
+    /* One 32-key sub-chunk at key c0 whose K tile and V fragment have been
+     * requested into kg / vf.  As soon as kg is parked in LDS it is reused for
+     * the K tile of the sub-chunk at cnext (when `more`), and vf for its V
+     * fragment once the second product has consumed it, so those rows travel
+     * while this and the following sub-chunks are worked on. */
+    auto sub_chunk = [&](auto touches_new_rows, float (&kg)[HALF], float (&vf)[DB][16], uint32_t c0,
+                         uint32_t cnext, bool more) __attribute__((always_inline)) {
+        /* NEW = false: this sub-chunk and the one requested at cnext lie in the cached prefix: nothing
+         * to rotate or write through, one address form.  That body has no branch around a load or a
+         * store, so its waits stay exact. */
+        constexpr bool NEW = decltype(touches_new_rows)::value;
+        constexpr std::integral_constant<bool, !NEW> next_cached{};
         /* K tile: write-through of new rows, then LDS -> fragment (lane = key row) */
 #pragma unroll
         for (int t = 0; t < HD / 8; t++) {
             const uint32_t r = t * (64 / LPR) + lane / LPR;
             float4 piece = make_float4(kg[4 * t + 0], kg[4 * t + 1], kg[4 * t + 2], kg[4 * t + 3]);
-            const uint32_t j = c0 + r;
-            if (a.rope_cos && c0 + 32u > len && j >= len && j < nk) { /* a new key row is rotated at its position j */
-                const size_t at = (size_t)j * HALF + 2u * (lane % LPR);
-                piece = rope_rotate4(piece, a.rope_cos + at, a.rope_sin + at);
+            if constexpr (NEW) {
+                const uint32_t j = c0 + r;
+                if (a.rope_cos && j >= len && j < nk) { /* a new key row is rotated at its position j */
+                    const size_t at = (size_t)j * HALF + 2u * (lane % LPR);
+                    piece = rope_rotate4(piece, a.rope_cos + at, a.rope_sin + at);
+                }
+                if (a.write_through && head_ok && j >= len && j < k_end)
+                    *reinterpret_cast<float4 *>(a.cache_k + (slab + j) * a.embed_dim + head * HD +
+                                                4u * (lane % LPR)) = piece;
             }
-            if (a.write_through && head_ok && c0 + 32u > len && j >= len && j < k_end)
-                *reinterpret_cast<float4 *>(a.cache_k + (slab + j) * a.embed_dim + head * HD + 4u * (lane % LPR)) = piece;
             *reinterpret_cast<float4 *>(my_k + r * ROW + 4u * (lane % LPR)) = piece;
         }
         float kf[HALF];
@@ -187,8 +204,10 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block_mfma_kernel(StepArgs a
             const float4 t = *reinterpret_cast<const float4 *>(my_k + c * ROW + h * HALF + s);
             kf[s + 0] = t.x, kf[s + 1] = t.y, kf[s + 2] = t.z, kf[s + 3] = t.w;
         }
-        /* the next sub-chunk's K rows travel while this one is worked on */
-        if (cn < k_end) REQUEST_K(cn);
+        if (more) request_k(next_cached, kg, cnext);
+        /* the requests stay where they are written: left alone, the scheduler moves loads whose
+         * results are not needed in this block to its end, which is the opposite of a prefetch */
+        __builtin_amdgcn_sched_barrier(0);
 
         floatx16 sacc;
 #pragma unroll
@@ -226,22 +245,43 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block_mfma_kernel(StepArgs a
             for (int s = 0; s < 16; s++) oacc[d] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf[d][s], x[s], oacc[d], 0, 0, 0);
         }
 
-        /* V: write-through of new rows from the values just used, then the next sub-chunk's rows */
-        if (a.write_through && head_ok && c0 + 32u > len) {
+        /* V: write-through of new rows from the values just used, then the next rows */
+        if constexpr (NEW) {
+            if (a.write_through && head_ok) {
 #pragma unroll
-            for (int s = 0; s < 16; s++) {
-                const uint32_t j = c0 + acc_key(s, h);
-                if (j >= len && j < k_end) {
+                for (int s = 0; s < 16; s++) {
+                    const uint32_t j = c0 + acc_key(s, h);
+                    if (j >= len && j < k_end) {
 #pragma unroll
-                    for (int d = 0; d < DB; d++) a.cache_v[(slab + j) * a.embed_dim + head * HD + 32 * d + c] = vf[d][s];
+                        for (int d = 0; d < DB; d++)
+                            a.cache_v[(slab + j) * a.embed_dim + head * HD + 32 * d + c] = vf[d][s];
+                    }
                 }
             }
         }
-        if (cn < k_end) REQUEST_V(cn);
+        if (more) request_v(next_cached, vf, cnext);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    constexpr std::false_type CACHED{};
+    constexpr std::true_type GENERAL{};
+
+    const uint32_t step = a.slices * 32u;
+    uint32_t c0 = k_begin + slice * 32u;
+    float kg[HALF];
+    float vf[DB][16];
+    if (c0 < k_end) {
+        request_k(std::false_type{}, kg, c0);
+        request_v(std::false_type{}, vf, c0);
+    }
+    while (c0 + step + 32u <= len && c0 + step < k_end) { /* this and the next sub-chunk are cached rows */
+        sub_chunk(CACHED, kg, vf, c0, c0 + step, true);
+        c0 += step;
+    }
+    while (c0 < k_end) {
+        const uint32_t cn = c0 + step;
+        sub_chunk(GENERAL, kg, vf, c0, cn, cn < k_end);
         c0 = cn;
     }
-#undef REQUEST_K
-#undef REQUEST_V
 
     l += __shfl_xor(l, 32, 64);
 
