@@ -324,14 +324,17 @@ __global__ __launch_bounds__(64 * NW, HD <= 64 ? 2 : 1) void attn_mfma_kernel(co
         float x[16];
         float mt = neg_inf();
         const bool all_seen = !DENSE && k0 >= flo && k0 + 32u <= fhi; /* uniform: no row masks any key */
+        /* lo <= j < hi as one unsigned compare, widened to "always" on tiles every row sees whole:
+         * written with && the sixteen tests become sixteen pairs of branches */
+        const uint32_t vlo = all_seen ? 0u : lo;
+        const uint32_t vlen = all_seen ? 0xFFFFFFFFu : (hi > lo ? hi - lo : 0u);
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const uint32_t j = k0 + acc_key(r, h);
             float t;
             if (DENSE) t = (sacc[r] * p.scale + mrow[min(j, p.nk - 1u)]) * LOG2E;
             else t = sacc[r] * scale2;
-            bool vis = isfinite(t);
-            if (!all_seen) vis = vis && j >= lo && j < hi;
+            const bool vis = ((j - vlo) < vlen) & isfinite(t);
             x[r] = vis ? t : neg_inf();
             mt = fmaxf(mt, x[r]);
         }
