@@ -126,15 +126,23 @@ __global__ __launch_bounds__(64 * WAVES) void kv_step_kernel(StepArgs a) {
         for (int r = 0; r < NQ; r++) {
             const uint32_t qi = a.q0 + r;
             const uint32_t p = len + qi; /* absolute position of the query */
+            /* the keys this row sees within the span, [vlo, vlo + vlen): everything up to the span's
+             * end for block rows, up to its own position and inside the window for causal rows
+             * (kv_cache.c:229-236), nothing for padding rows; one unsigned compare per key */
+            uint32_t vhi = k_end, vlo = 0u;
+            if (!a.block_kind) {
+                vhi = min(vhi, p + 1u);
+                if (a.window > 0u && p + 1u > a.window) vlo = p + 1u - a.window;
+            }
+            if (qi >= a.n) vhi = 0u;
+            const uint32_t vlen = vhi > vlo ? vhi - vlo : 0u;
             float x[LOADS];
             float mt = neg_inf();
 #pragma unroll
             for (int t = 0; t < LOADS; t++) {
                 const uint32_t j = c0 + grp + KPL * t;
                 const float s = group_sum<G>(dot4(q[r], kf[t])) * a.scale;
-                bool vis = j < k_end && qi < a.n;
-                if (!a.block_kind) vis = vis && j <= p && (a.window == 0u || p - j < a.window);
-                vis = vis && isfinite(s);
+                const bool vis = ((j - vlo) < vlen) & isfinite(s);
                 x[t] = vis ? s : neg_inf();
                 mt = fmaxf(mt, x[t]);
             }
