@@ -29,13 +29,13 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 # the plain 64 MiB streaming copy (--probe-copy-mib 64): x1.999 for FETCH_SIZE,
 # x1.000 for WRITE_SIZE.  The summaries under profiles/ hold the readings.
 MEASURED_TRAFFIC_BYTES = {
-    "c2_patch_block_causal": (6243.1 * 1.999 + 4096.0) * 1024,
-    "c1_local_decoder_causal": (708.6 * 1.999 + 256.0) * 1024,
+    "c2_patch_block_causal": (6225.1 * 1.999 + 4096.0) * 1024,
+    "c1_local_decoder_causal": (687.0 * 1.999 + 256.0) * 1024,
     "c3_encoder_cross": (4699.1 * 1.999 + 1024.0) * 1024,
-    "c4_kv_decode": (11865.7 * 1.999 + 108.0) * 1024,          # mean over the 256 growing steps
-    "c5_block_verify_B4": (9521.5 * 1.999 + 896.0) * 1024,     # the three block sizes run the same kernel
-    "c5_block_verify_B8": (9521.5 * 1.999 + 896.0) * 1024,     # and were collected together
-    "c5_block_verify_B16": (9521.5 * 1.999 + 896.0) * 1024,
+    "c4_kv_decode": (11868.6 * 1.999 + 108.0) * 1024,          # mean over the 256 growing steps
+    "c5_block_verify_B4": (9530.5 * 1.999 + 896.0) * 1024,     # the three block sizes run the same kernel
+    "c5_block_verify_B8": (9530.5 * 1.999 + 896.0) * 1024,     # and were collected together
+    "c5_block_verify_B16": (9530.5 * 1.999 + 896.0) * 1024,
 }
 
 
