@@ -188,31 +188,47 @@ __device__ __forceinline__ void splitk_tile(const MatmulArgs &g, const uint32_t 
 
     float ss = 0.f; /* this lane's share of sum_k a[row][k]^2 (norm_w only) */
     /* fragments of one 32-wide K chunk: lane (h, c) holds a[row][k0 + 16h + t] and b[k0 + 16h + t][col] */
+    /* Every load of a chunk is issued before anything waits: addresses past K are clamped to the
+     * last valid element and the value replaced by zero afterwards, so no load sits behind a
+     * branch, and the norm arithmetic (which needs the a values) comes after the b requests. */
     auto fetch = [&](uint32_t k0, float (&fa)[16], float (&fb)[16], float (&fg)[16]) __attribute__((always_inline)) {
         const uint32_t kb = k0 + 16u * h;
-        if (VEC) {
+        if (VEC) { /* K is a multiple of 4 here: a 16-byte piece is inside or outside as a whole */
 #pragma unroll
             for (int t = 0; t < 16; t += 4) {
-                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (kb + t < g.k) v = *reinterpret_cast<const float4 *>(arow + kb + t);
-                fa[t + 0] = v.x, fa[t + 1] = v.y, fa[t + 2] = v.z, fa[t + 3] = v.w;
+                const float4 v = *reinterpret_cast<const float4 *>(arow + min(kb + t, g.k - 4u));
+                const bool in = kb + t < g.k;
+                fa[t + 0] = in ? v.x : 0.f, fa[t + 1] = in ? v.y : 0.f;
+                fa[t + 2] = in ? v.z : 0.f, fa[t + 3] = in ? v.w : 0.f;
             }
         } else {
 #pragma unroll
-            for (int t = 0; t < 16; t++) fa[t] = kb + t < g.k ? arow[kb + t] : 0.f;
-        }
-        if (g.norm_w) { /* uniform: sum of squares of the raw row, then the norm weight folded into a */
-#pragma unroll
             for (int t = 0; t < 16; t++) {
-                ss += fa[t] * fa[t];
-                fa[t] *= kb + t < g.k ? g.norm_w[kb + t] : 0.f;
+                const float v = arow[min(kb + t, g.k - 1u)];
+                fa[t] = kb + t < g.k ? v : 0.f;
             }
         }
 #pragma unroll
-        for (int t = 0; t < 16; t++) fb[t] = kb + t < g.k ? bcol[(size_t)(kb + t) * g.ldb] : 0.f;
+        for (int t = 0; t < 16; t++) {
+            const float v = bcol[(size_t)min(kb + t, g.k - 1u) * g.ldb];
+            fb[t] = kb + t < g.k ? v : 0.f;
+        }
         if (GATED) {
 #pragma unroll
-            for (int t = 0; t < 16; t++) fg[t] = kb + t < g.k ? b2col[(size_t)(kb + t) * g.ldb] : 0.f;
+            for (int t = 0; t < 16; t++) {
+                const float v = b2col[(size_t)min(kb + t, g.k - 1u) * g.ldb];
+                fg[t] = kb + t < g.k ? v : 0.f;
+            }
+        }
+        if (g.norm_w) { /* uniform: sum of squares of the raw row, then the norm weight folded into a */
+            float nw[16];
+#pragma unroll
+            for (int t = 0; t < 16; t++) nw[t] = g.norm_w[min(kb + t, g.k - 1u)];
+#pragma unroll
+            for (int t = 0; t < 16; t++) {
+                ss += fa[t] * fa[t];
+                fa[t] *= nw[t]; /* fa is already zero past K */
+            }
         }
     };
 
