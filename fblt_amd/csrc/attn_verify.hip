@@ -27,6 +27,8 @@
 #include "launch.h"
 
 #include <algorithm>
+#include <cstdlib>
+#include <cstring>
 #include <type_traits>
 
 namespace {
@@ -329,6 +331,290 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block_mfma_kernel(StepArgs a
     kv_finish_sequence<HD>(a, (uint32_t)SLOTS, b, nk, &sm_ticket);
 }
 
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+/* The same step for blocks of at most 16 rows on 16x16x4 tiles
+ * (v_mfma_f32_16x16x4_f32: A[i = lane % 16][k = lane / 16], B[k = lane / 16][j = lane % 16],
+ * D[i = 4 * (lane / 16) + r][j = lane % 16]), so that no half of a tile is padding:
+ *
+ *   S^T[key, query]: two 16-key tiles per sub-chunk; lane group g = lane / 16 contracts the
+ *                    head's columns [g * HD/4, (g + 1) * HD/4), one per step;
+ *   O^T[d, query]:   HD/16 tiles; the contraction runs over the keys, lane group g taking key
+ *                    16 t + 4 g + r at step (t, r) -- exactly the key whose weight its S^T
+ *                    register (t, r) holds, so P^T needs no exchange.
+ *
+ * Half the matrix-core cycles and half the softmax arithmetic of the 32-wide kernel per
+ * sub-chunk.  K and V fragments come straight from global memory in fragment layout (a K row's
+ * 128 bytes are shared by the four lane groups), nothing is staged through LDS. */
+template <int HD, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 2) void kv_block16_mfma_kernel(StepArgs a) {
+    constexpr int HALF = HD / 2;
+    constexpr int QD = HD / 4;  /* columns of the head one lane group contracts */
+    constexpr int DT = HD / 16; /* 16-row tiles of O^T */
+    constexpr int PR = HD + 2;  /* a parked result row: HD columns, max, sum */
+    constexpr uint32_t ROWS = 16;
+
+    __shared__ float sm_o[WAVES][ROWS * PR];
+    __shared__ uint32_t sm_ticket;
+
+    const uint32_t b = blockIdx.y;
+    const uint32_t split = blockIdx.x;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t slice = wave / a.hpb;
+    const uint32_t head = blockIdx.z * a.hpb + wave % a.hpb;
+    const bool head_ok = head < a.num_heads;
+    const uint32_t hsafe = head_ok ? head : 0u;
+    const uint32_t g = lane >> 4;
+    const uint32_t c = lane & 15u;
+
+    const uint32_t len = a.self_len[b];
+    const uint32_t nk = len + a.n;
+    const size_t slab = (size_t)b * a.max_seq_len;
+    const uint32_t span = kv_span_of(a, nk);
+    const uint32_t k_begin = split * span;
+    const uint32_t k_end = min(k_begin + span, nk);
+    const size_t newrow0 = (size_t)b * a.n;
+
+    /* query fragment: row c of the block (clamped), columns [g*QD, (g+1)*QD) of the head */
+    const uint32_t qi = a.q0 + c;
+    const bool q_ok = qi < a.n;
+    float qf[QD];
+    {
+        const float *qrow = a.q_rows + (newrow0 + min(qi, a.n - 1u)) * a.q_stride + hsafe * HD + g * QD;
+#pragma unroll
+        for (int s = 0; s < QD; s += 4) {
+            float4 t = *reinterpret_cast<const float4 *>(qrow + s);
+            if (a.rope_cos) { /* the query sits at position len + qi */
+                const size_t at = (size_t)(len + min(qi, a.n - 1u)) * HALF + (g * QD + s) / 2;
+                t = rope_rotate4(t, a.rope_cos + at, a.rope_sin + at);
+            }
+            qf[s + 0] = t.x, qf[s + 1] = t.y, qf[s + 2] = t.z, qf[s + 3] = t.w;
+        }
+    }
+    uint32_t vis_lo = 0, vis_hi = k_end;
+    if (!a.block_kind) {
+        const uint32_t qpos = len + qi;
+        vis_hi = min(vis_hi, qpos + 1u);
+        if (a.window > 0u && qpos + 1u > a.window) vis_lo = qpos + 1u - a.window;
+    }
+    if (!q_ok) vis_hi = 0;
+    const uint32_t vis_len = vis_hi > vis_lo ? vis_hi - vis_lo : 0u;
+    const float scale2 = a.scale * LOG2E;
+
+    floatx4 oacc[DT];
+#pragma unroll
+    for (int d = 0; d < DT; d++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) oacc[d][r] = 0.f;
+    float m = neg_inf(), l = 0.f;
+
+    const float *const cache_k = a.cache_k, *const cache_v = a.cache_v;
+    const float *const new_k = a.k_rows, *const new_v = a.v_rows;
+    const size_t embed_dim = a.embed_dim, k_stride = a.k_stride, v_stride = a.v_stride;
+    auto k_row = [&](uint32_t j) __attribute__((always_inline)) -> const float * {
+        const size_t at = j < len ? (slab + j) * embed_dim : (newrow0 + (j - len)) * k_stride;
+        return (j < len ? cache_k : new_k) + at;
+    };
+    auto v_row = [&](uint32_t j) __attribute__((always_inline)) -> const float * {
+        const size_t at = j < len ? (slab + j) * embed_dim : (newrow0 + (j - len)) * v_stride;
+        return (j < len ? cache_v : new_v) + at;
+    };
+
+    /* K fragment of the sub-chunk at key cs: tile t holds key cs + 16 t + c, columns g*QD ...;
+     * V fragment: element (d, 4 t + r) is column 16 d + c of key cs + 16 t + 4 g + r */
+    auto request_k = [&](auto cached_only, float (&kf)[2][QD], uint32_t cs) __attribute__((always_inline)) {
+        if (decltype(cached_only)::value || cs + 32u <= len) {
+            const float *kb = cache_k + (slab + cs + c) * embed_dim + hsafe * HD + g * QD;
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int s = 0; s < QD; s += 4) {
+                    const float4 x = *reinterpret_cast<const float4 *>(kb + (size_t)(16 * t) * embed_dim + s);
+                    kf[t][s + 0] = x.x, kf[t][s + 1] = x.y, kf[t][s + 2] = x.z, kf[t][s + 3] = x.w;
+                }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                const uint32_t j = min(cs + 16u * t + c, nk - 1u);
+                const float *kr = k_row(j) + hsafe * HD + g * QD;
+#pragma unroll
+                for (int s = 0; s < QD; s += 4) {
+                    const float4 x = *reinterpret_cast<const float4 *>(kr + s);
+                    kf[t][s + 0] = x.x, kf[t][s + 1] = x.y, kf[t][s + 2] = x.z, kf[t][s + 3] = x.w;
+                }
+            }
+        }
+    };
+    auto request_v = [&](auto cached_only, float (&vf)[DT][8], uint32_t cs) __attribute__((always_inline)) {
+        if (decltype(cached_only)::value || cs + 32u <= len) {
+            const float *vb = cache_v + (slab + cs + 4u * g) * embed_dim + hsafe * HD + c;
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const float *vr = vb + (size_t)(16 * (u >> 2) + (u & 3)) * embed_dim;
+#pragma unroll
+                for (int d = 0; d < DT; d++) vf[d][u] = vr[16 * d];
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const uint32_t j = min(cs + 16u * (u >> 2) + 4u * g + (u & 3), nk - 1u);
+                const float *vr = v_row(j) + hsafe * HD + c;
+#pragma unroll
+                for (int d = 0; d < DT; d++) vf[d][u] = vr[16 * d];
+            }
+        }
+    };
+
+    auto sub_chunk = [&](auto touches_new_rows, float (&kf)[2][QD], float (&vf)[DT][8], uint32_t c0, uint32_t cnext,
+                         bool more) __attribute__((always_inline)) {
+        constexpr bool NEW = decltype(touches_new_rows)::value;
+        constexpr std::integral_constant<bool, !NEW> next_cached{};
+        float kc[2][QD]; /* this sub-chunk's K values; kf is handed to the next request at once */
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+#pragma unroll
+            for (int s = 0; s < QD; s += 4) {
+                float4 piece = make_float4(kf[t][s + 0], kf[t][s + 1], kf[t][s + 2], kf[t][s + 3]);
+                if constexpr (NEW) {
+                    const uint32_t j = c0 + 16u * t + c;
+                    if (a.rope_cos && j >= len && j < nk) { /* a new key row is rotated at its position j */
+                        const size_t at = (size_t)j * HALF + (g * QD + s) / 2;
+                        piece = rope_rotate4(piece, a.rope_cos + at, a.rope_sin + at);
+                    }
+                    if (a.write_through && head_ok && j >= len && j < k_end)
+                        *reinterpret_cast<float4 *>(a.cache_k + (slab + j) * a.embed_dim + head * HD + g * QD + s) =
+                            piece;
+                }
+                kc[t][s + 0] = piece.x, kc[t][s + 1] = piece.y, kc[t][s + 2] = piece.z, kc[t][s + 3] = piece.w;
+            }
+        }
+        if (more) request_k(next_cached, kf, cnext);
+        __builtin_amdgcn_sched_barrier(0); /* the requests stay ahead of the arithmetic */
+
+        floatx4 sacc[2];
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) sacc[t][r] = 0.f;
+#pragma unroll
+            for (int s = 0; s < QD; s++) sacc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kc[t][s], qf[s], sacc[t], 0, 0, 0);
+        }
+
+        float x[8];
+        float mt = neg_inf();
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const float t = sacc[u >> 2][u & 3] * scale2;
+            const uint32_t j = c0 + 16u * (u >> 2) + 4u * g + (u & 3);
+            const bool vis = ((j - vis_lo) < vis_len) & isfinite(t);
+            x[u] = vis ? t : neg_inf();
+            mt = fmaxf(mt, x[u]);
+        }
+        mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+        const float mn = fmaxf(m, mt);
+        const float ms = mn == neg_inf() ? 0.f : mn;
+        const float alpha = fast_exp2(m - ms);
+        float ps = 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            x[u] = fast_exp2(x[u] - ms);
+            ps += x[u];
+        }
+        l = l * alpha + ps;
+        m = mn;
+#pragma unroll
+        for (int d = 0; d < DT; d++) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) oacc[d][r] *= alpha;
+#pragma unroll
+            for (int u = 0; u < 8; u++) oacc[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[d][u], x[u], oacc[d], 0, 0, 0);
+        }
+
+        if constexpr (NEW) {
+            if (a.write_through && head_ok) {
+#pragma unroll
+                for (int u = 0; u < 8; u++) {
+                    const uint32_t j = c0 + 16u * (u >> 2) + 4u * g + (u & 3);
+                    if (j >= len && j < k_end) {
+#pragma unroll
+                        for (int d = 0; d < DT; d++)
+                            a.cache_v[(slab + j) * a.embed_dim + head * HD + 16 * d + c] = vf[d][u];
+                    }
+                }
+            }
+        }
+        if (more) request_v(next_cached, vf, cnext);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    constexpr std::false_type CACHED{};
+    constexpr std::true_type GENERAL{};
+
+    const uint32_t step = a.slices * 32u;
+    uint32_t c0 = k_begin + slice * 32u;
+    float kf[2][QD];
+    float vf[DT][8];
+    if (c0 < k_end) {
+        request_k(std::false_type{}, kf, c0);
+        request_v(std::false_type{}, vf, c0);
+    }
+    while (c0 + step + 32u <= len && c0 + step < k_end) { /* this and the next sub-chunk are cached rows */
+        sub_chunk(CACHED, kf, vf, c0, c0 + step, true);
+        c0 += step;
+    }
+    while (c0 < k_end) {
+        const uint32_t cn = c0 + step;
+        sub_chunk(GENERAL, kf, vf, c0, cn, cn < k_end);
+        c0 = cn;
+    }
+
+    /* the four lane groups of a column carry the same m, their sums add */
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+
+    /* lane (g, c) holds O^T[d = 16 dt + 4 g + r][query c]: park rows [query][HD columns, max, sum]
+     * in the wave's LDS tile, then merge the slices of each head as the 32-wide kernel does */
+    float *mine = sm_o[wave];
+#pragma unroll
+    for (int d = 0; d < DT; d++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) mine[c * PR + 16 * d + 4 * g + r] = oacc[d][r];
+    if (g == 0) {
+        mine[c * PR + HD + 0] = m * LN2; /* merges work in natural units */
+        mine[c * PR + HD + 1] = l;
+    }
+    __syncthreads();
+
+    const uint32_t rows = a.n - a.q0 < ROWS ? a.n - a.q0 : ROWS;
+    const uint32_t cells = a.hpb * rows * PR;
+    for (uint32_t t = threadIdx.x; t < cells; t += blockDim.x) {
+        const uint32_t col = t % PR;
+        const uint32_t r = (t / PR) % rows;
+        const uint32_t hl = t / (PR * rows);
+        const uint32_t hh = blockIdx.z * a.hpb + hl;
+        if (hh >= a.num_heads) continue;
+        float M = neg_inf();
+        for (uint32_t s = 0; s < a.slices; s++) M = fmaxf(M, sm_o[s * a.hpb + hl][r * PR + HD]);
+        float L = 0.f, acc = 0.f;
+        for (uint32_t s = 0; s < a.slices; s++) {
+            const float *ps = sm_o[s * a.hpb + hl] + r * PR;
+            const float f = ps[HD] == neg_inf() ? 0.f : softmax_exp(ps[HD] - M);
+            L += ps[HD + 1] * f;
+            if (col < (uint32_t)HD) acc += ps[col] * f;
+        }
+        if (a.splits == 1u) {
+            if (col < (uint32_t)HD)
+                a.combined[(newrow0 + a.q0 + r) * a.out_stride + hh * HD + col] = L > 0.f ? acc / L : 0.f;
+        } else {
+            float *dst = a.partial + ((((size_t)b * a.splits + split) * a.num_heads + hh) * SLOTS + r) * PR;
+            publish(dst + col, col < (uint32_t)HD ? acc : (col == (uint32_t)HD ? M : L));
+        }
+    }
+
+    kv_finish_sequence<HD>(a, (uint32_t)SLOTS, b, nk, &sm_ticket);
+}
+
 template <int HD, int WAVES>
 void launch_block(StepArgs a, uint32_t batch, hipStream_t s) {
     /* a.hpb heads per workgroup (the caller's choice, see kv_block_heads_per_group); the other waves are slices */
@@ -336,7 +622,15 @@ void launch_block(StepArgs a, uint32_t batch, hipStream_t s) {
     const uint32_t subs = (a.span + 31u) / 32u;
     a.slices = std::max(1u, std::min<uint32_t>((uint32_t)WAVES / a.hpb, subs));
     dim3 grid(a.splits, batch, (a.num_heads + a.hpb - 1) / a.hpb);
-    blt_launch("kv_block_mfma", kv_block_mfma_kernel<HD, WAVES>, grid, dim3(64 * a.hpb * a.slices), 0, s, a);
+    /* blocks of up to 16 rows on 16-wide tiles; BLT_HIP_BLOCK_TILE=32 keeps the 32-wide kernel (test hook) */
+    static const bool wide_only = [] {
+        const char *e = getenv("BLT_HIP_BLOCK_TILE");
+        return e && strcmp(e, "32") == 0;
+    }();
+    if (a.n - a.q0 <= 16u && !wide_only)
+        blt_launch("kv_block16_mfma", kv_block16_mfma_kernel<HD, WAVES>, grid, dim3(64 * a.hpb * a.slices), 0, s, a);
+    else
+        blt_launch("kv_block_mfma", kv_block_mfma_kernel<HD, WAVES>, grid, dim3(64 * a.hpb * a.slices), 0, s, a);
 }
 
 } // namespace
