@@ -439,10 +439,11 @@ void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_s
     a.partial = sc.partial;
     a.tickets = sc.tickets;
 
-    /* Blocks of four or more rows go to the matrix-core kernel (one launch for
-     * up to 32 rows; its cost does not depend on the row count) where it takes
-     * the head_dim; shorter blocks, single rows and the shapes it does not
-     * take go to the VALU kernel in slices of at most 16 rows.
+    /* Blocks of two or more rows go to the matrix-core kernels (one launch for
+     * up to 32 rows; the cost does not depend on the row count: measured 9.5 us
+     * at 64 sequences for 2 ... 16 rows against 9.9 / 14.6 us for 2 / 3 rows on
+     * the VALU kernel) where they take the head_dim; single rows and the shapes
+     * they do not take go to the VALU kernel in slices of at most 16 rows.
      * Every launch reads the new rows from the inputs, so only the first one
      * stores them and only the last one may advance the lengths.
      * BLT_HIP_BLOCK_KERNEL=valu|mfma pins the choice (tuning and test hook). */
@@ -450,7 +451,7 @@ void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_s
         const char *e = getenv("BLT_HIP_BLOCK_KERNEL");
         return e && strcmp(e, "valu") == 0 ? 1 : e && strcmp(e, "mfma") == 0 ? 2 : 0;
     }();
-    const bool want_mfma = pinned == 2 || (pinned == 0 && a.n >= 4u);
+    const bool want_mfma = pinned == 2 || (pinned == 0 && a.n >= 2u);
     if (want_mfma && (hd == 32 || hd == 64)) {
         /* the block kernel merges slices inside the workgroup, so it wants few,
          * long spans: just enough workgroups to cover the compute units */

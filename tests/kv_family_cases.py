@@ -39,6 +39,9 @@ CASES = {
     "chunk12_rope": lambda: chunked(12, True),
     "chunk20_rope_hd64": lambda: chunked(20, True, hd=64),
     "chunk6_rope_window": lambda: chunked(6, True, window=40),
+    "chunk9_rope_hd64_window": lambda: chunked(9, True, hd=64, window=33),
+    "chunk16": lambda: chunked(16, False),
+    "chunk17": lambda: chunked(17, False),
     "block8_rope": lambda: workloads.config5(batch=9, B=8, rope=True),
     "block16_rope_hd64": lambda: workloads.config5(batch=5, B=16, H=2, hd=64, rope=True),
 }

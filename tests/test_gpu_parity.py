@@ -411,16 +411,19 @@ def test_strided_copy_softmax_dot(oracle, dev):
     assert abs(got - float(np.dot(a.astype(np.float64), b.astype(np.float64)))) < 1e-3
 
 
-@pytest.mark.parametrize("kernel", ["valu", "mfma"])
+@pytest.mark.parametrize("kernel", ["valu", "mfma", "mfma32"])
 def test_kv_step_kernel_families_agree(kernel):
-    """Both kernels behind the KV step entry points (VALU and matrix-core) on the same cases -- block
-    rows, prefill chunks, rotation fused in or not -- pinned through BLT_HIP_BLOCK_KERNEL in a fresh
-    process (the hook is read once)."""
+    """The kernels behind the KV step entry points (VALU, matrix-core with 16-wide tiles for blocks of
+    up to 16 rows, matrix-core with 32-wide tiles only) on the same cases -- block rows, prefill
+    chunks, rotation fused in or not -- pinned through BLT_HIP_BLOCK_KERNEL / BLT_HIP_BLOCK_TILE in a
+    fresh process (the hooks are read once)."""
     import subprocess
     import sys
     import os
     here = os.path.dirname(os.path.abspath(__file__))
-    env = dict(os.environ, BLT_HIP_BLOCK_KERNEL=kernel)
+    env = dict(os.environ, BLT_HIP_BLOCK_KERNEL=kernel[:4])
+    if kernel == "mfma32":
+        env["BLT_HIP_BLOCK_TILE"] = "32"
     p = subprocess.run([sys.executable, "-u", os.path.join(here, "kv_family_cases.py")], capture_output=True,
                        text=True, timeout=600, env=env)
     assert p.returncode == 0 and "OK" in p.stdout, p.stdout[-2000:] + p.stderr[-2000:]
