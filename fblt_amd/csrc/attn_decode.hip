@@ -248,8 +248,27 @@ __global__ __launch_bounds__(64 * WAVES) void kv_step_kernel(StepArgs a) {
         }
     }
     __syncthreads();
+    /* every wave of the workgroup has long read the old length: draw the ticket now, look at it last */
+    const uint32_t early_ticket = kv_draw_early_ticket(a, b);
 
-    /* ---- merge the slices: thread t owns (local head, query, column) ---- */
+    /* ---- merge the slices, in two steps so that the exponentials are spread over all waves:
+     * every wave rescales its own parked state to the common maximum of its head's slices
+     * (nobody's maximum is overwritten), then thread t owns (local head, query, column) and adds
+     * the slices up ---- */
+    {
+        const uint32_t hl = wave % a.hpb;
+#pragma unroll
+        for (int r = 0; r < NQ; r++) {
+            float M = neg_inf();
+            for (uint32_t s = 0; s < a.slices; s++)
+                M = fmaxf(M, sm[((size_t)(s * a.hpb + hl) * NQ + r) * (HD + 2) + HD]);
+            const float own = mine[r * (HD + 2) + HD];
+            const float f = own == neg_inf() ? 0.f : softmax_exp(own - M);
+            for (uint32_t d = lane; d < (uint32_t)HD + 2u; d += 64u)
+                if (d != (uint32_t)HD) mine[r * (HD + 2) + d] *= f;
+        }
+    }
+    __syncthreads();
     const uint32_t cells = a.hpb * NQ * HD;
     for (uint32_t t = threadIdx.x; t < cells; t += blockDim.x) {
         const uint32_t d = t % HD;
@@ -258,15 +277,11 @@ __global__ __launch_bounds__(64 * WAVES) void kv_step_kernel(StepArgs a) {
         const uint32_t hh = blockIdx.z * a.hpb + hl;
         const uint32_t qi = a.q0 + r;
         if (hh >= a.num_heads || qi >= a.n) continue;
-        float M = neg_inf();
-        for (uint32_t s = 0; s < a.slices; s++)
-            M = fmaxf(M, sm[((size_t)(s * a.hpb + hl) * NQ + r) * (HD + 2) + HD]);
         float L = 0.f, acc = 0.f;
         for (uint32_t s = 0; s < a.slices; s++) {
             const float *ps = sm + ((size_t)(s * a.hpb + hl) * NQ + r) * (HD + 2);
-            const float f = ps[HD] == neg_inf() ? 0.f : softmax_exp(ps[HD] - M);
-            L += ps[HD + 1] * f;
-            acc += ps[d] * f;
+            L += ps[HD + 1];
+            acc += ps[d];
         }
         if (a.splits == 1u) {
             a.combined[((size_t)b * a.n + qi) * a.out_stride + hh * HD + d] = L > 0.f ? acc / L : 0.f;
@@ -274,13 +289,16 @@ __global__ __launch_bounds__(64 * WAVES) void kv_step_kernel(StepArgs a) {
             float *dst = a.partial + ((((size_t)b * a.splits + split) * a.num_heads + hh) * NQ + r) * (HD + 2);
             publish(dst + d, acc);
             if (d == 0) {
+                float M = neg_inf();
+                for (uint32_t s = 0; s < a.slices; s++)
+                    M = fmaxf(M, sm[((size_t)(s * a.hpb + hl) * NQ + r) * (HD + 2) + HD]);
                 publish(dst + HD + 0, M);
                 publish(dst + HD + 1, L);
             }
         }
     }
 
-    kv_finish_sequence<HD>(a, (uint32_t)NQ, b, nk, &sm_ticket);
+    kv_finish_sequence<HD>(a, (uint32_t)NQ, b, nk, &sm_ticket, early_ticket);
 }
 
 /* scratch the family owns: per-split softmax states and per-sequence tickets */

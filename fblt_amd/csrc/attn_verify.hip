@@ -301,6 +301,8 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block_mfma_kernel(StepArgs a
         my_k[c * PR + HD + 1] = l;
     }
     __syncthreads();
+    /* every wave of the workgroup has long read the old length: draw the ticket now, look at it last */
+    const uint32_t early_ticket = kv_draw_early_ticket(a, b);
 
     const uint32_t rows = a.n - a.q0 < (uint32_t)SLOTS ? a.n - a.q0 : (uint32_t)SLOTS;
     const uint32_t cells = a.hpb * rows * PR;
@@ -328,7 +330,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block_mfma_kernel(StepArgs a
         }
     }
 
-    kv_finish_sequence<HD>(a, (uint32_t)SLOTS, b, nk, &sm_ticket);
+    kv_finish_sequence<HD>(a, (uint32_t)SLOTS, b, nk, &sm_ticket, early_ticket);
 }
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -585,6 +587,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block16_mfma_kernel(StepArgs
         mine[c * PR + HD + 1] = l;
     }
     __syncthreads();
+    const uint32_t early_ticket = kv_draw_early_ticket(a, b); /* as in the 32-wide kernel */
 
     const uint32_t rows = a.n - a.q0 < ROWS ? a.n - a.q0 : ROWS;
     const uint32_t cells = a.hpb * rows * PR;
@@ -612,7 +615,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block16_mfma_kernel(StepArgs
         }
     }
 
-    kv_finish_sequence<HD>(a, (uint32_t)SLOTS, b, nk, &sm_ticket);
+    kv_finish_sequence<HD>(a, (uint32_t)SLOTS, b, nk, &sm_ticket, early_ticket);
 }
 
 template <int HD, int WAVES>

@@ -71,13 +71,36 @@ __device__ __forceinline__ float observe(const float *p) {
  * one die's L2 and no cache write-back or invalidate is needed; the barrier's
  * wait on outstanding memory operations orders the stores before this
  * workgroup's ticket. */
+/* The step commits, has one split per sequence but several workgroups (head
+ * groups): all that has to be known is when every workgroup of the sequence
+ * has read the old length.  Thread 0 of each workgroup draws its ticket at a
+ * point where all its waves have done that read (after the barrier that ends
+ * the key loop) -- the reply travels while the workgroup merges and stores --
+ * and the one that drew the last ticket writes the new length when it is done.  Returns
+ * the ticket (thread 0 only; KV_NO_TICKET when this scheme does not apply). */
+constexpr uint32_t KV_NO_TICKET = 0xFFFFFFFFu;
+__device__ __forceinline__ bool kv_early_ticket_applies(const StepArgs &a) {
+    return a.splits == 1u && gridDim.z > 1u && a.commit;
+}
+__device__ __forceinline__ uint32_t kv_draw_early_ticket(const StepArgs &a, uint32_t b) {
+    if (!kv_early_ticket_applies(a) || threadIdx.x != 0) return KV_NO_TICKET;
+    return __hip_atomic_fetch_add(&a.tickets[b], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 template <int HD>
 __device__ __forceinline__ void kv_finish_sequence(const StepArgs &a, uint32_t slots, uint32_t b, uint32_t nk,
-                                                   uint32_t *sm_ticket) {
+                                                   uint32_t *sm_ticket, uint32_t early_ticket) {
     if (a.splits == 1u && (gridDim.z == 1u || !a.commit)) {
         /* the output rows are written; the ticket is only needed to tell when the
          * last workgroup of the sequence has read the old length */
         if (a.commit && threadIdx.x == 0) a.self_len[b] = nk;
+        return;
+    }
+    if (kv_early_ticket_applies(a)) {
+        if (threadIdx.x == 0 && early_ticket == gridDim.z - 1u) {
+            a.tickets[b] = 0u; /* re-armed for the next launch */
+            a.self_len[b] = nk;
+        }
         return;
     }
     __syncthreads();
