@@ -67,7 +67,7 @@ __global__ __launch_bounds__(64 * WAVES) void kv_step_kernel(StepArgs a) {
     const uint32_t grp = lane / G;
     const bool head_ok = head < a.num_heads;
 
-    const uint32_t len = a.self_len[b];
+    const uint32_t len = a.self_len[b] + a.len_bias;
     const uint32_t nk = len + a.n;
     const size_t slab = (size_t)b * a.max_seq_len;
     const uint32_t col = (head_ok ? head : 0u) * HD + 4u * g;
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(64 * WAVES) void kv_step_kernel(StepArgs a) {
 #pragma unroll
     for (int r = 0; r < NQ; r++) {
         const uint32_t qi = min(a.q0 + r, a.n - 1u);
-        q[r] = *reinterpret_cast<const float4 *>(a.q_rows + ((size_t)b * a.n + qi) * a.q_stride + col);
+        q[r] = *reinterpret_cast<const float4 *>(a.q_rows + ((size_t)b * a.n_seq + qi) * a.q_stride + col);
         if (a.rope_cos) { /* the query sits at position len + qi */
             const size_t at = (size_t)(len + qi) * (HD / 2) + 2u * g;
             q[r] = rope_rotate4(q[r], a.rope_cos + at, a.rope_sin + at);
@@ -98,7 +98,7 @@ __global__ __launch_bounds__(64 * WAVES) void kv_step_kernel(StepArgs a) {
                 kf[t] = *reinterpret_cast<const float4 *>(a.cache_k + (slab + j) * a.embed_dim + col);
                 vf[t] = *reinterpret_cast<const float4 *>(a.cache_v + (slab + j) * a.embed_dim + col);
             } else {
-                const size_t r = (size_t)b * a.n + (j - len);
+                const size_t r = (size_t)b * a.n_seq + (j - len);
                 kf[t] = *reinterpret_cast<const float4 *>(a.k_rows + r * a.k_stride + col);
                 vf[t] = *reinterpret_cast<const float4 *>(a.v_rows + r * a.v_stride + col);
                 if (a.rope_cos) { /* a new key row is rotated at its own position j */
@@ -284,7 +284,7 @@ __global__ __launch_bounds__(64 * WAVES) void kv_step_kernel(StepArgs a) {
             acc += ps[d];
         }
         if (a.splits == 1u) {
-            a.combined[((size_t)b * a.n + qi) * a.out_stride + hh * HD + d] = L > 0.f ? acc / L : 0.f;
+            a.combined[((size_t)b * a.n_seq + qi) * a.out_stride + hh * HD + d] = L > 0.f ? acc / L : 0.f;
         } else {
             float *dst = a.partial + ((((size_t)b * a.splits + split) * a.num_heads + hh) * NQ + r) * (HD + 2);
             publish(dst + d, acc);
@@ -356,18 +356,44 @@ void dispatch_nq(const StepArgs &a, uint32_t nq, uint32_t batch, hipStream_t s) 
 
 namespace {
 
+/* One launch set for at most 32 new rows per sequence: rows [row0, row0 + n) of a step of
+ * n_seq rows per sequence, the row pointers already advanced to row0. */
+void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride, const float *k_rows,
+                   size_t k_stride, const float *v_rows, size_t v_stride, const float *rope_cos,
+                   const float *rope_sin, float *combined, size_t combined_stride, size_t n, size_t n_seq,
+                   size_t row0, int step_kind, int commit, size_t max_len_hint);
+
 void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride, const float *k_rows,
                  size_t k_stride, const float *v_rows, size_t v_stride, const float *rope_cos, const float *rope_sin,
                  float *combined, size_t combined_stride, size_t n, int step_kind, int commit, size_t max_len_hint) {
-    BLT_REQUIRE(cache != NULL && cache->self_k != NULL && cache->self_v != NULL && cache->self_len != NULL,
-                "blt_kv_attend_step: cache buffers must not be NULL");
     BLT_REQUIRE(q_rows != NULL && k_rows != NULL && v_rows != NULL && combined != NULL,
                 "blt_kv_attend_step: row buffers must not be NULL");
     BLT_REQUIRE(n >= 1, "blt_kv_attend_step: need at least one row");
-    BLT_REQUIRE(n <= 32, "blt_kv_attend_step: at most 32 new rows per sequence and step "
-                         "(longer prefill chunks go through blt_attention_batch_hip)");
     BLT_REQUIRE(step_kind == BLT_KV_STEP_CAUSAL || step_kind == BLT_KV_STEP_BLOCK,
                 "blt_kv_attend_step: unknown step_kind");
+    BLT_REQUIRE(n <= 32 || step_kind == BLT_KV_STEP_CAUSAL,
+                "blt_kv_attend_step: a block step takes at most 32 rows per sequence (every row sees every "
+                "new row, so the block cannot be cut)");
+    BLT_REQUIRE(max_len_hint >= n, "blt_kv_attend_step: exceeds cache capacity");
+    /* A causal chunk longer than 32 rows (a prompt prefill) runs as consecutive 32-row slices: a
+     * slice's rows see the cache, the earlier slices' rows (written through by then) and their
+     * own; only the last slice advances the lengths. */
+    for (size_t row0 = 0; row0 < n; row0 += 32) {
+        const size_t rows = std::min<size_t>(32, n - row0);
+        const bool last = row0 + rows == n;
+        kv_step_slice(cache, q_rows + row0 * q_stride, q_stride, k_rows + row0 * k_stride, k_stride,
+                      v_rows + row0 * v_stride, v_stride, rope_cos, rope_sin, combined + row0 * combined_stride,
+                      combined_stride, rows, n, row0, step_kind, last ? commit : 0,
+                      max_len_hint - (n - row0 - rows));
+    }
+}
+
+void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride, const float *k_rows,
+                   size_t k_stride, const float *v_rows, size_t v_stride, const float *rope_cos,
+                   const float *rope_sin, float *combined, size_t combined_stride, size_t n, size_t n_seq,
+                   size_t row0, int step_kind, int commit, size_t max_len_hint) {
+    BLT_REQUIRE(cache != NULL && cache->self_k != NULL && cache->self_v != NULL && cache->self_len != NULL,
+                "blt_kv_attend_step: cache buffers must not be NULL");
     const size_t E = cache->embed_dim, H = cache->num_heads;
     BLT_REQUIRE(H >= 1 && E % H == 0, "blt_kv_attend_step: embed_dim must be divisible by num_heads");
     const size_t hd = E / H;
@@ -402,6 +428,8 @@ void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_s
     a.num_heads = (uint32_t)H;
     a.window = (uint32_t)cache->window;
     a.n = (uint32_t)n;
+    a.n_seq = (uint32_t)n_seq;
+    a.len_bias = (uint32_t)row0;
     a.scale = 1.0f / sqrtf((float)hd);
     a.block_kind = step_kind == BLT_KV_STEP_BLOCK;
     a.hpb = 0, a.slices = 1;

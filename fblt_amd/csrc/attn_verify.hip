@@ -67,13 +67,13 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block_mfma_kernel(StepArgs a
     const uint32_t h = lane >> 5;
     const uint32_t c = lane & 31u;
 
-    const uint32_t len = a.self_len[b];
+    const uint32_t len = a.self_len[b] + a.len_bias;
     const uint32_t nk = len + a.n;
     const size_t slab = (size_t)b * a.max_seq_len;
     const uint32_t span = kv_span_of(a, nk);
     const uint32_t k_begin = split * span;
     const uint32_t k_end = min(k_begin + span, nk);
-    const size_t newrow0 = (size_t)b * a.n;
+    const size_t newrow0 = (size_t)b * a.n_seq;
 
     /* query fragment: row c of the block (clamped), floats [h*HALF, (h+1)*HALF) of the head */
     const uint32_t qi = a.q0 + c;
@@ -370,13 +370,13 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block16_mfma_kernel(StepArgs
     const uint32_t g = lane >> 4;
     const uint32_t c = lane & 15u;
 
-    const uint32_t len = a.self_len[b];
+    const uint32_t len = a.self_len[b] + a.len_bias;
     const uint32_t nk = len + a.n;
     const size_t slab = (size_t)b * a.max_seq_len;
     const uint32_t span = kv_span_of(a, nk);
     const uint32_t k_begin = split * span;
     const uint32_t k_end = min(k_begin + span, nk);
-    const size_t newrow0 = (size_t)b * a.n;
+    const size_t newrow0 = (size_t)b * a.n_seq;
 
     /* query fragment: row c of the block (clamped), columns [g*QD, (g+1)*QD) of the head */
     const uint32_t qi = a.q0 + c;

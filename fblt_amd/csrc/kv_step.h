@@ -28,7 +28,11 @@ struct StepArgs {
     uint32_t q_stride, k_stride, v_stride, out_stride;
     uint32_t max_seq_len, embed_dim, num_heads;
     uint32_t window;
-    uint32_t n;        /* new rows per sequence */
+    uint32_t n;        /* new rows per sequence this launch works on */
+    uint32_t n_seq;    /* rows per sequence in the row arrays: sequence b's rows start at row b * n_seq
+                          (the row pointers are already advanced to this launch's first row) */
+    uint32_t len_bias; /* rows of the same step already written through by earlier launches:
+                          the sequence's length for this launch is self_len[b] + len_bias */
     uint32_t q0;       /* first query row this launch handles */
     uint32_t splits;   /* gridDim.x */
     uint32_t span;     /* keys per split, a multiple of SUB */
@@ -138,7 +142,7 @@ __device__ __forceinline__ void kv_finish_sequence(const StepArgs &a, uint32_t s
                 L += pl[s] * f;
                 acc += po[s] * f;
             }
-            a.combined[((size_t)b * a.n + qi) * a.out_stride + hh * HD + d] = L > 0.f ? acc / L : 0.f;
+            a.combined[((size_t)b * a.n_seq + qi) * a.out_stride + hh * HD + d] = L > 0.f ? acc / L : 0.f;
         }
     }
     if (threadIdx.x == 0) {

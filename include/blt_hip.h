@@ -289,7 +289,10 @@ enum {
  * v_rows and combined are [batch*n, *] with the given row strides (elements);
  * K rows are already rotated.  max_len_hint >= max_b(self_len[b]) + n sizes
  * the launch (the host knows it, as the reference's host-side self_len does);
- * sequences shorter than the hint simply leave blocks idle. */
+ * sequences shorter than the hint simply leave blocks idle.  A causal step
+ * of more than 32 rows per sequence (a prompt prefill) is run as consecutive
+ * 32-row slices; a block step takes at most 32 rows (the reference's
+ * BLT_BLOCKGEN_MAX_B, csrc/infer/block_generation.c:154). */
 void blt_kv_attend_step_hip(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride,
                             const float *k_rows, size_t k_stride, const float *v_rows, size_t v_stride,
                             float *combined, size_t combined_stride, size_t n, int step_kind, int commit,

@@ -42,6 +42,8 @@ CASES = {
     "chunk9_rope_hd64_window": lambda: chunked(9, True, hd=64, window=33),
     "chunk16": lambda: chunked(16, False),
     "chunk17": lambda: chunked(17, False),
+    "chunk40_rope": lambda: chunked(40, True),                  # longer than one launch takes: 32 + 8 rows
+    "chunk70_window_hd64": lambda: chunked(70, True, hd=64, window=50),
     "block8_rope": lambda: workloads.config5(batch=9, B=8, rope=True),
     "block16_rope_hd64": lambda: workloads.config5(batch=5, B=16, H=2, hd=64, rope=True),
 }

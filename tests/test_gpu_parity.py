@@ -889,6 +889,53 @@ def test_kv_decode_step_single_sequence(case, oracle, dev):
         lib.blt_arena_destroy(arena)
 
 
+def test_kv_decode_step_long_prefill(oracle, dev):
+    """A prompt prefill in one call: more new rows than one attention launch takes (45, then 1, then
+    50 rows), against the restated step; logits and tiers after every call."""
+    import torch
+    from fblt_amd import decoder
+    lib = api.load()
+    c = dict(E=128, H=4, XH=4, L=2, hidden=256, V=256, max_len=128, k=1, window=0, all_layers=True, placement=0)
+    E, V, L = c["E"], c["V"], c["L"]
+    rs = np.random.RandomState(911)
+    host, device = _decoders(oracle, c, 912)
+    mine = decoder.HostCache(host, c["max_len"])
+    arena = lib.blt_arena_create(64 << 20, abi.BLT_BACKEND_HIP)
+    try:
+        cache = lib.blt_kv_cache_create(arena, device.ptr, c["max_len"])
+        mark = arena.contents.offset
+        lengths = [5, 7, 3, 9, 6, 8, 4, 10, 2, 9, 7, 11, 15]      # 96 bytes
+        P = len(lengths)
+        patches = decoder.patch_table(lengths)
+        patch_in = rs.randn(P, E).astype(np.float32)
+        tp = torch.from_numpy(patch_in).cuda()
+        vp = _dev_tensor(tp)
+        lib.blt_kv_cache_refresh_cross(cache, C.byref(vp), patches, P, 0, arena)
+        assert oracle.orc_kv_cache_refresh_cross(mine.ptr, 0, binding.fptr(patch_in.reshape(-1)), P, 0) == 0
+        done = 0
+        for n in (45, 1, 50):
+            rows = rs.randn(n, E).astype(np.float32)
+            ref = np.zeros((n, V), dtype=np.float32)
+            assert oracle.orc_kv_decode_step(mine.ptr, 0, done, patches, P, binding.fptr(rows.reshape(-1)), n, 0,
+                                             binding.fptr(ref.reshape(-1))) == 0
+            td = torch.from_numpy(rows).cuda()
+            tl = torch.full((n, V), 7.0, dtype=torch.float32, device="cuda")
+            vd, vl = _dev_tensor(td), _dev_tensor(tl)
+            arena.contents.offset = mark
+            lib.blt_kv_decode_step(cache, C.byref(vp), patches, P, C.byref(vd), 0, C.byref(vl), arena)
+            lib.blt_backend_pass_sync_hip()
+            done += n
+            assert cache.contents.self_len == done
+            assert_close(tl.cpu().numpy(), ref, "long prefill logits n=%d" % n)
+            for name in ("self_k", "self_v"):
+                for l in range(L):
+                    assert_close(_tier(lib, cache, name, l, c["max_len"], E), mine.tiers[name][l],
+                                 "%s[%d] after %d rows" % (name, l, done))
+        lib.blt_kv_cache_destroy(cache)
+    finally:
+        lib.blt_arena_destroy(arena)
+
+
 @pytest.mark.parametrize("batch,n,case", [(8, 1, 0), (64, 1, 2), (16, 4, 1), (5, 3, 3), (64, 8, 2)])
 def test_kv_decode_step_batched(batch, n, case, oracle, dev):
     """blt_kv_decode_step_batched_hip: every sequence of a batched cache in one pass, against the
