@@ -174,8 +174,9 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_kernel(MatmulArgs g) {
                      make_float4(acc[4 * q + 0], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]), vst);
 }
 
-/* 32x32 output tile (bx, by) per workgroup, K split over the four waves. */
-template <bool VEC, bool ROPE, bool GATED>
+/* 32x32 output tile (bx, by) per workgroup, K split over the NW waves (4, or 8 for long K:
+ * the serial chain of chunk loads per wave halves); the first four waves finish the tile. */
+template <bool VEC, bool ROPE, bool GATED, int NW = 4>
 __device__ __forceinline__ void splitk_tile(const MatmulArgs &g, const uint32_t bx, const uint32_t by,
                                             float (*part)[16][64], float (*part_ss)[32]) {
     const uint32_t lane = threadIdx.x & 63u;
@@ -245,7 +246,7 @@ __device__ __forceinline__ void splitk_tile(const MatmulArgs &g, const uint32_t 
         else fetch(ch * 32u, fa, fb, dummy);
     }
     while (ch < chunks) {
-        const uint32_t nx = ch + 4u;
+        const uint32_t nx = ch + (uint32_t)NW;
         float na[16], nb[16], ng[GATED ? 16 : 1];
         if (nx < chunks) {
             if constexpr (GATED) fetch(nx * 32u, na, nb, ng);
@@ -267,27 +268,35 @@ __device__ __forceinline__ void splitk_tile(const MatmulArgs &g, const uint32_t 
 #pragma unroll
     for (int r = 0; r < 16; r++) {
         part[wave][r][lane] = acc[r];
-        if (GATED) part[4 + wave][r][lane] = acc2[r];
+        if (GATED) part[NW + wave][r][lane] = acc2[r];
     }
     if (g.norm_w) {
         ss += __shfl_xor(ss, 32, 64);
         if (h == 0) part_ss[wave][c] = ss;
     }
     __syncthreads();
+    if (NW > 4 && wave >= 4u) return; /* no barrier follows */
     float row_scale = 1.0f;
     if (g.norm_w) {
-        const float tot = (part_ss[0][c] + part_ss[1][c]) + (part_ss[2][c] + part_ss[3][c]);
+        float tot = (part_ss[0][c] + part_ss[1][c]) + (part_ss[2][c] + part_ss[3][c]);
+        if (NW > 4) tot += (part_ss[4][c] + part_ss[5][c]) + (part_ss[6][c] + part_ss[7][c]);
         row_scale = 1.0f / sqrtf(tot / (float)g.k + 1e-6f); /* reductions_cpu.c:345-346 */
     }
-    /* wave w finishes register group w: out[row][col0 + 8w + 4h + 0..3] */
+    /* wave w < 4 finishes register group w: out[row][col0 + 8w + 4h + 0..3] */
+    auto total = [&](uint32_t first, uint32_t reg) __attribute__((always_inline)) {
+        float t = (part[first + 0][reg][lane] + part[first + 1][reg][lane]) +
+                  (part[first + 2][reg][lane] + part[first + 3][reg][lane]);
+        if (NW > 4)
+            t += (part[first + 4][reg][lane] + part[first + 5][reg][lane]) +
+                 (part[first + 6][reg][lane] + part[first + 7][reg][lane]);
+        return t;
+    };
     float v4[4], second[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        v4[i] = ((part[0][4 * wave + i][lane] + part[1][4 * wave + i][lane]) +
-                 (part[2][4 * wave + i][lane] + part[3][4 * wave + i][lane])) * row_scale;
+        v4[i] = total(0u, 4u * wave + i) * row_scale;
         if (GATED) {
-            const float gate = ((part[4][4 * wave + i][lane] + part[5][4 * wave + i][lane]) +
-                                (part[6][4 * wave + i][lane] + part[7][4 * wave + i][lane])) * row_scale;
+            const float gate = total((uint32_t)NW, 4u * wave + i) * row_scale;
             if (g.out2) second[i] = gate; /* two products, two outputs */
             else v4[i] = silu_times(gate, v4[i]);
         }
@@ -306,11 +315,11 @@ __device__ __forceinline__ void splitk_tile(const MatmulArgs &g, const uint32_t 
     }
 }
 
-template <bool VEC, bool ROPE, bool GATED>
-__global__ __launch_bounds__(256, 2) void matmul_splitk_kernel(MatmulArgs g) {
-    __shared__ float part[GATED ? 8 : 4][16][64];
-    __shared__ float part_ss[4][32];
-    splitk_tile<VEC, ROPE, GATED>(g, blockIdx.x, blockIdx.y, part, part_ss);
+template <bool VEC, bool ROPE, bool GATED, int NW = 4>
+__global__ __launch_bounds__(64 * NW, 2) void matmul_splitk_kernel(MatmulArgs g) {
+    __shared__ float part[(GATED ? 2 : 1) * NW][16][64];
+    __shared__ float part_ss[NW][32];
+    splitk_tile<VEC, ROPE, GATED, NW>(g, blockIdx.x, blockIdx.y, part, part_ss);
 }
 
 /* Two independent products in one launch: the tile rows of the second are
@@ -379,7 +388,10 @@ Path choose_path(const MatmulArgs &g) {
 
 template <bool VEC, bool ROPE>
 void launch_splitk(const MatmulArgs &g, dim3 grid, hipStream_t s) {
+    /* eight waves once every wave still gets a chunk (K >= 256) and the launch leaves the chip room for them */
+    const bool eight = g.k >= 256u && (uint64_t)grid.x * grid.y <= 512u;
     if (g.b2) blt_launch("matmul_splitk", matmul_splitk_kernel<VEC, ROPE, true>, grid, dim3(256), 0, s, g);
+    else if (eight) blt_launch("matmul_splitk", matmul_splitk_kernel<VEC, ROPE, false, 8>, grid, dim3(512), 0, s, g);
     else blt_launch("matmul_splitk", matmul_splitk_kernel<VEC, ROPE, false>, grid, dim3(256), 0, s, g);
 }
 
