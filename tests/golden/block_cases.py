@@ -1,0 +1,77 @@
+"""Seeded inputs of the block-level golden cases (attention block, cross-attention block, whole
+decoder step).  Shared by the generator (make_golden_blocks.py, which feeds them to the reference
+build) and by the tests (which feed them to the CPU checker and to the HIP library)."""
+import numpy as np
+
+from fblt_amd import decoder
+
+MHA_CASES = {
+    # T, E, H, rope, mask ("causal_flag", "causal_cfg", "window", "docs")
+    "mha_T96_E64_H2_rope": dict(T=96, E=64, H=2, rope=True, mask="causal_cfg"),
+    "mha_T50_E48_H3_window": dict(T=50, E=48, H=3, rope=True, mask="window"),
+    "mha_T33_E32_H4_docs": dict(T=33, E=32, H=4, rope=False, mask="docs"),
+}
+XATTN_CASES = {
+    "xattn_P16_T64_E64_H2": dict(P=16, T=64, E=64, H=2),
+    "xattn_P40_T150_E32_H4": dict(P=40, T=150, E=32, H=4),
+}
+STEP_CASES = {
+    # decoder configuration and a script of (patch lengths so far, from_patch, new rows, trailing_closed)
+    "step_E64_L2_k2_window": dict(E=64, H=2, XH=2, L=2, hidden=96, V=64, max_len=48, k=2, window=9,
+                                  all_layers=True, placement=0),
+    "step_E32_L3_last_only": dict(E=32, H=4, XH=1, L=3, hidden=48, V=256, max_len=40, k=1, window=0,
+                                  all_layers=False, placement=0),
+}
+STEP_SCRIPT = [([3, 4], 0, 7, 0), ([3, 4, 1], 2, 1, 0), ([3, 4, 2], 2, 1, 1), ([3, 4, 2, 5], 3, 5, 0),
+               ([3, 4, 2, 5, 1], 4, 1, 0), ([3, 4, 2, 5, 4], 4, 3, 1), ([3, 4, 2, 5, 4, 3], 5, 3, 0)]
+THETA = 500000.0
+
+
+def seed_of(name):
+    return sum(ord(ch) * (i + 1) for i, ch in enumerate(name)) % (2 ** 31)
+
+
+def mha_inputs(name):
+    c = MHA_CASES[name]
+    rs = np.random.RandomState(seed_of(name))
+    T, E = c["T"], c["E"]
+    x = rs.randn(T, E).astype(np.float32)
+    wqkv = (rs.randn(E, 3 * E) / np.sqrt(E)).astype(np.float32)
+    wproj = (rs.randn(E, E) / np.sqrt(E)).astype(np.float32)
+    return c, x, wqkv, wproj
+
+
+def mha_mask(c):
+    """(is_causal, sliding_window, doc boundary list or None) of the case's mask configuration."""
+    if c["mask"] == "window":
+        return True, 11, None
+    if c["mask"] == "docs":
+        return False, 0, [9, 20]
+    return True, 0, None
+
+
+def xattn_inputs(name):
+    c = XATTN_CASES[name]
+    rs = np.random.RandomState(seed_of(name))
+    P, T, E = c["P"], c["T"], c["E"]
+    xq, xkv = rs.randn(P, E).astype(np.float32), rs.randn(T, E).astype(np.float32)
+    ws = [(rs.randn(E, E) / np.sqrt(E)).astype(np.float32) for _ in range(4)]
+    groups = np.sort(np.concatenate([np.arange(P), rs.randint(0, P, size=T - P)]))
+    return c, xq, xkv, ws, groups
+
+
+def step_inputs(name):
+    """Decoder weights, the rows of every call of the script and the patch latents per call."""
+    c = STEP_CASES[name]
+    rs = np.random.RandomState(seed_of(name))
+    weights = decoder.random_weights(c["E"], c["hidden"], c["L"], c["V"], seed_of(name) + 1)
+    total = sum(n for _l, _f, n, _c in STEP_SCRIPT)
+    d0 = rs.randn(total, c["E"]).astype(np.float32)
+    latents, prev = [], None
+    for lengths, from_patch, _n, _closed in STEP_SCRIPT:
+        pin = rs.randn(len(lengths), c["k"] * c["E"]).astype(np.float32)
+        if from_patch:
+            pin[:from_patch] = prev[:from_patch]   # completed patches keep their latents
+        latents.append(pin)
+        prev = pin
+    return c, weights, d0, latents

@@ -1,0 +1,134 @@
+"""Writes tests/golden/blocks_golden.npz from the reference build (oracle/_ref):
+blt_multihead_attention, blt_cross_attention_forward and the script of
+blt_kv_cache_refresh_cross + blt_kv_decode_step calls of block_cases.py.
+
+Run in a container that holds the reference sources:
+    make -C oracle ref && python tests/golden/make_golden_blocks.py
+
+Stored per case: SHA-256 of the full outputs (bit-exact check for the CPU checker) and up to
+4096 sampled values (tolerance check for the GPU path).  Inputs are regenerated from the seed.
+"""
+import ctypes as C
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+
+from fblt_amd import abi, decoder  # noqa: E402
+from oracle import binding  # noqa: E402
+from tests.golden import block_cases as bc  # noqa: E402
+from tests.golden.make_golden import pack  # noqa: E402
+
+CPU = abi.BLT_BACKEND_CPU
+
+
+def view(a):
+    return abi.tensor_view(a.ctypes.data, a.shape, CPU)
+
+
+def rope_tables(ref, rows, hd):
+    cos, sin = np.zeros((rows, hd // 2), dtype=np.float32), np.zeros((rows, hd // 2), dtype=np.float32)
+    vc, vs = view(cos), view(sin)
+    cfg = binding.BltRopeConfig(bc.THETA, hd)
+    ref.blt_rope_precompute(rows, C.byref(cfg), C.byref(vc), C.byref(vs))
+    return cos, sin
+
+
+def run_mha(ref, arena, name):
+    c, x, wqkv, wproj = bc.mha_inputs(name)
+    T, E, H = c["T"], c["E"], c["H"]
+    causal, window, docs = bc.mha_mask(c)
+    cfg = abi.BltMaskConfig()
+    cfg.seq_len_q = cfg.seq_len_kv = T
+    cfg.is_causal, cfg.sliding_window = causal, window
+    keep = abi.size_array(docs) if docs else None
+    if docs:
+        cfg.doc_boundaries, cfg.num_docs = keep, len(docs) + 1
+    ac = abi.BltAttentionConfig()
+    ac.embed_dim, ac.num_heads, ac.head_dim = E, H, E // H
+    ac.use_rope, ac.rope_theta, ac.mask_config = c["rope"], bc.THETA, C.pointer(cfg)
+    out = np.zeros((T, E), dtype=np.float32)
+    tx, tq, tp, to = view(x), view(wqkv), view(wproj), view(out)
+    arena.contents.offset = 0
+    ref.blt_multihead_attention(C.byref(tx), C.byref(tq), C.byref(tp), C.byref(to), C.byref(ac), arena)
+    return out
+
+
+def run_xattn(ref, arena, name):
+    c, xq, xkv, ws, groups = bc.xattn_inputs(name)
+    P, T, E, H = c["P"], c["T"], c["E"], c["H"]
+    cfg = abi.BltMaskConfig()
+    cfg.seq_len_q, cfg.seq_len_kv = P, T
+    keep = (abi.size_array(list(range(P))), abi.size_array(groups.tolist()))
+    cfg.query_group_ids, cfg.kv_group_ids, cfg.bidirectional_within_group = keep[0], keep[1], True
+    out = np.zeros((P, E), dtype=np.float32)
+    tq, tkv, to = view(xq), view(xkv), view(out)
+    tw = [view(w) for w in ws]
+    wts = abi.BltCrossAttentionWeights(*(C.pointer(t) for t in tw))
+    cc = abi.BltCrossAttentionConfig()
+    cc.embed_dim, cc.num_heads, cc.head_dim, cc.mask_config = E, H, E // H, C.pointer(cfg)
+    arena.contents.offset = 0
+    ref.blt_cross_attention_forward(C.byref(tq), C.byref(tkv), C.byref(wts), C.byref(to), C.byref(cc), arena)
+    return out
+
+
+def run_step(ref, arena, name):
+    c, weights, d0, latents = bc.step_inputs(name)
+    E, V = c["E"], c["V"]
+    cos, sin = rope_tables(ref, c["max_len"], E // c["H"])
+    bound = decoder.bind(weights, cos, sin, CPU, decoder.host_place, E, c["H"], c["XH"], c["hidden"], V, c["max_len"],
+                         patch_dim=c["k"] * E, window=c["window"], all_layers=c["all_layers"],
+                         placement=c["placement"], theta=bc.THETA)
+    arena.contents.offset = 0
+    cache = ref.blt_kv_cache_create_batched(arena, bound.ptr, c["max_len"], 1)
+    mark = arena.contents.offset
+    logits, done = [], 0
+    for (lengths, from_patch, n, closed), pin in zip(bc.STEP_SCRIPT, latents):
+        P = len(lengths)
+        patches = decoder.patch_table(lengths)
+        tp = view(pin)
+        ref.blt_kv_cache_truncate(cache, cache.contents.self_len, min(from_patch, cache.contents.cross_num_patches))
+        arena.contents.offset = mark
+        ref.blt_kv_cache_refresh_cross(cache, C.byref(tp), patches, P, from_patch, arena)
+        rows = np.ascontiguousarray(d0[done:done + n])
+        out = np.zeros((n, V), dtype=np.float32)
+        td, tl = view(rows), view(out)
+        ref.blt_kv_decode_step(cache, C.byref(tp), patches, P, C.byref(td), closed, C.byref(tl), arena)
+        logits.append(out)
+        done += n
+    tiers = {}
+    for tier in ("self_k", "self_v", "cross_k", "cross_v"):
+        tiers[tier] = np.stack([np.ctypeslib.as_array(C.cast(getattr(cache.contents, tier)[l].data,
+                                                             C.POINTER(C.c_float)), shape=(c["max_len"], E)).copy()
+                                for l in range(c["L"])])
+    ref.blt_kv_cache_destroy(cache)
+    return np.concatenate(logits), tiers
+
+
+def main():
+    ref = binding.load_ref()
+    if ref is None:
+        raise SystemExit("oracle/_ref/libblt_ref.so is missing: run `make -C oracle ref` first")
+    rs = np.random.RandomState(20240701)
+    store = {}
+    arena = ref.blt_arena_create(64 << 20, CPU)
+    for name in bc.MHA_CASES:
+        pack(store, name + "/out", run_mha(ref, arena, name), rs)
+    for name in bc.XATTN_CASES:
+        pack(store, name + "/out", run_xattn(ref, arena, name), rs)
+    for name in bc.STEP_CASES:
+        logits, tiers = run_step(ref, arena, name)
+        pack(store, name + "/logits", logits, rs)
+        for tier, arr in tiers.items():
+            pack(store, name + "/" + tier, arr, rs)
+    ref.blt_arena_destroy(arena)
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "blocks_golden.npz")
+    np.savez_compressed(path, **store)
+    print(path, os.path.getsize(path), "bytes")
+
+
+if __name__ == "__main__":
+    main()
