@@ -13,7 +13,8 @@
  *    is bit-identical to blt_matmul_cpu.
  *
  *  - "mfma" (everything else): 64x64 output tiles per workgroup of four
- *    wavefronts, K in steps of 32 through double-buffered LDS tiles,
+ *    wavefronts (128x128, four MFMA tiles per wavefront, once there are 512
+ *    such tiles), K in steps of 32 (16) through double-buffered LDS tiles,
  *    v_mfma_f32_32x32x2_f32 accumulation.  The product is accumulated
  *    TRANSPOSED (MFMA A operand = b tile, B operand = a tile), which puts one
  *    output ROW in each lane with four consecutive columns per register
@@ -38,14 +39,13 @@
 #include "matmul.h"
 
 #include <stdint.h>
+#include <stdlib.h>
 
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int TM = 64, TN = 64, TK = 32;
-constexpr int A_PITCH = TK + 4; /* floats per LDS row of the a tile: 16-byte fragment reads of 32 rows hit all banks */
-constexpr int B_PITCH = TN + 4;
+constexpr int TM = 64, TN = 64, TK = 32; /* smallest workgroup tile of the mfma kernel */
 
 __device__ __forceinline__ float silu_times(float gate, float up) {
     const float silu = gate / (1.0f + expf(-gate));
@@ -79,99 +79,139 @@ __device__ __forceinline__ void store4(const MatmulArgs &g, uint32_t row, uint32
     }
 }
 
-/* VEC: a, b 16-byte aligned with lda, ldb, K, N multiples of 4, so a 16-byte
+/* One (64*WT)x(64*WT) output tile per workgroup of four wavefronts; each wave owns a quadrant of
+ * WT x WT MFMA tiles.  WT = 2 is for products large enough to give every compute unit several
+ * 128x128 tiles: a fragment read from LDS then feeds two matrix instructions, the four
+ * accumulators of a wave are independent, and operands come from L2 half as often.
+ * K in steps of 32/WT through double-buffered LDS tiles.
+ * VEC: a, b 16-byte aligned with lda, ldb, K, N multiples of 4, so a 16-byte
  * piece is either entirely inside or entirely outside the matrices.
  * ROPE: rotate pairs of the first g.rope_cols columns in the epilogue. */
-template <bool VEC, bool ROPE>
+template <bool VEC, bool ROPE, int WT>
 __global__ __launch_bounds__(256, 2) void matmul_mfma_kernel(MatmulArgs g) {
-    __shared__ __attribute__((aligned(16))) float sa[2][TM * A_PITCH];
-    __shared__ __attribute__((aligned(16))) float sb[2][TK * B_PITCH];
+    constexpr int BM = TM * WT, BN = TN * WT, BK = TK / WT, KH = BK / 2;
+    constexpr int AP = BK + 4; /* floats per LDS row of the a tile: 16-byte fragment reads of 32 rows hit all banks */
+    constexpr int BP = BN + 4;
+    __shared__ __attribute__((aligned(16))) float sa[2][BM * AP];
+    __shared__ __attribute__((aligned(16))) float sb[2][BK * BP];
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
     const uint32_t h = lane >> 5, c = lane & 31u;
-    const uint32_t wr = wave >> 1, wc = wave & 1u; /* wave's 32x32 quadrant of the tile */
-    const uint32_t row0 = blockIdx.y * TM, col0 = blockIdx.x * TN;
+    const uint32_t wr = wave >> 1, wc = wave & 1u; /* wave's quadrant of the tile */
+    const uint32_t row0 = blockIdx.y * BM, col0 = blockIdx.x * BN;
 
-    /* pieces of 4 floats this thread moves per K step: two of the a tile, two of the b tile */
+    /* pieces of 4 floats this thread moves per K step: two of the a tile, two of the b tile.
+     * Loads go to clamped addresses and land in registers untouched; pieces outside the matrices
+     * are zeroed only when they are parked in LDS, after the step's matrix instructions, so that
+     * nothing between the requests and those instructions waits for memory. */
     float pa[2][4], pb[2][4];
     auto request = [&](uint32_t k0) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             const uint32_t e = threadIdx.x + 256u * u;
             {
-                const uint32_t r = row0 + e / (TK / 4), k = k0 + 4u * (e % (TK / 4));
-                const float *src = g.a + (size_t)min(r, g.m - 1u) * g.lda + k;
+                const uint32_t r = row0 + e / (BK / 4), k = k0 + 4u * (e % (BK / 4));
+                const float *src = g.a + (size_t)min(r, g.m - 1u) * g.lda;
                 if (VEC) {
-                    float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-                    if (k < g.k) t = *reinterpret_cast<const float4 *>(src);
+                    const float4 t = *reinterpret_cast<const float4 *>(src + min(k, g.k - 4u));
                     pa[u][0] = t.x, pa[u][1] = t.y, pa[u][2] = t.z, pa[u][3] = t.w;
                 } else {
 #pragma unroll
-                    for (int i = 0; i < 4; i++) pa[u][i] = k + i < g.k ? src[i] : 0.f;
+                    for (int i = 0; i < 4; i++) pa[u][i] = src[min(k + i, g.k - 1u)];
                 }
             }
             {
-                const uint32_t k = k0 + e / (TN / 4), col = col0 + 4u * (e % (TN / 4));
-                const float *src = g.b + (size_t)min(k, g.k - 1u) * g.ldb + col;
+                const uint32_t k = k0 + e / (BN / 4), col = col0 + 4u * (e % (BN / 4));
+                const float *src = g.b + (size_t)min(k, g.k - 1u) * g.ldb;
                 if (VEC) {
-                    float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-                    if (k < g.k && col < g.n) t = *reinterpret_cast<const float4 *>(src);
+                    const float4 t = *reinterpret_cast<const float4 *>(src + min(col, g.n - 4u));
                     pb[u][0] = t.x, pb[u][1] = t.y, pb[u][2] = t.z, pb[u][3] = t.w;
                 } else {
 #pragma unroll
-                    for (int i = 0; i < 4; i++) pb[u][i] = (k < g.k && col + i < g.n) ? src[i] : 0.f;
+                    for (int i = 0; i < 4; i++) pb[u][i] = src[min(col + i, g.n - 1u)];
                 }
             }
         }
     };
-    auto park = [&](uint32_t buf) __attribute__((always_inline)) {
+    auto park = [&](uint32_t buf, uint32_t k0) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             const uint32_t e = threadIdx.x + 256u * u;
-            *reinterpret_cast<float4 *>(&sa[buf][(e / (TK / 4)) * A_PITCH + 4u * (e % (TK / 4))]) =
-                make_float4(pa[u][0], pa[u][1], pa[u][2], pa[u][3]);
-            *reinterpret_cast<float4 *>(&sb[buf][(e / (TN / 4)) * B_PITCH + 4u * (e % (TN / 4))]) =
-                make_float4(pb[u][0], pb[u][1], pb[u][2], pb[u][3]);
+            const uint32_t ka = k0 + 4u * (e % (BK / 4));
+            const uint32_t kb = k0 + e / (BN / 4), col = col0 + 4u * (e % (BN / 4));
+            float va[4], vb[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                va[i] = (VEC ? ka : ka + i) < g.k ? pa[u][i] : 0.f;
+                vb[i] = (kb < g.k && (VEC ? col : col + i) < g.n) ? pb[u][i] : 0.f;
+            }
+            *reinterpret_cast<float4 *>(&sa[buf][(e / (BK / 4)) * AP + 4u * (e % (BK / 4))]) =
+                make_float4(va[0], va[1], va[2], va[3]);
+            *reinterpret_cast<float4 *>(&sb[buf][(e / (BN / 4)) * BP + 4u * (e % (BN / 4))]) =
+                make_float4(vb[0], vb[1], vb[2], vb[3]);
         }
     };
 
-    floatx16 acc;
+    floatx16 acc[WT][WT];
 #pragma unroll
-    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    for (int i = 0; i < WT; i++)
+#pragma unroll
+        for (int j = 0; j < WT; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    const uint32_t steps = (g.k + TK - 1u) / TK;
+    const uint32_t steps = (g.k + BK - 1u) / BK;
     request(0);
-    park(0);
+    park(0, 0);
     __syncthreads();
     for (uint32_t s = 0; s < steps; s++) {
         const uint32_t buf = s & 1u;
-        if (s + 1u < steps) request((s + 1u) * TK);
-        /* MFMA A operand (rows of D = output columns): b[k][col], k = 16*h + t
+        if (s + 1u < steps) request((s + 1u) * BK);
+        /* MFMA A operand (rows of D = output columns): b[k][col], k = KH*h + t
          * MFMA B operand (columns of D = output rows):  a[row][k]            */
-        const float *ar = &sa[buf][(wr * 32u + c) * A_PITCH + 16u * h];
-        const float *bc = &sb[buf][(16u * h) * B_PITCH + wc * 32u + c];
+        const float *ar = &sa[buf][(wr * (32u * WT) + c) * AP + KH * h];
+        const float *bc = &sb[buf][(KH * h) * BP + wc * (32u * WT) + c];
 #pragma unroll
-        for (int t4 = 0; t4 < 16; t4 += 4) {
-            const float4 av = *reinterpret_cast<const float4 *>(ar + t4);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(bc[(t4 + 0) * B_PITCH], av.x, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(bc[(t4 + 1) * B_PITCH], av.y, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(bc[(t4 + 2) * B_PITCH], av.z, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(bc[(t4 + 3) * B_PITCH], av.w, acc, 0, 0, 0);
+        for (int t4 = 0; t4 < KH; t4 += 4) {
+            float av[WT][4];
+#pragma unroll
+            for (int i = 0; i < WT; i++) {
+                const float4 t = *reinterpret_cast<const float4 *>(ar + 32 * i * AP + t4);
+                av[i][0] = t.x, av[i][1] = t.y, av[i][2] = t.z, av[i][3] = t.w;
+            }
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                float bv[WT];
+#pragma unroll
+                for (int j = 0; j < WT; j++) bv[j] = bc[(t4 + t) * BP + 32 * j];
+#pragma unroll
+                for (int i = 0; i < WT; i++)
+#pragma unroll
+                    for (int j = 0; j < WT; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j], av[i][t], acc[i][j], 0, 0, 0);
+            }
         }
-        if (s + 1u < steps) park(buf ^ 1u);
+        if (s + 1u < steps) park(buf ^ 1u, (s + 1u) * BK);
         __syncthreads();
     }
 
-    /* lane (h, c) holds out[row0 + 32*wr + c][col0 + 32*wc + 8*q + 4*h + 0..3] in acc[4q..4q+3] */
-    const uint32_t row = row0 + wr * 32u + c;
-    if (row >= g.m) return;
+    /* lane (h, c) holds out[row0 + 32*(WT*wr + i) + c][col0 + 32*(WT*wc + j) + 8*q + 4*h + 0..3] in acc[i][j][4q..4q+3] */
     const bool vst = VEC && (g.ldo % 4u == 0u) && ((reinterpret_cast<uintptr_t>(g.out) & 15u) == 0u) &&
                      ((reinterpret_cast<uintptr_t>(g.residual) & 15u) == 0u);
 #pragma unroll
-    for (int q = 0; q < 4; q++)
-        store4<ROPE>(g, row, col0 + wc * 32u + 8u * q + 4u * h,
-                     make_float4(acc[4 * q + 0], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]), vst);
+    for (int i = 0; i < WT; i++) {
+        const uint32_t row = row0 + 32u * (WT * wr + i) + c;
+        if (row >= g.m) continue;
+#pragma unroll
+        for (int j = 0; j < WT; j++)
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+                store4<ROPE>(g, row, col0 + 32u * (WT * wc + j) + 8u * q + 4u * h,
+                             make_float4(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                                         acc[i][j][4 * q + 3]),
+                             vst);
+    }
 }
 
 /* 32x32 output tile (bx, by) per workgroup, K split over the NW waves (4, or 8 for long K:
@@ -454,13 +494,31 @@ void matmul_f32_launch(const MatmulArgs &g, hipStream_t s) {
         }
         return;
     }
+    /* 128x128 tiles once there are enough of them to load every compute unit twice over
+     * (BLT_HIP_MATMUL_TILE=64 keeps the 64x64 tiles: tuning hook) */
+    static const bool big_ok = [] {
+        const char *e = getenv("BLT_HIP_MATMUL_TILE");
+        return !(e && atoi(e) == 64);
+    }();
+    const uint32_t tx = (g.n + 2 * TN - 1) / (2 * TN), ty = (g.m + 2 * TM - 1) / (2 * TM);
+    if (big_ok && (uint64_t)tx * ty >= 512u) {
+        const dim3 grid(tx, ty);
+        if (rope) {
+            if (vec) blt_launch("matmul_mfma", matmul_mfma_kernel<true, true, 2>, grid, block, 0, s, g);
+            else blt_launch("matmul_mfma", matmul_mfma_kernel<false, true, 2>, grid, block, 0, s, g);
+        } else {
+            if (vec) blt_launch("matmul_mfma", matmul_mfma_kernel<true, false, 2>, grid, block, 0, s, g);
+            else blt_launch("matmul_mfma", matmul_mfma_kernel<false, false, 2>, grid, block, 0, s, g);
+        }
+        return;
+    }
     const dim3 grid((g.n + TN - 1) / TN, (g.m + TM - 1) / TM);
     if (rope) {
-        if (vec) blt_launch("matmul_mfma", matmul_mfma_kernel<true, true>, grid, block, 0, s, g);
-        else blt_launch("matmul_mfma", matmul_mfma_kernel<false, true>, grid, block, 0, s, g);
+        if (vec) blt_launch("matmul_mfma", matmul_mfma_kernel<true, true, 1>, grid, block, 0, s, g);
+        else blt_launch("matmul_mfma", matmul_mfma_kernel<false, true, 1>, grid, block, 0, s, g);
     } else {
-        if (vec) blt_launch("matmul_mfma", matmul_mfma_kernel<true, false>, grid, block, 0, s, g);
-        else blt_launch("matmul_mfma", matmul_mfma_kernel<false, false>, grid, block, 0, s, g);
+        if (vec) blt_launch("matmul_mfma", matmul_mfma_kernel<true, false, 1>, grid, block, 0, s, g);
+        else blt_launch("matmul_mfma", matmul_mfma_kernel<false, false, 1>, grid, block, 0, s, g);
     }
 }
 
