@@ -64,6 +64,7 @@ SYMBOLS = {
                                                   C.POINTER(abi.BltArena)]),
     "blt_strided_copy_hip": (None, [C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t,
                                     C.c_size_t]),
+    "blt_rows_gather_hip": (None, [C.POINTER(abi.BltTensor), abi.c_size_p, C.POINTER(abi.BltTensor)]),
     "blt_softmax_masked_row_inplace_hip": (None, [C.c_int, C.c_void_p, C.c_size_t, C.c_size_t, C.c_bool, C.c_void_p,
                                                   C.c_float]),
     "blt_vec_dot_hip": (C.c_float, [C.c_int, C.c_void_p, C.c_void_p, C.c_size_t]),
@@ -92,6 +93,9 @@ SYMBOLS = {
     "blt_softmax_masked_row_inplace": (None, [C.c_int, C.c_void_p, C.c_size_t, C.c_size_t, C.c_bool, C.c_void_p,
                                               C.c_float]),
     "blt_vec_dot": (C.c_float, [C.c_int, C.c_void_p, C.c_void_p, C.c_size_t]),
+    "blt_rows_gather": (None, [C.POINTER(abi.BltTensor), abi.c_size_p, C.POINTER(abi.BltTensor)]),
+    "blt_rope_position_gather": (None, [C.POINTER(abi.BltTensor), C.POINTER(abi.BltTensor), abi.c_size_p, C.c_size_t,
+                                        C.POINTER(abi.BltTensor), C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)]),
     "blt_patch_build_group_ids": (None, [C.POINTER(abi.BltPatchInfo), C.c_size_t, C.c_size_t, abi.c_size_p,
                                          abi.c_size_p]),
     "blt_patch_decoder_latent_at": (C.c_size_t, [C.POINTER(abi.BltPatchInfo), C.c_size_t, C.c_size_t]),

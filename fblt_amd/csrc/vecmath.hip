@@ -91,6 +91,27 @@ __global__ __launch_bounds__(256) void dot_kernel(const float *__restrict__ a, c
     if (threadIdx.x == 0) *out = (red[0] + red[1]) + (red[2] + red[3]);
 }
 
+/* dst[r, :] = src[pos[r], :] for up to GATHER_ROWS rows per launch; the row numbers travel in the
+ * kernel's argument block (the reference stages them in a device scratch arena, which this
+ * library does not keep), so the call neither allocates nor synchronises. */
+constexpr int GATHER_ROWS = 128;
+struct GatherRows {
+    uint64_t pos[GATHER_ROWS];
+};
+
+template <bool VEC>
+__global__ __launch_bounds__(256) void rows_gather_kernel(const float *__restrict__ src, float *__restrict__ dst,
+                                                          uint64_t row_len, GatherRows rows) {
+    const float *s = src + rows.pos[blockIdx.x] * row_len;
+    float *d = dst + (uint64_t)blockIdx.x * row_len;
+    if (VEC) {
+        for (uint64_t t = threadIdx.x; t < row_len / 4u; t += 256u)
+            reinterpret_cast<float4 *>(d)[t] = reinterpret_cast<const float4 *>(s)[t];
+    } else {
+        for (uint64_t t = threadIdx.x; t < row_len; t += 256u) d[t] = s[t];
+    }
+}
+
 } // namespace
 
 extern "C" void blt_strided_copy_hip(blt_backend backend, float *dst, size_t dst_stride, const float *src,
@@ -109,6 +130,36 @@ extern "C" void blt_strided_copy_hip(blt_backend backend, float *dst, size_t dst
         hipLaunchKernelGGL(strided_copy_kernel<false>, dim3(blocks), dim3(256), 0, blt_stream(), dst, (uint64_t)dst_stride, src,
                            (uint64_t)src_stride, (uint64_t)rows, (uint64_t)cols);
     HIP_CHECK_LAUNCH("blt_strided_copy");
+}
+
+extern "C" void blt_rows_gather_hip(const blt_tensor *src, const size_t *pos_host, blt_tensor *dst) {
+    BLT_REQUIRE(src != NULL && dst != NULL && pos_host != NULL, "blt_rows_gather: arguments cannot be NULL");
+    BLT_REQUIRE(src->backend == BLT_BACKEND_HIP && dst->backend == BLT_BACKEND_HIP,
+                "blt_rows_gather: HIP implementation called with non-HIP tensors");
+    BLT_REQUIRE(src->dtype == BLT_DTYPE_FP32 && dst->dtype == BLT_DTYPE_FP32, "blt_rows_gather: tensors must be FP32");
+    const size_t rows = dst->ndim >= 1 ? dst->shape[0] : 0;
+    if (rows == 0 || dst->numel == 0) return;
+    const size_t row_len = dst->numel / rows;
+    BLT_REQUIRE(src->ndim >= 1 && src->shape[src->ndim - 1] != 0 && src->numel % src->shape[src->ndim - 1] == 0,
+                "blt_rows_gather: src must be row-structured");
+    BLT_REQUIRE(src->numel >= row_len, "blt_rows_gather: position out of range");
+    for (size_t i = 0; i < rows; i++)
+        BLT_REQUIRE(pos_host[i] <= (src->numel - row_len) / row_len, "blt_rows_gather: position out of range");
+    const float *s = static_cast<const float *>(src->data);
+    float *d = static_cast<float *>(dst->data);
+    const bool vec = ((reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) & 15u) == 0 && row_len % 4 == 0;
+    for (size_t r0 = 0; r0 < rows; r0 += GATHER_ROWS) {
+        const size_t n = rows - r0 < (size_t)GATHER_ROWS ? rows - r0 : (size_t)GATHER_ROWS;
+        GatherRows g;
+        for (size_t i = 0; i < (size_t)GATHER_ROWS; i++) g.pos[i] = i < n ? pos_host[r0 + i] : 0;
+        if (vec)
+            hipLaunchKernelGGL(rows_gather_kernel<true>, dim3((unsigned)n), dim3(256), 0, blt_stream(), s,
+                               d + r0 * row_len, (uint64_t)row_len, g);
+        else
+            hipLaunchKernelGGL(rows_gather_kernel<false>, dim3((unsigned)n), dim3(256), 0, blt_stream(), s,
+                               d + r0 * row_len, (uint64_t)row_len, g);
+        HIP_CHECK_LAUNCH("blt_rows_gather");
+    }
 }
 
 extern "C" void blt_softmax_masked_row_inplace_hip(blt_backend backend, float *row, size_t row_len, size_t row_idx,

@@ -53,6 +53,12 @@ void blt_build_block_diffusion_mask_hip(const blt_block_diffusion_config *config
 void blt_strided_copy_hip(blt_backend backend, float *dst, size_t dst_stride, const float *src,
                           size_t src_stride, size_t rows, size_t cols);
 
+/* Replaces blt_rows_gather_cuda (csrc/ops/gather_scatter.cu:272-287; contract
+ * csrc/ops/gather_scatter.h:41-42): dst[i, :] = src[pos_host[i], :] with whole-row
+ * copies; pos_host is a HOST array (the rotary-table gather of the KV step,
+ * csrc/infer/rope_gather.c:33-34).  No allocation, no synchronisation. */
+void blt_rows_gather_hip(const blt_tensor *src, const size_t *pos_host, blt_tensor *dst);
+
 /* Replaces blt_softmax_masked_row_inplace_cuda (csrc/ops/vecmath.cu:71-114):
  * the row softmax of csrc/ops/vecmath.h:20-31 on one device row. */
 void blt_softmax_masked_row_inplace_hip(blt_backend backend, float *row, size_t row_len, size_t row_idx,
@@ -164,6 +170,12 @@ void blt_strided_copy(blt_backend backend, float *dst, size_t dst_stride, const 
 void blt_softmax_masked_row_inplace(blt_backend backend, float *row, size_t row_len, size_t row_idx,
                                     bool is_causal, const float *mask_row, float scale);
 float blt_vec_dot(blt_backend backend, const float *a, const float *b, size_t n);
+/* csrc/core/backend.c:532-534: the backend comes from src. */
+void blt_rows_gather(const blt_tensor *src, const size_t *pos_host, blt_tensor *dst);
+/* csrc/infer/rope_gather.h / rope_gather.c:5-35: rows positions[0..n) of the two rotary
+ * tables into new [n, half] tensors of the arena. */
+void blt_rope_position_gather(const blt_tensor *cos_cache, const blt_tensor *sin_cache, const size_t *positions,
+                              size_t n, blt_tensor *cos_out, blt_tensor *sin_out, blt_arena *arena);
 /* csrc/core/backend.c:397-399, 307-345; csrc/models/attention.h:24-26.  The
  * backend comes from the first tensor (matmul, rope_apply), the output
  * tensors (precompute), the explicit argument (packed) or the input tensor

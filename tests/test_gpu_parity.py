@@ -411,6 +411,47 @@ def test_strided_copy_softmax_dot(oracle, dev):
     assert abs(got - float(np.dot(a.astype(np.float64), b.astype(np.float64)))) < 1e-3
 
 
+@pytest.mark.parametrize("rows,src_rows,row_len", [(1, 7, 16), (5, 40, 33), (130, 512, 16), (300, 64, 64)])
+def test_rows_gather(rows, src_rows, row_len, dev):
+    """blt_rows_gather (csrc/ops/gather_scatter.h:41-42): dst[i, :] = src[pos[i], :], positions a host
+    array, repeats allowed, more rows than one launch carries, row lengths that are not a multiple
+    of four.  Copies are bit-exact."""
+    import torch
+    lib = api.load()
+    rs = np.random.RandomState(rows + row_len)
+    src = rs.randn(src_rows, row_len).astype(np.float32)
+    pos = rs.randint(0, src_rows, size=rows)
+    pos[-1] = src_rows - 1
+    tsrc = torch.from_numpy(src).cuda()
+    tdst = torch.full((rows, row_len), 7.0, dtype=torch.float32, device="cuda")
+    vs, vd = _dev_tensor(tsrc), _dev_tensor(tdst)
+    lib.blt_rows_gather(C.byref(vs), (C.c_size_t * rows)(*pos.tolist()), C.byref(vd))
+    lib.blt_backend_pass_sync_hip()
+    assert (tdst.cpu().numpy() == src[pos]).all()
+
+
+def test_rope_position_gather(dev):
+    """blt_rope_position_gather (csrc/infer/rope_gather.c:5-35): table rows of the given absolute
+    positions as two new [n, half] arena tensors."""
+    import torch
+    lib = api.load()
+    rs = np.random.RandomState(11)
+    cos, sin = rs.randn(96, 16).astype(np.float32), rs.randn(96, 16).astype(np.float32)
+    tc, ts = torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda()
+    vc, vs = _dev_tensor(tc), _dev_tensor(ts)
+    arena = lib.blt_arena_create(1 << 20, abi.BLT_BACKEND_HIP)
+    pos = [40, 41, 42, 95, 0]
+    oc, os_ = abi.BltTensor(), abi.BltTensor()
+    lib.blt_rope_position_gather(C.byref(vc), C.byref(vs), (C.c_size_t * 5)(*pos), 5, C.byref(oc), C.byref(os_), arena)
+    lib.blt_backend_pass_sync_hip()
+    assert (oc.ndim, oc.shape[0], oc.shape[1], oc.backend) == (2, 5, 16, abi.BLT_BACKEND_HIP)
+    got_c, got_s = np.empty((5, 16), dtype=np.float32), np.empty((5, 16), dtype=np.float32)
+    lib.blt_hip_memcpy_d2h(got_c.ctypes.data, oc.data, got_c.nbytes)
+    lib.blt_hip_memcpy_d2h(got_s.ctypes.data, os_.data, got_s.nbytes)
+    lib.blt_arena_destroy(arena)
+    assert (got_c == cos[pos]).all() and (got_s == sin[pos]).all()
+
+
 @pytest.mark.parametrize("kernel", ["valu", "mfma", "mfma32"])
 def test_kv_step_kernel_families_agree(kernel):
     """The kernels behind the KV step entry points (VALU, matrix-core with 16-wide tiles for blocks of

@@ -230,6 +230,20 @@ def test_host_arena_and_tensor():
 
 
 FATAL_SNIPPETS = {
+    "cpu_backend_rows_gather": """
+t = abi.BltTensor(); t.backend = abi.BLT_BACKEND_CPU
+pos = (C.c_size_t * 1)(0)
+lib.blt_rows_gather(C.byref(t), pos, C.byref(t))
+""",
+    "rope_position_gather_out_of_range": """
+import numpy as np
+tab = np.zeros((8, 4), dtype=np.float32)
+v = abi.tensor_view(tab.ctypes.data, tab.shape, abi.BLT_BACKEND_CPU)
+arena = lib.blt_arena_create(1 << 12, abi.BLT_BACKEND_CPU)
+pos = (C.c_size_t * 2)(1, 8)
+a, b = abi.BltTensor(), abi.BltTensor()
+lib.blt_rope_position_gather(C.byref(v), C.byref(v), pos, 2, C.byref(a), C.byref(b), arena)
+""",
     "cpu_backend_attention": """
 a = abi.BltAttentionHeadArgs()
 lib.blt_attention_head_core(abi.BLT_BACKEND_CPU, C.byref(a))
