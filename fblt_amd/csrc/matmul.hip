@@ -379,27 +379,107 @@ __global__ __launch_bounds__(256, 2) void matmul_splitk_pair_kernel(MatmulArgs g
     }
 }
 
-/* R rows of a per thread, one output column per thread. */
+constexpr uint32_t SKINNY_KC = 512; /* k values of the a rows staged in LDS at a time */
+
+/* One output column per thread, R rows of a per workgroup (grid.y walks the row groups).  Every
+ * output is the reference's own sum: k ascending, product and sum rounded separately.  What the
+ * kernel is built around is the latency of that serial chain: the rows of a sit in LDS (one
+ * broadcast 16-byte read per four k), the column of b is fetched sixteen k ahead of the chain --
+ * the requests of block t+1 are in flight while block t is summed -- and a decode step's single
+ * row gets a thread per column rather than a share of a thread. */
 template <int R, bool GATED>
 __global__ __launch_bounds__(256) void matmul_skinny_kernel(MatmulArgs g) {
 #pragma clang fp contract(off) /* product and sum rounded separately, as the reference's loop */
-    const uint32_t j = blockIdx.x * 256u + threadIdx.x;
+    constexpr uint32_t KC = SKINNY_KC, UN = 16;
+    __shared__ __attribute__((aligned(16))) float sa[R][KC];
+    __shared__ float inv_rms[R];
+    const uint32_t jj = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t j = min(jj, g.n - 1u);
     const uint32_t r0 = blockIdx.y * R;
-    if (j >= g.n) return;
     float acc[R], acc2[R];
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r] = 0.0f, acc2[r] = 0.0f;
-    for (uint32_t k = 0; k < g.k; k++) {
-        const float bj = g.b[(size_t)k * g.ldb + j];
-        const float gj = GATED ? g.b2[(size_t)k * g.ldb + j] : 0.0f;
-#pragma unroll
-        for (int r = 0; r < R; r++) {
+    const float *bcol = g.b + j;
+    const float *gcol = GATED ? g.b2 + j : nullptr;
+    for (uint32_t kc = 0; kc < g.k; kc += KC) {
+        const uint32_t klen = min(KC, g.k - kc);
+        __syncthreads(); /* the previous chunk has been consumed */
+        for (uint32_t t = threadIdx.x; t < R * KC; t += 256u) {
+            const uint32_t r = t / KC, kk = t % KC;
             const uint32_t row = min(r0 + r, g.m - 1u);
-            const float av = g.a[(size_t)row * g.lda + k];
-            acc[r] = acc[r] + av * bj;
-            if (GATED) acc2[r] = acc2[r] + av * gj;
+            sa[r][kk] = g.a[(size_t)row * g.lda + kc + min(kk, klen - 1u)];
+        }
+        __syncthreads();
+        if (g.norm_w) { /* uniform; the host sends such a product here only when k <= KC (one chunk) */
+            /* the reference's row norm (csrc/ops/reductions_cpu.c:325-352) on the staged rows: sum of
+             * squares in element order by one lane per row, then x * inv_rms * w element by element */
+            if ((threadIdx.x & 63u) == 0 && (threadIdx.x >> 6) < (uint32_t)R) {
+                const uint32_t r = threadIdx.x >> 6;
+                float sumsq = 0.0f;
+                uint32_t q = 0;
+                for (; q + 4u <= klen; q += 4u) {
+                    const float4 t = *reinterpret_cast<const float4 *>(&sa[r][q]);
+                    sumsq = sumsq + t.x * t.x;
+                    sumsq = sumsq + t.y * t.y;
+                    sumsq = sumsq + t.z * t.z;
+                    sumsq = sumsq + t.w * t.w;
+                }
+                for (; q < klen; q++) sumsq = sumsq + sa[r][q] * sa[r][q];
+                inv_rms[r] = 1.0f / sqrtf(sumsq / (float)klen + 1e-6f);
+            }
+            __syncthreads();
+            for (uint32_t t = threadIdx.x; t < R * KC; t += 256u) {
+                const uint32_t r = t / KC, kk = t % KC;
+                if (kk < klen) sa[r][kk] = sa[r][kk] * inv_rms[r] * g.norm_w[kk];
+            }
+            __syncthreads();
+        }
+        const uint32_t full = klen / UN * UN;
+        if (full) {
+            float bv[UN], gv[UN];
+#pragma unroll
+            for (uint32_t u = 0; u < UN; u++) {
+                bv[u] = bcol[(size_t)(kc + u) * g.ldb];
+                gv[u] = GATED ? gcol[(size_t)(kc + u) * g.ldb] : 0.0f;
+            }
+            for (uint32_t k0 = 0; k0 < full; k0 += UN) {
+                /* the next block's column values (the last round fetches its own block again) */
+                const uint32_t kn = kc + min(k0 + UN, full - UN);
+                float nb[UN], ng[UN];
+#pragma unroll
+                for (uint32_t u = 0; u < UN; u++) {
+                    nb[u] = bcol[(size_t)(kn + u) * g.ldb];
+                    ng[u] = GATED ? gcol[(size_t)(kn + u) * g.ldb] : 0.0f;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (uint32_t u4 = 0; u4 < UN; u4 += 4) {
+#pragma unroll
+                    for (int r = 0; r < R; r++) {
+                        const float4 a4 = *reinterpret_cast<const float4 *>(&sa[r][k0 + u4]);
+                        const float av[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+                        for (int t = 0; t < 4; t++) {
+                            acc[r] = acc[r] + av[t] * bv[u4 + t];
+                            if (GATED) acc2[r] = acc2[r] + av[t] * gv[u4 + t];
+                        }
+                    }
+                }
+#pragma unroll
+                for (uint32_t u = 0; u < UN; u++) bv[u] = nb[u], gv[u] = ng[u];
+            }
+        }
+        for (uint32_t k = full; k < klen; k++) {
+            const float bj = bcol[(size_t)(kc + k) * g.ldb];
+            const float gj = GATED ? gcol[(size_t)(kc + k) * g.ldb] : 0.0f;
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                acc[r] = acc[r] + sa[r][k] * bj;
+                if (GATED) acc2[r] = acc2[r] + sa[r][k] * gj;
+            }
         }
     }
+    if (jj >= g.n) return;
 #pragma unroll
     for (int r = 0; r < R; r++) {
         if (r0 + r >= g.m) continue;
@@ -408,6 +488,13 @@ __global__ __launch_bounds__(256) void matmul_skinny_kernel(MatmulArgs g) {
         g.out[(size_t)(r0 + r) * g.ldo + j] = v;
         if (GATED && g.out2) g.out2[(size_t)(r0 + r) * g.ldo + j] = acc2[r];
     }
+}
+
+template <int R>
+void launch_skinny(const MatmulArgs &g, hipStream_t s) {
+    const dim3 grid((g.n + 255u) / 256u, (g.m + R - 1u) / R);
+    if (g.b2) blt_launch("matmul_skinny", matmul_skinny_kernel<R, true>, grid, dim3(256), 0, s, g);
+    else blt_launch("matmul_skinny", matmul_skinny_kernel<R, false>, grid, dim3(256), 0, s, g);
 }
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -438,7 +525,10 @@ void launch_splitk(const MatmulArgs &g, dim3 grid, hipStream_t s) {
 } // namespace
 
 bool matmul_takes_gated(const MatmulArgs &g) { return choose_path(g) != PATH_MFMA; }
-bool matmul_takes_norm(const MatmulArgs &g) { return choose_path(g) == PATH_SPLITK; }
+bool matmul_takes_norm(const MatmulArgs &g) {
+    const Path path = choose_path(g);
+    return path == PATH_SPLITK || (path == PATH_SKINNY && g.k <= SKINNY_KC);
+}
 
 namespace {
 bool vec_ok(const MatmulArgs &g) {
@@ -469,17 +559,13 @@ void matmul_f32_launch(const MatmulArgs &g, hipStream_t s) {
     const bool rope = g.rope_cos != nullptr && g.rope_cols > 0;
     const Path path = choose_path(g);
     BLT_REQUIRE(g.b2 == nullptr || path != PATH_MFMA, "matmul: the gated product is not available for this shape");
-    BLT_REQUIRE(g.norm_w == nullptr || path == PATH_SPLITK, "matmul: the fused row norm is not available for this shape");
+    BLT_REQUIRE(g.norm_w == nullptr || matmul_takes_norm(g), "matmul: the fused row norm is not available for this shape");
     const dim3 block(256);
     if (path == PATH_SKINNY) {
-        const dim3 g4((g.n + 255u) / 256u, 1), g8((g.n + 255u) / 256u, (g.m + 7u) / 8u);
-        if (g.m <= 4u) {
-            if (g.b2) blt_launch("matmul_skinny", matmul_skinny_kernel<4, true>, g4, block, 0, s, g);
-            else blt_launch("matmul_skinny", matmul_skinny_kernel<4, false>, g4, block, 0, s, g);
-        } else {
-            if (g.b2) blt_launch("matmul_skinny", matmul_skinny_kernel<8, true>, g8, block, 0, s, g);
-            else blt_launch("matmul_skinny", matmul_skinny_kernel<8, false>, g8, block, 0, s, g);
-        }
+        /* rows per workgroup: the serial chains of a thread grow with it, the re-reads of b shrink */
+        if (g.m <= 4u) launch_skinny<1>(g, s);
+        else if (g.m <= 16u) launch_skinny<2>(g, s);
+        else launch_skinny<4>(g, s);
         return;
     }
     const bool vec = vec_ok(g);

@@ -28,10 +28,6 @@ extern "C" void blt_hip_memset(void *dst, int value, size_t bytes) {
     HIP_CHECK(hipMemsetAsync(dst, value, bytes, blt_stream()));
 }
 
-extern "C" void blt_hip_memcpy_h2d(void *dst, const void *src, size_t bytes) {
-    if (bytes == 0) return;
-    HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, blt_stream()));
-}
 
 namespace {
 
@@ -70,6 +66,19 @@ void blt_upload_staged(void *dst, const void *src, size_t bytes) {
     HIP_CHECK(hipMemcpyAsync(dst, s.host, bytes, hipMemcpyHostToDevice, blt_stream()));
     HIP_CHECK(hipEventRecord(s.copied, blt_stream()));
     s.in_flight = true;
+}
+
+/* The reference's callers free or reuse the host buffer as soon as the upload call returns
+ * (csrc/infer/kv_cache.c:237-238), so the source must be consumed before this returns: small
+ * uploads go through the pinned ring (no wait), large ones wait for the copy. */
+extern "C" void blt_hip_memcpy_h2d(void *dst, const void *src, size_t bytes) {
+    if (bytes == 0) return;
+    if (bytes <= (1u << 20) && !blt_stream_capturing()) {
+        blt_upload_staged(dst, src, bytes);
+        return;
+    }
+    HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, blt_stream()));
+    HIP_CHECK(hipStreamSynchronize(blt_stream()));
 }
 
 extern "C" void blt_hip_memcpy_d2h(void *dst, const void *src, size_t bytes) {

@@ -136,7 +136,7 @@ void blt_multihead_attention_hip(const blt_tensor *input, const blt_tensor *weig
 void *blt_hip_malloc(size_t bytes);
 void blt_hip_free(void *ptr);
 void blt_hip_memset(void *dst, int value, size_t bytes);                 /* async, default stream */
-void blt_hip_memcpy_h2d(void *dst, const void *src, size_t bytes);       /* async, default stream */
+void blt_hip_memcpy_h2d(void *dst, const void *src, size_t bytes);       /* src is consumed on return; the copy itself is ordered on the library's stream */
 void blt_hip_memcpy_d2h(void *dst, const void *src, size_t bytes);       /* blocking */
 void blt_backend_pass_sync_hip(void);                                    /* device sync + error check */
 

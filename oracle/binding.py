@@ -27,6 +27,8 @@ def build(ref=True):
     subprocess.check_call(["make", "-s", "-B", "-C", HERE, "all"])
     if ref and os.path.isdir(os.environ.get("REF_ROOT", "/root/reference")):
         subprocess.check_call(["make", "-s", "-B", "-C", HERE, "ref"])
+        if os.path.exists(os.path.join(HERE, "..", "fblt_amd", "lib", "libfblt_hip.so")):
+            subprocess.check_call(["make", "-s", "-C", HERE, "callers"])
 
 
 def load_oracle():
@@ -202,6 +204,43 @@ def load_ref():
     lib.blt_patch_decoder_latent_at.argtypes = [C.POINTER(abi.BltPatchInfo), C.c_size_t, C.c_size_t]
     lib.blt_patch_expand_group_ids.restype = None
     lib.blt_patch_expand_group_ids.argtypes = [_sp, C.c_size_t, C.c_size_t, _sp]
+    return lib
+
+
+CALLERS_SO = os.path.join(HERE, "_ref", "libblt_ref_callers.so")
+
+
+def load_ref_callers():
+    """The reference's attention blocks and KV-cache step, compiled unmodified and linked against
+    the HIP library so that every tensor op they call lands there (`make -C oracle callers`); None
+    where that was never built.  Import torch and load the HIP library before calling this (the
+    dependency must resolve to the copy that is already loaded)."""
+    if not os.path.exists(CALLERS_SO) or not os.path.exists(REF_SO):
+        return None
+    load_ref()          # its own scope first: its internal calls must keep resolving to itself
+    lib = C.CDLL(CALLERS_SO)
+    T = C.POINTER(abi.BltTensor)
+    K = C.POINTER(abi.BltKvCache)
+    A = C.POINTER(abi.BltArena)
+    P = C.POINTER(abi.BltPatchInfo)
+    lib.blt_multihead_attention.restype = None
+    lib.blt_multihead_attention.argtypes = [T, T, T, T, C.POINTER(abi.BltAttentionConfig), A]
+    lib.blt_cross_attention_forward.restype = None
+    lib.blt_cross_attention_forward.argtypes = [T, T, C.POINTER(abi.BltCrossAttentionWeights), T,
+                                                C.POINTER(abi.BltCrossAttentionConfig), A]
+    lib.blt_kv_cache_create.restype = K
+    lib.blt_kv_cache_create.argtypes = [A, C.POINTER(abi.BltLocalDecoder), C.c_size_t]
+    for name in ("blt_kv_cache_destroy", "blt_kv_cache_reset"):
+        getattr(lib, name).restype = None
+        getattr(lib, name).argtypes = [K]
+    lib.blt_kv_cache_truncate.restype = None
+    lib.blt_kv_cache_truncate.argtypes = [K, C.c_size_t, C.c_size_t]
+    lib.blt_kv_cache_common_patches.restype = C.c_size_t
+    lib.blt_kv_cache_common_patches.argtypes = [K, P, C.c_size_t]
+    lib.blt_kv_cache_refresh_cross.restype = None
+    lib.blt_kv_cache_refresh_cross.argtypes = [K, T, P, C.c_size_t, C.c_size_t, A]
+    lib.blt_kv_decode_step.restype = None
+    lib.blt_kv_decode_step.argtypes = [K, T, P, C.c_size_t, T, C.c_int, T, A]
     return lib
 
 

@@ -530,6 +530,7 @@ def _dev_tensor(t, shape=None):
 
 
 @pytest.mark.parametrize("m,k,n,exact", [(1, 128, 384, True), (5, 33, 17, True), (32, 512, 512, True),
+                                          (3, 1100, 70, True), (1, 7, 300, True), (9, 528, 257, True),
                                           (16, 128, 512, True), (33, 64, 64, False), (64, 128, 384, False),
                                           (512, 128, 384, False), (100, 70, 50, False), (513, 129, 130, False),
                                           (2048, 512, 1536, False), (4100, 70, 2050, False), (4096, 96, 2048, False)])
@@ -591,6 +592,22 @@ def test_rope_apply_bit_exact(oracle, dev):
     assert tq.cpu().numpy().tobytes() == want.tobytes()
 
 
+IMPLS = ["library", "reference_callers"]
+
+
+def _entry(impl, lib):
+    """Where the block-level calls go: the library's own entry points, or the reference's caller
+    code (models/attention.c, cross_attention.c, infer/kv_cache.c compiled unmodified) whose tensor
+    ops are served by the library -- the drop-in arrangement itself."""
+    if impl == "library":
+        return lib
+    callers = binding.load_ref_callers()
+    if callers is None:
+        pytest.skip("oracle/_ref/libblt_ref_callers.so was not built (needs the reference sources)")
+    return callers
+
+
+@pytest.mark.parametrize("impl", IMPLS)
 @pytest.mark.parametrize("T,E,H,causal,rope,mask,cached", [
     (2, 4, 2, False, False, None, False),          # the reference's identity-weight block
     (20, 32, 4, True, True, None, False),          # few rows: exact products, separate rotation pass
@@ -600,10 +617,11 @@ def test_rope_apply_bit_exact(oracle, dev):
     (70, 48, 3, False, False, "docs", False),        # dense mask from the device builder
     (128, 512, 8, False, False, "causal_cfg", False),  # the patch transformer's call at C2 size
 ])
-def test_multihead_attention_block(T, E, H, causal, rope, mask, cached, oracle, dev):
+def test_multihead_attention_block(T, E, H, causal, rope, mask, cached, impl, oracle, dev):
     """blt_multihead_attention on device tensors against the restated block."""
     import torch
     lib = api.load()
+    entry = _entry(impl, lib)
     rs = np.random.RandomState(T + E)
     hd, half = E // H, E // H // 2
     if (T, E, H) == (2, 4, 2):
@@ -651,7 +669,7 @@ def test_multihead_attention_block(T, E, H, causal, rope, mask, cached, oracle, 
     arena = lib.blt_arena_create(64 << 20, abi.BLT_BACKEND_HIP)
     try:
         vx, vq, vp, vo = _dev_tensor(tx), _dev_tensor(tq), _dev_tensor(tp), _dev_tensor(to)
-        lib.blt_multihead_attention(C.byref(vx), C.byref(vq), C.byref(vp), C.byref(vo), C.byref(ac), arena)
+        entry.blt_multihead_attention(C.byref(vx), C.byref(vq), C.byref(vp), C.byref(vo), C.byref(ac), arena)
         lib.blt_backend_pass_sync_hip()
         got = to.cpu().numpy()
     finally:
@@ -659,6 +677,7 @@ def test_multihead_attention_block(T, E, H, causal, rope, mask, cached, oracle, 
     assert_close(got, ref, "attention block T=%d E=%d H=%d" % (T, E, H))
 
 
+@pytest.mark.parametrize("impl", IMPLS)
 @pytest.mark.parametrize("P,T,E,H,kind", [
     (2, 4, 4, 2, "identity"),          # tests/unit/models/unit_cross_attention.c:24-117
     (9, 70, 32, 4, "groups"),          # few rows: exact products
@@ -668,10 +687,11 @@ def test_multihead_attention_block(T, E, H, causal, rope, mask, cached, oracle, 
     (33, 100, 48, 3, "interleaved"),   # groups not contiguous: dense mask from the device builder
     (64, 200, 64, 2, "window"),        # no groups: window-only visibility
 ])
-def test_cross_attention_block(P, T, E, H, kind, oracle, dev):
+def test_cross_attention_block(P, T, E, H, kind, impl, oracle, dev):
     """blt_cross_attention_forward on device tensors against the restated block."""
     import torch
     lib = api.load()
+    entry = _entry(impl, lib)
     rs = np.random.RandomState(P + T + E)
     if kind == "identity":
         xq = np.array([[1, 0, 1, 0], [0, 1, 0, 1]], dtype=np.float32)
@@ -712,7 +732,7 @@ def test_cross_attention_block(P, T, E, H, kind, oracle, dev):
     cc.mask_config = C.pointer(cfg)
     arena = lib.blt_arena_create(64 << 20, abi.BLT_BACKEND_HIP)
     try:
-        lib.blt_cross_attention_forward(C.byref(views[0]), C.byref(views[1]), C.byref(wts), C.byref(vo), C.byref(cc),
+        entry.blt_cross_attention_forward(C.byref(views[0]), C.byref(views[1]), C.byref(wts), C.byref(vo), C.byref(cc),
                                         arena)
         lib.blt_backend_pass_sync_hip()
         got = to.cpu().numpy()
@@ -870,13 +890,15 @@ def _tier(lib, cache, name, layer, rows, E):
     return out
 
 
+@pytest.mark.parametrize("impl", IMPLS)
 @pytest.mark.parametrize("case", range(len(STEP_CASES)))
-def test_kv_decode_step_single_sequence(case, oracle, dev):
+def test_kv_decode_step_single_sequence(case, impl, oracle, dev):
     """blt_kv_cache_refresh_cross + blt_kv_decode_step on device memory against the restated step:
     prefill chunk, single rows, re-segmentation; logits and all four cache tiers after every call."""
     import torch
     from fblt_amd import decoder
     lib = api.load()
+    entry = _entry(impl, lib)
     c = STEP_CASES[case]
     E, V, k, L = c["E"], c["V"], c["k"], c["L"]
     rs = np.random.RandomState(300 + case)
@@ -884,7 +906,7 @@ def test_kv_decode_step_single_sequence(case, oracle, dev):
     mine = decoder.HostCache(host, c["max_len"])
     arena = lib.blt_arena_create(64 << 20, abi.BLT_BACKEND_HIP)
     try:
-        cache = lib.blt_kv_cache_create(arena, device.ptr, c["max_len"])
+        cache = entry.blt_kv_cache_create(arena, device.ptr, c["max_len"])
         assert cache.contents.k == k and cache.contents.max_subtokens == c["max_len"]
         mark = arena.contents.offset
         d0_all = rs.randn(21, E).astype(np.float32)
@@ -898,13 +920,13 @@ def test_kv_decode_step_single_sequence(case, oracle, dev):
             if from_patch:
                 patch_in[:from_patch] = prev[:from_patch]
             prev = patch_in
-            same = lib.blt_kv_cache_common_patches(cache, patches, P)
+            same = entry.blt_kv_cache_common_patches(cache, patches, P)
             assert same == from_patch
-            lib.blt_kv_cache_truncate(cache, cache.contents.self_len, min(from_patch, cache.contents.cross_num_patches))
+            entry.blt_kv_cache_truncate(cache, cache.contents.self_len, min(from_patch, cache.contents.cross_num_patches))
             tp = torch.from_numpy(patch_in).cuda()
             vp = _dev_tensor(tp)
             arena.contents.offset = mark
-            lib.blt_kv_cache_refresh_cross(cache, C.byref(vp), patches, P, from_patch, arena)
+            entry.blt_kv_cache_refresh_cross(cache, C.byref(vp), patches, P, from_patch, arena)
             assert cache.contents.cross_num_patches == P
             assert oracle.orc_kv_cache_refresh_cross(mine.ptr, 0, binding.fptr(patch_in.reshape(-1)), P, from_patch) == 0
             rows = np.ascontiguousarray(d0_all[done:done + n])
@@ -914,7 +936,7 @@ def test_kv_decode_step_single_sequence(case, oracle, dev):
             td = torch.from_numpy(rows).cuda()
             tl = torch.full((n, V), 7.0, dtype=torch.float32, device="cuda")
             vd, vl = _dev_tensor(td), _dev_tensor(tl)
-            lib.blt_kv_decode_step(cache, C.byref(vp), patches, P, C.byref(vd), closed, C.byref(vl), arena)
+            entry.blt_kv_decode_step(cache, C.byref(vp), patches, P, C.byref(vd), closed, C.byref(vl), arena)
             lib.blt_backend_pass_sync_hip()
             done += n
             assert cache.contents.self_len == done
@@ -923,9 +945,9 @@ def test_kv_decode_step_single_sequence(case, oracle, dev):
                 for l in range(L):
                     assert_close(_tier(lib, cache, name, l, c["max_len"], E), mine.tiers[name][l],
                                  "%s[%d] case %d %s" % (name, l, case, lengths))
-        lib.blt_kv_cache_reset(cache)
+        entry.blt_kv_cache_reset(cache)
         assert cache.contents.self_len == 0 and cache.contents.cross_num_patches == 0
-        lib.blt_kv_cache_destroy(cache)
+        entry.blt_kv_cache_destroy(cache)
     finally:
         lib.blt_arena_destroy(arena)
 

@@ -32,6 +32,35 @@ def test_library_exports_every_declared_symbol():
     assert b"gfx950" in api.load().blt_hip_build_info()
 
 
+# what the reference's caller code references but this library leaves to the reference build:
+# training passes and ops of other model parts, none of them reached from the forward attention
+# blocks or the KV-cache step (csrc/models/attention.c:130-207, cross_attention.c:101-157,
+# csrc/infer/kv_cache.c:112-428)
+OFF_PATH = {"blt_attention_head_core_backward", "blt_matmul_backward", "blt_rmsnorm_backward",
+            "blt_rmsnorm_backward_add", "blt_rope_apply_packed_backward", "blt_swiglu_backward",
+            "blt_cross_entropy_forward", "blt_cross_entropy_backward", "blt_embedding_lookup", "blt_gelu_forward",
+            "blt_layernorm_forward", "blt_cast", "blt_container_alloc", "blt_tensor_view_2d", "blt_tensor_view_3d"}
+
+
+def test_reference_callers_find_their_ops_in_the_library():
+    """The reference's attention blocks and KV-cache step, compiled unmodified, leave their tensor
+    ops undefined; every one of those that is on the path is exported by the HIP library under the
+    reference's own name (the drop-in arrangement the GPU tests then run)."""
+    so = os.path.join(ROOT, "oracle", "_ref", "libblt_ref_callers.so")
+    if not os.path.exists(so):
+        pytest.skip("oracle/_ref/libblt_ref_callers.so was not built (needs the reference sources)")
+    out = subprocess.run(["nm", "-D", "-u", so], capture_output=True, text=True, check=True).stdout
+    wanted = {line.split()[-1] for line in out.splitlines() if line.split()[-1].startswith("blt_")}
+    assert len(wanted) >= 25
+    lib = C.CDLL(api.LIB_PATH)
+    missing = {n for n in wanted - OFF_PATH if not hasattr(lib, n)}
+    assert not missing, missing
+    for n in ("blt_attention_head_core", "blt_build_attention_mask", "blt_matmul", "blt_rope_apply", "blt_rows_gather",
+              "blt_strided_copy", "blt_rmsnorm_forward", "blt_swiglu_forward", "blt_add", "blt_tensor_create",
+              "blt_tensor_upload", "blt_arena_alloc"):
+        assert n in wanted, n
+
+
 def test_header_layout_assertions_compile():
     """include/blt_abi.h carries its own static assertions; compile it as C99 and C++17."""
     for cc, std, lang in (("gcc", "-std=c99", "c"), ("g++", "-std=c++17", "c++")):
