@@ -707,6 +707,11 @@ def main():
         if not args.no_cpu:
             others["decode_step"]["cpu_baseline"] = cpu_decode_step(2.0)
         log("decode_step", json.dumps(others["decode_step"]))
+        # the reference's own use of the step: one sequence, one new row per call
+        others["decode_step_b1"] = bench_decode_step(K, W, batch=1)
+        if not args.no_cpu:
+            others["decode_step_b1"]["cpu_baseline"] = cpu_decode_step(2.0, batch=1)
+        log("decode_step_b1", json.dumps(others["decode_step_b1"]))
 
     cpu_head = None
     if not args.no_cpu:
