@@ -553,14 +553,17 @@ def cpu_decode_step(budget_s, batch=64, L=2, E=128, H=4, hidden=512, V=256, len_
 
 
 def cpu_dense(w, budget_s):
-    """Checker on one host core over the same workload; repeated whole passes up to the budget."""
+    """One host core over the same workload; repeated whole passes up to the budget.  Through the
+    reference's own attention core where its build is present (kind "reference"), else through the
+    restatement (kind "port"); the two are bit-identical and compiled with the same flags."""
     from oracle import binding, runner as orunner
     lib = binding.load_oracle()
+    ref = binding.load_ref()
     passes, spent = 0, 0.0
     while passes < 1 or (spent < budget_s and passes < 200):
-        spent += orunner.run(w, lib=lib, timed=True)
+        spent += orunner.run_ref(w, ref, lib=lib, timed=True) if ref else orunner.run(w, lib=lib, timed=True)
         passes += 1
-    return {"value": w.tokens * passes / spent, "unit": "tokens/s", "cores": 1, "kind": "port",
+    return {"value": w.tokens * passes / spent, "unit": "tokens/s", "cores": 1, "kind": "reference" if ref else "port",
             "sample": "%d full passes of %s, %.1f s, dense mask passed in, one core call per (sequence, head)"
                       % (passes, w.name, spent), "ms_per_pass": spent / passes * 1e3}
 

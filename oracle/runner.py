@@ -100,6 +100,19 @@ def run(w, lib=None, use_causal_flag=False, weights=None, timed=False):
     return dt if timed else None
 
 
+def run_ref(w, ref, lib=None, timed=False):
+    """The same pass through the reference's own blt_attention_head_core (oracle/_ref build), one call
+    per (sequence, head) as its callers make them; masks come from the restated builder (untimed)."""
+    lib = lib or binding.load_oracle()
+    arr, keep = head_arg_array(lib, w)
+    t0 = time.perf_counter()
+    for t in range(len(w.heads)):
+        ref.blt_attention_head_core(abi.BLT_BACKEND_CPU, C.byref(arr[t]))
+    dt = time.perf_counter() - t0
+    del keep
+    return dt if timed else None
+
+
 def run_kv(kw, lib=None, steps=None, timed=False):
     """KV-cache workload: returns combined [steps, batch*n, E]; mutates a COPY of the cache."""
     lib = lib or binding.load_oracle()
