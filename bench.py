@@ -292,6 +292,76 @@ def bench_block(name, T, E, H, steps, warmup, gemm_only=None, cross=None, warm_m
     return res
 
 
+def bench_masks(steps, warmup, cpu):
+    """The device mask builders (blt_build_attention_mask / blt_build_block_diffusion_mask on a device
+    arena) at the shapes their callers use, and one large fill; per call: the fill kernel(s) by
+    events, the whole call by the host clock (it ends with the blocking read-back of the empty-row
+    check).  Algorithmic bytes = the mask written once.  `cpu`: time the restated builder beside it."""
+    import ctypes as C
+    import numpy as np
+    from fblt_amd import abi, api, synth
+    lib = api.load()
+    out = {}
+
+    def group_ids(P, T):
+        _, lens = synth.patch_lengths(synth.seed_for(3, synth.S_LEN), P, T)
+        return np.repeat(np.arange(P), lens)
+
+    cases = []
+    c1 = abi.BltMaskConfig(); c1.seq_len_q = c1.seq_len_kv = 512; c1.is_causal = True
+    cases.append(("mask_c1_causal_512", "attention", c1, None, 512 * 512))
+    c3 = abi.BltMaskConfig(); c3.seq_len_q, c3.seq_len_kv = 128, 512
+    qg, kg = abi.size_array(range(128)), abi.size_array(group_ids(128, 512).tolist())
+    c3.query_group_ids, c3.kv_group_ids, c3.bidirectional_within_group = qg, kg, True
+    cases.append(("mask_c3_patch_groups_128x512", "attention", c3, (qg, kg), 128 * 512))
+    c5 = abi.BltBlockDiffusionConfig(); c5.mode, c5.seq_len, c5.num_clean = abi.BLT_BDM_INFER, 524, 508
+    cases.append(("mask_c5_block_infer_524", "block", c5, None, 524 * 524))
+    big = abi.BltMaskConfig(); big.seq_len_q = big.seq_len_kv = 4096; big.is_causal = True; big.sliding_window = 1024
+    cases.append(("mask_causal_window_4096", "attention", big, None, 4096 * 4096))
+
+    arena = lib.blt_arena_create(160 << 20, abi.BLT_BACKEND_HIP)
+    mark = arena.contents.offset
+    for name, kind, cfg, keep, cells in cases:
+        t = abi.BltTensor()
+        fn = lib.blt_build_attention_mask if kind == "attention" else lib.blt_build_block_diffusion_mask
+
+        def run():
+            arena.contents.offset = mark
+            fn(C.byref(cfg), C.byref(t), arena)
+        n = max(10, steps // 4)
+        warm_up(lib, run, max(3, warmup // 4))
+        lib.blt_hip_profile_begin()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            run()
+        lib.blt_backend_pass_sync_hip()
+        wall = time.perf_counter() - t0
+        prof = api.profile_end()
+        fill = {k: v for k, v in prof.items() if k != "mask_row_check"}
+        avg_s = sum(v[1] for v in fill.values()) / 1e3 / n
+        nbytes = 4.0 * cells
+        res = {"workload": name, "kernel": "+".join(sorted(prof)), "launches_per_step": sum(v[0] for v in prof.values()) / n,
+               "us_per_call": wall / n * 1e6, "kernel_us_avg": avg_s * 1e6,
+               "per_kernel_us": {k: v[1] * 1e3 / n for k, v in prof.items()}, "bytes": nbytes,
+               "roofline": roofline("hbm", nbytes, avg_s)}
+        if cpu:
+            from oracle import binding
+            orc = binding.load_oracle()
+            buf = np.empty(cells, dtype=np.float32)
+            ofn = orc.orc_build_attention_mask if kind == "attention" else orc.orc_build_block_diffusion_mask
+            reps, spent = 0, 0.0
+            while reps < 1 or (spent < 1.0 and reps < 50):
+                t0 = time.perf_counter()
+                assert ofn(C.byref(cfg), binding.fptr(buf)) == 0
+                spent += time.perf_counter() - t0
+                reps += 1
+            res["cpu_baseline"] = {"value": spent / reps * 1e6, "unit": "us/call", "cores": 1, "kind": "port",
+                                   "sample": "%d calls, %.2f s" % (reps, spent)}
+        out[name] = res
+    lib.blt_arena_destroy(arena)
+    return out
+
+
 def bench_decode_layer(steps, warmup, batch=64, H=4, hd=32, hidden=512, len_hi=512):
     """blt_kv_decode_layer_hip: one decoder layer (self-attention block with fused RoPE and
     write-through, feed-forward block) for `batch` sequences, one new row each, per step."""
@@ -717,6 +787,12 @@ def main():
         if not args.no_cpu:
             others["decode_step_b1"]["cpu_baseline"] = cpu_decode_step(2.0, batch=1)
         log("decode_step_b1", json.dumps(others["decode_step_b1"]))
+
+    # the dense-mask builders the callers still use
+    if want("masks"):
+        for name, res in bench_masks(K, W, not args.no_cpu).items():
+            others[name] = res
+            log(name, json.dumps(res))
 
     cpu_head = None
     if not args.no_cpu:

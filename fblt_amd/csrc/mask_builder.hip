@@ -48,19 +48,28 @@ __device__ __forceinline__ bool pair_allowed(const MaskRecipe &r, uint64_t i, ui
     return ok;
 }
 
-/* grid.x covers the key axis in chunks of 256, grid.y strides over rows.
- * row_ok[i] ends up non-zero when row i has at least one allowed key. */
+/* grid.x covers the key axis in chunks of 256 * W cells (lane = W consecutive keys, stored as one
+ * 4*W-byte piece; W = 4 needs seq_len_kv % 4 == 0 so that every row starts 16-byte aligned),
+ * grid.y strides over rows.  row_ok[i] ends up non-zero when row i has at least one allowed key:
+ * a plain store of 1 by every wave that saw one (the same value from all of them, no atomic). */
+template <int W>
 __global__ __launch_bounds__(256) void attention_mask_kernel(float *__restrict__ out, MaskRecipe r,
                                                              uint32_t *__restrict__ row_ok) {
-    const uint64_t j = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    const uint64_t j0 = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * W;
     for (uint64_t i = blockIdx.y; i < r.nq; i += gridDim.y) {
-        bool ok = false;
-        if (j < r.nk) {
-            ok = pair_allowed(r, i, j);
-            out[i * r.nk + j] = ok ? 0.0f : -__builtin_huge_valf();
+        bool any_ok = false;
+        if (j0 < r.nk) { /* nk % W == 0: all W cells are inside */
+            float v[W];
+#pragma unroll
+            for (int t = 0; t < W; t++) {
+                const bool ok = pair_allowed(r, i, j0 + t);
+                any_ok |= ok;
+                v[t] = ok ? 0.0f : -__builtin_huge_valf();
+            }
+            if (W == 4) *reinterpret_cast<float4 *>(out + i * r.nk + j0) = make_float4(v[0], v[1], v[2], v[3]);
+            else out[i * r.nk + j0] = v[0];
         }
-        const unsigned long long any = __ballot(ok);
-        if (any != 0ull && (threadIdx.x & 63u) == 0u) atomicOr(&row_ok[i], 1u);
+        if (row_ok && __ballot(any_ok) != 0ull && (threadIdx.x & 63u) == 0u) row_ok[i] = 1u;
     }
 }
 
@@ -78,21 +87,29 @@ struct BlockRecipe {
     int infer;
 };
 
+template <int W>
 __global__ __launch_bounds__(256) void block_diffusion_mask_kernel(float *__restrict__ out, BlockRecipe r) {
-    const uint64_t j = (uint64_t)blockIdx.x * 256u + threadIdx.x;
-    if (j >= r.S) return;
+    const uint64_t j0 = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * W;
+    if (j0 >= r.S) return;
     for (uint64_t i = blockIdx.y; i < r.S; i += gridDim.y) {
-        bool ok;
-        if (i < r.N) {
-            ok = j < r.N && j <= i;
-        } else if (r.infer) {
-            ok = true;
-        } else {
-            const uint64_t blk = (i - r.N) / r.B;
-            const bool own = j >= r.N && (j - r.N) / r.B == blk;
-            ok = j < r.starts[blk] || own;
+        float v[W];
+#pragma unroll
+        for (int t = 0; t < W; t++) {
+            const uint64_t j = j0 + t;
+            bool ok;
+            if (i < r.N) {
+                ok = j < r.N && j <= i;
+            } else if (r.infer) {
+                ok = true;
+            } else {
+                const uint64_t blk = (i - r.N) / r.B;
+                const bool own = j >= r.N && (j - r.N) / r.B == blk;
+                ok = j < r.starts[blk] || own;
+            }
+            v[t] = ok ? 0.0f : -__builtin_huge_valf();
         }
-        out[i * r.S + j] = ok ? 0.0f : -__builtin_huge_valf();
+        if (W == 4) *reinterpret_cast<float4 *>(out + i * r.S + j0) = make_float4(v[0], v[1], v[2], v[3]);
+        else out[i * r.S + j0] = v[0];
     }
 }
 
@@ -113,8 +130,8 @@ void doc_ids_from_boundaries(const size_t *bounds, size_t num_docs, size_t len, 
     }
 }
 
-dim3 mask_grid(uint64_t rows, uint64_t cols) {
-    const uint64_t gx = (cols + 255u) / 256u;
+dim3 mask_grid(uint64_t rows, uint64_t cols, uint64_t per_lane) {
+    const uint64_t gx = (cols + 256u * per_lane - 1u) / (256u * per_lane);
     const uint64_t gy = rows < 4096u ? (rows ? rows : 1u) : 4096u;
     return dim3((unsigned)gx, (unsigned)gy, 1u);
 }
@@ -157,19 +174,37 @@ extern "C" void blt_build_attention_mask_hip(const blt_mask_config *config, blt_
         r.grp_kv = stage_u64(config->kv_group_ids, nk, arena);
     }
 
-    uint32_t *row_ok = static_cast<uint32_t *>(blt_arena_alloc(arena, (nq + 1) * sizeof(uint32_t), 16));
-    uint32_t *dead = row_ok + nq;
-    blt_hip_memset(row_ok, 0, (nq + 1) * sizeof(uint32_t));
+    /* "query position has no valid key" (mask_builder_cpu.c:93).  Whenever every row's allowed keys
+     * form one range -- causal, window, document and sorted-group recipes, i.e. every mask the
+     * callers build -- the host knows the answer in O(nq + nk) and the call stays asynchronous;
+     * otherwise the kernel flags the rows that have a key and one blocking read-back counts the rest. */
+    bool host_checked = false;
+    if (nq <= 0xFFFFFFFFu && nk <= 0xFFFFFFFFu) {
+        std::vector<uint32_t> lo(nq), hi(nq);
+        if (blt_mask_config_row_ranges(config, lo.data(), hi.data())) {
+            for (size_t i = 0; i < nq; i++)
+                BLT_REQUIRE(lo[i] < hi[i], "blt_build_attention_mask: query position has no valid key");
+            host_checked = true;
+        }
+    }
+    uint32_t *row_ok = nullptr, *dead = nullptr;
+    if (!host_checked) {
+        row_ok = static_cast<uint32_t *>(blt_arena_alloc(arena, (nq + 1) * sizeof(uint32_t), 16));
+        dead = row_ok + nq;
+        blt_hip_memset(row_ok, 0, (nq + 1) * sizeof(uint32_t));
+    }
 
-    hipLaunchKernelGGL(attention_mask_kernel, mask_grid(nq, nk), dim3(256), 0, blt_stream(),
-                       static_cast<float *>(out_mask->data), r, row_ok);
+    if (nk % 4u == 0u)
+        blt_launch("mask_attention", attention_mask_kernel<4>, mask_grid(nq, nk, 4), dim3(256), 0, 0,
+                   static_cast<float *>(out_mask->data), r, row_ok);
+    else
+        blt_launch("mask_attention", attention_mask_kernel<1>, mask_grid(nq, nk, 1), dim3(256), 0, 0,
+                   static_cast<float *>(out_mask->data), r, row_ok);
     HIP_CHECK_LAUNCH("blt_build_attention_mask");
+    if (host_checked) return; /* the id vectors staged above were consumed when their uploads returned */
     const unsigned cblocks = (unsigned)((nq + 255u) / 256u < 1024u ? (nq + 255u) / 256u : 1024u);
-    hipLaunchKernelGGL(count_dead_rows_kernel, dim3(cblocks), dim3(256), 0, blt_stream(), row_ok, (uint64_t)nq, dead);
+    blt_launch("mask_row_check", count_dead_rows_kernel, dim3(cblocks), dim3(256), 0, 0, row_ok, (uint64_t)nq, dead);
     HIP_CHECK_LAUNCH("blt_build_attention_mask row check");
-
-    /* The staged id vectors (dq, dk) must outlive the asynchronous copies:
-     * the blocking read below orders everything before they are destroyed. */
     uint32_t dead_rows = 0;
     blt_hip_memcpy_d2h(&dead_rows, dead, sizeof(dead_rows));
     BLT_REQUIRE(dead_rows == 0, "blt_build_attention_mask: query position has no valid key");
@@ -206,8 +241,12 @@ extern "C" void blt_build_block_diffusion_mask_hip(const blt_block_diffusion_con
     r.infer = train ? 0 : 1;
     r.starts = train ? stage_u64(config->block_starts, config->num_blocks, arena) : nullptr;
 
-    hipLaunchKernelGGL(block_diffusion_mask_kernel, mask_grid(S, S), dim3(256), 0, blt_stream(),
-                       static_cast<float *>(out_mask->data), r);
+    if (S % 4u == 0u)
+        blt_launch("mask_block_diffusion", block_diffusion_mask_kernel<4>, mask_grid(S, S, 4), dim3(256), 0, 0,
+                   static_cast<float *>(out_mask->data), r);
+    else
+        blt_launch("mask_block_diffusion", block_diffusion_mask_kernel<1>, mask_grid(S, S, 1), dim3(256), 0, 0,
+                   static_cast<float *>(out_mask->data), r);
     HIP_CHECK_LAUNCH("blt_build_block_diffusion_mask");
     /* Row i always sees column min(i, N-1) or itself, so no row can be empty
      * once the checks above hold; block_starts is caller memory and the copy

@@ -411,6 +411,39 @@ def test_strided_copy_softmax_dot(oracle, dev):
     assert abs(got - float(np.dot(a.astype(np.float64), b.astype(np.float64)))) < 1e-3
 
 
+DEAD_ROW_SNIPPETS = {
+    # ranges exist: the host answers, no read-back (rows 7.. of a 10 x 5 causal window have no key left)
+    "host_ranges": """
+cfg = abi.BltMaskConfig(); cfg.seq_len_q, cfg.seq_len_kv = 10, 5
+cfg.is_causal, cfg.sliding_window = True, 2
+""",
+    # interleaved groups: no ranges, the kernel flags live rows and the count is read back
+    "device_flags": """
+cfg = abi.BltMaskConfig(); cfg.seq_len_q, cfg.seq_len_kv = 3, 4
+qg, kg = abi.size_array([0, 1, 2]), abi.size_array([0, 1, 0, 1])
+cfg.query_group_ids, cfg.kv_group_ids, cfg.bidirectional_within_group = qg, kg, True
+""",
+}
+
+
+@pytest.mark.parametrize("name", list(DEAD_ROW_SNIPPETS))
+def test_mask_builder_dead_row_is_fatal(name, dev):
+    """A query row without any allowed key ends the process with the reference's message
+    (csrc/ops/mask_builder_cpu.c:93), on both ways the device builder has of finding it."""
+    import subprocess
+    import sys
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = ("import ctypes as C, sys\nsys.path.insert(0, %r)\nimport torch\nfrom fblt_amd import abi, api\n"
+            "lib = api.load()\n" % root) + DEAD_ROW_SNIPPETS[name] + (
+            "arena = lib.blt_arena_create(1 << 20, abi.BLT_BACKEND_HIP)\nt = abi.BltTensor()\n"
+            "lib.blt_build_attention_mask(C.byref(cfg), C.byref(t), arena)\nlib.blt_backend_pass_sync_hip()\n"
+            "print('SURVIVED')\n")
+    p = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert p.returncode == 1, (p.returncode, p.stdout, p.stderr)
+    assert "query position has no valid key" in p.stderr and "SURVIVED" not in p.stdout
+
+
 @pytest.mark.parametrize("rows,src_rows,row_len", [(1, 7, 16), (5, 40, 33), (130, 512, 16), (300, 64, 64)])
 def test_rows_gather(rows, src_rows, row_len, dev):
     """blt_rows_gather (csrc/ops/gather_scatter.h:41-42): dst[i, :] = src[pos[i], :], positions a host
