@@ -638,6 +638,15 @@ def cpu_dense(w, budget_s):
                       % (passes, w.name, spent), "ms_per_pass": spent / passes * 1e3}
 
 
+def _chunk_causal(kw):
+    """The block-verify workload with causal rows: row r of a chunk sees the prefix and rows <= r."""
+    import dataclasses
+    n, E = kw.n, kw.E
+    pairs = float(kw.lens.astype("int64").sum()) * n + kw.batch * n * (n + 1) / 2.0
+    return dataclasses.replace(kw, name="c5_chunk_causal_n%d" % n, kind="causal",
+                               flops=4.0 * kw.hd * kw.H * pairs)
+
+
 def cpu_kv(kw, budget_s, max_steps):
     from oracle import binding, runner as orunner
     lib = binding.load_oracle()
@@ -742,6 +751,11 @@ def main():
         for B in (4, 8, 16):
             others["c5_B%d" % B], k5 = bench_kv(workloads.config5(B=B), K, W)
             log("c5_B%d" % B, json.dumps(others["c5_B%d" % B]))
+        # the sibling shape the reference's KV path really runs: a chunk-causal block of 16 new rows
+        # over the cached prefix (a prefill chunk, kv_cache.c:229-236), not committed so that it repeats
+        others["c5_chunk_causal_n16"], _ = bench_kv(_chunk_causal(workloads.config5(B=16)), K, W)
+        others["c5_chunk_causal_n16"]["roofline_hbm"]["traffic"] = None
+        log("c5_chunk_causal_n16", json.dumps(others["c5_chunk_causal_n16"]))
     # batch-swept prefill: the same kernels away from the launch floor
     if want("sweep"):
         for name, make in (("c1_x64", lambda: workloads.config1(batch=64)),
@@ -807,6 +821,7 @@ def main():
         if want("c5"):
             for B in (4, 8, 16):
                 others["c5_B%d" % B]["cpu_baseline"] = cpu_kv(workloads.config5(B=B, steps=1), 1.0, 1)
+            others["c5_chunk_causal_n16"]["cpu_baseline"] = cpu_kv(_chunk_causal(workloads.config5(B=16, steps=1)), 1.0, 1)
 
     line = {
         "metric": "attn_tokens_per_s", "value": head["tokens_per_s"], "unit": "tokens/s",
