@@ -211,6 +211,46 @@ def test_single_head_shapes(nq, nk, hd, masked, oracle, dev):
         assert (got[0, 1:] == 0).all() and (gw[0] == 0).all()
 
 
+@pytest.mark.parametrize("seed", range(40))
+def test_single_head_randomised(seed, oracle, dev):
+    """Seeded draws of everything the per-head call leaves open: ragged sizes, head widths with and
+    without the 16-byte fast paths, padded row strides, a column offset in the output, the mask given
+    as nothing / the causal flag / a dense additive mask with -inf, finite biases and dead rows, and
+    the scale."""
+    lib = api.load()
+    rs = np.random.RandomState(7000 + seed)
+    nq = int(rs.choice([1, 2, 7, 31, 32, 33, 64, 100, 129, 200]))
+    nk = int(rs.choice([1, 3, 31, 32, 33, 65, 128, 257, 400]))
+    hd = int(rs.choice([4, 8, 12, 16, 32, 48, 64, 96, 128]))
+    pad = int(rs.choice([0, 0, 4, 3]))
+    qs, ks, vs = hd + pad, hd + int(rs.choice([0, 4, 5])), hd + int(rs.choice([0, 8, 1]))
+    col = int(rs.choice([0, 4, 1]))
+    os_ = hd + col + int(rs.choice([0, 4, 2]))
+    kind = rs.choice(["none", "causal", "dense"])
+    q = rs.randn(nq, qs).astype(np.float32)
+    k = rs.randn(nk, ks).astype(np.float32)
+    v = rs.randn(nk, vs).astype(np.float32)
+    scale = float(rs.choice([1.0 / np.sqrt(np.float32(hd)), 0.05, 1.0]))
+    mask = None
+    if kind == "dense":
+        mask = np.where(rs.rand(nq, nk) < 0.5, -np.inf, 0.0).astype(np.float32)
+        bias = rs.rand(nq, nk) < 0.2
+        mask[bias & np.isfinite(mask)] = rs.randn(int((bias & np.isfinite(mask)).sum())).astype(np.float32)
+        mask[rs.randint(nq), :] = -np.inf
+    out_ref = np.zeros((nq, os_), dtype=np.float32)
+    w_ref = np.zeros((nq, nk), dtype=np.float32)
+    flat = None if mask is None else mask.reshape(-1)
+    a = binding.head_args(q.reshape(-1), k.reshape(-1), v.reshape(-1), out_ref.reshape(-1), nq, nk, hd, scale,
+                          qs, ks, vs, os_, col, weights=w_ref.reshape(-1), mask=flat, causal=kind == "causal")
+    assert oracle.orc_attention_head_core(C.byref(a)) == 0
+    got, gw = _run_single(lib, q.reshape(-1), k.reshape(-1), v.reshape(-1), nq, nk, hd, scale, qs, ks, vs, os_, col,
+                          mask=flat, causal=kind == "causal")
+    what = "seed %d nq %d nk %d hd %d strides %d/%d/%d out %d+%d %s" % (seed, nq, nk, hd, qs, ks, vs, os_, col, kind)
+    assert (got[:, :col] == 5.0).all() and (got[:, col + hd:] == 5.0).all(), "columns outside the head slice: " + what
+    assert_close(got[:, col:col + hd], out_ref[:, col:col + hd], "out " + what)
+    assert_close(gw, w_ref, "weights " + what)
+
+
 def test_additive_mask_values(oracle, dev):
     """A dense mask is additive: finite biases shift the scores, +inf / nan entries drop the key."""
     lib = api.load()
@@ -376,6 +416,36 @@ def test_block_verify(B, batch, oracle, dev):
     assert (lens == kw.lens).all()   # verify does not commit
     assert ck.tobytes() == ref_k.tobytes() and cv.tobytes() == ref_v.tobytes()
     assert_close(out, ref_out, "block verify B=%d" % B)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_kv_step_randomised(seed, oracle, dev):
+    """Seeded draws over the KV step's free choices: sequences, heads, head width, cached lengths
+    (from empty to long), rows per step (single rows, blocks, chunks longer than one launch takes),
+    step kind, window, rotation fused in or not, committing steps in a row."""
+    rs = np.random.RandomState(9100 + seed)
+    batch = int(rs.choice([1, 2, 5, 17]))
+    H, hd = int(rs.choice([1, 2, 4])), int(rs.choice([8, 16, 32, 64]))
+    len_hi = int(rs.choice([1, 6, 40, 130, 300]))
+    kind = "causal" if rs.rand() < 0.6 else "block"
+    n = int(rs.choice([1, 2, 5, 16, 17, 32] + ([33, 40] if kind == "causal" else [])))
+    steps = int(rs.choice([1, 2, 3])) if kind == "causal" else 1
+    rope = bool(rs.rand() < 0.4)
+    kw = workloads.config4(batch=batch, steps=steps, H=H, hd=hd, len_lo=0 if rs.rand() < 0.3 else 1, len_hi=len_hi,
+                           max_seq_len=len_hi + steps * n + int(rs.choice([0, 3])), rope=rope)
+    kw.n, kw.kind, kw.commit = n, kind, kind == "causal"
+    if kind == "causal" and rs.rand() < 0.4:
+        kw.window = int(rs.choice([1, 7, 48]))
+    kw.q_new, kw.k_new, kw.v_new = (rs.randn(kw.steps, kw.batch * n, kw.E).astype(np.float32) for _ in range(3))
+    ref_out, ref_k, ref_v = orunner.run_kv(kw, lib=oracle)
+    d = dev.DeviceKvWorkload(kw)
+    d.run()
+    out, ck, cv, lens = d.results()
+    what = "seed %d batch %d H %d hd %d len<=%d n %d %s steps %d window %s rope %s" % (
+        seed, batch, H, hd, len_hi, n, kind, steps, getattr(kw, "window", 0), rope)
+    assert (lens == kw.lens.astype(np.int64) + (n * steps if kw.commit else 0)).all(), what
+    assert ck.tobytes() == ref_k.tobytes() and cv.tobytes() == ref_v.tobytes(), what
+    assert_close(out, ref_out, "kv step " + what)
 
 
 # ---------------------------------------------------------------------------
