@@ -352,6 +352,21 @@ void decode_step_run(const blt_kv_cache *cache, size_t batch, size_t n, const si
             MatmulArgs probe;
             std::memset(&probe, 0, sizeof(probe));
             probe.m = (uint32_t)rows, probe.k = (uint32_t)E, probe.n = (uint32_t)E;
+            if (xhd == 32 && matmul_takes_norm(probe) && matmul_takes_cross(probe)) {
+                /* norm, Q projection and the rows' cross attention in one launch: a 32x32 tile of the
+                 * projection is one head of 32 rows */
+                MatmulArgs g;
+                std::memset(&g, 0, sizeof(g));
+                g.a = cur, g.b = (const float *)s->cross_weight_q.data, g.out = xq;
+                g.norm_w = (const float *)s->cross_norm_weight.data;
+                g.m = (uint32_t)rows, g.k = (uint32_t)E, g.n = (uint32_t)E;
+                g.lda = g.ldb = g.ldo = (uint32_t)E;
+                g.cross_k = (const float *)cache->cross_k[l].data, g.cross_v = (const float *)cache->cross_v[l].data;
+                g.cross_out = xcomb, g.cross_lo = dev + batch, g.cross_hi = dev + batch + rows;
+                g.cross_rows_per_seq = (uint32_t)n, g.cross_slab_rows = (uint32_t)cache->max_subtokens;
+                g.cross_scale = 1.0f / sqrtf((float)xhd);
+                matmul_f32_launch(g, 0);
+            } else {
             if (matmul_takes_norm(probe)) {
                 gemm(cur, (const float *)s->cross_weight_q.data, xq, rows, E, E, nullptr, nullptr,
                      (const float *)s->cross_norm_weight.data);
@@ -369,6 +384,7 @@ void decode_step_run(const blt_kv_cache *cache, size_t batch, size_t n, const si
             c.slab_rows = cache->max_subtokens;
             c.scale = 1.0f / sqrtf((float)xhd);
             blt_launch("kv_cross_rows", kv_cross_rows_kernel, dim3((unsigned)rows, (unsigned)XH), dim3(64), 0, 0, c);
+            }
             gemm(xcomb, (const float *)s->cross_weight_proj.data, mid, rows, E, E, cur); /* + residual */
             in = mid;
         }

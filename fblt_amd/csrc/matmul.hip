@@ -216,9 +216,9 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_kernel(MatmulArgs g) {
 
 /* 32x32 output tile (bx, by) per workgroup, K split over the NW waves (4, or 8 for long K:
  * the serial chain of chunk loads per wave halves); the first four waves finish the tile. */
-template <bool VEC, bool ROPE, bool GATED, int NW = 4>
+template <bool VEC, bool ROPE, bool GATED, int NW = 4, bool CROSS = false>
 __device__ __forceinline__ void splitk_tile(const MatmulArgs &g, const uint32_t bx, const uint32_t by,
-                                            float (*part)[16][64], float (*part_ss)[32]) {
+                                            float (*part)[16][64], float (*part_ss)[32], float *qt = nullptr) {
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
     const uint32_t h = lane >> 5, c = lane & 31u;
@@ -341,6 +341,49 @@ __device__ __forceinline__ void splitk_tile(const MatmulArgs &g, const uint32_t 
             else v4[i] = silu_times(gate, v4[i]);
         }
     }
+    if (CROSS) {
+        /* The tile is the projected query of 32 rows for head bx: park it, then wave w takes rows
+         * 8w .. 8w+7 with eight lanes per row (four columns each).  Softmax as
+         * blt_softmax_masked_row_inplace: maximum over finite scores, non-finite scores weigh
+         * nothing, an empty or all-dead row gives zeros (same statements as kv_cross_rows_kernel). */
+#pragma unroll
+        for (int i = 0; i < 4; i++) qt[c * 33u + 8u * wave + 4u * h + i] = v4[i];
+        __syncthreads(); /* the waves past the fourth have left */
+        const uint32_t rr = 8u * wave + (lane >> 3), s8 = lane & 7u;
+        const uint32_t R = by * 32u + rr;
+        if (R >= g.m) return;
+        const float4 q4 = make_float4(qt[rr * 33u + 4u * s8], qt[rr * 33u + 4u * s8 + 1u], qt[rr * 33u + 4u * s8 + 2u],
+                                      qt[rr * 33u + 4u * s8 + 3u]);
+        const uint32_t lo = g.cross_lo[R], hi = g.cross_hi[R];
+        const size_t base = (size_t)(R / g.cross_rows_per_seq) * g.cross_slab_rows * g.n + bx * 32u + 4u * s8;
+        auto score = [&](uint32_t j) {
+            const float4 k4 = *reinterpret_cast<const float4 *>(g.cross_k + base + (size_t)j * g.n);
+            float p = q4.x * k4.x + q4.y * k4.y + q4.z * k4.z + q4.w * k4.w;
+            p += __shfl_xor(p, 1, 64);
+            p += __shfl_xor(p, 2, 64);
+            p += __shfl_xor(p, 4, 64);
+            return p * g.cross_scale;
+        };
+        float mx = -__builtin_huge_valf();
+        for (uint32_t j = lo; j < hi; j++) {
+            const float sc = score(j);
+            if (isfinite(sc)) mx = fmaxf(mx, sc);
+        }
+        float sum = 0.f;
+        float4 o4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (uint32_t j = lo; j < hi; j++) {
+            const float sc = score(j);
+            const float e = isfinite(sc) ? expf(sc - mx) : 0.f;
+            if (e == 0.f) continue;
+            sum += e;
+            const float4 vv = *reinterpret_cast<const float4 *>(g.cross_v + base + (size_t)j * g.n);
+            o4.x += e * vv.x, o4.y += e * vv.y, o4.z += e * vv.z, o4.w += e * vv.w;
+        }
+        const float inv = sum > 0.f ? 1.0f / sum : 0.f;
+        *reinterpret_cast<float4 *>(g.cross_out + (size_t)R * g.n + bx * 32u + 4u * s8) =
+            make_float4(o4.x * inv, o4.y * inv, o4.z * inv, o4.w * inv);
+        return;
+    }
     if (row >= g.m) return;
     const bool vst = VEC && (g.ldo % 4u == 0u) && ((reinterpret_cast<uintptr_t>(g.out) & 15u) == 0u) &&
                      ((reinterpret_cast<uintptr_t>(g.residual) & 15u) == 0u) &&
@@ -355,11 +398,12 @@ __device__ __forceinline__ void splitk_tile(const MatmulArgs &g, const uint32_t 
     }
 }
 
-template <bool VEC, bool ROPE, bool GATED, int NW = 4>
+template <bool VEC, bool ROPE, bool GATED, int NW = 4, bool CROSS = false>
 __global__ __launch_bounds__(64 * NW, 2) void matmul_splitk_kernel(MatmulArgs g) {
     __shared__ float part[(GATED ? 2 : 1) * NW][16][64];
     __shared__ float part_ss[NW][32];
-    splitk_tile<VEC, ROPE, GATED, NW>(g, blockIdx.x, blockIdx.y, part, part_ss);
+    __shared__ float qt[CROSS ? 32 * 33 : 1];
+    splitk_tile<VEC, ROPE, GATED, NW, CROSS>(g, blockIdx.x, blockIdx.y, part, part_ss, qt);
 }
 
 /* Two independent products in one launch: the tile rows of the second are
@@ -517,6 +561,11 @@ template <bool VEC, bool ROPE>
 void launch_splitk(const MatmulArgs &g, dim3 grid, hipStream_t s) {
     /* eight waves once every wave still gets a chunk (K >= 256) and the launch leaves the chip room for them */
     const bool eight = g.k >= 256u && (uint64_t)grid.x * grid.y <= 512u;
+    if (g.cross_k) {
+        if constexpr (VEC && !ROPE)
+            blt_launch("matmul_splitk_cross", matmul_splitk_kernel<true, false, false, 4, true>, grid, dim3(256), 0, s, g);
+        return;
+    }
     if (g.b2) blt_launch("matmul_splitk", matmul_splitk_kernel<VEC, ROPE, true>, grid, dim3(256), 0, s, g);
     else if (eight) blt_launch("matmul_splitk", matmul_splitk_kernel<VEC, ROPE, false, 8>, grid, dim3(512), 0, s, g);
     else blt_launch("matmul_splitk", matmul_splitk_kernel<VEC, ROPE, false>, grid, dim3(256), 0, s, g);
@@ -525,6 +574,10 @@ void launch_splitk(const MatmulArgs &g, dim3 grid, hipStream_t s) {
 } // namespace
 
 bool matmul_takes_gated(const MatmulArgs &g) { return choose_path(g) != PATH_MFMA; }
+bool matmul_takes_cross(const MatmulArgs &g) {
+    return g.m > 32u && choose_path(g) == PATH_SPLITK && g.n % 32u == 0u && g.k % 4u == 0u && !g.b2 && !g.residual &&
+           !(g.rope_cos != nullptr && g.rope_cols > 0);
+}
 bool matmul_takes_norm(const MatmulArgs &g) {
     const Path path = choose_path(g);
     return path == PATH_SPLITK || (path == PATH_SKINNY && g.k <= SKINNY_KC);
@@ -569,6 +622,12 @@ void matmul_f32_launch(const MatmulArgs &g, hipStream_t s) {
         return;
     }
     const bool vec = vec_ok(g);
+    if (g.cross_k) {
+        BLT_REQUIRE(matmul_takes_cross(g) && vec && g.cross_v && g.cross_out && g.cross_lo && g.cross_hi &&
+                        g.cross_rows_per_seq >= 1u && aligned16(g.cross_k) && aligned16(g.cross_v) &&
+                        aligned16(g.cross_out),
+                    "matmul: the cross-attention epilogue is not available for this shape");
+    }
     if (path == PATH_SPLITK) {
         const dim3 sgrid((g.n + 31u) / 32u, (g.m + 31u) / 32u);
         if (rope) {
