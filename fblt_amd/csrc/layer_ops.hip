@@ -16,6 +16,7 @@
 #include "hip_check.h"
 #include "launch.h"
 #include "matmul.h"
+#include "cross_rows_device.h"
 
 #include <algorithm>
 #include <cmath>
@@ -241,49 +242,13 @@ struct CrossRowsArgs {
     float scale;
 };
 
-/* One wave per (new row, head): the row sees the few sub-tokens of its latent
- * patch (kv_cache.c:240-251), so the keys are walked one after the other,
- * lanes over the head's columns.  Softmax as blt_softmax_masked_row_inplace:
- * maximum over finite scores, non-finite scores weigh nothing, an empty or
- * all-dead row gives zeros. */
+/* One wave per (new row, head), see cross_rows_device.h. */
 __global__ __launch_bounds__(64) void kv_cross_rows_kernel(CrossRowsArgs a) {
     const uint32_t R = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
     const uint32_t seq = R / a.n;
-    const uint32_t lo = a.lo[R], hi = a.hi[R];
-    const float *q = a.q + (size_t)R * a.E + head * a.xhd;
-    const float *kb = a.k + (size_t)seq * a.slab_rows * a.E + head * a.xhd;
-    const float *vb = a.v + (size_t)seq * a.slab_rows * a.E + head * a.xhd;
-    auto score = [&](uint32_t j) {
-        float p = 0.f;
-        for (uint32_t d = lane; d < a.xhd; d += 64u) p += q[d] * kb[(size_t)j * a.E + d];
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) p += __shfl_xor(p, off, 64);
-        return p * a.scale;
-    };
-    float mx = -INFINITY;
-    for (uint32_t j = lo; j < hi; j++) {
-        const float s = score(j);
-        if (isfinite(s)) mx = fmaxf(mx, s);
-    }
-    float sum = 0.f;
-    float acc[4] = {0.f, 0.f, 0.f, 0.f}; /* head widths up to 256 columns */
-    for (uint32_t j = lo; j < hi; j++) {
-        const float s = score(j);
-        const float e = isfinite(s) ? expf(s - mx) : 0.f;
-        if (e == 0.f) continue;
-        sum += e;
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            const uint32_t d = lane + 64u * t;
-            if (d < a.xhd) acc[t] += e * vb[(size_t)j * a.E + d];
-        }
-    }
-    const float inv = sum > 0.f ? 1.0f / sum : 0.f;
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-        const uint32_t d = lane + 64u * t;
-        if (d < a.xhd) a.out[(size_t)R * a.E + head * a.xhd + d] = acc[t] * inv;
-    }
+    cross_row_head(a.q + (size_t)R * a.E + head * a.xhd, a.k + (size_t)seq * a.slab_rows * a.E + head * a.xhd,
+                   a.v + (size_t)seq * a.slab_rows * a.E + head * a.xhd, a.lo[R], a.hi[R], a.E, a.xhd, a.scale,
+                   a.out + (size_t)R * a.E + head * a.xhd, lane);
 }
 
 bool cross_fires(const blt_local_decoder_config *c, size_t layer) {
@@ -352,9 +317,11 @@ void decode_step_run(const blt_kv_cache *cache, size_t batch, size_t n, const si
             MatmulArgs probe;
             std::memset(&probe, 0, sizeof(probe));
             probe.m = (uint32_t)rows, probe.k = (uint32_t)E, probe.n = (uint32_t)E;
-            if (xhd == 32 && matmul_takes_norm(probe) && matmul_takes_cross(probe)) {
-                /* norm, Q projection and the rows' cross attention in one launch: a 32x32 tile of the
-                 * projection is one head of 32 rows */
+            probe.cross_head_dim = (uint32_t)xhd;
+            if (matmul_takes_norm(probe) && matmul_takes_cross(probe)) {
+                /* norm, Q projection and the rows' cross attention in one launch: with more than 32
+                 * rows a 32x32 tile of the projection is one 32-wide head of 32 rows; up to 32 rows
+                 * one workgroup of the exact kernel holds the whole projected rows */
                 MatmulArgs g;
                 std::memset(&g, 0, sizeof(g));
                 g.a = cur, g.b = (const float *)s->cross_weight_q.data, g.out = xq;
@@ -364,7 +331,7 @@ void decode_step_run(const blt_kv_cache *cache, size_t batch, size_t n, const si
                 g.cross_k = (const float *)cache->cross_k[l].data, g.cross_v = (const float *)cache->cross_v[l].data;
                 g.cross_out = xcomb, g.cross_lo = dev + batch, g.cross_hi = dev + batch + rows;
                 g.cross_rows_per_seq = (uint32_t)n, g.cross_slab_rows = (uint32_t)cache->max_subtokens;
-                g.cross_scale = 1.0f / sqrtf((float)xhd);
+                g.cross_scale = 1.0f / sqrtf((float)xhd), g.cross_head_dim = (uint32_t)xhd;
                 matmul_f32_launch(g, 0);
             } else {
             if (matmul_takes_norm(probe)) {

@@ -29,18 +29,20 @@ struct MatmulArgs {
     uint32_t m, k, n;
     uint32_t lda, ldb, ldo;
     uint32_t rope_cols, head_dim;
-    /* Optional cross-attention epilogue of the split-K kernel (matmul_takes_cross): the product is
-     * the query projection of a cross block with 32-wide heads, so a 32x32 output tile is one head
-     * of 32 rows; instead of being stored, each row of the tile attends over the sub-tokens
-     * [cross_lo[row], cross_hi[row]) of its sequence's tier-2 slab (row / cross_rows_per_seq) and
-     * the weighted V row goes to cross_out[row, head columns] (csrc/infer/kv_cache.c:303-324).
+    /* Optional cross-attention epilogue (matmul_takes_cross): the product is the query projection
+     * of a cross block with heads cross_head_dim wide; instead of being stored, each projected row
+     * attends, head by head, over the sub-tokens [cross_lo[row], cross_hi[row]) of its sequence's
+     * tier-2 slab (sequence = row / cross_rows_per_seq) and the weighted V row goes to
+     * cross_out[row, head columns] (csrc/infer/kv_cache.c:303-324).  More than 32 rows: split-K
+     * kernel, 32-wide heads (a 32x32 output tile is one head of 32 rows).  Up to 32 rows: the exact
+     * kernel with n <= 256, whose single workgroup per row group holds whole projected rows.
      * out may be null. */
     const float *cross_k;
     const float *cross_v;
     float *cross_out;
     const uint32_t *cross_lo;
     const uint32_t *cross_hi;
-    uint32_t cross_rows_per_seq, cross_slab_rows;
+    uint32_t cross_rows_per_seq, cross_slab_rows, cross_head_dim;
     float cross_scale;
 };
 
@@ -50,7 +52,7 @@ bool matmul_pair_ok(const MatmulArgs &g0, const MatmulArgs &g1);
 void matmul_f32_launch_pair(const MatmulArgs &g0, const MatmulArgs &g1, hipStream_t s);
 /* b2 is only implemented by the kernels for small outputs; false = run the two products and the activation apart */
 bool matmul_takes_gated(const MatmulArgs &g);
-/* the cross-attention epilogue: split-K shapes with n a multiple of 32, no other epilogue */
+/* the cross-attention epilogue for this shape and g.cross_head_dim, no other epilogue set */
 bool matmul_takes_cross(const MatmulArgs &g);
 /* norm_w likewise */
 bool matmul_takes_norm(const MatmulArgs &g);

@@ -37,6 +37,7 @@
 #include "hip_check.h"
 #include "launch.h"
 #include "matmul.h"
+#include "cross_rows_device.h"
 
 #include <stdint.h>
 #include <stdlib.h>
@@ -431,12 +432,13 @@ constexpr uint32_t SKINNY_KC = 512; /* k values of the a rows staged in LDS at a
  * broadcast 16-byte read per four k), the column of b is fetched sixteen k ahead of the chain --
  * the requests of block t+1 are in flight while block t is summed -- and a decode step's single
  * row gets a thread per column rather than a share of a thread. */
-template <int R, bool GATED>
+template <int R, bool GATED, bool CROSS = false>
 __global__ __launch_bounds__(256) void matmul_skinny_kernel(MatmulArgs g) {
 #pragma clang fp contract(off) /* product and sum rounded separately, as the reference's loop */
     constexpr uint32_t KC = SKINNY_KC, UN = 16;
     __shared__ __attribute__((aligned(16))) float sa[R][KC];
     __shared__ float inv_rms[R];
+    __shared__ float sq[CROSS ? R : 1][CROSS ? 256 : 1]; /* the projected rows, for the cross-attention epilogue */
     const uint32_t jj = blockIdx.x * 256u + threadIdx.x;
     const uint32_t j = min(jj, g.n - 1u);
     const uint32_t r0 = blockIdx.y * R;
@@ -523,6 +525,20 @@ __global__ __launch_bounds__(256) void matmul_skinny_kernel(MatmulArgs g) {
             }
         }
     }
+    if (CROSS) { /* one workgroup holds whole rows (n <= 256): a wave per (row, head) */
+#pragma unroll
+        for (int r = 0; r < R; r++) sq[r][threadIdx.x] = acc[r];
+        __syncthreads();
+        const uint32_t xhd = g.cross_head_dim, heads = g.n / xhd;
+        for (uint32_t p = threadIdx.x >> 6; p < (uint32_t)R * heads; p += 4u) {
+            const uint32_t r = p / heads, hh = p % heads, row = r0 + r;
+            if (row >= g.m) continue;
+            const size_t slab = (size_t)(row / g.cross_rows_per_seq) * g.cross_slab_rows * g.n + hh * xhd;
+            cross_row_head(&sq[r][hh * xhd], g.cross_k + slab, g.cross_v + slab, g.cross_lo[row], g.cross_hi[row], g.n,
+                           xhd, g.cross_scale, g.cross_out + (size_t)row * g.n + hh * xhd, threadIdx.x & 63u);
+        }
+        return;
+    }
     if (jj >= g.n) return;
 #pragma unroll
     for (int r = 0; r < R; r++) {
@@ -537,7 +553,8 @@ __global__ __launch_bounds__(256) void matmul_skinny_kernel(MatmulArgs g) {
 template <int R>
 void launch_skinny(const MatmulArgs &g, hipStream_t s) {
     const dim3 grid((g.n + 255u) / 256u, (g.m + R - 1u) / R);
-    if (g.b2) blt_launch("matmul_skinny", matmul_skinny_kernel<R, true>, grid, dim3(256), 0, s, g);
+    if (g.cross_k) blt_launch("matmul_skinny_cross", matmul_skinny_kernel<R, false, true>, grid, dim3(256), 0, s, g);
+    else if (g.b2) blt_launch("matmul_skinny", matmul_skinny_kernel<R, true>, grid, dim3(256), 0, s, g);
     else blt_launch("matmul_skinny", matmul_skinny_kernel<R, false>, grid, dim3(256), 0, s, g);
 }
 
@@ -575,8 +592,12 @@ void launch_splitk(const MatmulArgs &g, dim3 grid, hipStream_t s) {
 
 bool matmul_takes_gated(const MatmulArgs &g) { return choose_path(g) != PATH_MFMA; }
 bool matmul_takes_cross(const MatmulArgs &g) {
-    return g.m > 32u && choose_path(g) == PATH_SPLITK && g.n % 32u == 0u && g.k % 4u == 0u && !g.b2 && !g.residual &&
-           !(g.rope_cos != nullptr && g.rope_cols > 0);
+    if (g.b2 || g.residual || (g.rope_cos != nullptr && g.rope_cols > 0) || g.cross_head_dim == 0u ||
+        g.n % g.cross_head_dim != 0u)
+        return false;
+    const Path path = choose_path(g);
+    if (path == PATH_SKINNY) return g.n <= 256u && g.cross_head_dim <= 256u;
+    return g.m > 32u && path == PATH_SPLITK && g.cross_head_dim == 32u && g.n % 32u == 0u && g.k % 4u == 0u;
 }
 bool matmul_takes_norm(const MatmulArgs &g) {
     const Path path = choose_path(g);
@@ -615,6 +636,9 @@ void matmul_f32_launch(const MatmulArgs &g, hipStream_t s) {
     BLT_REQUIRE(g.norm_w == nullptr || matmul_takes_norm(g), "matmul: the fused row norm is not available for this shape");
     const dim3 block(256);
     if (path == PATH_SKINNY) {
+        BLT_REQUIRE(g.cross_k == nullptr || (matmul_takes_cross(g) && g.cross_v && g.cross_out && g.cross_lo &&
+                                             g.cross_hi && g.cross_rows_per_seq >= 1u),
+                    "matmul: the cross-attention epilogue is not available for this shape");
         /* rows per workgroup: the serial chains of a thread grow with it, the re-reads of b shrink */
         if (g.m <= 4u) launch_skinny<1>(g, s);
         else if (g.m <= 16u) launch_skinny<2>(g, s);
