@@ -17,6 +17,7 @@
 #include "launch.h"
 #include "matmul.h"
 #include "cross_rows_device.h"
+#include "rope_device.h"
 
 #include <algorithm>
 #include <cmath>
@@ -160,10 +161,74 @@ extern "C" void blt_swiglu_forward_hip(const blt_tensor *gate, const blt_tensor 
     HIP_CHECK_LAUNCH("blt_swiglu_forward");
 }
 
-extern "C" void blt_kv_decode_layer_hip(const blt_kv_attn_cache *cache, const blt_transformer_weights *w,
-                                        const float *rows_in, float *rows_out, const float *rope_cos,
-                                        const float *rope_sin, size_t rope_positions, size_t n, int step_kind,
-                                        int commit, size_t max_len_hint, blt_arena *arena) {
+namespace {
+
+/* Prompt prefill through the step: `n` (> 32) new rows per sequence, causal.  The step kernels take
+ * 32 rows at a time, one slice after the other with few workgroups each; here the rows are staged
+ * once -- Q rotated into a scratch buffer, K rotated and V written through to the slabs, one small
+ * launch -- and the attention of all of them runs as one batch of (sequence, head) problems of the
+ * prefill kernels with the causal diagonal moved by the cached length (csrc/infer/kv_cache.c:
+ * 229-236: j <= base + r, base + r - j < window).  Needs the lengths on the host. */
+__global__ __launch_bounds__(256) void kv_chunk_stage_kernel(const float *__restrict__ qkv, float *__restrict__ q_rot,
+                                                             float *__restrict__ cache_k, float *__restrict__ cache_v,
+                                                             const uint32_t *__restrict__ self_len,
+                                                             const float *__restrict__ rope_cos,
+                                                             const float *__restrict__ rope_sin, uint32_t n, uint32_t E,
+                                                             uint32_t hd, uint64_t max_seq_len) {
+    const uint32_t row = blockIdx.x, b = row / n, r = row % n;
+    const uint32_t pos = self_len[b] + r;
+    const float *src = qkv + (size_t)row * 3u * E;
+    float *kd = cache_k + ((size_t)b * max_seq_len + pos) * E;
+    float *vd = cache_v + ((size_t)b * max_seq_len + pos) * E;
+    for (uint32_t col = 4u * threadIdx.x; col < E; col += 1024u) {
+        const size_t at = (size_t)pos * (hd / 2u) + (col % hd) / 2u;
+        const float4 q4 = *reinterpret_cast<const float4 *>(src + col);
+        const float4 k4 = *reinterpret_cast<const float4 *>(src + E + col);
+        *reinterpret_cast<float4 *>(q_rot + (size_t)row * E + col) = rope_rotate4(q4, rope_cos + at, rope_sin + at);
+        *reinterpret_cast<float4 *>(kd + col) = rope_rotate4(k4, rope_cos + at, rope_sin + at);
+        *reinterpret_cast<float4 *>(vd + col) = *reinterpret_cast<const float4 *>(src + 2u * E + col);
+    }
+}
+
+void long_chunk_attention(const blt_kv_attn_cache *cache, const float *qkv, const float *rope_cos,
+                          const float *rope_sin, size_t rope_positions, size_t n, const size_t *host_base,
+                          float *combined, blt_arena *arena) {
+    const size_t E = cache->embed_dim, H = cache->num_heads, hd = E / H, rows = cache->batch * n;
+    float *q_rot = (float *)blt_arena_alloc(arena, rows * E * sizeof(float), 64);
+    for (size_t b = 0; b < cache->batch; b++)
+        BLT_REQUIRE(host_base[b] + n <= rope_positions && host_base[b] + n <= cache->max_seq_len,
+                    "blt_kv_decode_step: positions exceed the rotary tables or the cache");
+    blt_launch("kv_chunk_stage", kv_chunk_stage_kernel, dim3((unsigned)rows), dim3(256), 0, 0, qkv, q_rot, cache->self_k,
+               cache->self_v, cache->self_len, rope_cos, rope_sin, (uint32_t)n, (uint32_t)E, (uint32_t)hd,
+               (uint64_t)cache->max_seq_len);
+    std::vector<blt_attention_problem> pr(cache->batch * H);
+    const float scale = 1.0f / sqrtf((float)hd);
+    for (size_t b = 0; b < cache->batch; b++) {
+        for (size_t head = 0; head < H; head++) {
+            blt_attention_problem &p = pr[b * H + head];
+            std::memset(&p, 0, sizeof(p));
+            p.head.q = q_rot + b * n * E + head * hd;
+            p.head.k = cache->self_k + b * cache->max_seq_len * E + head * hd;
+            p.head.v = cache->self_v + b * cache->max_seq_len * E + head * hd;
+            p.head.q_stride = p.head.k_stride = p.head.v_stride = E;
+            p.head.combined = combined + b * n * E;
+            p.head.combined_stride = E;
+            p.head.combined_col_offset = head * hd;
+            p.head.nq = n;
+            p.head.nk = host_base[b] + n;
+            p.head.head_dim = hd;
+            p.head.scale = scale;
+            p.mask_kind = BLT_ATTN_MASK_CAUSAL;
+            p.causal_offset = host_base[b];
+            p.window = cache->window;
+        }
+    }
+    blt_attention_batch_hip(pr.data(), pr.size());
+}
+
+void decode_layer_impl(const blt_kv_attn_cache *cache, const blt_transformer_weights *w, const float *rows_in,
+                       float *rows_out, const float *rope_cos, const float *rope_sin, size_t rope_positions, size_t n,
+                       int step_kind, int commit, size_t max_len_hint, blt_arena *arena, const size_t *host_base) {
     BLT_REQUIRE(cache != NULL && w != NULL && rows_in != NULL && rows_out != NULL && arena != NULL,
                 "blt_kv_decode_layer: arguments must not be NULL");
     BLT_REQUIRE(arena->backend == BLT_BACKEND_HIP, "blt_kv_decode_layer: needs a device arena");
@@ -204,8 +269,12 @@ extern "C" void blt_kv_decode_layer_hip(const blt_kv_attn_cache *cache, const bl
         rmsnorm_launch(rows_in, f32(w->norm1_weight), normed, rows, E);
         gemm(normed, f32(w->attn_qkv_w), qkv, rows, E, 3 * E);
     }
-    blt_kv_rope_attend_step_hip(cache, qkv, 3 * E, qkv + E, 3 * E, qkv + 2 * E, 3 * E, rope_cos, rope_sin,
-                                rope_positions, combined, E, n, step_kind, commit, max_len_hint);
+    if (host_base != nullptr && n > 32 && step_kind == BLT_KV_STEP_CAUSAL && commit == 0 &&
+        (E / cache->num_heads) % 4 == 0)
+        long_chunk_attention(cache, qkv, rope_cos, rope_sin, rope_positions, n, host_base, combined, arena);
+    else
+        blt_kv_rope_attend_step_hip(cache, qkv, 3 * E, qkv + E, 3 * E, qkv + 2 * E, 3 * E, rope_cos, rope_sin,
+                                    rope_positions, combined, E, n, step_kind, commit, max_len_hint);
     gemm(combined, f32(w->attn_proj_w), resid1, rows, E, E, rows_in); /* projection + residual in one pass */
     /* feed-forward block, kv_cache.c:396-414 */
     probe.n = (uint32_t)Hd;
@@ -222,6 +291,16 @@ extern "C" void blt_kv_decode_layer_hip(const blt_kv_attn_cache *cache, const bl
     }
     gemm(gate, f32(w->ffn_down_w), rows_out, rows, Hd, E, resid1); /* projection + residual */
     HIP_CHECK_LAUNCH("blt_kv_decode_layer");
+}
+
+} // namespace
+
+extern "C" void blt_kv_decode_layer_hip(const blt_kv_attn_cache *cache, const blt_transformer_weights *w,
+                                        const float *rows_in, float *rows_out, const float *rope_cos,
+                                        const float *rope_sin, size_t rope_positions, size_t n, int step_kind,
+                                        int commit, size_t max_len_hint, blt_arena *arena) {
+    decode_layer_impl(cache, w, rows_in, rows_out, rope_cos, rope_sin, rope_positions, n, step_kind, commit,
+                      max_len_hint, arena, nullptr);
 }
 
 /* ===================================================================== */
@@ -371,9 +450,9 @@ void decode_step_run(const blt_kv_cache *cache, size_t batch, size_t n, const si
         w.ffn_down_w = &s->ffn_down_w;
         float *next = (cur == ping) ? pong : ping;
         arena->offset = arena_mark; /* the layer's work buffers are reused by the next layer */
-        blt_kv_decode_layer_hip(&view, &w, in, next, (const float *)dec->rope_cos_cache.data,
-                                (const float *)dec->rope_sin_cache.data, cfg->max_seq_len, n, BLT_KV_STEP_CAUSAL, 0,
-                                max_total, arena);
+        decode_layer_impl(&view, &w, in, next, (const float *)dec->rope_cos_cache.data,
+                          (const float *)dec->rope_sin_cache.data, cfg->max_seq_len, n, BLT_KV_STEP_CAUSAL, 0, max_total,
+                          arena, base);
         cur = next;
     }
     gemm(cur, (const float *)dec->lm_head_weight.data, logits, rows, E, V); /* kv_cache.c:416 */

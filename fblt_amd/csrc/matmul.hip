@@ -430,8 +430,8 @@ constexpr uint32_t SKINNY_KC = 512; /* k values of the a rows staged in LDS at a
  * output is the reference's own sum: k ascending, product and sum rounded separately.  What the
  * kernel is built around is the latency of that serial chain: the rows of a sit in LDS (one
  * broadcast 16-byte read per four k), the column of b is fetched sixteen k ahead of the chain --
- * the requests of block t+1 are in flight while block t is summed -- and a decode step's single
- * row gets a thread per column rather than a share of a thread. */
+ * the requests of block t+1 are in flight while block t is summed -- and every row gets a thread
+ * per column of its own (R = 1 at launch) rather than a share of a thread. */
 template <int R, bool GATED, bool CROSS = false>
 __global__ __launch_bounds__(256) void matmul_skinny_kernel(MatmulArgs g) {
 #pragma clang fp contract(off) /* product and sum rounded separately, as the reference's loop */
@@ -639,10 +639,9 @@ void matmul_f32_launch(const MatmulArgs &g, hipStream_t s) {
         BLT_REQUIRE(g.cross_k == nullptr || (matmul_takes_cross(g) && g.cross_v && g.cross_out && g.cross_lo &&
                                              g.cross_hi && g.cross_rows_per_seq >= 1u),
                     "matmul: the cross-attention epilogue is not available for this shape");
-        /* rows per workgroup: the serial chains of a thread grow with it, the re-reads of b shrink */
-        if (g.m <= 4u) launch_skinny<1>(g, s);
-        else if (g.m <= 16u) launch_skinny<2>(g, s);
-        else launch_skinny<4>(g, s);
+        /* one row per workgroup (measured against 2 and 4 at every shape of the decoder: the extra
+         * chains of a lane cost more than the re-reads of b from L2) */
+        launch_skinny<1>(g, s);
         return;
     }
     const bool vec = vec_ok(g);

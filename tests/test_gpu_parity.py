@@ -1055,13 +1055,15 @@ def test_kv_decode_step_single_sequence(case, impl, oracle, dev):
         lib.blt_arena_destroy(arena)
 
 
-def test_kv_decode_step_long_prefill(oracle, dev):
-    """A prompt prefill in one call: more new rows than one attention launch takes (45, then 1, then
-    50 rows), against the restated step; logits and tiers after every call."""
+@pytest.mark.parametrize("window", [0, 20])
+def test_kv_decode_step_long_prefill(window, oracle, dev):
+    """A prompt prefill in one call: more new rows than one step launch takes (45, then 1, then
+    50 rows: staged once and attended as one batch of prefill problems), with and without a local
+    window, against the restated step; logits and tiers after every call."""
     import torch
     from fblt_amd import decoder
     lib = api.load()
-    c = dict(E=128, H=4, XH=4, L=2, hidden=256, V=256, max_len=128, k=1, window=0, all_layers=True, placement=0)
+    c = dict(E=128, H=4, XH=4, L=2, hidden=256, V=256, max_len=128, k=1, window=window, all_layers=True, placement=0)
     E, V, L = c["E"], c["V"], c["L"]
     rs = np.random.RandomState(911)
     host, device = _decoders(oracle, c, 912)
