@@ -100,12 +100,15 @@ void blt_cross_attention_forward_hip(const blt_tensor *query_in, const blt_tenso
  * weights and rows that live in device memory.  refresh_cross: one launch per
  * firing layer computes K and V of the new sub-tokens straight into the
  * tier-2 slabs.  decode_step: per layer the cross block (RMSNorm + Q
- * projection, the rows' few sub-tokens, projection + residual: 3 launches)
- * and the self-attention / feed-forward layer (5 launches), then the LM
- * head; the dense masks, strided copies and per-head calls of the reference
- * are gone, the row groups follow the same latent rule (kv_cache.c:199-213).
- * Up to 32 new rows every projection is bit-identical to the CPU reference;
- * attention is within fp32 tolerance. */
+ * projection with the rows' few sub-tokens attended in its epilogue where the
+ * shape allows, projection + residual: 2-3 launches) and the self-attention /
+ * feed-forward layer (5 launches), then the LM head; the dense masks, strided
+ * copies and per-head calls of the reference are gone, the row groups follow
+ * the same latent rule (kv_cache.c:199-213).  A prompt chunk of more than 32
+ * rows is staged once (rotation, write-through) and attended by the prefill
+ * kernels with the causal diagonal moved by the cached length.  Up to 32 new
+ * rows every projection is bit-identical to the CPU reference; attention is
+ * within fp32 tolerance. */
 void blt_kv_cache_refresh_cross_hip(blt_kv_cache *cache, const blt_tensor *patch_in, const blt_patch_info *patches,
                                     size_t num_patches, size_t from_patch, blt_arena *arena);
 void blt_kv_decode_step_hip(blt_kv_cache *cache, const blt_tensor *patch_in, const blt_patch_info *patches,
