@@ -315,17 +315,14 @@ void plan_launch(const blt_attention_plan &pl, const AttnProb *dev, const AttnTi
 }
 
 /* Staging for one-shot batches: descriptors go host vector -> pinned buffer ->
- * device buffer with a truly asynchronous copy on the null stream.  The
+ * device buffer with a truly asynchronous copy on the library's stream.  The
  * device buffer can be reused by the next call because that call's copy is
- * ordered behind this call's kernels; the pinned buffer is guarded by an
- * event recorded right after the copy. */
+ * ordered behind this call's kernels; the pinned side is the calling thread's
+ * ring of buffers (blt_upload_staged). */
 struct Staging {
     blt_attention_plan plan;
-    void *pinned = nullptr;
     void *device = nullptr;
     size_t capacity = 0;
-    hipEvent_t copied = nullptr;
-    bool in_flight = false;
 
     void run() {
         const size_t pbytes = plan.host.size() * sizeof(AttnProb);
@@ -335,26 +332,19 @@ struct Staging {
         BLT_REQUIRE(!blt_stream_capturing(),
                     "blt_attention_batch: this batch stages its descriptors through host memory, which a graph "
                     "cannot replay; use a resident plan (blt_attention_plan_*) or a strided batch under capture");
-        if (!copied) HIP_CHECK(hipEventCreateWithFlags(&copied, hipEventDisableTiming));
-        if (in_flight) {
-            HIP_CHECK(hipEventSynchronize(copied));
-            in_flight = false;
-        }
         if (need > capacity) {
             if (device) {
                 HIP_CHECK(hipDeviceSynchronize());
                 HIP_CHECK(hipFree(device));
-                HIP_CHECK(hipHostFree(pinned));
             }
             capacity = std::max<size_t>(2 * need, 64 * 1024);
             HIP_CHECK(hipMalloc(&device, capacity));
-            HIP_CHECK(hipHostMalloc(&pinned, capacity, hipHostMallocDefault));
         }
-        std::memcpy(pinned, plan.host.data(), pbytes);
-        if (tbytes) std::memcpy(static_cast<char *>(pinned) + pbytes, plan.tiles.data(), tbytes);
-        HIP_CHECK(hipMemcpyAsync(device, pinned, need, hipMemcpyHostToDevice, blt_stream()));
-        HIP_CHECK(hipEventRecord(copied, blt_stream()));
-        in_flight = true;
+        /* the device copy is rewritten in stream order, behind the kernels of the previous call that
+         * read it; the host side goes through the ring of pinned buffers, so consecutive calls do
+         * not wait for each other */
+        blt_upload_staged(device, plan.host.data(), pbytes);
+        if (tbytes) blt_upload_staged(static_cast<char *>(device) + pbytes, plan.tiles.data(), tbytes);
         plan_launch(plan, static_cast<const AttnProb *>(device),
                     reinterpret_cast<const AttnTile *>(static_cast<const char *>(device) + pbytes));
     }

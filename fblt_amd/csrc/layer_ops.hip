@@ -545,6 +545,40 @@ extern "C" void blt_kv_cache_refresh_cross_seq_hip(blt_kv_cache *cache, size_t s
     refresh_cross_seq(cache, seq, patch_in, patches, num_patches, from_patch);
 }
 
+namespace {
+
+/* blt_patch_decoder_latent_at (csrc/ops/patch_pool_cpu.c:114-131) for the consecutive positions
+ * base .. base + n - 1: when the table tiles its range (each patch starts where the previous one
+ * ends, the only kind the model builds) the owner only moves forward, so one walk serves all rows;
+ * any other table goes row by row through the general rule. */
+void latent_ids(const blt_patch_info *patches, size_t num_patches, size_t base, size_t n, size_t *out) {
+    bool tiling = n > 4; /* a few rows: the general rule's own scan is as short as the check below */
+    for (size_t p = 0; p < num_patches && tiling; p++)
+        tiling = patches[p].length >= 1 &&
+                 (p + 1 == num_patches || patches[p + 1].start_idx == patches[p].start_idx + patches[p].length);
+    if (!tiling) {
+        for (size_t r = 0; r < n; r++) out[r] = blt_patch_decoder_latent_at(patches, num_patches, base + r);
+        return;
+    }
+    size_t p = 0;
+    for (size_t r = 0; r < n; r++) {
+        const size_t pos = base + r;
+        if (pos < patches[0].start_idx) {
+            out[r] = 0;
+            continue;
+        }
+        while (p < num_patches && pos >= patches[p].start_idx + patches[p].length) p++;
+        if (p == num_patches) {
+            out[r] = num_patches - 1; /* past the last patch */
+            continue;
+        }
+        const bool closes = pos - patches[p].start_idx + 1 == patches[p].length;
+        out[r] = (closes && p + 1 < num_patches) ? p : (p == 0 ? 0 : p - 1);
+    }
+}
+
+} // namespace
+
 extern "C" void blt_kv_decode_step_hip(blt_kv_cache *cache, const blt_tensor *patch_in, const blt_patch_info *patches,
                                        size_t num_patches, const blt_tensor *d0_rows, int trailing_closed,
                                        blt_tensor *logits_out, blt_arena *arena) {
@@ -572,7 +606,7 @@ extern "C" void blt_kv_decode_step_hip(blt_kv_cache *cache, const blt_tensor *pa
     BLT_REQUIRE(num_patches * cache->k <= cache->max_subtokens,
                 "blt_kv_decode_step: sub-token count exceeds cache capacity");
     std::vector<size_t> group(n); /* kv_cache.c:199-213 */
-    for (size_t r = 0; r < n; r++) group[r] = blt_patch_decoder_latent_at(patches, num_patches, base + r);
+    latent_ids(patches, num_patches, base, n, group.data());
     if (trailing_closed) group[n - 1] = num_patches - 1;
     decode_step_run(cache, 1, n, &base, group.data(), (const float *)d0_rows->data, (float *)logits_out->data, arena);
     cache->self_len = total;
@@ -607,8 +641,7 @@ extern "C" void blt_kv_decode_step_batched_hip(blt_kv_cache *cache, size_t *self
         BLT_REQUIRE(self_len[b] + n <= cache->max_seq_len, "blt_kv_decode_step_batched: exceeds cache capacity");
         BLT_REQUIRE(num_patches[b] * cache->k <= cache->max_subtokens,
                     "blt_kv_decode_step_batched: sub-token count exceeds cache capacity");
-        for (size_t r = 0; r < n; r++)
-            group[b * n + r] = blt_patch_decoder_latent_at(patches[b], num_patches[b], self_len[b] + r);
+        latent_ids(patches[b], num_patches[b], self_len[b], n, group.data() + b * n);
         if (trailing_closed != NULL && trailing_closed[b]) group[b * n + n - 1] = num_patches[b] - 1;
     }
     decode_step_run(cache, batch, n, self_len, group.data(), (const float *)d0_rows->data,
