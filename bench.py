@@ -509,7 +509,7 @@ def _decode_step_setup(batch, L, E, H, hidden, V, len_hi, total_steps, seed=17):
     return max_len, lens, weights, tables
 
 
-def bench_decode_step(steps, warmup, batch=64, L=2, E=128, H=4, hidden=512, V=256, len_hi=512):
+def bench_decode_step(steps, warmup, batch=64, L=2, E=128, H=4, hidden=512, V=256, len_hi=512, n=1):
     """blt_kv_decode_step_batched_hip: the whole incremental decoder step (per layer the cross block
     over the tier-2 cache and the self-attention / feed-forward layer, then the LM head) for `batch`
     sequences, one new row each, per step."""
@@ -519,7 +519,10 @@ def bench_decode_step(steps, warmup, batch=64, L=2, E=128, H=4, hidden=512, V=25
     from fblt_amd import abi, api, decoder
     lib = api.load()
     hd, half = E // H, E // H // 2
-    max_len, lens, weights, tables = _decode_step_setup(batch, L, E, H, hidden, V, len_hi, 2 * (warmup + steps))
+    # n = 1: consecutive steps, the sequences grow; n > 1 (a prompt chunk): every call starts again from
+    # the same cached lengths
+    max_len, lens, weights, tables = _decode_step_setup(batch, L, E, H, hidden, V, len_hi,
+                                                        2 * (warmup + steps) if n == 1 else n)
     view = lambda t: abi.tensor_view(t.data_ptr(), tuple(t.shape), abi.BLT_BACKEND_HIP)
     cos, sin = torch.zeros((max_len, half), device="cuda"), torch.zeros((max_len, half), device="cuda")
     vc, vs = view(cos), view(sin)
@@ -544,14 +547,17 @@ def bench_decode_step(steps, warmup, batch=64, L=2, E=128, H=4, hidden=512, V=25
     mark = arena.contents.offset
     table_ptrs = (C.POINTER(abi.BltPatchInfo) * batch)(*(C.cast(t, C.POINTER(abi.BltPatchInfo)) for t in tables))
     num = abi.size_array([P] * batch)
-    x = torch.randn(batch, E, generator=g, dtype=torch.float32).cuda()
-    logits = torch.zeros((batch, V), device="cuda")
+    x = torch.randn(batch * n, E, generator=g, dtype=torch.float32).cuda()
+    logits = torch.zeros((batch * n, V), device="cuda")
     vx, vl = view(x), view(logits)
     self_len = abi.size_array(lens.tolist())
 
     def run(count):
         for _ in range(count):
             arena.contents.offset = mark
+            if n > 1:
+                for b in range(batch):
+                    self_len[b] = int(lens[b])
             lib.blt_kv_decode_step_batched_hip(cache, self_len, table_ptrs, num, None, C.byref(vx), C.byref(vl), arena)
     run(warmup)
     lib.blt_backend_pass_sync_hip()
@@ -570,31 +576,37 @@ def bench_decode_step(steps, warmup, batch=64, L=2, E=128, H=4, hidden=512, V=25
     lib.blt_kv_cache_destroy(cache)
     lib.blt_arena_destroy(arena)
     avg_s = sum(v[1] for v in prof.values()) / 1e3 / steps
-    mean_keys = float(lens.sum()) + batch * (warmup + (steps - 1) / 2.0) + batch
+    rows = batch * n
+    if n == 1:
+        mean_keys = float(lens.sum()) + batch * (warmup + (steps - 1) / 2.0) + batch   # keys attended per step
+        read_keys = mean_keys
+    else:
+        mean_keys = n * float(lens.sum()) + batch * n * (n + 1) / 2.0                  # (row, key) pairs per call
+        read_keys = float(lens.sum()) + rows
     per_layer_w = E * E * 2 + E * 3 * E + E * E + 3 * E * hidden   # cross q / proj, qkv, proj, up / gate / down
-    flops = L * (batch * 2.0 * per_layer_w + 4.0 * hd * H * mean_keys + 4.0 * E * batch) + batch * 2.0 * E * V
-    nbytes = 4.0 * (L * (2 * E * mean_keys + per_layer_w + 2 * E * batch) + E * V)
-    res = {"workload": "decoder step: %d sequences, %d layers (cross block in each), E=%d, H=%d, hidden=%d, V=%d, "
-                       "cached 1..%d" % (batch, L, E, H, hidden, V, len_hi),
+    flops = L * (rows * 2.0 * per_layer_w + 4.0 * hd * H * mean_keys + 4.0 * E * rows) + rows * 2.0 * E * V
+    nbytes = 4.0 * (L * (2 * E * read_keys + per_layer_w + 2 * E * rows) + E * V)
+    res = {"workload": "decoder step: %d sequences x %d new rows, %d layers (cross block in each), E=%d, H=%d, "
+                       "hidden=%d, V=%d, cached 1..%d" % (batch, n, L, E, H, hidden, V, len_hi),
            "kernel": "+".join(sorted(prof)), "launches_per_step": sum(v[0] for v in prof.values()) / steps,
-           "tokens_per_step": batch, "us_per_step": wall_plain / steps * 1e6,
+           "tokens_per_step": rows, "us_per_step": wall_plain / steps * 1e6,
            "us_per_step_with_events": wall / steps * 1e6, "kernel_us_avg": avg_s * 1e6,
            "kernel_us_min": min(v[2] for v in prof.values()) * 1e3,
            "per_kernel_us": {k: v[1] * 1e3 / steps for k, v in prof.items()},
-           "tokens_per_s": batch * steps / wall_plain, "tokens_per_s_kernel": batch / avg_s, "flops": flops,
+           "tokens_per_s": rows * steps / wall_plain, "tokens_per_s_kernel": rows / avg_s, "flops": flops,
            "bytes": nbytes, "roofline_hbm": roofline("hbm", nbytes, avg_s), "roofline_mfma": roofline("mfma", flops, avg_s)}
     res["roofline"] = res["roofline_hbm"]
     return res
 
 
-def cpu_decode_step(budget_s, batch=64, L=2, E=128, H=4, hidden=512, V=256, len_hi=512):
+def cpu_decode_step(budget_s, batch=64, L=2, E=128, H=4, hidden=512, V=256, len_hi=512, n=1):
     """The restated decoder step on one host core, one sequence at a time as the reference runs it."""
     import numpy as np
     from fblt_amd import abi, decoder
     from oracle import binding
     lib = binding.load_oracle()
     hd, half = E // H, E // H // 2
-    max_len, lens, weights, tables = _decode_step_setup(batch, L, E, H, hidden, V, len_hi, 40)
+    max_len, lens, weights, tables = _decode_step_setup(batch, L, E, H, hidden, V, len_hi, 40 if n == 1 else n)
     cos, sin = np.empty(max_len * half, dtype=np.float32), np.empty(max_len * half, dtype=np.float32)
     lib.orc_rope_precompute(max_len, 500000.0, hd, binding.fptr(cos), binding.fptr(sin))
     bound = decoder.bind(weights, cos.reshape(max_len, half), sin.reshape(max_len, half), abi.BLT_BACKEND_CPU,
@@ -608,14 +620,15 @@ def cpu_decode_step(budget_s, batch=64, L=2, E=128, H=4, hidden=512, V=256, len_
     for b in range(batch):
         pin = rs.randn(P, E).astype(np.float32)
         assert lib.orc_kv_cache_refresh_cross(cache.ptr, b, binding.fptr(pin.reshape(-1)), P, 0) == 0
-    x, o = rs.randn(batch, E).astype(np.float32), np.zeros((batch, V), dtype=np.float32)
+    x, o = rs.randn(batch * n, E).astype(np.float32), np.zeros((batch * n, V), dtype=np.float32)
     fp = lambda a: binding.fptr(a.reshape(-1))
     steps, spent = 0, 0.0
     while steps < 1 or (spent < budget_s and steps < 16):
         t0 = time.perf_counter()
         for b in range(batch):
-            assert lib.orc_kv_decode_step(cache.ptr, b, int(lens[b]) + steps, tables[b], P, fp(x[b:b + 1]), 1, 0,
-                                          fp(o[b:b + 1])) == 0
+            base = int(lens[b]) + (steps if n == 1 else 0)
+            assert lib.orc_kv_decode_step(cache.ptr, b, base, tables[b], P, fp(x[b * n:(b + 1) * n]), n, 0,
+                                          fp(o[b * n:(b + 1) * n])) == 0
         spent += time.perf_counter() - t0
         steps += 1
     return {"value": spent / steps * 1e6, "unit": "us/step", "cores": 1, "kind": "port",
@@ -801,6 +814,11 @@ def main():
         if not args.no_cpu:
             others["decode_step_b1"]["cpu_baseline"] = cpu_decode_step(2.0, batch=1)
         log("decode_step_b1", json.dumps(others["decode_step_b1"]))
+        # a 512-byte prompt through the same entry point in one call (time to the first token)
+        others["decode_step_prefill_512"] = bench_decode_step(max(10, K // 10), 3, batch=1, len_hi=1, n=512)
+        if not args.no_cpu:
+            others["decode_step_prefill_512"]["cpu_baseline"] = cpu_decode_step(2.0, batch=1, len_hi=1, n=512)
+        log("decode_step_prefill_512", json.dumps(others["decode_step_prefill_512"]))
 
     # the dense-mask builders the callers still use
     if want("masks"):
