@@ -969,6 +969,8 @@ STEP_CASES = [
     dict(E=24, H=3, XH=2, L=3, hidden=40, V=256, max_len=48, k=2, window=7, all_layers=False, placement=0),
     dict(E=128, H=4, XH=4, L=2, hidden=512, V=256, max_len=64, k=1, window=0, all_layers=True, placement=0),
     dict(E=64, H=2, XH=4, L=2, hidden=96, V=50, max_len=32, k=3, window=5, all_layers=False, placement=4),
+    dict(E=64, H=2, XH=2, L=2, hidden=96, V=52, max_len=200, k=1, window=0, all_layers=True, placement=0),
+    dict(E=128, H=4, XH=4, L=1, hidden=128, V=64, max_len=160, k=2, window=30, all_layers=True, placement=0),
 ]
 
 
@@ -1104,7 +1106,8 @@ def test_kv_decode_step_long_prefill(window, oracle, dev):
         lib.blt_arena_destroy(arena)
 
 
-@pytest.mark.parametrize("batch,n,case", [(8, 1, 0), (64, 1, 2), (16, 4, 1), (5, 3, 3), (64, 8, 2)])
+@pytest.mark.parametrize("batch,n,case", [(8, 1, 0), (64, 1, 2), (16, 4, 1), (5, 3, 3), (64, 8, 2),
+                                          (3, 40, 4), (5, 33, 5)])   # chunks of more than 32 rows per sequence
 def test_kv_decode_step_batched(batch, n, case, oracle, dev):
     """blt_kv_decode_step_batched_hip: every sequence of a batched cache in one pass, against the
     restated step run sequence by sequence; two steps in a row."""
