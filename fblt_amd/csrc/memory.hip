@@ -59,7 +59,7 @@ void blt_upload_staged(void *dst, const void *src, size_t bytes) {
     }
     if (bytes > s.capacity) {
         if (s.host) HIP_CHECK(hipHostFree(s.host));
-        s.capacity = bytes < 4096 ? 4096 : 2 * bytes;
+        s.capacity = bytes < 32768 ? 65536 : 2 * bytes; /* few re-allocations: pinning memory costs ~100 us */
         HIP_CHECK(hipHostMalloc(&s.host, s.capacity, hipHostMallocDefault));
     }
     __builtin_memcpy(s.host, src, bytes);
