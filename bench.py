@@ -854,6 +854,9 @@ def main():
         "roofline": head["roofline"],
         "roofline_mfma": head["roofline_mfma"],
         "cpu_baseline": cpu_head,
+        # the other parts of the composite headline metric (decode us/step, verify tokens/s), when they ran
+        "decode_us_per_step": others["c4"]["us_per_step"] if "c4" in others else None,
+        "verify_tokens_per_s": {k: others[k]["tokens_per_s"] for k in ("c5_B4", "c5_B8", "c5_B16") if k in others} or None,
         "workloads": others,
     }
     print(json.dumps(line), flush=True)
