@@ -6,11 +6,15 @@
 A "step" is one pass of the headline workload -- the patch-transformer
 block-causal attention (batch 16, 128 patches, 8 heads of 64, fp32) -- through
 the HIP library: one resident plan, one kernel launch per step, inputs already
-in HBM.  The single JSON line on stdout carries the whole-job throughput of
-that workload, the roofline figures of its kernel (duration from HIP events
-attached to every launch of the timed region), the CPU baseline (the checker
-under oracle/, one host core, bounded sample) and, under "workloads", the same
-figures for the other four attention shapes of the path.
+in HBM.  The last line on stdout is ONE compact JSON object (a few KB): the
+whole-job throughput of that workload, the roofline figures of its kernel
+(duration from HIP events attached to every launch of the timed region), the
+CPU baseline (the reference's own attention core where its build travelled
+with the tree, else the checker under oracle/; one host core, bounded sample),
+the other two parts of the composite metric (decode us/step, verify tokens/s)
+and one summary row per attention shape under "per_config".  The full
+per-workload records go to stderr as they are measured and, together, to
+gpurun_out/bench_detail.json.
 """
 import argparse
 import json
@@ -24,19 +28,33 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 
-# HBM bytes per launch from two `rocprofv3 --pmc` runs (FETCH_SIZE, then
-# WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for
-# the plain 64 MiB streaming copy (--probe-copy-mib 64): x1.999 for FETCH_SIZE,
-# x1.000 for WRITE_SIZE.  The summaries under profiles/ hold the readings.
-MEASURED_TRAFFIC_BYTES = {
-    "c2_patch_block_causal": (6225.1 * 1.999 + 4096.0) * 1024,
-    "c1_local_decoder_causal": (687.0 * 1.999 + 256.0) * 1024,
-    "c3_encoder_cross": (4699.1 * 1.999 + 1024.0) * 1024,
-    "c4_kv_decode": (11857.6 * 1.999 + 108.0) * 1024,          # mean over the 256 growing steps
-    "c5_block_verify_B4": (9488.0 * 1.999 + 896.0) * 1024,     # the three block sizes run the same kernel
-    "c5_block_verify_B8": (9488.0 * 1.999 + 896.0) * 1024,     # and were collected together
-    "c5_block_verify_B16": (9488.0 * 1.999 + 896.0) * 1024,
-}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.md")
+DETAIL_FILE = os.path.join(ROOT, "gpurun_out", "bench_detail.json")
+
+
+def measured_traffic():
+    """{workload name: HBM bytes per launch} from the committed counter summary: one table row per
+    workload holding the FETCH_SIZE and WRITE_SIZE readings (KiB per dispatch, `rocprofv3 --pmc`, one
+    counter per run) and the factors the same counters read for a plain copy of known size.  An
+    absent file or row gives no figure (traffic: null), never a stale constant."""
+    out = {}
+    try:
+        with open(TRAFFIC_FILE) as f:
+            for line in f:
+                cells = [c.strip().strip("`") for c in line.strip().strip("|").split("|")]
+                if len(cells) < 5 or cells[0] in ("workload", "") or set(cells[0]) <= set("-: "):
+                    continue
+                try:
+                    fetch, ffac, write, wfac = (float(c) for c in cells[1:5])
+                except ValueError:
+                    continue
+                out[cells[0]] = (fetch * ffac + write * wfac) * 1024.0
+    except OSError:
+        pass
+    return out
+
+
+MEASURED_TRAFFIC_BYTES = measured_traffic()
 
 
 def log(*a):
@@ -95,7 +113,7 @@ def time_plan(lib, api, plan, steps, warmup, warm_ms=0.0):
     return wall, api.profile_end()
 
 
-def bench_dense(make, steps, warmup, bound, mask_mode="descriptor", warm_ms=0.0):
+def bench_dense(make, steps, warmup, bound, mask_mode="descriptor", warm_ms=0.0, caller_path=False):
     from fblt_amd import api, runner
     lib = api.load()
     w = make()
@@ -112,6 +130,7 @@ def bench_dense(make, steps, warmup, bound, mask_mode="descriptor", warm_ms=0.0)
     wall_plain = time.perf_counter() - t0
     pct = step_percentiles(lib, api, lambda s_: lib.blt_attention_plan_run_hip(plan), min(steps, 256))
     lib.blt_attention_plan_destroy_hip(plan)
+    caller = bench_caller_path(w, d, steps, warmup) if caller_path else None
     d.close()
     launches = sum(v[0] for v in prof.values())
     kern_ms = sum(v[1] for v in prof.values())
@@ -130,8 +149,61 @@ def bench_dense(make, steps, warmup, bound, mask_mode="descriptor", warm_ms=0.0)
     }
     if warm_ms:
         res["warmup_ms"] = warm_ms
+    if caller:
+        res["reference_call_pattern"] = caller
     res["roofline"] = res["roofline_" + bound]
     return res, w
+
+
+def bench_caller_path(w, d, steps, warmup):
+    """The same workload the way an unmodified reference caller issues it on this library's ops
+    (csrc/models/attention.c:92-128, 197-202; cross_attention.c:70-96, 145-150): per sequence one
+    dense mask built on the device arena by blt_build_attention_mask, then one
+    blt_attention_head_core call per head with that mask and weights_out set.  Device time = the
+    launches' own durations summed; wall time includes this script's ctypes call overhead (a C
+    caller pays less per call)."""
+    import ctypes as C
+    import torch
+    from fblt_amd import abi, api
+    lib = api.load()
+    seqs = {}
+    for h in w.heads:
+        seqs.setdefault(h.seq, []).append(h)
+    scores = torch.empty(max(h.nq * h.nk for h in w.heads), dtype=torch.float32, device="cuda")
+    arena = lib.blt_arena_create(64 << 20, abi.BLT_BACKEND_HIP)
+    plan = []
+    for seq, heads in seqs.items():
+        cfg = d.mask_config(heads[0])
+        args = [d.head_args(h, "none", weights_ptr=scores.data_ptr()) for h in heads]
+        plan.append((cfg, args))
+    t = abi.BltTensor()
+
+    def one_pass():
+        for cfg, args in plan:
+            arena.contents.offset = 0
+            lib.blt_build_attention_mask(C.byref(cfg), C.byref(t), arena)
+            for a in args:
+                a.mask = t.data
+                lib.blt_attention_head_core(abi.BLT_BACKEND_HIP, C.byref(a))
+    n = max(5, steps // 10)
+    for _ in range(max(2, warmup // 4)):
+        one_pass()
+    lib.blt_backend_pass_sync_hip()
+    lib.blt_hip_profile_begin()
+    for _ in range(n):
+        one_pass()
+    prof = api.profile_end()
+    t0 = time.perf_counter()
+    for _ in range(n):
+        one_pass()
+    lib.blt_backend_pass_sync_hip()
+    wall = time.perf_counter() - t0
+    lib.blt_arena_destroy(arena)
+    return {"entry": "blt_build_attention_mask + one blt_attention_head_core per (sequence, head), dense mask, weights_out",
+            "launches_per_pass": sum(v[0] for v in prof.values()) / n,
+            "kernel_us_per_pass": sum(v[1] for v in prof.values()) * 1e3 / n,
+            "per_kernel_us": {k: v[1] * 1e3 / n for k, v in prof.items()},
+            "wall_us_per_pass": wall / n * 1e6, "tokens_per_s": w.tokens * n / wall}
 
 
 def bench_kv(kw, steps, warmup, warm_ms=0.0):
@@ -682,6 +754,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--only", default="", help="comma list of c1,c2,c3,c4,c5 (c2 always runs)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU budget of the headline workload")
+    ap.add_argument("--cpu-scale", type=float, default=1.0, help="scales the CPU budgets of the other workloads")
+    ap.add_argument("--detail", default=DETAIL_FILE, help="file the full per-workload records are written to")
     ap.add_argument("--probe-copy-mib", type=int, default=0,
                     help="only run the plain streaming copy of this many MiB --steps times (counter yardstick)")
     ap.add_argument("--probe-read-mib", default="",
@@ -699,39 +773,39 @@ def main():
     from fblt_amd import workloads
 
     if args.probe_copy_mib:
-        from fblt_amd import api
-        lib = api.load()
+        from fblt_amd import probes
+        lib = probes.load()
         nbytes = args.probe_copy_mib << 20
         src = torch.ones(nbytes // 4, dtype=torch.float32, device="cuda")
         dst = torch.empty_like(src)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(args.steps):
-            lib.blt_hip_stream_copy_probe(dst.data_ptr(), src.data_ptr(), nbytes)
-        lib.blt_backend_pass_sync_hip()
+            lib.blt_probe_stream_copy(dst.data_ptr(), src.data_ptr(), nbytes)
+        torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         print(json.dumps({"probe": "stream_copy", "bytes_in": nbytes, "bytes_out": nbytes, "launches": args.steps,
                           "GBps_read_plus_write": 2.0 * nbytes * args.steps / dt / 1e9}), flush=True)
         return
 
     if args.probe_read_mib:
-        from fblt_amd import api
-        lib = api.load()
+        from fblt_amd import probes
+        lib = probes.load()
         sizes = [int(x) for x in args.probe_read_mib.split(",") if x]
         buf = torch.ones((max(sizes) << 20) // 4, dtype=torch.float32, device="cuda")
         torch.cuda.synchronize()
         out = []
         for mib in sizes:
-            ms = lib.blt_hip_stream_read_probe(buf.data_ptr(), mib << 20, 10)
+            ms = lib.blt_probe_stream_read(buf.data_ptr(), mib << 20, 10)
             out.append({"MiB": mib, "us_per_launch": ms * 1e3, "GBps": (mib << 20) / ms / 1e6,
                         "frac_of_hbm_peak": (mib << 20) / ms / 1e6 / HBM_PEAK_GBS})
         print(json.dumps({"probe": "stream_read", "results": out}), flush=True)
         return
     if args.probe_issue:
-        from fblt_amd import api
-        lib = api.load()
+        from fblt_amd import probes
+        lib = probes.load()
         groups = 4000
-        ms = {m: min(lib.blt_hip_issue_probe(m, groups) for _ in range(3)) for m in (1, 2, 3)}
+        ms = {m: min(lib.blt_probe_issue(m, groups) for _ in range(3)) for m in (1, 2, 3)}
         tflops = 256 * 4 * groups * 8 * 4096 / (ms[1] * 1e-3) / 1e12   # one matrix wave per SIMD
         print(json.dumps({"probe": "issue", "groups": groups, "ms_matrix_only": ms[1], "ms_vector_only": ms[2],
                           "ms_both": ms[3], "both_over_sum": ms[3] / (ms[1] + ms[2]),
@@ -741,16 +815,16 @@ def main():
     only = set(x for x in args.only.split(",") if x)
     want = lambda c: not only or c in only
     K, W = args.steps, args.warmup
+    cs = args.cpu_scale
 
-    head, w2 = bench_dense(workloads.config2, K, W, "hbm")
+    head, w2 = bench_dense(workloads.config2, K, W, "hbm", caller_path=True)
     log("c2", json.dumps(head))
     others = {}
-    cpu = {}
     if want("c1"):
-        others["c1"], w1 = bench_dense(workloads.config1, K, W, "mfma")
+        others["c1"], w1 = bench_dense(workloads.config1, K, W, "mfma", caller_path=True)
         log("c1", json.dumps(others["c1"]))
     if want("c3"):
-        others["c3"], w3 = bench_dense(workloads.config3, K, W, "hbm")
+        others["c3"], w3 = bench_dense(workloads.config3, K, W, "hbm", caller_path=True)
         log("c3", json.dumps(others["c3"]))
     if want("c4"):
         others["c4"], k4 = bench_kv(workloads.config4(steps=W + 256, max_seq_len=512 + W + 256), 256, W)
@@ -776,13 +850,14 @@ def main():
                            ("c1_T4096", lambda: workloads.config1(batch=8, T=4096)),
                            ("c2_P2048", lambda: workloads.config2(batch=8, P=2048, T_bytes=8192))):
             others[name], _ = bench_dense(make, max(10, K // 10), 3, "mfma", warm_ms=100.0)
+            others[name]["roofline_hbm"]["traffic"] = None   # counters were read at the BASELINE sizes only
             log(name, json.dumps(others[name]))
 
         # decode and block verify with enough cached keys to leave the launch floor
         big = workloads.config4(batch=128, steps=3 + 20, len_lo=1024, len_hi=2048, max_seq_len=2048 + 32,
                                cache_period=8)
         others["c4_b128_L2048"], _ = bench_kv(big, 20, 3)
-        others["c4_b128_L2048"]["roofline_hbm"]["traffic"] = None   # counters were read at the BASELINE size only
+        others["c4_b128_L2048"]["roofline_hbm"]["traffic"] = None
         log("c4_b128_L2048", json.dumps(others["c4_b128_L2048"]))
         bigv = workloads.config5(batch=128, B=16, len_lo=1024, len_hi=2032, max_seq_len=2048, cache_period=8)
         others["c5_B16_b128_L2048"], _ = bench_kv(bigv, 20, 3, warm_ms=100.0)
@@ -803,21 +878,21 @@ def main():
         log("matmul", json.dumps(others["matmul_8192x512x1536"]))
         others["decode_layer"] = bench_decode_layer(K, W)
         if not args.no_cpu:
-            others["decode_layer"]["cpu_baseline"] = cpu_decode_layer(2.0)
+            others["decode_layer"]["cpu_baseline"] = cpu_decode_layer(2.0 * cs)
         log("decode_layer", json.dumps(others["decode_layer"]))
         others["decode_step"] = bench_decode_step(K, W)
         if not args.no_cpu:
-            others["decode_step"]["cpu_baseline"] = cpu_decode_step(2.0)
+            others["decode_step"]["cpu_baseline"] = cpu_decode_step(2.0 * cs)
         log("decode_step", json.dumps(others["decode_step"]))
         # the reference's own use of the step: one sequence, one new row per call
         others["decode_step_b1"] = bench_decode_step(K, W, batch=1)
         if not args.no_cpu:
-            others["decode_step_b1"]["cpu_baseline"] = cpu_decode_step(2.0, batch=1)
+            others["decode_step_b1"]["cpu_baseline"] = cpu_decode_step(2.0 * cs, batch=1)
         log("decode_step_b1", json.dumps(others["decode_step_b1"]))
         # a 512-byte prompt through the same entry point in one call (time to the first token)
         others["decode_step_prefill_512"] = bench_decode_step(max(10, K // 10), 3, batch=1, len_hi=1, n=512)
         if not args.no_cpu:
-            others["decode_step_prefill_512"]["cpu_baseline"] = cpu_decode_step(2.0, batch=1, len_hi=1, n=512)
+            others["decode_step_prefill_512"]["cpu_baseline"] = cpu_decode_step(2.0 * cs, batch=1, len_hi=1, n=512)
         log("decode_step_prefill_512", json.dumps(others["decode_step_prefill_512"]))
 
     # the dense-mask builders the callers still use
@@ -831,17 +906,70 @@ def main():
         cpu_head = cpu_dense(w2, args.cpu_seconds)
         log("cpu c2", json.dumps(cpu_head))
         if want("c1"):
-            others["c1"]["cpu_baseline"] = cpu_dense(w1, 2.0)
+            others["c1"]["cpu_baseline"] = cpu_dense(w1, 2.0 * cs)
         if want("c3"):
-            others["c3"]["cpu_baseline"] = cpu_dense(w3, 2.0)
+            others["c3"]["cpu_baseline"] = cpu_dense(w3, 2.0 * cs)
         if want("c4"):
-            others["c4"]["cpu_baseline"] = cpu_kv(workloads.config4(steps=64), 3.0, 64)
+            others["c4"]["cpu_baseline"] = cpu_kv(workloads.config4(steps=64), 3.0 * cs, 64)
         if want("c5"):
             for B in (4, 8, 16):
-                others["c5_B%d" % B]["cpu_baseline"] = cpu_kv(workloads.config5(B=B, steps=1), 1.0, 1)
-            others["c5_chunk_causal_n16"]["cpu_baseline"] = cpu_kv(_chunk_causal(workloads.config5(B=16, steps=1)), 1.0, 1)
+                others["c5_B%d" % B]["cpu_baseline"] = cpu_kv(workloads.config5(B=B, steps=1), 1.0 * cs, 1)
+            others["c5_chunk_causal_n16"]["cpu_baseline"] = cpu_kv(_chunk_causal(workloads.config5(B=16, steps=1)), 1.0 * cs, 1)
 
-    line = {
+    head["cpu_baseline"] = cpu_head
+    detail = dict(others)
+    detail["c2"] = head
+    detail_path = None
+    try:
+        os.makedirs(os.path.dirname(args.detail) or ".", exist_ok=True)
+        with open(args.detail, "w") as f:
+            json.dump({"steps": K, "warmup": W, "workloads": detail}, f, indent=1)
+        detail_path = os.path.relpath(args.detail, ROOT)
+    except OSError as e:
+        log("detail file not written:", e)
+    print(json.dumps(compact_line(head, others, cpu_head, K, W, detail_path)), flush=True)
+
+
+def _sig(x, digits=4):
+    """Floats cut to a few significant digits: the summary line stays short."""
+    if isinstance(x, float):
+        return float("%.*g" % (digits, x))
+    if isinstance(x, dict):
+        return {k: _sig(v, digits) for k, v in x.items()}
+    return x
+
+
+def compact_line(head, others, cpu_head, K, W, detail_path):
+    """The one JSON object printed last on stdout: headline figures in full precision, one short
+    summary row per attention shape (kernel, its device microseconds, fraction of the binding
+    roofline, the reference call pattern beside it, CPU figure)."""
+    def row(r):
+        if r is None:
+            return None
+        o = {"kernel": r["kernel"][:40], "launches": r["launches_per_step"], "kernel_us": r["kernel_us_avg"],
+             "bound": r["roofline"]["bound"], "frac": r["roofline"]["frac"],
+             "tokens_per_s": r["tokens_per_s"]}
+        if r.get("roofline_hbm", {}).get("traffic"):
+            o["traffic_x"] = r["roofline_hbm"]["traffic"] / r["bytes"]   # measured HBM bytes over algorithmic bytes
+        c = r.get("reference_call_pattern")
+        if c:
+            # the reference's call pattern on this library's ops: [launches, device us, wall us] per pass
+            o["caller"] = [c["launches_per_pass"], _sig(c["kernel_us_per_pass"]), _sig(c["wall_us_per_pass"])]
+        b = r.get("cpu_baseline")
+        if b:
+            o["cpu"] = [_sig(b["value"]), b["unit"]]
+        return _sig(o)
+    per = {"c2": row(head)}
+    for k in ("c1", "c3", "c4", "c4_rope", "c5_B4", "c5_B8", "c5_B16"):
+        if k in others:
+            per[k] = row(others[k])
+    # the same kernels away from the launch floor: [kernel us, binding roofline, fraction of it]
+    scaled = {k: [_sig(others[k]["kernel_us_avg"]), others[k]["roofline"]["bound"], _sig(others[k]["roofline"]["frac"])]
+              for k in ("c1_x64", "c2_x8", "c1_T4096", "c2_P2048", "c4_b128_L2048", "c5_B16_b128_L2048") if k in others}
+    # whole decoder step (all layers + LM head): [launches per step, device us, wall us]
+    steps_ = {k: [others[k]["launches_per_step"], _sig(others[k]["kernel_us_avg"]), _sig(others[k]["us_per_step"])]
+              for k in ("decode_step", "decode_step_b1") if k in others}
+    return {
         "metric": "attn_tokens_per_s", "value": head["tokens_per_s"], "unit": "tokens/s",
         "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": head["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
@@ -850,16 +978,19 @@ def main():
                    "entry": "blt_attention_plan_run_hip, causal descriptor, one launch per step",
                    "kernel": head["kernel"], "tokens_per_step": head["tokens_per_step"]},
         "kernel_us_avg": head["kernel_us_avg"],
-        "kernel_us_percentiles": head["kernel_us_percentiles"],
+        "kernel_us_p50": head["kernel_us_percentiles"]["p50"],
         "roofline": head["roofline"],
         "roofline_mfma": head["roofline_mfma"],
         "cpu_baseline": cpu_head,
+        "cpu_cores": cpu_head["cores"] if cpu_head else None,
         # the other parts of the composite headline metric (decode us/step, verify tokens/s), when they ran
         "decode_us_per_step": others["c4"]["us_per_step"] if "c4" in others else None,
         "verify_tokens_per_s": {k: others[k]["tokens_per_s"] for k in ("c5_B4", "c5_B8", "c5_B16") if k in others} or None,
-        "workloads": others,
+        "per_config": per,
+        "at_scale": scaled or None,
+        "decoder_step": steps_ or None,
+        "detail": detail_path,
     }
-    print(json.dumps(line), flush=True)
 
 
 if __name__ == "__main__":

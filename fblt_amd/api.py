@@ -169,9 +169,6 @@ SYMBOLS = {
     "blt_hip_graph_destroy": (None, [C.c_void_p]),
     "blt_hip_profile_begin": (None, []),
     "blt_hip_profile_end": (C.c_size_t, [C.POINTER(BltHipKernelTime), C.c_size_t]),
-    "blt_hip_stream_copy_probe": (None, [C.c_void_p, C.c_void_p, C.c_size_t]),
-    "blt_hip_stream_read_probe": (C.c_float, [C.c_void_p, C.c_size_t, C.c_int]),
-    "blt_hip_issue_probe": (C.c_float, [C.c_int, C.c_int]),
     "blt_hip_build_info": (C.c_char_p, []),
 }
 

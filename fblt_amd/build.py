@@ -1,4 +1,5 @@
-"""Builds fblt_amd/lib/libfblt_hip.so: host C99 (gcc) + gfx950 HIP (hipcc).
+"""Builds fblt_amd/lib/libfblt_hip.so: host C99 (gcc) + gfx950 HIP (hipcc); and the
+bench-only yardsticks fblt_amd/lib/libfblt_probes.so.
 
 `python -m fblt_amd.build` or `fblt_amd.build.build()`.  Objects go to
 fblt_amd/lib/obj; nothing is compiled at import time, and loading the library
@@ -15,8 +16,11 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(LIBDIR, "obj")
 LIB = os.path.join(LIBDIR, "libfblt_hip.so")
+# measurement yardsticks of bench.py's --probe-* modes: their own small library, not in the backend's ABI
+PROBES_SRC = os.path.join(HERE, "probes", "probes.hip")
+PROBES_LIB = os.path.join(LIBDIR, "libfblt_probes.so")
 
-HIP_SOURCES = ["memory.hip", "mask_builder.hip", "vecmath.hip", "attn_rows.hip", "attn_mfma.hip", "attn_wide.hip", "matmul.hip", "rope.hip", "mha.hip", "layer_ops.hip", "probes.hip", "stream.hip",
+HIP_SOURCES = ["memory.hip", "mask_builder.hip", "vecmath.hip", "attn_rows.hip", "attn_mfma.hip", "attn_wide.hip", "matmul.hip", "rope.hip", "mha.hip", "layer_ops.hip", "stream.hip",
                "attn_decode.hip", "attn_verify.hip", "attn_api.hip", "profile.hip"]
 C_SOURCES = ["host/blt_host.c"]
 
@@ -48,6 +52,7 @@ def build(verbose=False, jobs=8):
         obj = os.path.join(OBJDIR, os.path.basename(src) + ".o")
         objs.append(obj)
         steps.append(["gcc"] + C_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
+    steps.append([HIPCC] + HIP_FLAGS + ["-shared", PROBES_SRC, "-o", PROBES_LIB])
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         for out in ex.map(_run, steps):
             if verbose and out.strip():

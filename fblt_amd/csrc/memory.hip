@@ -94,20 +94,4 @@ extern "C" void blt_backend_pass_sync_hip(void) {
     if (e != hipSuccess) BLT_FATAL("blt_backend_pass_sync: %s", hipGetErrorString(e));
 }
 
-/* Plain streaming copy, 16 bytes per thread and step: the yardstick the
- * hardware-counter readings of the attention kernels are scaled by (it moves
- * exactly `bytes` in and `bytes` out). */
-__global__ __launch_bounds__(256) void stream_copy_kernel(float4 *__restrict__ dst, const float4 *__restrict__ src,
-                                                          size_t n16) {
-    for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256u) dst[i] = src[i];
-}
-
-extern "C" void blt_hip_stream_copy_probe(void *dst, const void *src, size_t bytes) {
-    BLT_REQUIRE(dst != NULL && src != NULL && bytes % 16 == 0, "blt_hip_stream_copy_probe: need 16-byte multiples");
-    if (bytes == 0) return;
-    hipLaunchKernelGGL(stream_copy_kernel, dim3(2048), dim3(256), 0, blt_stream(), static_cast<float4 *>(dst),
-                       static_cast<const float4 *>(src), bytes / 16);
-    HIP_CHECK_LAUNCH("blt_hip_stream_copy_probe");
-}
-
 extern "C" const char *blt_hip_build_info(void) { return "fblt_amd attention backend; kernels: gfx950"; }

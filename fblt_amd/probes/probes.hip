@@ -1,8 +1,12 @@
 /*
- * Hardware yardsticks the kernel designs and the reported rooflines lean on,
- * callable through the C-ABI so that the figures can be re-measured with the
- * shipped library (bench.py --probe-read-mib / --probe-issue):
+ * Hardware yardsticks the kernel designs and the reported rooflines lean on.
+ * They are measurement helpers, not part of the attention backend: they build
+ * into their own small library (libfblt_probes.so) that only bench.py's
+ * --probe-* modes load, so that the figures can be re-measured:
  *
+ *  - a plain streaming COPY of a buffer (the yardstick hardware-counter
+ *    readings of the attention kernels are scaled by: it moves exactly
+ *    `bytes` in and `bytes` out);
  *  - a plain streaming READ of a buffer (what a purely bandwidth-bound kernel
  *    attains on this part, against the published HBM peak);
  *  - an issue probe: wavefronts that run only v_mfma_f32_32x32x2_f32, only
@@ -11,15 +15,21 @@
  *    different waves overlap on a SIMD (they do not on gfx950: the mixed run
  *    takes the sum of the two separate times).
  */
-#include "blt_hip.h"
 #include "blt_fatal.h"
 #include "hip_check.h"
+
+#include <stddef.h>
 
 #include <stdint.h>
 
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(256) void stream_copy_kernel(float4 *__restrict__ dst, const float4 *__restrict__ src,
+                                                          size_t n16) {
+    for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256u) dst[i] = src[i];
+}
 
 __global__ __launch_bounds__(256) void stream_read_kernel(const float4 *__restrict__ src, size_t n16,
                                                           float *__restrict__ sink) {
@@ -84,9 +94,20 @@ float timed_ms(hipEvent_t e0, hipEvent_t e1) {
 
 } // namespace
 
-extern "C" float blt_hip_stream_read_probe(const void *src, size_t bytes, int launches) {
+/* Plain device-to-device streaming copy of `bytes` (a multiple of 16) on the null stream. */
+extern "C" void blt_probe_stream_copy(void *dst, const void *src, size_t bytes) {
+    BLT_REQUIRE(dst != NULL && src != NULL && bytes % 16 == 0, "blt_probe_stream_copy: need 16-byte multiples");
+    if (bytes == 0) return;
+    hipLaunchKernelGGL(stream_copy_kernel, dim3(2048), dim3(256), 0, 0, static_cast<float4 *>(dst),
+                       static_cast<const float4 *>(src), bytes / 16);
+    HIP_CHECK_LAUNCH("blt_probe_stream_copy");
+}
+
+/* Plain streaming read of `bytes` device bytes, `launches` times back to back after one warm-up;
+ * returns milliseconds per launch (HIP events). */
+extern "C" float blt_probe_stream_read(const void *src, size_t bytes, int launches) {
     BLT_REQUIRE(src != NULL && bytes % 16 == 0 && bytes > 0 && launches >= 1,
-                "blt_hip_stream_read_probe: need a buffer of 16-byte multiples");
+                "blt_probe_stream_read: need a buffer of 16-byte multiples");
     float *sink = nullptr;
     HIP_CHECK(hipMalloc((void **)&sink, 64));
     hipEvent_t e0, e1;
@@ -106,8 +127,11 @@ extern "C" float blt_hip_stream_read_probe(const void *src, size_t bytes, int la
     return ms / launches;
 }
 
-extern "C" float blt_hip_issue_probe(int mode, int groups) {
-    BLT_REQUIRE(mode >= 1 && mode <= 3 && groups >= 1, "blt_hip_issue_probe: mode is 1 (matrix), 2 (vector) or 3 (both)");
+/* One launch of 256 workgroups of 8 waves (2 per SIMD) in which one wave per SIMD runs `groups` x 8
+ * v_mfma_f32_32x32x2_f32 (mode & 1) and / or the other runs `groups` x 64 v_fma_f32 (mode & 2).
+ * Returns the launch's milliseconds: mode 3 ~ mode 1 + mode 2 means the two do not overlap. */
+extern "C" float blt_probe_issue(int mode, int groups) {
+    BLT_REQUIRE(mode >= 1 && mode <= 3 && groups >= 1, "blt_probe_issue: mode is 1 (matrix), 2 (vector) or 3 (both)");
     float *sink = nullptr;
     HIP_CHECK(hipMalloc((void **)&sink, 256u * 512u * sizeof(float)));
     hipEvent_t e0, e1;

@@ -59,6 +59,32 @@ class DeviceWorkload:
             self.lib.blt_arena_destroy(self.arena)
             self.arena = None
 
+    def mask_config(self, h):
+        """The blt_mask_config a reference caller would fill for head h's sequence (index arrays
+        on the host, as the reference passes them): causal (+ offset, window) for the
+        self-attention blocks (csrc/models/local_common.c:110, global_transformer.c:19-28), patch
+        groups for the cross block (csrc/models/local_encoder.c:56-74)."""
+        cfg = abi.BltMaskConfig()
+        cfg.seq_len_q, cfg.seq_len_kv = h.nq, h.nk
+        if h.mask == "causal":
+            cfg.is_causal = True
+            cfg.causal_offset = h.causal_offset
+            cfg.sliding_window = h.window
+        elif h.mask == "range":
+            lo_name, hi_name, off = h.mask_ref
+            lo = self.w.ranges[lo_name][off:off + h.nq]
+            hi = self.w.ranges[hi_name][off:off + h.nq]
+            kv = np.full(h.nk, h.nq, dtype=np.uint64)
+            for i in range(h.nq):
+                kv[lo[i]:hi[i]] = i
+            qg, kg = abi.size_array(range(h.nq)), abi.size_array(kv)
+            self._keep += [qg, kg]
+            cfg.query_group_ids, cfg.kv_group_ids = qg, kg
+            cfg.bidirectional_within_group = True
+        else:
+            raise ValueError(h.mask)
+        return cfg
+
     def dense_mask_ptr(self, h):
         """Device address of the dense additive mask of head h, built by the
         device mask builder in the arena (the reference's flow)."""
@@ -72,23 +98,7 @@ class DeviceWorkload:
             raise ValueError(h.mask)
         if key in self._mask_cache:
             return self._mask_cache[key]
-        cfg = abi.BltMaskConfig()
-        cfg.seq_len_q, cfg.seq_len_kv = h.nq, h.nk
-        if h.mask == "causal":
-            cfg.is_causal = True
-            cfg.causal_offset = h.causal_offset
-            cfg.sliding_window = h.window
-        else:
-            lo_name, hi_name, off = h.mask_ref
-            lo = self.w.ranges[lo_name][off:off + h.nq]
-            hi = self.w.ranges[hi_name][off:off + h.nq]
-            kv = np.full(h.nk, h.nq, dtype=np.uint64)
-            for i in range(h.nq):
-                kv[lo[i]:hi[i]] = i
-            qg, kg = abi.size_array(range(h.nq)), abi.size_array(kv)
-            self._keep += [qg, kg]
-            cfg.query_group_ids, cfg.kv_group_ids = qg, kg
-            cfg.bidirectional_within_group = True
+        cfg = self.mask_config(h)
         t = abi.BltTensor()
         self.lib.blt_build_attention_mask_hip(C.byref(cfg), C.byref(t), self._arena())
         self._mask_cache[key] = t.data

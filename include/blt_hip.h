@@ -404,20 +404,6 @@ typedef struct {
 void blt_hip_profile_begin(void);
 size_t blt_hip_profile_end(blt_hip_kernel_time *out, size_t capacity);
 
-/* Measurement yardstick: a plain device-to-device streaming copy of `bytes`
- * (a multiple of 16) on the default stream.  Hardware-counter readings of the
- * attention kernels are scaled by what the same counters read for this copy. */
-void blt_hip_stream_copy_probe(void *dst, const void *src, size_t bytes);
-/* Plain streaming read of `bytes` device bytes, `launches` times back to back
- * after one warm-up; returns milliseconds per launch (HIP events).  What a
- * purely bandwidth-bound read attains on the device. */
-float blt_hip_stream_read_probe(const void *src, size_t bytes, int launches);
-/* Issue probe: one launch of 256 workgroups of 8 waves (2 per SIMD) in which
- * one wave per SIMD runs `groups` x 8 v_mfma_f32_32x32x2_f32 (mode & 1) and /
- * or the other runs `groups` x 64 v_fma_f32 (mode & 2).  Returns the launch's
- * milliseconds: mode 3 ~ mode 1 + mode 2 means the two do not overlap. */
-float blt_hip_issue_probe(int mode, int groups);
-
 /* Library build tag and the architecture its kernels were compiled for. */
 const char *blt_hip_build_info(void);
 
