@@ -13,6 +13,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <vector>
 
 namespace {
@@ -317,8 +318,9 @@ void plan_launch(const blt_attention_plan &pl, const AttnProb *dev, const AttnTi
 /* Staging for one-shot batches: descriptors go host vector -> pinned buffer ->
  * device buffer with a truly asynchronous copy on the library's stream.  The
  * device buffer can be reused by the next call because that call's copy is
- * ordered behind this call's kernels; the pinned side is the calling thread's
- * ring of buffers (blt_upload_staged). */
+ * ordered behind this call's kernels -- which holds per stream, so there is
+ * one staging buffer per (host thread, stream); the pinned side is the calling
+ * thread's ring of buffers (blt_upload_staged). */
 struct Staging {
     blt_attention_plan plan;
     void *device = nullptr;
@@ -351,8 +353,8 @@ struct Staging {
 };
 
 Staging &staging() {
-    static thread_local Staging st;
-    return st;
+    static thread_local std::map<hipStream_t, Staging> by_stream;
+    return by_stream[blt_stream_key()];
 }
 
 } // namespace

@@ -30,8 +30,12 @@
 #include "launch.h"
 
 #include <algorithm>
+#include <atomic>
 #include <cstdlib>
 #include <cstring>
+#include <map>
+#include <mutex>
+#include <vector>
 
 namespace {
 
@@ -69,6 +73,7 @@ __global__ __launch_bounds__(64 * WAVES) void kv_step_kernel(StepArgs a) {
 
     const uint32_t len = a.self_len[b] + a.len_bias;
     const uint32_t nk = len + a.n;
+    if (kv_over_capacity(a, nk)) return; /* uniform over the sequence's workgroups */
     const size_t slab = (size_t)b * a.max_seq_len;
     const uint32_t col = (head_ok ? head : 0u) * HD + 4u * g;
     const uint32_t span = kv_span_of(a, nk);
@@ -301,7 +306,18 @@ __global__ __launch_bounds__(64 * WAVES) void kv_step_kernel(StepArgs a) {
     kv_finish_sequence<HD>(a, (uint32_t)NQ, b, nk, &sm_ticket, early_ticket);
 }
 
-/* scratch the family owns: per-split softmax states and per-sequence tickets */
+/* ---- device memory the family owns beyond inputs and outputs ----
+ * per-split softmax records [batch][splits][heads][slots][hd + 2], per-sequence tickets [batch]
+ * and one sticky error word.
+ *
+ * Growing entry points (blt_kv_attend_step_hip and everything built on it): one set per (host
+ * thread, stream), so that steps issued on two streams never share tickets or records.  The
+ * buffers only grow, and a buffer that is replaced by a larger one is kept until the process
+ * ends: a graph captured earlier holds the old addresses in its kernel arguments and must stay
+ * replayable.
+ *
+ * blt_kv_attend_step_noalloc_hip: the same records and tickets in a file-scope device array of
+ * fixed size (`scratch`), one copy per GPU, whose address is looked up once per device. */
 struct Scratch {
     float *partial = nullptr;
     size_t partial_floats = 0;
@@ -309,9 +325,55 @@ struct Scratch {
     size_t ticket_count = 0;
 };
 
-Scratch &scratch() {
-    static thread_local Scratch s;
-    return s;
+constexpr size_t STATIC_PARTIAL_FLOATS = (size_t)1 << 20; /* 4 MiB of per-split records            */
+constexpr size_t STATIC_TICKETS = 4096;                   /* sequences per call                     */
+constexpr size_t STATIC_WORDS = 64;                       /* error word + padding to 256 bytes      */
+constexpr size_t STATIC_BYTES = STATIC_PARTIAL_FLOATS * sizeof(float) + STATIC_TICKETS * sizeof(uint32_t) +
+                                STATIC_WORDS * sizeof(uint32_t);
+static __device__ __align__(256) unsigned char scratch[STATIC_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+struct DeviceStatics {
+    unsigned char *base = nullptr; /* device address of `scratch` on this GPU */
+    float *partial() const { return reinterpret_cast<float *>(base); }
+    uint32_t *tickets() const { return reinterpret_cast<uint32_t *>(base + STATIC_PARTIAL_FLOATS * sizeof(float)); }
+    uint32_t *error() const { return tickets() + STATIC_TICKETS; }
+};
+DeviceStatics g_statics[MAX_DEVICES];
+std::mutex g_statics_lock;
+std::atomic<uint32_t> g_unchecked_steps{0}; /* device-length steps issued since the error word was last read */
+
+/* The current device's copy of `scratch`: looked up on the first call on that device (each GPU
+ * holds its own copy at its own address).  The array is zero when the code object is loaded and
+ * every launch leaves tickets and error word as it found them, so nothing has to be cleared. */
+const DeviceStatics &statics() {
+    int dev = 0;
+    HIP_CHECK(hipGetDevice(&dev));
+    BLT_REQUIRE(dev >= 0 && dev < MAX_DEVICES, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> hold(g_statics_lock);
+    if (!g_statics[dev].base) {
+        void *ptr = nullptr;
+        HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        BLT_REQUIRE(ptr != nullptr, "hipGetSymbolAddress returned no address for the KV step scratch");
+        g_statics[dev].base = static_cast<unsigned char *>(ptr);
+    }
+    return g_statics[dev];
+}
+
+struct GrowingScratch {
+    std::map<hipStream_t, Scratch> by_stream;
+    std::vector<void *> retired; /* replaced by larger buffers; live graphs may still name them */
+};
+
+GrowingScratch &growing() {
+    static thread_local GrowingScratch g;
+    return g;
+}
+
+/* tickets must start at zero; a fill kernel, not a memset node, so that a capture could hold it */
+__global__ void kv_clear_words_kernel(uint32_t *p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
 }
 
 template <int G, int NQ, int WAVES>
@@ -360,12 +422,13 @@ namespace {
  * n_seq rows per sequence, the row pointers already advanced to row0. */
 void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride, const float *k_rows,
                    size_t k_stride, const float *v_rows, size_t v_stride, const float *rope_cos,
-                   const float *rope_sin, float *combined, size_t combined_stride, size_t n, size_t n_seq,
-                   size_t row0, int step_kind, int commit, size_t max_len_hint);
+                   const float *rope_sin, size_t rope_positions, float *combined, size_t combined_stride, size_t n,
+                   size_t n_seq, size_t row0, int step_kind, int commit, size_t max_len_hint, bool static_scratch);
 
 void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride, const float *k_rows,
                  size_t k_stride, const float *v_rows, size_t v_stride, const float *rope_cos, const float *rope_sin,
-                 float *combined, size_t combined_stride, size_t n, int step_kind, int commit, size_t max_len_hint) {
+                 size_t rope_positions, float *combined, size_t combined_stride, size_t n, int step_kind, int commit,
+                 size_t max_len_hint, bool static_scratch) {
     BLT_REQUIRE(q_rows != NULL && k_rows != NULL && v_rows != NULL && combined != NULL,
                 "blt_kv_attend_step: row buffers must not be NULL");
     BLT_REQUIRE(n >= 1, "blt_kv_attend_step: need at least one row");
@@ -382,16 +445,57 @@ void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_s
         const size_t rows = std::min<size_t>(32, n - row0);
         const bool last = row0 + rows == n;
         kv_step_slice(cache, q_rows + row0 * q_stride, q_stride, k_rows + row0 * k_stride, k_stride,
-                      v_rows + row0 * v_stride, v_stride, rope_cos, rope_sin, combined + row0 * combined_stride,
-                      combined_stride, rows, n, row0, step_kind, last ? commit : 0,
-                      max_len_hint - (n - row0 - rows));
+                      v_rows + row0 * v_stride, v_stride, rope_cos, rope_sin, rope_positions,
+                      combined + row0 * combined_stride, combined_stride, rows, n, row0, step_kind, last ? commit : 0,
+                      max_len_hint - (n - row0 - rows), static_scratch);
     }
+    g_unchecked_steps.fetch_add(1, std::memory_order_relaxed);
+}
+
+/* Query capacity of the per-split record layout a launch of `nq` rows uses: the VALU kernel's
+ * row template, 32 for the matrix-core kernels. */
+uint32_t valu_slots(uint32_t nq) { return nq <= 1 ? 1u : nq <= 2 ? 2u : nq <= 4 ? 4u : nq <= 8 ? 8u : 16u; }
+
+/* Records and tickets for a launch set that needs `floats` floats of per-split records and
+ * `batch` tickets, from the fixed device array or from the growing per-stream buffers. */
+void acquire_scratch(StepArgs &a, size_t floats, size_t batch, bool static_scratch) {
+    const DeviceStatics &st = statics();
+    a.error = st.error();
+    if (static_scratch) {
+        BLT_REQUIRE(floats <= STATIC_PARTIAL_FLOATS && batch <= STATIC_TICKETS,
+                    "blt_kv_attend_step_noalloc: this step needs %zu bytes of per-split records for %zu sequences; "
+                    "the fixed scratch holds %zu bytes and %zu sequences (use blt_kv_attend_step_hip, which "
+                    "allocates, or a smaller batch)",
+                    floats * sizeof(float), batch, STATIC_PARTIAL_FLOATS * sizeof(float), STATIC_TICKETS);
+        a.partial = st.partial();
+        a.tickets = st.tickets();
+        return;
+    }
+    GrowingScratch &g = growing();
+    Scratch &sc = g.by_stream[blt_stream_key()];
+    BLT_REQUIRE(!blt_stream_capturing() || (floats <= sc.partial_floats && batch <= sc.ticket_count),
+                "blt_kv_attend_step: the step would allocate its scratch while a graph capture is open; run it once "
+                "eagerly with this batch size on this stream first");
+    if (floats > sc.partial_floats) {
+        if (sc.partial) g.retired.push_back(sc.partial);
+        sc.partial_floats = std::max(floats, 2 * sc.partial_floats);
+        HIP_CHECK(hipMalloc((void **)&sc.partial, sc.partial_floats * sizeof(float)));
+    }
+    if (batch > sc.ticket_count) {
+        if (sc.tickets) g.retired.push_back(sc.tickets);
+        sc.ticket_count = std::max<size_t>(2 * batch, 1024);
+        HIP_CHECK(hipMalloc((void **)&sc.tickets, sc.ticket_count * sizeof(uint32_t)));
+        hipLaunchKernelGGL(kv_clear_words_kernel, dim3((unsigned)((sc.ticket_count + 255) / 256)), dim3(256), 0,
+                           blt_stream(), sc.tickets, sc.ticket_count);
+    }
+    a.partial = sc.partial;
+    a.tickets = sc.tickets;
 }
 
 void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride, const float *k_rows,
                    size_t k_stride, const float *v_rows, size_t v_stride, const float *rope_cos,
-                   const float *rope_sin, float *combined, size_t combined_stride, size_t n, size_t n_seq,
-                   size_t row0, int step_kind, int commit, size_t max_len_hint) {
+                   const float *rope_sin, size_t rope_positions, float *combined, size_t combined_stride, size_t n,
+                   size_t n_seq, size_t row0, int step_kind, int commit, size_t max_len_hint, bool static_scratch) {
     BLT_REQUIRE(cache != NULL && cache->self_k != NULL && cache->self_v != NULL && cache->self_len != NULL,
                 "blt_kv_attend_step: cache buffers must not be NULL");
     const size_t E = cache->embed_dim, H = cache->num_heads;
@@ -460,31 +564,6 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
         a.span = (uint32_t)(subs * SUB);
     }
 
-    Scratch &sc = scratch();
-    const size_t need = cache->batch * (size_t)MAX_SPLITS * H * 32u * (hd + 2); /* 32 = widest query block */
-    BLT_REQUIRE(!blt_stream_capturing() || (need <= sc.partial_floats && cache->batch <= sc.ticket_count),
-                "blt_kv_attend_step: the step would allocate its scratch while a graph capture is open; run it once "
-                "eagerly with this batch size first");
-    if (need > sc.partial_floats) {
-        if (sc.partial) {
-            HIP_CHECK(hipDeviceSynchronize());
-            HIP_CHECK(hipFree(sc.partial));
-        }
-        sc.partial_floats = need;
-        HIP_CHECK(hipMalloc((void **)&sc.partial, need * sizeof(float)));
-    }
-    if (cache->batch > sc.ticket_count) {
-        if (sc.tickets) {
-            HIP_CHECK(hipDeviceSynchronize());
-            HIP_CHECK(hipFree(sc.tickets));
-        }
-        sc.ticket_count = std::max<size_t>(cache->batch, 1024);
-        HIP_CHECK(hipMalloc((void **)&sc.tickets, sc.ticket_count * sizeof(uint32_t)));
-        HIP_CHECK(hipMemsetAsync(sc.tickets, 0, sc.ticket_count * sizeof(uint32_t), blt_stream()));
-    }
-    a.partial = sc.partial;
-    a.tickets = sc.tickets;
-
     /* Blocks of two or more rows go to the matrix-core kernels (one launch for
      * up to 32 rows; the cost does not depend on the row count: measured 9.5 us
      * at 64 sequences for 2 ... 16 rows against 9.9 / 14.6 us for 2 / 3 rows on
@@ -498,7 +577,8 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
         return e && strcmp(e, "valu") == 0 ? 1 : e && strcmp(e, "mfma") == 0 ? 2 : 0;
     }();
     const bool want_mfma = pinned == 2 || (pinned == 0 && a.n >= 2u);
-    if (want_mfma && (hd == 32 || hd == 64)) {
+    const bool mfma = want_mfma && (hd == 32 || hd == 64);
+    if (mfma) {
         /* the block kernel merges slices inside the workgroup, so it wants few,
          * long spans: just enough workgroups to cover the compute units */
         a.hpb = kv_block_heads_per_group((uint32_t)cache->batch, (uint32_t)subs, (uint32_t)H);
@@ -515,6 +595,16 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
         const size_t bspan = (subs + bs - 1) / bs;
         a.splits = (uint32_t)((subs + bspan - 1) / bspan);
         a.span = (uint32_t)(bspan * SUB);
+    }
+    /* what a sequence may attend at most: beyond it the kernels leave the sequence alone and raise
+     * the error word (lengths are device data; the hint is all the host knows) */
+    a.cap = (uint32_t)std::min<size_t>({(size_t)a.splits * a.span, (size_t)cache->max_seq_len,
+                                        rope_cos ? rope_positions : (size_t)UINT32_MAX});
+    const uint32_t slots = mfma ? 32u : valu_slots((uint32_t)std::min<size_t>(16, n));
+    acquire_scratch(a, a.splits > 1u ? cache->batch * (size_t)a.splits * H * slots * (hd + 2) : 0, cache->batch,
+                    static_scratch);
+
+    if (mfma) {
         a.q0 = 0;
         a.write_through = 1;
         a.commit = commit;
@@ -541,12 +631,23 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
 
 } // namespace
 
+/* Reads the sticky device error word when a device-length step was issued since the last look;
+ * called by the library's synchronising entry points after their wait. */
+void blt_kv_check_device_errors() {
+    if (g_unchecked_steps.exchange(0, std::memory_order_relaxed) == 0) return;
+    uint32_t word = 0;
+    HIP_CHECK(hipMemcpy(&word, statics().error(), sizeof(word), hipMemcpyDeviceToHost));
+    if (word & KV_ERR_CAPACITY)
+        BLT_FATAL("blt_kv_attend_step: exceeds cache capacity (on the device a sequence's length plus its new rows "
+                  "went past max_len_hint, max_seq_len or the rotation tables; that sequence was left untouched)");
+}
+
 extern "C" void blt_kv_attend_step_hip(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride,
                                        const float *k_rows, size_t k_stride, const float *v_rows, size_t v_stride,
                                        float *combined, size_t combined_stride, size_t n, int step_kind, int commit,
                                        size_t max_len_hint) {
-    kv_step_run(cache, q_rows, q_stride, k_rows, k_stride, v_rows, v_stride, nullptr, nullptr, combined,
-                combined_stride, n, step_kind, commit, max_len_hint);
+    kv_step_run(cache, q_rows, q_stride, k_rows, k_stride, v_rows, v_stride, nullptr, nullptr, 0, combined,
+                combined_stride, n, step_kind, commit, max_len_hint, false);
 }
 
 extern "C" void blt_kv_rope_attend_step_hip(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride,
@@ -560,6 +661,6 @@ extern "C" void blt_kv_rope_attend_step_hip(const blt_kv_attn_cache *cache, cons
     BLT_REQUIRE(max_len_hint <= rope_positions,
                 "blt_kv_rope_attend_step: positions up to %zu exceed the rotation tables (%zu rows)", max_len_hint,
                 rope_positions);
-    kv_step_run(cache, q_rows, q_stride, k_rows, k_stride, v_rows, v_stride, rope_cos, rope_sin, combined,
-                combined_stride, n, step_kind, commit, max_len_hint);
+    kv_step_run(cache, q_rows, q_stride, k_rows, k_stride, v_rows, v_stride, rope_cos, rope_sin, rope_positions,
+                combined, combined_stride, n, step_kind, commit, max_len_hint, false);
 }

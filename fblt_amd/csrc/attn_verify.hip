@@ -69,6 +69,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block_mfma_kernel(StepArgs a
 
     const uint32_t len = a.self_len[b] + a.len_bias;
     const uint32_t nk = len + a.n;
+    if (kv_over_capacity(a, nk)) return; /* uniform over the sequence's workgroups */
     const size_t slab = (size_t)b * a.max_seq_len;
     const uint32_t span = kv_span_of(a, nk);
     const uint32_t k_begin = split * span;
@@ -372,6 +373,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block16_mfma_kernel(StepArgs
 
     const uint32_t len = a.self_len[b] + a.len_bias;
     const uint32_t nk = len + a.n;
+    if (kv_over_capacity(a, nk)) return; /* uniform over the sequence's workgroups */
     const size_t slab = (size_t)b * a.max_seq_len;
     const uint32_t span = kv_span_of(a, nk);
     const uint32_t k_begin = split * span;

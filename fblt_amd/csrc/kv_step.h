@@ -25,6 +25,7 @@ struct StepArgs {
     const float *rope_sin;
     float *partial;    /* [batch][splits][heads][NQ][hd + 2] */
     uint32_t *tickets; /* [batch] */
+    uint32_t *error;   /* sticky device word: KV_ERR_* bits, read back by the host at its next synchronisation */
     uint32_t q_stride, k_stride, v_stride, out_stride;
     uint32_t max_seq_len, embed_dim, num_heads;
     uint32_t window;
@@ -36,6 +37,8 @@ struct StepArgs {
     uint32_t q0;       /* first query row this launch handles */
     uint32_t splits;   /* gridDim.x */
     uint32_t span;     /* keys per split, a multiple of SUB */
+    uint32_t cap;      /* most keys (cached + new) a sequence may attend in this launch: what the slab, the
+                          launch's splits * span and the rotation tables all hold */
     uint32_t hpb;      /* heads per workgroup */
     uint32_t slices;   /* waves per head in a workgroup */
     float scale;
@@ -44,6 +47,21 @@ struct StepArgs {
     int commit;        /* advance self_len when the sequence is done */
 };
 
+
+/* The lengths live in device memory and the launch was sized from a host-side hint.  A sequence
+ * whose length + new rows went past what the launch, its slab or the rotation tables hold must
+ * neither drop keys silently nor store past its slab: every workgroup of such a sequence leaves
+ * before its first load -- no write-through, no output rows, no ticket, no commit -- and one of them
+ * raises a sticky error bit that the host turns into the reference's "exceeds cache capacity" fatal
+ * error (csrc/infer/kv_cache.c:191) at its next synchronisation.  The condition depends on the
+ * sequence only, so all workgroups of the sequence agree and the ticket stays armed. */
+constexpr uint32_t KV_ERR_CAPACITY = 1u;
+__device__ __forceinline__ bool kv_over_capacity(const StepArgs &a, uint32_t nk) {
+    if (nk <= a.cap) return false;
+    if (threadIdx.x == 0 && blockIdx.x == 0 && blockIdx.z == 0)
+        __hip_atomic_fetch_or(a.error, KV_ERR_CAPACITY, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return true;
+}
 
 /* Keys per split for a sequence that attends nk keys: the sequence's own
  * sub-chunks divided evenly over the launch's splits, so that every workgroup

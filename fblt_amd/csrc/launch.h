@@ -18,10 +18,18 @@ bool blt_profile_is_open();
  * graph capture is open on it (stream.hip). */
 hipStream_t blt_stream();
 bool blt_stream_capturing();
+/* The stream library-owned scratch is keyed by: the current stream, or, while a capture is open,
+ * the stream the thread was on when it began (the one the graph will be replayed on). */
+hipStream_t blt_stream_key();
 /* Host-to-device copy that returns at once and lets the caller reuse `src`
  * right away: the bytes go through a small ring of pinned buffers owned by
  * the calling thread (memory.hip).  Not usable while a graph is captured. */
 void blt_upload_staged(void *dst, const void *src, size_t bytes);
+/* Turns a sticky error the KV step kernels raised on the device (a sequence outgrew what its
+ * launch, slab or rotation tables hold) into the fatal error; costs one 4-byte read-back, and
+ * only when such a step was issued since the last look.  Called after a host wait
+ * (attn_decode.hip). */
+void blt_kv_check_device_errors();
 /* A fresh (start, stop) event pair owned by the open profile, booked under `tag`. */
 void blt_profile_book(const char *tag, hipEvent_t *start, hipEvent_t *stop);
 

@@ -701,7 +701,11 @@ extern "C" void blt_matmul_hip(const blt_tensor *a, const blt_tensor *b, blt_ten
     BLT_REQUIRE(a->shape[1] == b->shape[0], "matmul inner dimensions do not match");
     BLT_REQUIRE(out->shape[0] == a->shape[0] && out->shape[1] == b->shape[1], "matmul output shape is incorrect");
     const size_t m = a->shape[0], k = a->shape[1], n = b->shape[1];
-    if (m == 0 || k == 0 || n == 0) return;
+    if (m == 0 || n == 0) return;
+    if (k == 0) { /* an empty sum: the product is all zeros (csrc/ops/linalg_cpu.c:8-18 stores sum = 0) */
+        blt_hip_memset(out->data, 0, m * n * sizeof(float));
+        return;
+    }
     BLT_REQUIRE(m <= 0x7FFFFFFFu && k <= 0x7FFFFFFFu && n <= 0x7FFFFFFFu, "matmul: dimensions exceed 2^31-1");
     MatmulArgs g;
     __builtin_memset(&g, 0, sizeof(g));

@@ -11,6 +11,9 @@
 #include "hip_check.h"
 #include "launch.h"
 
+#include <algorithm>
+#include <stdint.h>
+
 extern "C" void *blt_hip_malloc(size_t bytes) {
     void *p = nullptr;
     HIP_CHECK(hipMalloc(&p, bytes));
@@ -23,9 +26,39 @@ extern "C" void blt_hip_free(void *ptr) {
     if (e != hipSuccess) BLT_WARN("HIP hipFree failed: %s", hipGetErrorString(e));
 }
 
+namespace {
+
+/* Byte fill as a kernel: 16-byte stores over the aligned body, single bytes at the ragged ends. */
+__global__ __launch_bounds__(256) void fill_bytes_kernel(unsigned char *dst, unsigned int pattern, size_t head,
+                                                         size_t body16, size_t bytes) {
+    const size_t t = (size_t)blockIdx.x * 256u + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * 256u;
+    uint4 *body = reinterpret_cast<uint4 *>(dst + head);
+    for (size_t i = t; i < body16; i += stride) body[i] = make_uint4(pattern, pattern, pattern, pattern);
+    const size_t tail0 = head + 16u * body16;
+    for (size_t i = t; i < head; i += stride) dst[i] = (unsigned char)pattern;
+    for (size_t i = tail0 + t; i < bytes; i += stride) dst[i] = (unsigned char)pattern;
+}
+
+} // namespace
+
+/* While a graph is being captured the fill is a kernel node: memset nodes recorded into a graph
+ * have replayed wrongly on this platform, and blt_tensor_create (zero-filled tensors) reaches this
+ * from inside captured calls. */
 extern "C" void blt_hip_memset(void *dst, int value, size_t bytes) {
     if (bytes == 0) return;
-    HIP_CHECK(hipMemsetAsync(dst, value, bytes, blt_stream()));
+    if (!blt_stream_capturing()) {
+        HIP_CHECK(hipMemsetAsync(dst, value, bytes, blt_stream()));
+        return;
+    }
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(dst);
+    const size_t head = std::min<size_t>(bytes, (16u - (addr & 15u)) & 15u);
+    const size_t body16 = (bytes - head) / 16u;
+    const unsigned int b = (unsigned int)(value & 0xFF), pattern = b | (b << 8) | (b << 16) | (b << 24);
+    const unsigned blocks = (unsigned)std::min<size_t>(2048, std::max<size_t>(1, (body16 + 255) / 256));
+    hipLaunchKernelGGL(fill_bytes_kernel, dim3(blocks), dim3(256), 0, blt_stream(), static_cast<unsigned char *>(dst),
+                       pattern, head, body16, bytes);
+    HIP_CHECK_LAUNCH("blt_hip_memset");
 }
 
 
@@ -86,12 +119,14 @@ extern "C" void blt_hip_memcpy_d2h(void *dst, const void *src, size_t bytes) {
     /* the copy waits for the library's current stream, whichever it is */
     HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, blt_stream()));
     HIP_CHECK(hipStreamSynchronize(blt_stream()));
+    blt_kv_check_device_errors();
 }
 
 extern "C" void blt_backend_pass_sync_hip(void) {
     hipError_t e = hipGetLastError();
     if (e == hipSuccess) e = hipDeviceSynchronize();
     if (e != hipSuccess) BLT_FATAL("blt_backend_pass_sync: %s", hipGetErrorString(e));
+    blt_kv_check_device_errors();
 }
 
 extern "C" const char *blt_hip_build_info(void) { return "fblt_amd attention backend; kernels: gfx950"; }

@@ -35,6 +35,7 @@ struct blt_hip_graph {
 };
 
 hipStream_t blt_stream() { return t_stream; }
+hipStream_t blt_stream_key() { return t_capturing ? t_saved : t_stream; }
 bool blt_stream_capturing() { return t_capturing; }
 
 extern "C" void blt_hip_set_stream(void *stream) {

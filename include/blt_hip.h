@@ -304,7 +304,13 @@ enum {
  * v_rows and combined are [batch*n, *] with the given row strides (elements);
  * K rows are already rotated.  max_len_hint >= max_b(self_len[b]) + n sizes
  * the launch (the host knows it, as the reference's host-side self_len does);
- * sequences shorter than the hint simply leave blocks idle.  A causal step
+ * sequences shorter than the hint simply leave blocks idle.  A sequence whose
+ * device-side length + n exceeds the hint (rounded up to the launch's span),
+ * max_seq_len or the rotation tables is left untouched -- no write-through, no
+ * output rows, no commit -- and the next synchronising call of the library
+ * (blt_backend_pass_sync_hip, blt_hip_memcpy_d2h, blt_tensor_download) ends
+ * with "exceeds cache capacity", the reference's check of csrc/infer/
+ * kv_cache.c:191 made where the lengths live.  A causal step
  * of more than 32 rows per sequence (a prompt prefill) is run as consecutive
  * 32-row slices; a block step takes at most 32 rows (the reference's
  * BLT_BLOCKGEN_MAX_B, csrc/infer/block_generation.c:154). */

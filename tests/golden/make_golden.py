@@ -38,6 +38,7 @@ DENSE_CASES = {
 }
 KV_CASES = {
     "c4_full_8steps": lambda: workloads.config4(steps=8),
+    "c4_full_256steps": lambda: workloads.config4(),   # BASELINE config 4 as stated: 64 sequences, 256 consecutive steps
     "c4_small": lambda: workloads.config4(batch=3, steps=5, len_hi=70),
     "c5_B4": lambda: workloads.config5(B=4),
     "c5_B8": lambda: workloads.config5(B=8),

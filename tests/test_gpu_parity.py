@@ -10,6 +10,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
+from tests import lse_check
 from fblt_amd import abi, api, workloads
 from oracle import binding, runner as orunner
 
@@ -74,8 +75,6 @@ def test_dense_configs(name, entry, oracle, dev):
     w = (SMALL.get(name) or FULL[name])()
     if entry == "per_head_flag" and w.heads[0].mask != "causal":
         pytest.skip("is_causal flag only describes causal problems")
-    if name in FULL and entry in ("batch_dense",):
-        pytest.skip("covered at reduced size")
     ref = _oracle_out(w, oracle)
     d = dev.DeviceWorkload(w)
     try:
@@ -121,12 +120,18 @@ def test_weights_and_lse(name, mask_mode, oracle, dev):
             gw = wbufs[t].cpu().numpy()
             assert_close(gw, host_w[t], "%s weights head %d" % (name, t))
             assert ((gw == 0) == (host_w[t] == 0)).all(), "masked pattern differs"
-            lse = lbufs[t].cpu().numpy().reshape(h.nq, 2)
-            # (m, l): weights = exp(x - m) / l, so sum of ref weights * l == sum exp == l
-            assert np.isfinite(lse).all()
-            assert (lse[:, 1] >= 1.0 - 1e-4).all()  # the max term contributes exp(0) = 1
+        # (m, l) in natural units: the weights rebuilt from the pair must be the checker's weights
+        cache = {}
+        lse_check.check_workload(w, [t.cpu().numpy() for t in lbufs], host_w,
+                                 lambda h: orunner._mask_for(oracle, w, h, cache))
     finally:
         d.close()
+
+
+def test_lse_pair_single_head(oracle, dev):
+    """lse_out alone (the reference's BLT_FLASH_ATTN output mode) and together with weights_out:
+    dead rows, additive biases, causal flag, no mask."""
+    lse_check.run_single_head_cases(api.load(), oracle, api, abi, binding)
 
 
 # ---------------------------------------------------------------------------
@@ -366,7 +371,8 @@ def test_block_diffusion_mask_bit_exact(mode, S, N, B, starts, oracle, dev):
 # KV-cache step (config 4) and block verify (config 5)
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("batch,steps,H,hd,len_hi", [(3, 5, 4, 32, 70), (64, 6, 4, 32, 512), (5, 4, 2, 64, 100),
-                                                     (4, 3, 8, 16, 40), (2, 40, 4, 32, 3)])
+                                                     (4, 3, 8, 16, 40), (2, 40, 4, 32, 3),
+                                                     (64, 256, 4, 32, 512)])   # the last: config 4 at full size
 def test_kv_decode_steps(batch, steps, H, hd, len_hi, oracle, dev):
     kw = workloads.config4(batch=batch, steps=steps, H=H, hd=hd, len_hi=len_hi)
     ref_out, ref_k, ref_v = orunner.run_kv(kw, lib=oracle)
@@ -416,6 +422,116 @@ def test_block_verify(B, batch, oracle, dev):
     assert (lens == kw.lens).all()   # verify does not commit
     assert ck.tobytes() == ref_k.tobytes() and cv.tobytes() == ref_v.tobytes()
     assert_close(out, ref_out, "block verify B=%d" % B)
+
+
+@pytest.mark.parametrize("B,nseq", [(4, 12), (8, 12), (16, 64)])
+def test_diffusion_self_attention_call_pattern(B, nseq, oracle, dev):
+    """The reference's own route to config 5 (csrc/models/block_diffusion.c:196-204, 293-319): the whole
+    [prefix ; block] sequence of S = N + B rows through one blt_attention_head_core call per head with
+    nq = nk = S and the dense INFER mask blt_build_block_diffusion_mask builds on the device.  All S rows
+    against the checker; the block rows also against what the cached-prefix block kernel returns
+    for the same sequence (blt_kv_attend_step_hip, BLT_KV_STEP_BLOCK)."""
+    import torch
+    lib = api.load()
+    kw = workloads.config5(B=B)
+    d = dev.DeviceKvWorkload(kw)
+    d.run()
+    step_out = d.results()[0][0]                      # [batch * B, E] of the single step
+    E, H, hd = kw.E, kw.H, kw.hd
+    scale = float(np.float32(1.0) / np.sqrt(np.float32(hd)))
+    arena = lib.blt_arena_create(16 << 20, abi.BLT_BACKEND_HIP)
+    rs = np.random.RandomState(B)
+    for b in range(nseq):
+        N = int(kw.lens[b])
+        S = N + B
+        slab = slice(b * kw.max_seq_len, b * kw.max_seq_len + N)
+        k = np.concatenate([kw.cache_k[slab], kw.k_new[0, b * B:(b + 1) * B]]).astype(np.float32)
+        v = np.concatenate([kw.cache_v[slab], kw.v_new[0, b * B:(b + 1) * B]]).astype(np.float32)
+        q = np.concatenate([rs.randn(N, E).astype(np.float32), kw.q_new[0, b * B:(b + 1) * B]])
+        cfg = abi.BltBlockDiffusionConfig()
+        cfg.mode, cfg.seq_len, cfg.num_clean, cfg.block_size = abi.BLT_BDM_INFER, S, N, B
+        # checker: restated mask builder + one core call per head
+        mask = np.empty(S * S, dtype=np.float32)
+        assert oracle.orc_build_block_diffusion_mask(C.byref(cfg), binding.fptr(mask)) == 0
+        ref = np.zeros((S, E), dtype=np.float32)
+        scratch = np.empty(S * S, dtype=np.float32)
+        for h in range(H):
+            a = binding.head_args(q.reshape(-1), k.reshape(-1), v.reshape(-1), ref.reshape(-1), S, S, hd, scale, E, E,
+                                  E, E, h * hd, q_off=h * hd, k_off=h * hd, v_off=h * hd, scratch=scratch, mask=mask)
+            assert oracle.orc_attention_head_core(C.byref(a)) == 0
+        # device: the reference caller's statements on this library's ops
+        arena.contents.offset = 0
+        t = abi.BltTensor()
+        lib.blt_build_block_diffusion_mask(C.byref(cfg), C.byref(t), arena)
+        got_mask = np.empty(S * S, dtype=np.float32)
+        lib.blt_tensor_download(C.byref(t), got_mask.ctypes.data, got_mask.nbytes)
+        assert got_mask.tobytes() == mask.tobytes()
+        tq, tk, tv = (torch.from_numpy(x).cuda() for x in (q, k, v))
+        comb = torch.zeros((S, E), dtype=torch.float32, device="cuda")
+        scores = torch.empty(S * S, dtype=torch.float32, device="cuda")
+        for h in range(H):
+            a = api.head_args(tq.data_ptr() + 4 * h * hd, tk.data_ptr() + 4 * h * hd, tv.data_ptr() + 4 * h * hd,
+                              comb.data_ptr(), S, S, hd, scale, E, E, E, E, h * hd, weights=scores.data_ptr(),
+                              mask=t.data)
+            lib.blt_attention_head_core(abi.BLT_BACKEND_HIP, C.byref(a))
+        lib.blt_backend_pass_sync_hip()
+        got = comb.cpu().numpy()
+        assert_close(got, ref, "sequence %d: [prefix ; block] rows" % b)
+        assert_close(step_out[b * B:(b + 1) * B], ref[N:], "sequence %d: block kernel against the dense route" % b)
+    lib.blt_arena_destroy(arena)
+
+
+def test_zero_weight_key_with_non_finite_value_row(oracle, dev):
+    """Documents the one place where results can differ from the reference: the reference's weighted
+    sum skips keys whose weight is exactly zero (csrc/ops/attn_core_cpu.c:47-50), so a masked key
+    whose V row holds inf / NaN leaves the output finite; the kernels here multiply (0 * inf = NaN).
+    What is guaranteed and checked: (1) only the columns that are non-finite in that V row can
+    differ; (2) wherever the reference's output is non-finite, so is this library's; (3) rows whose
+    key range ends before the bad key's 32-key tile (the kernels never load tiles no row of a
+    32-row query tile can see) are untouched; (4) elsewhere in those columns the value is either
+    the reference's (within tolerance) or NaN."""
+    lib = api.load()
+    rs = np.random.RandomState(11)
+    nq = nk = 160
+    hd = 32
+    q, k, v = (rs.randn(n, hd).astype(np.float32) for n in (nq, nk, nk))
+    bad_key, bad_col = 100, 5
+    v[bad_key, bad_col] = np.inf
+    scale = float(np.float32(1.0) / np.sqrt(np.float32(hd)))
+    out_ref = np.zeros((nq, hd), dtype=np.float32)
+    w_ref = np.zeros((nq, nk), dtype=np.float32)
+    a = binding.head_args(q.reshape(-1), k.reshape(-1), v.reshape(-1), out_ref.reshape(-1), nq, nk, hd, scale, hd, hd,
+                          hd, hd, 0, weights=w_ref.reshape(-1), causal=True)
+    assert oracle.orc_attention_head_core(C.byref(a)) == 0
+    assert np.isfinite(out_ref[:bad_key]).all() and not np.isfinite(out_ref[bad_key:, bad_col]).any()
+    got, _ = _run_single(lib, q.reshape(-1), k.reshape(-1), v.reshape(-1), nq, nk, hd, scale, hd, hd, hd, hd, 0,
+                         causal=True)
+    other = [c for c in range(hd) if c != bad_col]
+    assert_close(got[:, other], out_ref[:, other], "columns the bad value is not in")          # (1)
+    assert not np.isfinite(got[bad_key:, bad_col]).any()                                       # (2)
+    first_tile_row = (bad_key // 32) * 32
+    assert_close(got[:first_tile_row, bad_col], out_ref[:first_tile_row, bad_col], "rows before the key's tile")  # (3)
+    mid = got[first_tile_row:bad_key, bad_col]                                                 # (4)
+    fin = np.isfinite(mid)
+    assert np.isnan(mid[~fin]).all()
+    if fin.any():
+        assert_close(mid[fin], out_ref[first_tile_row:bad_key, bad_col][fin], "finite cells of the key's tile")
+
+
+@pytest.mark.parametrize("mode", ["hint", "slab", "tables"])
+def test_kv_step_length_beyond_capacity_is_reported(mode):
+    """The lengths of the KV step live on the device; the host sizes the launch from a hint.  A
+    sequence that outgrew the hint, its slab or the rotation tables is left alone by the kernels
+    (which all exit normally) and the next synchronising call ends with the reference's "exceeds
+    cache capacity" error (csrc/infer/kv_cache.c:191).  Runs in its own process: the error is fatal."""
+    import os
+    import subprocess
+    import sys
+    here = os.path.dirname(os.path.abspath(__file__))
+    p = subprocess.run([sys.executable, "-u", os.path.join(here, "kv_guard_case.py"), mode], capture_output=True,
+                       text=True, timeout=300)
+    assert "CHECKED" in p.stdout and "NOT REACHED" not in p.stdout, p.stdout[-2000:] + p.stderr[-2000:]
+    assert p.returncode == 1 and "exceeds cache capacity" in p.stderr, (p.returncode, p.stderr[-2000:])
 
 
 @pytest.mark.parametrize("seed", range(24))
