@@ -650,6 +650,14 @@ extern "C" void blt_kv_attend_step_hip(const blt_kv_attn_cache *cache, const flo
                 combined_stride, n, step_kind, commit, max_len_hint, false);
 }
 
+extern "C" void blt_kv_attend_step_noalloc_hip(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride,
+                                               const float *k_rows, size_t k_stride, const float *v_rows,
+                                               size_t v_stride, float *combined, size_t combined_stride, size_t n,
+                                               int step_kind, int commit, size_t max_len_hint) {
+    kv_step_run(cache, q_rows, q_stride, k_rows, k_stride, v_rows, v_stride, nullptr, nullptr, 0, combined,
+                combined_stride, n, step_kind, commit, max_len_hint, true);
+}
+
 extern "C" void blt_kv_rope_attend_step_hip(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride,
                                             const float *k_rows, size_t k_stride, const float *v_rows,
                                             size_t v_stride, const float *rope_cos, const float *rope_sin,

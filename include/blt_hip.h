@@ -319,6 +319,20 @@ void blt_kv_attend_step_hip(const blt_kv_attn_cache *cache, const float *q_rows,
                             float *combined, size_t combined_stride, size_t n, int step_kind, int commit,
                             size_t max_len_hint);
 
+/* blt_kv_attend_step_hip for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid it).  No counterpart in the reference.  Same
+ * arguments, same kernels, same results; the per-split softmax records, the per-sequence tickets
+ * and the error word come from a fixed device array inside the library (4 MiB of records, 4096
+ * sequences; one copy per GPU, held until the process ends) instead of buffers that grow on demand,
+ * and the call issues no hipMalloc / hipFree.  A step that needs more (batch * splits * heads *
+ * row slots * (head_dim + 2) floats of records with splits > 1, or more than 4096 sequences) ends
+ * with a message naming both figures.  All calls on one GPU share the array: calls that overlap
+ * on that GPU (two streams, two threads) race; issue them in order on one stream. */
+void blt_kv_attend_step_noalloc_hip(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride,
+                                    const float *k_rows, size_t k_stride, const float *v_rows, size_t v_stride,
+                                    float *combined, size_t combined_stride, size_t n, int step_kind, int commit,
+                                    size_t max_len_hint);
+
 /* blt_kv_attend_step_hip with the rotation of the new rows fused in: the step
  * of blt_kv_decode_step from the QKV projection's output to `combined`
  * (csrc/infer/kv_cache.c:262-271 position gather, 343-366 per-head copy-out,
