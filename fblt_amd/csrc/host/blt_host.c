@@ -200,43 +200,75 @@ void blt_cross_attention_forward(const blt_tensor *query_in, const blt_tensor *k
 /* ------------------------------------------------------------------ */
 /* two-tier KV cache container (csrc/infer/kv_cache.c:27-110)          */
 /* ------------------------------------------------------------------ */
+/* Geometry of a cache for a decoder, checked in one place.  The struct contract
+ * (include/blt_abi.h, mirroring csrc/infer/kv_cache.h:45-65): per layer four [rows, embed]
+ * fp32 tensors, tier 1 with batch * max_seq_len byte rows, tier 2 with batch * max_subtokens
+ * sub-token rows; a patch of patch_dim columns splits into patch_dim / embed sub-tokens. */
+typedef struct {
+    size_t layers;
+    size_t embed;
+    size_t patch_dim;
+    size_t split;      /* sub-tokens per patch */
+    size_t subtokens;  /* tier-2 rows per sequence */
+    size_t batch;
+} kv_geometry;
+
+static kv_geometry kv_geometry_of(const blt_local_decoder *decoder, size_t max_seq_len, size_t batch_size) {
+    const blt_local_decoder_config *cfg = &decoder->config;
+    kv_geometry g;
+    g.layers = cfg->num_layers;
+    g.embed = cfg->embed_dim;
+    g.patch_dim = cfg->patch_dim != 0 ? cfg->patch_dim : cfg->embed_dim;
+    BLT_REQUIRE(g.embed > 0 && g.patch_dim % g.embed == 0,
+                "blt_kv_cache_create: patch_dim (%zu) must be a positive multiple of embed_dim (%zu)", g.patch_dim,
+                g.embed);
+    BLT_REQUIRE(max_seq_len >= 2 && max_seq_len <= cfg->max_seq_len,
+                "blt_kv_cache_create: max_seq_len %zu outside [2, %zu], the decoder's own limit", max_seq_len,
+                cfg->max_seq_len);
+    g.split = g.patch_dim / g.embed;
+    g.subtokens = max_seq_len; /* every patch covers at least one byte, so tier 2 never needs more rows */
+    g.batch = batch_size != 0 ? batch_size : 1;
+    return g;
+}
+
 blt_kv_cache *blt_kv_cache_create_batched(blt_arena *arena, const blt_local_decoder *decoder, size_t max_seq_len,
                                           size_t batch_size) {
-    if (batch_size == 0) batch_size = 1;
     BLT_REQUIRE(arena != NULL && decoder != NULL, "blt_kv_cache_create: arena and decoder cannot be NULL");
-    BLT_REQUIRE(max_seq_len >= 2 && max_seq_len <= decoder->config.max_seq_len,
-                "blt_kv_cache_create: max_seq_len must be in [2, decoder max_seq_len]");
-    const size_t E = decoder->config.embed_dim;
-    const size_t patch_dim = decoder->config.patch_dim ? decoder->config.patch_dim : E;
-    BLT_REQUIRE(E != 0 && patch_dim % E == 0, "blt_kv_cache_create: patch_dim must be a multiple of embed_dim");
-    const size_t L = decoder->config.num_layers;
-    blt_kv_cache *c = (blt_kv_cache *)calloc(1, sizeof(*c));
-    BLT_REQUIRE(c != NULL, "blt_kv_cache_create: failed to allocate cache container");
-    c->decoder = decoder;
-    c->max_seq_len = max_seq_len;
-    c->batch_size = batch_size;
-    c->max_subtokens = max_seq_len; /* a patch holds at least one byte */
-    c->embed_dim = E;
-    c->patch_dim = patch_dim;
-    c->k = patch_dim / E;
-    /* four separate heap arrays, as the reference's destroy frees them one by one (kv_cache.c:77-87) */
-    c->self_k = (blt_tensor *)calloc(L ? L : 1, sizeof(blt_tensor));
-    c->self_v = (blt_tensor *)calloc(L ? L : 1, sizeof(blt_tensor));
-    c->cross_k = (blt_tensor *)calloc(L ? L : 1, sizeof(blt_tensor));
-    c->cross_v = (blt_tensor *)calloc(L ? L : 1, sizeof(blt_tensor));
-    BLT_REQUIRE(c->self_k && c->self_v && c->cross_k && c->cross_v,
-                "blt_kv_cache_create: failed to allocate layer handle arrays");
-    const size_t self_shape[2] = {batch_size * max_seq_len, E};
-    const size_t cross_shape[2] = {batch_size * c->max_subtokens, E};
-    for (size_t l = 0; l < L; l++) {
-        c->self_k[l] = blt_tensor_create(arena, self_shape, 2, BLT_DTYPE_FP32);
-        c->self_v[l] = blt_tensor_create(arena, self_shape, 2, BLT_DTYPE_FP32);
-        c->cross_k[l] = blt_tensor_create(arena, cross_shape, 2, BLT_DTYPE_FP32);
-        c->cross_v[l] = blt_tensor_create(arena, cross_shape, 2, BLT_DTYPE_FP32);
+    const kv_geometry g = kv_geometry_of(decoder, max_seq_len, batch_size);
+    blt_kv_cache *cache = (blt_kv_cache *)calloc(1, sizeof(*cache));
+    BLT_REQUIRE(cache != NULL, "blt_kv_cache_create: out of host memory for the container");
+    cache->decoder = decoder;
+    cache->batch_size = g.batch;
+    cache->max_seq_len = max_seq_len;
+    cache->max_subtokens = g.subtokens;
+    cache->embed_dim = g.embed;
+    cache->patch_dim = g.patch_dim;
+    cache->k = g.split;
+
+    /* The four tiers: where the container keeps each handle array, and the rows of one layer's
+     * tensor.  Each handle array is a heap block of its own (destroy releases them one by one,
+     * and so does the reference's, csrc/infer/kv_cache.c:77-87); the payloads are zero-filled
+     * arena tensors, placed layer by layer. */
+    const struct {
+        blt_tensor **handles;
+        size_t rows;
+    } tiers[4] = {{&cache->self_k, g.batch * max_seq_len},
+                  {&cache->self_v, g.batch * max_seq_len},
+                  {&cache->cross_k, g.batch * g.subtokens},
+                  {&cache->cross_v, g.batch * g.subtokens}};
+    for (size_t t = 0; t < 4; t++) {
+        *tiers[t].handles = (blt_tensor *)calloc(g.layers != 0 ? g.layers : 1, sizeof(blt_tensor));
+        BLT_REQUIRE(*tiers[t].handles != NULL, "blt_kv_cache_create: out of host memory for %zu layer handles", g.layers);
     }
-    c->cached_patches = (blt_patch_info *)calloc(batch_size * max_seq_len, sizeof(blt_patch_info));
-    BLT_REQUIRE(c->cached_patches != NULL, "blt_kv_cache_create: failed to allocate patch table");
-    return c;
+    for (size_t layer = 0; layer < g.layers; layer++) {
+        for (size_t t = 0; t < 4; t++) {
+            const size_t shape[2] = {tiers[t].rows, g.embed};
+            (*tiers[t].handles)[layer] = blt_tensor_create(arena, shape, 2, BLT_DTYPE_FP32);
+        }
+    }
+    cache->cached_patches = (blt_patch_info *)calloc(g.batch * max_seq_len, sizeof(blt_patch_info));
+    BLT_REQUIRE(cache->cached_patches != NULL, "blt_kv_cache_create: out of host memory for the patch table");
+    return cache;
 }
 
 blt_kv_cache *blt_kv_cache_create(blt_arena *arena, const blt_local_decoder *decoder, size_t max_seq_len) {
@@ -244,34 +276,36 @@ blt_kv_cache *blt_kv_cache_create(blt_arena *arena, const blt_local_decoder *dec
 }
 
 void blt_kv_cache_destroy(blt_kv_cache *cache) {
-    if (!cache) return;
-    free(cache->self_k);
-    free(cache->self_v);
-    free(cache->cross_k);
-    free(cache->cross_v);
+    if (cache == NULL) return;
+    blt_tensor *const handle_arrays[4] = {cache->self_k, cache->self_v, cache->cross_k, cache->cross_v};
+    for (size_t t = 0; t < 4; t++) free(handle_arrays[t]);
     free(cache->cached_patches);
     free(cache);
 }
 
-void blt_kv_cache_reset(blt_kv_cache *cache) {
-    cache->self_len = 0;
-    cache->cross_num_patches = 0;
-}
-
+/* Rollback is bookkeeping only: rows past the valid counts are dead by contract
+ * (csrc/infer/kv_cache.c:89-99). */
 void blt_kv_cache_truncate(blt_kv_cache *cache, size_t self_len, size_t num_patches) {
-    BLT_REQUIRE(self_len <= cache->max_seq_len, "blt_kv_cache_truncate: self_len out of range");
-    BLT_REQUIRE(num_patches <= cache->max_subtokens, "blt_kv_cache_truncate: num_patches out of range");
+    BLT_REQUIRE(cache != NULL, "blt_kv_cache_truncate: cache cannot be NULL");
+    BLT_REQUIRE(self_len <= cache->max_seq_len, "blt_kv_cache_truncate: %zu byte rows exceed the cache's %zu",
+                self_len, cache->max_seq_len);
+    BLT_REQUIRE(num_patches <= cache->max_subtokens, "blt_kv_cache_truncate: %zu patches exceed the cache's %zu",
+                num_patches, cache->max_subtokens);
     cache->self_len = self_len;
     cache->cross_num_patches = num_patches;
 }
 
+void blt_kv_cache_reset(blt_kv_cache *cache) { blt_kv_cache_truncate(cache, 0, 0); }
+
+/* Length of the common prefix of the cached patch table and a new segmentation: patches agree
+ * when start and length agree (csrc/infer/kv_cache.c:101-109). */
 size_t blt_kv_cache_common_patches(const blt_kv_cache *cache, const blt_patch_info *patches, size_t num_patches) {
-    size_t same = 0;
-    while (same < cache->cross_num_patches && same < num_patches &&
-           cache->cached_patches[same].start_idx == patches[same].start_idx &&
-           cache->cached_patches[same].length == patches[same].length)
-        same++;
-    return same;
+    const size_t limit = num_patches < cache->cross_num_patches ? num_patches : cache->cross_num_patches;
+    for (size_t p = 0; p < limit; p++) {
+        const blt_patch_info *old = &cache->cached_patches[p];
+        if (old->start_idx != patches[p].start_idx || old->length != patches[p].length) return p;
+    }
+    return limit;
 }
 
 bool blt_local_cross_attn_fires(blt_xattn_placement placement, bool cross_attn_all_layers, size_t num_layers,
