@@ -116,6 +116,9 @@ SYMBOLS = {
     "blt_kv_rope_attend_step_hip": (None, [C.POINTER(BltKvAttnCache), C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t,
                                            C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p,
                                            C.c_size_t, C.c_size_t, C.c_int, C.c_int, C.c_size_t]),
+    "blt_kv_attend_step_lens_hip": (None, [C.POINTER(BltKvAttnCache), C.POINTER(C.c_uint32), C.c_void_p, C.c_size_t,
+                                           C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p,
+                                           C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t, C.c_int]),
     "blt_matmul_hip": (None, [C.POINTER(abi.BltTensor)] * 3),
     "blt_matmul": (None, [C.POINTER(abi.BltTensor)] * 3),
     "blt_rope_apply_hip": (None, [C.POINTER(abi.BltTensor)] * 4),

@@ -362,12 +362,28 @@ const DeviceStatics &statics() {
 
 struct GrowingScratch {
     std::map<hipStream_t, Scratch> by_stream;
+    std::map<hipStream_t, std::pair<uint32_t *, size_t>> lens_by_stream; /* staged host lengths */
     std::vector<void *> retired; /* replaced by larger buffers; live graphs may still name them */
 };
 
 GrowingScratch &growing() {
     static thread_local GrowingScratch g;
     return g;
+}
+
+/* Device copy of the caller's host lengths for this step (grow-only, per stream; ordered on the
+ * stream like every launch, so the next step's copy cannot overtake this step's kernels). */
+uint32_t *staged_lengths(const uint32_t *host_lens, size_t batch) {
+    GrowingScratch &g = growing();
+    auto &slot = g.lens_by_stream[blt_stream_key()];
+    BLT_REQUIRE(!blt_stream_capturing(), "blt_kv_attend_step_lens: host lengths cannot be staged while a graph capture is open");
+    if (batch > slot.second) {
+        if (slot.first) g.retired.push_back(slot.first);
+        slot.second = std::max<size_t>(2 * batch, 1024);
+        HIP_CHECK(hipMalloc((void **)&slot.first, slot.second * sizeof(uint32_t)));
+    }
+    blt_upload_staged(slot.first, host_lens, batch * sizeof(uint32_t));
+    return slot.first;
 }
 
 /* tickets must start at zero; a fill kernel, not a memset node, so that a capture could hold it */
@@ -423,12 +439,13 @@ namespace {
 void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride, const float *k_rows,
                    size_t k_stride, const float *v_rows, size_t v_stride, const float *rope_cos,
                    const float *rope_sin, size_t rope_positions, float *combined, size_t combined_stride, size_t n,
-                   size_t n_seq, size_t row0, int step_kind, int commit, size_t max_len_hint, bool static_scratch);
+                   size_t n_seq, size_t row0, int step_kind, int commit, size_t max_len_hint, bool static_scratch,
+                   const uint32_t *host_lens);
 
 void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride, const float *k_rows,
                  size_t k_stride, const float *v_rows, size_t v_stride, const float *rope_cos, const float *rope_sin,
                  size_t rope_positions, float *combined, size_t combined_stride, size_t n, int step_kind, int commit,
-                 size_t max_len_hint, bool static_scratch) {
+                 size_t max_len_hint, bool static_scratch, const uint32_t *host_lens = nullptr) {
     BLT_REQUIRE(q_rows != NULL && k_rows != NULL && v_rows != NULL && combined != NULL,
                 "blt_kv_attend_step: row buffers must not be NULL");
     BLT_REQUIRE(n >= 1, "blt_kv_attend_step: need at least one row");
@@ -438,6 +455,21 @@ void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_s
                 "blt_kv_attend_step: a block step takes at most 32 rows per sequence (every row sees every "
                 "new row, so the block cannot be cut)");
     BLT_REQUIRE(max_len_hint >= n, "blt_kv_attend_step: exceeds cache capacity");
+    /* Host lengths and a shape none of the kernel-argument kernels takes (several rows per sequence
+     * at a head width the matrix-core block kernels do not have): the lengths go to a device array
+     * of the library's through the pinned ring and the step runs as a non-committing device-length
+     * step. */
+    blt_kv_attn_cache staged_cache;
+    if (host_lens && cache != NULL && n > 1) {
+        const size_t hd = cache->num_heads ? cache->embed_dim / cache->num_heads : 0;
+        if (hd != 32 && hd != 64) {
+            staged_cache = *cache;
+            staged_cache.self_len = staged_lengths(host_lens, cache->batch);
+            cache = &staged_cache;
+            host_lens = nullptr;
+            commit = 0;
+        }
+    }
     /* A causal chunk longer than 32 rows (a prompt prefill) runs as consecutive 32-row slices: a
      * slice's rows see the cache, the earlier slices' rows (written through by then) and their
      * own; only the last slice advances the lengths. */
@@ -447,9 +479,9 @@ void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_s
         kv_step_slice(cache, q_rows + row0 * q_stride, q_stride, k_rows + row0 * k_stride, k_stride,
                       v_rows + row0 * v_stride, v_stride, rope_cos, rope_sin, rope_positions,
                       combined + row0 * combined_stride, combined_stride, rows, n, row0, step_kind, last ? commit : 0,
-                      max_len_hint - (n - row0 - rows), static_scratch);
+                      max_len_hint - (n - row0 - rows), static_scratch, host_lens);
     }
-    g_unchecked_steps.fetch_add(1, std::memory_order_relaxed);
+    if (!host_lens) g_unchecked_steps.fetch_add(1, std::memory_order_relaxed);
 }
 
 /* Query capacity of the per-split record layout a launch of `nq` rows uses: the VALU kernel's
@@ -495,8 +527,10 @@ void acquire_scratch(StepArgs &a, size_t floats, size_t batch, bool static_scrat
 void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_stride, const float *k_rows,
                    size_t k_stride, const float *v_rows, size_t v_stride, const float *rope_cos,
                    const float *rope_sin, size_t rope_positions, float *combined, size_t combined_stride, size_t n,
-                   size_t n_seq, size_t row0, int step_kind, int commit, size_t max_len_hint, bool static_scratch) {
-    BLT_REQUIRE(cache != NULL && cache->self_k != NULL && cache->self_v != NULL && cache->self_len != NULL,
+                   size_t n_seq, size_t row0, int step_kind, int commit, size_t max_len_hint, bool static_scratch,
+                   const uint32_t *host_lens) {
+    BLT_REQUIRE(cache != NULL && cache->self_k != NULL && cache->self_v != NULL &&
+                    (cache->self_len != NULL || host_lens != NULL),
                 "blt_kv_attend_step: cache buffers must not be NULL");
     const size_t E = cache->embed_dim, H = cache->num_heads;
     BLT_REQUIRE(H >= 1 && E % H == 0, "blt_kv_attend_step: embed_dim must be divisible by num_heads");
@@ -538,11 +572,48 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
     a.block_kind = step_kind == BLT_KV_STEP_BLOCK;
     a.hpb = 0, a.slices = 1;
 
+    static const int span_env = env_int("BLT_HIP_DECODE_SPAN", 0);
+    const size_t subs = (max_len_hint + SUB - 1) / SUB;
+
+    /* Lengths on the host (the reference keeps self_len there, csrc/infer/kv_cache.h:56-60): they
+     * travel in the kernel arguments, KARG_SEQS sequences per launch; the capacity check was made
+     * by the entry point.  Sequences [b0, b0 + nb) of the step as a launch of their own: */
+    auto chunk_of = [&](const StepArgs &all, size_t b0) {
+        StepArgs c = all;
+        c.cache_k += b0 * cache->max_seq_len * E, c.cache_v += b0 * cache->max_seq_len * E;
+        c.q_rows += b0 * n_seq * q_stride, c.k_rows += b0 * n_seq * k_stride, c.v_rows += b0 * n_seq * v_stride;
+        c.combined += b0 * n_seq * combined_stride;
+        return c;
+    };
+    if (host_lens && n_seq == 1) {
+        a.self_len = nullptr, a.partial = nullptr, a.tickets = nullptr, a.error = nullptr;
+        a.splits = 1, a.span = 0, a.cap = (uint32_t)cache->max_seq_len, a.q0 = 0, a.write_through = 1, a.commit = 0;
+        for (size_t b0 = 0; b0 < cache->batch; b0 += KARG_SEQS) {
+            const size_t nb = std::min<size_t>(KARG_SEQS, cache->batch - b0);
+            uint32_t longest = 0;
+            for (size_t b = 0; b < nb; b++) longest = std::max(longest, host_lens[b0 + b] + 1u);
+            kv_row_launch(chunk_of(a, b0), (uint32_t)nb, (uint32_t)hd, host_lens + b0, longest, 0);
+        }
+        HIP_CHECK_LAUNCH("blt_kv_attend_step_lens");
+        return;
+    }
+    /* Single rows of a batch that one workgroup per (sequence, head) spreads over the chip: the
+     * waves of a workgroup slice one head's keys and meet once in LDS, nothing crosses workgroups
+     * but the length ticket.  BLT_HIP_DECODE_ROW=0 keeps the split layout (tuning hook). */
+    static const int row_env = env_int("BLT_HIP_DECODE_ROW", 1);
+    if (n_seq == 1 && span_env == 0 &&
+        (row_env == 2 || (row_env == 1 && subs >= 4 && subs <= 64 && cache->batch * H >= 128 && cache->batch * H <= 512))) {
+        a.splits = 1, a.span = 0, a.q0 = 0, a.write_through = 1, a.commit = commit;
+        a.cap = (uint32_t)std::min<size_t>((size_t)cache->max_seq_len, rope_cos ? rope_positions : (size_t)UINT32_MAX);
+        acquire_scratch(a, 0, cache->batch, static_scratch);
+        kv_row_launch(a, (uint32_t)cache->batch, (uint32_t)hd, nullptr, (uint32_t)max_len_hint, 0);
+        HIP_CHECK_LAUNCH("blt_kv_attend_step");
+        return;
+    }
+
     /* enough workgroups to fill 256 compute units a few times over (sequences
      * shorter than the hint leave theirs idle), but no span shorter than two
      * sub-chunks */
-    static const int span_env = env_int("BLT_HIP_DECODE_SPAN", 0);
-    const size_t subs = (max_len_hint + SUB - 1) / SUB;
     size_t splits = (1024 + cache->batch - 1) / cache->batch;
     splits = std::min<size_t>(splits, (subs + 1) / 2);
     if (span_env > 0) splits = (subs + span_env - 1) / span_env;
@@ -576,8 +647,9 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
         const char *e = getenv("BLT_HIP_BLOCK_KERNEL");
         return e && strcmp(e, "valu") == 0 ? 1 : e && strcmp(e, "mfma") == 0 ? 2 : 0;
     }();
-    const bool want_mfma = pinned == 2 || (pinned == 0 && a.n >= 2u);
+    const bool want_mfma = pinned == 2 || (pinned == 0 && a.n >= 2u) || host_lens != nullptr;
     const bool mfma = want_mfma && (hd == 32 || hd == 64);
+    BLT_REQUIRE(mfma || !host_lens, "blt_kv_attend_step_lens: internal: host lengths reached a kernel without them");
     if (mfma) {
         /* the block kernel merges slices inside the workgroup, so it wants few,
          * long spans: just enough workgroups to cover the compute units */
@@ -607,8 +679,16 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
     if (mfma) {
         a.q0 = 0;
         a.write_through = 1;
-        a.commit = commit;
-        kv_block_mfma_launch(a, (uint32_t)cache->batch, (uint32_t)hd, 0);
+        a.commit = host_lens ? 0 : commit;
+        if (host_lens) {
+            a.self_len = nullptr;
+            for (size_t b0 = 0; b0 < cache->batch; b0 += KARG_SEQS) {
+                const size_t nb = std::min<size_t>(KARG_SEQS, cache->batch - b0);
+                kv_block_mfma_launch(chunk_of(a, b0), (uint32_t)nb, (uint32_t)hd, host_lens + b0, 0);
+            }
+        } else {
+            kv_block_mfma_launch(a, (uint32_t)cache->batch, (uint32_t)hd, nullptr, 0);
+        }
         HIP_CHECK_LAUNCH("blt_kv_attend_step");
         return;
     }
@@ -671,4 +751,23 @@ extern "C" void blt_kv_rope_attend_step_hip(const blt_kv_attn_cache *cache, cons
                 rope_positions);
     kv_step_run(cache, q_rows, q_stride, k_rows, k_stride, v_rows, v_stride, rope_cos, rope_sin, rope_positions,
                 combined, combined_stride, n, step_kind, commit, max_len_hint, false);
+}
+
+extern "C" void blt_kv_attend_step_lens_hip(const blt_kv_attn_cache *cache, const uint32_t *self_len_host,
+                                            const float *q_rows, size_t q_stride, const float *k_rows, size_t k_stride,
+                                            const float *v_rows, size_t v_stride, const float *rope_cos,
+                                            const float *rope_sin, size_t rope_positions, float *combined,
+                                            size_t combined_stride, size_t n, int step_kind) {
+    BLT_REQUIRE(self_len_host != NULL, "blt_kv_attend_step_lens: the host lengths must not be NULL");
+    BLT_REQUIRE((rope_cos == NULL) == (rope_sin == NULL), "blt_kv_attend_step_lens: both rotation tables or none");
+    BLT_REQUIRE(((reinterpret_cast<uintptr_t>(rope_cos) | reinterpret_cast<uintptr_t>(rope_sin)) & 7u) == 0,
+                "blt_kv_attend_step_lens: rotation tables must be 8-byte aligned");
+    BLT_REQUIRE(cache != NULL, "blt_kv_attend_step_lens: cache must not be NULL");
+    /* the reference's check (csrc/infer/kv_cache.c:191), made where the lengths live */
+    const size_t limit = std::min<size_t>(cache->max_seq_len, rope_cos ? rope_positions : SIZE_MAX);
+    size_t longest = 0;
+    for (size_t b = 0; b < cache->batch; b++) longest = std::max<size_t>(longest, self_len_host[b]);
+    BLT_REQUIRE(longest + n <= limit, "blt_kv_attend_step_lens: exceeds cache capacity");
+    kv_step_run(cache, q_rows, q_stride, k_rows, k_stride, v_rows, v_stride, rope_cos, rope_sin, rope_positions,
+                combined, combined_stride, n, step_kind, 0, longest + n, false, self_len_host);
 }

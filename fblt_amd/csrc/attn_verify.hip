@@ -45,8 +45,8 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 /* One wavefront per (head, slice): blockDim.x = 64 * hpb * slices, head =
  * blockIdx.z * hpb + wave % hpb, slice = wave / hpb.  The slices of a head
  * take the span's 32-key sub-chunks round-robin and merge through LDS. */
-template <int HD, int WAVES>
-__global__ __launch_bounds__(64 * WAVES, 2) void kv_block_mfma_kernel(StepArgs a) {
+template <int HD, int WAVES, bool KARG>
+__global__ __launch_bounds__(64 * WAVES, 2) void kv_block_mfma_kernel(StepArgs a, LensArg<KARG> lens) {
     constexpr int HALF = HD / 2;
     constexpr int DB = HD / 32;
     constexpr int ROW = HD + 4;
@@ -67,9 +67,9 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block_mfma_kernel(StepArgs a
     const uint32_t h = lane >> 5;
     const uint32_t c = lane & 31u;
 
-    const uint32_t len = a.self_len[b] + a.len_bias;
+    const uint32_t len = kv_len_of(a, lens, b) + a.len_bias;
     const uint32_t nk = len + a.n;
-    if (kv_over_capacity(a, nk)) return; /* uniform over the sequence's workgroups */
+    if (!KARG && kv_over_capacity(a, nk)) return; /* uniform over the sequence's workgroups */
     const size_t slab = (size_t)b * a.max_seq_len;
     const uint32_t span = kv_span_of(a, nk);
     const uint32_t k_begin = split * span;
@@ -349,8 +349,8 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
  * Half the matrix-core cycles and half the softmax arithmetic of the 32-wide kernel per
  * sub-chunk.  K and V fragments come straight from global memory in fragment layout (a K row's
  * 128 bytes are shared by the four lane groups), nothing is staged through LDS. */
-template <int HD, int WAVES>
-__global__ __launch_bounds__(64 * WAVES, 2) void kv_block16_mfma_kernel(StepArgs a) {
+template <int HD, int WAVES, bool KARG>
+__global__ __launch_bounds__(64 * WAVES, 2) void kv_block16_mfma_kernel(StepArgs a, LensArg<KARG> lens) {
     constexpr int HALF = HD / 2;
     constexpr int QD = HD / 4;  /* columns of the head one lane group contracts */
     constexpr int DT = HD / 16; /* 16-row tiles of O^T */
@@ -371,9 +371,9 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block16_mfma_kernel(StepArgs
     const uint32_t g = lane >> 4;
     const uint32_t c = lane & 15u;
 
-    const uint32_t len = a.self_len[b] + a.len_bias;
+    const uint32_t len = kv_len_of(a, lens, b) + a.len_bias;
     const uint32_t nk = len + a.n;
-    if (kv_over_capacity(a, nk)) return; /* uniform over the sequence's workgroups */
+    if (!KARG && kv_over_capacity(a, nk)) return; /* uniform over the sequence's workgroups */
     const size_t slab = (size_t)b * a.max_seq_len;
     const uint32_t span = kv_span_of(a, nk);
     const uint32_t k_begin = split * span;
@@ -621,7 +621,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void kv_block16_mfma_kernel(StepArgs
 }
 
 template <int HD, int WAVES>
-void launch_block(StepArgs a, uint32_t batch, hipStream_t s) {
+void launch_block(StepArgs a, uint32_t batch, const uint32_t *host_lens, hipStream_t s) {
     /* a.hpb heads per workgroup (the caller's choice, see kv_block_heads_per_group); the other waves are slices */
     a.hpb = std::max(1u, std::min<uint32_t>(std::min<uint32_t>(a.hpb, a.num_heads), (uint32_t)WAVES));
     const uint32_t subs = (a.span + 31u) / 32u;
@@ -632,10 +632,18 @@ void launch_block(StepArgs a, uint32_t batch, hipStream_t s) {
         const char *e = getenv("BLT_HIP_BLOCK_TILE");
         return e && strcmp(e, "32") == 0;
     }();
-    if (a.n - a.q0 <= 16u && !wide_only)
-        blt_launch("kv_block16_mfma", kv_block16_mfma_kernel<HD, WAVES>, grid, dim3(64 * a.hpb * a.slices), 0, s, a);
-    else
-        blt_launch("kv_block_mfma", kv_block_mfma_kernel<HD, WAVES>, grid, dim3(64 * a.hpb * a.slices), 0, s, a);
+    const dim3 block(64 * a.hpb * a.slices);
+    const bool narrow = a.n - a.q0 <= 16u && !wide_only;
+    if (host_lens) {
+        KargLens lens;
+        for (uint32_t b = 0; b < batch; b++) lens.v[b] = host_lens[b];
+        if (narrow) blt_launch("kv_block16_mfma", kv_block16_mfma_kernel<HD, WAVES, true>, grid, block, 0, s, a, lens);
+        else blt_launch("kv_block_mfma", kv_block_mfma_kernel<HD, WAVES, true>, grid, block, 0, s, a, lens);
+    } else {
+        const DeviceLens lens{0u};
+        if (narrow) blt_launch("kv_block16_mfma", kv_block16_mfma_kernel<HD, WAVES, false>, grid, block, 0, s, a, lens);
+        else blt_launch("kv_block_mfma", kv_block_mfma_kernel<HD, WAVES, false>, grid, block, 0, s, a, lens);
+    }
 }
 
 } // namespace
@@ -653,10 +661,11 @@ uint32_t kv_block_heads_per_group(uint32_t batch, uint32_t subs, uint32_t num_he
 /* Takes head_dim 32 and 64 (the K tiles of four waves fit the static LDS
  * budget); the caller falls back to the VALU kernel otherwise.  Handles up to
  * 32 query rows per launch: a.q0 .. a.q0 + 31. */
-bool kv_block_mfma_launch(const StepArgs &a, uint32_t batch, uint32_t head_dim, hipStream_t s) {
+bool kv_block_mfma_launch(const StepArgs &a, uint32_t batch, uint32_t head_dim, const uint32_t *host_lens,
+                          hipStream_t s) {
     /* the per-wave K tiles bound the workgroup: 8 waves of 4.6 KB or 4 of 8.7 KB */
-    if (head_dim == 32u) launch_block<32, 8>(a, batch, s);
-    else if (head_dim == 64u) launch_block<64, 4>(a, batch, s);
+    if (head_dim == 32u) launch_block<32, 8>(a, batch, host_lens, s);
+    else if (head_dim == 64u) launch_block<64, 4>(a, batch, host_lens, s);
     else return false;
     return true;
 }

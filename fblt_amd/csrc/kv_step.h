@@ -48,6 +48,33 @@ struct StepArgs {
 };
 
 
+/* Where a launch takes the sequences' lengths from: a.self_len in device memory, or -- when the
+ * caller keeps the lengths on the host, as the reference does (csrc/infer/kv_cache.h:56-60) -- the
+ * kernel arguments themselves, KARG_SEQS sequences per launch.  With the lengths in the argument
+ * block the first K/V requests of a workgroup depend on nothing but that block: one dependent
+ * trip to memory less.  Such a launch checks nothing and commits nothing on the device (the host
+ * did the capacity check and owns the lengths). */
+constexpr int KARG_SEQS = 256;
+struct KargLens {
+    uint32_t v[KARG_SEQS];
+};
+struct DeviceLens {
+    uint32_t unused;
+};
+template <bool KARG>
+struct LensArgOf {
+    typedef DeviceLens type;
+};
+template <>
+struct LensArgOf<true> {
+    typedef KargLens type;
+};
+template <bool KARG>
+using LensArg = typename LensArgOf<KARG>::type;
+
+__device__ __forceinline__ uint32_t kv_len_of(const StepArgs &a, const KargLens &lens, uint32_t b) { return lens.v[b]; }
+__device__ __forceinline__ uint32_t kv_len_of(const StepArgs &a, const DeviceLens &, uint32_t b) { return a.self_len[b]; }
+
 /* The lengths live in device memory and the launch was sized from a host-side hint.  A sequence
  * whose length + new rows went past what the launch, its slab or the rotation tables hold must
  * neither drop keys silently nor store past its slab: every workgroup of such a sequence leaves
@@ -171,7 +198,16 @@ __device__ __forceinline__ void kv_finish_sequence(const StepArgs &a, uint32_t s
 
 /* heads per workgroup the MFMA block kernel should be launched with (set StepArgs.hpb to it) */
 uint32_t kv_block_heads_per_group(uint32_t batch, uint32_t subs, uint32_t num_heads);
-/* launch of the MFMA block kernel (attn_verify.hip); false when it does not take the shape */
-bool kv_block_mfma_launch(const StepArgs &a, uint32_t batch, uint32_t head_dim, hipStream_t s);
+/* launch of the MFMA block kernel (attn_verify.hip); false when it does not take the shape.
+ * host_lens: NULL (device lengths) or `batch` <= KARG_SEQS lengths for the argument block */
+bool kv_block_mfma_launch(const StepArgs &a, uint32_t batch, uint32_t head_dim, const uint32_t *host_lens,
+                          hipStream_t s);
+
+/* single-row steps with one workgroup per (sequence, head) (attn_decode_row.hip): lengths from
+ * `host_lens` (at most KARG_SEQS sequences, carried in the kernel arguments; nothing is
+ * committed) or, when NULL, from a.self_len with the commit through a.tickets; max_keys sizes
+ * the workgroups; false when the head width is not taken */
+bool kv_row_launch(const StepArgs &a, uint32_t batch, uint32_t head_dim, const uint32_t *host_lens, uint32_t max_keys,
+                   hipStream_t s);
 
 #endif

@@ -162,11 +162,17 @@ class DeviceWorkload:
 
 class DeviceKvWorkload:
     """Device-resident KV-cache workload driving blt_kv_attend_step_hip, or
-    blt_kv_rope_attend_step_hip when the workload carries rotation tables."""
+    blt_kv_rope_attend_step_hip when the workload carries rotation tables.  With
+    lens="host" the lengths stay on the host (as the reference keeps them) and single-row
+    steps go through blt_kv_attend_step_lens_hip; the device copy of the lengths is then
+    not used."""
 
-    def __init__(self, kw):
+    def __init__(self, kw, lens="device"):
         torch = _torch()
         self.kw = kw
+        self.lens_mode = lens
+        self.host_lens = kw.lens.astype(np.uint32)  # the caller's own lengths (lens="host")
+        self._host_lens_p = self.host_lens.ctypes.data_as(C.POINTER(C.c_uint32))
         self.lib = api.load()
         self.cache_k = torch.from_numpy(kw.cache_k).cuda()
         self.cache_v = torch.from_numpy(kw.cache_v).cuda()
@@ -192,13 +198,22 @@ class DeviceKvWorkload:
         """Lengths back to the start; cache rows past them are dead by contract."""
         self.lens.copy_(self.lens0)
         self.host_max_len = int(self.kw.lens.max())
+        self.host_lens[:] = self.kw.lens
         _torch().cuda.synchronize()
 
     def step(self, s):
         kw = self.kw
         E = kw.E
         hint = self.host_max_len + kw.n
-        if self.rope is not None:
+        if self.lens_mode == "host":
+            cos, sin, rows = ((self.rope[0].data_ptr(), self.rope[1].data_ptr(), self.rope[0].shape[0])
+                              if self.rope is not None else (None, None, 0))
+            self.lib.blt_kv_attend_step_lens_hip(C.byref(self.c), self._host_lens_p, self.q_new[s].data_ptr(), E,
+                                                 self.k_new[s].data_ptr(), E, self.v_new[s].data_ptr(), E, cos, sin,
+                                                 rows, self.out[s].data_ptr(), E, kw.n, self.kind)
+            if kw.commit:  # the caller advances its lengths, as the reference does after a step
+                self.host_lens += np.uint32(kw.n)
+        elif self.rope is not None:
             self.lib.blt_kv_rope_attend_step_hip(C.byref(self.c), self.q_new[s].data_ptr(), E,
                                                  self.k_new[s].data_ptr(), E, self.v_new[s].data_ptr(), E,
                                                  self.rope[0].data_ptr(), self.rope[1].data_ptr(),
@@ -219,5 +234,6 @@ class DeviceKvWorkload:
 
     def results(self):
         _torch().cuda.synchronize()
-        return (self.out.cpu().numpy(), self.cache_k.cpu().numpy(), self.cache_v.cpu().numpy(),
-                self.lens.cpu().numpy())
+        lens = (self.host_lens.astype(np.int32) if self.lens_mode == "host"
+                else self.lens.cpu().numpy())
+        return self.out.cpu().numpy(), self.cache_k.cpu().numpy(), self.cache_v.cpu().numpy(), lens

@@ -353,6 +353,28 @@ void blt_kv_rope_attend_step_hip(const blt_kv_attn_cache *cache, const float *q_
                                  float *combined, size_t combined_stride, size_t n, int step_kind, int commit,
                                  size_t max_len_hint);
 
+/* The single-row step with the lengths where the reference keeps them: on the
+ * host (blt_kv_cache.self_len, csrc/infer/kv_cache.h:56-60; advanced by the
+ * caller after the step, kv_cache.c:416).  self_len_host[b] is the number of
+ * valid rows of sequence b; cache->self_len (the device array) is neither read
+ * nor written and may be NULL.  The lengths travel in the kernel arguments, so
+ * the first K/V requests of a workgroup depend on nothing but the argument
+ * block -- one memory round trip less than the device-length step -- and the
+ * capacity check of kv_cache.c:191 is made on the host before anything is
+ * launched ("exceeds cache capacity").  rope_cos / rope_sin as in
+ * blt_kv_rope_attend_step_hip, or both NULL for rows that arrive rotated.
+ * n and step_kind as in blt_kv_attend_step_hip (single rows, causal chunks,
+ * blocks of at most 32 rows); nothing is committed on the device.  Head
+ * widths the matrix-core block kernels do not take (anything but 32 and 64)
+ * with n > 1 stage the lengths to a device array of the library's and run the
+ * device-length kernels.  Not for replay from a graph: the lengths are frozen
+ * into the launch. */
+void blt_kv_attend_step_lens_hip(const blt_kv_attn_cache *cache, const uint32_t *self_len_host,
+                                 const float *q_rows, size_t q_stride, const float *k_rows, size_t k_stride,
+                                 const float *v_rows, size_t v_stride, const float *rope_cos, const float *rope_sin,
+                                 size_t rope_positions, float *combined, size_t combined_stride, size_t n,
+                                 int step_kind);
+
 /* One decoder layer of blt_kv_decode_step (csrc/infer/kv_cache.c:326-414
  * without the optional cross-attention: RMSNorm, QKV projection, rotation +
  * write-through + attention of the new rows, output projection, residual;

@@ -373,10 +373,13 @@ def test_block_diffusion_mask_bit_exact(mode, S, N, B, starts, oracle, dev):
 @pytest.mark.parametrize("batch,steps,H,hd,len_hi", [(3, 5, 4, 32, 70), (64, 6, 4, 32, 512), (5, 4, 2, 64, 100),
                                                      (4, 3, 8, 16, 40), (2, 40, 4, 32, 3),
                                                      (64, 256, 4, 32, 512)])   # the last: config 4 at full size
-def test_kv_decode_steps(batch, steps, H, hd, len_hi, oracle, dev):
+@pytest.mark.parametrize("lens_mode", ["device", "host"])
+def test_kv_decode_steps(batch, steps, H, hd, len_hi, lens_mode, oracle, dev):
+    """lens_mode host: blt_kv_attend_step_lens_hip, the lengths kept by the caller as the reference
+    keeps them (kv_cache.h:56-60) and carried in the kernel arguments."""
     kw = workloads.config4(batch=batch, steps=steps, H=H, hd=hd, len_hi=len_hi)
     ref_out, ref_k, ref_v = orunner.run_kv(kw, lib=oracle)
-    d = dev.DeviceKvWorkload(kw)
+    d = dev.DeviceKvWorkload(kw, lens=lens_mode)
     d.run()
     out, ck, cv, lens = d.results()
     assert (lens == kw.lens.astype(np.int64) + steps).all()          # slot bookkeeping: exact
@@ -384,26 +387,58 @@ def test_kv_decode_steps(batch, steps, H, hd, len_hi, oracle, dev):
     assert_close(out, ref_out, "kv decode")
 
 
-def test_kv_decode_window(oracle, dev):
+@pytest.mark.parametrize("lens_mode", ["device", "host"])
+def test_kv_decode_window(lens_mode, oracle, dev):
     kw = workloads.config4(batch=6, steps=4, H=4, hd=32, len_hi=200)
     kw.window = 48
     ref_out, ref_k, ref_v = orunner.run_kv(kw, lib=oracle)
-    d = dev.DeviceKvWorkload(kw)
+    d = dev.DeviceKvWorkload(kw, lens=lens_mode)
     d.run()
     out, ck, cv, lens = d.results()
     assert ck.tobytes() == ref_k.tobytes()
     assert_close(out, ref_out, "kv decode window")
 
 
+@pytest.mark.parametrize("lens_mode", ["device", "host"])
+@pytest.mark.parametrize("batch,H,hd,len_lo,len_hi,window,rope", [
+    (64, 4, 32, 0, 300, 0, False),     # from empty caches
+    (64, 4, 32, 100, 700, 0, True),    # rotation fused in
+    (40, 4, 32, 1, 900, 130, False),   # window that skips whole rounds of keys
+    (32, 8, 16, 1, 400, 0, True),
+    (64, 2, 64, 1, 500, 77, True),
+    (128, 1, 128, 1, 260, 0, False),
+    (70, 2, 8, 0, 200, 0, False),
+    (140, 1, 4, 1, 150, 5, False),
+    (300, 1, 32, 1, 140, 0, True),     # host lengths: more sequences than one launch carries
+    (130, 2, 32, 1000, 2040, 0, False),
+])
+def test_kv_single_row_steps(batch, H, hd, len_lo, len_hi, window, rope, lens_mode, oracle, dev):
+    """One new row per sequence at batch sizes that give one workgroup per (sequence, head): every
+    head width, empty caches, windows, fused rotation, three committing steps in a row; lengths
+    in device memory or in the caller's hands."""
+    steps = 3
+    kw = workloads.config4(batch=batch, steps=steps, H=H, hd=hd, len_lo=len_lo, len_hi=len_hi,
+                           max_seq_len=len_hi + steps, rope=rope)
+    kw.window = window
+    ref_out, ref_k, ref_v = orunner.run_kv(kw, lib=oracle)
+    d = dev.DeviceKvWorkload(kw, lens=lens_mode)
+    d.run()
+    out, ck, cv, lens = d.results()
+    assert (lens == kw.lens.astype(np.int64) + steps).all()
+    assert ck.tobytes() == ref_k.tobytes() and cv.tobytes() == ref_v.tobytes()
+    assert_close(out, ref_out, "kv single rows")
+
+
+@pytest.mark.parametrize("lens_mode", ["device", "host"])
 @pytest.mark.parametrize("n", [2, 3, 8, 20])
-def test_kv_prefill_chunk(n, oracle, dev):
+def test_kv_prefill_chunk(n, lens_mode, oracle, dev):
     """n > 1 rows per step, chunk-causal (kv_cache.c:229-236): same kernel, causal kind."""
     kw = workloads.config4(batch=5, steps=3, H=4, hd=32, len_hi=90, max_seq_len=90 + 3 * n)
     rs = np.random.RandomState(n)
     kw.n = n
     kw.q_new, kw.k_new, kw.v_new = (rs.randn(kw.steps, kw.batch * n, kw.E).astype(np.float32) for _ in range(3))
     ref_out, ref_k, ref_v = orunner.run_kv(kw, lib=oracle)
-    d = dev.DeviceKvWorkload(kw)
+    d = dev.DeviceKvWorkload(kw, lens=lens_mode)
     d.run()
     out, ck, cv, lens = d.results()
     assert (lens == kw.lens.astype(np.int64) + n * kw.steps).all()
@@ -411,12 +446,13 @@ def test_kv_prefill_chunk(n, oracle, dev):
     assert_close(out, ref_out, "kv chunk n=%d" % n)
 
 
+@pytest.mark.parametrize("lens_mode", ["device", "host"])
 @pytest.mark.parametrize("B", [4, 8, 16, 32])
 @pytest.mark.parametrize("batch", [3, 64])
-def test_block_verify(B, batch, oracle, dev):
+def test_block_verify(B, batch, lens_mode, oracle, dev):
     kw = workloads.config5(batch=batch, B=B)
     ref_out, ref_k, ref_v = orunner.run_kv(kw, lib=oracle)
-    d = dev.DeviceKvWorkload(kw)
+    d = dev.DeviceKvWorkload(kw, lens=lens_mode)
     d.run()
     out, ck, cv, lens = d.results()
     assert (lens == kw.lens).all()   # verify does not commit
@@ -534,8 +570,9 @@ def test_kv_step_length_beyond_capacity_is_reported(mode):
     assert p.returncode == 1 and "exceeds cache capacity" in p.stderr, (p.returncode, p.stderr[-2000:])
 
 
+@pytest.mark.parametrize("lens_mode", ["device", "host"])
 @pytest.mark.parametrize("seed", range(24))
-def test_kv_step_randomised(seed, oracle, dev):
+def test_kv_step_randomised(seed, lens_mode, oracle, dev):
     """Seeded draws over the KV step's free choices: sequences, heads, head width, cached lengths
     (from empty to long), rows per step (single rows, blocks, chunks longer than one launch takes),
     step kind, window, rotation fused in or not, committing steps in a row."""
@@ -554,7 +591,7 @@ def test_kv_step_randomised(seed, oracle, dev):
         kw.window = int(rs.choice([1, 7, 48]))
     kw.q_new, kw.k_new, kw.v_new = (rs.randn(kw.steps, kw.batch * n, kw.E).astype(np.float32) for _ in range(3))
     ref_out, ref_k, ref_v = orunner.run_kv(kw, lib=oracle)
-    d = dev.DeviceKvWorkload(kw)
+    d = dev.DeviceKvWorkload(kw, lens=lens_mode)
     d.run()
     out, ck, cv, lens = d.results()
     what = "seed %d batch %d H %d hd %d len<=%d n %d %s steps %d window %s rope %s" % (
