@@ -10,6 +10,18 @@
 #include "attn_device.h"
 #include "rope_device.h"
 
+#ifdef BLT_MARKS /* experiment builds only: cycle marks of wave 0 of every workgroup */
+extern __device__ unsigned long long blt_marks[];
+#define BLT_MARK(i)                                                                                        \
+    do {                                                                                                   \
+        if (threadIdx.x == 0)                                                                              \
+            blt_marks[((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 16 + (i)] =       \
+                __builtin_readcyclecounter();                                                              \
+    } while (0)
+#else
+#define BLT_MARK(i) do { } while (0)
+#endif
+
 constexpr int SUB = 32;        /* keys per sub-chunk (one wave, one head)       */
 constexpr int MAX_SPLITS = 16; /* workgroups per sequence                        */
 
