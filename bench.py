@@ -206,14 +206,15 @@ def bench_caller_path(w, d, steps, warmup):
             "wall_us_per_pass": wall / n * 1e6, "tokens_per_s": w.tokens * n / wall}
 
 
-def bench_kv(kw, steps, warmup, warm_ms=0.0):
+def bench_kv(kw, steps, warmup, warm_ms=0.0, lens="device"):
     """KV-cache workloads: `steps` consecutive step calls after `warmup` calls.  A
     committing workload (decode) appends one row per call and needs kw.steps >=
     warmup + steps; a non-committing one (verify) repeats its single step (and can be
-    warmed by time, see warm_up)."""
+    warmed by time, see warm_up).  lens="host": the caller keeps the lengths, as the
+    reference does, and the steps go through blt_kv_attend_step_lens_hip."""
     from fblt_amd import api, runner
     lib = api.load()
-    d = runner.DeviceKvWorkload(kw)
+    d = runner.DeviceKvWorkload(kw, lens=lens)
     idx = (lambda s: s) if kw.commit else (lambda s: 0)
 
     def one_pass(profiled):
@@ -260,6 +261,8 @@ def bench_kv(kw, steps, warmup, warm_ms=0.0):
         "flops": flops_step, "bytes": bytes_step,
         "roofline_hbm": roofline("hbm", bytes_step, avg_s, MEASURED_TRAFFIC_BYTES.get(kw.name)),
         "roofline_mfma": roofline("mfma", flops_step, avg_s),
+        "entry": ("blt_kv_attend_step_lens_hip (lengths on the host, carried in the kernel arguments)"
+                  if lens == "host" else "blt_kv_attend_step_hip / blt_kv_rope_attend_step_hip (lengths in device memory)"),
     }
     if warm_ms and not kw.commit:
         res["warmup_ms"] = warm_ms
@@ -671,6 +674,104 @@ def bench_decode_step(steps, warmup, batch=64, L=2, E=128, H=4, hidden=512, V=25
     return res
 
 
+def bench_draft_pass(steps, warmup, cpu_budget_s, N=400, B=8, L=2, E=128, H=4, hidden=512, V=256):
+    """One denoising pass of the reference's draft loop (csrc/infer/block_generation.c:156-266: one
+    sequence, N clean bytes, a block of B [MASK] rows on the last latent) three ways: the reference's
+    call blt_local_decoder_forward_diffusion_infer (the whole [N + B] forward again on every pass),
+    blt_kv_block_step_hip over a cache that holds the prefix (the block rows only), and the restated
+    dense forward on one host core."""
+    import ctypes as C
+    import numpy as np
+    import torch
+    from fblt_amd import abi, api, decoder
+    lib = api.load()
+    hd, half = E // H, E // H // 2
+    max_len = N + 32 + (-(N + 32)) % 4
+    weights = decoder.random_weights(E, hidden, L, V, 23)
+    view = lambda t: abi.tensor_view(t.data_ptr(), tuple(t.shape), abi.BLT_BACKEND_HIP)
+    cos, sin = torch.zeros((max_len, half), device="cuda"), torch.zeros((max_len, half), device="cuda")
+    vc, vs = view(cos), view(sin)
+    rcfg = abi.BltRopeConfig(500000.0, hd)
+    lib.blt_rope_precompute(max_len, C.byref(rcfg), C.byref(vc), C.byref(vs))
+    tables = (cos.cpu().numpy(), sin.cpu().numpy())
+    bound = decoder.bind(weights, *tables, abi.BLT_BACKEND_HIP, decoder.device_place, E, H, H, hidden, V, max_len)
+    lengths = [4] * (N // 4)
+    P = len(lengths)
+    patches = decoder.patch_table(lengths)
+    rs = np.random.RandomState(29)
+    hidden_rows, latents = rs.randn(N, E).astype(np.float32), rs.randn(P, E).astype(np.float32)
+    batch = decoder.BlockBatch(N, B, P)
+    th, tp = torch.from_numpy(hidden_rows).cuda(), torch.from_numpy(latents).cuda()
+    full, block = torch.zeros((N + B, V), device="cuda"), torch.zeros((B, V), device="cuda")
+    vh, vp, vf, vb = view(th), view(tp), view(full), view(block)
+    arena = lib.blt_arena_create(1 << 30, abi.BLT_BACKEND_HIP)
+    cache = lib.blt_kv_cache_create(arena, bound.ptr, max_len)
+    lib.blt_kv_cache_refresh_cross(cache, C.byref(vp), patches, P, 0, arena)
+    prefix = torch.zeros((N, V), device="cuda")
+    vpre = view(prefix)
+    lib.blt_kv_decode_step(cache, C.byref(vp), patches, P, C.byref(vh), 1, C.byref(vpre), arena)
+    lib.blt_backend_pass_sync_hip()
+    mark = arena.contents.offset
+
+    def timed(call):
+        def run(count):
+            for _ in range(count):
+                arena.contents.offset = mark
+                call()
+        run(warmup)
+        lib.blt_backend_pass_sync_hip()
+        lib.blt_hip_profile_begin()
+        run(steps)
+        lib.blt_backend_pass_sync_hip()
+        prof = api.profile_end()
+        t0 = time.perf_counter()
+        run(steps)
+        lib.blt_backend_pass_sync_hip()
+        wall = (time.perf_counter() - t0) / steps
+        return {"launches_per_pass": sum(v[0] for v in prof.values()) / steps,
+                "kernel_us_per_pass": sum(v[1] for v in prof.values()) * 1e3 / steps, "wall_us_per_pass": wall * 1e6,
+                "per_kernel_us": {k: v[1] * 1e3 / steps for k, v in prof.items()}}
+
+    dense = timed(lambda: lib.blt_local_decoder_forward_diffusion_infer(
+        bound.ptr, C.byref(vh), C.byref(vp), patches, P, batch.ptr, abi.BLT_D0_LEARNED, C.byref(vf), arena))
+    cached = timed(lambda: lib.blt_kv_block_step_hip(cache, P, batch.ptr, abi.BLT_D0_LEARNED, C.byref(vb), arena))
+    lib.blt_backend_pass_sync_hip()
+    agree = float((full[N:] - block).abs().max().item())
+    lib.blt_kv_cache_destroy(cache)
+    lib.blt_arena_destroy(arena)
+    avg_s = cached["kernel_us_per_pass"] * 1e-6
+    per_layer_w = E * E * 2 + E * 3 * E + E * E + 3 * E * hidden
+    nbytes = 4.0 * (L * (2 * E * (N + B) + per_layer_w + 2 * E * B) + E * V)
+    flops = L * (B * 2.0 * per_layer_w + 4.0 * hd * H * B * (N + B)) + B * 2.0 * E * V
+    res = {"workload": "draft pass: 1 sequence, %d clean bytes, block of %d rows, %d layers (cross block in each), "
+                       "E=%d, H=%d, hidden=%d, V=%d" % (N, B, L, E, H, hidden, V),
+           "entry": "blt_kv_block_step_hip over the cached prefix",
+           "kernel": "+".join(sorted(cached["per_kernel_us"])), "launches_per_step": cached["launches_per_pass"],
+           "tokens_per_step": B, "us_per_step": cached["wall_us_per_pass"], "kernel_us_avg": cached["kernel_us_per_pass"],
+           "kernel_us_min": min(cached["per_kernel_us"].values()), "per_kernel_us": cached["per_kernel_us"],
+           "tokens_per_s": B / (cached["wall_us_per_pass"] * 1e-6), "flops": flops, "bytes": nbytes,
+           "roofline_hbm": roofline("hbm", nbytes, avg_s), "roofline_mfma": roofline("mfma", flops, avg_s),
+           "reference_call": dict(dense, entry="blt_local_decoder_forward_diffusion_infer (prefix recomputed per pass)"),
+           "block_rows_max_abs_difference_between_the_two": agree}
+    res["roofline"] = res["roofline_hbm"]
+    if cpu_budget_s > 0:
+        from oracle import binding
+        orc = binding.load_oracle()
+        host = decoder.bind(weights, *tables, abi.BLT_BACKEND_CPU, decoder.host_place, E, H, H, hidden, V, max_len)
+        out = np.zeros((N + B, V), dtype=np.float32)
+        fp = lambda a: binding.fptr(a.reshape(-1))
+        t0, passes = time.perf_counter(), 0
+        while passes == 0 or time.perf_counter() - t0 < cpu_budget_s:
+            assert orc.orc_local_decoder_forward_diffusion_infer(host.ptr, fp(hidden_rows), fp(latents), patches, P,
+                                                                 batch.ptr, abi.BLT_D0_LEARNED, fp(out)) == 0
+            passes += 1
+        dt = (time.perf_counter() - t0) / passes
+        res["cpu_baseline"] = {"value": B / dt, "unit": "tokens/s", "cores": 1, "kind": "port",
+                               "sample": "%d dense passes of the restated forward, %.1f s" % (passes, dt * passes),
+                               "ms_per_pass": dt * 1e3}
+    return res
+
+
 def cpu_decode_step(budget_s, batch=64, L=2, E=128, H=4, hidden=512, V=256, len_hi=512, n=1):
     """The restated decoder step on one host core, one sequence at a time as the reference runs it."""
     import numpy as np
@@ -829,6 +930,10 @@ def main():
     if want("c4"):
         others["c4"], k4 = bench_kv(workloads.config4(steps=W + 256, max_seq_len=512 + W + 256), 256, W)
         log("c4", json.dumps(others["c4"]))
+        # the same steps with the lengths where the reference keeps them (on the host)
+        others["c4_host_lens"], _ = bench_kv(workloads.config4(steps=W + 256, max_seq_len=512 + W + 256), 256, W,
+                                             lens="host")
+        log("c4_host_lens", json.dumps(others["c4_host_lens"]))
         # the same steps with the rotation of the new Q/K rows fused in (un-rotated inputs + tables)
         others["c4_rope"], _ = bench_kv(workloads.config4(steps=W + 256, max_seq_len=512 + W + 256, rope=True), 256,
                                         W)
@@ -859,6 +964,9 @@ def main():
         others["c4_b128_L2048"], _ = bench_kv(big, 20, 3)
         others["c4_b128_L2048"]["roofline_hbm"]["traffic"] = None
         log("c4_b128_L2048", json.dumps(others["c4_b128_L2048"]))
+        others["c4_b128_L2048_host_lens"], _ = bench_kv(big, 20, 3, lens="host")
+        others["c4_b128_L2048_host_lens"]["roofline_hbm"]["traffic"] = None
+        log("c4_b128_L2048_host_lens", json.dumps(others["c4_b128_L2048_host_lens"]))
         bigv = workloads.config5(batch=128, B=16, len_lo=1024, len_hi=2032, max_seq_len=2048, cache_period=8)
         others["c5_B16_b128_L2048"], _ = bench_kv(bigv, 20, 3, warm_ms=100.0)
         others["c5_B16_b128_L2048"]["roofline_hbm"]["traffic"] = None
@@ -894,6 +1002,9 @@ def main():
         if not args.no_cpu:
             others["decode_step_prefill_512"]["cpu_baseline"] = cpu_decode_step(2.0 * cs, batch=1, len_hi=1, n=512)
         log("decode_step_prefill_512", json.dumps(others["decode_step_prefill_512"]))
+        # BLT-D drafting: one denoising pass over a 400-byte prefix, block of 8
+        others["draft_pass"] = bench_draft_pass(K, W, 0.0 if args.no_cpu else 2.0 * cs)
+        log("draft_pass", json.dumps(others["draft_pass"]))
 
     # the dense-mask builders the callers still use
     if want("masks"):
@@ -960,15 +1071,20 @@ def compact_line(head, others, cpu_head, K, W, detail_path):
             o["cpu"] = [_sig(b["value"]), b["unit"]]
         return _sig(o)
     per = {"c2": row(head)}
-    for k in ("c1", "c3", "c4", "c4_rope", "c5_B4", "c5_B8", "c5_B16"):
+    for k in ("c1", "c3", "c4", "c4_host_lens", "c4_rope", "c5_B4", "c5_B8", "c5_B16"):
         if k in others:
             per[k] = row(others[k])
     # the same kernels away from the launch floor: [kernel us, binding roofline, fraction of it]
     scaled = {k: [_sig(others[k]["kernel_us_avg"]), others[k]["roofline"]["bound"], _sig(others[k]["roofline"]["frac"])]
-              for k in ("c1_x64", "c2_x8", "c1_T4096", "c2_P2048", "c4_b128_L2048", "c5_B16_b128_L2048") if k in others}
+              for k in ("c1_x64", "c2_x8", "c1_T4096", "c2_P2048", "c4_b128_L2048", "c4_b128_L2048_host_lens",
+                        "c5_B16_b128_L2048") if k in others}
     # whole decoder step (all layers + LM head): [launches per step, device us, wall us]
     steps_ = {k: [others[k]["launches_per_step"], _sig(others[k]["kernel_us_avg"]), _sig(others[k]["us_per_step"])]
-              for k in ("decode_step", "decode_step_b1") if k in others}
+              for k in ("decode_step", "decode_step_b1", "draft_pass") if k in others}
+    if "draft_pass" in others:   # the reference's call (prefix recomputed per pass) beside the cached block step
+        c = others["draft_pass"]["reference_call"]
+        steps_["draft_pass_reference_call"] = [c["launches_per_pass"], _sig(c["kernel_us_per_pass"]),
+                                               _sig(c["wall_us_per_pass"])]
     return {
         "metric": "attn_tokens_per_s", "value": head["tokens_per_s"], "unit": "tokens/s",
         "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": head["ms_per_step"],
@@ -984,7 +1100,10 @@ def compact_line(head, others, cpu_head, K, W, detail_path):
         "cpu_baseline": cpu_head,
         "cpu_cores": cpu_head["cores"] if cpu_head else None,
         # the other parts of the composite headline metric (decode us/step, verify tokens/s), when they ran
-        "decode_us_per_step": others["c4"]["us_per_step"] if "c4" in others else None,
+        # decode: wall microseconds per step of the 256 consecutive steps; the lengths on the host as in the
+        # reference's blt_kv_decode_step (the device-length entry, which graphs can replay, is beside it)
+        "decode_us_per_step": others["c4_host_lens"]["us_per_step"] if "c4_host_lens" in others else None,
+        "decode_us_per_step_device_lens": others["c4"]["us_per_step"] if "c4" in others else None,
         "verify_tokens_per_s": {k: others[k]["tokens_per_s"] for k in ("c5_B4", "c5_B8", "c5_B16") if k in others} or None,
         "per_config": per,
         "at_scale": scaled or None,

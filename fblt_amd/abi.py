@@ -197,9 +197,34 @@ class BltKvCache(C.Structure):
 
 
 BLT_XATTN_DEFAULT, BLT_XATTN_NONE, BLT_XATTN_LAST, BLT_XATTN_ALL, BLT_XATTN_FIRST = range(5)
+BLT_D0_HFINAL, BLT_D0_ZEROS, BLT_D0_LEARNED = range(3)
+BLT_MASK_TOKEN_ID = 256
+
+
+class BltBlockBatch(C.Structure):
+    """csrc/models/block_diffusion.h:37-86"""
+    _fields_ = [
+        ("num_clean", C.c_size_t),
+        ("block_size", C.c_size_t),
+        ("num_blocks", C.c_size_t),
+        ("n_block_rows", C.c_size_t),
+        ("t", C.c_float),
+        ("tokens", C.POINTER(C.c_uint32)),
+        ("positions", C.POINTER(C.c_size_t)),
+        ("targets", C.POINTER(C.c_uint8)),
+        ("cell_valid", C.POINTER(C.c_uint8)),
+        ("cell_masked", C.POINTER(C.c_uint8)),
+        ("groups", C.POINTER(C.c_size_t)),
+        ("loss_scale", C.c_float),
+        ("last_row_scale", C.c_float),
+        ("clean_sum", C.c_int),
+        ("mask_norm", C.c_int),
+        ("trailing_closed", C.c_int),
+    ]
 
 
 def check_layout():
+    assert C.sizeof(BltBlockBatch) == 112
     assert C.sizeof(BltTensor) == 104
     assert C.sizeof(BltArena) == 32
     assert C.sizeof(BltAttentionHeadArgs) == 136

@@ -119,6 +119,18 @@ SYMBOLS = {
     "blt_kv_attend_step_lens_hip": (None, [C.POINTER(BltKvAttnCache), C.POINTER(C.c_uint32), C.c_void_p, C.c_size_t,
                                            C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p,
                                            C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t, C.c_int]),
+    "blt_local_decoder_forward_diffusion_infer_hip": (None, [C.POINTER(abi.BltLocalDecoder), C.POINTER(abi.BltTensor),
+                                                             C.POINTER(abi.BltTensor), C.POINTER(abi.BltPatchInfo),
+                                                             C.c_size_t, C.POINTER(abi.BltBlockBatch), C.c_int,
+                                                             C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)]),
+    "blt_local_decoder_forward_diffusion_infer": (None, [C.POINTER(abi.BltLocalDecoder), C.POINTER(abi.BltTensor),
+                                                         C.POINTER(abi.BltTensor), C.POINTER(abi.BltPatchInfo),
+                                                         C.c_size_t, C.POINTER(abi.BltBlockBatch), C.c_int,
+                                                         C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)]),
+    "blt_embedding_lookup": (None, [C.POINTER(abi.BltTensor), C.POINTER(C.c_uint32), C.POINTER(abi.BltTensor)]),
+    "blt_embedding_lookup_hip": (None, [C.POINTER(abi.BltTensor), C.POINTER(C.c_uint32), C.POINTER(abi.BltTensor)]),
+    "blt_kv_block_step_hip": (None, [C.POINTER(abi.BltKvCache), C.c_size_t, C.POINTER(abi.BltBlockBatch), C.c_int,
+                                     C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)]),
     "blt_matmul_hip": (None, [C.POINTER(abi.BltTensor)] * 3),
     "blt_matmul": (None, [C.POINTER(abi.BltTensor)] * 3),
     "blt_rope_apply_hip": (None, [C.POINTER(abi.BltTensor)] * 4),

@@ -460,9 +460,12 @@ void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_s
      * of the library's through the pinned ring and the step runs as a non-committing device-length
      * step. */
     blt_kv_attn_cache staged_cache;
-    if (host_lens && cache != NULL && n > 1) {
+    if (host_lens && cache != NULL) {
         const size_t hd = cache->num_heads ? cache->embed_dim / cache->num_heads : 0;
-        if (hd != 32 && hd != 64) {
+        /* ... and single rows of a few long sequences, which the split kernel spreads over more
+         * compute units than one workgroup per (sequence, head) reaches */
+        const bool few_long = n == 1 && cache->batch * cache->num_heads < 64 && max_len_hint > 4096;
+        if ((n > 1 && hd != 32 && hd != 64) || few_long) {
             staged_cache = *cache;
             staged_cache.self_len = staged_lengths(host_lens, cache->batch);
             cache = &staged_cache;

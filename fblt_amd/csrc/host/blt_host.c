@@ -159,6 +159,12 @@ void blt_rows_gather(const blt_tensor *src, const size_t *pos_host, blt_tensor *
     blt_rows_gather_hip(src, pos_host, dst);
 }
 
+void blt_embedding_lookup(const blt_tensor *table, const uint32_t *ids_host, blt_tensor *out) {
+    BLT_REQUIRE(table != NULL, "blt_embedding_lookup: arguments cannot be NULL");
+    BLT_DEVICE_ONLY(table->backend, "blt_embedding_lookup");
+    blt_embedding_lookup_hip(table, ids_host, out);
+}
+
 void blt_rope_position_gather(const blt_tensor *cos_cache, const blt_tensor *sin_cache, const size_t *positions,
                               size_t n, blt_tensor *cos_out, blt_tensor *sin_out, blt_arena *arena) {
     BLT_REQUIRE(cos_cache != NULL && sin_cache != NULL && positions != NULL && cos_out != NULL && sin_out != NULL &&
@@ -333,6 +339,16 @@ void blt_kv_decode_step(blt_kv_cache *cache, const blt_tensor *patch_in, const b
     BLT_REQUIRE(d0_rows != NULL, "blt_kv_decode_step: arguments cannot be NULL");
     BLT_DEVICE_ONLY(d0_rows->backend, "blt_kv_decode_step");
     blt_kv_decode_step_hip(cache, patch_in, patches, num_patches, d0_rows, trailing_closed, logits_out, arena);
+}
+
+void blt_local_decoder_forward_diffusion_infer(const blt_local_decoder *model, const blt_tensor *byte_hidden_in,
+                                               const blt_tensor *patch_in, const blt_patch_info *patches,
+                                               size_t num_patches, const blt_block_batch *batch, blt_d0_mode d0_mode,
+                                               blt_tensor *logits_out, blt_arena *arena) {
+    BLT_REQUIRE(byte_hidden_in != NULL, "forward_diffusion_infer: arguments cannot be NULL");
+    BLT_DEVICE_ONLY(byte_hidden_in->backend, "blt_local_decoder_forward_diffusion_infer");
+    blt_local_decoder_forward_diffusion_infer_hip(model, byte_hidden_in, patch_in, patches, num_patches, batch, d0_mode,
+                                                  logits_out, arena);
 }
 
 void blt_add(const blt_tensor *a, const blt_tensor *b, blt_tensor *out) {

@@ -226,9 +226,29 @@ void long_chunk_attention(const blt_kv_attn_cache *cache, const float *qkv, cons
     blt_attention_batch_hip(pr.data(), pr.size());
 }
 
+/* Q and K column blocks of packed [rows, 3E] projection rows rotated in place, row R at the
+ * position positions[R] (block rows carry their own positions, csrc/models/block_diffusion.c:
+ * 148-157; the arithmetic of csrc/ops/reductions_cpu.c:219-226). */
+__global__ __launch_bounds__(256) void rope_rows_at_kernel(float *__restrict__ qkv, const uint32_t *__restrict__ positions,
+                                                           const float *__restrict__ rope_cos,
+                                                           const float *__restrict__ rope_sin, uint32_t E, uint32_t hd) {
+    const uint32_t row = blockIdx.x;
+    const uint32_t pos = positions[row];
+    float *src = qkv + (size_t)row * 3u * E;
+    for (uint32_t col = 4u * threadIdx.x; col < 2u * E; col += 1024u) { /* Q block, then K block */
+        const size_t at = (size_t)pos * (hd / 2u) + (col % hd) / 2u;
+        float4 *cell = reinterpret_cast<float4 *>(src + col);
+        *cell = rope_rotate4(*cell, rope_cos + at, rope_sin + at);
+    }
+}
+
+/* host_base: the sequences' lengths where the caller keeps them (NULL: device lengths in
+ * cache->self_len); they then travel in the step kernels' arguments.  dev_positions: device array
+ * [rows] of rotary positions when they are not base + r (NULL otherwise). */
 void decode_layer_impl(const blt_kv_attn_cache *cache, const blt_transformer_weights *w, const float *rows_in,
                        float *rows_out, const float *rope_cos, const float *rope_sin, size_t rope_positions, size_t n,
-                       int step_kind, int commit, size_t max_len_hint, blt_arena *arena, const size_t *host_base) {
+                       int step_kind, int commit, size_t max_len_hint, blt_arena *arena, const size_t *host_base,
+                       const uint32_t *dev_positions = nullptr) {
     BLT_REQUIRE(cache != NULL && w != NULL && rows_in != NULL && rows_out != NULL && arena != NULL,
                 "blt_kv_decode_layer: arguments must not be NULL");
     BLT_REQUIRE(arena->backend == BLT_BACKEND_HIP, "blt_kv_decode_layer: needs a device arena");
@@ -269,12 +289,27 @@ void decode_layer_impl(const blt_kv_attn_cache *cache, const blt_transformer_wei
         rmsnorm_launch(rows_in, f32(w->norm1_weight), normed, rows, E);
         gemm(normed, f32(w->attn_qkv_w), qkv, rows, E, 3 * E);
     }
-    if (host_base != nullptr && n > 32 && step_kind == BLT_KV_STEP_CAUSAL && commit == 0 &&
-        (E / cache->num_heads) % 4 == 0)
+    if (host_base != nullptr && n > 32 && step_kind == BLT_KV_STEP_CAUSAL && commit == 0 && dev_positions == nullptr &&
+        (E / cache->num_heads) % 4 == 0) {
         long_chunk_attention(cache, qkv, rope_cos, rope_sin, rope_positions, n, host_base, combined, arena);
-    else
+    } else if (host_base != nullptr && commit == 0) {
+        /* the caller keeps the lengths: they go into the kernel arguments */
+        std::vector<uint32_t> lens(cache->batch);
+        for (size_t b = 0; b < cache->batch; b++) lens[b] = (uint32_t)host_base[b];
+        if (dev_positions != nullptr) { /* rows rotated at their own positions first, then a plain step */
+            BLT_REQUIRE((E / cache->num_heads) % 4 == 0, "blt_kv_block_step: explicit row positions need head_dim %% 4 == 0");
+            blt_launch("rope_rows_at", rope_rows_at_kernel, dim3((unsigned)rows), dim3(256), 0, 0, qkv, dev_positions,
+                       rope_cos, rope_sin, (uint32_t)E, (uint32_t)(E / cache->num_heads));
+            blt_kv_attend_step_lens_hip(cache, lens.data(), qkv, 3 * E, qkv + E, 3 * E, qkv + 2 * E, 3 * E, nullptr,
+                                        nullptr, 0, combined, E, n, step_kind);
+        } else {
+            blt_kv_attend_step_lens_hip(cache, lens.data(), qkv, 3 * E, qkv + E, 3 * E, qkv + 2 * E, 3 * E, rope_cos,
+                                        rope_sin, rope_positions, combined, E, n, step_kind);
+        }
+    } else {
         blt_kv_rope_attend_step_hip(cache, qkv, 3 * E, qkv + E, 3 * E, qkv + 2 * E, 3 * E, rope_cos, rope_sin,
                                     rope_positions, combined, E, n, step_kind, commit, max_len_hint);
+    }
     gemm(combined, f32(w->attn_proj_w), resid1, rows, E, E, rows_in); /* projection + residual in one pass */
     /* feed-forward block, kv_cache.c:396-414 */
     probe.n = (uint32_t)Hd;
@@ -349,8 +384,12 @@ void check_vec(const blt_tensor &t, size_t dim, const char *what) {
 /* The step for `batch` sequences with n new rows each: base[b] is sequence b's
  * valid length, group[b*n + r] the latent patch of its row r.  Lengths and
  * group ranges travel to the device in one staged copy. */
+/* step_kind / window: BLT_KV_STEP_CAUSAL with the decoder's local window for the incremental step;
+ * the diffusion forward runs its clean rows causally without a window and its block rows as
+ * BLT_KV_STEP_BLOCK.  positions (host, [batch*n]) when a row's rotary position is not base + r. */
 void decode_step_run(const blt_kv_cache *cache, size_t batch, size_t n, const size_t *base, const size_t *group,
-                     const float *d0_rows, float *logits, blt_arena *arena) {
+                     const float *d0_rows, float *logits, blt_arena *arena, int step_kind = BLT_KV_STEP_CAUSAL,
+                     size_t window = SIZE_MAX, const size_t *positions = nullptr) {
     const blt_local_decoder *dec = cache->decoder;
     const blt_local_decoder_config *cfg = &dec->config;
     const size_t E = cache->embed_dim, L = cfg->num_layers, H = cfg->num_heads, XH = cfg->cross_attn_heads;
@@ -363,7 +402,16 @@ void decode_step_run(const blt_kv_cache *cache, size_t batch, size_t n, const si
                  "blt_kv_decode_step: rope_sin_cache must be [max_seq_len, head_dim/2]");
 
     /* lengths, then lo / hi of every row's sub-token range, in one upload */
-    std::vector<uint32_t> host(batch + 2 * rows);
+    bool own_positions = false; /* any row whose rotary position is not base + r */
+    if (positions != nullptr)
+        for (size_t b = 0; b < batch; b++)
+            for (size_t r = 0; r < n; r++) {
+                BLT_REQUIRE(positions[b * n + r] < cfg->max_seq_len, "rope_position_gather: position index out of range");
+                own_positions = own_positions || positions[b * n + r] != base[b] + r;
+            }
+    std::vector<uint32_t> host(batch + 2 * rows + (own_positions ? rows : 0));
+    if (own_positions)
+        for (size_t i = 0; i < rows; i++) host[batch + 2 * rows + i] = (uint32_t)positions[i];
     size_t max_total = 0;
     for (size_t b = 0; b < batch; b++) {
         host[b] = (uint32_t)base[b];
@@ -442,7 +490,7 @@ void decode_step_run(const blt_kv_cache *cache, size_t batch, size_t n, const si
         view.max_seq_len = cache->max_seq_len;
         view.embed_dim = E;
         view.num_heads = H;
-        view.window = cfg->local_window;
+        view.window = window == SIZE_MAX ? cfg->local_window : window;
         blt_transformer_weights w;
         std::memset(&w, 0, sizeof(w));
         w.norm1_weight = &s->norm1_weight, w.attn_qkv_w = &s->attn_qkv_w, w.attn_proj_w = &s->attn_proj_w;
@@ -451,8 +499,8 @@ void decode_step_run(const blt_kv_cache *cache, size_t batch, size_t n, const si
         float *next = (cur == ping) ? pong : ping;
         arena->offset = arena_mark; /* the layer's work buffers are reused by the next layer */
         decode_layer_impl(&view, &w, in, next, (const float *)dec->rope_cos_cache.data,
-                          (const float *)dec->rope_sin_cache.data, cfg->max_seq_len, n, BLT_KV_STEP_CAUSAL, 0, max_total,
-                          arena, base);
+                          (const float *)dec->rope_sin_cache.data, cfg->max_seq_len, n, step_kind, 0, max_total, arena,
+                          base, own_positions ? dev + batch + 2 * rows : nullptr);
         cur = next;
     }
     gemm(cur, (const float *)dec->lm_head_weight.data, logits, rows, E, V); /* kv_cache.c:416 */
@@ -647,4 +695,140 @@ extern "C" void blt_kv_decode_step_batched_hip(blt_kv_cache *cache, size_t *self
     decode_step_run(cache, batch, n, self_len, group.data(), (const float *)d0_rows->data,
                     (float *)logits_out->data, arena);
     for (size_t b = 0; b < batch; b++) self_len[b] += n;
+}
+
+/* ===================================================================== */
+/* Inference-mode diffusion forward (csrc/models/block_diffusion.c:776-795) */
+/* ===================================================================== */
+namespace {
+
+/* D_0 rows of the block section (block_diffusion.c:137-146): zeros, or row tokens[r] of the
+ * learned table (csrc/ops/gather_scatter_cpu.c:7-29). */
+const float *block_d0_rows(const blt_local_decoder *dec, const blt_block_batch *batch, blt_d0_mode d0_mode,
+                           blt_arena *arena) {
+    const size_t E = dec->config.embed_dim, R = batch->n_block_rows;
+    const size_t shape[2] = {R, E};
+    if (d0_mode != BLT_D0_LEARNED) {
+        blt_tensor zeros = blt_tensor_create(arena, shape, 2, BLT_DTYPE_FP32); /* zero-filled */
+        return (const float *)zeros.data;
+    }
+    BLT_REQUIRE(batch->tokens != NULL, "forward_diffusion_infer: batch->tokens cannot be NULL with the learned D_0 table");
+    BLT_REQUIRE(dec->d0_embed_weight.data != NULL, "forward_diffusion_infer: the decoder has no learned D_0 table");
+    blt_tensor out = blt_tensor_create_uninit(arena, shape, 2, BLT_DTYPE_FP32);
+    blt_embedding_lookup_hip(&dec->d0_embed_weight, batch->tokens, &out);
+    return (const float *)out.data;
+}
+
+void check_block_batch(const blt_block_batch *batch, const char *fn) {
+    BLT_REQUIRE(batch != NULL, "%s: arguments cannot be NULL", fn);
+    BLT_REQUIRE(batch->n_block_rows >= 1 && batch->positions != NULL && batch->groups != NULL,
+                "%s: the batch needs at least one block row with positions and groups", fn);
+    BLT_REQUIRE(batch->n_block_rows <= 32,
+                "%s: at most 32 block rows (csrc/infer/block_generation.c:154); the rows of a block all see each "
+                "other, so the block cannot be cut",
+                fn);
+}
+
+/* The block rows over a cache whose sequence 0 holds the clean prefix. */
+void block_step_run(const blt_kv_cache *cache, size_t num_patches, const blt_block_batch *batch, blt_d0_mode d0_mode,
+                    float *logits, blt_arena *arena) {
+    const size_t base = batch->num_clean, R = batch->n_block_rows;
+    for (size_t r = 0; r < R; r++)
+        BLT_REQUIRE(batch->groups[r] < num_patches, "forward_diffusion_infer: a block row's latent group is out of range");
+    const float *d0 = block_d0_rows(cache->decoder, batch, d0_mode, arena);
+    decode_step_run(cache, 1, R, &base, batch->groups, d0, logits, arena, BLT_KV_STEP_BLOCK, 0, batch->positions);
+}
+
+} // namespace
+
+extern "C" void blt_kv_block_step_hip(blt_kv_cache *cache, size_t num_patches, const blt_block_batch *batch,
+                                      blt_d0_mode d0_mode, blt_tensor *logits_out, blt_arena *arena) {
+    check_cache(cache, "blt_kv_block_step");
+    check_block_batch(batch, "blt_kv_block_step");
+    const blt_local_decoder_config *cfg = &cache->decoder->config;
+    const size_t hd = cache->embed_dim / cfg->num_heads;
+    BLT_REQUIRE(hd > 0 && hd % 2 == 0, "blt_kv_block_step: RoPE requires an even head_dim");
+    BLT_REQUIRE(logits_out != NULL && arena != NULL, "blt_kv_block_step: arguments cannot be NULL");
+    BLT_REQUIRE(arena->backend == BLT_BACKEND_HIP, "blt_kv_block_step: HIP implementation needs a device arena");
+    BLT_REQUIRE(batch->num_clean == cache->self_len,
+                "blt_kv_block_step: the cache holds %zu byte rows, the batch says %zu clean rows", cache->self_len,
+                batch->num_clean);
+    BLT_REQUIRE(num_patches >= 1 && num_patches == cache->cross_num_patches,
+                "blt_kv_block_step: tier-2 cache must cover all patches (refresh first)");
+    BLT_REQUIRE(cache->self_len + batch->n_block_rows <= cache->max_seq_len, "blt_kv_block_step: exceeds cache capacity");
+    BLT_REQUIRE(logits_out->data != NULL && logits_out->ndim == 2 && logits_out->shape[0] == batch->n_block_rows &&
+                    logits_out->shape[1] == cfg->vocab_size && logits_out->dtype == BLT_DTYPE_FP32 &&
+                    logits_out->backend == BLT_BACKEND_HIP,
+                "blt_kv_block_step: logits_out must be [n_block_rows, vocab_size] FP32 in device memory");
+    block_step_run(cache, num_patches, batch, d0_mode, (float *)logits_out->data, arena);
+}
+
+extern "C" void blt_local_decoder_forward_diffusion_infer_hip(const blt_local_decoder *model,
+                                                              const blt_tensor *byte_hidden_in,
+                                                              const blt_tensor *patch_in, const blt_patch_info *patches,
+                                                              size_t num_patches, const blt_block_batch *batch,
+                                                              blt_d0_mode d0_mode, blt_tensor *logits_out,
+                                                              blt_arena *arena) {
+    BLT_REQUIRE(model != NULL && logits_out != NULL && arena != NULL && batch != NULL,
+                "forward_diffusion_infer: arguments cannot be NULL");
+    const blt_local_decoder_config *cfg = &model->config;
+    const size_t E = cfg->embed_dim, V = cfg->vocab_size, L = cfg->num_layers;
+    const size_t N = batch->num_clean, R = batch->n_block_rows, S = N + R;
+    const size_t pdim = cfg->patch_dim ? cfg->patch_dim : E, k = pdim / E;
+    BLT_REQUIRE(cfg->num_heads != 0 && E % cfg->num_heads == 0 && (E / cfg->num_heads) % 2 == 0,
+                "diffusion: RoPE requires an even head_dim");
+    BLT_REQUIRE(byte_hidden_in != NULL && patch_in != NULL && patches != NULL, "diffusion: arguments cannot be NULL");
+    BLT_REQUIRE(arena->backend == BLT_BACKEND_HIP && byte_hidden_in->backend == BLT_BACKEND_HIP &&
+                    patch_in->backend == BLT_BACKEND_HIP,
+                "forward_diffusion_infer: HIP implementation called with a non-HIP tensor");
+    BLT_REQUIRE(byte_hidden_in->ndim == 2 && byte_hidden_in->shape[0] == N && byte_hidden_in->shape[1] == E && N >= 1,
+                "diffusion: byte_hidden_in must be [N, embed_dim]");
+    BLT_REQUIRE(patch_in->ndim == 2 && patch_in->shape[0] == num_patches && patch_in->shape[1] == pdim && num_patches >= 1,
+                "diffusion: patch_in must be [num_patches, patch_dim]");
+    BLT_REQUIRE(S >= 2 && S <= cfg->max_seq_len, "diffusion: total sequence length outside [2, decoder max_seq_len]");
+    check_block_batch(batch, "forward_diffusion_infer");
+    BLT_REQUIRE(logits_out->data != NULL && logits_out->ndim == 2 && logits_out->shape[0] == S &&
+                    logits_out->shape[1] == V && logits_out->dtype == BLT_DTYPE_FP32 &&
+                    logits_out->backend == BLT_BACKEND_HIP,
+                "forward_diffusion_infer: logits_out must be [N + n_block_rows, vocab_size] FP32");
+
+    /* A clean row never sees a block row (csrc/ops/mask_builder_cpu.c:128-131), so the clean rows
+     * are the incremental step over an empty cache -- causal, no window (the INFER mask has none),
+     * the last row on the last latent when the patch is closed -- and the block rows are one block
+     * step over what that step cached (133-135: all clean rows plus the whole block).  The cache
+     * lives in the caller's arena like every other work buffer of this forward; nothing of it needs
+     * clearing, every row that is read was written first. */
+    std::vector<blt_tensor> tiers(4 * L);
+    const size_t subtokens = num_patches * k;
+    for (size_t l = 0; l < L; l++) {
+        const size_t self_shape[2] = {S, E}, cross_shape[2] = {subtokens, E};
+        tiers[0 * L + l] = blt_tensor_create_uninit(arena, self_shape, 2, BLT_DTYPE_FP32);
+        tiers[1 * L + l] = blt_tensor_create_uninit(arena, self_shape, 2, BLT_DTYPE_FP32);
+        tiers[2 * L + l] = blt_tensor_create_uninit(arena, cross_shape, 2, BLT_DTYPE_FP32);
+        tiers[3 * L + l] = blt_tensor_create_uninit(arena, cross_shape, 2, BLT_DTYPE_FP32);
+    }
+    std::vector<blt_patch_info> table(num_patches);
+    blt_kv_cache cache;
+    std::memset(&cache, 0, sizeof(cache));
+    cache.decoder = model;
+    cache.max_seq_len = S, cache.batch_size = 1, cache.max_subtokens = subtokens;
+    cache.embed_dim = E, cache.k = k, cache.patch_dim = pdim;
+    cache.self_k = tiers.data(), cache.self_v = tiers.data() + L;
+    cache.cross_k = tiers.data() + 2 * L, cache.cross_v = tiers.data() + 3 * L;
+    cache.cached_patches = table.data();
+    check_cache(&cache, "forward_diffusion_infer");
+
+    /* refresh_cross_seq indexes the snapshot by seq * max_seq_len: sequence 0 */
+    refresh_cross_seq(&cache, 0, patch_in, patches, num_patches, 0);
+    cache.cross_num_patches = num_patches;
+
+    std::vector<size_t> group(N); /* block_diffusion.c:163-172 */
+    latent_ids(patches, num_patches, 0, N, group.data());
+    if (batch->trailing_closed) group[N - 1] = num_patches - 1;
+    const size_t zero = 0;
+    float *logits = (float *)logits_out->data;
+    decode_step_run(&cache, 1, N, &zero, group.data(), (const float *)byte_hidden_in->data, logits, arena,
+                    BLT_KV_STEP_CAUSAL, 0);
+    cache.self_len = N;
+    block_step_run(&cache, num_patches, batch, d0_mode, logits + N * V, arena);
 }

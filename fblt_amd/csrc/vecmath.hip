@@ -4,6 +4,7 @@
  * product (reference contracts: csrc/ops/vecmath.h:14-37).
  */
 #include "blt_hip.h"
+#include <cstdlib>
 #include "blt_fatal.h"
 #include "hip_check.h"
 #include "launch.h"
@@ -160,6 +161,25 @@ extern "C" void blt_rows_gather_hip(const blt_tensor *src, const size_t *pos_hos
                                d + r0 * row_len, (uint64_t)row_len, g);
         HIP_CHECK_LAUNCH("blt_rows_gather");
     }
+}
+
+/* csrc/ops/gather_scatter_cpu.c:7-21: out row i = table row ids_host[i] */
+extern "C" void blt_embedding_lookup_hip(const blt_tensor *table, const uint32_t *ids_host, blt_tensor *out) {
+    BLT_REQUIRE(table != NULL && ids_host != NULL && out != NULL, "blt_embedding_lookup: arguments cannot be NULL");
+    BLT_REQUIRE(table->backend == BLT_BACKEND_HIP && out->backend == BLT_BACKEND_HIP,
+                "blt_embedding_lookup: HIP implementation called with non-HIP tensors");
+    BLT_REQUIRE(table->ndim == 2 && out->ndim == 2 && table->dtype == BLT_DTYPE_FP32 && out->dtype == BLT_DTYPE_FP32,
+                "blt_embedding_lookup: table and out must be 2D FP32 tensors");
+    BLT_REQUIRE(table->shape[1] == out->shape[1], "blt_embedding_lookup: embed_dim mismatch");
+    const size_t rows = out->shape[0];
+    size_t *pos = (size_t *)malloc((rows ? rows : 1) * sizeof(size_t));
+    BLT_REQUIRE(pos != NULL, "blt_embedding_lookup: out of host memory");
+    for (size_t i = 0; i < rows; i++) {
+        BLT_REQUIRE(ids_host[i] < table->shape[0], "blt_embedding_lookup: id out of range");
+        pos[i] = ids_host[i];
+    }
+    blt_rows_gather_hip(table, pos, out);
+    free(pos);
 }
 
 extern "C" void blt_softmax_masked_row_inplace_hip(blt_backend backend, float *row, size_t row_len, size_t row_idx,

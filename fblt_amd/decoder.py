@@ -35,7 +35,10 @@ def random_weights(E, hidden, L, V, seed):
             else:
                 w[name] = (rs.randn(*shape) / np.sqrt(shape[0])).astype(np.float32)
         layers.append(w)
-    return {"layers": layers, "lm_head_weight": (rs.randn(E, V) / np.sqrt(E)).astype(np.float32)}
+    lm_head = (rs.randn(E, V) / np.sqrt(E)).astype(np.float32)
+    # drawn last, so that the weights above are what they were before the table existed
+    d0_embed = (0.5 * rs.randn(257, E)).astype(np.float32)   # [BLT_D0_VOCAB, E], local_decoder.h:40
+    return {"layers": layers, "lm_head_weight": lm_head, "d0_embed_weight": d0_embed}
 
 
 class BoundDecoder:
@@ -74,6 +77,8 @@ def bind(weights, rope_cos, rope_sin, backend, place, E, H, XH, hidden, V, max_s
     dec.rope_cos_cache, dec.rope_sin_cache = tensor(rope_cos), tensor(rope_sin)
     dec.layers = C.cast(layers, C.POINTER(abi.BltLocalLayerStorage))
     dec.lm_head_weight = tensor(weights["lm_head_weight"])
+    if "d0_embed_weight" in weights:
+        dec.d0_embed_weight = tensor(weights["d0_embed_weight"])
     return BoundDecoder(dec, layers, keep)
 
 
@@ -107,6 +112,32 @@ class HostCache:
             setattr(c, name, C.cast(self.handles[name], C.POINTER(abi.BltTensor)))
         c.cached_patches = C.cast(self.patch_table, C.POINTER(abi.BltPatchInfo))
         self.struct, self.bound = c, bound
+
+    @property
+    def ptr(self):
+        return C.pointer(self.struct)
+
+
+class BlockBatch:
+    """A blt_block_batch for the inference forward (csrc/models/block_diffusion.h:37-86,
+    filled as csrc/infer/block_generation.c:171-215 fills it): R block rows behind num_clean
+    clean rows; tokens / positions / groups as given (defaults: all [MASK], positions
+    num_clean + r, every row on the last latent)."""
+
+    def __init__(self, num_clean, R, num_patches, tokens=None, positions=None, groups=None, trailing_closed=1,
+                 num_blocks=1):
+        self.tokens = (C.c_uint32 * R)(*(tokens if tokens is not None else [abi.BLT_MASK_TOKEN_ID] * R))
+        self.positions = (C.c_size_t * R)(*(positions if positions is not None else range(num_clean, num_clean + R)))
+        self.groups = (C.c_size_t * R)(*(groups if groups is not None else [num_patches - 1] * R))
+        self.masked = (C.c_uint8 * R)(*([1] * R))
+        self.valid = (C.c_uint8 * R)(*([1] * R))
+        self.targets = (C.c_uint8 * R)()
+        b = abi.BltBlockBatch()
+        b.num_clean, b.block_size, b.num_blocks, b.n_block_rows = num_clean, R // num_blocks, num_blocks, R
+        b.tokens, b.positions, b.groups = self.tokens, self.positions, self.groups
+        b.targets, b.cell_valid, b.cell_masked = self.targets, self.valid, self.masked
+        b.trailing_closed = trailing_closed
+        self.struct = b
 
     @property
     def ptr(self):

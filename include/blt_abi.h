@@ -253,6 +253,37 @@ typedef struct {
     blt_patch_info *cached_patches; /* [batch_size*max_seq_len] boundary snapshot */
 } blt_kv_cache;
 
+/* csrc/models/local_decoder.h:42-46 */
+typedef enum {
+    BLT_D0_HFINAL = 0, /* every row of byte_hidden_in is a real encoder state */
+    BLT_D0_ZEROS,      /* block rows start from zero vectors */
+    BLT_D0_LEARNED     /* block rows read d0_embed_weight[token] */
+} blt_d0_mode;
+
+#define BLT_MASK_TOKEN_ID 256u /* csrc/models/block_diffusion.h:32 */
+
+/* csrc/models/block_diffusion.h:37-86: the block section behind a clean prefix.  The inference
+ * forward reads num_clean, n_block_rows, block_size, num_blocks, tokens, positions, groups and
+ * trailing_closed; the rest belongs to the training loss. */
+typedef struct {
+    size_t num_clean;
+    size_t block_size;
+    size_t num_blocks;
+    size_t n_block_rows;
+    float t;
+    uint32_t *tokens;     /* [n_block_rows] byte value or BLT_MASK_TOKEN_ID */
+    size_t *positions;    /* [n_block_rows] byte position of every block row (rotary tables) */
+    uint8_t *targets;
+    uint8_t *cell_valid;
+    uint8_t *cell_masked;
+    size_t *groups;       /* [n_block_rows] latent patch the row cross-attends */
+    float loss_scale;
+    float last_row_scale;
+    int clean_sum;
+    int mask_norm;
+    int trailing_closed;  /* the last clean byte closes its patch and reads the last latent */
+} blt_block_batch;
+
 #ifdef __cplusplus
 }
 #define BLT_ABI_ASSERT(c, m) static_assert(c, m)
@@ -294,5 +325,9 @@ BLT_ABI_ASSERT(sizeof(blt_local_decoder) == 512 && offsetof(blt_local_decoder, l
 BLT_ABI_ASSERT(sizeof(blt_kv_cache) == 112 && offsetof(blt_kv_cache, self_len) == 72 &&
                    offsetof(blt_kv_cache, cached_patches) == 104,
                "blt_kv_cache layout");
+
+BLT_ABI_ASSERT(sizeof(blt_block_batch) == 112 && offsetof(blt_block_batch, tokens) == 40 &&
+                   offsetof(blt_block_batch, groups) == 80 && offsetof(blt_block_batch, trailing_closed) == 104,
+               "blt_block_batch layout");
 
 #endif /* FBLT_AMD_BLT_ABI_H */

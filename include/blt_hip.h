@@ -58,6 +58,9 @@ void blt_strided_copy_hip(blt_backend backend, float *dst, size_t dst_stride, co
  * copies; pos_host is a HOST array (the rotary-table gather of the KV step,
  * csrc/infer/rope_gather.c:33-34).  No allocation, no synchronisation. */
 void blt_rows_gather_hip(const blt_tensor *src, const size_t *pos_host, blt_tensor *dst);
+/* csrc/ops/gather_scatter.h:21 (gather_scatter_cpu.c:7-21): out[i, :] = table[ids_host[i], :]; the
+ * diffusion forward's learned D_0 rows (csrc/models/block_diffusion.c:140-146) */
+void blt_embedding_lookup_hip(const blt_tensor *table, const uint32_t *ids_host, blt_tensor *out);
 
 /* Replaces blt_softmax_masked_row_inplace_cuda (csrc/ops/vecmath.cu:71-114):
  * the row softmax of csrc/ops/vecmath.h:20-31 on one device row. */
@@ -175,6 +178,7 @@ void blt_softmax_masked_row_inplace(blt_backend backend, float *row, size_t row_
 float blt_vec_dot(blt_backend backend, const float *a, const float *b, size_t n);
 /* csrc/core/backend.c:532-534: the backend comes from src. */
 void blt_rows_gather(const blt_tensor *src, const size_t *pos_host, blt_tensor *dst);
+void blt_embedding_lookup(const blt_tensor *table, const uint32_t *ids_host, blt_tensor *out);
 /* csrc/infer/rope_gather.h / rope_gather.c:5-35: rows positions[0..n) of the two rotary
  * tables into new [n, half] tensors of the arena. */
 void blt_rope_position_gather(const blt_tensor *cos_cache, const blt_tensor *sin_cache, const size_t *positions,
@@ -218,6 +222,10 @@ void blt_kv_cache_refresh_cross(blt_kv_cache *cache, const blt_tensor *patch_in,
 void blt_kv_decode_step(blt_kv_cache *cache, const blt_tensor *patch_in, const blt_patch_info *patches,
                         size_t num_patches, const blt_tensor *d0_rows, int trailing_closed, blt_tensor *logits_out,
                         blt_arena *arena);
+void blt_local_decoder_forward_diffusion_infer(const blt_local_decoder *model, const blt_tensor *byte_hidden_in,
+                                               const blt_tensor *patch_in, const blt_patch_info *patches,
+                                               size_t num_patches, const blt_block_batch *batch, blt_d0_mode d0_mode,
+                                               blt_tensor *logits_out, blt_arena *arena);
 bool blt_local_cross_attn_fires(blt_xattn_placement placement, bool cross_attn_all_layers, size_t num_layers,
                                 size_t layer);
 
@@ -410,6 +418,33 @@ void blt_kv_cache_refresh_cross_seq_hip(blt_kv_cache *cache, size_t seq, const b
 void blt_kv_decode_step_batched_hip(blt_kv_cache *cache, size_t *self_len, const blt_patch_info *const *patches,
                                     const size_t *num_patches, const int *trailing_closed, const blt_tensor *d0_rows,
                                     blt_tensor *logits_out, blt_arena *arena);
+
+/* csrc/models/block_diffusion.h:131-134 (block_diffusion.c:776-795): the inference-mode diffusion
+ * forward over [clean prefix ; block rows] -- the call blt_draft_block makes once per denoising
+ * pass (csrc/infer/block_generation.c:156-266).  Same parameter list; every tensor and the arena
+ * in device memory; logits_out is [num_clean + n_block_rows, vocab_size].  The reference runs all
+ * S rows through S x S attention against the dense INFER mask; here the clean rows are the
+ * incremental decoder step over an empty cache (a clean row never sees a block row,
+ * csrc/ops/mask_builder_cpu.c:128-131) and the block rows one block step over what it cached
+ * (133-135) -- the same arithmetic per row, projections in their summation order above 32 rows
+ * apart.  At most 32 block rows (the reference's BLT_BLOCKGEN_MAX_B).  As in the reference the
+ * decoder's local_window plays no part. */
+void blt_local_decoder_forward_diffusion_infer_hip(const blt_local_decoder *model, const blt_tensor *byte_hidden_in,
+                                                   const blt_tensor *patch_in, const blt_patch_info *patches,
+                                                   size_t num_patches, const blt_block_batch *batch,
+                                                   blt_d0_mode d0_mode, blt_tensor *logits_out, blt_arena *arena);
+
+/* The block rows of that forward over a cache that already holds the clean prefix (sequence 0:
+ * cache->self_len == batch->num_clean rows, tier 2 refreshed for num_patches patches): what a
+ * denoising pass needs when the prefix was decoded through blt_kv_decode_step, without
+ * recomputing it -- the cost of a pass no longer depends on the prefix length beyond reading its
+ * K and V once.  logits_out is [n_block_rows, vocab_size]; row r cross-attends latent
+ * batch->groups[r], sits at rotary position batch->positions[r] and starts from zeros or from
+ * d0_embed_weight[batch->tokens[r]].  Nothing is committed: the cache's lengths stay, rows past
+ * self_len are scratch.  No counterpart in the reference, whose draft loop recomputes the prefix
+ * on every pass. */
+void blt_kv_block_step_hip(blt_kv_cache *cache, size_t num_patches, const blt_block_batch *batch, blt_d0_mode d0_mode,
+                           blt_tensor *logits_out, blt_arena *arena);
 
 /* The stream every launch, asynchronous copy and memset of the library goes
  * to, per calling thread: the null stream (the reference's behaviour) unless

@@ -103,6 +103,13 @@ def load_oracle():
     lib.orc_kv_decode_step.restype = C.c_int
     lib.orc_kv_decode_step.argtypes = [C.POINTER(abi.BltKvCache), C.c_size_t, C.c_size_t,
                                        C.POINTER(abi.BltPatchInfo), C.c_size_t, _fp, C.c_size_t, C.c_int, _fp]
+    lib.orc_local_decoder_forward_diffusion_infer.restype = C.c_int
+    lib.orc_local_decoder_forward_diffusion_infer.argtypes = [C.POINTER(abi.BltLocalDecoder), _fp, _fp,
+                                                              C.POINTER(abi.BltPatchInfo), C.c_size_t,
+                                                              C.POINTER(abi.BltBlockBatch), C.c_int, _fp]
+    lib.orc_kv_block_step.restype = C.c_int
+    lib.orc_kv_block_step.argtypes = [C.POINTER(abi.BltKvCache), C.c_size_t, C.c_size_t, C.c_size_t,
+                                      C.POINTER(abi.BltBlockBatch), C.c_int, _fp]
     lib.orc_kv_rope_attend_step.restype = C.c_int
     lib.orc_kv_rope_attend_step.argtypes = [_fp, _fp] + [C.c_size_t] * 7 + [_fp, C.c_size_t, _fp, C.c_size_t, _fp,
                                                                            C.c_size_t, _fp, _fp, C.c_size_t, _fp]
@@ -195,6 +202,12 @@ def load_ref():
     lib.blt_local_decoder_forward_ext.argtypes = [C.POINTER(abi.BltLocalDecoder), T, T, C.POINTER(abi.BltPatchInfo),
                                                   C.c_size_t, T, T, abi.c_size_p, C.c_size_t, C.c_void_p, C.c_int, T,
                                                   T, C.POINTER(abi.BltArena)]
+    if hasattr(lib, "blt_local_decoder_forward_diffusion_infer"):   # csrc/models/block_diffusion.h:131-134
+        lib.blt_local_decoder_forward_diffusion_infer.restype = None
+        lib.blt_local_decoder_forward_diffusion_infer.argtypes = [C.POINTER(abi.BltLocalDecoder), T, T,
+                                                                  C.POINTER(abi.BltPatchInfo), C.c_size_t,
+                                                                  C.POINTER(abi.BltBlockBatch), C.c_int, T,
+                                                                  C.POINTER(abi.BltArena)]
     lib.blt_build_block_diffusion_mask.restype = None
     lib.blt_build_block_diffusion_mask.argtypes = [C.POINTER(abi.BltBlockDiffusionConfig),
                                                    C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)]
@@ -241,6 +254,10 @@ def load_ref_callers():
     lib.blt_kv_cache_refresh_cross.argtypes = [K, T, P, C.c_size_t, C.c_size_t, A]
     lib.blt_kv_decode_step.restype = None
     lib.blt_kv_decode_step.argtypes = [K, T, P, C.c_size_t, T, C.c_int, T, A]
+    if hasattr(lib, "blt_local_decoder_forward_diffusion_infer"):
+        lib.blt_local_decoder_forward_diffusion_infer.restype = None
+        lib.blt_local_decoder_forward_diffusion_infer.argtypes = [C.POINTER(abi.BltLocalDecoder), T, T, P, C.c_size_t,
+                                                                  C.POINTER(abi.BltBlockBatch), C.c_int, T, A]
     return lib
 
 

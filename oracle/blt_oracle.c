@@ -277,6 +277,15 @@ void orc_kv_cross_mask(float *out, const size_t *q_ids, size_t n, const size_t *
 int orc_kv_attend_step(float *self_k, float *self_v, size_t max_seq_len, size_t E, size_t H, size_t b,
                        size_t base, size_t n, size_t window, const float *q_rows, const float *k_rows,
                        const float *v_rows, float *combined) {
+    return orc_kv_attend_step_kind(self_k, self_v, max_seq_len, E, H, b, base, n, window, 0, q_rows, k_rows, v_rows,
+                                   combined);
+}
+
+/* The same statements; block_kind != 0: every new row sees all base + n keys, the rows of a single
+ * live block under the INFER rule (csrc/ops/mask_builder_cpu.c:133-135), cached prefix included. */
+int orc_kv_attend_step_kind(float *self_k, float *self_v, size_t max_seq_len, size_t E, size_t H, size_t b,
+                            size_t base, size_t n, size_t window, int block_kind, const float *q_rows,
+                            const float *k_rows, const float *v_rows, float *combined) {
     const size_t total = base + n;
     if (total > max_seq_len) return ORC_ERR_CAPACITY;
     const size_t hd = E / H;
@@ -291,7 +300,11 @@ int orc_kv_attend_step(float *self_k, float *self_v, size_t max_seq_len, size_t 
 
     float *mask = (float *)malloc(n * total * sizeof(float));
     float *scratch = (float *)malloc(n * total * sizeof(float));
-    orc_kv_self_mask(mask, n, base, window);
+    if (block_kind) {
+        for (size_t e = 0; e < n * total; e++) mask[e] = 0.0f;
+    } else {
+        orc_kv_self_mask(mask, n, base, window);
+    }
     memset(combined, 0, n * E * sizeof(float));
 
     int rc = ORC_OK;
@@ -376,6 +389,19 @@ int orc_kv_rope_attend_step(float *self_k, float *self_v, size_t max_seq_len, si
                             size_t base, size_t n, size_t window, const float *q_rows, size_t q_stride,
                             const float *k_rows, size_t k_stride, const float *v_rows, size_t v_stride,
                             const float *cos_cache, const float *sin_cache, size_t cache_rows, float *combined) {
+    return orc_kv_rope_attend_step_kind(self_k, self_v, max_seq_len, E, H, b, base, n, window, 0, NULL, q_rows,
+                                        q_stride, k_rows, k_stride, v_rows, v_stride, cos_cache, sin_cache,
+                                        cache_rows, combined);
+}
+
+/* The same with the step kind of orc_kv_attend_step_kind and, when row_positions is given, the
+ * rotary position of every new row taken from it (block rows carry their own positions,
+ * csrc/models/block_diffusion.c:148-157) instead of base + r. */
+int orc_kv_rope_attend_step_kind(float *self_k, float *self_v, size_t max_seq_len, size_t E, size_t H, size_t b,
+                                 size_t base, size_t n, size_t window, int block_kind, const size_t *row_positions,
+                                 const float *q_rows, size_t q_stride, const float *k_rows, size_t k_stride,
+                                 const float *v_rows, size_t v_stride, const float *cos_cache,
+                                 const float *sin_cache, size_t cache_rows, float *combined) {
     if (base + n > max_seq_len) return ORC_ERR_CAPACITY;
     const size_t hd = E / H, half = hd / 2;
     size_t *positions = (size_t *)malloc(n * sizeof(size_t));
@@ -388,7 +414,7 @@ int orc_kv_rope_attend_step(float *self_k, float *self_v, size_t max_seq_len, si
     float *q_full = (float *)malloc(n * E * sizeof(float));
     float *k_full = (float *)malloc(n * E * sizeof(float));
     float *v_full = (float *)malloc(n * E * sizeof(float));
-    for (size_t r = 0; r < n; r++) positions[r] = base + r;
+    for (size_t r = 0; r < n; r++) positions[r] = row_positions ? row_positions[r] : base + r;
     int rcode = orc_rope_position_gather(cos_cache, sin_cache, cache_rows, half, positions, n, rc, rs);
     if (rcode == ORC_OK) {
         for (size_t h = 0; h < H; h++) {
@@ -400,8 +426,8 @@ int orc_kv_rope_attend_step(float *self_k, float *self_v, size_t max_seq_len, si
             orc_strided_copy(k_full + h * hd, E, k_rot, hd, n, hd);
             orc_strided_copy(v_full + h * hd, E, v_rows + h * hd, v_stride, n, hd);
         }
-        rcode = orc_kv_attend_step(self_k, self_v, max_seq_len, E, H, b, base, n, window, q_full, k_full, v_full,
-                                   combined);
+        rcode = orc_kv_attend_step_kind(self_k, self_v, max_seq_len, E, H, b, base, n, window, block_kind, q_full,
+                                        k_full, v_full, combined);
     }
     free(positions), free(rc), free(rs), free(q_head), free(k_head), free(q_rot), free(k_rot);
     free(q_full), free(k_full), free(v_full);
@@ -531,6 +557,17 @@ int orc_kv_decode_layer(float *self_k, float *self_v, size_t max_seq_len, size_t
                         const float *norm2_w, const float *up_w, const float *gate_w, const float *down_w,
                         size_t hidden, const float *cos_cache, const float *sin_cache, size_t cache_rows,
                         const float *rows_in, float *rows_out) {
+    return orc_kv_decode_layer_kind(self_k, self_v, max_seq_len, E, H, b, base, n, window, 0, NULL, norm1_w, qkv_w,
+                                    proj_w, norm2_w, up_w, gate_w, down_w, hidden, cos_cache, sin_cache, cache_rows,
+                                    rows_in, rows_out);
+}
+
+int orc_kv_decode_layer_kind(float *self_k, float *self_v, size_t max_seq_len, size_t E, size_t H, size_t b,
+                             size_t base, size_t n, size_t window, int block_kind, const size_t *row_positions,
+                             const float *norm1_w, const float *qkv_w, const float *proj_w, const float *norm2_w,
+                             const float *up_w, const float *gate_w, const float *down_w, size_t hidden,
+                             const float *cos_cache, const float *sin_cache, size_t cache_rows, const float *rows_in,
+                             float *rows_out) {
     float *normed = (float *)malloc(n * E * sizeof(float));
     float *qkv = (float *)malloc(n * 3 * E * sizeof(float));
     float *combined = (float *)malloc(n * E * sizeof(float));
@@ -541,8 +578,9 @@ int orc_kv_decode_layer(float *self_k, float *self_v, size_t max_seq_len, size_t
     float *act = (float *)malloc(n * hidden * sizeof(float));
     orc_rmsnorm_forward(rows_in, norm1_w, normed, n, E);
     orc_matmul(normed, qkv_w, qkv, n, E, 3 * E);
-    int rc = orc_kv_rope_attend_step(self_k, self_v, max_seq_len, E, H, b, base, n, window, qkv, 3 * E, qkv + E,
-                                     3 * E, qkv + 2 * E, 3 * E, cos_cache, sin_cache, cache_rows, combined);
+    int rc = orc_kv_rope_attend_step_kind(self_k, self_v, max_seq_len, E, H, b, base, n, window, block_kind,
+                                          row_positions, qkv, 3 * E, qkv + E, 3 * E, qkv + 2 * E, 3 * E, cos_cache,
+                                          sin_cache, cache_rows, combined);
     if (rc == ORC_OK) {
         orc_matmul(combined, proj_w, attn_out, n, E, E);
         orc_add(rows_in, attn_out, resid1, n * E);
@@ -720,5 +758,180 @@ int orc_kv_decode_step(blt_kv_cache *cache, size_t b, size_t base, const blt_pat
     }
     if (rc == ORC_OK) orc_matmul(cur, (const float *)dec->lm_head_weight.data, logits_out, n, E, cfg->vocab_size);
     free(q_group), free(cur), free(mid);
+    return rc;
+}
+
+/* D_0 rows of the block section (csrc/models/block_diffusion.c:137-146): zeros, or row tokens[r] of
+ * the learned table (csrc/ops/gather_scatter_cpu.c:7-29) */
+static int orc_block_d0_rows(const blt_local_decoder *dec, const blt_block_batch *batch, int d0_mode, float *rows) {
+    const size_t E = dec->config.embed_dim, R = batch->n_block_rows;
+    memset(rows, 0, R * E * sizeof(float));
+    if (d0_mode != BLT_D0_LEARNED) return ORC_OK;
+    const blt_tensor *table = &dec->d0_embed_weight;
+    if (table->data == NULL || table->ndim != 2 || table->shape[1] != E || batch->tokens == NULL) return ORC_ERR_ARG;
+    for (size_t r = 0; r < R; r++) {
+        if (batch->tokens[r] >= table->shape[0]) return ORC_ERR_ARG;
+        memcpy(rows + r * E, (const float *)table->data + (size_t)batch->tokens[r] * E, E * sizeof(float));
+    }
+    return ORC_OK;
+}
+
+/* csrc/models/block_diffusion.c:776-795: the inference-mode forward over [clean prefix ; block
+ * rows] as the reference computes it -- all S = N + R rows densely: context 110-204 (D_0, gathered
+ * rotary rows, group ids, the S x S INFER mask), layers 336-398 (cross block where it fires,
+ * self-attention 246-323 with one core call per head against the mask, feed-forward), LM head.
+ * byte_hidden is [N, E], patch_in [num_patches, patch_dim], logits_out [S, vocab]. */
+int orc_local_decoder_forward_diffusion_infer(const blt_local_decoder *dec, const float *byte_hidden,
+                                              const float *patch_in, const blt_patch_info *patches,
+                                              size_t num_patches, const blt_block_batch *batch, int d0_mode,
+                                              float *logits_out) {
+    const blt_local_decoder_config *cfg = &dec->config;
+    const size_t N = batch->num_clean, R = batch->n_block_rows, S = N + R;
+    const size_t E = cfg->embed_dim, V = cfg->vocab_size, H = cfg->num_heads, XH = cfg->cross_attn_heads;
+    const size_t hd = E / H, half = hd / 2, L = cfg->num_layers;
+    const size_t pdim = cfg->patch_dim ? cfg->patch_dim : E, k = pdim / E;
+    if (hd == 0 || hd % 2 != 0 || N < 1 || num_patches < 1) return ORC_ERR_ARG;
+    if (S < 2 || S > cfg->max_seq_len) return ORC_ERR_ARG;
+
+    float *cur = (float *)calloc(S * E, sizeof(float));
+    float *next = (float *)malloc(S * E * sizeof(float));
+    memcpy(cur, byte_hidden, N * E * sizeof(float));
+    int rc = orc_block_d0_rows(dec, batch, d0_mode, cur + N * E);
+
+    size_t *positions = (size_t *)malloc(S * sizeof(size_t));
+    for (size_t i = 0; i < N; i++) positions[i] = i;
+    for (size_t r = 0; r < R; r++) positions[N + r] = batch->positions[r];
+    float *rope_c = (float *)malloc(S * half * sizeof(float));
+    float *rope_s = (float *)malloc(S * half * sizeof(float));
+    if (rc == ORC_OK)
+        rc = orc_rope_position_gather((const float *)dec->rope_cos_cache.data, (const float *)dec->rope_sin_cache.data,
+                                      dec->rope_cos_cache.shape[0], half, positions, S, rope_c, rope_s);
+
+    size_t *q_ids = (size_t *)malloc(S * sizeof(size_t));
+    size_t *kv_ids = (size_t *)malloc(num_patches * k * sizeof(size_t));
+    for (size_t i = 0; i < N; i++) q_ids[i] = orc_patch_decoder_latent_at(patches, num_patches, i);
+    if (batch->trailing_closed) q_ids[N - 1] = num_patches - 1;
+    for (size_t r = 0; r < R; r++) q_ids[N + r] = batch->groups[r];
+    for (size_t p = 0; p < num_patches; p++)
+        for (size_t s2 = 0; s2 < k; s2++) kv_ids[p * k + s2] = p;
+
+    float *mask = (float *)malloc(S * S * sizeof(float));
+    float *weights = (float *)malloc(S * S * sizeof(float));
+    if (rc == ORC_OK) {
+        blt_block_diffusion_config mc;
+        memset(&mc, 0, sizeof(mc));
+        mc.mode = BLT_BDM_INFER, mc.seq_len = S, mc.num_clean = N, mc.block_size = batch->block_size;
+        mc.num_blocks = batch->num_blocks; /* the INFER rule reads neither block_starts nor block_size */
+        rc = orc_build_block_diffusion_mask(&mc, mask);
+    }
+
+    const size_t hidden = L ? dec->layers[0].ffn_up_w.shape[1] : 0;
+    float *normed = (float *)malloc(S * E * sizeof(float));
+    float *mid = (float *)malloc(S * E * sizeof(float));
+    float *qkv = (float *)malloc(S * 3 * E * sizeof(float));
+    float *combined = (float *)malloc(S * E * sizeof(float));
+    float *tmp = (float *)malloc(S * E * sizeof(float));
+    float *resid1 = (float *)malloc(S * E * sizeof(float));
+    float *up = (float *)malloc(S * (hidden ? hidden : 1) * sizeof(float));
+    float *gate = (float *)malloc(S * (hidden ? hidden : 1) * sizeof(float));
+    float *act = (float *)malloc(S * (hidden ? hidden : 1) * sizeof(float));
+
+    for (size_t l = 0; l < L && rc == ORC_OK; l++) {
+        const blt_local_layer_storage *s = &dec->layers[l];
+        const float *b_in = cur;
+        if (orc_local_cross_attn_fires(cfg->cross_attn_placement, cfg->cross_attn_all_layers, L, l)) {
+            blt_mask_config xm;
+            memset(&xm, 0, sizeof(xm));
+            xm.seq_len_q = S, xm.seq_len_kv = num_patches * k;
+            xm.query_group_ids = q_ids, xm.kv_group_ids = kv_ids;
+            xm.bidirectional_within_group = true, xm.is_causal = false;
+            orc_rmsnorm_forward(cur, (const float *)s->cross_norm_weight.data, normed, S, E);
+            rc = orc_cross_attention_forward(normed, patch_in, (const float *)s->cross_weight_q.data,
+                                             (const float *)s->cross_weight_k.data, (const float *)s->cross_weight_v.data,
+                                             (const float *)s->cross_weight_proj.data, tmp, S, num_patches * k, E, XH, &xm);
+            if (rc != ORC_OK) break;
+            orc_add(cur, tmp, mid, S * E);
+            b_in = mid;
+        }
+        orc_rmsnorm_forward(b_in, (const float *)s->norm1_weight.data, normed, S, E);
+        orc_matmul(normed, (const float *)s->attn_qkv_w.data, qkv, S, E, 3 * E);
+        for (size_t h = 0; h < H; h++) { /* rotate Q and K of every head in place, rows by their gathered tables */
+            orc_rope_apply_packed(qkv, 3 * E, h * hd, S, hd, rope_c, rope_s);
+            orc_rope_apply_packed(qkv, 3 * E, E + h * hd, S, hd, rope_c, rope_s);
+        }
+        memset(combined, 0, S * E * sizeof(float));
+        for (size_t h = 0; h < H && rc == ORC_OK; h++) {
+            blt_attention_head_args a;
+            memset(&a, 0, sizeof(a));
+            a.q = qkv + h * hd, a.k = qkv + E + h * hd, a.v = qkv + 2 * E + h * hd;
+            a.q_stride = a.k_stride = a.v_stride = 3 * E;
+            a.combined = combined, a.combined_stride = E, a.combined_col_offset = h * hd;
+            a.weights_out = weights;
+            a.mask = mask;
+            a.nq = S, a.nk = S, a.head_dim = hd;
+            a.is_causal = false;
+            a.scale = 1.0f / sqrtf((float)hd);
+            rc = orc_attention_head_core(&a);
+        }
+        if (rc != ORC_OK) break;
+        orc_matmul(combined, (const float *)s->attn_proj_w.data, tmp, S, E, E);
+        orc_add(b_in, tmp, resid1, S * E);
+        orc_rmsnorm_forward(resid1, (const float *)s->norm2_weight.data, normed, S, E);
+        const size_t hid = s->ffn_up_w.shape[1];
+        orc_matmul(normed, (const float *)s->ffn_up_w.data, up, S, E, hid);
+        orc_matmul(normed, (const float *)s->ffn_gate_w.data, gate, S, E, hid);
+        orc_swiglu_forward(gate, up, act, S * hid);
+        orc_matmul(act, (const float *)s->ffn_down_w.data, tmp, S, hid, E);
+        orc_add(resid1, tmp, next, S * E);
+        float *t = cur;
+        cur = next, next = t;
+    }
+    if (rc == ORC_OK) orc_matmul(cur, (const float *)dec->lm_head_weight.data, logits_out, S, E, V);
+    free(cur), free(next), free(positions), free(rope_c), free(rope_s), free(q_ids), free(kv_ids), free(mask);
+    free(weights), free(normed), free(mid), free(qkv), free(combined), free(tmp), free(resid1), free(up), free(gate);
+    free(act);
+    return rc;
+}
+
+/* The block rows of the same forward over a cache that already holds the clean prefix (`base` =
+ * num_clean valid rows of sequence b, tier 2 refreshed): the rows of
+ * orc_local_decoder_forward_diffusion_infer's logits from num_clean on, computed without touching
+ * the prefix -- a clean row never sees a block row (csrc/ops/mask_builder_cpu.c:128-131), so the
+ * prefix's K and V are what the incremental step cached, and a block row sees all of them plus the
+ * whole block (133-135).  Group of row r: batch->groups[r]; rotary row: batch->positions[r]; no
+ * window (the INFER mask has none); nothing is committed.  logits_out is [n_block_rows, vocab]. */
+int orc_kv_block_step(blt_kv_cache *cache, size_t b, size_t base, size_t num_patches, const blt_block_batch *batch,
+                      int d0_mode, float *logits_out) {
+    const blt_local_decoder *dec = cache->decoder;
+    const blt_local_decoder_config *cfg = &dec->config;
+    const size_t E = cache->embed_dim, L = cfg->num_layers, H = cfg->num_heads, XH = cfg->cross_attn_heads;
+    const size_t n = batch->n_block_rows;
+    if (n < 1 || num_patches < 1 || batch->num_clean != base) return ORC_ERR_ARG;
+    if (base + n > cache->max_seq_len || num_patches * cache->k > cache->max_subtokens) return ORC_ERR_CAPACITY;
+    float *cur = (float *)malloc(n * E * sizeof(float));
+    float *mid = (float *)malloc(n * E * sizeof(float));
+    int rc = orc_block_d0_rows(dec, batch, d0_mode, cur);
+    for (size_t l = 0; l < L && rc == ORC_OK; l++) {
+        const blt_local_layer_storage *s = &dec->layers[l];
+        const float *in = cur;
+        if (orc_local_cross_attn_fires(cfg->cross_attn_placement, cfg->cross_attn_all_layers, L, l)) {
+            rc = orc_kv_cross_block((const float *)cache->cross_k[l].data, (const float *)cache->cross_v[l].data,
+                                    cache->max_subtokens, E, XH, b, num_patches * cache->k, cache->k, batch->groups, n,
+                                    (const float *)s->cross_norm_weight.data, (const float *)s->cross_weight_q.data,
+                                    (const float *)s->cross_weight_proj.data, cur, mid);
+            in = mid;
+        }
+        if (rc != ORC_OK) break;
+        rc = orc_kv_decode_layer_kind((float *)cache->self_k[l].data, (float *)cache->self_v[l].data,
+                                      cache->max_seq_len, E, H, b, base, n, 0, 1, batch->positions,
+                                      (const float *)s->norm1_weight.data, (const float *)s->attn_qkv_w.data,
+                                      (const float *)s->attn_proj_w.data, (const float *)s->norm2_weight.data,
+                                      (const float *)s->ffn_up_w.data, (const float *)s->ffn_gate_w.data,
+                                      (const float *)s->ffn_down_w.data, s->ffn_up_w.shape[1],
+                                      (const float *)dec->rope_cos_cache.data, (const float *)dec->rope_sin_cache.data,
+                                      dec->rope_cos_cache.shape[0], in, cur);
+    }
+    if (rc == ORC_OK) orc_matmul(cur, (const float *)dec->lm_head_weight.data, logits_out, n, E, cfg->vocab_size);
+    free(cur), free(mid);
     return rc;
 }

@@ -240,6 +240,36 @@ int orc_kv_decode_step(blt_kv_cache *cache, size_t b, size_t base, const blt_pat
                        size_t num_patches, const float *d0_rows, size_t n, int trailing_closed,
                        float *logits_out);
 
+/* The KV step statements with the step kind (block_kind != 0: every new row sees all keys, the
+ * INFER rule of ops/mask_builder_cpu.c:133-135) and optional rotary positions of the new rows. */
+int orc_kv_attend_step_kind(float *self_k, float *self_v, size_t max_seq_len, size_t E, size_t H, size_t b,
+                            size_t base, size_t n, size_t window, int block_kind, const float *q_rows,
+                            const float *k_rows, const float *v_rows, float *combined);
+int orc_kv_rope_attend_step_kind(float *self_k, float *self_v, size_t max_seq_len, size_t E, size_t H, size_t b,
+                                 size_t base, size_t n, size_t window, int block_kind, const size_t *row_positions,
+                                 const float *q_rows, size_t q_stride, const float *k_rows, size_t k_stride,
+                                 const float *v_rows, size_t v_stride, const float *cos_cache,
+                                 const float *sin_cache, size_t cache_rows, float *combined);
+int orc_kv_decode_layer_kind(float *self_k, float *self_v, size_t max_seq_len, size_t E, size_t H, size_t b,
+                             size_t base, size_t n, size_t window, int block_kind, const size_t *row_positions,
+                             const float *norm1_w, const float *qkv_w, const float *proj_w, const float *norm2_w,
+                             const float *up_w, const float *gate_w, const float *down_w, size_t hidden,
+                             const float *cos_cache, const float *sin_cache, size_t cache_rows, const float *rows_in,
+                             float *rows_out);
+
+/* models/block_diffusion.c:776-795 (context 110-204, self-attention 246-323, layers 336-398): the
+ * inference-mode diffusion forward over [clean prefix ; block rows], all rows densely.
+ * byte_hidden [num_clean, E], patch_in [num_patches, patch_dim], logits_out [S, vocab]. */
+int orc_local_decoder_forward_diffusion_infer(const blt_local_decoder *dec, const float *byte_hidden,
+                                              const float *patch_in, const blt_patch_info *patches,
+                                              size_t num_patches, const blt_block_batch *batch, int d0_mode,
+                                              float *logits_out);
+
+/* The block rows of that forward over a host cache holding the clean prefix of sequence b (`base`
+ * = num_clean rows, tier 2 refreshed); logits_out [n_block_rows, vocab]; nothing is committed. */
+int orc_kv_block_step(blt_kv_cache *cache, size_t b, size_t base, size_t num_patches, const blt_block_batch *batch,
+                      int d0_mode, float *logits_out);
+
 #ifdef __cplusplus
 }
 #endif

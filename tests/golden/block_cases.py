@@ -24,6 +24,19 @@ STEP_CASES = {
 }
 STEP_SCRIPT = [([3, 4], 0, 7, 0), ([3, 4, 1], 2, 1, 0), ([3, 4, 2], 2, 1, 1), ([3, 4, 2, 5], 3, 5, 0),
                ([3, 4, 2, 5, 1], 4, 1, 0), ([3, 4, 2, 5, 4], 4, 3, 1), ([3, 4, 2, 5, 4, 3], 5, 3, 0)]
+# inference-mode diffusion forward: decoder configuration, patch lengths of the clean prefix, block
+# rows, trailing_closed, learned D_0 table or zeros, "draft" (all [MASK], positions N + r, every row
+# on the last latent -- csrc/infer/block_generation.c:171-215) or "mixed" (seeded tokens, positions
+# and groups)
+DIFFUSION_CASES = {
+    "diff_E64_k2_draft_B8": dict(E=64, H=2, XH=2, L=2, hidden=96, V=64, max_len=80, k=2, window=9, all_layers=True,
+                                 placement=0, lengths=[5, 9, 3, 12, 7], R=8, closed=1, learned=True, fill="draft"),
+    "diff_E32_last_mixed_B4": dict(E=32, H=4, XH=1, L=3, hidden=48, V=256, max_len=48, k=1, window=0,
+                                   all_layers=False, placement=0, lengths=[4, 6, 5], R=4, closed=0, learned=True,
+                                   fill="mixed"),
+    "diff_E128_zeros_B16": dict(E=128, H=4, XH=4, L=2, hidden=256, V=256, max_len=128, k=1, window=0, all_layers=True,
+                                placement=0, lengths=[16, 9, 20, 11, 14], R=16, closed=1, learned=False, fill="draft"),
+}
 THETA = 500000.0
 
 
@@ -75,3 +88,22 @@ def step_inputs(name):
         latents.append(pin)
         prev = pin
     return c, weights, d0, latents
+
+
+def diffusion_inputs(name):
+    """Decoder weights, clean-row states, patch latents and the block section of a diffusion case."""
+    c = DIFFUSION_CASES[name]
+    rs = np.random.RandomState(seed_of(name))
+    weights = decoder.random_weights(c["E"], c["hidden"], c["L"], c["V"], seed_of(name) + 1)
+    N, P, R = sum(c["lengths"]), len(c["lengths"]), c["R"]
+    hidden = rs.randn(N, c["E"]).astype(np.float32)
+    latents = rs.randn(P, c["k"] * c["E"]).astype(np.float32)
+    if c["fill"] == "draft":
+        batch = decoder.BlockBatch(N, R, P, trailing_closed=c["closed"])
+    else:
+        tokens = [int(rs.randint(0, 256)) if rs.rand() < 0.5 else 256 for _ in range(R)]
+        positions = [int(x) for x in np.sort(rs.randint(0, c["max_len"], size=R))]
+        groups = [int(rs.randint(0, P)) for _ in range(R)]
+        batch = decoder.BlockBatch(N, R, P, tokens=tokens, positions=positions, groups=groups,
+                                   trailing_closed=c["closed"])
+    return c, weights, hidden, latents, batch

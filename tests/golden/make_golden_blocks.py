@@ -1,6 +1,7 @@
 """Writes tests/golden/blocks_golden.npz from the reference build (oracle/_ref):
-blt_multihead_attention, blt_cross_attention_forward and the script of
-blt_kv_cache_refresh_cross + blt_kv_decode_step calls of block_cases.py.
+blt_multihead_attention, blt_cross_attention_forward, the script of
+blt_kv_cache_refresh_cross + blt_kv_decode_step calls and the
+blt_local_decoder_forward_diffusion_infer cases of block_cases.py.
 
 Run in a container that holds the reference sources:
     make -C oracle ref && python tests/golden/make_golden_blocks.py
@@ -108,6 +109,23 @@ def run_step(ref, arena, name):
     return np.concatenate(logits), tiers
 
 
+def run_diffusion(ref, arena, name):
+    c, weights, hidden, latents, batch = bc.diffusion_inputs(name)
+    E, V = c["E"], c["V"]
+    cos, sin = rope_tables(ref, c["max_len"], E // c["H"])
+    bound = decoder.bind(weights, cos, sin, CPU, decoder.host_place, E, c["H"], c["XH"], c["hidden"], V, c["max_len"],
+                         patch_dim=c["k"] * E, window=c["window"], all_layers=c["all_layers"],
+                         placement=c["placement"], theta=bc.THETA)
+    N, P = sum(c["lengths"]), len(c["lengths"])
+    out = np.zeros((N + c["R"], V), dtype=np.float32)
+    th, tp, tl = view(hidden), view(latents), view(out)
+    arena.contents.offset = 0
+    ref.blt_local_decoder_forward_diffusion_infer(bound.ptr, C.byref(th), C.byref(tp), decoder.patch_table(c["lengths"]),
+                                                  P, batch.ptr, abi.BLT_D0_LEARNED if c["learned"] else abi.BLT_D0_ZEROS,
+                                                  C.byref(tl), arena)
+    return out
+
+
 def main():
     ref = binding.load_ref()
     if ref is None:
@@ -124,6 +142,8 @@ def main():
         pack(store, name + "/logits", logits, rs)
         for tier, arr in tiers.items():
             pack(store, name + "/" + tier, arr, rs)
+    for name in bc.DIFFUSION_CASES:
+        pack(store, name + "/logits", run_diffusion(ref, arena, name), rs)
     ref.blt_arena_destroy(arena)
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "blocks_golden.npz")
     np.savez_compressed(path, **store)

@@ -39,7 +39,7 @@ def test_summary_line_stays_short_with_every_workload_present():
     """The driver keeps a bounded tail of stdout: the line that carries metric, value, roofline and
     cpu_baseline must fit it with every workload of a full run present."""
     import bench
-    names = ["c1", "c3", "c4", "c4_rope", "c5_B4", "c5_B8", "c5_B16", "c5_chunk_causal_n16", "c1_x64", "c2_x8",
+    names = ["c1", "c3", "c4", "c4_host_lens", "c4_b128_L2048_host_lens", "draft_pass", "c4_rope", "c5_B4", "c5_B8", "c5_B16", "c5_chunk_causal_n16", "c1_x64", "c2_x8",
              "c1_T4096", "c2_P2048", "c4_b128_L2048", "c5_B16_b128_L2048", "mha_c1", "xattn_c3", "mha_c2",
              "matmul_8192x512x1536", "decode_layer", "decode_step", "decode_step_b1", "decode_step_prefill_512",
              "mask_c1_causal_512", "mask_c3_patch_groups_128x512", "mask_c5_block_infer_524", "mask_causal_window_4096"]

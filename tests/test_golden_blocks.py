@@ -1,6 +1,6 @@
 """Golden vectors of the block-level entry points, written by tests/golden/make_golden_blocks.py
-from the reference build: blt_multihead_attention, blt_cross_attention_forward and a script of
-blt_kv_cache_refresh_cross + blt_kv_decode_step calls.  CPU: the checker reproduces every output
+from the reference build: blt_multihead_attention, blt_cross_attention_forward, a script of
+blt_kv_cache_refresh_cross + blt_kv_decode_step calls and blt_local_decoder_forward_diffusion_infer.  CPU: the checker reproduces every output
 bit for bit (SHA-256).  GPU: the HIP library matches the stored samples within
 |got - ref| <= 1e-5 + 1e-4 |ref|."""
 import ctypes as C
@@ -99,6 +99,37 @@ def test_oracle_reproduces_reference_decoder_steps(name, oracle):
         check(np.stack(cache.tiers[tier]), name + "/" + tier, exact=True)
 
 
+def _diffusion_decoder(oracle, c, weights, backend, place):
+    cos, sin = host_tables(oracle, c["max_len"], c["E"] // c["H"])
+    return decoder.bind(weights, cos, sin, backend, place, c["E"], c["H"], c["XH"], c["hidden"], c["V"], c["max_len"],
+                        patch_dim=c["k"] * c["E"], window=c["window"], all_layers=c["all_layers"],
+                        placement=c["placement"], theta=bc.THETA)
+
+
+@pytest.mark.parametrize("name", list(bc.DIFFUSION_CASES))
+def test_oracle_reproduces_reference_diffusion_forward(name, oracle):
+    """The dense restatement, and the cached form (prefix through the incremental step without a
+    window, block rows through the block step), both bit for bit what the reference build wrote."""
+    c, weights, hidden, latents, batch = bc.diffusion_inputs(name)
+    bound = _diffusion_decoder(oracle, c, weights, CPU, decoder.host_place)
+    N, P, R, V = sum(c["lengths"]), len(c["lengths"]), c["R"], c["V"]
+    mode = abi.BLT_D0_LEARNED if c["learned"] else abi.BLT_D0_ZEROS
+    patches = decoder.patch_table(c["lengths"])
+    out = np.zeros((N + R, V), dtype=np.float32)
+    assert oracle.orc_local_decoder_forward_diffusion_infer(
+        bound.ptr, binding.fptr(hidden.reshape(-1)), binding.fptr(latents.reshape(-1)), patches, P, batch.ptr, mode,
+        binding.fptr(out.reshape(-1))) == 0
+    check(out, name + "/logits", exact=True)
+    bound.struct.config.local_window = 0
+    cache = decoder.HostCache(bound, c["max_len"])
+    assert oracle.orc_kv_cache_refresh_cross(cache.ptr, 0, binding.fptr(latents.reshape(-1)), P, 0) == 0
+    two = np.zeros((N + R, V), dtype=np.float32)
+    assert oracle.orc_kv_decode_step(cache.ptr, 0, 0, patches, P, binding.fptr(hidden.reshape(-1)), N, c["closed"],
+                                     binding.fptr(two[:N].reshape(-1))) == 0
+    assert oracle.orc_kv_block_step(cache.ptr, 0, N, P, batch.ptr, mode, binding.fptr(two[N:].reshape(-1))) == 0
+    check(two, name + "/logits", exact=True)
+
+
 # ---------------------------------------------------------------------------- GPU: the library
 def dev_view(t):
     return abi.tensor_view(t.data_ptr(), tuple(t.shape), HIP)
@@ -188,3 +219,25 @@ def test_hip_matches_reference_decoder_steps(name, oracle):
         check(got, name + "/" + tier, exact=False)
     lib.blt_kv_cache_destroy(cache)
     lib.blt_arena_destroy(arena)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", list(bc.DIFFUSION_CASES))
+def test_hip_matches_reference_diffusion_forward(name, oracle):
+    import torch
+    from fblt_amd import api
+    lib = api.load()
+    c, weights, hidden, latents, batch = bc.diffusion_inputs(name)
+    bound = _diffusion_decoder(oracle, c, weights, HIP, decoder.device_place)
+    N, P, R, V = sum(c["lengths"]), len(c["lengths"]), c["R"], c["V"]
+    mode = abi.BLT_D0_LEARNED if c["learned"] else abi.BLT_D0_ZEROS
+    th, tp = torch.from_numpy(hidden).cuda(), torch.from_numpy(latents).cuda()
+    tl = torch.full((N + R, V), 7.0, dtype=torch.float32, device="cuda")
+    vh, vp, vl = dev_view(th), dev_view(tp), dev_view(tl)
+    arena = lib.blt_arena_create(128 << 20, HIP)
+    lib.blt_local_decoder_forward_diffusion_infer(bound.ptr, C.byref(vh), C.byref(vp), decoder.patch_table(c["lengths"]),
+                                                  P, batch.ptr, mode, C.byref(vl), arena)
+    lib.blt_backend_pass_sync_hip()
+    out = tl.cpu().numpy()
+    lib.blt_arena_destroy(arena)
+    check(out, name + "/logits", exact=False)

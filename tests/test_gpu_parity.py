@@ -1210,6 +1210,90 @@ def test_kv_decode_step_single_sequence(case, impl, oracle, dev):
         lib.blt_arena_destroy(arena)
 
 
+# (patch lengths of the clean prefix, block rows, trailing_closed, d0 mode, how the block is filled)
+DIFFUSION_SCRIPTS = [
+    ([3, 4, 2], 4, 1, abi.BLT_D0_ZEROS, "draft"),      # blt_draft_block's batch: all [MASK], positions N + r, o_M
+    ([3, 4, 2, 5], 8, 1, abi.BLT_D0_LEARNED, "draft"),
+    ([5, 1, 6], 3, 0, abi.BLT_D0_LEARNED, "mixed"),    # some cells unmasked, groups and positions of the caller's
+    ([2, 2, 2, 2, 3], 16, 1, abi.BLT_D0_ZEROS, "mixed"),
+    ([7], 1, 1, abi.BLT_D0_LEARNED, "draft"),
+    ([9, 8, 12, 7, 11, 3], 32, 1, abi.BLT_D0_LEARNED, "draft"),   # 50 clean rows: the prefill kernels
+    ([30, 31, 29, 33, 17], 4, 0, abi.BLT_D0_ZEROS, "mixed"),      # 140 clean rows
+]
+
+
+def _diffusion_batch(rs, N, R, P, fill, closed, max_len):
+    from fblt_amd import decoder
+    if fill == "draft":
+        return decoder.BlockBatch(N, R, P, trailing_closed=closed)
+    tokens = [int(rs.randint(0, 256)) if rs.rand() < 0.5 else abi.BLT_MASK_TOKEN_ID for _ in range(R)]
+    positions = [int(x) for x in np.sort(rs.randint(0, max_len, size=R))]
+    groups = [int(rs.randint(0, P)) for _ in range(R)]
+    return decoder.BlockBatch(N, R, P, tokens=tokens, positions=positions, groups=groups, trailing_closed=closed)
+
+
+@pytest.mark.parametrize("impl", IMPLS)
+@pytest.mark.parametrize("script", range(len(DIFFUSION_SCRIPTS)))
+@pytest.mark.parametrize("case", range(len(STEP_CASES)))
+def test_diffusion_infer_forward(case, script, impl, oracle, dev):
+    """blt_local_decoder_forward_diffusion_infer on device tensors against the restated dense
+    forward (csrc/models/block_diffusion.c:776-795): logits of all N + R rows.  impl =
+    reference_callers runs the reference's own block_diffusion.c (S x S attention through one core
+    call per head against the dense INFER mask) on this library's ops.  Then the block rows alone
+    through blt_kv_block_step_hip over a cache that blt_kv_decode_step filled with the prefix."""
+    import torch
+    from fblt_amd import decoder
+    lib = api.load()
+    entry = _entry(impl, lib)
+    c = STEP_CASES[case]
+    lengths, R, closed, d0_mode, fill = DIFFUSION_SCRIPTS[script]
+    E, V, k = c["E"], c["V"], c["k"]
+    N, P = sum(lengths), len(lengths)
+    if N + R > c["max_len"]:
+        pytest.skip("sequence longer than this decoder's tables")
+    rs = np.random.RandomState(8000 + 10 * case + script)
+    host, device = _decoders(oracle, c, 500 + case)
+    patches = decoder.patch_table(lengths)
+    hidden = rs.randn(N, E).astype(np.float32)
+    patch_in = rs.randn(P, k * E).astype(np.float32)
+    batch = _diffusion_batch(rs, N, R, P, fill, closed, c["max_len"])
+    ref = np.zeros((N + R, V), dtype=np.float32)
+    assert oracle.orc_local_decoder_forward_diffusion_infer(
+        host.ptr, binding.fptr(hidden.reshape(-1)), binding.fptr(patch_in.reshape(-1)), patches, P, batch.ptr, d0_mode,
+        binding.fptr(ref.reshape(-1))) == 0
+    arena = lib.blt_arena_create(256 << 20, abi.BLT_BACKEND_HIP)
+    try:
+        th, tp = torch.from_numpy(hidden).cuda(), torch.from_numpy(patch_in).cuda()
+        tl = torch.full((N + R, V), 7.0, dtype=torch.float32, device="cuda")
+        vh, vp, vl = _dev_tensor(th), _dev_tensor(tp), _dev_tensor(tl)
+        entry.blt_local_decoder_forward_diffusion_infer(device.ptr, C.byref(vh), C.byref(vp), patches, P, batch.ptr,
+                                                        d0_mode, C.byref(vl), arena)
+        lib.blt_backend_pass_sync_hip()
+        assert_close(tl.cpu().numpy(), ref, "diffusion forward case %d script %d" % (case, script))
+        if impl != "library":
+            return
+        # the draft loop's form: prefix decoded once through the incremental step, block rows per pass
+        device.struct.config.local_window = 0      # the diffusion forward has no window
+        lib.blt_arena_reset(arena)
+        cache = lib.blt_kv_cache_create(arena, device.ptr, c["max_len"])
+        lib.blt_kv_cache_refresh_cross(cache, C.byref(vp), patches, P, 0, arena)
+        tc = torch.zeros((N, V), dtype=torch.float32, device="cuda")
+        vc = _dev_tensor(tc)
+        lib.blt_kv_decode_step(cache, C.byref(vp), patches, P, C.byref(vh), closed, C.byref(vc), arena)
+        assert cache.contents.self_len == N
+        for _ in range(2):                         # a pass changes nothing in the cache
+            tb = torch.full((R, V), 7.0, dtype=torch.float32, device="cuda")
+            vb = _dev_tensor(tb)
+            lib.blt_kv_block_step_hip(cache, P, batch.ptr, d0_mode, C.byref(vb), arena)
+            lib.blt_backend_pass_sync_hip()
+            assert cache.contents.self_len == N
+            assert_close(tb.cpu().numpy(), ref[N:], "block step case %d script %d" % (case, script))
+        assert_close(tc.cpu().numpy(), ref[:N], "prefix step case %d script %d" % (case, script))
+        lib.blt_kv_cache_destroy(cache)
+    finally:
+        lib.blt_arena_destroy(arena)
+
+
 @pytest.mark.parametrize("window", [0, 20])
 def test_kv_decode_step_long_prefill(window, oracle, dev):
     """A prompt prefill in one call: more new rows than one step launch takes (45, then 1, then

@@ -35,11 +35,13 @@ def test_library_exports_every_declared_symbol():
 # what the reference's caller code references but this library leaves to the reference build:
 # training passes and ops of other model parts, none of them reached from the forward attention
 # blocks or the KV-cache step (csrc/models/attention.c:130-207, cross_attention.c:101-157,
-# csrc/infer/kv_cache.c:112-428)
+# csrc/infer/kv_cache.c:112-428, csrc/models/block_diffusion.c:776-795)
 OFF_PATH = {"blt_attention_head_core_backward", "blt_matmul_backward", "blt_rmsnorm_backward",
             "blt_rmsnorm_backward_add", "blt_rope_apply_packed_backward", "blt_swiglu_backward",
-            "blt_cross_entropy_forward", "blt_cross_entropy_backward", "blt_embedding_lookup", "blt_gelu_forward",
-            "blt_layernorm_forward", "blt_cast", "blt_container_alloc", "blt_tensor_view_2d", "blt_tensor_view_3d"}
+            "blt_cross_entropy_forward", "blt_cross_entropy_backward", "blt_gelu_forward",
+            "blt_layernorm_forward", "blt_cast", "blt_container_alloc", "blt_tensor_view_2d", "blt_tensor_view_3d",
+            # training side of csrc/models/block_diffusion.c (loss scaling, D_0 table gradient)
+            "blt_indexed_row_scatter_add", "blt_scale"}
 
 
 def test_reference_callers_find_their_ops_in_the_library():
@@ -96,8 +98,10 @@ int main(void) {
     O(blt_local_decoder, lm_head_weight); O(blt_local_decoder, d0_embed_weight);
     S(blt_kv_cache); O(blt_kv_cache, k); O(blt_kv_cache, self_k); O(blt_kv_cache, self_len); O(blt_kv_cache, cross_k);
     O(blt_kv_cache, cross_num_patches); O(blt_kv_cache, cached_patches);
-    printf("enum %%d %%d %%d %%d\n", (int)BLT_XATTN_FIRST, (int)BLT_DTYPE_FP32, (int)BLT_BACKEND_CPU,
-           (int)BLT_CROSS_ATTN_SPLIT_KV);
+    S(blt_block_batch); O(blt_block_batch, t); O(blt_block_batch, tokens); O(blt_block_batch, positions);
+    O(blt_block_batch, groups); O(blt_block_batch, loss_scale); O(blt_block_batch, trailing_closed);
+    printf("enum %%d %%d %%d %%d %%d %%u\n", (int)BLT_XATTN_FIRST, (int)BLT_DTYPE_FP32, (int)BLT_BACKEND_CPU,
+           (int)BLT_CROSS_ATTN_SPLIT_KV, (int)BLT_D0_LEARNED, (unsigned)BLT_MASK_TOKEN_ID);
     return 0;
 }
 """
@@ -112,7 +116,7 @@ def test_layout_matches_reference_headers(tmp_path):
     ref_inc = "\n".join('#include "%s"' % h for h in (
         "core/tensor.h", "core/allocator.h", "ops/attn_core.h", "ops/mask_builder.h", "ops/rope.h",
         "models/attention.h", "models/cross_attention.h", "models/transformer.h", "models/patcher.h",
-        "models/local_decoder.h", "infer/kv_cache.h"))
+        "models/local_decoder.h", "infer/kv_cache.h", "models/block_diffusion.h"))
     outs = []
     for tag, inc_dir, inc in (("ref", REF_ROOT, ref_inc), ("own", os.path.join(ROOT, "include"), '#include "blt_abi.h"')):
         src = tmp_path / (tag + ".c")

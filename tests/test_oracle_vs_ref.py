@@ -489,3 +489,77 @@ def test_kv_decode_step_bit_exact(case, oracle, ref):
                 at += n
     finally:
         ref.blt_arena_destroy(arena)
+
+
+# ---------------------------------------------------------------------------
+# inference-mode diffusion forward (csrc/models/block_diffusion.c:776-795)
+# ---------------------------------------------------------------------------
+# (patch lengths of the clean prefix, block rows, trailing_closed, d0 mode, how the block is filled)
+DIFFUSION_SCRIPTS = [
+    ([3, 4, 2], 4, 1, abi.BLT_D0_ZEROS, "draft"),      # blt_draft_block's batch: all [MASK], positions N + r, o_M
+    ([3, 4, 2, 5], 8, 1, abi.BLT_D0_LEARNED, "draft"),
+    ([5, 1, 6], 3, 0, abi.BLT_D0_LEARNED, "mixed"),    # some cells unmasked, groups and positions of the caller's
+    ([2, 2, 2, 2, 3], 16, 1, abi.BLT_D0_ZEROS, "mixed"),
+    ([7], 1, 1, abi.BLT_D0_LEARNED, "draft"),
+]
+
+
+def _block_batch(decoder, rs, N, R, P, fill, closed, max_len):
+    if fill == "draft":
+        return decoder.BlockBatch(N, R, P, trailing_closed=closed)
+    tokens = [int(rs.randint(0, 256)) if rs.rand() < 0.5 else abi.BLT_MASK_TOKEN_ID for _ in range(R)]
+    positions = [int(x) for x in np.sort(rs.randint(0, max_len, size=R))]
+    groups = [int(rs.randint(0, P)) for _ in range(R)]
+    return decoder.BlockBatch(N, R, P, tokens=tokens, positions=positions, groups=groups, trailing_closed=closed)
+
+
+@pytest.mark.parametrize("script", range(len(DIFFUSION_SCRIPTS)))
+@pytest.mark.parametrize("case", range(len(DECODER_CASES)))
+def test_diffusion_infer_bit_exact(case, script, oracle, ref):
+    """orc_local_decoder_forward_diffusion_infer against blt_local_decoder_forward_diffusion_infer
+    compiled from the reference: logits of all N + R rows bit for bit, for four decoder
+    configurations (sub-token split, cross-attention placements, window set -- which this forward
+    ignores) and block sections as the draft loop builds them and as a caller may.  Then the
+    cached form: the prefix through orc_kv_decode_step, the block rows through orc_kv_block_step
+    -- the dense forward's block rows bit for bit (a clean row never sees a block row)."""
+    from fblt_amd import decoder
+    c = dict(DECODER_CASES[case])
+    lengths, R, closed, d0_mode, fill = DIFFUSION_SCRIPTS[script]
+    E, V, k = c["E"], c["V"], c["k"]
+    N, P = sum(lengths), len(lengths)
+    if N + R > c["max_len"]:
+        pytest.skip("sequence longer than this decoder's tables")
+    rs = np.random.RandomState(7000 + 10 * case + script)
+    bound = _host_decoder(oracle, c, 300 + case)
+    patches = decoder.patch_table(lengths)
+    hidden = rs.randn(N, E).astype(np.float32)
+    patch_in = rs.randn(P, k * E).astype(np.float32)
+    batch = _block_batch(decoder, rs, N, R, P, fill, closed, c["max_len"])
+    got = np.zeros((N + R, V), dtype=np.float32)
+    assert oracle.orc_local_decoder_forward_diffusion_infer(
+        bound.ptr, binding.fptr(hidden.reshape(-1)), binding.fptr(patch_in.reshape(-1)), patches, P, batch.ptr,
+        d0_mode, binding.fptr(got.reshape(-1))) == 0
+    want = np.zeros((N + R, V), dtype=np.float32)
+    arena = ref.blt_arena_create(64 << 20, CPU)
+    try:
+        th = abi.tensor_view(hidden.ctypes.data, hidden.shape, CPU)
+        tp = abi.tensor_view(patch_in.ctypes.data, patch_in.shape, CPU)
+        tl = abi.tensor_view(want.ctypes.data, want.shape, CPU)
+        ref.blt_local_decoder_forward_diffusion_infer(bound.ptr, C.byref(th), C.byref(tp), patches, P, batch.ptr,
+                                                      d0_mode, C.byref(tl), arena)
+    finally:
+        ref.blt_arena_destroy(arena)
+    assert np.isfinite(want).all()
+    assert got.tobytes() == want.tobytes(), (case, script)
+
+    # cached form; the dense forward has no window, so the prefix is cached without one
+    bound.struct.config.local_window = 0
+    cache = decoder.HostCache(bound, c["max_len"])
+    assert oracle.orc_kv_cache_refresh_cross(cache.ptr, 0, binding.fptr(patch_in.reshape(-1)), P, 0) == 0
+    clean = np.zeros((N, V), dtype=np.float32)
+    assert oracle.orc_kv_decode_step(cache.ptr, 0, 0, patches, P, binding.fptr(hidden.reshape(-1)), N, closed,
+                                     binding.fptr(clean.reshape(-1))) == 0
+    assert clean.tobytes() == want[:N].tobytes(), (case, script, "clean rows")
+    block = np.zeros((R, V), dtype=np.float32)
+    assert oracle.orc_kv_block_step(cache.ptr, 0, N, P, batch.ptr, d0_mode, binding.fptr(block.reshape(-1))) == 0
+    assert block.tobytes() == want[N:].tobytes(), (case, script, "block rows")
