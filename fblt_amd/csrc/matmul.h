@@ -44,6 +44,12 @@ struct MatmulArgs {
     const uint32_t *cross_hi;
     uint32_t cross_rows_per_seq, cross_slab_rows, cross_head_dim;
     float cross_scale;
+    /* Products of up to 32 rows normally run on the thread-per-column kernel, whose sums follow the
+     * reference's order (bit-identical results) at the price of a serial chain of k additions.
+     * tolerant != 0: the caller accepts fp32-tolerance results for such shapes too, and they go to
+     * the matrix cores with K split over the waves (the whole decoder step sets it: a one-row
+     * step takes 72 us instead of 112). */
+    uint32_t tolerant;
 };
 
 void matmul_f32_launch(const MatmulArgs &g, hipStream_t s);

@@ -568,7 +568,13 @@ enum Path { PATH_SKINNY, PATH_SPLITK, PATH_MFMA };
 
 Path choose_path(const MatmulArgs &g) {
     const bool rope = g.rope_cos != nullptr && g.rope_cols > 0;
-    if (g.m <= 32u && !rope) return PATH_SKINNY;
+    /* up to this many rows the thread-per-column kernel, whose sums run in the reference's order
+     * (bit-identical results); BLT_HIP_EXACT_PRODUCT_ROWS lowers it (0: matrix cores for every shape) */
+    static const uint32_t exact_rows = [] {
+        const char *e = getenv("BLT_HIP_EXACT_PRODUCT_ROWS");
+        return e && *e ? (uint32_t)atoi(e) : 32u;
+    }();
+    if (g.m <= exact_rows && !rope && !g.tolerant) return PATH_SKINNY;
     /* fewer 64x64 tiles than half the compute units: quarter tiles, K split over the waves */
     if ((uint64_t)((g.n + TN - 1) / TN) * ((g.m + TM - 1) / TM) < 128u) return PATH_SPLITK;
     return PATH_MFMA;
@@ -597,7 +603,7 @@ bool matmul_takes_cross(const MatmulArgs &g) {
         return false;
     const Path path = choose_path(g);
     if (path == PATH_SKINNY) return g.n <= 256u && g.cross_head_dim <= 256u;
-    return g.m > 32u && path == PATH_SPLITK && g.cross_head_dim == 32u && g.n % 32u == 0u && g.k % 4u == 0u;
+    return path == PATH_SPLITK && g.cross_head_dim == 32u && g.n % 32u == 0u && g.k % 4u == 0u;
 }
 bool matmul_takes_norm(const MatmulArgs &g) {
     const Path path = choose_path(g);

@@ -1478,3 +1478,21 @@ def test_library_follows_the_chosen_stream(oracle, dev):
         lib.blt_hip_set_stream(None)
         d.close()
     assert_close(got, ref["out"], "side stream")
+
+
+@pytest.mark.gpu
+def test_decoder_step_with_exact_projections():
+    """The decoder step takes its projections on the matrix cores by default; BLT_HIP_EXACT_STEP=1
+    keeps the thread-per-column kernel (sums in the reference's order) for steps of up to 32 rows.
+    The switch is read once per process, so the step, layer and diffusion tests run again in a
+    process of their own with it set."""
+    import os
+    import subprocess
+    import sys
+    here = os.path.dirname(os.path.abspath(__file__))
+    env = dict(os.environ, BLT_HIP_EXACT_STEP="1")
+    p = subprocess.run([sys.executable, "-u", "-m", "pytest", os.path.join(here, "test_gpu_parity.py"), "-x", "-q", "-m",
+                        "gpu", "-k", "kv_decode_step_single_sequence or kv_decode_layer or diffusion_infer_forward "
+                        "or kv_decode_step_batched", "-p", "no:cacheprovider"],
+                       capture_output=True, text=True, timeout=900, env=env, cwd=os.path.dirname(here))
+    assert p.returncode == 0, p.stdout[-3000:] + p.stderr[-2000:]
