@@ -270,10 +270,12 @@ def bench_kv(kw, steps, warmup, warm_ms=0.0, lens="device"):
     return res, kw
 
 
-def bench_block(name, T, E, H, steps, warmup, gemm_only=None, cross=None, warm_ms=0.0):
+def bench_block(name, T, E, H, steps, warmup, gemm_only=None, cross=None, warm_ms=0.0, hidden=None):
     """blt_multihead_attention (projection, rotation, all heads, projection) on random
     device tensors; with gemm_only=(m, k, n) one blt_matmul of that shape; with cross=P
-    blt_cross_attention_forward of P patches over T bytes (T / P bytes per patch)."""
+    blt_cross_attention_forward of P patches over T bytes (T / P bytes per patch); with
+    hidden=h the whole blt_transformer_forward block (RMSNorm, attention, gated feed-forward of
+    width h, residuals) under a document-causal mask."""
     import ctypes as C
     import numpy as np
     import torch
@@ -338,6 +340,26 @@ def bench_block(name, T, E, H, steps, warmup, gemm_only=None, cross=None, warm_m
         flops = 2.0 * T * E * 3 * E + 4.0 * hd * pairs + 2.0 * T * E * E
         nbytes = 4.0 * (T * E + 3 * E * E + E * E + T * E)
         tokens = T
+        if hidden:
+            docs = abi.size_array([T // 3, (2 * T) // 3])
+            mc.doc_boundaries, mc.num_docs = docs, 3
+            n1, n2 = torch.ones(E, device="cuda"), torch.ones(E, device="cuda")
+            up, gate = (rnd(E, hidden) / E ** 0.5).cuda(), (rnd(E, hidden) / E ** 0.5).cuda()
+            down = (rnd(hidden, E) / hidden ** 0.5).cuda()
+            tv = [view(t) for t in (n1, wq, wp, n2, up, gate, down)]
+            wt = abi.BltTransformerWeights()
+            wt.norm1_weight, wt.attn_qkv_w, wt.attn_proj_w, wt.norm2_weight = (C.pointer(v) for v in tv[:4])
+            wt.ffn_up_w, wt.ffn_gate_w, wt.ffn_down_w = (C.pointer(v) for v in tv[4:])
+            tc = abi.BltTransformerConfig()
+            tc.attn_config = ac
+            tc.hidden_dim, tc.norm_type, tc.activation_type = hidden, abi.BLT_NORM_RMSNORM, abi.BLT_ACTIVATION_SWIGLU
+            keep += [docs, n1, n2, up, gate, down, tv, wt]
+
+            def run():
+                arena.contents.offset = 0
+                lib.blt_transformer_forward(C.byref(vx), C.byref(wt), C.byref(vo), C.byref(tc), arena)
+            flops += 2.0 * T * E * hidden * 3
+            nbytes += 4.0 * 3 * E * hidden
     warm_up(lib, run, warmup, warm_ms)
     lib.blt_hip_profile_begin()
     t0 = time.perf_counter()
@@ -981,6 +1003,13 @@ def main():
         log("xattn_c3", json.dumps(others["xattn_c3"]))
         others["mha_c2"] = bench_block("blt_multihead_attention T=128 E=512 H=8 rope causal", 128, 512, 8, K, W)
         log("mha_c2", json.dumps(others["mha_c2"]))
+        # a whole layer of the patch transformer (C2's caller once more removed) and of the local encoder
+        others["layer_c2"] = bench_block("blt_transformer_forward T=128 E=512 H=8 hidden=2048 rope document-causal",
+                                         128, 512, 8, K, W, hidden=2048)
+        log("layer_c2", json.dumps(others["layer_c2"]))
+        others["layer_c1"] = bench_block("blt_transformer_forward T=512 E=128 H=4 hidden=512 rope document-causal",
+                                         512, 128, 4, K, W, hidden=512)
+        log("layer_c1", json.dumps(others["layer_c1"]))
         others["matmul_8192x512x1536"] = bench_block("blt_matmul 8192x512x1536", 0, 0, 0, max(10, K // 10), 3,
                                                      gemm_only=(8192, 512, 1536), warm_ms=100.0)
         log("matmul", json.dumps(others["matmul_8192x512x1536"]))
@@ -1081,7 +1110,7 @@ def compact_line(head, others, cpu_head, K, W, detail_path):
     # whole decoder step (all layers + LM head): [launches per step, device us, wall us]
     steps_ = {k: [others[k]["launches_per_step"], _sig(others[k]["kernel_us_avg"]), _sig(others[k]["us_per_step"])]
               for k in ("decode_step", "decode_step_b1", "draft_pass") if k in others}
-    if "draft_pass" in others:   # the reference's call (prefix recomputed per pass) beside the cached block step
+    if "reference_call" in others.get("draft_pass", {}):   # the reference's call (prefix recomputed per pass) beside the cached block step
         c = others["draft_pass"]["reference_call"]
         steps_["draft_pass_reference_call"] = [c["launches_per_pass"], _sig(c["kernel_us_per_pass"]),
                                                _sig(c["wall_us_per_pass"])]

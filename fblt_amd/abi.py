@@ -109,6 +109,22 @@ class BltAttentionConfig(C.Structure):
     ]
 
 
+BLT_NORM_LAYERNORM, BLT_NORM_RMSNORM = 0, 1
+BLT_ACTIVATION_GELU, BLT_ACTIVATION_SWIGLU = 0, 1
+
+
+class BltTransformerConfig(C.Structure):
+    """csrc/models/transformer.h:31-38"""
+    _fields_ = [
+        ("attn_config", BltAttentionConfig),
+        ("hidden_dim", C.c_size_t),
+        ("layer_norm_eps", C.c_float),
+        ("norm_type", C.c_int),
+        ("activation_type", C.c_int),
+        ("use_bf16", C.c_int),
+    ]
+
+
 class BltCrossAttentionConfig(C.Structure):
     """csrc/models/cross_attention.h:27-34"""
     _fields_ = [
@@ -224,6 +240,7 @@ class BltBlockBatch(C.Structure):
 
 
 def check_layout():
+    assert C.sizeof(BltTransformerConfig) == 80
     assert C.sizeof(BltBlockBatch) == 112
     assert C.sizeof(BltTensor) == 104
     assert C.sizeof(BltArena) == 32

@@ -127,6 +127,12 @@ SYMBOLS = {
                                                          C.POINTER(abi.BltTensor), C.POINTER(abi.BltPatchInfo),
                                                          C.c_size_t, C.POINTER(abi.BltBlockBatch), C.c_int,
                                                          C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)]),
+    "blt_transformer_forward": (None, [C.POINTER(abi.BltTensor), C.POINTER(abi.BltTransformerWeights),
+                                       C.POINTER(abi.BltTensor), C.POINTER(abi.BltTransformerConfig),
+                                       C.POINTER(abi.BltArena)]),
+    "blt_transformer_forward_hip": (None, [C.POINTER(abi.BltTensor), C.POINTER(abi.BltTransformerWeights),
+                                           C.POINTER(abi.BltTensor), C.POINTER(abi.BltTransformerConfig),
+                                           C.POINTER(abi.BltArena)]),
     "blt_embedding_lookup": (None, [C.POINTER(abi.BltTensor), C.POINTER(C.c_uint32), C.POINTER(abi.BltTensor)]),
     "blt_embedding_lookup_hip": (None, [C.POINTER(abi.BltTensor), C.POINTER(C.c_uint32), C.POINTER(abi.BltTensor)]),
     "blt_kv_block_step_hip": (None, [C.POINTER(abi.BltKvCache), C.c_size_t, C.POINTER(abi.BltBlockBatch), C.c_int,

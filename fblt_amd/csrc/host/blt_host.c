@@ -351,6 +351,13 @@ void blt_local_decoder_forward_diffusion_infer(const blt_local_decoder *model, c
                                                   logits_out, arena);
 }
 
+void blt_transformer_forward(const blt_tensor *input, const blt_transformer_weights *weights, blt_tensor *output,
+                             const blt_transformer_config *config, blt_arena *arena) {
+    BLT_REQUIRE(input != NULL, "Transformer: input, weights, output, and config cannot be NULL");
+    BLT_DEVICE_ONLY(input->backend, "blt_transformer_forward");
+    blt_transformer_forward_hip(input, weights, output, config, arena);
+}
+
 void blt_add(const blt_tensor *a, const blt_tensor *b, blt_tensor *out) {
     BLT_REQUIRE(a != NULL, "blt_add: input tensors must be FP32 with matching element count");
     BLT_DEVICE_ONLY(a->backend, "blt_add");

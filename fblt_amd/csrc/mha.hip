@@ -33,9 +33,14 @@ void check_2d_fp32(const blt_tensor *t, size_t rows, size_t cols, const char *wh
 
 } // namespace
 
-extern "C" void blt_multihead_attention_hip(const blt_tensor *input, const blt_tensor *weight_qkv,
-                                            const blt_tensor *weight_proj, blt_tensor *output,
-                                            const blt_attention_config *config, blt_arena *arena) {
+namespace {
+
+/* The attention block; with norm_w the rows of `input` are RMS-normalised first (in the packed
+ * projection's own pass where that kernel takes it, csrc/models/transformer.c:60-66), with
+ * residual that [seq_len, embed_dim] array is added to the projected output (transformer.c:
+ * 116-117) -- the two statements a transformer block wraps around its attention. */
+void mha_run(const blt_tensor *input, const blt_tensor *weight_qkv, const blt_tensor *weight_proj, blt_tensor *output,
+             const blt_attention_config *config, blt_arena *arena, const float *norm_w, const float *residual) {
     BLT_REQUIRE(config != NULL && arena != NULL, "blt_multihead_attention: config and arena cannot be NULL");
     BLT_REQUIRE(arena->backend == BLT_BACKEND_HIP, "blt_multihead_attention: HIP implementation needs a device arena");
     const size_t E = config->embed_dim, H = config->num_heads;
@@ -104,6 +109,20 @@ extern "C" void blt_multihead_attention_hip(const blt_tensor *input, const blt_t
         g.rope_cos = rope_cos, g.rope_sin = rope_sin;
         g.rope_cols = (uint32_t)(2 * E), g.head_dim = (uint32_t)hd;
     }
+    if (norm_w != nullptr) {
+        if (matmul_takes_norm(g)) {
+            g.norm_w = norm_w;
+        } else { /* the row norm as a pass of its own */
+            const size_t shape[2] = {T, E};
+            blt_tensor normed = blt_tensor_create_uninit(arena, shape, 2, BLT_DTYPE_FP32);
+            blt_tensor wt;
+            std::memset(&wt, 0, sizeof(wt));
+            wt.data = const_cast<float *>(norm_w), wt.ndim = 1, wt.shape[0] = E, wt.strides[0] = 1, wt.numel = E;
+            wt.dtype = BLT_DTYPE_FP32, wt.backend = BLT_BACKEND_HIP, wt.is_view = true;
+            blt_rmsnorm_forward_hip(input, &wt, &normed);
+            g.a = (const float *)normed.data;
+        }
+    }
     matmul_f32_launch(g, 0);
     if (config->use_rope && !fuse_rope) {
         for (size_t head = 0; head < H; head++) {
@@ -115,6 +134,7 @@ extern "C" void blt_multihead_attention_hip(const blt_tensor *input, const blt_t
     /* 2. every head in one launch */
     const blt_mask_config *mc = config->mask_config;
     const float *dense = nullptr;
+    const uint32_t *row_lo = nullptr, *row_hi = nullptr;
     bool causal_desc = false;
     size_t causal_off = 0, window = 0;
     if (mc != NULL) {
@@ -128,10 +148,23 @@ extern "C" void blt_multihead_attention_hip(const blt_tensor *input, const blt_t
         } else if (plain && mc->sliding_window == 0) {
             /* nothing masked */
         } else {
-            blt_tensor mask_tensor;
-            std::memset(&mask_tensor, 0, sizeof(mask_tensor));
-            blt_build_attention_mask_hip(mc, &mask_tensor, arena);
-            dense = (const float *)mask_tensor.data;
+            /* document boundaries, groups: one key range per row when the allowed keys of every row
+             * are contiguous (they are for the document-causal masks of the patch transformer and of
+             * the local encoder, csrc/models/global_transformer.c:19-33), 8 bytes per row through
+             * the pinned ring; the dense matrix from the device builder otherwise */
+            std::vector<uint32_t> lohi(2 * T);
+            if (blt_mask_config_row_ranges(mc, lohi.data(), lohi.data() + T) == 1) {
+                for (size_t i = 0; i < T; i++) /* the dense builder refuses such a mask (mask_builder_cpu.c:93) */
+                    BLT_REQUIRE(lohi[i] < lohi[T + i], "blt_build_attention_mask: query position has no valid key");
+                uint32_t *dev = (uint32_t *)blt_arena_alloc(arena, 2 * T * sizeof(uint32_t), 64);
+                blt_upload_staged(dev, lohi.data(), 2 * T * sizeof(uint32_t));
+                row_lo = dev, row_hi = dev + T;
+            } else {
+                blt_tensor mask_tensor;
+                std::memset(&mask_tensor, 0, sizeof(mask_tensor));
+                blt_build_attention_mask_hip(mc, &mask_tensor, arena);
+                dense = (const float *)mask_tensor.data;
+            }
         }
     }
     std::vector<blt_attention_problem> pr(H);
@@ -153,6 +186,10 @@ extern "C" void blt_multihead_attention_hip(const blt_tensor *input, const blt_t
             p.mask_kind = BLT_ATTN_MASK_CAUSAL;
             p.causal_offset = causal_off;
             p.window = window;
+        } else if (row_lo != nullptr) {
+            p.mask_kind = BLT_ATTN_MASK_ROW_RANGE;
+            p.row_lo = row_lo;
+            p.row_hi = row_hi;
         } else {
             p.mask_kind = BLT_ATTN_MASK_FROM_HEAD;
             p.head.mask = dense;
@@ -161,15 +198,112 @@ extern "C" void blt_multihead_attention_hip(const blt_tensor *input, const blt_t
     }
     blt_attention_batch_hip(pr.data(), H);
 
-    /* 3. output projection */
+    /* 3. output projection (+ residual) */
     std::memset(&g, 0, sizeof(g));
     g.a = combined;
     g.b = (const float *)weight_proj->data;
     g.out = (float *)output->data;
+    g.residual = residual;
     g.m = (uint32_t)T, g.k = (uint32_t)E, g.n = (uint32_t)E;
     g.lda = g.ldb = g.ldo = (uint32_t)E;
     matmul_f32_launch(g, 0);
     HIP_CHECK_LAUNCH("blt_multihead_attention");
+}
+
+} // namespace
+
+extern "C" void blt_multihead_attention_hip(const blt_tensor *input, const blt_tensor *weight_qkv,
+                                            const blt_tensor *weight_proj, blt_tensor *output,
+                                            const blt_attention_config *config, blt_arena *arena) {
+    mha_run(input, weight_qkv, weight_proj, output, config, arena, nullptr, nullptr);
+}
+
+/*
+ * blt_transformer_forward on the device (reference: csrc/models/transformer.c:97-128), the block
+ * the patch transformer stacks (csrc/models/global_transformer.c:69-97 through
+ * transformer_stack.c:228-248) and the local encoder runs per byte layer (csrc/models/
+ * local_encoder.c:243-248): RMSNorm, attention block, residual, RMSNorm, gated feed-forward,
+ * residual -- five launches where the small-output projection kernel takes the fused forms:
+ *
+ *   1. qkv = RMSNorm(input) * attn_qkv_w, Q and K rotated in the epilogue;
+ *   2. all heads in one attention launch (mask as a descriptor or as row ranges);
+ *   3. attn_residual = input + combined * attn_proj_w;
+ *   4. act = silu(RMSNorm(attn_residual) * ffn_gate_w) .* (RMSNorm(attn_residual) * ffn_up_w);
+ *   5. output = attn_residual + act * ffn_down_w.
+ *
+ * RMSNorm + SwiGLU blocks with FP32 weights (what every BLT block is, csrc/models/
+ * local_common.c:99-115); LayerNorm / GELU blocks and BF16 weight copies end with a message.
+ */
+extern "C" void blt_transformer_forward_hip(const blt_tensor *input, const blt_transformer_weights *w, blt_tensor *output,
+                                            const blt_transformer_config *config, blt_arena *arena) {
+    BLT_REQUIRE(input != NULL && w != NULL && output != NULL && config != NULL,
+                "Transformer: input, weights, output, and config cannot be NULL");
+    BLT_REQUIRE(arena != NULL, "Transformer: arena cannot be NULL");
+    BLT_REQUIRE(arena->backend == BLT_BACKEND_HIP, "Transformer: HIP implementation needs a device arena");
+    BLT_REQUIRE(config->norm_type == BLT_NORM_RMSNORM && config->activation_type == BLT_ACTIVATION_SWIGLU,
+                "Transformer: the HIP backend implements RMSNorm + SwiGLU blocks only");
+    BLT_REQUIRE(config->use_bf16 == 0, "Transformer: the HIP backend takes FP32 weights only (BF16 copies are not supported)");
+    BLT_REQUIRE(input->ndim == 2 && input->dtype == BLT_DTYPE_FP32, "Transformer: input must be a 2D FP32 tensor [seq_len, embed_dim]");
+    const size_t T = input->shape[0], E = input->shape[1];
+    check_2d_fp32(input, T, E, "Transformer: input must be a 2D FP32 tensor [seq_len, embed_dim]");
+    check_2d_fp32(output, T, E, "Transformer: output shape must match input [seq_len, embed_dim]");
+    BLT_REQUIRE(w->norm1_weight != NULL && w->norm1_weight->ndim == 1 && w->norm1_weight->shape[0] == E &&
+                    w->norm1_weight->dtype == BLT_DTYPE_FP32 && w->norm1_weight->backend == BLT_BACKEND_HIP,
+                "Transformer: norm1_weight must be [embed_dim] FP32");
+    BLT_REQUIRE(w->norm2_weight != NULL && w->norm2_weight->ndim == 1 && w->norm2_weight->shape[0] == E &&
+                    w->norm2_weight->dtype == BLT_DTYPE_FP32 && w->norm2_weight->backend == BLT_BACKEND_HIP,
+                "Transformer: norm2_weight must be [embed_dim] FP32");
+    BLT_REQUIRE(w->attn_qkv_w != NULL && w->attn_proj_w != NULL, "Transformer: attn_qkv_w and attn_proj_w cannot be NULL");
+    BLT_REQUIRE(w->ffn_up_w != NULL && w->ffn_up_w->ndim == 2 && w->ffn_up_w->shape[0] == E,
+                "Transformer: ffn_up_w must be [embed_dim, hidden_dim]");
+    const size_t hidden = w->ffn_up_w->shape[1];
+    BLT_REQUIRE(hidden == config->hidden_dim, "Transformer: ffn_up_w hidden dimension mismatch with config");
+    check_2d_fp32(w->ffn_up_w, E, hidden, "Transformer: ffn_up_w must be FP32 or BF16");
+    check_2d_fp32(w->ffn_gate_w, E, hidden, "Transformer: ffn_gate_w must be [embed_dim, hidden_dim] for SwiGLU");
+    check_2d_fp32(w->ffn_down_w, hidden, E, "Transformer: ffn_down_w must be [hidden_dim, embed_dim]");
+    if (T == 0) return;
+
+    const size_t embed_shape[2] = {T, E}, hidden_shape[2] = {T, hidden};
+    blt_tensor attn_residual = blt_tensor_create_uninit(arena, embed_shape, 2, BLT_DTYPE_FP32);
+    mha_run(input, w->attn_qkv_w, w->attn_proj_w, &attn_residual, &config->attn_config, arena,
+            (const float *)w->norm1_weight->data, (const float *)input->data);
+
+    blt_tensor act = blt_tensor_create_uninit(arena, hidden_shape, 2, BLT_DTYPE_FP32);
+    MatmulArgs g;
+    std::memset(&g, 0, sizeof(g));
+    g.a = (const float *)attn_residual.data;
+    g.b = (const float *)w->ffn_up_w->data;
+    g.out = (float *)act.data;
+    g.m = (uint32_t)T, g.k = (uint32_t)E, g.n = (uint32_t)hidden;
+    g.lda = (uint32_t)E, g.ldb = g.ldo = (uint32_t)hidden;
+    if (matmul_takes_gated(g) && matmul_takes_norm(g)) { /* norm, up, gate and the activation in one pass */
+        g.b2 = (const float *)w->ffn_gate_w->data;
+        g.norm_w = (const float *)w->norm2_weight->data;
+        matmul_f32_launch(g, 0);
+    } else {
+        blt_tensor normed = blt_tensor_create_uninit(arena, embed_shape, 2, BLT_DTYPE_FP32);
+        blt_rmsnorm_forward_hip(&attn_residual, w->norm2_weight, &normed);
+        g.a = (const float *)normed.data;
+        if (matmul_takes_gated(g)) {
+            g.b2 = (const float *)w->ffn_gate_w->data;
+            matmul_f32_launch(g, 0);
+        } else {
+            blt_tensor gate = blt_tensor_create_uninit(arena, hidden_shape, 2, BLT_DTYPE_FP32);
+            matmul_f32_launch(g, 0);
+            g.b = (const float *)w->ffn_gate_w->data, g.out = (float *)gate.data;
+            matmul_f32_launch(g, 0);
+            blt_swiglu_forward_hip(&gate, &act, &act);
+        }
+    }
+    std::memset(&g, 0, sizeof(g));
+    g.a = (const float *)act.data;
+    g.b = (const float *)w->ffn_down_w->data;
+    g.out = (float *)output->data;
+    g.residual = (const float *)attn_residual.data;
+    g.m = (uint32_t)T, g.k = (uint32_t)hidden, g.n = (uint32_t)E;
+    g.lda = (uint32_t)hidden, g.ldb = g.ldo = (uint32_t)E;
+    matmul_f32_launch(g, 0);
+    HIP_CHECK_LAUNCH("blt_transformer_forward");
 }
 
 /*

@@ -253,6 +253,26 @@ typedef struct {
     blt_patch_info *cached_patches; /* [batch_size*max_seq_len] boundary snapshot */
 } blt_kv_cache;
 
+/* csrc/models/transformer.h:15-38 */
+typedef enum {
+    BLT_NORM_LAYERNORM = 0,
+    BLT_NORM_RMSNORM = 1
+} blt_norm_type;
+
+typedef enum {
+    BLT_ACTIVATION_GELU = 0,
+    BLT_ACTIVATION_SWIGLU = 1
+} blt_activation_type;
+
+typedef struct {
+    blt_attention_config attn_config;
+    size_t hidden_dim;
+    float layer_norm_eps;
+    blt_norm_type norm_type;
+    blt_activation_type activation_type;
+    int use_bf16;
+} blt_transformer_config;
+
 /* csrc/models/local_decoder.h:42-46 */
 typedef enum {
     BLT_D0_HFINAL = 0, /* every row of byte_hidden_in is a real encoder state */
@@ -326,6 +346,9 @@ BLT_ABI_ASSERT(sizeof(blt_kv_cache) == 112 && offsetof(blt_kv_cache, self_len) =
                    offsetof(blt_kv_cache, cached_patches) == 104,
                "blt_kv_cache layout");
 
+BLT_ABI_ASSERT(sizeof(blt_transformer_config) == 80 && offsetof(blt_transformer_config, hidden_dim) == 56 &&
+                   offsetof(blt_transformer_config, norm_type) == 68 && offsetof(blt_transformer_config, use_bf16) == 76,
+               "blt_transformer_config layout");
 BLT_ABI_ASSERT(sizeof(blt_block_batch) == 112 && offsetof(blt_block_batch, tokens) == 40 &&
                    offsetof(blt_block_batch, groups) == 80 && offsetof(blt_block_batch, trailing_closed) == 104,
                "blt_block_batch layout");

@@ -135,6 +135,14 @@ void blt_multihead_attention_hip(const blt_tensor *input, const blt_tensor *weig
                                  const blt_tensor *weight_proj, blt_tensor *output,
                                  const blt_attention_config *config, blt_arena *arena);
 
+/* csrc/models/transformer.h (transformer.c:97-128): the pre-norm block every BLT transformer is
+ * made of -- RMSNorm, attention block, residual, RMSNorm, SwiGLU feed-forward, residual; called
+ * once per layer by the patch transformer (csrc/models/transformer_stack.c:228-248 under
+ * global_transformer.c:69-97) and by the local encoder (csrc/models/local_encoder.c:243-248).
+ * RMSNorm + SwiGLU with FP32 weights only. */
+void blt_transformer_forward_hip(const blt_tensor *input, const blt_transformer_weights *weights, blt_tensor *output,
+                                 const blt_transformer_config *config, blt_arena *arena);
+
 /* ===================================================================== */
 /* Part 2 -- device memory shim (csrc/core/cuda_shim.h:18-31,             */
 /*           csrc/ops/memory.cu:19-77)                                    */
@@ -202,6 +210,8 @@ void blt_cross_attention_forward(const blt_tensor *query_in, const blt_tensor *k
                                  const blt_cross_attention_weights *weights, blt_tensor *output,
                                  const blt_cross_attention_config *config, blt_arena *arena);
 /* csrc/core/backend.c:254-256, 276-278, 380-382 */
+void blt_transformer_forward(const blt_tensor *input, const blt_transformer_weights *weights, blt_tensor *output,
+                             const blt_transformer_config *config, blt_arena *arena);
 void blt_add(const blt_tensor *a, const blt_tensor *b, blt_tensor *out);
 void blt_swiglu_forward(const blt_tensor *gate, const blt_tensor *up, blt_tensor *out);
 void blt_rmsnorm_forward(const blt_tensor *x, const blt_tensor *weight, blt_tensor *out);

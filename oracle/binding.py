@@ -28,7 +28,7 @@ def build(ref=True):
     if ref and os.path.isdir(os.environ.get("REF_ROOT", "/root/reference")):
         subprocess.check_call(["make", "-s", "-B", "-C", HERE, "ref"])
         if os.path.exists(os.path.join(HERE, "..", "fblt_amd", "lib", "libfblt_hip.so")):
-            subprocess.check_call(["make", "-s", "-C", HERE, "callers"])
+            subprocess.check_call(["make", "-s", "-C", HERE, "callers", "stack_callers"])
 
 
 def load_oracle():
@@ -83,6 +83,9 @@ def load_oracle():
     lib.orc_multihead_attention.restype = C.c_int
     lib.orc_multihead_attention.argtypes = [_fp, _fp, _fp, _fp, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int, C.c_int,
                                             C.c_float, _fp, _fp, C.POINTER(abi.BltMaskConfig)]
+    lib.orc_transformer_forward.restype = C.c_int
+    lib.orc_transformer_forward.argtypes = [_fp] * 9 + [C.c_size_t] * 4 + [C.c_int, C.c_int, C.c_float, _fp, _fp,
+                                                                         C.POINTER(abi.BltMaskConfig)]
     lib.orc_rmsnorm_forward.restype = None
     lib.orc_rmsnorm_forward.argtypes = [_fp, _fp, _fp, C.c_size_t, C.c_size_t]
     lib.orc_add.restype = None
@@ -176,6 +179,9 @@ def load_ref():
     lib.blt_rope_apply_packed.argtypes = [_fp, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, _fp, _fp, C.c_int]
     lib.blt_multihead_attention.restype = None
     lib.blt_multihead_attention.argtypes = [T, T, T, T, C.POINTER(abi.BltAttentionConfig), C.POINTER(abi.BltArena)]
+    lib.blt_transformer_forward.restype = None
+    lib.blt_transformer_forward.argtypes = [T, C.POINTER(abi.BltTransformerWeights), T,
+                                            C.POINTER(abi.BltTransformerConfig), C.POINTER(abi.BltArena)]
     lib.blt_cross_attention_forward.restype = None
     lib.blt_cross_attention_forward.argtypes = [T, T, C.POINTER(abi.BltCrossAttentionWeights), T,
                                                 C.POINTER(abi.BltCrossAttentionConfig), C.POINTER(abi.BltArena)]
@@ -223,6 +229,48 @@ def load_ref():
 CALLERS_SO = os.path.join(HERE, "_ref", "libblt_ref_callers.so")
 
 
+STACK_CALLERS_SO = os.path.join(HERE, "_ref", "libblt_ref_stack_callers.so")
+
+
+class BltGlobalTransformerConfig(C.Structure):
+    """csrc/models/global_transformer.h:15-24"""
+    _fields_ = [("embed_dim", C.c_size_t), ("num_layers", C.c_size_t), ("hidden_dim", C.c_size_t),
+                ("num_heads", C.c_size_t), ("rope_theta", C.c_float), ("max_seq_len", C.c_size_t),
+                ("use_bf16", C.c_bool), ("use_fp8", C.c_bool)]
+
+
+class BltTransformerStack(C.Structure):
+    """csrc/models/transformer_stack.h:14-33"""
+    _fields_ = [("layer_config", abi.BltTransformerConfig), ("layer_storage", C.c_void_p),
+                ("layer_weights", C.POINTER(abi.BltTransformerWeights)), ("layer_weights_bf16", C.c_void_p),
+                ("layer_weights_fp8", C.c_void_p), ("rope_cos_cache", abi.BltTensor), ("rope_sin_cache", abi.BltTensor),
+                ("num_layers", C.c_size_t), ("embed_dim", C.c_size_t), ("hidden_dim", C.c_size_t),
+                ("num_heads", C.c_size_t), ("head_dim", C.c_size_t), ("max_seq_len", C.c_size_t),
+                ("use_bf16", C.c_int), ("use_fp8", C.c_int)]
+
+
+class BltGlobalTransformer(C.Structure):
+    """csrc/models/global_transformer.h:26-29"""
+    _fields_ = [("config", BltGlobalTransformerConfig), ("stack", BltTransformerStack)]
+
+
+def load_ref_stack_callers():
+    """The reference's transformer_stack.c and global_transformer.c, compiled unmodified and linked
+    against the HIP library without the reference's transformer.c, so that every layer of the
+    patch transformer runs through the library's blt_transformer_forward (`make -C oracle
+    stack_callers`); None where that was never built."""
+    if not os.path.exists(STACK_CALLERS_SO) or not os.path.exists(REF_SO):
+        return None
+    load_ref()
+    lib = C.CDLL(STACK_CALLERS_SO)
+    T, A = C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)
+    lib.blt_global_transformer_create.restype = C.POINTER(BltGlobalTransformer)
+    lib.blt_global_transformer_create.argtypes = [A, C.POINTER(BltGlobalTransformerConfig)]
+    lib.blt_global_transformer_forward.restype = None
+    lib.blt_global_transformer_forward.argtypes = [C.POINTER(BltGlobalTransformer), T, abi.c_size_p, C.c_size_t, T, A]
+    return lib
+
+
 def load_ref_callers():
     """The reference's attention blocks and KV-cache step, compiled unmodified and linked against
     the HIP library so that every tensor op they call lands there (`make -C oracle callers`); None
@@ -241,6 +289,9 @@ def load_ref_callers():
     lib.blt_cross_attention_forward.restype = None
     lib.blt_cross_attention_forward.argtypes = [T, T, C.POINTER(abi.BltCrossAttentionWeights), T,
                                                 C.POINTER(abi.BltCrossAttentionConfig), A]
+    lib.blt_transformer_forward.restype = None
+    lib.blt_transformer_forward.argtypes = [T, C.POINTER(abi.BltTransformerWeights), T,
+                                            C.POINTER(abi.BltTransformerConfig), A]
     lib.blt_kv_cache_create.restype = K
     lib.blt_kv_cache_create.argtypes = [A, C.POINTER(abi.BltLocalDecoder), C.c_size_t]
     for name in ("blt_kv_cache_destroy", "blt_kv_cache_reset"):

@@ -935,3 +935,34 @@ int orc_kv_block_step(blt_kv_cache *cache, size_t b, size_t base, size_t num_pat
     free(cur), free(mid);
     return rc;
 }
+
+/* csrc/models/transformer.c:97-128 for an RMSNorm + SwiGLU block (what csrc/models/local_common.c:
+ * 99-115 and csrc/models/transformer_stack.c configure): norm, attention block, residual, norm,
+ * up / gate projections, SwiGLU, down projection, residual.  input / output are [seq_len, E]. */
+int orc_transformer_forward(const float *input, const float *norm1_w, const float *qkv_w, const float *proj_w,
+                            const float *norm2_w, const float *up_w, const float *gate_w, const float *down_w,
+                            float *output, size_t seq_len, size_t embed_dim, size_t hidden_dim, size_t num_heads,
+                            int is_causal, int use_rope, float rope_theta, const float *rope_cos_cache,
+                            const float *rope_sin_cache, const blt_mask_config *mask_config) {
+    const size_t T = seq_len, E = embed_dim, Hd = hidden_dim;
+    float *normed = (float *)malloc(T * E * sizeof(float));
+    float *attn = (float *)malloc(T * E * sizeof(float));
+    float *resid = (float *)malloc(T * E * sizeof(float));
+    float *up = (float *)malloc(T * Hd * sizeof(float));
+    float *gate = (float *)malloc(T * Hd * sizeof(float));
+    float *act = (float *)malloc(T * Hd * sizeof(float));
+    orc_rmsnorm_forward(input, norm1_w, normed, T, E);
+    int rc = orc_multihead_attention(normed, qkv_w, proj_w, attn, T, E, num_heads, is_causal, use_rope, rope_theta,
+                                     rope_cos_cache, rope_sin_cache, mask_config);
+    if (rc == ORC_OK) {
+        orc_add(input, attn, resid, T * E);
+        orc_rmsnorm_forward(resid, norm2_w, normed, T, E);
+        orc_matmul(normed, up_w, up, T, E, Hd);
+        orc_matmul(normed, gate_w, gate, T, E, Hd);
+        orc_swiglu_forward(gate, up, act, T * Hd);
+        orc_matmul(act, down_w, output, T, Hd, E);
+        orc_add(resid, output, output, T * E);
+    }
+    free(normed), free(attn), free(resid), free(up), free(gate), free(act);
+    return rc;
+}

@@ -270,6 +270,13 @@ int orc_local_decoder_forward_diffusion_infer(const blt_local_decoder *dec, cons
 int orc_kv_block_step(blt_kv_cache *cache, size_t b, size_t base, size_t num_patches, const blt_block_batch *batch,
                       int d0_mode, float *logits_out);
 
+/* models/transformer.c:97-128, RMSNorm + SwiGLU block */
+int orc_transformer_forward(const float *input, const float *norm1_w, const float *qkv_w, const float *proj_w,
+                            const float *norm2_w, const float *up_w, const float *gate_w, const float *down_w,
+                            float *output, size_t seq_len, size_t embed_dim, size_t hidden_dim, size_t num_heads,
+                            int is_causal, int use_rope, float rope_theta, const float *rope_cos_cache,
+                            const float *rope_sin_cache, const blt_mask_config *mask_config);
+
 #ifdef __cplusplus
 }
 #endif

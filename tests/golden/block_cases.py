@@ -3,7 +3,7 @@ decoder step).  Shared by the generator (make_golden_blocks.py, which feeds them
 build) and by the tests (which feed them to the CPU checker and to the HIP library)."""
 import numpy as np
 
-from fblt_amd import decoder
+from fblt_amd import abi, decoder
 
 MHA_CASES = {
     # T, E, H, rope, mask ("causal_flag", "causal_cfg", "window", "docs")
@@ -36,6 +36,11 @@ DIFFUSION_CASES = {
                                    fill="mixed"),
     "diff_E128_zeros_B16": dict(E=128, H=4, XH=4, L=2, hidden=256, V=256, max_len=128, k=1, window=0, all_layers=True,
                                 placement=0, lengths=[16, 9, 20, 11, 14], R=16, closed=1, learned=False, fill="draft"),
+}
+# the transformer block (csrc/models/transformer.c:97-128): T, E, H, hidden, mask kind
+TRANSFORMER_CASES = {
+    "block_T128_E512_H8_docs": (128, 512, 8, 1024, "docs"),           # a layer of the patch transformer at C2 size
+    "block_T96_E64_H2_docs_window": (96, 64, 2, 160, "docs_window"),  # a byte layer of the local encoder
 }
 THETA = 500000.0
 
@@ -107,3 +112,31 @@ def diffusion_inputs(name):
         batch = decoder.BlockBatch(N, R, P, tokens=tokens, positions=positions, groups=groups,
                                    trailing_closed=c["closed"])
     return c, weights, hidden, latents, batch
+
+
+def transformer_case(rs, T, E, H, hidden, mask):
+    """Seeded inputs of one RMSNorm + SwiGLU block and its mask configuration: "causal" (the
+    decoder's), "window" (causal + sliding window), "docs" (document-causal: the patch transformer's,
+    csrc/models/global_transformer.c:19-33), "docs_window" (the local encoder's)."""
+    x = rs.randn(T, E).astype(np.float32)
+    w = {"norm1": (1.0 + 0.1 * rs.randn(E)).astype(np.float32), "qkv": (rs.randn(E, 3 * E) / np.sqrt(E)).astype(np.float32),
+         "proj": (rs.randn(E, E) / np.sqrt(E)).astype(np.float32), "norm2": (1.0 + 0.1 * rs.randn(E)).astype(np.float32),
+         "up": (rs.randn(E, hidden) / np.sqrt(E)).astype(np.float32),
+         "gate": (rs.randn(E, hidden) / np.sqrt(E)).astype(np.float32),
+         "down": (rs.randn(hidden, E) / np.sqrt(hidden)).astype(np.float32)}
+    cfg = abi.BltMaskConfig()
+    cfg.seq_len_q = cfg.seq_len_kv = T
+    cfg.is_causal = True
+    keep = None
+    if "window" in mask:
+        cfg.sliding_window = max(2, T // 5)
+    if "docs" in mask:
+        cuts = sorted(set(int(v) for v in rs.randint(1, T, size=3))) if T > 4 else [1]
+        keep = abi.size_array(cuts)
+        cfg.doc_boundaries, cfg.num_docs = keep, len(cuts) + 1
+    return x, w, cfg, keep
+
+
+def transformer_inputs(name):
+    T, E, H, hidden, mask = TRANSFORMER_CASES[name]
+    return (T, E, H, hidden, mask) + transformer_case(np.random.RandomState(seed_of(name)), T, E, H, hidden, mask)

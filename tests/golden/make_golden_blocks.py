@@ -1,7 +1,7 @@
 """Writes tests/golden/blocks_golden.npz from the reference build (oracle/_ref):
 blt_multihead_attention, blt_cross_attention_forward, the script of
 blt_kv_cache_refresh_cross + blt_kv_decode_step calls and the
-blt_local_decoder_forward_diffusion_infer cases of block_cases.py.
+blt_transformer_forward and blt_local_decoder_forward_diffusion_infer cases of block_cases.py.
 
 Run in a container that holds the reference sources:
     make -C oracle ref && python tests/golden/make_golden_blocks.py
@@ -126,6 +126,34 @@ def run_diffusion(ref, arena, name):
     return out
 
 
+WEIGHT_ORDER = ("norm1", "qkv", "proj", "norm2", "up", "gate", "down")
+
+
+def transformer_structs(w, cfg, E, H, hidden, make_view):
+    """blt_transformer_weights / blt_transformer_config over the case's arrays (views kept alive by the caller)."""
+    tv = {n: make_view(w[n]) for n in WEIGHT_ORDER}
+    wt = abi.BltTransformerWeights()
+    wt.norm1_weight, wt.attn_qkv_w, wt.attn_proj_w = C.pointer(tv["norm1"]), C.pointer(tv["qkv"]), C.pointer(tv["proj"])
+    wt.norm2_weight, wt.ffn_up_w, wt.ffn_gate_w = C.pointer(tv["norm2"]), C.pointer(tv["up"]), C.pointer(tv["gate"])
+    wt.ffn_down_w = C.pointer(tv["down"])
+    tc = abi.BltTransformerConfig()
+    ac = tc.attn_config
+    ac.embed_dim, ac.num_heads, ac.head_dim, ac.is_causal, ac.use_rope, ac.rope_theta = E, H, E // H, True, True, bc.THETA
+    ac.mask_config = C.pointer(cfg)
+    tc.hidden_dim, tc.norm_type, tc.activation_type = hidden, abi.BLT_NORM_RMSNORM, abi.BLT_ACTIVATION_SWIGLU
+    return wt, tc, tv
+
+
+def run_transformer(ref, arena, name):
+    T, E, H, hidden, _mask, x, w, cfg, _keep = bc.transformer_inputs(name)
+    wt, tc, _tv = transformer_structs(w, cfg, E, H, hidden, view)
+    out = np.zeros((T, E), dtype=np.float32)
+    tx, to = view(x), view(out)
+    arena.contents.offset = 0
+    ref.blt_transformer_forward(C.byref(tx), C.byref(wt), C.byref(to), C.byref(tc), arena)
+    return out
+
+
 def main():
     ref = binding.load_ref()
     if ref is None:
@@ -142,6 +170,8 @@ def main():
         pack(store, name + "/logits", logits, rs)
         for tier, arr in tiers.items():
             pack(store, name + "/" + tier, arr, rs)
+    for name in bc.TRANSFORMER_CASES:
+        pack(store, name + "/out", run_transformer(ref, arena, name), rs)
     for name in bc.DIFFUSION_CASES:
         pack(store, name + "/logits", run_diffusion(ref, arena, name), rs)
     ref.blt_arena_destroy(arena)

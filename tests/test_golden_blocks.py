@@ -99,6 +99,17 @@ def test_oracle_reproduces_reference_decoder_steps(name, oracle):
         check(np.stack(cache.tiers[tier]), name + "/" + tier, exact=True)
 
 
+@pytest.mark.parametrize("name", list(bc.TRANSFORMER_CASES))
+def test_oracle_reproduces_reference_transformer_block(name, oracle):
+    T, E, H, hidden, _mask, x, w, cfg, _keep = bc.transformer_inputs(name)
+    out = np.zeros((T, E), dtype=np.float32)
+    order = ("norm1", "qkv", "proj", "norm2", "up", "gate", "down")
+    assert oracle.orc_transformer_forward(binding.fptr(x.reshape(-1)), *(binding.fptr(w[n].reshape(-1)) for n in order),
+                                          binding.fptr(out.reshape(-1)), T, E, hidden, H, 1, 1, bc.THETA, None, None,
+                                          C.byref(cfg)) == 0
+    check(out, name + "/out", exact=True)
+
+
 def _diffusion_decoder(oracle, c, weights, backend, place):
     cos, sin = host_tables(oracle, c["max_len"], c["E"] // c["H"])
     return decoder.bind(weights, cos, sin, backend, place, c["E"], c["H"], c["XH"], c["hidden"], c["V"], c["max_len"],
@@ -241,3 +252,24 @@ def test_hip_matches_reference_diffusion_forward(name, oracle):
     out = tl.cpu().numpy()
     lib.blt_arena_destroy(arena)
     check(out, name + "/logits", exact=False)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", list(bc.TRANSFORMER_CASES))
+def test_hip_matches_reference_transformer_block(name):
+    import torch
+    from fblt_amd import api
+    from tests.golden.make_golden_blocks import transformer_structs
+    lib = api.load()
+    T, E, H, hidden, _mask, x, w, cfg, _keep = bc.transformer_inputs(name)
+    tens = {n: torch.from_numpy(a).cuda() for n, a in w.items()}
+    wt, tc, _tv = transformer_structs(tens, cfg, E, H, hidden, dev_view)
+    tx = torch.from_numpy(x).cuda()
+    to = torch.full((T, E), 7.0, dtype=torch.float32, device="cuda")
+    vx, vo = dev_view(tx), dev_view(to)
+    arena = lib.blt_arena_create(128 << 20, HIP)
+    lib.blt_transformer_forward(C.byref(vx), C.byref(wt), C.byref(vo), C.byref(tc), arena)
+    lib.blt_backend_pass_sync_hip()
+    out = to.cpu().numpy()
+    lib.blt_arena_destroy(arena)
+    check(out, name + "/out", exact=False)

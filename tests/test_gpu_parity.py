@@ -1210,6 +1210,110 @@ def test_kv_decode_step_single_sequence(case, impl, oracle, dev):
         lib.blt_arena_destroy(arena)
 
 
+@pytest.mark.parametrize("impl", IMPLS)
+@pytest.mark.parametrize("shape", [(2, 8, 2, 12, "causal"), (33, 32, 4, 48, "window"), (70, 48, 3, 64, "docs"),
+                                   (40, 64, 2, 96, "docs_window"),
+                                   (512, 128, 4, 512, "docs_window"),    # a byte layer of the local encoder at C1 size
+                                   (128, 512, 8, 1024, "docs"),          # a layer of the patch transformer at C2 size
+                                   (300, 256, 4, 768, "causal")])
+def test_transformer_block(shape, impl, oracle, dev):
+    """blt_transformer_forward on device tensors against the restated block (csrc/models/
+    transformer.c:97-128); impl = reference_callers runs the reference's transformer.c on this
+    library's ops."""
+    import torch
+    from tests.golden.block_cases import transformer_case
+    lib = api.load()
+    entry = _entry(impl, lib)
+    T, E, H, hidden, mask = shape
+    rs = np.random.RandomState(T * 131 + E)
+    x, w, cfg, _keep = transformer_case(rs, T, E, H, hidden, mask)
+    order = ("norm1", "qkv", "proj", "norm2", "up", "gate", "down")
+    ref = np.zeros((T, E), dtype=np.float32)
+    assert oracle.orc_transformer_forward(binding.fptr(x.reshape(-1)), *(binding.fptr(w[n].reshape(-1)) for n in order),
+                                          binding.fptr(ref.reshape(-1)), T, E, hidden, H, 1, 1, 500000.0, None, None,
+                                          C.byref(cfg)) == 0
+    tens = {n: torch.from_numpy(w[n]).cuda() for n in order}
+    tv = {n: _dev_tensor(t) for n, t in tens.items()}
+    wt = abi.BltTransformerWeights()
+    wt.norm1_weight, wt.attn_qkv_w, wt.attn_proj_w = C.pointer(tv["norm1"]), C.pointer(tv["qkv"]), C.pointer(tv["proj"])
+    wt.norm2_weight, wt.ffn_up_w, wt.ffn_gate_w = C.pointer(tv["norm2"]), C.pointer(tv["up"]), C.pointer(tv["gate"])
+    wt.ffn_down_w = C.pointer(tv["down"])
+    tc = abi.BltTransformerConfig()
+    ac = tc.attn_config
+    ac.embed_dim, ac.num_heads, ac.head_dim, ac.is_causal, ac.use_rope, ac.rope_theta = E, H, E // H, True, True, 500000.0
+    ac.mask_config = C.pointer(cfg)
+    tc.hidden_dim, tc.norm_type, tc.activation_type = hidden, abi.BLT_NORM_RMSNORM, abi.BLT_ACTIVATION_SWIGLU
+    tx = torch.from_numpy(x).cuda()
+    to = torch.full((T, E), 7.0, dtype=torch.float32, device="cuda")
+    vx, vo = _dev_tensor(tx), _dev_tensor(to)
+    arena = lib.blt_arena_create(256 << 20, abi.BLT_BACKEND_HIP)
+    try:
+        entry.blt_transformer_forward(C.byref(vx), C.byref(wt), C.byref(vo), C.byref(tc), arena)
+        lib.blt_backend_pass_sync_hip()
+        assert_close(to.cpu().numpy(), ref, "transformer block %s" % (shape,))
+    finally:
+        lib.blt_arena_destroy(arena)
+
+
+@pytest.mark.parametrize("P,E,H,hidden,L,docs", [(128, 512, 8, 1024, 2, [40, 90]),   # C2's caller: one window of patches
+                                                 (50, 64, 2, 96, 3, []), (200, 128, 4, 256, 1, [7, 8, 150])])
+def test_global_transformer_on_the_fused_block(P, E, H, hidden, L, docs, oracle, dev):
+    """The reference's patch transformer -- csrc/models/global_transformer.c:69-97 over
+    transformer_stack.c:228-248, both compiled unmodified -- with this library's
+    blt_transformer_forward under it (and blt_build_attention_mask, blt_rope_precompute,
+    blt_tensor_create, blt_strided_copy): the model is created in a device arena by the
+    reference's own constructor, filled with seeded weights, and compared with the restated
+    block applied layer by layer under the document-causal mask."""
+    import torch
+    lib = api.load()
+    stack_lib = binding.load_ref_stack_callers()
+    if stack_lib is None:
+        pytest.skip("oracle/_ref/libblt_ref_stack_callers.so was not built (needs the reference sources)")
+    rs = np.random.RandomState(P * 7 + E)
+    arena = lib.blt_arena_create(512 << 20, abi.BLT_BACKEND_HIP)
+    try:
+        cfg = binding.BltGlobalTransformerConfig(E, L, hidden, H, 500000.0, 256, False, False)
+        model = stack_lib.blt_global_transformer_create(arena, C.byref(cfg))
+        assert model.contents.stack.num_layers == L and model.contents.stack.head_dim == E // H
+        order = ("norm1_weight", "attn_qkv_w", "attn_proj_w", "norm2_weight", "ffn_up_w", "ffn_gate_w", "ffn_down_w")
+        layers = []
+        for l in range(L):
+            w = {"norm1_weight": (1.0 + 0.1 * rs.randn(E)), "attn_qkv_w": rs.randn(E, 3 * E) / np.sqrt(E),
+                 "attn_proj_w": rs.randn(E, E) / np.sqrt(E), "norm2_weight": (1.0 + 0.1 * rs.randn(E)),
+                 "ffn_up_w": rs.randn(E, hidden) / np.sqrt(E), "ffn_gate_w": rs.randn(E, hidden) / np.sqrt(E),
+                 "ffn_down_w": rs.randn(hidden, E) / np.sqrt(hidden)}
+            w = {n: np.ascontiguousarray(a, dtype=np.float32) for n, a in w.items()}
+            for n in order:
+                t = getattr(model.contents.stack.layer_weights[l], n)
+                assert tuple(t.contents.shape[:t.contents.ndim]) == w[n].shape
+                lib.blt_tensor_upload(t, w[n].ctypes.data, w[n].nbytes)
+            layers.append(w)
+        x = rs.randn(P, E).astype(np.float32)
+        tx = torch.from_numpy(x).cuda()
+        to = torch.full((P, E), 7.0, dtype=torch.float32, device="cuda")
+        vx, vo = _dev_tensor(tx), _dev_tensor(to)
+        bounds = abi.size_array(docs) if docs else None
+        stack_lib.blt_global_transformer_forward(model, C.byref(vx), bounds, len(docs) + 1 if docs else 0, C.byref(vo),
+                                                 arena)
+        lib.blt_backend_pass_sync_hip()
+        got = to.cpu().numpy()
+    finally:
+        lib.blt_arena_destroy(arena)
+    mc = abi.BltMaskConfig()
+    mc.seq_len_q = mc.seq_len_kv = P
+    mc.is_causal = True
+    if docs:
+        mc.doc_boundaries, mc.num_docs = bounds, len(docs) + 1
+    cur = x
+    for w in layers:
+        nxt = np.zeros((P, E), dtype=np.float32)
+        assert oracle.orc_transformer_forward(binding.fptr(cur.reshape(-1)), *(binding.fptr(w[n].reshape(-1)) for n in order),
+                                              binding.fptr(nxt.reshape(-1)), P, E, hidden, H, 1, 1, 500000.0, None, None,
+                                              C.byref(mc)) == 0
+        cur = nxt
+    assert_close(got, cur, "global transformer P=%d E=%d L=%d" % (P, E, L))
+
+
 # (patch lengths of the clean prefix, block rows, trailing_closed, d0 mode, how the block is filled)
 DIFFUSION_SCRIPTS = [
     ([3, 4, 2], 4, 1, abi.BLT_D0_ZEROS, "draft"),      # blt_draft_block's batch: all [MASK], positions N + r, o_M

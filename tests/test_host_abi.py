@@ -98,10 +98,13 @@ int main(void) {
     O(blt_local_decoder, lm_head_weight); O(blt_local_decoder, d0_embed_weight);
     S(blt_kv_cache); O(blt_kv_cache, k); O(blt_kv_cache, self_k); O(blt_kv_cache, self_len); O(blt_kv_cache, cross_k);
     O(blt_kv_cache, cross_num_patches); O(blt_kv_cache, cached_patches);
+    S(blt_transformer_config); O(blt_transformer_config, hidden_dim); O(blt_transformer_config, layer_norm_eps);
+    O(blt_transformer_config, norm_type); O(blt_transformer_config, activation_type); O(blt_transformer_config, use_bf16);
     S(blt_block_batch); O(blt_block_batch, t); O(blt_block_batch, tokens); O(blt_block_batch, positions);
     O(blt_block_batch, groups); O(blt_block_batch, loss_scale); O(blt_block_batch, trailing_closed);
     printf("enum %%d %%d %%d %%d %%d %%u\n", (int)BLT_XATTN_FIRST, (int)BLT_DTYPE_FP32, (int)BLT_BACKEND_CPU,
            (int)BLT_CROSS_ATTN_SPLIT_KV, (int)BLT_D0_LEARNED, (unsigned)BLT_MASK_TOKEN_ID);
+    printf("enum2 %%d %%d\n", (int)BLT_NORM_RMSNORM, (int)BLT_ACTIVATION_SWIGLU);
     return 0;
 }
 """

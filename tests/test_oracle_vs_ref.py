@@ -563,3 +563,45 @@ def test_diffusion_infer_bit_exact(case, script, oracle, ref):
     block = np.zeros((R, V), dtype=np.float32)
     assert oracle.orc_kv_block_step(cache.ptr, 0, N, P, batch.ptr, d0_mode, binding.fptr(block.reshape(-1))) == 0
     assert block.tobytes() == want[N:].tobytes(), (case, script, "block rows")
+
+
+# ---------------------------------------------------------------------------
+# the transformer block (csrc/models/transformer.c:97-128)
+# ---------------------------------------------------------------------------
+from tests.golden.block_cases import transformer_case  # noqa: E402
+
+
+TRANSFORMER_SHAPES = [(2, 8, 2, 12, "causal"), (33, 32, 4, 48, "window"), (70, 48, 3, 64, "docs"),
+                      (40, 64, 2, 96, "docs_window")]
+
+
+@pytest.mark.parametrize("shape", TRANSFORMER_SHAPES)
+def test_transformer_block_bit_exact(shape, oracle, ref):
+    """orc_transformer_forward against blt_transformer_forward compiled from the reference."""
+    T, E, H, hidden, mask = shape
+    rs = np.random.RandomState(T * 131 + E)
+    x, w, cfg, _keep = transformer_case(rs, T, E, H, hidden, mask)
+    mine = np.zeros((T, E), dtype=np.float32)
+    order = ("norm1", "qkv", "proj", "norm2", "up", "gate", "down")
+    assert oracle.orc_transformer_forward(binding.fptr(x.reshape(-1)), *(binding.fptr(w[n].reshape(-1)) for n in order),
+                                          binding.fptr(mine.reshape(-1)), T, E, hidden, H, 1, 1, 500000.0, None, None,
+                                          C.byref(cfg)) == 0
+    theirs = np.zeros((T, E), dtype=np.float32)
+    tv = {n: abi.tensor_view(w[n].ctypes.data, w[n].shape, CPU) for n in order}
+    wt = abi.BltTransformerWeights()
+    wt.norm1_weight, wt.attn_qkv_w, wt.attn_proj_w = C.pointer(tv["norm1"]), C.pointer(tv["qkv"]), C.pointer(tv["proj"])
+    wt.norm2_weight, wt.ffn_up_w, wt.ffn_gate_w = C.pointer(tv["norm2"]), C.pointer(tv["up"]), C.pointer(tv["gate"])
+    wt.ffn_down_w = C.pointer(tv["down"])
+    tc = abi.BltTransformerConfig()
+    ac = tc.attn_config
+    ac.embed_dim, ac.num_heads, ac.head_dim, ac.is_causal, ac.use_rope, ac.rope_theta = E, H, E // H, True, True, 500000.0
+    ac.mask_config = C.pointer(cfg)
+    tc.hidden_dim, tc.norm_type, tc.activation_type = hidden, abi.BLT_NORM_RMSNORM, abi.BLT_ACTIVATION_SWIGLU
+    tx, to = abi.tensor_view(x.ctypes.data, x.shape, CPU), abi.tensor_view(theirs.ctypes.data, theirs.shape, CPU)
+    arena = ref.blt_arena_create(64 << 20, CPU)
+    try:
+        ref.blt_transformer_forward(C.byref(tx), C.byref(wt), C.byref(to), C.byref(tc), arena)
+    finally:
+        ref.blt_arena_destroy(arena)
+    assert np.isfinite(theirs).all()
+    assert mine.tobytes() == theirs.tobytes(), shape
