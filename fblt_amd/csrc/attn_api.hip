@@ -2,7 +2,7 @@
  * Entry points of the attention forward path: the per-head device twin the
  * reference's dispatcher binds, the whole-batch launch and the resident plan.
  * Host code only (argument checks, descriptor translation, kernel choice);
- * the kernels live in attn_rows.hip, attn_mfma.hip and attn_wide.hip.
+ * the kernels live in attn_rows.hip, attn_mfma.hip, attn_wide.hip and attn_fine.hip.
  */
 #include "blt_hip.h"
 #include "blt_fatal.h"
@@ -19,7 +19,7 @@
 namespace {
 
 /* Kernel family a problem is routed to. */
-enum Family : uint32_t { FAM_ROWS = 0, FAM_MFMA = 1, FAM_WIDE = 2 };
+enum Family : uint32_t { FAM_ROWS = 0, FAM_MFMA = 1, FAM_WIDE = 2, FAM_FINE = 3 };
 
 struct Bucket {
     Family fam;
@@ -33,6 +33,7 @@ struct Bucket {
     uint32_t max_nq;
     uint32_t tiles;   /* mfma: number of work items; first item index in tile array = tile_base */
     uint32_t tile_base;
+    uint32_t span;    /* fine: keys the longest 32-row tile needs */
 };
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -105,7 +106,7 @@ AttnProb translate(const blt_attention_problem &pr, bool need_score_buffer, cons
     return d;
 }
 
-/* BLT_HIP_ATTN_FAMILY=rows|mfma|wide pins the kernel family wherever the
+/* BLT_HIP_ATTN_FAMILY=rows|mfma|wide|fine pins the kernel family wherever the
  * shape allows it (tuning and test hook); unset or anything else = automatic. */
 int family_override() {
     static const int cached = [] {
@@ -113,6 +114,7 @@ int family_override() {
         if (e && std::strcmp(e, "rows") == 0) return 1;
         if (e && std::strcmp(e, "mfma") == 0) return 2;
         if (e && std::strcmp(e, "wide") == 0) return 3;
+        if (e && std::strcmp(e, "fine") == 0) return 4;
         return 0;
     }();
     return cached;
@@ -145,7 +147,7 @@ uint32_t wide_min_groups(uint32_t max_nk) {
 /* Do problems p[0..n), all routed to the mfma family, go to the wide kernel instead? */
 bool choose_wide(const AttnProb *p, uint32_t n) {
     const int forced = family_override();
-    if (forced == 1 || forced == 2) return false;
+    if (forced == 1 || forced == 2 || forced == 4) return false;
     uint64_t groups = 0;
     uint32_t max_nk = 0;
     for (uint32_t i = 0; i < n; i++) {
@@ -154,6 +156,32 @@ bool choose_wide(const AttnProb *p, uint32_t n) {
         max_nk = std::max(max_nk, p[i].nk);
     }
     return forced == 3 || groups >= wide_min_groups(max_nk);
+}
+
+/* Do problems p[0..n), all routed to the mfma family, go to the fine kernel?  `span` gets the keys
+ * its longest 32-row tile needs.  Measured at head width 64, batches of (8 heads x) 4..128
+ * sequences of 64 and 128 rows: it is ahead of both other matrix-core kernels where one LDS fill
+ * holds every key a tile needs and the launch is neither tiny (up to one 4-wave workgroup per
+ * compute unit: the mfma kernel's shorter prologue wins from 128 keys on) nor so large that
+ * workgroups queue up behind each other several deep (the wide kernel overlaps its fetches with
+ * its arithmetic, this one fetches, then computes). */
+bool choose_fine(const AttnProb *p, uint32_t n, uint32_t &span) {
+    const int forced = family_override();
+    if (forced != 0 && forced != 4) return false;
+    span = 0;
+    uint64_t tiles = 0, groups = 0;
+    uint32_t max_nk = 0;
+    for (uint32_t i = 0; i < n; i++) {
+        if (!attn_fine_can(p[i])) return false;
+        span = std::max(span, attn_fine_span(p[i]));
+        tiles += (p[i].nq + 31u) / 32u;
+        groups += attn_wide_can(p[i]) ? attn_wide_groups(p[i]) : 0u;
+        max_nk = std::max(max_nk, p[i].nk);
+    }
+    if (forced == 4) return true;
+    if (span > attn_fine_fill_max(p[0].hd)) return false;
+    if (tiles <= 256u && span > 64u) return false;
+    return groups < (max_nk <= 64u ? 640u : 448u);
 }
 
 /* Element distance between two float pointers (either both NULL or both set). */
@@ -284,19 +312,24 @@ void plan_build(blt_attention_plan &pl, const blt_attention_problem *problems, s
     }
     for (Bucket &b : pl.buckets) {
         if (b.fam != FAM_MFMA) continue;
-        if (choose_wide(pl.host.data() + b.base, b.count)) b.fam = FAM_WIDE;
+        if (choose_fine(pl.host.data() + b.base, b.count, b.span)) b.fam = FAM_FINE;
+        else if (choose_wide(pl.host.data() + b.base, b.count)) b.fam = FAM_WIDE;
         b.affine = detect_affine(pl.host.data() + b.base, b.count, b.aff);
         if (b.affine) continue; /* no descriptor or tile memory needed */
         b.tile_base = (uint32_t)pl.tiles.size();
         if (b.fam == FAM_WIDE) attn_wide_make_tiles(pl.host.data(), b.base, b.count, pl.tiles);
+        else if (b.fam == FAM_FINE) attn_fine_make_tiles(pl.host.data(), b.base, b.count, pl.tiles);
         else attn_mfma_make_tiles(pl.host.data(), b.base, b.count, pl.tiles);
         b.tiles = (uint32_t)pl.tiles.size() - b.tile_base;
     }
-    bool any[3] = {false, false, false};
+    bool any[4] = {false, false, false, false};
     for (const Bucket &b : pl.buckets) any[b.fam] = true;
-    static const char *const names[8] = {"none",      "rows",      "mfma",      "mfma+rows",
-                                         "wide",      "wide+rows", "wide+mfma", "wide+mfma+rows"};
-    pl.kernel = names[(any[FAM_ROWS] ? 1 : 0) | (any[FAM_MFMA] ? 2 : 0) | (any[FAM_WIDE] ? 4 : 0)];
+    static const char *const names[16] = {"none",           "rows",           "mfma",           "mfma+rows",
+                                          "wide",           "wide+rows",      "wide+mfma",      "wide+mfma+rows",
+                                          "fine",           "fine+rows",      "fine+mfma",      "fine+mfma+rows",
+                                          "fine+wide",      "fine+wide+rows", "fine+wide+mfma", "fine+wide+mfma+rows"};
+    pl.kernel = names[(any[FAM_ROWS] ? 1 : 0) | (any[FAM_MFMA] ? 2 : 0) | (any[FAM_WIDE] ? 4 : 0) |
+                      (any[FAM_FINE] ? 8 : 0)];
 }
 
 void plan_launch(const blt_attention_plan &pl, const AttnProb *dev, const AttnTile *dev_tiles) {
@@ -305,6 +338,10 @@ void plan_launch(const blt_attention_plan &pl, const AttnProb *dev, const AttnTi
             attn_wide_launch_affine(b.aff, 0);
         else if (b.fam == FAM_WIDE)
             attn_wide_launch(dev, dev_tiles + b.tile_base, b.tiles, b.hd, b.dense, 0);
+        else if (b.fam == FAM_FINE && b.affine)
+            attn_fine_launch_affine(b.aff, 0);
+        else if (b.fam == FAM_FINE)
+            attn_fine_launch(dev, dev_tiles + b.tile_base, b.tiles, b.hd, b.span, 0);
         else if (b.fam == FAM_MFMA && b.affine)
             attn_mfma_launch_affine(b.aff, 0);
         else if (b.fam == FAM_MFMA)
@@ -370,7 +407,9 @@ extern "C" void blt_attention_head_core_hip(blt_backend backend, const blt_atten
     const AttnProb d = translate(pr, true, "blt_attention_head_core");
     if (d.nq == 0) return;
     const Family f = choose_family(d);
-    if (f == FAM_MFMA && choose_wide(&d, 1)) attn_wide_launch_single(d, 0);
+    uint32_t span = 0;
+    if (f == FAM_MFMA && choose_fine(&d, 1, span)) attn_fine_launch_single(d, 0);
+    else if (f == FAM_MFMA && choose_wide(&d, 1)) attn_wide_launch_single(d, 0);
     else if (f == FAM_MFMA) attn_mfma_launch_single(d, 0);
     else attn_rows_launch_single(d, 0);
     HIP_CHECK_LAUNCH("blt_attention_head_core");

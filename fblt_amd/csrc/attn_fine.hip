@@ -1,0 +1,464 @@
+/*
+ * "fine" kernel family: fused QK^T -> online softmax -> PV for prefill shapes
+ * whose launches hold about as many 32-row query tiles as the chip has
+ * compute-unit slots (a patch transformer over 128 patches, a few heads of a
+ * short byte window).  There a workgroup's time is the matrix-core time of its
+ * busiest SIMD, so the work is cut finer than a 32x32 score tile:
+ *
+ *   unit          = 16 query rows x 16 keys on v_mfma_f32_16x16x4_f32
+ *                   (HD/4 instructions for S^T, HD/4 for O^T);
+ *   workgroup     = one tile of 32 query rows, eight waves: waves 0..3 own rows
+ *                   0..15 of the tile, waves 4..7 rows 16..31;
+ *   unit -> wave  : the units of the tile are numbered row half by row half,
+ *                   key tile by key tile, and unit u goes to wave u % 4 of its
+ *                   row half, so the four SIMDs of the compute unit differ by at
+ *                   most one unit whatever the causal triangle leaves of each
+ *                   row half, and fully masked 16x16 corners are never computed.
+ *
+ * Every K and V row a tile needs is used by both row halves, so the workgroup
+ * fetches them once, with consecutive lanes on consecutive 16-byte pieces of a
+ * row, into LDS (rows padded by four floats: fragment reads of sixteen lanes
+ * fall on distinct banks); the waves read their fragments from there.  Keys
+ * beyond what one fill holds are walked in further fills.
+ *
+ * Both contractions are computed transposed, as in the other matrix-core
+ * kernels, so that a lane's scores, weights and output accumulators all
+ * belong to one query (column c = lane % 16):
+ *
+ *   S^T[key, query] = sum_d K[key, d] Q[query, d]        A = K,   B = Q^T
+ *   O^T[d,   query] = sum_key V[key, d] P^T[key, query]   A = V^T, B = P^T
+ *
+ * register r of lane (g = lane / 16, c) of an accumulator is row 4 g + r,
+ * column c.  The eight partial (max, sum, O) of a tile meet once in LDS.
+ *
+ * Takes closed-form visibility (all keys, causal with optional window), head
+ * widths 32 and 64 with 16-byte aligned rows, no weights output.
+ */
+#include "attn_device.h"
+#include "attn_launch.h"
+#include "attn_tile.h"
+#include "hip_check.h"
+#include "lane_ops.h"
+#include "launch.h"
+#include <algorithm>
+#include <cstdlib>
+
+namespace {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr uint32_t FINE_THREADS = 512;
+#ifndef FINE_PIECES_PER_STAGE
+#define FINE_PIECES_PER_STAGE 2 /* pieces of a fill parked between two barriers: 1, 2 or 4 */
+#endif
+constexpr uint32_t FINE_MIN_FILL = 64; /* keys an LDS fill holds at least (the merge needs that much) */
+/* keys one LDS fill holds at most: 4 float4 pieces of K and of V per thread */
+template <int HD>
+struct FineShape {
+    static constexpr int ROW = HD + 4;                        /* floats per parked row          */
+    static constexpr int LPR4 = HD / 4;                       /* 16-byte pieces per row         */
+    static constexpr int PIECES = 4;                          /* pieces per thread and matrix   */
+    static constexpr int KC_MAX = PIECES * FINE_THREADS / LPR4; /* 128 keys at 64, 256 at 32   */
+    static constexpr int MERGE_FLOATS = 8 * 16 * ROW;         /* eight partial tiles of 16 rows */
+};
+
+/* Query tile of the o-th workgroup of a problem with nqt tiles: the long tiles of a causal problem
+ * first, and tile t at the same distance from the start of its half of the order as tile
+ * nqt - 1 - t, so that workgroups dispatched half a launch apart add up to the same work. */
+__device__ __forceinline__ uint32_t fine_tile_order(uint32_t o, uint32_t nqt) {
+    const uint32_t first_half = (nqt + 1u) / 2u;
+    return o < first_half ? nqt - 1u - o : o - first_half;
+}
+
+/* Keys row i sees, [lo, hi), for the two visibility kinds the kernel takes; selects only. */
+__device__ __forceinline__ void fine_row_range(const AttnProb &p, uint32_t i, uint32_t &lo, uint32_t &hi) {
+    const bool causal = p.vis == ATTN_VIS_CAUSAL;
+    const uint32_t diag1 = i + p.causal_off + 1u; /* below 2^32: both terms are below 2^31 */
+    hi = causal ? min(p.nk, diag1) : p.nk;
+    lo = causal && p.window > 0u && diag1 > p.window ? min(diag1 - p.window, p.nk) : 0u;
+    lo = min(lo, hi);
+}
+
+/* Key span of rows [first, last]: keys any of them sees [tlo, thi) (thi <= tlo: none) and keys all of
+ * them see [flo, fhi); both ends of a row's range grow with the row. */
+__device__ __forceinline__ void fine_span(const AttnProb &p, uint32_t first, uint32_t last, uint32_t &tlo, uint32_t &thi,
+                                          uint32_t &flo, uint32_t &fhi) {
+    uint32_t lo_a, hi_a, lo_b, hi_b;
+    fine_row_range(p, first, lo_a, hi_a);
+    fine_row_range(p, last, lo_b, hi_b);
+    const bool any = hi_a > lo_a;
+    tlo = any ? lo_a : 0xFFFFFFFFu, thi = any ? hi_b : 0u;
+    flo = lo_b, fhi = hi_a;
+}
+
+template <int HD, int SRC>
+__global__ __launch_bounds__(FINE_THREADS, 4) void attn_fine_kernel(const AttnProb *__restrict__ probs,
+                                                                    const AttnTile *__restrict__ tiles,
+                                                                    AttnAffine aff, uint32_t kc) {
+    using Shape = FineShape<HD>;
+    constexpr int ROW = Shape::ROW;
+    constexpr int LPR4 = Shape::LPR4;
+    constexpr int QD = HD / 4;  /* columns of the head one lane group contracts */
+    constexpr int DT = HD / 16; /* 16-row tiles of O^T */
+
+    extern __shared__ __attribute__((aligned(16))) float sm[];
+    float *const sm_k = sm;
+    float *const sm_v = sm + (size_t)kc * ROW;
+
+    if (SRC != SRC_TILES) {
+        /* every kernel argument the workgroup will read is asked for here, in one go: left to
+         * itself the compiler fetches them group by group where they are first needed, and each
+         * group is a round trip through a cold scalar cache */
+        asm volatile("" ::"s"(aff.first.q), "s"(aff.first.k), "s"(aff.first.v), "s"(aff.first.out), "s"(aff.first.lse));
+        asm volatile("" ::"s"(aff.first.q_stride), "s"(aff.first.k_stride), "s"(aff.first.v_stride),
+                     "s"(aff.first.out_stride), "s"(aff.first.nq), "s"(aff.first.nk), "s"(aff.first.vis),
+                     "s"(aff.first.causal_off), "s"(aff.first.window), "s"(aff.first.scale));
+        asm volatile("" ::"s"(aff.q_seq), "s"(aff.q_head), "s"(aff.k_seq), "s"(aff.k_head), "s"(aff.v_seq),
+                     "s"(aff.v_head), "s"(aff.o_seq), "s"(aff.o_head), "s"(aff.lse_seq), "s"(aff.lse_head));
+        asm volatile("" ::"s"(aff.count), "s"(aff.heads), "s"(aff.nqt), "s"(kc));
+    }
+    uint32_t qtile;
+    AttnProb p;
+    if (SRC == SRC_TILES) {
+        qtile = tiles[blockIdx.x].qtile;
+        p = probs[tiles[blockIdx.x].prob];
+    } else if (SRC == SRC_SINGLE) {
+        qtile = fine_tile_order(blockIdx.x, gridDim.x);
+        p = aff.first;
+    } else {
+        const uint32_t prob = blockIdx.x % aff.count;
+        qtile = fine_tile_order(blockIdx.x / aff.count, aff.nqt);
+        affine_problem(p, aff, prob, false);
+    }
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t half = wave >> 2; /* row half of the tile */
+    const uint32_t wi = wave & 3u;   /* wave of the row half */
+    const uint32_t g = lane >> 4;
+    const uint32_t c = lane & 15u;
+
+    const uint32_t q0 = qtile * 32u;
+    const uint32_t last_row = min(q0 + 31u, p.nq - 1u);
+
+    /* keys the tile needs, as 16-key tiles [t0, t1) */
+    uint32_t tlo, thi, flo, fhi;
+    fine_span(p, q0, last_row, tlo, thi, flo, fhi);
+    const uint32_t t0 = thi > tlo ? tlo / 16u : 0u;
+    const uint32_t t1 = thi > tlo ? (thi + 15u) / 16u : 0u;
+
+    /* the row halves' own key tiles [h0, h1) and where their units start in the numbering */
+    uint32_t h0[2], h1[2];
+#pragma unroll
+    for (int a = 0; a < 2; a++) {
+        const uint32_t first = q0 + 16u * a;
+        h0[a] = h1[a] = 0;
+        if (first < p.nq) {
+            uint32_t lo_a, hi_a, f0, f1;
+            fine_span(p, first, min(first + 15u, p.nq - 1u), lo_a, hi_a, f0, f1);
+            if (hi_a > lo_a) h0[a] = lo_a / 16u, h1[a] = (hi_a + 15u) / 16u;
+        }
+    }
+    const uint32_t my0 = half ? h0[1] : h0[0], my1 = half ? h1[1] : h1[0];
+    /* this wave's key tiles: kt = wi - 2 half (mod 4), so that the units a stage of 32 keys completes
+     * (two key tiles, two row halves) fall on four different SIMDs */
+    uint32_t kt = my0 + ((wi - 2u * half - my0) & 3u);
+
+    /* this lane's query row and what it sees */
+    const uint32_t row = q0 + 16u * half + c;
+    const bool live = row < p.nq;
+    const uint32_t qi = live ? row : p.nq - 1u;
+    uint32_t lo, hi;
+    fine_row_range(p, qi, lo, hi);
+    if (!live) hi = lo;
+    /* keys every row of the half sees whole: no per-key test on those tiles */
+    uint32_t half_flo, half_fhi;
+    {
+        const uint32_t first = min(q0 + 16u * half, p.nq - 1u);
+        uint32_t a_, b_;
+        fine_span(p, first, min(first + 15u, p.nq - 1u), a_, b_, half_flo, half_fhi);
+        if (q0 + 16u * half + 15u >= p.nq) half_fhi = half_flo; /* padding rows see nothing */
+    }
+    const float scale2 = p.scale * LOG2E;
+
+    floatx4 oacc[DT];
+#pragma unroll
+    for (int d = 0; d < DT; d++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) oacc[d][r] = 0.f;
+    float m = neg_inf(), l = 0.f;
+
+    /* the query fragment: row c of the half, columns [g*QD, (g+1)*QD) */
+    float qf[QD];
+    {
+        const float *qrow = p.q + (size_t)qi * p.q_stride + g * QD;
+#pragma unroll
+        for (int s = 0; s < QD; s += 4) {
+            const float4 t = *reinterpret_cast<const float4 *>(qrow + s);
+            qf[s + 0] = t.x, qf[s + 1] = t.y, qf[s + 2] = t.z, qf[s + 3] = t.w;
+        }
+    }
+
+    /* ---- fill: rows [c0, c0 + kc) of K and V, clamped to the last row the tile needs; the first
+     * fill is requested here, the later ones at the end of the loop's body, so that nothing at the
+     * head of the loop waits for what the previous round left in flight ---- */
+    const uint32_t key_end = t1 * 16u;
+    const uint32_t last_key = min(max(key_end, 1u), p.nk) - 1u; /* row 0 when the tile sees nothing */
+    float4 kp[Shape::PIECES], vp[Shape::PIECES];
+    auto request = [&](uint32_t c0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < Shape::PIECES; t++) {
+            const uint32_t e = tid + FINE_THREADS * t;
+            const uint32_t r = e / LPR4, f = e % LPR4;
+            const uint32_t j = min(c0 + r, last_key);
+            kp[t] = *reinterpret_cast<const float4 *>(p.k + (size_t)j * p.k_stride + 4u * f);
+            vp[t] = *reinterpret_cast<const float4 *>(p.v + (size_t)j * p.v_stride + 4u * f);
+        }
+    };
+    uint32_t c0 = t0 * 16u;
+    request(c0); /* unconditionally: a branch here would make the code after it wait for every request */
+    /* the query fragment is pinned down here, where the compiler still counts the requests in flight
+     * one by one: inside the loops below a use of a value that is still on its way makes it wait for
+     * every request, the later pieces of the fill included */
+#pragma unroll
+    for (int s = 0; s < QD; s++) asm volatile("" : "+v"(qf[s]));
+    while (c0 < key_end) {
+        /* ---- the pieces land in the order they were requested: piece by piece, park it and work
+         * on the key tiles it completes while the later pieces are still on their way ---- */
+        const uint32_t fill_end = min(c0 + kc, key_end);
+        constexpr uint32_t RPP = FINE_THREADS / LPR4; /* rows per piece */
+        auto park = [&](const uint32_t pc, const float4 k_piece, const float4 v_piece) __attribute__((always_inline)) {
+            const uint32_t e = tid + FINE_THREADS * pc;
+            const uint32_t r = e / LPR4, f = e % LPR4;
+            /* a fill holds 64 keys at least: no test (and nothing for the compiler to sink the
+             * piece's loads behind) on the pieces below that */
+            if (RPP * (pc + 1u) <= FINE_MIN_FILL || r < kc) {
+                *reinterpret_cast<float4 *>(sm_k + r * ROW + 4u * f) = k_piece;
+                *reinterpret_cast<float4 *>(sm_v + r * ROW + 4u * f) = v_piece;
+            }
+        };
+        /* one stage = the units of the key tiles that pieces [0, pieces_done) complete */
+        auto stage = [&](const uint32_t pieces_done) __attribute__((always_inline)) {
+            __syncthreads();
+            const uint32_t stage_end = min(c0 + RPP * pieces_done, fill_end);
+            while (kt < my1 && kt * 16u < stage_end) {
+                const uint32_t k0 = kt * 16u;
+                const float *krow = sm_k + (k0 - c0 + c) * ROW + g * QD;
+                const float *vrow = sm_v + (k0 - c0 + 4u * g) * ROW + c;
+                float kf[QD];
+#pragma unroll
+                for (int s = 0; s < QD; s += 4) {
+                    const float4 t = *reinterpret_cast<const float4 *>(krow + s);
+                    kf[s + 0] = t.x, kf[s + 1] = t.y, kf[s + 2] = t.z, kf[s + 3] = t.w;
+                }
+                float vf[DT][4];
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+#pragma unroll
+                    for (int d = 0; d < DT; d++) vf[d][r] = vrow[r * ROW + 16 * d];
+
+                /* S^T on two accumulators: neither chain waits for its own previous result */
+                floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < QD; s += 2) {
+                    s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[s], qf[s], s0, 0, 0, 0);
+                    s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[s + 1], qf[s + 1], s1, 0, 0, 0);
+                }
+
+                const bool all_seen = k0 >= half_flo && k0 + 16u <= half_fhi; /* uniform over the wave */
+                const uint32_t vlo = all_seen ? 0u : lo;
+                const uint32_t vlen = all_seen ? 0xFFFFFFFFu : (hi > lo ? hi - lo : 0u);
+                float x[4];
+                float mt = neg_inf();
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const float t = (s0[r] + s1[r]) * scale2;
+                    const bool vis = ((k0 + 4u * g + r - vlo) < vlen) & isfinite(t);
+                    x[r] = vis ? t : neg_inf();
+                    mt = fmaxf(mt, x[r]);
+                }
+                mt = swap32(swap16(mt, OpMax()), OpMax());
+                const float mn = fmaxf(m, mt);
+                const float ms = mn == neg_inf() ? 0.f : mn;
+                const float alpha = fast_exp2(m - ms);
+                float ps = 0.f;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    x[r] = fast_exp2(x[r] - ms);
+                    ps += x[r];
+                }
+                l = l * alpha + ps;
+                m = mn;
+#pragma unroll
+                for (int d = 0; d < DT; d++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) oacc[d][r] *= alpha;
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+#pragma unroll
+                    for (int d = 0; d < DT; d++)
+                        oacc[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[d][r], x[r], oacc[d], 0, 0, 0);
+                kt += 4u;
+            }
+            return c0 + RPP * pieces_done < fill_end; /* more keys to come: uniform over the workgroup */
+        };
+        static_assert(Shape::PIECES == 4, "four pieces are spelled out");
+        if (FINE_PIECES_PER_STAGE == 1) {
+            park(0, kp[0], vp[0]);
+            if (stage(1)) {
+                park(1, kp[1], vp[1]);
+                if (stage(2)) {
+                    park(2, kp[2], vp[2]);
+                    if (stage(3)) {
+                        park(3, kp[3], vp[3]);
+                        stage(4);
+                    }
+                }
+            }
+        } else if (FINE_PIECES_PER_STAGE == 2) {
+            park(0, kp[0], vp[0]);
+            park(1, kp[1], vp[1]);
+            if (stage(2)) {
+                park(2, kp[2], vp[2]);
+                park(3, kp[3], vp[3]);
+                stage(4);
+            }
+        } else {
+            park(0, kp[0], vp[0]);
+            park(1, kp[1], vp[1]);
+            park(2, kp[2], vp[2]);
+            park(3, kp[3], vp[3]);
+            stage(4);
+        }
+        __syncthreads(); /* the fill is consumed: the next fill, or the merge, may overwrite it */
+        c0 += kc;
+        if (c0 < key_end) request(c0);
+    }
+
+    /* the four lane groups of a column carry the same m, their sums add */
+    l = swap32(swap16(l, OpSum()), OpSum());
+
+    /* ---- merge: every wave parks [16 queries][HD columns, max, sum] ---- */
+    float *mine = sm + wave * (16 * ROW);
+#pragma unroll
+    for (int d = 0; d < DT; d++)
+        *reinterpret_cast<float4 *>(mine + c * ROW + 16 * d + 4 * g) =
+            make_float4(oacc[d][0], oacc[d][1], oacc[d][2], oacc[d][3]);
+    if (g == 0) *reinterpret_cast<float2 *>(mine + c * ROW + HD) = make_float2(m, l);
+    __syncthreads();
+
+    /* 256 threads per row half: thread = (row, 16-byte piece of the row) */
+    const uint32_t mh = tid >> 8, idx = tid & 255u;
+    const uint32_t mr = idx / LPR4, mf = idx % LPR4;
+    if (mr < 16u) {
+        const float *part = sm + (4u * mh) * (16 * ROW) + mr * ROW;
+        float pm[4], pl[4];
+        float M = neg_inf();
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float2 t = *reinterpret_cast<const float2 *>(part + w * (16 * ROW) + HD);
+            pm[w] = t.x, pl[w] = t.y;
+            M = fmaxf(M, pm[w]);
+        }
+        const float Ms = M == neg_inf() ? 0.f : M;
+        float L = 0.f;
+        float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float f = fast_exp2(pm[w] - Ms);
+            const float4 t = *reinterpret_cast<const float4 *>(part + w * (16 * ROW) + 4u * mf);
+            L += pl[w] * f;
+            o.x += t.x * f, o.y += t.y * f, o.z += t.z * f, o.w += t.w * f;
+        }
+        const float inv = L > 0.f ? 1.0f / L : 0.f;
+        const uint32_t orow = q0 + 16u * mh + mr;
+        if (orow < p.nq) {
+            *reinterpret_cast<float4 *>(p.out + (size_t)orow * p.out_stride + 4u * mf) =
+                make_float4(o.x * inv, o.y * inv, o.z * inv, o.w * inv);
+            if (mf == 0 && p.lse) {
+                p.lse[2 * (size_t)orow + 0] = M * LN2; /* back to natural units */
+                p.lse[2 * (size_t)orow + 1] = L;
+            }
+        }
+    }
+}
+
+/* keys per fill for a launch whose longest tile needs `span` keys, and the LDS that takes */
+template <int HD>
+uint32_t fine_fill_keys(uint32_t span) {
+    using Shape = FineShape<HD>;
+    const uint32_t want = std::max<uint32_t>(16u, (span + 15u) / 16u * 16u + 16u); /* a span may straddle a tile */
+    static_assert(2 * FINE_MIN_FILL * Shape::ROW >= Shape::MERGE_FLOATS, "the merge overlays the fill");
+    return std::min<uint32_t>(Shape::KC_MAX, std::max<uint32_t>(FINE_MIN_FILL, want));
+}
+
+template <int HD, int SRC>
+void fine_launch_as(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t nblocks, const AttnAffine &aff,
+                    uint32_t span, hipStream_t s) {
+    using Shape = FineShape<HD>;
+    const uint32_t kc = fine_fill_keys<HD>(span);
+    const size_t lds = (size_t)2 * kc * Shape::ROW * sizeof(float);
+    static const bool raised = [] { /* more than the 64 KB a kernel may use without asking */
+        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_fine_kernel<HD, SRC>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      2 * Shape::KC_MAX * Shape::ROW * (int)sizeof(float)));
+        return true;
+    }();
+    (void)raised;
+    blt_launch("attn_fine", attn_fine_kernel<HD, SRC>, dim3(nblocks), dim3(FINE_THREADS), lds, s, dprobs, dtiles, aff,
+               kc);
+}
+
+template <int SRC>
+void fine_launch_hd(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t nblocks, const AttnAffine &aff,
+                    uint32_t hd, uint32_t span, hipStream_t s) {
+    if (hd == 32u) fine_launch_as<32, SRC>(dprobs, dtiles, nblocks, aff, span, s);
+    else fine_launch_as<64, SRC>(dprobs, dtiles, nblocks, aff, span, s);
+}
+
+} // namespace
+
+/* Keys the longest 32-row tile of the problem needs. */
+uint32_t attn_fine_span(const AttnProb &d) {
+    if (d.vis != ATTN_VIS_CAUSAL) return d.nk;
+    if (d.window > 0) return std::min<uint64_t>(d.nk, (uint64_t)d.window + 31u);
+    return (uint32_t)std::min<uint64_t>(d.nk, (uint64_t)d.nq + d.causal_off);
+}
+
+/* keys one LDS fill holds at head width hd */
+uint32_t attn_fine_fill_max(uint32_t hd) { return hd == 32u ? FineShape<32>::KC_MAX : FineShape<64>::KC_MAX; }
+
+/* shapes the kernel is able to run */
+bool attn_fine_can(const AttnProb &d) {
+    return (d.hd == 32u || d.hd == 64u) && (d.flags & ATTN_FLAG_VEC4) != 0 && d.weights == nullptr &&
+           (d.vis == ATTN_VIS_ALL || d.vis == ATTN_VIS_CAUSAL) && d.nq >= 1u && d.nk >= 1u;
+}
+
+/* Work items for problems [base, base+count), longest first. */
+void attn_fine_make_tiles(const AttnProb *host, uint32_t base, uint32_t count, std::vector<AttnTile> &tiles) {
+    attn_mfma_make_tiles(host, base, count, tiles);
+}
+
+void attn_fine_launch(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t ntiles, uint32_t hd, uint32_t span,
+                      hipStream_t s) {
+    if (ntiles == 0) return;
+    AttnAffine none;
+    __builtin_memset(&none, 0, sizeof(none));
+    fine_launch_hd<SRC_TILES>(dprobs, dtiles, ntiles, none, hd, span, s);
+}
+
+void attn_fine_launch_single(const AttnProb &single, hipStream_t s) {
+    const uint32_t ntiles = (single.nq + 31u) / 32u;
+    if (ntiles == 0) return;
+    AttnAffine a;
+    __builtin_memset(&a, 0, sizeof(a));
+    a.first = single;
+    fine_launch_hd<SRC_SINGLE>(nullptr, nullptr, ntiles, a, single.hd, attn_fine_span(single), s);
+}
+
+void attn_fine_launch_affine(const AttnAffine &aff, hipStream_t s) {
+    const uint32_t blocks = aff.count * aff.nqt;
+    if (blocks == 0) return;
+    fine_launch_hd<SRC_AFFINE>(nullptr, nullptr, blocks, aff, aff.first.hd, attn_fine_span(aff.first), s);
+}

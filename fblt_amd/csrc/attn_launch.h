@@ -53,4 +53,15 @@ void attn_wide_launch(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t n
 void attn_wide_launch_single(const AttnProb &single, hipStream_t s);
 void attn_wide_launch_affine(const AttnAffine &aff, hipStream_t s);
 
+/* fine family: 32-row tiles cut into 16 x 16 units over eight waves, K/V rows of a tile shared
+ * through LDS; `span` = keys the longest tile of the launch needs */
+bool attn_fine_can(const AttnProb &d);
+uint32_t attn_fine_span(const AttnProb &d);
+uint32_t attn_fine_fill_max(uint32_t hd);
+void attn_fine_make_tiles(const AttnProb *host, uint32_t base, uint32_t count, std::vector<AttnTile> &tiles);
+void attn_fine_launch(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t ntiles, uint32_t hd, uint32_t span,
+                      hipStream_t s);
+void attn_fine_launch_single(const AttnProb &single, hipStream_t s);
+void attn_fine_launch_affine(const AttnAffine &aff, hipStream_t s);
+
 #endif

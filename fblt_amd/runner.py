@@ -193,6 +193,13 @@ class DeviceKvWorkload:
         self.c.batch, self.c.max_seq_len = kw.batch, kw.max_seq_len
         self.c.embed_dim, self.c.num_heads, self.c.window = kw.E, kw.H, kw.window
         self.kind = api.BLT_KV_STEP_CAUSAL if kw.kind == "causal" else api.BLT_KV_STEP_BLOCK
+        # addresses of every step's rows, taken once: slicing a tensor per step costs more host
+        # time than the step's launch
+        self._rows = [tuple(t[s].data_ptr() for t in (self.q_new, self.k_new, self.v_new, self.out))
+                      for s in range(kw.steps)]
+        self._cache_ref = C.byref(self.c)
+        self._rope_args = ((self.rope[0].data_ptr(), self.rope[1].data_ptr(), self.rope[0].shape[0])
+                           if self.rope is not None else (None, None, 0))
 
     def reset(self):
         """Lengths back to the start; cache rows past them are dead by contract."""
@@ -205,24 +212,19 @@ class DeviceKvWorkload:
         kw = self.kw
         E = kw.E
         hint = self.host_max_len + kw.n
+        q, k, v, out = self._rows[s]
+        cos, sin, rows = self._rope_args
         if self.lens_mode == "host":
-            cos, sin, rows = ((self.rope[0].data_ptr(), self.rope[1].data_ptr(), self.rope[0].shape[0])
-                              if self.rope is not None else (None, None, 0))
-            self.lib.blt_kv_attend_step_lens_hip(C.byref(self.c), self._host_lens_p, self.q_new[s].data_ptr(), E,
-                                                 self.k_new[s].data_ptr(), E, self.v_new[s].data_ptr(), E, cos, sin,
-                                                 rows, self.out[s].data_ptr(), E, kw.n, self.kind)
+            self.lib.blt_kv_attend_step_lens_hip(self._cache_ref, self._host_lens_p, q, E, k, E, v, E, cos, sin, rows,
+                                                 out, E, kw.n, self.kind)
             if kw.commit:  # the caller advances its lengths, as the reference does after a step
                 self.host_lens += np.uint32(kw.n)
         elif self.rope is not None:
-            self.lib.blt_kv_rope_attend_step_hip(C.byref(self.c), self.q_new[s].data_ptr(), E,
-                                                 self.k_new[s].data_ptr(), E, self.v_new[s].data_ptr(), E,
-                                                 self.rope[0].data_ptr(), self.rope[1].data_ptr(),
-                                                 self.rope[0].shape[0], self.out[s].data_ptr(), E, kw.n, self.kind,
-                                                 1 if kw.commit else 0, hint)
+            self.lib.blt_kv_rope_attend_step_hip(self._cache_ref, q, E, k, E, v, E, cos, sin, rows, out, E, kw.n,
+                                                 self.kind, 1 if kw.commit else 0, hint)
         else:
-            self.lib.blt_kv_attend_step_hip(C.byref(self.c), self.q_new[s].data_ptr(), E, self.k_new[s].data_ptr(),
-                                            E, self.v_new[s].data_ptr(), E, self.out[s].data_ptr(), E, kw.n,
-                                            self.kind, 1 if kw.commit else 0, hint)
+            self.lib.blt_kv_attend_step_hip(self._cache_ref, q, E, k, E, v, E, out, E, kw.n, self.kind,
+                                            1 if kw.commit else 0, hint)
         if kw.commit:
             self.host_max_len += kw.n
 

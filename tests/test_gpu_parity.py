@@ -726,7 +726,7 @@ def test_kv_step_kernel_families_agree(kernel):
     assert p.returncode == 0 and "OK" in p.stdout, p.stdout[-2000:] + p.stderr[-2000:]
 
 
-@pytest.mark.parametrize("family", ["rows", "mfma", "wide"])
+@pytest.mark.parametrize("family", ["rows", "mfma", "wide", "fine"])
 def test_attention_kernel_families(family):
     """Every attention kernel family on the same cases (causal, chunked prefill, sliding window,
     dense masks, lse output), pinned through BLT_HIP_ATTN_FAMILY in a fresh process."""
