@@ -34,6 +34,7 @@ struct Bucket {
     uint32_t tiles;   /* mfma: number of work items; first item index in tile array = tile_base */
     uint32_t tile_base;
     uint32_t span;    /* fine: keys the longest 32-row tile needs */
+    bool tall;        /* fine: 16-row workgroups of sixteen waves */
 };
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -158,15 +159,29 @@ bool choose_wide(const AttnProb *p, uint32_t n) {
     return forced == 3 || groups >= wide_min_groups(max_nk);
 }
 
-/* Do problems p[0..n), all routed to the mfma family, go to the fine kernel?  `span` gets the keys
- * its longest 32-row tile needs.  Measured at head width 64, batches of (8 heads x) 4..128
- * sequences of 64 and 128 rows: it is ahead of both other matrix-core kernels where one LDS fill
- * holds every key a tile needs and the launch is neither tiny (up to one 4-wave workgroup per
- * compute unit: the mfma kernel's shorter prologue wins from 128 keys on) nor so large that
- * workgroups queue up behind each other several deep (the wide kernel overlaps its fetches with
- * its arithmetic, this one fetches, then computes). */
-bool choose_fine(const AttnProb *p, uint32_t n, uint32_t &span) {
+/* Do problems p[0..n), all routed to the mfma family, go to the fine kernel, and in which workgroup
+ * shape?  `span` gets the keys its longest 32-row tile needs.  Measured at both head widths (4 heads
+ * of 32, 8 heads of 64), 1..128 sequences of 64..2048 rows, against the other two matrix-core
+ * kernels:
+ *   - few long problems (at most 128 tiles of 32 rows, rows of 256 keys and more): workgroups of 16
+ *     rows and sixteen waves double the workgroups and halve the chain of matrix instructions on the
+ *     busiest SIMD (512 rows x 4 heads: 8.9 -> 8.0 us; 1024 rows: 15.1 -> 11.7 us).  Only strided
+ *     batches and single problems have this shape;
+ *   - one LDS fill holds every key a tile needs (128 keys at width 64, 256 at 32): ahead unless the
+ *     launch is tiny (up to one 4-wave workgroup per compute unit: the mfma kernel's shorter
+ *     prologue wins from 128 keys on) or so large that workgroups queue up several deep (the wide
+ *     kernel overlaps its fetches with its arithmetic, this one fetches, then computes);
+ *   - longer rows when the launch is just what the chip holds at once, two 8-wave workgroups per
+ *     compute unit (512 tiles: 10..25 % ahead of the mfma kernel, behind it at 256 and at 1024). */
+bool choose_fine(const AttnProb *p, uint32_t n, bool strided, uint32_t &span, bool &tall) {
+    /* BLT_HIP_FINE_ROWS=16|32 pins the workgroup shape (tuning and test hook) */
+    static const int rows_pinned = [] {
+        const char *e = getenv("BLT_HIP_FINE_ROWS");
+        const int v = e ? std::atoi(e) : 0;
+        return v == 16 || v == 32 ? v : 0;
+    }();
     const int forced = family_override();
+    tall = false;
     if (forced != 0 && forced != 4) return false;
     span = 0;
     uint64_t tiles = 0, groups = 0;
@@ -178,8 +193,16 @@ bool choose_fine(const AttnProb *p, uint32_t n, uint32_t &span) {
         groups += attn_wide_can(p[i]) ? attn_wide_groups(p[i]) : 0u;
         max_nk = std::max(max_nk, p[i].nk);
     }
-    if (forced == 4) return true;
-    if (span > attn_fine_fill_max(p[0].hd)) return false;
+    const bool tall_fits = strided && tiles <= 128u && span >= 256u;
+    if (forced == 4) {
+        tall = strided && (rows_pinned == 16 || (rows_pinned == 0 && tall_fits));
+        return true;
+    }
+    if (rows_pinned != 32 && (tall_fits || (rows_pinned == 16 && strided))) {
+        tall = true;
+        return true;
+    }
+    if (span > attn_fine_fill_max(p[0].hd)) return tiles > 448u && tiles <= 512u;
     if (tiles <= 256u && span > 64u) return false;
     return groups < (max_nk <= 64u ? 640u : 448u);
 }
@@ -312,9 +335,9 @@ void plan_build(blt_attention_plan &pl, const blt_attention_problem *problems, s
     }
     for (Bucket &b : pl.buckets) {
         if (b.fam != FAM_MFMA) continue;
-        if (choose_fine(pl.host.data() + b.base, b.count, b.span)) b.fam = FAM_FINE;
-        else if (choose_wide(pl.host.data() + b.base, b.count)) b.fam = FAM_WIDE;
         b.affine = detect_affine(pl.host.data() + b.base, b.count, b.aff);
+        if (choose_fine(pl.host.data() + b.base, b.count, b.affine, b.span, b.tall)) b.fam = FAM_FINE;
+        else if (choose_wide(pl.host.data() + b.base, b.count)) b.fam = FAM_WIDE;
         if (b.affine) continue; /* no descriptor or tile memory needed */
         b.tile_base = (uint32_t)pl.tiles.size();
         if (b.fam == FAM_WIDE) attn_wide_make_tiles(pl.host.data(), b.base, b.count, pl.tiles);
@@ -339,7 +362,7 @@ void plan_launch(const blt_attention_plan &pl, const AttnProb *dev, const AttnTi
         else if (b.fam == FAM_WIDE)
             attn_wide_launch(dev, dev_tiles + b.tile_base, b.tiles, b.hd, b.dense, 0);
         else if (b.fam == FAM_FINE && b.affine)
-            attn_fine_launch_affine(b.aff, 0);
+            attn_fine_launch_affine(b.aff, b.tall, 0);
         else if (b.fam == FAM_FINE)
             attn_fine_launch(dev, dev_tiles + b.tile_base, b.tiles, b.hd, b.span, 0);
         else if (b.fam == FAM_MFMA && b.affine)
@@ -408,7 +431,8 @@ extern "C" void blt_attention_head_core_hip(blt_backend backend, const blt_atten
     if (d.nq == 0) return;
     const Family f = choose_family(d);
     uint32_t span = 0;
-    if (f == FAM_MFMA && choose_fine(&d, 1, span)) attn_fine_launch_single(d, 0);
+    bool tall = false;
+    if (f == FAM_MFMA && choose_fine(&d, 1, true, span, tall)) attn_fine_launch_single(d, tall, 0);
     else if (f == FAM_MFMA && choose_wide(&d, 1)) attn_wide_launch_single(d, 0);
     else if (f == FAM_MFMA) attn_mfma_launch_single(d, 0);
     else attn_rows_launch_single(d, 0);

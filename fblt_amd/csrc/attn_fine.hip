@@ -31,6 +31,14 @@
  * register r of lane (g = lane / 16, c) of an accumulator is row 4 g + r,
  * column c.  The eight partial (max, sum, O) of a tile meet once in LDS.
  *
+ * A second shape of the same kernel serves launches with few, long problems (a
+ * byte window of 512 rows over 4 heads: 64 tiles of 32 rows on 256 compute
+ * units): the workgroup is one tile of 16 query rows and all of its sixteen
+ * waves take key tiles of those rows, so the launch has twice the workgroups,
+ * each with half the matrix-core work and four waves per SIMD to hide a unit's
+ * latency chain; the next fill is requested before the units of the current one
+ * start.
+ *
  * Takes closed-form visibility (all keys, causal with optional window), head
  * widths 32 and 64 with 16-byte aligned rows, no weights output.
  */
@@ -47,19 +55,24 @@ namespace {
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-constexpr uint32_t FINE_THREADS = 512;
-#ifndef FINE_PIECES_PER_STAGE
-#define FINE_PIECES_PER_STAGE 2 /* pieces of a fill parked between two barriers: 1, 2 or 4 */
-#endif
-constexpr uint32_t FINE_MIN_FILL = 64; /* keys an LDS fill holds at least (the merge needs that much) */
-/* keys one LDS fill holds at most: 4 float4 pieces of K and of V per thread */
-template <int HD>
+/* HALVES row halves of 16 query rows per workgroup, WAVES waves in all (WAVES / HALVES per half). */
+template <int HD, int HALVES, int WAVES>
 struct FineShape {
-    static constexpr int ROW = HD + 4;                        /* floats per parked row          */
-    static constexpr int LPR4 = HD / 4;                       /* 16-byte pieces per row         */
-    static constexpr int PIECES = 4;                          /* pieces per thread and matrix   */
-    static constexpr int KC_MAX = PIECES * FINE_THREADS / LPR4; /* 128 keys at 64, 256 at 32   */
-    static constexpr int MERGE_FLOATS = 8 * 16 * ROW;         /* eight partial tiles of 16 rows */
+    static constexpr uint32_t THREADS = 64u * WAVES;
+    static constexpr int ROW = HD + 4;  /* floats per parked row  */
+    static constexpr int LPR4 = HD / 4; /* 16-byte pieces per row */
+    /* keys one LDS fill holds at most (K and V together: 68 KB at 64 columns, 72 KB at 32) */
+    static constexpr uint32_t KC_MAX = HD == 64 ? 128u : 256u;
+    static constexpr int PIECES = (int)(KC_MAX * LPR4 / THREADS); /* 16-byte pieces per thread and matrix */
+    static constexpr uint32_t RPP = THREADS / LPR4;               /* rows per piece                      */
+    /* a fill is parked and worked on in two stages where each wave finds a unit in either (eight
+     * waves, two halves); with sixteen waves on one half a stage would leave half of them idle */
+    static constexpr int STAGES = WAVES == 8 ? 2 : 1;
+    static constexpr int MERGE_FLOATS = WAVES * 16 * ROW; /* one partial tile of 16 rows per wave */
+    /* keys a fill holds at least: the merge overlays it */
+    static constexpr uint32_t MIN_FILL = (MERGE_FLOATS + 2 * ROW - 1) / (2 * ROW);
+    static_assert(PIECES * THREADS == KC_MAX * LPR4 && PIECES % STAGES == 0, "pieces tile the fill");
+    static_assert(MIN_FILL % 16 == 0 && MIN_FILL <= KC_MAX, "the merge fits the smallest fill");
 };
 
 /* Query tile of the o-th workgroup of a problem with nqt tiles: the long tiles of a causal problem
@@ -91,11 +104,14 @@ __device__ __forceinline__ void fine_span(const AttnProb &p, uint32_t first, uin
     flo = lo_b, fhi = hi_a;
 }
 
-template <int HD, int SRC>
-__global__ __launch_bounds__(FINE_THREADS, 4) void attn_fine_kernel(const AttnProb *__restrict__ probs,
-                                                                    const AttnTile *__restrict__ tiles,
-                                                                    AttnAffine aff, uint32_t kc) {
-    using Shape = FineShape<HD>;
+template <int HD, int SRC, int HALVES, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 4) void attn_fine_kernel(const AttnProb *__restrict__ probs,
+                                                                  const AttnTile *__restrict__ tiles, AttnAffine aff,
+                                                                  uint32_t kc) {
+    using Shape = FineShape<HD, HALVES, WAVES>;
+    constexpr uint32_t FINE_THREADS = Shape::THREADS;
+    constexpr uint32_t ROWS = 16u * HALVES; /* query rows of a workgroup            */
+    constexpr uint32_t WPH = WAVES / HALVES; /* waves of a row half (a power of two) */
     constexpr int ROW = Shape::ROW;
     constexpr int LPR4 = Shape::LPR4;
     constexpr int QD = HD / 4;  /* columns of the head one lane group contracts */
@@ -127,20 +143,20 @@ __global__ __launch_bounds__(FINE_THREADS, 4) void attn_fine_kernel(const AttnPr
         p = aff.first;
     } else {
         const uint32_t prob = blockIdx.x % aff.count;
-        qtile = fine_tile_order(blockIdx.x / aff.count, aff.nqt);
+        qtile = fine_tile_order(blockIdx.x / aff.count, (aff.first.nq + ROWS - 1u) / ROWS);
         affine_problem(p, aff, prob, false);
     }
 
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t half = wave >> 2; /* row half of the tile */
-    const uint32_t wi = wave & 3u;   /* wave of the row half */
+    const uint32_t half = HALVES == 1 ? 0u : wave / WPH; /* row half of the tile */
+    const uint32_t wi = wave & (WPH - 1u);               /* wave of the row half */
     const uint32_t g = lane >> 4;
     const uint32_t c = lane & 15u;
 
-    const uint32_t q0 = qtile * 32u;
-    const uint32_t last_row = min(q0 + 31u, p.nq - 1u);
+    const uint32_t q0 = qtile * ROWS;
+    const uint32_t last_row = min(q0 + ROWS - 1u, p.nq - 1u);
 
     /* keys the tile needs, as 16-key tiles [t0, t1) */
     uint32_t tlo, thi, flo, fhi;
@@ -148,22 +164,18 @@ __global__ __launch_bounds__(FINE_THREADS, 4) void attn_fine_kernel(const AttnPr
     const uint32_t t0 = thi > tlo ? tlo / 16u : 0u;
     const uint32_t t1 = thi > tlo ? (thi + 15u) / 16u : 0u;
 
-    /* the row halves' own key tiles [h0, h1) and where their units start in the numbering */
-    uint32_t h0[2], h1[2];
-#pragma unroll
-    for (int a = 0; a < 2; a++) {
-        const uint32_t first = q0 + 16u * a;
-        h0[a] = h1[a] = 0;
-        if (first < p.nq) {
-            uint32_t lo_a, hi_a, f0, f1;
-            fine_span(p, first, min(first + 15u, p.nq - 1u), lo_a, hi_a, f0, f1);
-            if (hi_a > lo_a) h0[a] = lo_a / 16u, h1[a] = (hi_a + 15u) / 16u;
-        }
+    /* this wave's row half: its own key tiles [my0, my1) */
+    uint32_t my0 = 0, my1 = 0;
+    {
+        const uint32_t first = q0 + 16u * half;
+        uint32_t lo_a, hi_a, f0, f1;
+        fine_span(p, min(first, p.nq - 1u), min(first + 15u, p.nq - 1u), lo_a, hi_a, f0, f1);
+        if (first < p.nq && hi_a > lo_a) my0 = lo_a / 16u, my1 = (hi_a + 15u) / 16u;
     }
-    const uint32_t my0 = half ? h0[1] : h0[0], my1 = half ? h1[1] : h1[0];
-    /* this wave's key tiles: kt = wi - 2 half (mod 4), so that the units a stage of 32 keys completes
-     * (two key tiles, two row halves) fall on four different SIMDs */
-    uint32_t kt = my0 + ((wi - 2u * half - my0) & 3u);
+    /* this wave's key tiles: kt = wi - 2 half (mod WPH), one in every WPH; with two halves of four
+     * waves the units a stage of 32 keys completes (two key tiles, two row halves) fall on four
+     * different SIMDs */
+    uint32_t kt = my0 + ((wi - 2u * half - my0) & (WPH - 1u));
 
     /* this lane's query row and what it sees */
     const uint32_t row = q0 + 16u * half + c;
@@ -227,13 +239,13 @@ __global__ __launch_bounds__(FINE_THREADS, 4) void attn_fine_kernel(const AttnPr
         /* ---- the pieces land in the order they were requested: piece by piece, park it and work
          * on the key tiles it completes while the later pieces are still on their way ---- */
         const uint32_t fill_end = min(c0 + kc, key_end);
-        constexpr uint32_t RPP = FINE_THREADS / LPR4; /* rows per piece */
+        constexpr uint32_t RPP = Shape::RPP; /* rows per piece */
         auto park = [&](const uint32_t pc, const float4 k_piece, const float4 v_piece) __attribute__((always_inline)) {
             const uint32_t e = tid + FINE_THREADS * pc;
             const uint32_t r = e / LPR4, f = e % LPR4;
-            /* a fill holds 64 keys at least: no test (and nothing for the compiler to sink the
-             * piece's loads behind) on the pieces below that */
-            if (RPP * (pc + 1u) <= FINE_MIN_FILL || r < kc) {
+            /* no test (and nothing for the compiler to sink the piece's loads behind) on the pieces
+             * below what every fill holds */
+            if (RPP * (pc + 1u) <= Shape::MIN_FILL || r < kc) {
                 *reinterpret_cast<float4 *>(sm_k + r * ROW + 4u * f) = k_piece;
                 *reinterpret_cast<float4 *>(sm_v + r * ROW + 4u * f) = v_piece;
             }
@@ -299,41 +311,27 @@ __global__ __launch_bounds__(FINE_THREADS, 4) void attn_fine_kernel(const AttnPr
 #pragma unroll
                     for (int d = 0; d < DT; d++)
                         oacc[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[d][r], x[r], oacc[d], 0, 0, 0);
-                kt += 4u;
+                kt += WPH;
             }
             return c0 + RPP * pieces_done < fill_end; /* more keys to come: uniform over the workgroup */
         };
-        static_assert(Shape::PIECES == 4, "four pieces are spelled out");
-        if (FINE_PIECES_PER_STAGE == 1) {
-            park(0, kp[0], vp[0]);
-            if (stage(1)) {
-                park(1, kp[1], vp[1]);
-                if (stage(2)) {
-                    park(2, kp[2], vp[2]);
-                    if (stage(3)) {
-                        park(3, kp[3], vp[3]);
-                        stage(4);
-                    }
-                }
-            }
-        } else if (FINE_PIECES_PER_STAGE == 2) {
-            park(0, kp[0], vp[0]);
-            park(1, kp[1], vp[1]);
-            if (stage(2)) {
-                park(2, kp[2], vp[2]);
-                park(3, kp[3], vp[3]);
-                stage(4);
-            }
-        } else {
-            park(0, kp[0], vp[0]);
-            park(1, kp[1], vp[1]);
-            park(2, kp[2], vp[2]);
-            park(3, kp[3], vp[3]);
-            stage(4);
+        /* The next fill is requested as soon as this one has left the registers, before the last
+         * stage's units start (past the end of the keys the requests repeat the last row: no branch
+         * around them).  The two fills' requests never overlap in the registers. */
+        constexpr int PPS = Shape::PIECES / Shape::STAGES;
+#pragma unroll
+        for (int t = 0; t < PPS; t++) park(t, kp[t], vp[t]);
+        if (Shape::STAGES == 1) {
+            request(c0 + kc);
+            stage(Shape::PIECES);
+        } else if (stage(PPS)) {
+#pragma unroll
+            for (int t = PPS; t < Shape::PIECES; t++) park(t, kp[t], vp[t]);
+            request(c0 + kc);
+            stage(Shape::PIECES);
         }
         __syncthreads(); /* the fill is consumed: the next fill, or the merge, may overwrite it */
         c0 += kc;
-        if (c0 < key_end) request(c0);
     }
 
     /* the four lane groups of a column carry the same m, their sums add */
@@ -348,15 +346,16 @@ __global__ __launch_bounds__(FINE_THREADS, 4) void attn_fine_kernel(const AttnPr
     if (g == 0) *reinterpret_cast<float2 *>(mine + c * ROW + HD) = make_float2(m, l);
     __syncthreads();
 
-    /* 256 threads per row half: thread = (row, 16-byte piece of the row) */
-    const uint32_t mh = tid >> 8, idx = tid & 255u;
+    /* the threads of a row half: thread = (row, 16-byte piece of the row) */
+    constexpr uint32_t TPH = FINE_THREADS / HALVES;
+    const uint32_t mh = HALVES == 1 ? 0u : tid / TPH, idx = tid % TPH;
     const uint32_t mr = idx / LPR4, mf = idx % LPR4;
     if (mr < 16u) {
-        const float *part = sm + (4u * mh) * (16 * ROW) + mr * ROW;
-        float pm[4], pl[4];
+        const float *part = sm + (WPH * mh) * (16 * ROW) + mr * ROW;
+        float pm[WPH], pl[WPH];
         float M = neg_inf();
 #pragma unroll
-        for (int w = 0; w < 4; w++) {
+        for (int w = 0; w < (int)WPH; w++) {
             const float2 t = *reinterpret_cast<const float2 *>(part + w * (16 * ROW) + HD);
             pm[w] = t.x, pl[w] = t.y;
             M = fmaxf(M, pm[w]);
@@ -365,7 +364,7 @@ __global__ __launch_bounds__(FINE_THREADS, 4) void attn_fine_kernel(const AttnPr
         float L = 0.f;
         float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-        for (int w = 0; w < 4; w++) {
+        for (int w = 0; w < (int)WPH; w++) {
             const float f = fast_exp2(pm[w] - Ms);
             const float4 t = *reinterpret_cast<const float4 *>(part + w * (16 * ROW) + 4u * mf);
             L += pl[w] * f;
@@ -384,37 +383,43 @@ __global__ __launch_bounds__(FINE_THREADS, 4) void attn_fine_kernel(const AttnPr
     }
 }
 
-/* keys per fill for a launch whose longest tile needs `span` keys, and the LDS that takes */
-template <int HD>
+/* keys per fill for a launch whose longest tile needs `span` keys */
+template <typename Shape>
 uint32_t fine_fill_keys(uint32_t span) {
-    using Shape = FineShape<HD>;
     const uint32_t want = std::max<uint32_t>(16u, (span + 15u) / 16u * 16u + 16u); /* a span may straddle a tile */
-    static_assert(2 * FINE_MIN_FILL * Shape::ROW >= Shape::MERGE_FLOATS, "the merge overlays the fill");
-    return std::min<uint32_t>(Shape::KC_MAX, std::max<uint32_t>(FINE_MIN_FILL, want));
+    return std::min<uint32_t>(Shape::KC_MAX, std::max<uint32_t>(Shape::MIN_FILL, want));
 }
 
-template <int HD, int SRC>
+template <int HD, int SRC, int HALVES, int WAVES>
 void fine_launch_as(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t nblocks, const AttnAffine &aff,
                     uint32_t span, hipStream_t s) {
-    using Shape = FineShape<HD>;
-    const uint32_t kc = fine_fill_keys<HD>(span);
+    using Shape = FineShape<HD, HALVES, WAVES>;
+    const uint32_t kc = fine_fill_keys<Shape>(span);
     const size_t lds = (size_t)2 * kc * Shape::ROW * sizeof(float);
     static const bool raised = [] { /* more than the 64 KB a kernel may use without asking */
-        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_fine_kernel<HD, SRC>),
+        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_fine_kernel<HD, SRC, HALVES, WAVES>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      2 * Shape::KC_MAX * Shape::ROW * (int)sizeof(float)));
+                                      2 * (int)Shape::KC_MAX * Shape::ROW * (int)sizeof(float)));
         return true;
     }();
     (void)raised;
-    blt_launch("attn_fine", attn_fine_kernel<HD, SRC>, dim3(nblocks), dim3(FINE_THREADS), lds, s, dprobs, dtiles, aff,
-               kc);
+    blt_launch("attn_fine", attn_fine_kernel<HD, SRC, HALVES, WAVES>, dim3(nblocks), dim3(Shape::THREADS), lds, s,
+               dprobs, dtiles, aff, kc);
 }
 
+/* tall: workgroups of one 16-row tile and sixteen waves (strided batches and single problems) */
 template <int SRC>
 void fine_launch_hd(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t nblocks, const AttnAffine &aff,
-                    uint32_t hd, uint32_t span, hipStream_t s) {
-    if (hd == 32u) fine_launch_as<32, SRC>(dprobs, dtiles, nblocks, aff, span, s);
-    else fine_launch_as<64, SRC>(dprobs, dtiles, nblocks, aff, span, s);
+                    uint32_t hd, uint32_t span, bool tall, hipStream_t s) {
+    if constexpr (SRC != SRC_TILES) {
+        if (tall) {
+            if (hd == 32u) fine_launch_as<32, SRC, 1, 16>(dprobs, dtiles, nblocks, aff, span, s);
+            else fine_launch_as<64, SRC, 1, 16>(dprobs, dtiles, nblocks, aff, span, s);
+            return;
+        }
+    }
+    if (hd == 32u) fine_launch_as<32, SRC, 2, 8>(dprobs, dtiles, nblocks, aff, span, s);
+    else fine_launch_as<64, SRC, 2, 8>(dprobs, dtiles, nblocks, aff, span, s);
 }
 
 } // namespace
@@ -427,7 +432,7 @@ uint32_t attn_fine_span(const AttnProb &d) {
 }
 
 /* keys one LDS fill holds at head width hd */
-uint32_t attn_fine_fill_max(uint32_t hd) { return hd == 32u ? FineShape<32>::KC_MAX : FineShape<64>::KC_MAX; }
+uint32_t attn_fine_fill_max(uint32_t hd) { return hd == 32u ? FineShape<32, 2, 8>::KC_MAX : FineShape<64, 2, 8>::KC_MAX; }
 
 /* shapes the kernel is able to run */
 bool attn_fine_can(const AttnProb &d) {
@@ -445,20 +450,22 @@ void attn_fine_launch(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t n
     if (ntiles == 0) return;
     AttnAffine none;
     __builtin_memset(&none, 0, sizeof(none));
-    fine_launch_hd<SRC_TILES>(dprobs, dtiles, ntiles, none, hd, span, s);
+    fine_launch_hd<SRC_TILES>(dprobs, dtiles, ntiles, none, hd, span, false, s);
 }
 
-void attn_fine_launch_single(const AttnProb &single, hipStream_t s) {
-    const uint32_t ntiles = (single.nq + 31u) / 32u;
+void attn_fine_launch_single(const AttnProb &single, bool tall, hipStream_t s) {
+    const uint32_t rows = tall ? 16u : 32u;
+    const uint32_t ntiles = (single.nq + rows - 1u) / rows;
     if (ntiles == 0) return;
     AttnAffine a;
     __builtin_memset(&a, 0, sizeof(a));
     a.first = single;
-    fine_launch_hd<SRC_SINGLE>(nullptr, nullptr, ntiles, a, single.hd, attn_fine_span(single), s);
+    fine_launch_hd<SRC_SINGLE>(nullptr, nullptr, ntiles, a, single.hd, attn_fine_span(single), tall, s);
 }
 
-void attn_fine_launch_affine(const AttnAffine &aff, hipStream_t s) {
-    const uint32_t blocks = aff.count * aff.nqt;
+void attn_fine_launch_affine(const AttnAffine &aff, bool tall, hipStream_t s) {
+    const uint32_t rows = tall ? 16u : 32u;
+    const uint32_t blocks = aff.count * ((aff.first.nq + rows - 1u) / rows);
     if (blocks == 0) return;
-    fine_launch_hd<SRC_AFFINE>(nullptr, nullptr, blocks, aff, aff.first.hd, attn_fine_span(aff.first), s);
+    fine_launch_hd<SRC_AFFINE>(nullptr, nullptr, blocks, aff, aff.first.hd, attn_fine_span(aff.first), tall, s);
 }

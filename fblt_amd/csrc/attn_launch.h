@@ -61,7 +61,8 @@ uint32_t attn_fine_fill_max(uint32_t hd);
 void attn_fine_make_tiles(const AttnProb *host, uint32_t base, uint32_t count, std::vector<AttnTile> &tiles);
 void attn_fine_launch(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t ntiles, uint32_t hd, uint32_t span,
                       hipStream_t s);
-void attn_fine_launch_single(const AttnProb &single, hipStream_t s);
-void attn_fine_launch_affine(const AttnAffine &aff, hipStream_t s);
+/* tall: workgroups of one 16-row tile and sixteen waves instead of 32 rows and eight waves */
+void attn_fine_launch_single(const AttnProb &single, bool tall, hipStream_t s);
+void attn_fine_launch_affine(const AttnAffine &aff, bool tall, hipStream_t s);
 
 #endif
