@@ -872,8 +872,8 @@ def cpu_kv(kw, budget_s, max_steps):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--only", default="", help="comma list of c1,c2,c3,c4,c5 (c2 always runs)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU budget of the headline workload")
