@@ -696,6 +696,92 @@ def bench_decode_step(steps, warmup, batch=64, L=2, E=128, H=4, hidden=512, V=25
     return res
 
 
+def bench_encoder(steps, warmup, cpu_budget_s):
+    """The local encoder's forward (csrc/models/local_encoder.c:193-281) at C3's caller size -- 512
+    bytes in about 128 patches, E = 128, 4 heads, 2 layers with a cross block each, three hashed
+    n-gram tables: this library's blt_local_encoder_forward, and the restated forward on one host
+    core beside it."""
+    import ctypes as C
+    import numpy as np
+    import torch
+    from fblt_amd import abi, api, decoder, encoder
+    lib = api.load()
+    c = dict(T=512, E=128, H=4, XH=4, L=2, hidden=256, ngrams=(3, 4, 5), vocab=2048)
+    rs = np.random.RandomState(31)
+    lengths = []
+    while sum(lengths) < c["T"]:
+        lengths.append(int(min(c["T"] - sum(lengths), rs.poisson(3) + 1)))
+    P = len(lengths)
+    data = rs.randint(0, 256, size=c["T"]).astype(np.uint8)
+    weights = encoder.random_weights(c["E"], c["hidden"], c["L"], c["ngrams"], c["vocab"], 37)
+    hd = c["E"] // c["H"]
+    view = lambda t, dt=abi.BLT_DTYPE_FP32: abi.tensor_view(t.data_ptr(), tuple(t.shape), abi.BLT_BACKEND_HIP, dtype=dt)
+    cos, sin = torch.zeros((c["T"], hd // 2), device="cuda"), torch.zeros((c["T"], hd // 2), device="cuda")
+    vc, vs = view(cos), view(sin)
+    rcfg = abi.BltRopeConfig(500000.0, hd)
+    lib.blt_rope_precompute(c["T"], C.byref(rcfg), C.byref(vc), C.byref(vs))
+    tables = (cos.cpu().numpy(), sin.cpu().numpy())
+    args = (c["E"], c["H"], c["XH"], c["hidden"], c["T"], c["ngrams"], c["vocab"], 1000003)
+    dev = encoder.bind(weights, *tables, abi.BLT_BACKEND_HIP, decoder.device_place, *args)
+    patches = decoder.patch_table(lengths)
+    tbytes = torch.from_numpy(data).cuda()
+    p_out, h_out = torch.zeros((P, c["E"]), device="cuda"), torch.zeros((c["T"], c["E"]), device="cuda")
+    vb, vp, vh = view(tbytes, abi.BLT_DTYPE_UINT8), view(p_out), view(h_out)
+    arena = lib.blt_arena_create(256 << 20, abi.BLT_BACKEND_HIP)
+
+    def timed(entry):
+        def run(count):
+            for _ in range(count):
+                arena.contents.offset = 0
+                entry(dev.ptr, C.byref(vb), patches, P, None, 0, C.byref(vp), C.byref(vh), arena)
+        run(warmup)
+        lib.blt_backend_pass_sync_hip()
+        lib.blt_hip_profile_begin()
+        run(steps)
+        lib.blt_backend_pass_sync_hip()
+        prof = api.profile_end()
+        t0 = time.perf_counter()
+        run(steps)
+        lib.blt_backend_pass_sync_hip()
+        wall = (time.perf_counter() - t0) / steps
+        return {"launches_per_pass": sum(v[0] for v in prof.values()) / steps,
+                "kernel_us_per_pass": sum(v[1] for v in prof.values()) * 1e3 / steps, "wall_us_per_pass": wall * 1e6,
+                "per_kernel_us": {k: v[1] * 1e3 / steps for k, v in prof.items()}}
+
+    steps = max(10, steps // 5)
+    mine = timed(lib.blt_local_encoder_forward)
+    lib.blt_arena_destroy(arena)
+    avg_s = mine["kernel_us_per_pass"] * 1e-6
+    E, T, hidden, L = c["E"], c["T"], c["hidden"], c["L"]
+    per_layer_w = E * 3 * E + E * E + 3 * E * hidden + 4 * E * E
+    flops = L * (2.0 * T * (E * 3 * E + E * E + 3 * E * hidden) + 4.0 * hd * c["H"] * T * (T + 1) / 2 +
+                 2.0 * (P * 2 * E * E + T * 2 * E * E) + 4.0 * E * T)
+    nbytes = 4.0 * (L * (per_layer_w + 6 * T * E) + T * E * (1 + len(c["ngrams"])))
+    res = {"workload": "local encoder forward: %d bytes, %d patches, %d layers (cross block in each), E=%d, H=%d, "
+                       "hidden=%d, %d hashed n-gram tables" % (T, P, L, E, c["H"], hidden, len(c["ngrams"])),
+           "entry": "blt_local_encoder_forward", "kernel": "+".join(sorted(mine["per_kernel_us"])),
+           "launches_per_step": mine["launches_per_pass"], "tokens_per_step": T, "us_per_step": mine["wall_us_per_pass"],
+           "kernel_us_avg": mine["kernel_us_per_pass"], "kernel_us_min": min(mine["per_kernel_us"].values()),
+           "per_kernel_us": mine["per_kernel_us"], "tokens_per_s": T / (mine["wall_us_per_pass"] * 1e-6), "flops": flops,
+           "bytes": nbytes, "roofline_hbm": roofline("hbm", nbytes, avg_s), "roofline_mfma": roofline("mfma", flops, avg_s)}
+    res["roofline"] = res["roofline_mfma"]
+    if cpu_budget_s > 0:
+        from oracle import binding
+        orc = binding.load_oracle()
+        host = encoder.bind(weights, *tables, abi.BLT_BACKEND_CPU, decoder.host_place, *args)
+        po, ho = np.zeros((P, E), dtype=np.float32), np.zeros((T, E), dtype=np.float32)
+        t0, passes = time.perf_counter(), 0
+        while passes == 0 or time.perf_counter() - t0 < cpu_budget_s:
+            assert orc.orc_local_encoder_forward(host.ptr, data.ctypes.data_as(C.POINTER(C.c_uint8)), T, patches, P, None,
+                                                 0, binding.fptr(po.reshape(-1)), binding.fptr(ho.reshape(-1))) == 0
+            passes += 1
+        dt = (time.perf_counter() - t0) / passes
+        res["cpu_baseline"] = {"value": T / dt, "unit": "tokens/s", "cores": 1, "kind": "port",
+                               "sample": "%d passes of the restated forward, %.1f s" % (passes, dt * passes),
+                               "ms_per_pass": dt * 1e3}
+    return res
+
+
 def bench_draft_pass(steps, warmup, cpu_budget_s, N=400, B=8, L=2, E=128, H=4, hidden=512, V=256):
     """One denoising pass of the reference's draft loop (csrc/infer/block_generation.c:156-266: one
     sequence, N clean bytes, a block of B [MASK] rows on the last latent) three ways: the reference's
@@ -1034,6 +1120,8 @@ def main():
         # BLT-D drafting: one denoising pass over a 400-byte prefix, block of 8
         others["draft_pass"] = bench_draft_pass(K, W, 0.0 if args.no_cpu else 2.0 * cs)
         log("draft_pass", json.dumps(others["draft_pass"]))
+        others["encoder"] = bench_encoder(K, W, 0.0 if args.no_cpu else 2.0 * cs)
+        log("encoder", json.dumps(others["encoder"]))
 
     # the dense-mask builders the callers still use
     if want("masks"):
@@ -1109,7 +1197,7 @@ def compact_line(head, others, cpu_head, K, W, detail_path):
                         "c5_B16_b128_L2048") if k in others}
     # whole decoder step (all layers + LM head): [launches per step, device us, wall us]
     steps_ = {k: [others[k]["launches_per_step"], _sig(others[k]["kernel_us_avg"]), _sig(others[k]["us_per_step"])]
-              for k in ("decode_step", "decode_step_b1", "draft_pass") if k in others}
+              for k in ("decode_step", "decode_step_b1", "draft_pass", "encoder") if k in others}
     if "reference_call" in others.get("draft_pass", {}):   # the reference's call (prefix recomputed per pass) beside the cached block step
         c = others["draft_pass"]["reference_call"]
         steps_["draft_pass_reference_call"] = [c["launches_per_pass"], _sig(c["kernel_us_per_pass"]),

@@ -239,7 +239,65 @@ class BltBlockBatch(C.Structure):
     ]
 
 
+BLT_POOL_MEAN, BLT_POOL_MAX = range(2)
+BLT_IDX_SENTINEL = 0xFFFFFFFF
+BLT_MAX_NGRAM_SIZES = 6
+BLT_DTYPE_UINT8 = 3
+
+
+class BltHashNgramConfig(C.Structure):
+    """csrc/models/hash_ngram.h:13-22"""
+    _fields_ = [
+        ("ngram_sizes", C.c_size_t * BLT_MAX_NGRAM_SIZES),
+        ("num_ngram_sizes", C.c_size_t),
+        ("per_ngram_vocab", C.c_size_t),
+        ("hash_prime", C.c_uint64),
+        ("normalize", C.c_bool),
+        ("embed_dim", C.c_size_t),
+    ]
+
+
+class BltHashNgramWeights(C.Structure):
+    """csrc/models/hash_ngram.h:24-27"""
+    _fields_ = [("tables", BltTensor * BLT_MAX_NGRAM_SIZES), ("num_tables", C.c_size_t)]
+
+
+class BltLocalEncoderConfig(C.Structure):
+    """csrc/models/local_encoder.h:22-36"""
+    _fields_ = [
+        ("embed_dim", C.c_size_t),
+        ("num_layers", C.c_size_t),
+        ("patch_dim", C.c_size_t),
+        ("hidden_dim", C.c_size_t),
+        ("num_heads", C.c_size_t),
+        ("cross_attn_heads", C.c_size_t),
+        ("local_window", C.c_size_t),
+        ("cross_attn_all_layers", C.c_bool),
+        ("cross_attn_placement", C.c_int),
+        ("pool_type", C.c_int),
+        ("ngram_config", BltHashNgramConfig),
+        ("rope_theta", C.c_float),
+        ("max_seq_len", C.c_size_t),
+    ]
+
+
+class BltLocalEncoder(C.Structure):
+    """csrc/models/local_encoder.h:40-47"""
+    _fields_ = [
+        ("config", BltLocalEncoderConfig),
+        ("byte_embedding_weight", BltTensor),
+        ("ngram_weights", BltHashNgramWeights),
+        ("rope_cos_cache", BltTensor),
+        ("rope_sin_cache", BltTensor),
+        ("layers", C.POINTER(BltLocalLayerStorage)),
+    ]
+
+
 def check_layout():
+    assert C.sizeof(BltHashNgramConfig) == 88 and BltHashNgramConfig.hash_prime.offset == 64
+    assert C.sizeof(BltHashNgramWeights) == 632
+    assert C.sizeof(BltLocalEncoderConfig) == 176 and BltLocalEncoderConfig.ngram_config.offset == 72
+    assert C.sizeof(BltLocalEncoder) == 1128 and BltLocalEncoder.layers.offset == 1120
     assert C.sizeof(BltTransformerConfig) == 80
     assert C.sizeof(BltBlockBatch) == 112
     assert C.sizeof(BltTensor) == 104

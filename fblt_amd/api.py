@@ -133,6 +133,22 @@ SYMBOLS = {
     "blt_transformer_forward_hip": (None, [C.POINTER(abi.BltTensor), C.POINTER(abi.BltTransformerWeights),
                                            C.POINTER(abi.BltTensor), C.POINTER(abi.BltTransformerConfig),
                                            C.POINTER(abi.BltArena)]),
+    "blt_indexed_row_accumulate": (None, [C.POINTER(abi.BltTensor), C.POINTER(C.c_uint32), C.POINTER(abi.BltTensor)]),
+    "blt_indexed_row_accumulate_hip": (None, [C.POINTER(abi.BltTensor), C.POINTER(C.c_uint32),
+                                              C.POINTER(abi.BltTensor)]),
+    "blt_scale": (None, [C.POINTER(abi.BltTensor), C.c_float]),
+    "blt_scale_hip": (None, [C.POINTER(abi.BltTensor), C.c_float]),
+    "blt_patch_pool_forward": (None, [C.POINTER(abi.BltTensor), C.POINTER(abi.BltPatchInfo), C.c_size_t, C.c_int,
+                                      C.POINTER(abi.BltTensor)]),
+    "blt_patch_pool_forward_hip": (None, [C.POINTER(abi.BltTensor), C.POINTER(abi.BltPatchInfo), C.c_size_t, C.c_int,
+                                          C.POINTER(abi.BltTensor)]),
+    "blt_local_encoder_forward": (None, [C.POINTER(abi.BltLocalEncoder), C.POINTER(abi.BltTensor),
+                                         C.POINTER(abi.BltPatchInfo), C.c_size_t, abi.c_size_p, C.c_size_t,
+                                         C.POINTER(abi.BltTensor), C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)]),
+    "blt_local_encoder_forward_hip": (None, [C.POINTER(abi.BltLocalEncoder), C.POINTER(abi.BltTensor),
+                                             C.POINTER(abi.BltPatchInfo), C.c_size_t, abi.c_size_p, C.c_size_t,
+                                             C.POINTER(abi.BltTensor), C.POINTER(abi.BltTensor),
+                                             C.POINTER(abi.BltArena)]),
     "blt_embedding_lookup": (None, [C.POINTER(abi.BltTensor), C.POINTER(C.c_uint32), C.POINTER(abi.BltTensor)]),
     "blt_embedding_lookup_hip": (None, [C.POINTER(abi.BltTensor), C.POINTER(C.c_uint32), C.POINTER(abi.BltTensor)]),
     "blt_kv_block_step_hip": (None, [C.POINTER(abi.BltKvCache), C.c_size_t, C.POINTER(abi.BltBlockBatch), C.c_int,

@@ -358,6 +358,34 @@ void blt_transformer_forward(const blt_tensor *input, const blt_transformer_weig
     blt_transformer_forward_hip(input, weights, output, config, arena);
 }
 
+void blt_indexed_row_accumulate(const blt_tensor *table, const uint32_t *idx_host, blt_tensor *io) {
+    BLT_REQUIRE(table != NULL, "blt_indexed_row_accumulate: arguments cannot be NULL");
+    BLT_DEVICE_ONLY(table->backend, "blt_indexed_row_accumulate");
+    blt_indexed_row_accumulate_hip(table, idx_host, io);
+}
+
+void blt_scale(blt_tensor *t, float scalar) {
+    BLT_REQUIRE(t != NULL, "blt_scale: tensor must not be null");
+    BLT_DEVICE_ONLY(t->backend, "blt_scale");
+    blt_scale_hip(t, scalar);
+}
+
+void blt_patch_pool_forward(const blt_tensor *byte_hidden, const blt_patch_info *patches, size_t num_patches,
+                            blt_patch_pool_type pool_type, blt_tensor *out) {
+    BLT_REQUIRE(byte_hidden != NULL, "patch_pool: NULL tensor");
+    BLT_DEVICE_ONLY(byte_hidden->backend, "blt_patch_pool_forward");
+    blt_patch_pool_forward_hip(byte_hidden, patches, num_patches, pool_type, out);
+}
+
+void blt_local_encoder_forward(const blt_local_encoder *model, const blt_tensor *bytes_in, const blt_patch_info *patches,
+                               size_t num_patches, const size_t *doc_boundaries, size_t num_docs, blt_tensor *patch_out,
+                               blt_tensor *byte_hidden_out, blt_arena *arena) {
+    BLT_REQUIRE(patch_out != NULL, "blt_local_encoder_forward: patch_out and byte_hidden_out cannot be NULL");
+    BLT_DEVICE_ONLY(patch_out->backend, "blt_local_encoder_forward");
+    blt_local_encoder_forward_hip(model, bytes_in, patches, num_patches, doc_boundaries, num_docs, patch_out,
+                                  byte_hidden_out, arena);
+}
+
 void blt_add(const blt_tensor *a, const blt_tensor *b, blt_tensor *out) {
     BLT_REQUIRE(a != NULL, "blt_add: input tensors must be FP32 with matching element count");
     BLT_DEVICE_ONLY(a->backend, "blt_add");

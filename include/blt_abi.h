@@ -304,6 +304,55 @@ typedef struct {
     int trailing_closed;  /* the last clean byte closes its patch and reads the last latent */
 } blt_block_batch;
 
+/* csrc/ops/patch_pool.h:13-16 */
+typedef enum {
+    BLT_POOL_MEAN = 0, /* average of the patch's byte rows       */
+    BLT_POOL_MAX = 1   /* per-column maximum of the patch's rows */
+} blt_patch_pool_type;
+
+#define BLT_IDX_SENTINEL 0xFFFFFFFFu /* csrc/ops/gather_scatter.h:27: "no row" in an index list */
+
+/* csrc/models/hash_ngram.h:13-27 */
+#define BLT_MAX_NGRAM_SIZES 6
+typedef struct {
+    size_t ngram_sizes[BLT_MAX_NGRAM_SIZES];
+    size_t num_ngram_sizes;
+    size_t per_ngram_vocab; /* rows of every table = modulus of the rolling hash */
+    uint64_t hash_prime;
+    bool normalize;         /* divide the sum by num_ngram_sizes + 1 */
+    size_t embed_dim;
+} blt_hash_ngram_config;
+
+typedef struct {
+    blt_tensor tables[BLT_MAX_NGRAM_SIZES]; /* each [per_ngram_vocab, embed_dim] */
+    size_t num_tables;
+} blt_hash_ngram_weights;
+
+/* csrc/models/local_encoder.h:22-48 */
+typedef struct {
+    size_t embed_dim;
+    size_t num_layers;
+    size_t patch_dim; /* 0 = embed_dim */
+    size_t hidden_dim;
+    size_t num_heads;
+    size_t cross_attn_heads;
+    size_t local_window; /* 0 = full causal */
+    bool cross_attn_all_layers;
+    blt_xattn_placement cross_attn_placement;
+    blt_patch_pool_type pool_type;
+    blt_hash_ngram_config ngram_config;
+    float rope_theta;
+    size_t max_seq_len;
+} blt_local_encoder_config;
+
+typedef struct {
+    blt_local_encoder_config config;
+    blt_tensor byte_embedding_weight; /* [256, embed_dim] */
+    blt_hash_ngram_weights ngram_weights;
+    blt_tensor rope_cos_cache, rope_sin_cache; /* [max_seq_len, head_dim/2] */
+    blt_local_layer_storage *layers;           /* [num_layers] */
+} blt_local_encoder;
+
 #ifdef __cplusplus
 }
 #define BLT_ABI_ASSERT(c, m) static_assert(c, m)
@@ -349,6 +398,16 @@ BLT_ABI_ASSERT(sizeof(blt_kv_cache) == 112 && offsetof(blt_kv_cache, self_len) =
 BLT_ABI_ASSERT(sizeof(blt_transformer_config) == 80 && offsetof(blt_transformer_config, hidden_dim) == 56 &&
                    offsetof(blt_transformer_config, norm_type) == 68 && offsetof(blt_transformer_config, use_bf16) == 76,
                "blt_transformer_config layout");
+BLT_ABI_ASSERT(sizeof(blt_hash_ngram_config) == 88 && offsetof(blt_hash_ngram_config, hash_prime) == 64 &&
+                   sizeof(blt_hash_ngram_weights) == 632 && offsetof(blt_hash_ngram_weights, num_tables) == 624,
+               "blt_hash_ngram_config / _weights layout");
+BLT_ABI_ASSERT(sizeof(blt_local_encoder_config) == 176 && offsetof(blt_local_encoder_config, pool_type) == 64 &&
+                   offsetof(blt_local_encoder_config, ngram_config) == 72 &&
+                   offsetof(blt_local_encoder_config, rope_theta) == 160,
+               "blt_local_encoder_config layout");
+BLT_ABI_ASSERT(sizeof(blt_local_encoder) == 1128 && offsetof(blt_local_encoder, ngram_weights) == 280 &&
+                   offsetof(blt_local_encoder, rope_cos_cache) == 912 && offsetof(blt_local_encoder, layers) == 1120,
+               "blt_local_encoder layout");
 BLT_ABI_ASSERT(sizeof(blt_block_batch) == 112 && offsetof(blt_block_batch, tokens) == 40 &&
                    offsetof(blt_block_batch, groups) == 80 && offsetof(blt_block_batch, trailing_closed) == 104,
                "blt_block_batch layout");

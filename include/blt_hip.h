@@ -61,6 +61,20 @@ void blt_rows_gather_hip(const blt_tensor *src, const size_t *pos_host, blt_tens
 /* csrc/ops/gather_scatter.h:21 (gather_scatter_cpu.c:7-21): out[i, :] = table[ids_host[i], :]; the
  * diffusion forward's learned D_0 rows (csrc/models/block_diffusion.c:140-146) */
 void blt_embedding_lookup_hip(const blt_tensor *table, const uint32_t *ids_host, blt_tensor *out);
+/* Replaces blt_indexed_row_accumulate_cuda (csrc/core/backend.c:515-518; contract
+ * csrc/ops/gather_scatter.h:23-28, gather_scatter_cpu.c:41-61): io[i, :] += table[idx_host[i], :]
+ * for every i whose index is not BLT_IDX_SENTINEL; idx_host is a HOST array [io rows].  The
+ * hashed n-gram tables of the local encoder (csrc/models/hash_ngram.c:176-194).  Bit-identical. */
+void blt_indexed_row_accumulate_hip(const blt_tensor *table, const uint32_t *idx_host, blt_tensor *io);
+/* Replaces blt_scale_cuda (csrc/core/backend.c:262; csrc/ops/elementwise.h:10,
+ * elementwise_cpu.c:31-40): t *= scalar in place.  Bit-identical. */
+void blt_scale_hip(blt_tensor *t, float scalar);
+/* Replaces blt_patch_pool_forward_cuda (contract csrc/ops/patch_pool.h:18-21, patch_pool_cpu.c:3-48):
+ * out[j, :] = mean, or per-column maximum, of byte_hidden rows [start_j, start_j + len_j); patches
+ * is a HOST array; empty or out-of-range patches are fatal as in the reference.  The rows of a
+ * patch are added first to last and scaled by 1 / len: bit-identical. */
+void blt_patch_pool_forward_hip(const blt_tensor *byte_hidden, const blt_patch_info *patches, size_t num_patches,
+                                blt_patch_pool_type pool_type, blt_tensor *out);
 
 /* Replaces blt_softmax_masked_row_inplace_cuda (csrc/ops/vecmath.cu:71-114):
  * the row softmax of csrc/ops/vecmath.h:20-31 on one device row. */
@@ -143,6 +157,18 @@ void blt_multihead_attention_hip(const blt_tensor *input, const blt_tensor *weig
 void blt_transformer_forward_hip(const blt_tensor *input, const blt_transformer_weights *weights, blt_tensor *output,
                                  const blt_transformer_config *config, blt_arena *arena);
 
+/* csrc/models/local_encoder.h:71-73 (local_encoder.c:193-281): bytes -> byte embedding + hashed
+ * n-gram embeddings -> P_0 = pooled patches (repeated over the k sub-token column blocks) -> per
+ * layer the byte transformer block and, where it fires, P += cross_attention(RMSNorm(P), h).
+ * bytes_in [seq_len] UINT8 on either side (the ids are hashed on the host, as in the reference);
+ * weights, outputs and the arena are device memory; patches, doc_boundaries are HOST arrays.
+ * Unlike the reference's body on a device arena, sub-token splits (patch_dim = k * embed_dim,
+ * k > 1) work: the expanded group ids are host memory here. */
+void blt_local_encoder_forward_hip(const blt_local_encoder *model, const blt_tensor *bytes_in,
+                                   const blt_patch_info *patches, size_t num_patches, const size_t *doc_boundaries,
+                                   size_t num_docs, blt_tensor *patch_out, blt_tensor *byte_hidden_out,
+                                   blt_arena *arena);
+
 /* ===================================================================== */
 /* Part 2 -- device memory shim (csrc/core/cuda_shim.h:18-31,             */
 /*           csrc/ops/memory.cu:19-77)                                    */
@@ -187,6 +213,11 @@ float blt_vec_dot(blt_backend backend, const float *a, const float *b, size_t n)
 /* csrc/core/backend.c:532-534: the backend comes from src. */
 void blt_rows_gather(const blt_tensor *src, const size_t *pos_host, blt_tensor *dst);
 void blt_embedding_lookup(const blt_tensor *table, const uint32_t *ids_host, blt_tensor *out);
+/* csrc/core/backend.c:515-518, 262; csrc/ops/patch_pool.h:20: the backend comes from the first tensor. */
+void blt_indexed_row_accumulate(const blt_tensor *table, const uint32_t *idx_host, blt_tensor *io);
+void blt_scale(blt_tensor *t, float scalar);
+void blt_patch_pool_forward(const blt_tensor *byte_hidden, const blt_patch_info *patches, size_t num_patches,
+                            blt_patch_pool_type pool_type, blt_tensor *out);
 /* csrc/infer/rope_gather.h / rope_gather.c:5-35: rows positions[0..n) of the two rotary
  * tables into new [n, half] tensors of the arena. */
 void blt_rope_position_gather(const blt_tensor *cos_cache, const blt_tensor *sin_cache, const size_t *positions,
@@ -212,6 +243,10 @@ void blt_cross_attention_forward(const blt_tensor *query_in, const blt_tensor *k
 /* csrc/core/backend.c:254-256, 276-278, 380-382 */
 void blt_transformer_forward(const blt_tensor *input, const blt_transformer_weights *weights, blt_tensor *output,
                              const blt_transformer_config *config, blt_arena *arena);
+/* csrc/models/local_encoder.h:71-73 */
+void blt_local_encoder_forward(const blt_local_encoder *model, const blt_tensor *bytes_in, const blt_patch_info *patches,
+                               size_t num_patches, const size_t *doc_boundaries, size_t num_docs, blt_tensor *patch_out,
+                               blt_tensor *byte_hidden_out, blt_arena *arena);
 void blt_add(const blt_tensor *a, const blt_tensor *b, blt_tensor *out);
 void blt_swiglu_forward(const blt_tensor *gate, const blt_tensor *up, blt_tensor *out);
 void blt_rmsnorm_forward(const blt_tensor *x, const blt_tensor *weight, blt_tensor *out);

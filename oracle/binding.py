@@ -83,6 +83,23 @@ def load_oracle():
     lib.orc_multihead_attention.restype = C.c_int
     lib.orc_multihead_attention.argtypes = [_fp, _fp, _fp, _fp, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int, C.c_int,
                                             C.c_float, _fp, _fp, C.POINTER(abi.BltMaskConfig)]
+    _u8 = C.POINTER(C.c_uint8)
+    _u32 = C.POINTER(C.c_uint32)
+    lib.orc_indexed_row_accumulate.restype = C.c_int
+    lib.orc_indexed_row_accumulate.argtypes = [_fp, C.c_size_t, _u32, _fp, C.c_size_t, C.c_size_t]
+    lib.orc_scale.restype = None
+    lib.orc_scale.argtypes = [_fp, C.c_size_t, C.c_float]
+    lib.orc_patch_pool_forward.restype = C.c_int
+    lib.orc_patch_pool_forward.argtypes = [_fp, C.c_size_t, C.c_size_t, C.POINTER(abi.BltPatchInfo), C.c_size_t, C.c_int,
+                                           _fp]
+    lib.orc_ngram_indices.restype = C.c_int
+    lib.orc_ngram_indices.argtypes = [_u8, C.c_size_t, C.c_size_t, C.c_uint64, C.c_uint64, _u32]
+    lib.orc_embed_bytes.restype = C.c_int
+    lib.orc_embed_bytes.argtypes = [_fp, C.POINTER(abi.BltHashNgramConfig), C.POINTER(abi.BltHashNgramWeights), _u8,
+                                    C.c_size_t, _fp]
+    lib.orc_local_encoder_forward.restype = C.c_int
+    lib.orc_local_encoder_forward.argtypes = [C.POINTER(abi.BltLocalEncoder), _u8, C.c_size_t,
+                                              C.POINTER(abi.BltPatchInfo), C.c_size_t, abi.c_size_p, C.c_size_t, _fp, _fp]
     lib.orc_transformer_forward.restype = C.c_int
     lib.orc_transformer_forward.argtypes = [_fp] * 9 + [C.c_size_t] * 4 + [C.c_int, C.c_int, C.c_float, _fp, _fp,
                                                                          C.POINTER(abi.BltMaskConfig)]
@@ -214,6 +231,14 @@ def load_ref():
                                                                   C.POINTER(abi.BltPatchInfo), C.c_size_t,
                                                                   C.POINTER(abi.BltBlockBatch), C.c_int, T,
                                                                   C.POINTER(abi.BltArena)]
+    if hasattr(lib, "blt_local_encoder_forward"):   # csrc/models/local_encoder.h:71-73
+        _encoder_entry(lib)
+        lib.blt_indexed_row_accumulate.restype = None
+        lib.blt_indexed_row_accumulate.argtypes = [T, C.POINTER(C.c_uint32), T]
+        lib.blt_scale.restype = None
+        lib.blt_scale.argtypes = [T, C.c_float]
+        lib.blt_patch_pool_forward.restype = None
+        lib.blt_patch_pool_forward.argtypes = [T, C.POINTER(abi.BltPatchInfo), C.c_size_t, C.c_int, T]
     lib.blt_build_block_diffusion_mask.restype = None
     lib.blt_build_block_diffusion_mask.argtypes = [C.POINTER(abi.BltBlockDiffusionConfig),
                                                    C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)]
@@ -224,6 +249,13 @@ def load_ref():
     lib.blt_patch_expand_group_ids.restype = None
     lib.blt_patch_expand_group_ids.argtypes = [_sp, C.c_size_t, C.c_size_t, _sp]
     return lib
+
+
+def _encoder_entry(lib):
+    T = C.POINTER(abi.BltTensor)
+    lib.blt_local_encoder_forward.restype = None
+    lib.blt_local_encoder_forward.argtypes = [C.POINTER(abi.BltLocalEncoder), T, C.POINTER(abi.BltPatchInfo), C.c_size_t,
+                                              abi.c_size_p, C.c_size_t, T, T, C.POINTER(abi.BltArena)]
 
 
 CALLERS_SO = os.path.join(HERE, "_ref", "libblt_ref_callers.so")
@@ -268,6 +300,8 @@ def load_ref_stack_callers():
     lib.blt_global_transformer_create.argtypes = [A, C.POINTER(BltGlobalTransformerConfig)]
     lib.blt_global_transformer_forward.restype = None
     lib.blt_global_transformer_forward.argtypes = [C.POINTER(BltGlobalTransformer), T, abi.c_size_p, C.c_size_t, T, A]
+    if hasattr(lib, "blt_local_encoder_forward"):
+        _encoder_entry(lib)
     return lib
 
 

@@ -966,3 +966,183 @@ int orc_transformer_forward(const float *input, const float *norm1_w, const floa
     free(normed), free(attn), free(resid), free(up), free(gate), free(act);
     return rc;
 }
+
+/* ------------------------------------------------------------------------- */
+/* local encoder: embedding + hashed n-grams, patch pooling, layer loop        */
+/* ------------------------------------------------------------------------- */
+
+/* ops/gather_scatter_cpu.c:41-61 */
+int orc_indexed_row_accumulate(const float *table, size_t vocab, const uint32_t *idx, float *io, size_t rows,
+                               size_t embed_dim) {
+    for (size_t i = 0; i < rows; i++) {
+        if (idx[i] == BLT_IDX_SENTINEL) continue;
+        if (idx[i] >= vocab) return ORC_ERR_ARG;
+        const float *row = table + (size_t)idx[i] * embed_dim;
+        float *dst = io + i * embed_dim;
+        for (size_t d = 0; d < embed_dim; d++) dst[d] += row[d];
+    }
+    return ORC_OK;
+}
+
+/* ops/elementwise_cpu.c:31-40 */
+void orc_scale(float *x, size_t n, float scalar) {
+    for (size_t i = 0; i < n; i++) x[i] *= scalar;
+}
+
+/* ops/patch_pool_cpu.c:3-48 */
+int orc_patch_pool_forward(const float *byte_hidden, size_t seq_len, size_t embed_dim, const blt_patch_info *patches,
+                           size_t num_patches, int pool_type, float *out) {
+    if (pool_type != BLT_POOL_MEAN && pool_type != BLT_POOL_MAX) return ORC_ERR_ARG;
+    for (size_t j = 0; j < num_patches; j++) {
+        const size_t start = patches[j].start_idx, len = patches[j].length;
+        if (len < 1 || start + len > seq_len) return ORC_ERR_ARG;
+        float *dst = out + j * embed_dim;
+        const float *src0 = byte_hidden + start * embed_dim;
+        if (pool_type == BLT_POOL_MEAN) {
+            for (size_t d = 0; d < embed_dim; d++) dst[d] = 0.0f;
+            for (size_t i = 0; i < len; i++)
+                for (size_t d = 0; d < embed_dim; d++) dst[d] += src0[i * embed_dim + d];
+            const float inv_len = 1.0f / (float)len;
+            for (size_t d = 0; d < embed_dim; d++) dst[d] *= inv_len;
+        } else {
+            memcpy(dst, src0, embed_dim * sizeof(float));
+            for (size_t i = 1; i < len; i++)
+                for (size_t d = 0; d < embed_dim; d++)
+                    if (src0[i * embed_dim + d] > dst[d]) dst[d] = src0[i * embed_dim + d];
+        }
+    }
+    return ORC_OK;
+}
+
+/* models/hash_ngram.c:16-79 (state, first window, rolling update), 183-191 (the index list) */
+int orc_ngram_indices(const uint8_t *bytes, size_t seq_len, size_t n, uint64_t prime, uint64_t modulus,
+                      uint32_t *idx) {
+    if (n == 0 || n > 8 || modulus <= 1 || prime == 0 || prime > (UINT64_MAX - 255) / modulus) return ORC_ERR_ARG;
+    uint64_t pow_n = 1ULL % modulus;
+    for (size_t i = 0; i < n; i++) pow_n = (pow_n * prime) % modulus;
+    uint8_t window[8] = {0};
+    size_t window_start = 0, seen = 0;
+    uint64_t current = 0;
+    for (size_t i = 0; i < seq_len; i++) {
+        const uint8_t outgoing = window[window_start];
+        window[window_start] = bytes[i];
+        window_start = (window_start + 1) % n;
+        seen++;
+        if (seen < n) {
+            idx[i] = BLT_IDX_SENTINEL;
+            continue;
+        }
+        if (seen == n) {
+            uint64_t hash = 0;
+            size_t at = window_start;
+            for (size_t t = 0; t < n; t++) {
+                hash = (hash * prime + window[at]) % modulus;
+                at = (at + 1) % n;
+            }
+            current = hash;
+        } else {
+            uint64_t updated = (current * prime + bytes[i]) % modulus;
+            const uint64_t gone = ((uint64_t)outgoing * pow_n) % modulus;
+            current = (updated + modulus - gone) % modulus;
+        }
+        idx[i] = (uint32_t)current;
+    }
+    return ORC_OK;
+}
+
+/* models/byte_embedding.c:16-53 then models/hash_ngram.c:142-207 */
+int orc_embed_bytes(const float *byte_table, const blt_hash_ngram_config *config,
+                    const blt_hash_ngram_weights *weights, const uint8_t *bytes, size_t seq_len, float *out) {
+    const size_t E = config->embed_dim;
+    if (config->num_ngram_sizes > BLT_MAX_NGRAM_SIZES) return ORC_ERR_ARG;
+    for (size_t i = 0; i < seq_len; i++) memcpy(out + i * E, byte_table + (size_t)bytes[i] * E, E * sizeof(float));
+    uint32_t *idx = (uint32_t *)malloc((seq_len ? seq_len : 1) * sizeof(uint32_t));
+    int rc = ORC_OK;
+    for (size_t t = 0; t < config->num_ngram_sizes && rc == ORC_OK; t++) {
+        const size_t n = config->ngram_sizes[t];
+        if (n == 0 || n > seq_len) continue;
+        rc = orc_ngram_indices(bytes, seq_len, n, config->hash_prime, config->per_ngram_vocab, idx);
+        if (rc == ORC_OK)
+            rc = orc_indexed_row_accumulate((const float *)weights->tables[t].data, config->per_ngram_vocab, idx, out,
+                                            seq_len, E);
+    }
+    free(idx);
+    if (rc == ORC_OK && config->normalize) orc_scale(out, seq_len * E, 1.0f / (float)(config->num_ngram_sizes + 1));
+    return rc;
+}
+
+/* models/local_encoder.c:193-281; masks and views as make_context / make_cross_attn_config /
+ * setup_query_split_mask build them (52-113), layer configuration as local_common.c:99-115 */
+int orc_local_encoder_forward(const blt_local_encoder *enc, const uint8_t *bytes, size_t seq_len,
+                              const blt_patch_info *patches, size_t num_patches, const size_t *doc_boundaries,
+                              size_t num_docs, float *patch_out, float *byte_hidden_out) {
+    const blt_local_encoder_config *cfg = &enc->config;
+    const size_t E = cfg->embed_dim, T = seq_len, P = num_patches;
+    const size_t patch_dim = cfg->patch_dim == 0 ? E : cfg->patch_dim;
+    if (E == 0 || patch_dim % E != 0 || P < 1 || T < 1 || T > cfg->max_seq_len) return ORC_ERR_ARG;
+    const size_t k = patch_dim / E;
+
+    size_t *q_groups = (size_t *)malloc(P * sizeof(size_t));
+    size_t *kv_groups = (size_t *)malloc(T * sizeof(size_t));
+    size_t *q_split = (size_t *)malloc(P * k * sizeof(size_t));
+    float *h = (float *)malloc(T * E * sizeof(float));
+    float *h_next = (float *)malloc(T * E * sizeof(float));
+    float *pooled = (float *)malloc(P * E * sizeof(float));
+    float *p = (float *)malloc(P * patch_dim * sizeof(float));
+    float *query = (float *)malloc(P * patch_dim * sizeof(float));
+    float *cross = (float *)malloc(P * patch_dim * sizeof(float));
+    int rc = orc_patch_build_group_ids(patches, P, T, q_groups, kv_groups);
+
+    blt_mask_config local_mask, cross_mask;
+    memset(&local_mask, 0, sizeof(local_mask));
+    memset(&cross_mask, 0, sizeof(cross_mask));
+    local_mask.seq_len_q = local_mask.seq_len_kv = T;
+    local_mask.sliding_window = cfg->local_window;
+    local_mask.doc_boundaries = doc_boundaries;
+    local_mask.num_docs = num_docs;
+    local_mask.is_causal = true;
+    cross_mask.seq_len_q = P * k;
+    cross_mask.seq_len_kv = T;
+    cross_mask.query_group_ids = q_groups;
+    cross_mask.kv_group_ids = kv_groups;
+    cross_mask.bidirectional_within_group = true;
+    if (k > 1) {
+        orc_patch_expand_group_ids(q_groups, P, k, q_split);
+        cross_mask.query_group_ids = q_split;
+    }
+
+    if (rc == ORC_OK)
+        rc = orc_embed_bytes((const float *)enc->byte_embedding_weight.data, &cfg->ngram_config, &enc->ngram_weights,
+                             bytes, T, h);
+    if (rc == ORC_OK) rc = orc_patch_pool_forward(h, T, E, patches, P, (int)cfg->pool_type, pooled);
+    if (rc == ORC_OK)
+        for (size_t sj = 0; sj < k; sj++) orc_strided_copy(p + sj * E, patch_dim, pooled, E, P, E);
+
+    for (size_t l = 0; l < cfg->num_layers && rc == ORC_OK; l++) {
+        const blt_local_layer_storage *s = &enc->layers[l];
+        rc = orc_transformer_forward(h, (const float *)s->norm1_weight.data, (const float *)s->attn_qkv_w.data,
+                                     (const float *)s->attn_proj_w.data, (const float *)s->norm2_weight.data,
+                                     (const float *)s->ffn_up_w.data, (const float *)s->ffn_gate_w.data,
+                                     (const float *)s->ffn_down_w.data, h_next, T, E, cfg->hidden_dim, cfg->num_heads, 1,
+                                     1, cfg->rope_theta, (const float *)enc->rope_cos_cache.data,
+                                     (const float *)enc->rope_sin_cache.data, &local_mask);
+        if (rc != ORC_OK) break;
+        float *swap = h;
+        h = h_next, h_next = swap;
+        if (!orc_local_cross_attn_fires((int)cfg->cross_attn_placement, cfg->cross_attn_all_layers, cfg->num_layers, l))
+            continue;
+        orc_rmsnorm_forward(p, (const float *)s->cross_norm_weight.data, query, P * k, E);
+        rc = orc_cross_attention_forward(query, h, (const float *)s->cross_weight_q.data,
+                                         (const float *)s->cross_weight_k.data, (const float *)s->cross_weight_v.data,
+                                         (const float *)s->cross_weight_proj.data, cross, P * k, T, E,
+                                         cfg->cross_attn_heads, &cross_mask);
+        if (rc == ORC_OK) orc_add(p, cross, p, P * patch_dim);
+    }
+    if (rc == ORC_OK) {
+        memcpy(patch_out, p, P * patch_dim * sizeof(float));
+        memcpy(byte_hidden_out, h, T * E * sizeof(float));
+    }
+    free(q_groups), free(kv_groups), free(q_split), free(h), free(h_next), free(pooled), free(p), free(query), free(cross);
+    return rc;
+}
+

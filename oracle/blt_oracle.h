@@ -277,6 +277,28 @@ int orc_transformer_forward(const float *input, const float *norm1_w, const floa
                             int is_causal, int use_rope, float rope_theta, const float *rope_cos_cache,
                             const float *rope_sin_cache, const blt_mask_config *mask_config);
 
+/* ops/gather_scatter_cpu.c:41-61: io[i, :] += table[idx[i], :], BLT_IDX_SENTINEL entries skipped. */
+int orc_indexed_row_accumulate(const float *table, size_t vocab, const uint32_t *idx, float *io, size_t rows,
+                               size_t embed_dim);
+/* ops/elementwise_cpu.c:31-40 */
+void orc_scale(float *x, size_t n, float scalar);
+/* ops/patch_pool_cpu.c:3-48: pool_type 0 = mean, 1 = per-column maximum. */
+int orc_patch_pool_forward(const float *byte_hidden, size_t seq_len, size_t embed_dim, const blt_patch_info *patches,
+                           size_t num_patches, int pool_type, float *out);
+/* models/hash_ngram.c:16-79, 176-191: the bucket index of every position for n-gram size n (rolling
+ * polynomial hash with the circular window); BLT_IDX_SENTINEL before the first full window. */
+int orc_ngram_indices(const uint8_t *bytes, size_t seq_len, size_t n, uint64_t prime, uint64_t modulus,
+                      uint32_t *idx);
+/* models/hash_ngram.c:142-207 on top of models/byte_embedding.c:16-53: out = byte_table[bytes] +
+ * sum of the hashed tables (in order), scaled by 1 / (num_ngram_sizes + 1) when normalize is set. */
+int orc_embed_bytes(const float *byte_table, const blt_hash_ngram_config *config,
+                    const blt_hash_ngram_weights *weights, const uint8_t *bytes, size_t seq_len, float *out);
+/* models/local_encoder.c:193-281 with host tensors in `enc` (context 52-113): patch_out
+ * [num_patches, patch_dim], byte_hidden_out [seq_len, embed_dim]. */
+int orc_local_encoder_forward(const blt_local_encoder *enc, const uint8_t *bytes, size_t seq_len,
+                              const blt_patch_info *patches, size_t num_patches, const size_t *doc_boundaries,
+                              size_t num_docs, float *patch_out, float *byte_hidden_out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -42,6 +42,16 @@ TRANSFORMER_CASES = {
     "block_T128_E512_H8_docs": (128, 512, 8, 1024, "docs"),           # a layer of the patch transformer at C2 size
     "block_T96_E64_H2_docs_window": (96, 64, 2, 160, "docs_window"),  # a byte layer of the local encoder
 }
+# the local encoder (csrc/models/local_encoder.c:193-281): bytes, patch lengths, sizes, options
+ENCODER_CASES = {
+    # C3's caller at its size: 512 bytes in 128 patches, 4 x 32 heads, cross block in every layer
+    "enc_T512_L2": dict(T=512, E=128, H=4, XH=4, L=2, hidden=256, ngrams=(3, 4, 5), vocab=2048, k=1, window=0,
+                             placement=0, all_layers=True, pool="mean", docs=None, normalize=True, mean_patch=4),
+    # sub-token split, window, documents, max pooling, cross block after the last layer only
+    "enc_T150_k2_window_docs_max": dict(T=150, E=64, H=2, XH=4, L=3, hidden=96, ngrams=(2, 3, 8), vocab=257, k=2,
+                                        window=40, placement=0, all_layers=False, pool="max", docs=[60, 111],
+                                        normalize=False, mean_patch=6),
+}
 THETA = 500000.0
 
 
@@ -135,6 +145,24 @@ def transformer_case(rs, T, E, H, hidden, mask):
         keep = abi.size_array(cuts)
         cfg.doc_boundaries, cfg.num_docs = keep, len(cuts) + 1
     return x, w, cfg, keep
+
+
+def encoder_case(rs, c):
+    """Bytes, patch lengths and weights of one encoder configuration."""
+    from fblt_amd import encoder
+    T = c["T"]
+    lengths = []
+    while sum(lengths) < T:
+        lengths.append(int(min(T - sum(lengths), max(1, rs.poisson(c["mean_patch"] - 1) + 1))))
+    data = rs.randint(0, 256, size=T).astype(np.uint8)
+    data[rs.randint(0, T, size=T // 4)] = 32   # repeated bytes: hash buckets get hit more than once
+    weights = encoder.random_weights(c["E"], c["hidden"], c["L"], c["ngrams"], c["vocab"], int(rs.randint(1 << 30)))
+    return data, lengths, weights
+
+
+def encoder_inputs(name):
+    c = ENCODER_CASES[name]
+    return (c,) + encoder_case(np.random.RandomState(seed_of(name)), c)
 
 
 def transformer_inputs(name):

@@ -154,6 +154,13 @@ def run_transformer(ref, arena, name):
     return out
 
 
+def run_encoder(ref, name):
+    """blt_local_encoder_forward of the reference build on host tensors."""
+    from tests import encoder_runs
+    c, data, lengths, weights = bc.encoder_inputs(name)
+    return encoder_runs.run_reference(ref, binding.load_oracle(), c, data, lengths, weights)
+
+
 def main():
     ref = binding.load_ref()
     if ref is None:
@@ -174,6 +181,10 @@ def main():
         pack(store, name + "/out", run_transformer(ref, arena, name), rs)
     for name in bc.DIFFUSION_CASES:
         pack(store, name + "/logits", run_diffusion(ref, arena, name), rs)
+    for name in bc.ENCODER_CASES:
+        patch_out, byte_hidden = run_encoder(ref, name)
+        pack(store, name + "/patch_out", patch_out, rs)
+        pack(store, name + "/byte_hidden_out", byte_hidden, rs)
     ref.blt_arena_destroy(arena)
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "blocks_golden.npz")
     np.savez_compressed(path, **store)

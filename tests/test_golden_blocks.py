@@ -110,6 +110,15 @@ def test_oracle_reproduces_reference_transformer_block(name, oracle):
     check(out, name + "/out", exact=True)
 
 
+@pytest.mark.parametrize("name", list(bc.ENCODER_CASES))
+def test_oracle_reproduces_reference_local_encoder(name, oracle):
+    from tests import encoder_runs
+    c, data, lengths, weights = bc.encoder_inputs(name)
+    patch_out, byte_hidden = encoder_runs.run_oracle(oracle, c, data, lengths, weights)
+    check(patch_out, name + "/patch_out", exact=True)
+    check(byte_hidden, name + "/byte_hidden_out", exact=True)
+
+
 def _diffusion_decoder(oracle, c, weights, backend, place):
     cos, sin = host_tables(oracle, c["max_len"], c["E"] // c["H"])
     return decoder.bind(weights, cos, sin, backend, place, c["E"], c["H"], c["XH"], c["hidden"], c["V"], c["max_len"],
@@ -273,3 +282,17 @@ def test_hip_matches_reference_transformer_block(name):
     out = to.cpu().numpy()
     lib.blt_arena_destroy(arena)
     check(out, name + "/out", exact=False)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", list(bc.ENCODER_CASES))
+def test_hip_matches_reference_local_encoder(name, oracle):
+    from fblt_amd import api
+    from tests import encoder_runs
+    lib = api.load()
+    c, data, lengths, weights = bc.encoder_inputs(name)
+    patch_out, byte_hidden = encoder_runs.run_device(lib.blt_local_encoder_forward, lib, oracle, c, data, lengths,
+                                                     weights)
+    check(patch_out, name + "/patch_out", exact=False)
+    check(byte_hidden, name + "/byte_hidden_out", exact=False)
+

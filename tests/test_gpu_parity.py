@@ -1606,3 +1606,91 @@ def test_decoder_step_with_exact_projections():
                         "or kv_decode_step_batched", "-p", "no:cacheprovider"],
                        capture_output=True, text=True, timeout=900, env=env, cwd=os.path.dirname(here))
     assert p.returncode == 0, p.stdout[-3000:] + p.stderr[-2000:]
+
+
+def test_encoder_ops(oracle, dev):
+    """blt_indexed_row_accumulate / blt_scale / blt_patch_pool_forward on device tensors against the
+    restated ops: bit for bit (the kernels keep the reference's order of additions).  Index lists
+    longer than one launch carries, sentinel entries, both pools, patches of 1 ... 300 rows."""
+    import torch
+    from fblt_amd import decoder
+    lib = api.load()
+    rs = np.random.RandomState(5)
+    T, E, V = 1300, 48, 97
+    table = rs.randn(V, E).astype(np.float32)
+    idx = rs.randint(0, V, size=T).astype(np.uint32)
+    idx[rs.randint(0, T, size=150)] = abi.BLT_IDX_SENTINEL
+    io = rs.randn(T, E).astype(np.float32)
+    want = io.copy()
+    u32 = C.POINTER(C.c_uint32)
+    assert oracle.orc_indexed_row_accumulate(binding.fptr(table.reshape(-1)), V, idx.ctypes.data_as(u32),
+                                             binding.fptr(want.reshape(-1)), T, E) == 0
+    oracle.orc_scale(binding.fptr(want.reshape(-1)), want.size, 0.25)
+    tt, ti = torch.from_numpy(table).cuda(), torch.from_numpy(io).cuda()
+    vt, vi = _dev_tensor(tt), _dev_tensor(ti)
+    lib.blt_indexed_row_accumulate(C.byref(vt), idx.ctypes.data_as(u32), C.byref(vi))
+    lib.blt_scale(C.byref(vi), 0.25)
+    lib.blt_backend_pass_sync_hip()
+    assert ti.cpu().numpy().tobytes() == want.tobytes()
+
+    lengths = [1, 300, 2, 7, 1, 13] + [3] * 290   # more patches than one launch carries
+    patches = decoder.patch_table(lengths)
+    h = rs.randn(sum(lengths), E).astype(np.float32)
+    th = torch.from_numpy(h).cuda()
+    vh = _dev_tensor(th)
+    for pool in (abi.BLT_POOL_MEAN, abi.BLT_POOL_MAX):
+        want = np.zeros((len(lengths), E), dtype=np.float32)
+        assert oracle.orc_patch_pool_forward(binding.fptr(h.reshape(-1)), h.shape[0], E, patches, len(lengths), pool,
+                                             binding.fptr(want.reshape(-1))) == 0
+        to = torch.full((len(lengths), E), 9.0, dtype=torch.float32, device="cuda")
+        vo = _dev_tensor(to)
+        lib.blt_patch_pool_forward(C.byref(vh), patches, len(lengths), pool, C.byref(vo))
+        lib.blt_backend_pass_sync_hip()
+        assert to.cpu().numpy().tobytes() == want.tobytes(), pool
+
+
+ENCODER_GPU_SHAPES = {
+    "small_k1": dict(T=37, E=32, H=2, XH=2, L=1, hidden=48, ngrams=(3,), vocab=101, k=1, window=0, placement=0,
+                     all_layers=True, pool="mean", docs=None, normalize=True, mean_patch=3),
+    "k3_docs_first": dict(T=90, E=64, H=2, XH=1, L=3, hidden=96, ngrams=(0, 4, 200), vocab=64, k=3, window=0,
+                          placement=4, all_layers=False, pool="mean", docs=[25], normalize=True, mean_patch=2),
+    "no_cross_window": dict(T=130, E=32, H=1, XH=2, L=2, hidden=32, ngrams=(), vocab=8, k=1, window=17, placement=1,
+                            all_layers=True, pool="max", docs=None, normalize=True, mean_patch=7),
+    "six_tables_all": dict(T=300, E=128, H=4, XH=4, L=2, hidden=256, ngrams=(3, 4, 5, 6, 7, 8), vocab=509, k=1, window=0,
+                           placement=3, all_layers=False, pool="max", docs=[100, 101], normalize=True, mean_patch=4),
+}
+
+
+@pytest.mark.parametrize("impl", ["library", "reference_callers"])
+@pytest.mark.parametrize("name", list(ENCODER_GPU_SHAPES) + ["enc_T512_L2", "enc_T150_k2_window_docs_max"])
+def test_local_encoder_forward(name, impl, oracle, dev):
+    """blt_local_encoder_forward on device tensors against the restated forward: patch_out and
+    byte_hidden_out within the fp32 tolerance.  `library` = this library's entry point (bytes given
+    on the device and, for one case, on the host); `reference_callers` = the reference's own
+    local_encoder.c / hash_ngram.c / byte_embedding.c, compiled unmodified, with this library's
+    ops and fused blocks under them -- for configurations without a sub-token split only: with
+    k > 1 the reference writes its expanded group ids through a host pointer into arena memory
+    (csrc/models/local_encoder.c:100-103), which a device arena does not allow."""
+    from tests import encoder_runs
+    from tests.golden import block_cases
+    lib = api.load()
+    if name in ENCODER_GPU_SHAPES:
+        c = ENCODER_GPU_SHAPES[name]
+        data, lengths, weights = block_cases.encoder_case(np.random.RandomState(len(name) * 31 + c["T"]), c)
+    else:
+        c, data, lengths, weights = block_cases.encoder_inputs(name)
+    if impl == "library":
+        entry = lib.blt_local_encoder_forward
+    else:
+        if c["k"] > 1:
+            pytest.skip("the reference's encoder body cannot split patches on a device arena")
+        stack_lib = binding.load_ref_stack_callers()
+        if stack_lib is None or not hasattr(stack_lib, "blt_local_encoder_forward"):
+            pytest.skip("oracle/_ref/libblt_ref_stack_callers.so was not built (needs the reference sources)")
+        entry = stack_lib.blt_local_encoder_forward
+    want_p, want_h = encoder_runs.run_oracle(oracle, c, data, lengths, weights)
+    got_p, got_h = encoder_runs.run_device(entry, lib, oracle, c, data, lengths, weights,
+                                           bytes_on_device=name != "small_k1")
+    assert_close(got_h, want_h, name + " byte_hidden_out")
+    assert_close(got_p, want_p, name + " patch_out")
+

@@ -40,8 +40,17 @@ OFF_PATH = {"blt_attention_head_core_backward", "blt_matmul_backward", "blt_rmsn
             "blt_rmsnorm_backward_add", "blt_rope_apply_packed_backward", "blt_swiglu_backward",
             "blt_cross_entropy_forward", "blt_cross_entropy_backward", "blt_gelu_forward",
             "blt_layernorm_forward", "blt_cast", "blt_container_alloc", "blt_tensor_view_2d", "blt_tensor_view_3d",
-            # training side of csrc/models/block_diffusion.c (loss scaling, D_0 table gradient)
-            "blt_indexed_row_scatter_add", "blt_scale"}
+            # training side of csrc/models/block_diffusion.c (D_0 table gradient)
+            "blt_indexed_row_scatter_add"}
+# the same for the layer stack, patch transformer and local encoder (csrc/models/transformer_stack.c,
+# global_transformer.c, local_encoder.c, hash_ngram.c, byte_embedding.c): backward passes, weight
+# casts for the reduced-precision modes and pure host helpers that stay with the reference build
+STACK_OFF_PATH = OFF_PATH | {"blt_cross_attention_backward", "blt_multihead_attention_backward", "blt_patch_pool_backward",
+                             "blt_embedding_scatter_add", "blt_indexed_row_scatter_add_normalized", "blt_scaled_copy",
+                             "blt_local_byte_grad_view", "blt_local_byte_layer_config", "blt_local_byte_weights_view",
+                             "blt_local_cross_weights_view", "blt_local_layer_grad_alloc",
+                             "blt_local_layer_storage_alloc", "blt_transformer_backward", "blt_transformer_forward_cached",
+                             "blt_cast_fp32_to_bf16", "blt_cast_fp32_to_fp8", "blt_matmul_bf16", "blt_matmul_fp8"}
 
 
 def test_reference_callers_find_their_ops_in_the_library():
@@ -61,6 +70,27 @@ def test_reference_callers_find_their_ops_in_the_library():
               "blt_strided_copy", "blt_rmsnorm_forward", "blt_swiglu_forward", "blt_add", "blt_tensor_create",
               "blt_tensor_upload", "blt_arena_alloc"):
         assert n in wanted, n
+
+
+def test_reference_encoder_and_stack_find_their_ops_in_the_library():
+    """The same for the reference's layer stack, patch transformer and local encoder: everything
+    their forward passes call is exported here, the two fused blocks (blt_transformer_forward,
+    blt_cross_attention_forward) and the encoder's small ops included."""
+    so = os.path.join(ROOT, "oracle", "_ref", "libblt_ref_stack_callers.so")
+    if not os.path.exists(so):
+        pytest.skip("oracle/_ref/libblt_ref_stack_callers.so was not built (needs the reference sources)")
+    out = subprocess.run(["nm", "-D", "-u", so], capture_output=True, text=True, check=True).stdout
+    wanted = {line.split()[-1] for line in out.splitlines() if line.split()[-1].startswith("blt_")}
+    lib = C.CDLL(api.LIB_PATH)
+    ref = C.CDLL(os.path.join(ROOT, "oracle", "_ref", "libblt_ref.so"))
+    missing = {n for n in wanted if not hasattr(lib, n) and not hasattr(ref, n)}
+    assert not missing, missing
+    for n in ("blt_transformer_forward", "blt_cross_attention_forward", "blt_embedding_lookup",
+              "blt_indexed_row_accumulate", "blt_scale", "blt_patch_pool_forward", "blt_rmsnorm_forward", "blt_add",
+              "blt_strided_copy", "blt_tensor_create", "blt_tensor_download", "blt_patch_build_group_ids"):
+        assert n in wanted and hasattr(lib, n), n
+    off = {n for n in wanted if not hasattr(lib, n)}
+    assert off <= STACK_OFF_PATH, off - STACK_OFF_PATH
 
 
 def test_header_layout_assertions_compile():
@@ -102,6 +132,16 @@ int main(void) {
     O(blt_transformer_config, norm_type); O(blt_transformer_config, activation_type); O(blt_transformer_config, use_bf16);
     S(blt_block_batch); O(blt_block_batch, t); O(blt_block_batch, tokens); O(blt_block_batch, positions);
     O(blt_block_batch, groups); O(blt_block_batch, loss_scale); O(blt_block_batch, trailing_closed);
+    S(blt_hash_ngram_config); O(blt_hash_ngram_config, num_ngram_sizes); O(blt_hash_ngram_config, per_ngram_vocab);
+    O(blt_hash_ngram_config, hash_prime); O(blt_hash_ngram_config, normalize); O(blt_hash_ngram_config, embed_dim);
+    S(blt_hash_ngram_weights); O(blt_hash_ngram_weights, num_tables);
+    S(blt_local_encoder_config); O(blt_local_encoder_config, patch_dim); O(blt_local_encoder_config, cross_attn_all_layers);
+    O(blt_local_encoder_config, cross_attn_placement); O(blt_local_encoder_config, pool_type);
+    O(blt_local_encoder_config, ngram_config); O(blt_local_encoder_config, rope_theta);
+    O(blt_local_encoder_config, max_seq_len);
+    S(blt_local_encoder); O(blt_local_encoder, byte_embedding_weight); O(blt_local_encoder, ngram_weights);
+    O(blt_local_encoder, rope_cos_cache); O(blt_local_encoder, rope_sin_cache); O(blt_local_encoder, layers);
+    printf("enum3 %%d %%u %%d\n", (int)BLT_POOL_MAX, (unsigned)BLT_IDX_SENTINEL, (int)BLT_MAX_NGRAM_SIZES);
     printf("enum %%d %%d %%d %%d %%d %%u\n", (int)BLT_XATTN_FIRST, (int)BLT_DTYPE_FP32, (int)BLT_BACKEND_CPU,
            (int)BLT_CROSS_ATTN_SPLIT_KV, (int)BLT_D0_LEARNED, (unsigned)BLT_MASK_TOKEN_ID);
     printf("enum2 %%d %%d\n", (int)BLT_NORM_RMSNORM, (int)BLT_ACTIVATION_SWIGLU);
@@ -119,7 +159,8 @@ def test_layout_matches_reference_headers(tmp_path):
     ref_inc = "\n".join('#include "%s"' % h for h in (
         "core/tensor.h", "core/allocator.h", "ops/attn_core.h", "ops/mask_builder.h", "ops/rope.h",
         "models/attention.h", "models/cross_attention.h", "models/transformer.h", "models/patcher.h",
-        "models/local_decoder.h", "infer/kv_cache.h", "models/block_diffusion.h"))
+        "models/local_decoder.h", "infer/kv_cache.h", "models/block_diffusion.h", "models/local_encoder.h",
+        "ops/gather_scatter.h"))
     outs = []
     for tag, inc_dir, inc in (("ref", REF_ROOT, ref_inc), ("own", os.path.join(ROOT, "include"), '#include "blt_abi.h"')):
         src = tmp_path / (tag + ".c")

@@ -7,7 +7,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from fblt_amd import abi
+from fblt_amd import abi, decoder
 from oracle import binding
 
 CPU = abi.BLT_BACKEND_CPU
@@ -605,3 +605,92 @@ def test_transformer_block_bit_exact(shape, oracle, ref):
         ref.blt_arena_destroy(arena)
     assert np.isfinite(theirs).all()
     assert mine.tobytes() == theirs.tobytes(), shape
+
+
+def test_encoder_ops_bit_exact(oracle, ref):
+    """The encoder's three small ops and its hashing against the reference build: indexed row
+    accumulation with sentinel entries, in-place scale, patch pooling (mean and maximum, patches of
+    1 ... 30 rows), and the bucket index list of every n-gram size 1 ... 8 out of the reference's
+    own rolling-hash state machine (csrc/models/hash_ngram.c:16-79)."""
+    rs = np.random.RandomState(77)
+    T, E, V = 91, 24, 131
+    table = rs.randn(V, E).astype(np.float32)
+    idx = rs.randint(0, V, size=T).astype(np.uint32)
+    idx[rs.randint(0, T, size=9)] = abi.BLT_IDX_SENTINEL
+    io0 = rs.randn(T, E).astype(np.float32)
+    mine, theirs = io0.copy(), io0.copy()
+    u32 = C.POINTER(C.c_uint32)
+    assert oracle.orc_indexed_row_accumulate(binding.fptr(table.reshape(-1)), V, idx.ctypes.data_as(u32),
+                                             binding.fptr(mine.reshape(-1)), T, E) == 0
+    tt, ti = abi.tensor_view(table.ctypes.data, table.shape, CPU), abi.tensor_view(theirs.ctypes.data, theirs.shape, CPU)
+    ref.blt_indexed_row_accumulate(C.byref(tt), idx.ctypes.data_as(u32), C.byref(ti))
+    assert mine.tobytes() == theirs.tobytes() and not np.array_equal(mine, io0)
+    oracle.orc_scale(binding.fptr(mine.reshape(-1)), mine.size, 1.0 / 7.0)
+    ref.blt_scale(C.byref(ti), 1.0 / 7.0)
+    assert mine.tobytes() == theirs.tobytes()
+
+    lengths = [1, 30, 2, 7, 1, 13, 5, 9, 23]
+    patches = decoder.patch_table(lengths)
+    h = rs.randn(sum(lengths), E).astype(np.float32)
+    for pool in (abi.BLT_POOL_MEAN, abi.BLT_POOL_MAX):
+        a, b = (np.zeros((len(lengths), E), dtype=np.float32) for _ in range(2))
+        assert oracle.orc_patch_pool_forward(binding.fptr(h.reshape(-1)), h.shape[0], E, patches, len(lengths), pool,
+                                             binding.fptr(a.reshape(-1))) == 0
+        th, tb = abi.tensor_view(h.ctypes.data, h.shape, CPU), abi.tensor_view(b.ctypes.data, b.shape, CPU)
+        ref.blt_patch_pool_forward(C.byref(th), patches, len(lengths), pool, C.byref(tb))
+        assert a.tobytes() == b.tobytes() and np.abs(a).sum() > 0
+
+    class State(C.Structure):   # csrc/models/hash_ngram.h:29-38
+        _fields_ = [("current_hash", C.c_uint64), ("prime", C.c_uint64), ("modulus", C.c_uint64),
+                    ("prime_pow_n", C.c_uint64), ("window", C.c_uint8 * 8), ("window_start", C.c_size_t),
+                    ("n", C.c_size_t), ("positions_seen", C.c_size_t)]
+    ref.blt_rolling_hash_init.restype = None
+    ref.blt_rolling_hash_init.argtypes = [C.POINTER(State), C.c_size_t, C.c_uint64, C.c_uint64]
+    ref.blt_rolling_hash_update.restype = C.c_uint64
+    ref.blt_rolling_hash_update.argtypes = [C.POINTER(State), C.c_uint8]
+    data = rs.randint(0, 256, size=300).astype(np.uint8)
+    data[40:60] = 7
+    for n in range(1, 9):
+        for prime, modulus in ((1000003, 50021), (31, 2), (2 ** 31 - 1, 2 ** 31 + 11)):
+            got = np.zeros(data.size, dtype=np.uint32)
+            assert oracle.orc_ngram_indices(data.ctypes.data_as(C.POINTER(C.c_uint8)), data.size, n, prime, modulus,
+                                            got.ctypes.data_as(u32)) == 0
+            st = State()
+            ref.blt_rolling_hash_init(C.byref(st), n, prime, modulus)
+            want = []
+            for b in data:
+                hv = ref.blt_rolling_hash_update(C.byref(st), int(b))
+                want.append(abi.BLT_IDX_SENTINEL if hv == 2 ** 64 - 1 else hv & 0xFFFFFFFF)
+            assert got.tolist() == want, (n, prime, modulus)
+
+
+ENCODER_SHAPES = [
+    dict(T=37, E=16, H=2, XH=2, L=1, hidden=24, ngrams=(3,), vocab=101, k=1, window=0, placement=0, all_layers=True,
+         pool="mean", docs=None, normalize=True, mean_patch=3),
+    dict(T=64, E=32, H=2, XH=4, L=2, hidden=40, ngrams=(2, 5, 8), vocab=257, k=2, window=9, placement=0,
+         all_layers=False, pool="max", docs=[20, 41], normalize=False, mean_patch=5),
+    dict(T=50, E=24, H=3, XH=1, L=3, hidden=32, ngrams=(0, 4, 60), vocab=64, k=3, window=0, placement=4,
+         all_layers=False, pool="mean", docs=[25], normalize=True, mean_patch=2),
+    dict(T=29, E=16, H=1, XH=2, L=2, hidden=16, ngrams=(), vocab=8, k=1, window=5, placement=1, all_layers=True,
+         pool="mean", docs=None, normalize=True, mean_patch=7),
+    dict(T=48, E=32, H=4, XH=2, L=2, hidden=48, ngrams=(3, 4, 5, 6, 7, 8), vocab=509, k=1, window=0, placement=3,
+         all_layers=False, pool="max", docs=None, normalize=True, mean_patch=4),
+]
+
+
+@pytest.mark.parametrize("shape", range(len(ENCODER_SHAPES)))
+def test_local_encoder_bit_exact(shape, oracle, ref):
+    """orc_local_encoder_forward against blt_local_encoder_forward compiled from the reference:
+    patch_out and byte_hidden_out bit for bit, over sub-token splits, window, documents, every kind
+    of cross placement (none at all included), both pools, 0 ... 6 n-gram tables (sizes of 0 and
+    beyond the sequence are skipped as the reference skips them)."""
+    from tests import encoder_runs
+    from tests.golden.block_cases import encoder_case
+    c = ENCODER_SHAPES[shape]
+    data, lengths, weights = encoder_case(np.random.RandomState(900 + shape), c)
+    mine = encoder_runs.run_oracle(oracle, c, data, lengths, weights)
+    theirs = encoder_runs.run_reference(ref, oracle, c, data, lengths, weights)
+    for a, b in zip(mine, theirs):
+        assert np.isfinite(b).all() and np.abs(b).sum() > 0
+        assert a.tobytes() == b.tobytes(), shape
+
