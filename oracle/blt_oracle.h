@@ -63,6 +63,20 @@
  *       two-token block -> {0.6697615, 0.3302385, ...}, causal row 0 one-hot
  *       (tests/unit/models/unit_attention.c:82-88, 160-171); a float64 numpy
  *       product; the block against its parts called by hand.
+ *   orc_rmsnorm_forward, orc_add, orc_swiglu_forward, orc_kv_decode_layer, orc_transformer_forward
+ *       bit-for-bit against oracle/_ref (blt_rmsnorm_forward, blt_add, blt_swiglu_forward,
+ *       blt_transformer_forward); RMSNorm of a constant row = +-weight, silu(0) = 0, float64.
+ *   orc_local_decoder_forward_diffusion_infer, orc_kv_block_step, orc_kv_*_step_kind
+ *       bit-for-bit against oracle/_ref's blt_local_decoder_forward_diffusion_infer over D_0
+ *       modes, sub-token split, window, placements and block geometry; the cached form (prefix as
+ *       an incremental step, block rows as one block step) bit-for-bit against the dense one.
+ *   orc_indexed_row_accumulate, orc_scale, orc_patch_pool_forward, orc_ngram_indices,
+ *   orc_embed_bytes, orc_local_encoder_forward
+ *       bit-for-bit against oracle/_ref: the three ops on random inputs with sentinel entries and
+ *       patches of 1..30 rows, the index lists of n = 1..8 against the reference's own
+ *       blt_rolling_hash_init / _update state machine (three prime / modulus pairs, a run of equal
+ *       bytes), the whole forward (patch_out and byte_hidden_out) over sub-token splits, window,
+ *       documents, every cross placement, both pools and 0..6 tables.
  */
 #ifndef FBLT_AMD_ORACLE_H
 #define FBLT_AMD_ORACLE_H
