@@ -334,6 +334,10 @@ void plan_build(blt_attention_plan &pl, const blt_attention_problem *problems, s
         pl.host.push_back(d);
     }
     for (Bucket &b : pl.buckets) {
+        if (b.fam == FAM_ROWS) { /* strided batches need no descriptor memory in this family either */
+            b.affine = detect_affine(pl.host.data() + b.base, b.count, b.aff);
+            continue;
+        }
         if (b.fam != FAM_MFMA) continue;
         b.affine = detect_affine(pl.host.data() + b.base, b.count, b.aff);
         if (choose_fine(pl.host.data() + b.base, b.count, b.affine, b.span, b.tall)) b.fam = FAM_FINE;
@@ -369,6 +373,8 @@ void plan_launch(const blt_attention_plan &pl, const AttnProb *dev, const AttnTi
             attn_mfma_launch_affine(b.aff, 0);
         else if (b.fam == FAM_MFMA)
             attn_mfma_launch(dev, dev_tiles + b.tile_base, b.tiles, b.hd, b.vec4, b.dense, 0);
+        else if (b.affine)
+            attn_rows_launch_affine(b.aff, 0);
         else
             attn_rows_launch(dev, b.base, b.count, b.hd, b.max_nq, 0);
     }
@@ -391,6 +397,12 @@ struct Staging {
         const size_t tbytes = plan.tiles.size() * sizeof(AttnTile);
         const size_t need = pbytes + tbytes;
         if (need == 0) return;
+        bool strided = true; /* every bucket travels in kernel arguments: nothing to stage */
+        for (const Bucket &b : plan.buckets) strided = strided && b.affine;
+        if (strided) {
+            plan_launch(plan, nullptr, nullptr);
+            return;
+        }
         BLT_REQUIRE(!blt_stream_capturing(),
                     "blt_attention_batch: this batch stages its descriptors through host memory, which a graph "
                     "cannot replay; use a resident plan (blt_attention_plan_*) or a strided batch under capture");

@@ -33,6 +33,9 @@ void attn_rows_launch(const AttnProb *dprobs, uint32_t base, uint32_t count, uin
                       hipStream_t s);
 /* one problem, descriptor passed as a kernel argument (nothing staged) */
 void attn_rows_launch_single(const AttnProb &single, hipStream_t s);
+/* a strided batch, descriptors in the kernel arguments (declared below the AttnAffine struct) */
+
+void attn_rows_launch_affine(const AttnAffine &aff, hipStream_t s);
 
 /* mfma family */
 bool attn_mfma_can(const AttnProb &d);

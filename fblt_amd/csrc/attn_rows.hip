@@ -13,6 +13,7 @@
  */
 #include "attn_device.h"
 #include "attn_launch.h"
+#include "attn_tile.h"
 #include "launch.h"
 
 namespace {
@@ -51,13 +52,19 @@ __device__ __forceinline__ void store4(float *row, uint32_t d, uint32_t hd, bool
 
 __device__ __forceinline__ float dot4(float4 a, float4 b) { return a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w; }
 
-template <int G, int T, bool SINGLE>
+/* SRC: where the workgroup finds its problem (attn_tile.h): a device array, the kernel arguments
+ * (one problem), or the kernel arguments of a strided batch -- the last two need no trip to memory
+ * before the row ranges and the rows themselves can be requested. */
+template <int G, int T, int SRC>
 __global__ __launch_bounds__(256) void attn_rows_kernel(const AttnProb *__restrict__ probs, uint32_t prob_base,
-                                                        AttnProb single) {
+                                                        AttnAffine aff) {
     constexpr int ROWS_PER_WAVE = 64 / G;
     constexpr int ROWS_PER_BLOCK = 4 * ROWS_PER_WAVE;
 
-    const AttnProb p = SINGLE ? single : probs[prob_base + blockIdx.y];
+    AttnProb p;
+    if (SRC == SRC_TILES) p = probs[prob_base + blockIdx.y];
+    else if (SRC == SRC_SINGLE) p = aff.first;
+    else affine_problem(p, aff, prob_base + blockIdx.y, aff.first.vis == ATTN_VIS_DENSE);
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
     const uint32_t g = lane % G;
@@ -183,22 +190,26 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const AttnProb *__restri
     }
 }
 
+/* `aff`: NULL = problems [base, base + count) of the device array; count == 0 in it = its first
+ * problem alone; else the strided batch it describes, problems [base, base + count) of it */
 template <int G, int T>
-void launch_rows(const AttnProb *dprobs, uint32_t base, uint32_t count, uint32_t max_nq, const AttnProb *single,
+void launch_rows(const AttnProb *dprobs, uint32_t base, uint32_t count, uint32_t max_nq, const AttnAffine *aff,
                  hipStream_t s) {
     constexpr int ROWS_PER_BLOCK = 4 * (64 / G);
     dim3 grid((max_nq + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK, count, 1);
-    if (single) {
-        blt_launch("attn_rows", attn_rows_kernel<G, T, true>, grid, dim3(256), 0, s, dprobs, base, *single);
+    if (aff && aff->count == 0) {
+        blt_launch("attn_rows", attn_rows_kernel<G, T, SRC_SINGLE>, grid, dim3(256), 0, s, dprobs, base, *aff);
+    } else if (aff) {
+        blt_launch("attn_rows", attn_rows_kernel<G, T, SRC_AFFINE>, grid, dim3(256), 0, s, dprobs, base, *aff);
     } else {
-        AttnProb none;
+        AttnAffine none;
         __builtin_memset(&none, 0, sizeof(none));
-        blt_launch("attn_rows", attn_rows_kernel<G, T, false>, grid, dim3(256), 0, s, dprobs, base, none);
+        blt_launch("attn_rows", attn_rows_kernel<G, T, SRC_TILES>, grid, dim3(256), 0, s, dprobs, base, none);
     }
 }
 
 void dispatch_rows(const AttnProb *dprobs, uint32_t b, uint32_t n, uint32_t hd, uint32_t max_nq,
-                   const AttnProb *single, hipStream_t s) {
+                   const AttnAffine *single, hipStream_t s) {
     const uint32_t chunks = (hd + 3) / 4;
     if (chunks <= 1) launch_rows<1, 1>(dprobs, b, n, max_nq, single, s);
     else if (chunks <= 2) launch_rows<2, 1>(dprobs, b, n, max_nq, single, s);
@@ -227,5 +238,18 @@ void attn_rows_launch(const AttnProb *dprobs, uint32_t base, uint32_t count, uin
 
 void attn_rows_launch_single(const AttnProb &single, hipStream_t s) {
     if (single.nq == 0) return;
-    dispatch_rows(nullptr, 0, 1, single.hd, single.nq, &single, s);
+    AttnAffine a;
+    __builtin_memset(&a, 0, sizeof(a));
+    a.first = single; /* count stays 0: one problem */
+    dispatch_rows(nullptr, 0, 1, single.hd, single.nq, &a, s);
+}
+
+/* A strided batch: the descriptors travel in the kernel arguments. */
+void attn_rows_launch_affine(const AttnAffine &aff, hipStream_t s) {
+    if (aff.count == 0 || aff.first.nq == 0) return;
+    for (uint32_t done = 0; done < aff.count;) { /* grid.y is limited to 65535 */
+        const uint32_t n = aff.count - done < 65535u ? aff.count - done : 65535u;
+        dispatch_rows(nullptr, done, n, aff.first.hd, aff.first.nq, &aff, s);
+        done += n;
+    }
 }
