@@ -55,6 +55,7 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
  * take the span's 32-key sub-chunks round-robin and merge through LDS. */
 template <int HD, int WAVES, bool KARG>
 __global__ __launch_bounds__(64 * WAVES, 2) void kv_block_mfma_kernel(StepArgs a, LensArg<KARG> lens) {
+    kv_fetch_arguments(a);
     constexpr int HALF = HD / 2;
     constexpr int DB = HD / 32;
     constexpr int ROW = HD + 4;
@@ -427,6 +428,7 @@ __device__ __forceinline__ void kv_merge_slices(const StepArgs &a, const float (
  *   - the slices meet once in LDS; the merge issues all of a cell's reads before it adds. */
 template <int HD, int WAVES, bool KARG>
 __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs a, LensArg<KARG> lens) {
+    kv_fetch_arguments(a);
     constexpr int HALF = HD / 2;
     constexpr int QD = HD / 4;  /* columns of the head one lane group contracts */
     constexpr int DT = HD / 16; /* 16-row tiles of O^T */
@@ -686,6 +688,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
  * rows; which of the two a sub-chunk is, is uniform over the wave. */
 template <int WAVES, int MAXW, bool LOOP, bool KARG> /* WAVES: slots of the merge (a power of two), MAXW <= WAVES: most waves launched */
 __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a, LensArg<KARG> lens) {
+    kv_fetch_arguments(a);
     constexpr int HD = 32, HALF = 16;
     constexpr int LPR = HD + 4; /* a parked result row in LDS, 16-byte aligned */
     constexpr uint32_t ROWS = 4, CH = 64;

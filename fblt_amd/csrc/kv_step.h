@@ -60,6 +60,18 @@ struct StepArgs {
 };
 
 
+/* Asks for every member of the launch's argument block at once, at kernel entry: left to itself the
+ * compiler fetches them group by group where they are first needed, and each group is a round
+ * trip through a scalar cache that is cold at the start of a launch. */
+__device__ __forceinline__ void kv_fetch_arguments(const StepArgs &a) {
+    asm volatile("" ::"s"(a.cache_k), "s"(a.cache_v), "s"(a.self_len), "s"(a.q_rows), "s"(a.k_rows), "s"(a.v_rows),
+                 "s"(a.combined), "s"(a.rope_cos), "s"(a.rope_sin));
+    asm volatile("" ::"s"(a.partial), "s"(a.tickets), "s"(a.error), "s"(a.q_stride), "s"(a.k_stride), "s"(a.v_stride),
+                 "s"(a.out_stride), "s"(a.max_seq_len), "s"(a.embed_dim), "s"(a.num_heads), "s"(a.window));
+    asm volatile("" ::"s"(a.n), "s"(a.n_seq), "s"(a.len_bias), "s"(a.q0), "s"(a.splits), "s"(a.span), "s"(a.cap),
+                 "s"(a.hpb), "s"(a.slices), "s"(a.scale), "s"(a.block_kind), "s"(a.write_through), "s"(a.commit));
+}
+
 /* Where a launch takes the sequences' lengths from: a.self_len in device memory, or -- when the
  * caller keeps the lengths on the host, as the reference does (csrc/infer/kv_cache.h:56-60) -- the
  * kernel arguments themselves, KARG_SEQS sequences per launch.  With the lengths in the argument
