@@ -407,7 +407,10 @@ __device__ __forceinline__ void kv_merge_slices(const StepArgs &a, const float (
  *                    head's columns [g * HD/4, (g + 1) * HD/4), one per step;
  *   O^T[d, query]:   HD/16 tiles; the contraction runs over the keys, lane group g taking key
  *                    16 t + 4 g + r at step (t, r) -- exactly the key whose weight its S^T
- *                    register (t, r) holds, so P^T needs no exchange.
+ *                    register (t, r) holds, so P^T needs no exchange.  Row i of tile e is column
+ *                    (HD/16) i + e of the head: a lane's HD/16 operands of one key are
+ *                    consecutive floats, one 8- or 16-byte load, and the sixteen lanes of a group
+ *                    read the key's row as one contiguous piece.
  *
  * Half the matrix-core cycles and half the softmax arithmetic of the 32-wide kernel per
  * sub-chunk.  K and V fragments come straight from global memory in fragment layout (a K row's
@@ -472,10 +475,10 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
     const float *const new_v = a.v_rows + newrow0 * a.v_stride + hsafe * HD;
     const uint32_t cache_pitch = a.embed_dim * 4u, newk_pitch = a.k_stride * 4u, newv_pitch = a.v_stride * 4u;
     const uint32_t last_cached = len > 0u ? len - 1u : 0u, last_new = a.n - 1u;
-    const uint32_t lane_k = g * (QD * 4u), lane_v = c * 4u; /* byte offsets inside a row */
+    const uint32_t lane_k = g * (QD * 4u), lane_v = c * (DT * 4u); /* byte offsets inside a row */
 
     /* K fragment of sub-chunk si: tile t holds its row 16 t + c, columns g*QD ...;
-     * V fragment: element (d, 4 t + r) is column 16 d + c of its row 16 t + 4 g + r */
+     * V fragment: element (e, 4 t + r) is column DT c + e of its row 16 t + 4 g + r */
     auto request = [&](float (&kf)[2][QD], float (&vf)[DT][8], uint32_t si) __attribute__((always_inline)) {
         const bool fresh = si >= cached_subs; /* wave-uniform: scalar selects */
         const char *kb = reinterpret_cast<const char *>(fresh ? new_k : cache_k);
@@ -494,8 +497,14 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
 #pragma unroll
         for (int u = 0; u < 8; u++) {
             const uint32_t off = min(row0 + 16u * (u >> 2) + (u & 3) + 4u * g, limit) * vp + lane_v;
-#pragma unroll
-            for (int d = 0; d < DT; d++) vf[d][u] = *reinterpret_cast<const float *>(vb + off + 64 * d);
+            if constexpr (DT == 2) {
+                const float2 x = *reinterpret_cast<const float2 *>(vb + off);
+                vf[0][u] = x.x, vf[1][u] = x.y;
+            } else {
+                static_assert(DT == 4, "head widths 32 and 64");
+                const float4 x = *reinterpret_cast<const float4 *>(vb + off);
+                vf[0][u] = x.x, vf[1][u] = x.y, vf[2][u] = x.z, vf[3][u] = x.w;
+            }
         }
     };
 
@@ -576,9 +585,9 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
                 for (int u = 0; u < 8; u++) {
                     const uint32_t r = 16u * (u >> 2) + 4u * g + (u & 3);
                     if (r < a.n) {
-#pragma unroll
-                        for (int d = 0; d < DT; d++)
-                            a.cache_v[(slab + len + r) * a.embed_dim + head * HD + 16 * d + c] = vf[d][u];
+                        float *dst = a.cache_v + (slab + len + r) * a.embed_dim + head * HD + DT * c;
+                        if constexpr (DT == 2) *reinterpret_cast<float2 *>(dst) = make_float2(vf[0][u], vf[1][u]);
+                        else *reinterpret_cast<float4 *>(dst) = make_float4(vf[0][u], vf[1][u], vf[2][u], vf[3][u]);
                     }
                 }
             }
@@ -648,12 +657,21 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
     /* the four lane groups of a column carry the same m, their sums add */
     l = swap32(swap16(l, OpSum()), OpSum());
 
-    /* lane (g, c) holds O^T[d = 16 dt + 4 g + r][query c]: park rows [query][HD columns, max, sum]
-     * in the wave's LDS tile */
+    /* lane (g, c) holds O^T[column DT (4 g + r) + e][query c] in oacc[e][r], i.e. the 4 DT
+     * consecutive columns from 4 DT g on: park rows [query][HD columns, max, sum] in the wave's
+     * LDS tile */
     float *mine = sm_o[wave];
+    if constexpr (DT == 2) {
 #pragma unroll
-    for (int d = 0; d < DT; d++)
-        *reinterpret_cast<float4 *>(mine + c * LPR + 16 * d + 4 * g) = make_float4(oacc[d][0], oacc[d][1], oacc[d][2], oacc[d][3]);
+        for (int r = 0; r < 4; r += 2)
+            *reinterpret_cast<float4 *>(mine + c * LPR + 8 * g + 2 * r) =
+                make_float4(oacc[0][r], oacc[1][r], oacc[0][r + 1], oacc[1][r + 1]);
+    } else {
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+            *reinterpret_cast<float4 *>(mine + c * LPR + 16 * g + 4 * r) =
+                make_float4(oacc[0][r], oacc[1][r], oacc[2][r], oacc[3][r]);
+    }
     if (g == 0) *reinterpret_cast<float2 *>(mine + c * LPR + HD) = make_float2(m * LN2, l); /* merges work in natural units */
     BLT_MARK(5);
     __syncthreads();
