@@ -35,6 +35,7 @@ struct Bucket {
     uint32_t tile_base;
     uint32_t span;    /* fine: keys the longest 32-row tile needs */
     bool tall;        /* fine: 16-row workgroups of sixteen waves */
+    bool whole;       /* fine: one four-wave workgroup per whole problem (strided batches) */
 };
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -207,6 +208,32 @@ bool choose_fine(const AttnProb *p, uint32_t n, bool strided, uint32_t &span, bo
     return groups < (max_nk <= 64u ? 640u : 448u);
 }
 
+/* Does a strided batch of n problems like `d` go to the fine family's whole-problem shape (one
+ * four-wave workgroup per problem of at most 128 rows whose keys fit one LDS fill)?  It fetches
+ * K and V once per problem and balances the causal triangle inside the workgroup, which pays once
+ * the batch is several workgroups deep on every compute unit.  BLT_HIP_FINE_ROWS=128 pins it
+ * wherever the shape allows (tuning and test hook), BLT_HIP_WHOLE_MIN moves the threshold. */
+bool choose_whole(const AttnProb &d, uint32_t n, bool strided) {
+    static const int rows_pinned = [] {
+        const char *e = getenv("BLT_HIP_FINE_ROWS");
+        return e ? std::atoi(e) : 0;
+    }();
+    static const uint32_t min_problems = [] {
+        const char *e = getenv("BLT_HIP_WHOLE_MIN");
+        const long v = e ? std::atol(e) : 0;
+        return v > 0 ? (uint32_t)v : 0u;
+    }();
+    const int forced = family_override();
+    if (!strided || (forced != 0 && forced != 4) || !attn_whole_can(d)) return false;
+    if (rows_pinned != 0) return rows_pinned == 128;
+    if (forced != 0 || d.nq < 48u) return false; /* three row halves and fewer leave most of the waves idle */
+    if (min_problems) return n >= min_problems;
+    /* measured against the family's other shapes and the wide kernel (8 heads of 64 and 4 heads
+     * of 32): 128 rows ahead from 144 problems on (11.9 against 12.4 us; 12.5 against 15.6 at
+     * 256, 38.7 against 45.5 at 1024, 72.5 against 86 at 2048), 64 rows from 768 on */
+    return n >= (d.nq > 64u ? 144u : 640u);
+}
+
 /* Element distance between two float pointers (either both NULL or both set). */
 bool elem_delta(const void *a, const void *b, int64_t &out) {
     if ((a == nullptr) != (b == nullptr)) return false;
@@ -340,7 +367,9 @@ void plan_build(blt_attention_plan &pl, const blt_attention_problem *problems, s
         }
         if (b.fam != FAM_MFMA) continue;
         b.affine = detect_affine(pl.host.data() + b.base, b.count, b.aff);
-        if (choose_fine(pl.host.data() + b.base, b.count, b.affine, b.span, b.tall)) b.fam = FAM_FINE;
+        b.whole = choose_whole(pl.host[b.base], b.count, b.affine);
+        if (b.whole) b.fam = FAM_FINE;
+        else if (choose_fine(pl.host.data() + b.base, b.count, b.affine, b.span, b.tall)) b.fam = FAM_FINE;
         else if (choose_wide(pl.host.data() + b.base, b.count)) b.fam = FAM_WIDE;
         if (b.affine) continue; /* no descriptor or tile memory needed */
         b.tile_base = (uint32_t)pl.tiles.size();
@@ -365,6 +394,8 @@ void plan_launch(const blt_attention_plan &pl, const AttnProb *dev, const AttnTi
             attn_wide_launch_affine(b.aff, 0);
         else if (b.fam == FAM_WIDE)
             attn_wide_launch(dev, dev_tiles + b.tile_base, b.tiles, b.hd, b.dense, 0);
+        else if (b.fam == FAM_FINE && b.whole)
+            attn_whole_launch_affine(b.aff, 0);
         else if (b.fam == FAM_FINE && b.affine)
             attn_fine_launch_affine(b.aff, b.tall, 0);
         else if (b.fam == FAM_FINE)

@@ -39,6 +39,11 @@
  * latency chain; the next fill is requested before the units of the current one
  * start.
  *
+ * A third shape (attn_whole_kernel) serves strided batches of many short problems
+ * (at most 128 rows, keys within one fill), where the launch is several workgroups
+ * deep on every compute unit and the time is the bytes moved: one four-wave
+ * workgroup per problem fetches K and V once for all of its rows.
+ *
  * Takes closed-form visibility (all keys, causal with optional window), head
  * widths 32 and 64 with 16-byte aligned rows, no weights output.
  */
@@ -102,6 +107,148 @@ __device__ __forceinline__ void fine_span(const AttnProb &p, uint32_t first, uin
     const bool any = hi_a > lo_a;
     tlo = any ? lo_a : 0xFFFFFFFFu, thi = any ? hi_b : 0u;
     flo = lo_b, fhi = hi_a;
+}
+
+/* One unit: 16 query rows (fragment qf, pre-loaded) against the 16 keys whose K rows start at
+ * krow (this lane: row c, columns g*HD/4 ...) and whose V rows start at vrow (this lane: rows 4 g + r,
+ * column c) in LDS, rows ROW = HD + 4 floats apart.  Register r of the lane's scores is key
+ * 4 g + r of the tile; that key is visible iff rel + r < len (unsigned: rel = the key's offset
+ * into the row's range).  Running maximum m (log2 units), sum l and O^T accumulators are updated. */
+template <int HD>
+__device__ __forceinline__ void fine_unit(const float *krow, const float *vrow, const float (&qf)[HD / 4],
+                                          floatx4 (&oacc)[HD / 16], float &m, float &l, const uint32_t rel,
+                                          const uint32_t len, const float scale2) {
+    constexpr int QD = HD / 4, DT = HD / 16, ROW = HD + 4;
+    float kf[QD];
+#pragma unroll
+    for (int s = 0; s < QD; s += 4) {
+        const float4 t = *reinterpret_cast<const float4 *>(krow + s);
+        kf[s + 0] = t.x, kf[s + 1] = t.y, kf[s + 2] = t.z, kf[s + 3] = t.w;
+    }
+    float vf[DT][4];
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+#pragma unroll
+        for (int d = 0; d < DT; d++) vf[d][r] = vrow[r * ROW + 16 * d];
+
+    /* S^T on two accumulators: neither chain waits for its own previous result */
+    floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < QD; s += 2) {
+        s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[s], qf[s], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[s + 1], qf[s + 1], s1, 0, 0, 0);
+    }
+
+    float x[4];
+    float mt = neg_inf();
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const float t = (s0[r] + s1[r]) * scale2;
+        const bool vis = ((rel + r) < len) & isfinite(t);
+        x[r] = vis ? t : neg_inf();
+        mt = fmaxf(mt, x[r]);
+    }
+    mt = swap32(swap16(mt, OpMax()), OpMax());
+    const float mn = fmaxf(m, mt);
+    const float ms = mn == neg_inf() ? 0.f : mn;
+    const float alpha = fast_exp2(m - ms);
+    float ps = 0.f;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        x[r] = fast_exp2(x[r] - ms);
+        ps += x[r];
+    }
+    l = l * alpha + ps;
+    m = mn;
+#pragma unroll
+    for (int d = 0; d < DT; d++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) oacc[d][r] *= alpha;
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+#pragma unroll
+        for (int d = 0; d < DT; d++) oacc[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[d][r], x[r], oacc[d], 0, 0, 0);
+}
+
+/* Two units of the same query rows side by side -- key tiles at (krow0, vrow0) and (krow1, vrow1),
+ * each with a running state of its own -- written out interleaved, so that one unit's softmax
+ * arithmetic fills the time the other's matrix instructions take.  The two states are merged by
+ * the caller (fine_merge_states). */
+template <int HD>
+__device__ __forceinline__ void fine_unit2(const float *krow0, const float *vrow0, const float *krow1, const float *vrow1,
+                                           const float (&qf)[HD / 4], floatx4 (&oa)[HD / 16], float &ma, float &la,
+                                           floatx4 (&ob)[HD / 16], float &mb, float &lb, const uint32_t rel0,
+                                           const uint32_t rel1, const uint32_t len, const float scale2) {
+    constexpr int QD = HD / 4, DT = HD / 16, ROW = HD + 4;
+    float ka[QD], kb[QD];
+#pragma unroll
+    for (int s = 0; s < QD; s += 4) {
+        const float4 t = *reinterpret_cast<const float4 *>(krow0 + s);
+        const float4 u = *reinterpret_cast<const float4 *>(krow1 + s);
+        ka[s + 0] = t.x, ka[s + 1] = t.y, ka[s + 2] = t.z, ka[s + 3] = t.w;
+        kb[s + 0] = u.x, kb[s + 1] = u.y, kb[s + 2] = u.z, kb[s + 3] = u.w;
+    }
+    float va[DT][4], vb[DT][4];
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+#pragma unroll
+        for (int d = 0; d < DT; d++) va[d][r] = vrow0[r * ROW + 16 * d], vb[d][r] = vrow1[r * ROW + 16 * d];
+
+    floatx4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < QD; s++) {
+        sa = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[s], qf[s], sa, 0, 0, 0);
+        sb = __builtin_amdgcn_mfma_f32_16x16x4f32(kb[s], qf[s], sb, 0, 0, 0);
+    }
+
+    float xa[4], xb[4];
+    float ta = neg_inf(), tb = neg_inf();
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const float a = sa[r] * scale2, b = sb[r] * scale2;
+        xa[r] = (((rel0 + r) < len) & isfinite(a)) ? a : neg_inf();
+        xb[r] = (((rel1 + r) < len) & isfinite(b)) ? b : neg_inf();
+        ta = fmaxf(ta, xa[r]), tb = fmaxf(tb, xb[r]);
+    }
+    ta = swap32(swap16(ta, OpMax()), OpMax());
+    tb = swap32(swap16(tb, OpMax()), OpMax());
+    const float na = fmaxf(ma, ta), nb = fmaxf(mb, tb);
+    const float za = na == neg_inf() ? 0.f : na, zb = nb == neg_inf() ? 0.f : nb;
+    const float fa = fast_exp2(ma - za), fb = fast_exp2(mb - zb);
+    float pa = 0.f, pb = 0.f;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        xa[r] = fast_exp2(xa[r] - za), xb[r] = fast_exp2(xb[r] - zb);
+        pa += xa[r], pb += xb[r];
+    }
+    la = la * fa + pa, lb = lb * fb + pb;
+    ma = na, mb = nb;
+#pragma unroll
+    for (int d = 0; d < DT; d++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) oa[d][r] *= fa, ob[d][r] *= fb;
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+#pragma unroll
+        for (int d = 0; d < DT; d++) {
+            oa[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(va[d][r], xa[r], oa[d], 0, 0, 0);
+            ob[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(vb[d][r], xb[r], ob[d], 0, 0, 0);
+        }
+}
+
+/* state b folded into state a (log2-unit maxima) */
+template <int DT>
+__device__ __forceinline__ void fine_merge_states(floatx4 (&oa)[DT], float &ma, float &la, const floatx4 (&ob)[DT],
+                                                  const float mb, const float lb) {
+    const float mn = fmaxf(ma, mb);
+    const float ms = mn == neg_inf() ? 0.f : mn;
+    const float fa = fast_exp2(ma - ms), fb = fast_exp2(mb - ms);
+    la = la * fa + lb * fb;
+    ma = mn;
+#pragma unroll
+    for (int d = 0; d < DT; d++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) oa[d][r] = oa[d][r] * fa + ob[d][r] * fb;
 }
 
 template <int HD, int SRC, int HALVES, int WAVES>
@@ -258,59 +405,9 @@ __global__ __launch_bounds__(64 * WAVES, 4) void attn_fine_kernel(const AttnProb
                 const uint32_t k0 = kt * 16u;
                 const float *krow = sm_k + (k0 - c0 + c) * ROW + g * QD;
                 const float *vrow = sm_v + (k0 - c0 + 4u * g) * ROW + c;
-                float kf[QD];
-#pragma unroll
-                for (int s = 0; s < QD; s += 4) {
-                    const float4 t = *reinterpret_cast<const float4 *>(krow + s);
-                    kf[s + 0] = t.x, kf[s + 1] = t.y, kf[s + 2] = t.z, kf[s + 3] = t.w;
-                }
-                float vf[DT][4];
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-#pragma unroll
-                    for (int d = 0; d < DT; d++) vf[d][r] = vrow[r * ROW + 16 * d];
-
-                /* S^T on two accumulators: neither chain waits for its own previous result */
-                floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int s = 0; s < QD; s += 2) {
-                    s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[s], qf[s], s0, 0, 0, 0);
-                    s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[s + 1], qf[s + 1], s1, 0, 0, 0);
-                }
-
                 const bool all_seen = k0 >= half_flo && k0 + 16u <= half_fhi; /* uniform over the wave */
-                const uint32_t vlo = all_seen ? 0u : lo;
-                const uint32_t vlen = all_seen ? 0xFFFFFFFFu : (hi > lo ? hi - lo : 0u);
-                float x[4];
-                float mt = neg_inf();
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const float t = (s0[r] + s1[r]) * scale2;
-                    const bool vis = ((k0 + 4u * g + r - vlo) < vlen) & isfinite(t);
-                    x[r] = vis ? t : neg_inf();
-                    mt = fmaxf(mt, x[r]);
-                }
-                mt = swap32(swap16(mt, OpMax()), OpMax());
-                const float mn = fmaxf(m, mt);
-                const float ms = mn == neg_inf() ? 0.f : mn;
-                const float alpha = fast_exp2(m - ms);
-                float ps = 0.f;
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    x[r] = fast_exp2(x[r] - ms);
-                    ps += x[r];
-                }
-                l = l * alpha + ps;
-                m = mn;
-#pragma unroll
-                for (int d = 0; d < DT; d++)
-#pragma unroll
-                    for (int r = 0; r < 4; r++) oacc[d][r] *= alpha;
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-#pragma unroll
-                    for (int d = 0; d < DT; d++)
-                        oacc[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[d][r], x[r], oacc[d], 0, 0, 0);
+                fine_unit<HD>(krow, vrow, qf, oacc, m, l, k0 + 4u * g - (all_seen ? 0u : lo),
+                              all_seen ? 0xFFFFFFFFu : (hi > lo ? hi - lo : 0u), scale2);
                 kt += WPH;
             }
             return c0 + RPP * pieces_done < fill_end; /* more keys to come: uniform over the workgroup */
@@ -381,6 +478,159 @@ __global__ __launch_bounds__(64 * WAVES, 4) void attn_fine_kernel(const AttnProb
             }
         }
     }
+}
+
+/* Whole short problems (at most 128 query rows, keys that fit one fill), for strided batches of
+ * so many of them that throughput matters and the launch floor does not: the workgroup -- four
+ * waves -- fetches the problem's K and V rows ONCE into LDS, meets once, and from there on its
+ * waves run on their own.  Wave w takes the row halves (of 16 rows) n-1-w and w, one after the
+ * other: under a causal mask the two add up to the same number of units for every wave, and a
+ * half's keys are all the wave's own, so nothing is merged; the finished rows go to global
+ * memory straight from the accumulators.  Two workgroups fit a compute unit (LDS), so one
+ * fetches while the other computes. */
+template <int HD>
+struct WholeShape {
+    static constexpr uint32_t THREADS = 256;
+    static constexpr uint32_t MAX_ROWS = 128;
+    static constexpr uint32_t KC_MAX = FineShape<HD, 2, 8>::KC_MAX;
+    static constexpr int ROW = HD + 4, LPR4 = HD / 4;
+    static constexpr int PIECES = (int)(KC_MAX * LPR4 / THREADS);
+};
+
+template <int HD>
+__global__ __launch_bounds__(256, 2) void attn_whole_kernel(AttnAffine aff, uint32_t kc) {
+    using Shape = WholeShape<HD>;
+    constexpr int ROW = Shape::ROW, LPR4 = Shape::LPR4, QD = HD / 4, DT = HD / 16;
+    extern __shared__ __attribute__((aligned(16))) float sm[];
+    float *const sm_k = sm;
+    float *const sm_v = sm + (size_t)kc * ROW;
+
+    asm volatile("" ::"s"(aff.first.q), "s"(aff.first.k), "s"(aff.first.v), "s"(aff.first.out), "s"(aff.first.lse));
+    asm volatile("" ::"s"(aff.first.q_stride), "s"(aff.first.k_stride), "s"(aff.first.v_stride),
+                 "s"(aff.first.out_stride), "s"(aff.first.nq), "s"(aff.first.nk), "s"(aff.first.vis),
+                 "s"(aff.first.causal_off), "s"(aff.first.window), "s"(aff.first.scale));
+    asm volatile("" ::"s"(aff.q_seq), "s"(aff.q_head), "s"(aff.k_seq), "s"(aff.k_head), "s"(aff.v_seq), "s"(aff.v_head),
+                 "s"(aff.o_seq), "s"(aff.o_head), "s"(aff.lse_seq), "s"(aff.lse_head));
+    asm volatile("" ::"s"(aff.count), "s"(aff.heads), "s"(kc));
+    AttnProb p;
+    affine_problem(p, aff, blockIdx.x, false);
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t g = lane >> 4, c = lane & 15u;
+    const uint32_t halves = (p.nq + 15u) / 16u; /* at most 8 */
+
+    /* keys the problem needs: rows [c0, key_end), at most kc of them */
+    uint32_t tlo, thi, flo, fhi;
+    fine_span(p, 0u, p.nq - 1u, tlo, thi, flo, fhi);
+    const uint32_t c0 = thi > tlo ? tlo / 16u * 16u : 0u;
+    const uint32_t key_end = thi > tlo ? (thi + 15u) / 16u * 16u : 0u;
+    const uint32_t last_key = min(max(key_end, 1u), p.nk) - 1u;
+
+    /* the wave's two row halves; hb == NONE: one half, ha == NONE: nothing */
+    constexpr uint32_t NONE = 0xFFFFFFFFu;
+    const uint32_t ha = wave < halves && halves - 1u - wave >= wave ? halves - 1u - wave : NONE;
+    const uint32_t hb = ha != NONE && ha > wave ? wave : NONE;
+
+    auto load_q = [&](float (&qf)[QD], const uint32_t half) __attribute__((always_inline)) {
+        const uint32_t row = min(16u * (half == NONE ? 0u : half) + c, p.nq - 1u);
+        const float *qrow = p.q + (size_t)row * p.q_stride + g * QD;
+#pragma unroll
+        for (int s = 0; s < QD; s += 4) {
+            const float4 t = *reinterpret_cast<const float4 *>(qrow + s);
+            qf[s + 0] = t.x, qf[s + 1] = t.y, qf[s + 2] = t.z, qf[s + 3] = t.w;
+        }
+    };
+    float qa[QD], qb[QD];
+    load_q(qa, ha);
+    load_q(qb, hb);
+
+    /* ---- the fill: every piece is requested, then parked in the order it was requested ---- */
+    float4 kp[Shape::PIECES], vp[Shape::PIECES];
+#pragma unroll
+    for (int t = 0; t < Shape::PIECES; t++) {
+        const uint32_t e = tid + Shape::THREADS * t;
+        const uint32_t r = e / LPR4, f = e % LPR4;
+        const uint32_t j = min(c0 + r, last_key);
+        kp[t] = *reinterpret_cast<const float4 *>(p.k + (size_t)j * p.k_stride + 4u * f);
+        vp[t] = *reinterpret_cast<const float4 *>(p.v + (size_t)j * p.v_stride + 4u * f);
+    }
+#pragma unroll
+    for (int s = 0; s < QD; s++) asm volatile("" : "+v"(qa[s]), "+v"(qb[s]));
+    /* the pieces go to the lambda by value: indexed inside it, the arrays would live in scratch memory */
+    auto park = [&](const uint32_t pc, const float4 k_piece, const float4 v_piece) __attribute__((always_inline)) {
+        const uint32_t e = tid + Shape::THREADS * pc;
+        const uint32_t r = e / LPR4, f = e % LPR4;
+        if (r < kc) {
+            *reinterpret_cast<float4 *>(sm_k + r * ROW + 4u * f) = k_piece;
+            *reinterpret_cast<float4 *>(sm_v + r * ROW + 4u * f) = v_piece;
+        }
+    };
+#pragma unroll
+    for (int t = 0; t < Shape::PIECES; t++) park(t, kp[t], vp[t]);
+    __syncthreads(); /* the only one: from here on no wave waits for another */
+
+    const float scale2 = p.scale * LOG2E;
+    auto run_half = [&](const float (&qf)[QD], const uint32_t half) __attribute__((always_inline)) {
+        const uint32_t first = 16u * half;
+        const uint32_t row = first + c;
+        const bool live = row < p.nq;
+        uint32_t lo, hi;
+        fine_row_range(p, live ? row : p.nq - 1u, lo, hi);
+        if (!live) hi = lo;
+        /* key tiles of the half: [my0, my1) */
+        uint32_t lo_a, hi_a, all_lo, all_hi;
+        fine_span(p, first, min(first + 15u, p.nq - 1u), lo_a, hi_a, all_lo, all_hi);
+        (void)all_lo, (void)all_hi;
+        const uint32_t my0 = hi_a > lo_a ? lo_a / 16u : 0u, my1 = hi_a > lo_a ? (hi_a + 15u) / 16u : 0u;
+
+        floatx4 oacc[DT];
+#pragma unroll
+        for (int d = 0; d < DT; d++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) oacc[d][r] = 0.f;
+        float m = neg_inf(), l = 0.f;
+        /* key tiles two at a time on two running states, folded together at the end */
+        floatx4 oodd[DT];
+#pragma unroll
+        for (int d = 0; d < DT; d++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) oodd[d][r] = 0.f;
+        float modd = neg_inf(), lodd = 0.f;
+        const uint32_t vlen = hi > lo ? hi - lo : 0u;
+        uint32_t kt = my0;
+        for (; kt + 1u < my1; kt += 2u) {
+            const uint32_t k0 = kt * 16u;
+            const float *krow = sm_k + (k0 - c0 + c) * ROW + g * QD;
+            const float *vrow = sm_v + (k0 - c0 + 4u * g) * ROW + c;
+            fine_unit2<HD>(krow, vrow, krow + 16 * ROW, vrow + 16 * ROW, qf, oacc, m, l, oodd, modd, lodd,
+                           k0 + 4u * g - lo, k0 + 16u + 4u * g - lo, vlen, scale2);
+        }
+        if (kt < my1) {
+            const uint32_t k0 = kt * 16u;
+            const float *krow = sm_k + (k0 - c0 + c) * ROW + g * QD;
+            const float *vrow = sm_v + (k0 - c0 + 4u * g) * ROW + c;
+            fine_unit<HD>(krow, vrow, qf, oacc, m, l, k0 + 4u * g - lo, vlen, scale2);
+        }
+        fine_merge_states<DT>(oacc, m, l, oodd, modd, lodd);
+        /* the four lane groups of a column carry the same m, their sums add; lane (g, c) holds
+         * columns 16 d + 4 g + 0..3 of query row c */
+        l = swap32(swap16(l, OpSum()), OpSum());
+        if (!live) return;
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        float *orow = p.out + (size_t)row * p.out_stride + 4u * g;
+#pragma unroll
+        for (int d = 0; d < DT; d++)
+            *reinterpret_cast<float4 *>(orow + 16 * d) =
+                make_float4(oacc[d][0] * inv, oacc[d][1] * inv, oacc[d][2] * inv, oacc[d][3] * inv);
+        if (g == 0 && p.lse) {
+            p.lse[2 * (size_t)row + 0] = m * LN2; /* back to natural units */
+            p.lse[2 * (size_t)row + 1] = l;
+        }
+    };
+    if (ha != NONE) run_half(qa, ha);
+    if (hb != NONE) run_half(qb, hb);
 }
 
 /* keys per fill for a launch whose longest tile needs `span` keys */
@@ -461,6 +711,52 @@ void attn_fine_launch_single(const AttnProb &single, bool tall, hipStream_t s) {
     __builtin_memset(&a, 0, sizeof(a));
     a.first = single;
     fine_launch_hd<SRC_SINGLE>(nullptr, nullptr, ntiles, a, single.hd, attn_fine_span(single), tall, s);
+}
+
+/* the whole-problem kernel takes strided batches of problems like this one */
+bool attn_whole_can(const AttnProb &d) {
+    if (!attn_fine_can(d) || d.nq > WholeShape<64>::MAX_ROWS) return false;
+    /* keys the rows see, from the first row's first to the last row's last, in 16-key tiles */
+    uint64_t lo = 0, hi = d.nk;
+    if (d.vis == ATTN_VIS_CAUSAL) {
+        hi = std::min<uint64_t>(d.nk, (uint64_t)d.nq + d.causal_off);
+        if (d.window > 0 && (uint64_t)d.causal_off + 1u > d.window) lo = std::min<uint64_t>((uint64_t)d.causal_off + 1u - d.window, hi);
+    }
+    const uint64_t span = (hi + 15u) / 16u * 16u - lo / 16u * 16u;
+    return span <= attn_fine_fill_max(d.hd);
+}
+
+void attn_whole_launch_affine(const AttnAffine &aff, hipStream_t s) {
+    if (aff.count == 0) return;
+    const AttnProb &d = aff.first;
+    BLT_REQUIRE(attn_whole_can(d), "attention: internal: the whole-problem kernel was given a shape it does not take");
+    uint64_t lo = 0, hi = d.nk;
+    if (d.vis == ATTN_VIS_CAUSAL) {
+        hi = std::min<uint64_t>(d.nk, (uint64_t)d.nq + d.causal_off);
+        if (d.window > 0 && (uint64_t)d.causal_off + 1u > d.window) lo = std::min<uint64_t>((uint64_t)d.causal_off + 1u - d.window, hi);
+    }
+    const uint32_t kc = std::max<uint32_t>(16u, (uint32_t)((hi + 15u) / 16u * 16u - lo / 16u * 16u));
+    if (d.hd == 32u) {
+        const size_t lds = (size_t)2 * kc * WholeShape<32>::ROW * sizeof(float);
+        static const bool raised = [] {
+            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_whole_kernel<32>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          2 * (int)WholeShape<32>::KC_MAX * WholeShape<32>::ROW * (int)sizeof(float)));
+            return true;
+        }();
+        (void)raised;
+        blt_launch("attn_whole", attn_whole_kernel<32>, dim3(aff.count), dim3(256), lds, s, aff, kc);
+    } else {
+        const size_t lds = (size_t)2 * kc * WholeShape<64>::ROW * sizeof(float);
+        static const bool raised = [] {
+            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_whole_kernel<64>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          2 * (int)WholeShape<64>::KC_MAX * WholeShape<64>::ROW * (int)sizeof(float)));
+            return true;
+        }();
+        (void)raised;
+        blt_launch("attn_whole", attn_whole_kernel<64>, dim3(aff.count), dim3(256), lds, s, aff, kc);
+    }
 }
 
 void attn_fine_launch_affine(const AttnAffine &aff, bool tall, hipStream_t s) {

@@ -67,5 +67,8 @@ void attn_fine_launch(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t n
 /* tall: workgroups of one 16-row tile and sixteen waves instead of 32 rows and eight waves */
 void attn_fine_launch_single(const AttnProb &single, bool tall, hipStream_t s);
 void attn_fine_launch_affine(const AttnAffine &aff, bool tall, hipStream_t s);
+/* whole short problems of a strided batch, one workgroup each (attn_fine.hip) */
+bool attn_whole_can(const AttnProb &d);
+void attn_whole_launch_affine(const AttnAffine &aff, hipStream_t s);
 
 #endif

@@ -41,6 +41,9 @@ CASES = {
     "mixed_shapes": lambda: workloads.merged("mixed", [workloads.config1(batch=1, T=96, H=2, hd=32),
                                                        workloads.config1(batch=2, T=300, H=1, hd=32),
                                                        workloads.offset_causal(batch=1, nq=70, nk=200, H=3, hd=32)]),
+    # short problems with a sliding window, with and without an offset of the diagonal
+    "short_window": lambda: workloads.offset_causal(batch=2, nq=120, nk=120, H=2, hd=64, window=40),
+    "short_window_offset": lambda: workloads.offset_causal(batch=2, nq=90, nk=250, H=2, hd=32, window=70),
     # 512 problems of 64 rows: more 32-row (and 16-row) tiles than the chip holds at once, in a
     # multiple that lets resident workgroups walk them
     "c2_many": lambda: workloads.config2(batch=64, P=64, H=8, hd=64, T_bytes=256),
@@ -63,6 +66,7 @@ def main():
     import torch
     orc = binding.load_oracle()
     kernels = set()
+    launched = set()  # names of the kernels the plans launched
     for name, make in CASES.items():
         w = make()
         orunner.run(w, lib=orc)
@@ -87,8 +91,10 @@ def main():
                     arr = d.problems("descriptor", None, [t.data_ptr() for t in lse])
                     plan = d.lib.blt_attention_plan_create_hip(arr, len(w.heads))
                     kernels.add(d.lib.blt_attention_plan_kernel_hip(plan).decode())
+                    d.lib.blt_hip_profile_begin()
                     d.lib.blt_attention_plan_run_hip(plan)
                     d.lib.blt_backend_pass_sync_hip()
+                    launched.update(api.profile_end().keys())
                     d.lib.blt_attention_plan_destroy_hip(plan)
                     if name != "nonfinite_keys" and not name.endswith("_full") and name != "c2_many":
                         # the returned (max, sum) pairs rebuild the checker's weights
@@ -111,6 +117,7 @@ def main():
     print("case lse pairs, single-head calls", flush=True)
     lse_check.run_single_head_cases(api.load(), orc, api, abi, binding)
     print("KERNELS", ",".join(sorted(kernels)))
+    print("LAUNCHED", ",".join(sorted(launched)))
     print("OK")
 
 

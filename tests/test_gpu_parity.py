@@ -726,26 +726,31 @@ def test_kv_step_kernel_families_agree(kernel):
     assert p.returncode == 0 and "OK" in p.stdout, p.stdout[-2000:] + p.stderr[-2000:]
 
 
-@pytest.mark.parametrize("family", ["rows", "mfma", "wide", "fine", "fine16"])
+@pytest.mark.parametrize("family", ["rows", "mfma", "wide", "fine", "fine16", "fine128"])
 def test_attention_kernel_families(family):
     """Every attention kernel family on the same cases (causal, chunked prefill, sliding window,
     dense masks, lse output), pinned through BLT_HIP_ATTN_FAMILY in a fresh process; the fine
-    kernel in both workgroup shapes (BLT_HIP_FINE_ROWS: 32 rows and eight waves, 16 rows and
-    sixteen waves wherever the batch is strided)."""
+    kernel in its workgroup shapes (BLT_HIP_FINE_ROWS: 32 rows and eight waves, 16 rows and
+    sixteen waves wherever the batch is strided, whole problems of up to 128 rows on four waves
+    wherever the batch is strided and the keys fit one fill)."""
     import subprocess
     import sys
     import os
     here = os.path.dirname(os.path.abspath(__file__))
     env = dict(os.environ, BLT_HIP_ATTN_FAMILY=family)
+    shape = family
     if family.startswith("fine"):
         env["BLT_HIP_ATTN_FAMILY"] = "fine"
-        env["BLT_HIP_FINE_ROWS"] = "16" if family == "fine16" else "32"
+        env["BLT_HIP_FINE_ROWS"] = {"fine": "32", "fine16": "16", "fine128": "128"}[family]
         family = "fine"
     p = subprocess.run([sys.executable, "-u", os.path.join(here, "family_cases.py")], capture_output=True, text=True,
                        timeout=600, env=env)
     assert p.returncode == 0 and "OK" in p.stdout, p.stdout[-2000:] + p.stderr[-2000:]
     kernels = [ln for ln in p.stdout.splitlines() if ln.startswith("KERNELS")][0].split()[1]
     assert kernels == family, kernels
+    launched = [ln for ln in p.stdout.splitlines() if ln.startswith("LAUNCHED")][0].split()[1].split(",")
+    if family == "fine":
+        assert ("attn_whole" in launched) == (shape == "fine128"), launched
 
 
 @pytest.mark.parametrize("case", ["decode", "chunk5", "block16", "packed"])
