@@ -551,6 +551,7 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
                 "blt_kv_attend_step: buffers must be 16-byte aligned");
 
     StepArgs a;
+    a.by_length = 0; /* the block launcher decides */
     a.cache_k = cache->self_k;
     a.cache_v = cache->self_v;
     a.self_len = cache->self_len;

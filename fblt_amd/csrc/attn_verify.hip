@@ -355,7 +355,8 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
  * workgroup's per-split records. */
 template <int HD, int WAVES, int LPR, int ROWCAP>
 __device__ __forceinline__ void kv_merge_slices(const StepArgs &a, const float (*sm_o)[ROWCAP * LPR], uint32_t hshift,
-                                                uint32_t wave, uint32_t b, uint32_t split, size_t newrow0) {
+                                                uint32_t wave, uint32_t b, uint32_t split, size_t newrow0,
+                                                const uint32_t zblock) {
     static_assert(WAVES == 4 || WAVES == 8 || WAVES == 16, "slices map onto lane groups of a wave");
     constexpr int PR = HD + 2; /* a per-split record in global memory: HD columns, max, sum */
     constexpr uint32_t QUADS = HD / 4;
@@ -372,7 +373,7 @@ __device__ __forceinline__ void kv_merge_slices(const StepArgs &a, const float (
         const uint32_t quad = cc % QUADS;
         const uint32_t r = (cc / QUADS) % rows;
         const uint32_t hl = cc / (QUADS * rows);
-        const uint32_t hh = blockIdx.z * a.hpb + hl;
+        const uint32_t hh = zblock * a.hpb + hl;
         const float *ps = sm_o[(min(s, a.slices - 1u) << hshift) + hl] + r * LPR;
         const float2 ml = *reinterpret_cast<const float2 *>(ps + HD);
         const float4 o4 = *reinterpret_cast<const float4 *>(ps + 4u * quad);
@@ -442,13 +443,24 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
     __shared__ __attribute__((aligned(16))) float sm_o[WAVES][ROWS * LPR];
     __shared__ uint32_t sm_ticket;
 
-    const uint32_t b = blockIdx.y;
+    /* Which (sequence, head group) the workgroup takes.  Launches by length walk the pairs sequence
+     * by sequence, longest first, in the order workgroups are handed out (y before z): with more
+     * pairs than compute units the units that finish the shortest of the first round pick up the
+     * longest of the rest, so every unit ends up with about the same number of keys. */
+    uint32_t b = blockIdx.y, zblock = blockIdx.z;
+    if constexpr (KARG) {
+        if (a.by_length) {
+            const uint32_t at = blockIdx.y + gridDim.y * blockIdx.z;
+            zblock = at % gridDim.z;
+            b = lens.order[at / gridDim.z];
+        }
+    }
     const uint32_t split = blockIdx.x;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); /* uniform, and known to be */
     const uint32_t hshift = (uint32_t)__builtin_ctz(a.hpb);                 /* heads per workgroup: a power of two */
     const uint32_t slice = wave >> hshift;
-    const uint32_t head = blockIdx.z * a.hpb + (wave & (a.hpb - 1u));
+    const uint32_t head = zblock * a.hpb + (wave & (a.hpb - 1u));
     const bool head_ok = head < a.num_heads;
     const uint32_t hsafe = head_ok ? head : 0u;
     const uint32_t g = lane >> 4;
@@ -678,7 +690,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
     BLT_MARK(6);
     const uint32_t early_ticket = kv_draw_early_ticket(a, b); /* as in the 32-wide kernel */
 
-    kv_merge_slices<HD, WAVES, LPR, (int)ROWS>(a, sm_o, hshift, wave, b, split, newrow0);
+    kv_merge_slices<HD, WAVES, LPR, (int)ROWS>(a, sm_o, hshift, wave, b, split, newrow0, zblock);
     BLT_MARK(7);
 
     kv_finish_sequence<HD>(a, (uint32_t)SLOTS, b, nk, &sm_ticket, early_ticket);
@@ -949,7 +961,7 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
     __syncthreads();
     BLT_MARK(6);
     const uint32_t early_ticket = kv_draw_early_ticket(a, b);
-    kv_merge_slices<HD, WAVES, LPR, (int)ROWS>(a, sm_o, hshift, wave, b, split, newrow0);
+    kv_merge_slices<HD, WAVES, LPR, (int)ROWS>(a, sm_o, hshift, wave, b, split, newrow0, blockIdx.z);
     BLT_MARK(7);
     kv_finish_sequence<HD>(a, (uint32_t)SLOTS, b, nk, &sm_ticket, early_ticket);
 }
@@ -961,11 +973,35 @@ void launch_block_as(StepArgs a, uint32_t batch, const uint32_t *host_lens, hipS
     a.hpb = std::max(1u, std::min<uint32_t>(std::min<uint32_t>(a.hpb, a.num_heads), (uint32_t)WAVES));
     while (a.hpb & (a.hpb - 1u)) a.hpb &= a.hpb - 1u;
     const uint32_t subs = (a.span + 31u) / 32u;
+    /* Long sequences of unequal lengths, more (sequence, head) pairs than compute units, lengths
+     * known here: a launch of one workgroup per sequence and head pair ends with its longest
+     * sequence (2032 keys against a mean of 1528 is a quarter of the time lost), so the pairs
+     * become workgroups of their own, handed out longest first.  BLT_HIP_BLOCK_BY_LENGTH=0|1
+     * switches it off / on wherever it applies (tuning and test hook). */
+    KargLens lens;
+    a.by_length = 0;
+    if (NARROW && host_lens && a.splits == 1u && a.num_heads >= 2u && batch >= 2u) {
+        static const int pinned = [] {
+            const char *e = getenv("BLT_HIP_BLOCK_BY_LENGTH");
+            return e && *e ? atoi(e) : -1;
+        }();
+        uint32_t shortest = host_lens[0], longest = host_lens[0];
+        for (uint32_t b = 1; b < batch; b++)
+            shortest = std::min(shortest, host_lens[b]), longest = std::max(longest, host_lens[b]);
+        const bool pays = (uint64_t)batch * a.num_heads > 256u && subs >= 32u && (longest - shortest) * 5u >= longest;
+        if (pinned < 0 ? pays : pinned != 0) {
+            a.by_length = 1;
+            a.hpb = 1;
+            uint32_t idx[KARG_SEQS];
+            for (uint32_t b = 0; b < batch; b++) idx[b] = b;
+            std::stable_sort(idx, idx + batch, [&](uint32_t x, uint32_t y) { return host_lens[x] > host_lens[y]; });
+            for (uint32_t b = 0; b < batch; b++) lens.order[b] = (uint8_t)idx[b];
+        }
+    }
     a.slices = std::max(1u, std::min<uint32_t>((uint32_t)WAVES / a.hpb, subs));
     dim3 grid(a.splits, batch, (a.num_heads + a.hpb - 1) / a.hpb);
     const dim3 block(64 * a.hpb * a.slices);
     if (host_lens) {
-        KargLens lens;
         for (uint32_t b = 0; b < batch; b++) lens.v[b] = host_lens[b];
         if constexpr (NARROW) blt_launch("kv_block16_mfma", kv_block16_mfma_kernel<HD, WAVES, true>, grid, block, 0, s, a, lens);
         else blt_launch("kv_block_mfma", kv_block_mfma_kernel<HD, WAVES, true>, grid, block, 0, s, a, lens);

@@ -57,6 +57,8 @@ struct StepArgs {
     int block_kind;    /* every new row sees all keys */
     int write_through; /* this launch stores the new rows into the cache */
     int commit;        /* advance self_len when the sequence is done */
+    int by_length;     /* block step with the lengths in the arguments: workgroups take the (sequence, head
+                          group) pairs in the order of KargLens::order, longest sequences first */
 };
 
 
@@ -81,6 +83,7 @@ __device__ __forceinline__ void kv_fetch_arguments(const StepArgs &a) {
 constexpr int KARG_SEQS = 256;
 struct KargLens {
     uint32_t v[KARG_SEQS];
+    uint8_t order[KARG_SEQS]; /* by_length launches: the sequences of the launch, longest first */
 };
 struct DeviceLens {
     uint32_t unused;

@@ -460,6 +460,26 @@ def test_block_verify(B, batch, lens_mode, oracle, dev):
     assert_close(out, ref_out, "block verify B=%d" % B)
 
 
+@pytest.mark.parametrize("kind", ["block", "causal_chunk"])
+def test_block_step_long_unequal_sequences(kind, oracle, dev):
+    """More (sequence, head) pairs than compute units, prefixes of 300 ... 1100 keys, lengths on the
+    host: the block step hands the pairs out as workgroups of their own, longest sequence first
+    (blt_kv_attend_step_lens_hip).  Same results as the checker; the caches take the new rows bit
+    for bit; the device-length entry point, which cannot reorder, agrees."""
+    kw = workloads.config5(batch=72, B=16, len_lo=300, len_hi=1100, max_seq_len=1152)
+    if kind == "causal_chunk":
+        kw.kind = "causal"
+        kw.commit = True
+    ref_out, ref_k, ref_v = orunner.run_kv(kw, lib=oracle)
+    for lens_mode in ("host", "device"):
+        d = dev.DeviceKvWorkload(kw, lens=lens_mode)
+        d.run()
+        out, ck, cv, lens = d.results()
+        assert (lens == kw.lens.astype(np.int64) + (16 if kw.commit else 0)).all()
+        assert ck.tobytes() == ref_k.tobytes() and cv.tobytes() == ref_v.tobytes()
+        assert_close(out, ref_out, "block step by length, %s, %s lengths" % (kind, lens_mode))
+
+
 @pytest.mark.parametrize("B,nseq", [(4, 12), (8, 12), (16, 64)])
 def test_diffusion_self_attention_call_pattern(B, nseq, oracle, dev):
     """The reference's own route to config 5 (csrc/models/block_diffusion.c:196-204, 293-319): the whole
