@@ -1079,6 +1079,9 @@ def main():
         others["c5_B16_b128_L2048"], _ = bench_kv(bigv, 20, 3, warm_ms=100.0)
         others["c5_B16_b128_L2048"]["roofline_hbm"]["traffic"] = None
         log("c5_B16_b128_L2048", json.dumps(others["c5_B16_b128_L2048"]))
+        others["c5_B16_b128_L2048_host_lens"], _ = bench_kv(bigv, 20, 3, warm_ms=100.0, lens="host")
+        others["c5_B16_b128_L2048_host_lens"]["roofline_hbm"]["traffic"] = None
+        log("c5_B16_b128_L2048_host_lens", json.dumps(others["c5_B16_b128_L2048_host_lens"]))
 
     # the callers either side of the core: the whole attention block and its projection
     if want("block"):
@@ -1194,7 +1197,7 @@ def compact_line(head, others, cpu_head, K, W, detail_path):
     # the same kernels away from the launch floor: [kernel us, binding roofline, fraction of it]
     scaled = {k: [_sig(others[k]["kernel_us_avg"]), others[k]["roofline"]["bound"], _sig(others[k]["roofline"]["frac"])]
               for k in ("c1_x64", "c2_x8", "c1_T4096", "c2_P2048", "c4_b128_L2048", "c4_b128_L2048_host_lens",
-                        "c5_B16_b128_L2048") if k in others}
+                        "c5_B16_b128_L2048", "c5_B16_b128_L2048_host_lens") if k in others}
     # whole decoder step (all layers + LM head): [launches per step, device us, wall us]
     steps_ = {k: [others[k]["launches_per_step"], _sig(others[k]["kernel_us_avg"]), _sig(others[k]["us_per_step"])]
               for k in ("decode_step", "decode_step_b1", "draft_pass", "encoder") if k in others}
