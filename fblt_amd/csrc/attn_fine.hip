@@ -29,7 +29,9 @@
  *   O^T[d,   query] = sum_key V[key, d] P^T[key, query]   A = V^T, B = P^T
  *
  * register r of lane (g = lane / 16, c) of an accumulator is row 4 g + r,
- * column c.  The eight partial (max, sum, O) of a tile meet once in LDS.
+ * column c.  Row i of the e-th O^T tile stands for column (HD/16) i + e of the
+ * head, so that a lane's V operands of one key are consecutive floats in LDS.
+ * The eight partial (max, sum, O) of a tile meet once in LDS.
  *
  * A second shape of the same kernel serves launches with few, long problems (a
  * byte window of 512 rows over 4 heads: 64 tiles of 32 rows on 256 compute
@@ -109,8 +111,40 @@ __device__ __forceinline__ void fine_span(const AttnProb &p, uint32_t first, uin
     flo = lo_b, fhi = hi_a;
 }
 
+/* The V operands of one key for this lane: row i of tile e of O^T is column DT i + e of the head,
+ * so the lane's DT operands are consecutive floats, one 8- or 16-byte LDS read (vrow points at
+ * column DT c of the key's row). */
+template <int DT>
+__device__ __forceinline__ void fine_v_operands(const float *vrow, float (&vf)[DT][4], const int r) {
+    if constexpr (DT == 2) {
+        const float2 t = *reinterpret_cast<const float2 *>(vrow);
+        vf[0][r] = t.x, vf[1][r] = t.y;
+    } else {
+        static_assert(DT == 4, "head widths 32 and 64");
+        const float4 t = *reinterpret_cast<const float4 *>(vrow);
+        vf[0][r] = t.x, vf[1][r] = t.y, vf[2][r] = t.z, vf[3][r] = t.w;
+    }
+}
+
+/* The finished columns DT (4 g + r) + e of a query row, from accumulators oacc[e][r] scaled by f:
+ * the 4 DT consecutive floats from column 4 DT g on, written to dst (which points there). */
+template <int DT>
+__device__ __forceinline__ void fine_store_columns(float *dst, const floatx4 (&oacc)[DT], const float f) {
+    if constexpr (DT == 2) {
+#pragma unroll
+        for (int r = 0; r < 4; r += 2)
+            *reinterpret_cast<float4 *>(dst + 2 * r) =
+                make_float4(oacc[0][r] * f, oacc[1][r] * f, oacc[0][r + 1] * f, oacc[1][r + 1] * f);
+    } else {
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+            *reinterpret_cast<float4 *>(dst + 4 * r) =
+                make_float4(oacc[0][r] * f, oacc[1][r] * f, oacc[2][r] * f, oacc[3][r] * f);
+    }
+}
+
 /* One unit: 16 query rows (fragment qf, pre-loaded) against the 16 keys whose K rows start at
- * krow (this lane: row c, columns g*HD/4 ...) and whose V rows start at vrow (this lane: rows 4 g + r,
+ * krow (this lane: row c, columns g*HD/4 ...) and whose V rows start at vrow (this lane: rows 4 g + r, columns HD/16 c ...,
  * column c) in LDS, rows ROW = HD + 4 floats apart.  Register r of the lane's scores is key
  * 4 g + r of the tile; that key is visible iff rel + r < len (unsigned: rel = the key's offset
  * into the row's range).  Running maximum m (log2 units), sum l and O^T accumulators are updated. */
@@ -127,9 +161,7 @@ __device__ __forceinline__ void fine_unit(const float *krow, const float *vrow, 
     }
     float vf[DT][4];
 #pragma unroll
-    for (int r = 0; r < 4; r++)
-#pragma unroll
-        for (int d = 0; d < DT; d++) vf[d][r] = vrow[r * ROW + 16 * d];
+    for (int r = 0; r < 4; r++) fine_v_operands<DT>(vrow + r * ROW, vf, r);
 
     /* S^T on two accumulators: neither chain waits for its own previous result */
     floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
@@ -190,9 +222,10 @@ __device__ __forceinline__ void fine_unit2(const float *krow0, const float *vrow
     }
     float va[DT][4], vb[DT][4];
 #pragma unroll
-    for (int r = 0; r < 4; r++)
-#pragma unroll
-        for (int d = 0; d < DT; d++) va[d][r] = vrow0[r * ROW + 16 * d], vb[d][r] = vrow1[r * ROW + 16 * d];
+    for (int r = 0; r < 4; r++) {
+        fine_v_operands<DT>(vrow0 + r * ROW, va, r);
+        fine_v_operands<DT>(vrow1 + r * ROW, vb, r);
+    }
 
     floatx4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -404,7 +437,7 @@ __global__ __launch_bounds__(64 * WAVES, 4) void attn_fine_kernel(const AttnProb
             while (kt < my1 && kt * 16u < stage_end) {
                 const uint32_t k0 = kt * 16u;
                 const float *krow = sm_k + (k0 - c0 + c) * ROW + g * QD;
-                const float *vrow = sm_v + (k0 - c0 + 4u * g) * ROW + c;
+                const float *vrow = sm_v + (k0 - c0 + 4u * g) * ROW + DT * c;
                 const bool all_seen = k0 >= half_flo && k0 + 16u <= half_fhi; /* uniform over the wave */
                 fine_unit<HD>(krow, vrow, qf, oacc, m, l, k0 + 4u * g - (all_seen ? 0u : lo),
                               all_seen ? 0xFFFFFFFFu : (hi > lo ? hi - lo : 0u), scale2);
@@ -436,10 +469,7 @@ __global__ __launch_bounds__(64 * WAVES, 4) void attn_fine_kernel(const AttnProb
 
     /* ---- merge: every wave parks [16 queries][HD columns, max, sum] ---- */
     float *mine = sm + wave * (16 * ROW);
-#pragma unroll
-    for (int d = 0; d < DT; d++)
-        *reinterpret_cast<float4 *>(mine + c * ROW + 16 * d + 4 * g) =
-            make_float4(oacc[d][0], oacc[d][1], oacc[d][2], oacc[d][3]);
+    fine_store_columns<DT>(mine + c * ROW + 4 * DT * g, oacc, 1.0f);
     if (g == 0) *reinterpret_cast<float2 *>(mine + c * ROW + HD) = make_float2(m, l);
     __syncthreads();
 
@@ -603,27 +633,23 @@ __global__ __launch_bounds__(256, 2) void attn_whole_kernel(AttnAffine aff, uint
         for (; kt + 1u < my1; kt += 2u) {
             const uint32_t k0 = kt * 16u;
             const float *krow = sm_k + (k0 - c0 + c) * ROW + g * QD;
-            const float *vrow = sm_v + (k0 - c0 + 4u * g) * ROW + c;
+            const float *vrow = sm_v + (k0 - c0 + 4u * g) * ROW + DT * c;
             fine_unit2<HD>(krow, vrow, krow + 16 * ROW, vrow + 16 * ROW, qf, oacc, m, l, oodd, modd, lodd,
                            k0 + 4u * g - lo, k0 + 16u + 4u * g - lo, vlen, scale2);
         }
         if (kt < my1) {
             const uint32_t k0 = kt * 16u;
             const float *krow = sm_k + (k0 - c0 + c) * ROW + g * QD;
-            const float *vrow = sm_v + (k0 - c0 + 4u * g) * ROW + c;
+            const float *vrow = sm_v + (k0 - c0 + 4u * g) * ROW + DT * c;
             fine_unit<HD>(krow, vrow, qf, oacc, m, l, k0 + 4u * g - lo, vlen, scale2);
         }
         fine_merge_states<DT>(oacc, m, l, oodd, modd, lodd);
         /* the four lane groups of a column carry the same m, their sums add; lane (g, c) holds
-         * columns 16 d + 4 g + 0..3 of query row c */
+         * the HD/4 consecutive columns from (HD/4) g on of query row c */
         l = swap32(swap16(l, OpSum()), OpSum());
         if (!live) return;
         const float inv = l > 0.f ? 1.0f / l : 0.f;
-        float *orow = p.out + (size_t)row * p.out_stride + 4u * g;
-#pragma unroll
-        for (int d = 0; d < DT; d++)
-            *reinterpret_cast<float4 *>(orow + 16 * d) =
-                make_float4(oacc[d][0] * inv, oacc[d][1] * inv, oacc[d][2] * inv, oacc[d][3] * inv);
+        fine_store_columns<DT>(p.out + (size_t)row * p.out_stride + 4u * DT * g, oacc, inv);
         if (g == 0 && p.lse) {
             p.lse[2 * (size_t)row + 0] = m * LN2; /* back to natural units */
             p.lse[2 * (size_t)row + 1] = l;
