@@ -605,8 +605,13 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
      * waves of a workgroup slice one head's keys and meet once in LDS, nothing crosses workgroups
      * but the length ticket.  BLT_HIP_DECODE_ROW=0 keeps the split layout (tuning hook). */
     static const int row_env = env_int("BLT_HIP_DECODE_ROW", 1);
+    /* measured against the split layout at 32 / 64 / 128 sequences of 4 heads: ahead or level up to
+     * 8192 cached keys with up to 256 (sequence, head) pairs (21.2 against 24.2 us at 32 x 2048..4096,
+     * 35.5 against 39.4 at 64), with 512 pairs ahead at 2048 keys (33.2 against 39.2) and behind at
+     * 4096 (86.1 against 81.8) */
+    const size_t pairs = cache->batch * H;
     if (n_seq == 1 && span_env == 0 &&
-        (row_env == 2 || (row_env == 1 && subs >= 4 && subs <= 64 && cache->batch * H >= 128 && cache->batch * H <= 512))) {
+        (row_env == 2 || (row_env == 1 && subs >= 4 && pairs >= 128 && pairs <= 512 && subs <= (pairs <= 256 ? 256u : 96u)))) {
         a.splits = 1, a.span = 0, a.q0 = 0, a.write_through = 1, a.commit = commit;
         a.cap = (uint32_t)std::min<size_t>((size_t)cache->max_seq_len, rope_cos ? rope_positions : (size_t)UINT32_MAX);
         acquire_scratch(a, 0, cache->batch, static_scratch);

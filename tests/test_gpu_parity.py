@@ -411,6 +411,8 @@ def test_kv_decode_window(lens_mode, oracle, dev):
     (140, 1, 4, 1, 150, 5, False),
     (300, 1, 32, 1, 140, 0, True),     # host lengths: more sequences than one launch carries
     (130, 2, 32, 1000, 2040, 0, False),
+    (34, 4, 32, 2000, 4090, 0, False),  # long caches, 136 (sequence, head) pairs: still one workgroup per pair
+    (120, 4, 32, 1500, 2900, 600, True),
 ])
 def test_kv_single_row_steps(batch, H, hd, len_lo, len_hi, window, rope, lens_mode, oracle, dev):
     """One new row per sequence at batch sizes that give one workgroup per (sequence, head): every
