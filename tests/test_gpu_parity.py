@@ -775,6 +775,29 @@ def test_attention_kernel_families(family):
         assert ("attn_whole" in launched) == (shape == "fine128"), launched
 
 
+@pytest.mark.parametrize("family", ["auto", "rows", "mfma", "wide", "fine", "fine16", "fine128"])
+def test_attention_random_shapes(family):
+    """72 randomly shaped strided batches per routing (automatic, and every family / workgroup shape
+    pinned wherever the shape allows it) through the one-shot batch entry and a plan, against the
+    checker (tests/random_cases.py, fresh process: the routing hooks are read once)."""
+    import subprocess
+    import sys
+    import os
+    here = os.path.dirname(os.path.abspath(__file__))
+    env = dict(os.environ)
+    if family.startswith("fine"):
+        env["BLT_HIP_ATTN_FAMILY"] = "fine"
+        env["BLT_HIP_FINE_ROWS"] = {"fine": "32", "fine16": "16", "fine128": "128"}[family]
+    elif family != "auto":
+        env["BLT_HIP_ATTN_FAMILY"] = family
+    p = subprocess.run([sys.executable, "-u", os.path.join(here, "random_cases.py"), "11", "12", "13", "14", "15", "16"],
+                       capture_output=True, text=True, timeout=600, env=env)
+    assert p.returncode == 0 and "OK" in p.stdout, p.stdout[-2000:] + p.stderr[-2000:]
+    launched = [ln for ln in p.stdout.splitlines() if ln.startswith("LAUNCHED")][0].split()[1].split(",")
+    if family == "fine128":
+        assert "attn_whole" in launched, launched
+
+
 @pytest.mark.parametrize("case", ["decode", "chunk5", "block16", "packed"])
 def test_kv_rope_step(case, oracle, dev):
     """blt_kv_rope_attend_step_hip: rotation of the new Q/K rows fused into the step.  Rotated K rows
