@@ -99,7 +99,7 @@ struct LensArgOf<true> {
 template <bool KARG>
 using LensArg = typename LensArgOf<KARG>::type;
 
-__device__ __forceinline__ uint32_t kv_len_of(const StepArgs &a, const KargLens &lens, uint32_t b) { return lens.v[b]; }
+__device__ __forceinline__ uint32_t kv_len_of(const StepArgs &, const KargLens &lens, uint32_t b) { return lens.v[b]; }
 __device__ __forceinline__ uint32_t kv_len_of(const StepArgs &a, const DeviceLens &, uint32_t b) { return a.self_len[b]; }
 
 /* The lengths live in device memory and the launch was sized from a host-side hint.  A sequence
