@@ -100,6 +100,10 @@ def load_oracle():
     lib.orc_local_encoder_forward.restype = C.c_int
     lib.orc_local_encoder_forward.argtypes = [C.POINTER(abi.BltLocalEncoder), _u8, C.c_size_t,
                                               C.POINTER(abi.BltPatchInfo), C.c_size_t, abi.c_size_p, C.c_size_t, _fp, _fp]
+    lib.orc_local_decoder_forward.restype = C.c_int
+    lib.orc_local_decoder_forward.argtypes = [C.POINTER(abi.BltLocalDecoder), _fp, C.c_size_t, _fp,
+                                              C.POINTER(abi.BltPatchInfo), C.c_size_t, abi.c_size_p, C.c_size_t, C.c_int,
+                                              _fp]
     lib.orc_transformer_forward.restype = C.c_int
     lib.orc_transformer_forward.argtypes = [_fp] * 9 + [C.c_size_t] * 4 + [C.c_int, C.c_int, C.c_float, _fp, _fp,
                                                                          C.POINTER(abi.BltMaskConfig)]
@@ -233,6 +237,8 @@ def load_ref():
                                                                   C.POINTER(abi.BltArena)]
     if hasattr(lib, "blt_local_encoder_forward"):   # csrc/models/local_encoder.h:71-73
         _encoder_entry(lib)
+    if hasattr(lib, "blt_model_encode"):
+        _model_entry(lib)
         lib.blt_indexed_row_accumulate.restype = None
         lib.blt_indexed_row_accumulate.argtypes = [T, C.POINTER(C.c_uint32), T]
         lib.blt_scale.restype = None
@@ -286,6 +292,39 @@ class BltGlobalTransformer(C.Structure):
     _fields_ = [("config", BltGlobalTransformerConfig), ("stack", BltTransformerStack)]
 
 
+class BltModelConfig(C.Structure):
+    """csrc/models/model.h:16-20"""
+    _fields_ = [("encoder_config", abi.BltLocalEncoderConfig), ("global_config", BltGlobalTransformerConfig),
+                ("decoder_config", abi.BltLocalDecoderConfig)]
+
+
+class BltModel(C.Structure):
+    """csrc/models/model.h:22-27"""
+    _fields_ = [("config", BltModelConfig), ("encoder", C.POINTER(abi.BltLocalEncoder)),
+                ("global_", C.POINTER(BltGlobalTransformer)), ("decoder", C.POINTER(abi.BltLocalDecoder))]
+
+
+class BltModelEncOut(C.Structure):
+    """csrc/models/model.h:42-47"""
+    _fields_ = [("patch_out", abi.BltTensor), ("global_out", abi.BltTensor), ("byte_hidden_out", abi.BltTensor),
+                ("patch_doc_boundaries", abi.c_size_p)]
+
+
+def _model_entry(lib):
+    """The two stages of the model's inference forward, blt_model_encode and blt_model_decode
+    (csrc/models/model.c:68-131; blt_model_forward itself always asks for the loss), and the patch
+    transformer's constructor."""
+    T, A = C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)
+    lib.blt_global_transformer_create.restype = C.POINTER(BltGlobalTransformer)
+    lib.blt_global_transformer_create.argtypes = [A, C.POINTER(BltGlobalTransformerConfig)]
+    lib.blt_model_encode.restype = None
+    lib.blt_model_encode.argtypes = [C.POINTER(BltModel), T, C.POINTER(abi.BltPatchInfo), C.c_size_t, abi.c_size_p,
+                                     C.c_size_t, C.POINTER(BltModelEncOut), A]
+    lib.blt_model_decode.restype = None
+    lib.blt_model_decode.argtypes = [C.POINTER(BltModel), C.POINTER(BltModelEncOut), C.POINTER(abi.BltPatchInfo),
+                                     C.c_size_t, T, T, abi.c_size_p, C.c_size_t, C.c_void_p, T, T, A]
+
+
 def load_ref_stack_callers():
     """The reference's transformer_stack.c and global_transformer.c, compiled unmodified and linked
     against the HIP library without the reference's transformer.c, so that every layer of the
@@ -302,6 +341,8 @@ def load_ref_stack_callers():
     lib.blt_global_transformer_forward.argtypes = [C.POINTER(BltGlobalTransformer), T, abi.c_size_p, C.c_size_t, T, A]
     if hasattr(lib, "blt_local_encoder_forward"):
         _encoder_entry(lib)
+    if hasattr(lib, "blt_model_encode"):
+        _model_entry(lib)
     return lib
 
 

@@ -776,6 +776,73 @@ static int orc_block_d0_rows(const blt_local_decoder *dec, const blt_block_batch
     return ORC_OK;
 }
 
+
+/* csrc/models/local_decoder.c:233-351 with d0_opts == NULL and loss_out == NULL: D_0 is the encoder's
+ * byte states; per layer the cross block where it fires -- queries RMSNorm(D), keys and values the
+ * k sub-tokens of every patch, byte i reading the latent blt_patch_decoder_latent_at assigns it
+ * (:75-88), the last byte its own patch when trailing_closed -- then the byte transformer block
+ * under the causal / window / document mask (:96-102); logits = D_L * lm_head (:340).
+ * doc_boundaries in the mask builder's convention (entry d starts document d + 1). */
+int orc_local_decoder_forward(const blt_local_decoder *dec, const float *byte_hidden, size_t seq_len,
+                              const float *patch_in, const blt_patch_info *patches, size_t num_patches,
+                              const size_t *doc_boundaries, size_t num_docs, int trailing_closed, float *logits_out) {
+    const blt_local_decoder_config *cfg = &dec->config;
+    const size_t E = cfg->embed_dim, V = cfg->vocab_size, L = cfg->num_layers;
+    const size_t pdim = cfg->patch_dim ? cfg->patch_dim : E, k = pdim / E;
+    if (seq_len < 2 || seq_len > cfg->max_seq_len || num_patches < 1 || k < 1 || pdim % E != 0) return ORC_ERR_ARG;
+
+    size_t *q_ids = (size_t *)malloc(seq_len * sizeof(size_t));
+    size_t *kv_ids = (size_t *)malloc(num_patches * k * sizeof(size_t));
+    for (size_t i = 0; i < seq_len; i++) q_ids[i] = orc_patch_decoder_latent_at(patches, num_patches, i);
+    if (trailing_closed) q_ids[seq_len - 1] = num_patches - 1;
+    for (size_t p = 0; p < num_patches; p++)
+        for (size_t s2 = 0; s2 < k; s2++) kv_ids[p * k + s2] = p;
+
+    blt_mask_config local, cross;
+    memset(&local, 0, sizeof(local));
+    memset(&cross, 0, sizeof(cross));
+    local.seq_len_q = local.seq_len_kv = seq_len;
+    local.sliding_window = cfg->local_window;
+    local.doc_boundaries = doc_boundaries, local.num_docs = num_docs;
+    local.is_causal = true;
+    cross.seq_len_q = seq_len, cross.seq_len_kv = num_patches * k;
+    cross.query_group_ids = q_ids, cross.kv_group_ids = kv_ids;
+    cross.bidirectional_within_group = true;
+
+    float *cur = (float *)malloc(seq_len * E * sizeof(float));
+    float *next = (float *)malloc(seq_len * E * sizeof(float));
+    float *normed = (float *)malloc(seq_len * E * sizeof(float));
+    float *tmp = (float *)malloc(seq_len * E * sizeof(float));
+    float *mid = (float *)malloc(seq_len * E * sizeof(float));
+    memcpy(cur, byte_hidden, seq_len * E * sizeof(float));
+    int rc = ORC_OK;
+    for (size_t l = 0; l < L && rc == ORC_OK; l++) {
+        const blt_local_layer_storage *s = &dec->layers[l];
+        const float *b_in = cur;
+        if (orc_local_cross_attn_fires(cfg->cross_attn_placement, cfg->cross_attn_all_layers, L, l)) {
+            orc_rmsnorm_forward(cur, (const float *)s->cross_norm_weight.data, normed, seq_len, E);
+            rc = orc_cross_attention_forward(normed, patch_in, (const float *)s->cross_weight_q.data,
+                                             (const float *)s->cross_weight_k.data, (const float *)s->cross_weight_v.data,
+                                             (const float *)s->cross_weight_proj.data, tmp, seq_len, num_patches * k, E,
+                                             cfg->cross_attn_heads, &cross);
+            if (rc != ORC_OK) break;
+            orc_add(cur, tmp, mid, seq_len * E);
+            b_in = mid;
+        }
+        rc = orc_transformer_forward(b_in, (const float *)s->norm1_weight.data, (const float *)s->attn_qkv_w.data,
+                                     (const float *)s->attn_proj_w.data, (const float *)s->norm2_weight.data,
+                                     (const float *)s->ffn_up_w.data, (const float *)s->ffn_gate_w.data,
+                                     (const float *)s->ffn_down_w.data, next, seq_len, E, s->ffn_up_w.shape[1],
+                                     cfg->num_heads, 1, 1, cfg->rope_theta, (const float *)dec->rope_cos_cache.data,
+                                     (const float *)dec->rope_sin_cache.data, &local);
+        float *t = cur;
+        cur = next, next = t;
+    }
+    if (rc == ORC_OK) orc_matmul(cur, (const float *)dec->lm_head_weight.data, logits_out, seq_len, E, V);
+    free(q_ids), free(kv_ids), free(cur), free(next), free(normed), free(tmp), free(mid);
+    return rc;
+}
+
 /* csrc/models/block_diffusion.c:776-795: the inference-mode forward over [clean prefix ; block
  * rows] as the reference computes it -- all S = N + R rows densely: context 110-204 (D_0, gathered
  * rotary rows, group ids, the S x S INFER mask), layers 336-398 (cross block where it fires,

@@ -66,6 +66,10 @@
  *   orc_rmsnorm_forward, orc_add, orc_swiglu_forward, orc_kv_decode_layer, orc_transformer_forward
  *       bit-for-bit against oracle/_ref (blt_rmsnorm_forward, blt_add, blt_swiglu_forward,
  *       blt_transformer_forward); RMSNorm of a constant row = +-weight, silu(0) = 0, float64.
+ *   orc_local_decoder_forward
+ *       bit-for-bit against oracle/_ref's blt_local_decoder_forward_ext (window, documents,
+ *       sub-token split, trailing_closed) and against the incremental decoder step over the same
+ *       rows; with the encoder and the block restatement, the whole blt_model_forward.
  *   orc_local_decoder_forward_diffusion_infer, orc_kv_block_step, orc_kv_*_step_kind
  *       bit-for-bit against oracle/_ref's blt_local_decoder_forward_diffusion_infer over D_0
  *       modes, sub-token split, window, placements and block geometry; the cached form (prefix as
@@ -283,6 +287,11 @@ int orc_local_decoder_forward_diffusion_infer(const blt_local_decoder *dec, cons
  * = num_clean rows, tier 2 refreshed); logits_out [n_block_rows, vocab]; nothing is committed. */
 int orc_kv_block_step(blt_kv_cache *cache, size_t b, size_t base, size_t num_patches, const blt_block_batch *batch,
                       int d0_mode, float *logits_out);
+
+/* models/local_decoder.c:233-351 without D_0 options and without the loss: logits [seq_len, vocab]. */
+int orc_local_decoder_forward(const blt_local_decoder *dec, const float *byte_hidden, size_t seq_len,
+                              const float *patch_in, const blt_patch_info *patches, size_t num_patches,
+                              const size_t *doc_boundaries, size_t num_docs, int trailing_closed, float *logits_out);
 
 /* models/transformer.c:97-128, RMSNorm + SwiGLU block */
 int orc_transformer_forward(const float *input, const float *norm1_w, const float *qkv_w, const float *proj_w,

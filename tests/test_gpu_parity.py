@@ -1744,3 +1744,31 @@ def test_local_encoder_forward(name, impl, oracle, dev):
     assert_close(got_h, want_h, name + " byte_hidden_out")
     assert_close(got_p, want_p, name + " patch_out")
 
+
+
+@pytest.mark.parametrize("name", ["model_T96", "model_T200_docs_window"])
+def test_model_forward_on_the_library(name, oracle, dev):
+    """The reference's whole-model inference forward -- blt_model_encode + blt_model_decode of
+    csrc/models/model.c:68-131 over its local_encoder.c, global_transformer.c / transformer_stack.c
+    and local_decoder.c, all compiled unmodified -- on device tensors, with this library's ops and
+    fused blocks under them (blt_transformer_forward, blt_cross_attention_forward, the embedding,
+    n-gram, pooling, norm, add and product twins, the mask builders and the memory shim): logits
+    against the composition of the restated stages, which tests/test_oracle_vs_ref.py pins bit for
+    bit against the reference's CPU build."""
+    from fblt_amd import decoder
+    from tests import model_runs
+    lib = api.load()
+    stack_lib = binding.load_ref_stack_callers()
+    if stack_lib is None or not hasattr(stack_lib, "blt_model_encode"):
+        pytest.skip("oracle/_ref/libblt_ref_stack_callers.so was not built with the model driver (needs the reference sources)")
+    args = model_runs.inputs(name)
+
+    def fill(t, arr):
+        assert tuple(t.contents.shape[:t.contents.ndim]) == arr.shape
+        lib.blt_tensor_upload(t, arr.ctypes.data, arr.nbytes)
+
+    got = model_runs.run(stack_lib, lib, oracle, abi.BLT_BACKEND_HIP, decoder.device_place, fill,
+                         lib.blt_backend_pass_sync_hip, *args)
+    want = model_runs.run_oracle(oracle, *args)
+    assert np.abs(want).max() > 1e-3
+    assert_close(got, want, name + " logits")

@@ -694,3 +694,61 @@ def test_local_encoder_bit_exact(shape, oracle, ref):
         assert np.isfinite(b).all() and np.abs(b).sum() > 0
         assert a.tobytes() == b.tobytes(), shape
 
+
+
+# ---------------------------------------------------------------------------
+# the plain decoder forward and the whole-model forward (csrc/models/local_decoder.c:233-351,
+# csrc/models/model.c:68-144)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("case", range(len(DECODER_CASES)))
+@pytest.mark.parametrize("closed,docs", [(0, []), (1, []), (0, [5, 11])])
+def test_local_decoder_forward_bit_exact(case, closed, docs, oracle, ref):
+    """orc_local_decoder_forward against blt_local_decoder_forward_ext of the reference build: every
+    decoder configuration of this file (sub-token split, window, placements), trailing_closed, and
+    document boundaries in the byte mask."""
+    from fblt_amd import decoder
+    c = DECODER_CASES[case]
+    CPU = abi.BLT_BACKEND_CPU
+    bound = _host_decoder(oracle, c, 900 + case)
+    rs = np.random.RandomState(900 + case)
+    lengths = [3, 4, 2, 5, 1, 6]
+    T, P, E, V = sum(lengths), len(lengths), c["E"], c["V"]
+    patches = decoder.patch_table(lengths)
+    pdim = c["E"] * c["k"]
+    hidden = rs.randn(T, E).astype(np.float32)
+    patch_in = rs.randn(P, pdim).astype(np.float32)
+    bounds = abi.size_array(docs) if docs else None
+    num_docs = len(docs) + 1 if docs else 0
+    want, got = np.zeros((T, V), dtype=np.float32), np.zeros((T, V), dtype=np.float32)
+    th, tp = abi.tensor_view(hidden.ctypes.data, hidden.shape, CPU), abi.tensor_view(patch_in.ctypes.data, patch_in.shape, CPU)
+    tl = abi.tensor_view(want.ctypes.data, want.shape, CPU)
+    arena = ref.blt_arena_create(64 << 20, CPU)
+    try:
+        ref.blt_local_decoder_forward_ext(bound.ptr, C.byref(th), C.byref(tp), patches, P, None, None, bounds, num_docs,
+                                          None, closed, C.byref(tl), None, arena)
+    finally:
+        ref.blt_arena_destroy(arena)
+    assert oracle.orc_local_decoder_forward(bound.ptr, binding.fptr(hidden.reshape(-1)), T,
+                                            binding.fptr(patch_in.reshape(-1)), patches, P, bounds, num_docs, closed,
+                                            binding.fptr(got.reshape(-1))) == 0
+    assert got.tobytes() == want.tobytes()
+
+
+@pytest.mark.parametrize("name", ["model_T96", "model_T200_docs_window"])
+def test_model_forward_bit_exact(name, oracle, ref):
+    """blt_model_encode + blt_model_decode of the reference build (encoder, patch transformer,
+    decoder, LM head; the inference forward without the loss) against the composition of the
+    restated stages: logits bit for bit."""
+    from fblt_amd import decoder
+    from tests import model_runs
+    if not hasattr(ref, "blt_model_encode"):
+        pytest.skip("oracle/_ref/libblt_ref.so predates the model driver: rebuild it (make -C oracle ref)")
+    args = model_runs.inputs(name)
+
+    def fill(t, arr):
+        C.memmove(t.contents.data, arr.ctypes.data, arr.nbytes)
+
+    want = model_runs.run(ref, ref, oracle, abi.BLT_BACKEND_CPU, decoder.host_place, fill, lambda: None, *args)
+    got = model_runs.run_oracle(oracle, *args)
+    assert np.isfinite(want).all() and np.abs(want).max() > 1e-3
+    assert got.tobytes() == want.tobytes()
