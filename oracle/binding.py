@@ -28,7 +28,7 @@ def build(ref=True):
     if ref and os.path.isdir(os.environ.get("REF_ROOT", "/root/reference")):
         subprocess.check_call(["make", "-s", "-B", "-C", HERE, "ref"])
         if os.path.exists(os.path.join(HERE, "..", "fblt_amd", "lib", "libfblt_hip.so")):
-            subprocess.check_call(["make", "-s", "-C", HERE, "callers", "stack_callers"])
+            subprocess.check_call(["make", "-s", "-C", HERE, "callers", "stack_callers", "model_callers"])
 
 
 def load_oracle():
@@ -343,6 +343,22 @@ def load_ref_stack_callers():
         _encoder_entry(lib)
     if hasattr(lib, "blt_model_encode"):
         _model_entry(lib)
+    return lib
+
+
+MODEL_CALLERS_SO = os.path.join(HERE, "_ref", "libblt_ref_model_callers.so")
+
+
+def load_ref_model_callers():
+    """The reference's whole-model driver, patch transformer and local decoder, compiled unmodified
+    and linked against the HIP library WITHOUT the reference's encoder sources, so that
+    blt_model_encode runs the library's own blt_local_encoder_forward (`make -C oracle
+    model_callers`); None where that was never built."""
+    if not os.path.exists(MODEL_CALLERS_SO) or not os.path.exists(REF_SO):
+        return None
+    load_ref()
+    lib = C.CDLL(MODEL_CALLERS_SO)
+    _model_entry(lib)
     return lib
 
 

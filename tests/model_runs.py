@@ -12,7 +12,7 @@ from tests import encoder_runs
 
 GLOBAL_ORDER = ("norm1_weight", "attn_qkv_w", "attn_proj_w", "norm2_weight", "ffn_up_w", "ffn_gate_w", "ffn_down_w")
 
-# embed_dim shared by the three stages (csrc/models/model.c:37-39); the encoder case dictionary of
+# embed_dim shared by the three stages and patch_dim == embed_dim (csrc/models/model.c:37-39, 80-86); the encoder case dictionary of
 # tests/golden/block_cases.py plus the patch transformer's and the decoder's own sizes
 CASES = {
     "model_T96": dict(T=96, E=64, H=2, XH=2, hidden=96, L=2, k=1, ngrams=[3, 4], vocab=257, normalize=True, window=0,

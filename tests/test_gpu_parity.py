@@ -1746,21 +1746,24 @@ def test_local_encoder_forward(name, impl, oracle, dev):
 
 
 
+@pytest.mark.parametrize("driver", ["reference_encoder", "library_encoder"])
 @pytest.mark.parametrize("name", ["model_T96", "model_T200_docs_window"])
-def test_model_forward_on_the_library(name, oracle, dev):
+def test_model_forward_on_the_library(name, driver, oracle, dev):
     """The reference's whole-model inference forward -- blt_model_encode + blt_model_decode of
     csrc/models/model.c:68-131 over its local_encoder.c, global_transformer.c / transformer_stack.c
     and local_decoder.c, all compiled unmodified -- on device tensors, with this library's ops and
     fused blocks under them (blt_transformer_forward, blt_cross_attention_forward, the embedding,
     n-gram, pooling, norm, add and product twins, the mask builders and the memory shim): logits
     against the composition of the restated stages, which tests/test_oracle_vs_ref.py pins bit for
-    bit against the reference's CPU build."""
+    bit against the reference's CPU build.  `library_encoder`: the same driver built without the
+    reference's encoder sources, so that blt_model_encode runs this library's own
+    blt_local_encoder_forward."""
     from fblt_amd import decoder
     from tests import model_runs
     lib = api.load()
-    stack_lib = binding.load_ref_stack_callers()
+    stack_lib = binding.load_ref_stack_callers() if driver == "reference_encoder" else binding.load_ref_model_callers()
     if stack_lib is None or not hasattr(stack_lib, "blt_model_encode"):
-        pytest.skip("oracle/_ref/libblt_ref_stack_callers.so was not built with the model driver (needs the reference sources)")
+        pytest.skip("oracle/_ref does not hold the model driver build (needs the reference sources)")
     args = model_runs.inputs(name)
 
     def fill(t, arr):
