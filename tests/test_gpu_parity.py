@@ -413,6 +413,7 @@ def test_kv_decode_window(lens_mode, oracle, dev):
     (130, 2, 32, 1000, 2040, 0, False),
     (34, 4, 32, 2000, 4090, 0, False),  # long caches, 136 (sequence, head) pairs: still one workgroup per pair
     (120, 4, 32, 1500, 2900, 600, True),
+    (32, 4, 32, 6000, 8180, 0, False),   # the longest caches the single-row kernel is routed
 ])
 def test_kv_single_row_steps(batch, H, hd, len_lo, len_hi, window, rope, lens_mode, oracle, dev):
     """One new row per sequence at batch sizes that give one workgroup per (sequence, head): every
