@@ -78,6 +78,7 @@ SYMBOLS = {
     "blt_arena_destroy": (None, [C.POINTER(abi.BltArena)]),
     "blt_arena_reset": (None, [C.POINTER(abi.BltArena)]),
     "blt_arena_alloc": (C.c_void_p, [C.POINTER(abi.BltArena), C.c_size_t, C.c_size_t]),
+    "blt_container_alloc": (C.c_void_p, [C.POINTER(abi.BltArena), C.c_size_t]),
     "blt_tensor_create": (abi.BltTensor, [C.POINTER(abi.BltArena), C.POINTER(C.c_size_t), C.c_size_t, C.c_int]),
     "blt_tensor_create_uninit": (abi.BltTensor, [C.POINTER(abi.BltArena), C.POINTER(C.c_size_t), C.c_size_t,
                                                  C.c_int]),

@@ -29,7 +29,7 @@ INCLUDES = ["-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
 # -packed-fp32-ops off: hipcc must not form packed fp32 instructions on this pool
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"] + INCLUDES
-C_FLAGS = ["-std=c99", "-O2", "-fPIC", "-Wall", "-Wextra", "-D_POSIX_C_SOURCE=200809L"] + INCLUDES
+C_FLAGS = ["-std=c99", "-O2", "-fPIC", "-Wall", "-Wextra", "-Werror=implicit-function-declaration", "-D_POSIX_C_SOURCE=200809L"] + INCLUDES
 
 
 def _run(cmd):

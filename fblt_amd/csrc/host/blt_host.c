@@ -10,6 +10,7 @@
 #include "blt_fatal.h"
 
 #include <math.h>
+#include <pthread.h>
 #include <stdlib.h>
 #include <string.h>
 
@@ -48,15 +49,53 @@ blt_arena *blt_arena_create(size_t capacity_bytes, blt_backend backend) {
     return a;
 }
 
+/* Host blocks handed out by blt_container_alloc() for device arenas, newest first. */
+typedef struct host_block {
+    struct host_block *next;
+    const blt_arena *arena;
+    size_t at; /* the arena's offset when the block was handed out */
+} host_block;
+#define HOST_BLOCK_HEADER 64 /* keeps the payload 64-byte aligned, as arena containers are */
+
+static host_block *g_host_blocks = NULL;
+static pthread_mutex_t g_host_blocks_lock = PTHREAD_MUTEX_INITIALIZER;
+
+/* Frees the arena's host blocks that were handed out above `keep_to` (all of them for 0 with
+ * `all` set).  Caller holds the lock. */
+static void host_blocks_release(const blt_arena *a, size_t keep_to, int all) {
+    host_block **link = &g_host_blocks;
+    while (*link) {
+        host_block *b = *link;
+        if (b->arena == a && (all || b->at > keep_to)) {
+            *link = b->next;
+            free(b);
+        } else {
+            link = &b->next;
+        }
+    }
+}
+
 void blt_arena_destroy(blt_arena *a) {
     if (!a) return;
-    if (a->backend == BLT_BACKEND_HIP) blt_hip_free(a->buffer);
-    else free(a->buffer);
+    if (a->backend == BLT_BACKEND_HIP) {
+        pthread_mutex_lock(&g_host_blocks_lock);
+        host_blocks_release(a, 0, 1);
+        pthread_mutex_unlock(&g_host_blocks_lock);
+        blt_hip_free(a->buffer);
+    } else {
+        free(a->buffer);
+    }
     free(a);
 }
 
 void blt_arena_reset(blt_arena *a) {
-    if (a) a->offset = 0;
+    if (!a) return;
+    a->offset = 0;
+    if (a->backend == BLT_BACKEND_HIP) {
+        pthread_mutex_lock(&g_host_blocks_lock);
+        host_blocks_release(a, 0, 1);
+        pthread_mutex_unlock(&g_host_blocks_lock);
+    }
 }
 
 void *blt_arena_alloc(blt_arena *a, size_t bytes, size_t alignment) {
@@ -68,6 +107,33 @@ void *blt_arena_alloc(blt_arena *a, size_t bytes, size_t alignment) {
                   a->offset, a->capacity);
     a->offset = at + bytes;
     return (char *)a->buffer + at;
+}
+
+/* Containers are what callers fill and read on the host: group-id arrays, weight-view structs,
+ * model structs (csrc/models/local_decoder.c:76-80, transformer_stack.c:85).  On the CPU backend
+ * they live in the arena (csrc/core/tensor.c:154); for a device arena the reference hands out
+ * zeroed host memory instead (tensor.c:156-162, backend.c:494-501) and never releases it.  Here a
+ * block belongs to its arena: it is released when the arena is reset or destroyed, or once the
+ * caller has rewound the arena's offset below the point the block was handed out at
+ * (csrc/infer/self_speculation.c:359-401 rewinds that way), which is when a container of the CPU
+ * backend would be dead too. */
+void *blt_container_alloc(blt_arena *a, size_t bytes) {
+    if (!a || !a->buffer) BLT_FATAL("invalid arena");
+    if (a->backend != BLT_BACKEND_HIP) return blt_arena_alloc(a, bytes, 64);
+    BLT_REQUIRE(bytes <= (size_t)-1 - HOST_BLOCK_HEADER, "blt_container_alloc: size overflows");
+    void *raw = NULL;
+    if (posix_memalign(&raw, 64, HOST_BLOCK_HEADER + bytes) != 0) raw = NULL;
+    BLT_REQUIRE(raw != NULL, "blt_container_alloc: host allocation failed");
+    host_block *b = (host_block *)raw;
+    memset(b, 0, HOST_BLOCK_HEADER + bytes);
+    b->arena = a;
+    b->at = a->offset;
+    pthread_mutex_lock(&g_host_blocks_lock);
+    host_blocks_release(a, a->offset, 0);
+    b->next = g_host_blocks;
+    g_host_blocks = b;
+    pthread_mutex_unlock(&g_host_blocks_lock);
+    return (char *)b + HOST_BLOCK_HEADER;
 }
 
 static blt_tensor tensor_make(blt_arena *arena, const size_t *shape, size_t ndim, blt_dtype dtype, int clear) {

@@ -39,7 +39,7 @@ def test_library_exports_every_declared_symbol():
 OFF_PATH = {"blt_attention_head_core_backward", "blt_matmul_backward", "blt_rmsnorm_backward",
             "blt_rmsnorm_backward_add", "blt_rope_apply_packed_backward", "blt_swiglu_backward",
             "blt_cross_entropy_forward", "blt_cross_entropy_backward", "blt_gelu_forward",
-            "blt_layernorm_forward", "blt_cast", "blt_container_alloc", "blt_tensor_view_2d", "blt_tensor_view_3d",
+            "blt_layernorm_forward", "blt_cast", "blt_tensor_view_2d", "blt_tensor_view_3d",
             # training side of csrc/models/block_diffusion.c (D_0 table gradient)
             "blt_indexed_row_scatter_add"}
 # the same for the layer stack, patch transformer and local encoder (csrc/models/transformer_stack.c,
@@ -304,6 +304,34 @@ def test_host_arena_and_tensor():
     lib.blt_arena_reset(arena)
     assert arena.contents.offset == 0
     lib.blt_arena_destroy(arena)
+
+
+def test_containers_are_host_memory_for_a_device_arena():
+    """blt_container_alloc (csrc/core/tensor.c:154-162): arena memory on the CPU backend; for a device arena zeroed,
+    64-byte aligned host memory that leaves the arena's offset alone, released with the arena's reset.  The device
+    arena here is a hand-made struct whose buffer is never touched, so this runs without a GPU."""
+    lib = api.load()
+    host = lib.blt_arena_create(4096, abi.BLT_BACKEND_CPU)
+    p = lib.blt_container_alloc(host, 100)
+    assert p % 64 == 0 and host.contents.buffer <= p < host.contents.buffer + 4096 and host.contents.offset >= 100
+    lib.blt_arena_destroy(host)
+
+    dev = abi.BltArena()
+    dev.buffer, dev.capacity, dev.offset, dev.backend = 0x10000, 1 << 20, 0, abi.BLT_BACKEND_HIP
+    blocks = []
+    for at, size in ((0, 100), (512, 8), (512, 4000), (256, 64), (256, 1)):  # the fourth follows a rewind
+        dev.offset = at
+        q = lib.blt_container_alloc(C.byref(dev), size)
+        assert q % 64 == 0 and dev.offset == at
+        view = (C.c_ubyte * size).from_address(q)
+        assert not any(view)
+        for i in range(size):
+            view[i] = 0xA5  # host-writable
+        blocks.append(q)
+    first = (C.c_ubyte * 100).from_address(blocks[0])
+    assert all(b == 0xA5 for b in first)  # handed out below the rewind point: still alive
+    lib.blt_arena_reset(C.byref(dev))
+    assert dev.offset == 0
 
 
 FATAL_SNIPPETS = {
