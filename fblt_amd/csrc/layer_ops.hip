@@ -31,7 +31,11 @@ constexpr float RMSNORM_EPS = 1e-6f; /* csrc/ops/reductions_cpu.c:325 */
 
 /* `parts` lanes (a power of two, 8..64) share a row's loads (coalesced, into
  * LDS), one of them then walks the row in element order.  256 / parts rows
- * per workgroup. */
+ * per workgroup.
+ * VEC (dim a multiple of 4, 16-byte aligned pointers): a lane moves float4s, four requests in
+ * flight; with the trip count unknown at compile time the scalar loops wait for memory once per
+ * element instead. */
+template <bool VEC>
 __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const float *__restrict__ x, const float *__restrict__ w,
                                                            float *__restrict__ out, uint32_t rows, uint32_t dim,
                                                            uint32_t parts) {
@@ -42,7 +46,27 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const float *__restri
     const uint32_t row = blockIdx.x * (256u / parts) + r_local;
     const bool ok = row < rows;
     const float *src = x + (size_t)(ok ? row : rows - 1u) * dim;
-    for (uint32_t j = part; j < dim; j += parts) stage[r_local * pitch + j] = src[j];
+    const uint32_t quads = dim / 4u;
+    if constexpr (VEC) {
+        const float4 *src4 = reinterpret_cast<const float4 *>(src);
+        float4 *st4 = reinterpret_cast<float4 *>(stage + r_local * pitch);
+        for (uint32_t j = part; j < quads; j += 4u * parts) {
+            float4 t[4];
+#pragma unroll
+            for (uint32_t u = 0; u < 4u; u++) t[u] = src4[min(j + u * parts, quads - 1u)];
+#pragma unroll
+            for (uint32_t u = 0; u < 4u; u++)
+                if (j + u * parts < quads) st4[j + u * parts] = t[u];
+        }
+    } else {
+        for (uint32_t j = part; j < dim; j += parts) stage[r_local * pitch + j] = src[j];
+    }
+    float4 w_first[4]; /* the weights of the first round of stores, requested before the row walk */
+    if constexpr (VEC) {
+#pragma unroll
+        for (uint32_t u = 0; u < 4u; u++)
+            w_first[u] = reinterpret_cast<const float4 *>(w)[min(part + u * parts, quads - 1u)];
+    }
     __syncthreads();
     float inv_rms = 0.f;
     if (part == 0) {
@@ -66,7 +90,27 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const float *__restri
     inv_rms = __shfl(inv_rms, (int)((threadIdx.x & 63u) & ~(parts - 1u)), 64);
     if (!ok) return;
     float *dst = out + (size_t)row * dim;
-    for (uint32_t j = part; j < dim; j += parts) dst[j] = stage[r_local * pitch + j] * inv_rms * w[j];
+    if constexpr (VEC) {
+        const float4 *w4 = reinterpret_cast<const float4 *>(w);
+        const float4 *st4 = reinterpret_cast<const float4 *>(stage + r_local * pitch);
+        float4 *dst4 = reinterpret_cast<float4 *>(dst);
+        for (uint32_t j = part; j < quads; j += 4u * parts) {
+            float4 wv[4];
+#pragma unroll
+            for (uint32_t u = 0; u < 4u; u++) wv[u] = j == part ? w_first[u] : w4[min(j + u * parts, quads - 1u)];
+#pragma unroll
+            for (uint32_t u = 0; u < 4u; u++) {
+                if (j + u * parts >= quads) continue;
+                const float4 v = st4[j + u * parts];
+                float4 o;
+                o.x = v.x * inv_rms * wv[u].x, o.y = v.y * inv_rms * wv[u].y;
+                o.z = v.z * inv_rms * wv[u].z, o.w = v.w * inv_rms * wv[u].w;
+                dst4[j + u * parts] = o;
+            }
+        }
+    } else {
+        for (uint32_t j = part; j < dim; j += parts) dst[j] = stage[r_local * pitch + j] * inv_rms * w[j];
+    }
 }
 
 __global__ __launch_bounds__(256) void add_kernel(const float *__restrict__ a, const float *__restrict__ b,
@@ -94,8 +138,14 @@ void rmsnorm_launch(const float *x, const float *w, float *out, size_t rows, siz
     const uint32_t rpw = 256u / parts;
     const size_t lds = rpw * pitch * sizeof(float);
     BLT_REQUIRE(lds <= 64u * 1024u, "RMSNorm: embed_dim up to 4088 is supported by the HIP backend (got %zu)", dim);
-    blt_launch("rmsnorm_rows", rmsnorm_rows_kernel, dim3((uint32_t)((rows + rpw - 1u) / rpw)), dim3(256), lds, 0, x, w,
-               out, (uint32_t)rows, (uint32_t)dim, parts);
+    const bool vec = dim % 4u == 0u && (((uintptr_t)x | (uintptr_t)w | (uintptr_t)out) & 15u) == 0u;
+    const dim3 grid((uint32_t)((rows + rpw - 1u) / rpw));
+    if (vec)
+        blt_launch("rmsnorm_rows", rmsnorm_rows_kernel<true>, grid, dim3(256), lds, 0, x, w, out, (uint32_t)rows,
+                   (uint32_t)dim, parts);
+    else
+        blt_launch("rmsnorm_rows", rmsnorm_rows_kernel<false>, grid, dim3(256), lds, 0, x, w, out, (uint32_t)rows,
+                   (uint32_t)dim, parts);
 }
 void add_launch(const float *a, const float *b, float *out, size_t n) {
     if (n) blt_launch("add", add_kernel, dim3(blocks_for(n)), dim3(256), 0, 0, a, b, out, (uint64_t)n);

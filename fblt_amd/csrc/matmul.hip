@@ -575,8 +575,13 @@ Path choose_path(const MatmulArgs &g) {
         return e && *e ? (uint32_t)atoi(e) : 32u;
     }();
     if (g.m <= exact_rows && !rope && !g.tolerant) return PATH_SKINNY;
-    /* fewer 64x64 tiles than half the compute units: quarter tiles, K split over the waves */
-    if ((uint64_t)((g.n + TN - 1) / TN) * ((g.m + TM - 1) / TM) < 128u) return PATH_SPLITK;
+    /* fewer 64x64 tiles than half the compute units: quarter tiles, K split over the waves
+     * (BLT_HIP_MATMUL_SPLITK_BELOW moves the limit: tuning hook) */
+    static const uint64_t splitk_below = [] {
+        const char *e = getenv("BLT_HIP_MATMUL_SPLITK_BELOW");
+        return e && *e ? (uint64_t)atoll(e) : (uint64_t)128u;
+    }();
+    if ((uint64_t)((g.n + TN - 1) / TN) * ((g.m + TM - 1) / TM) < splitk_below) return PATH_SPLITK;
     return PATH_MFMA;
 }
 

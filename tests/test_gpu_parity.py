@@ -1059,7 +1059,7 @@ def test_row_ops(oracle, dev):
     import torch
     lib = api.load()
     rs = np.random.RandomState(61)
-    for rows, dim in ((1, 128), (64, 128), (100, 512), (7, 33), (2048, 128), (3, 1000)):
+    for rows, dim in ((1, 128), (64, 128), (100, 512), (7, 33), (2048, 128), (3, 1000), (5, 20), (118, 132), (33, 4088), (9, 4)):
         x = (rs.randn(rows, dim) * 2).astype(np.float32)
         w = rs.randn(dim).astype(np.float32)
         y = rs.randn(rows, dim).astype(np.float32)
