@@ -88,29 +88,47 @@ __device__ __forceinline__ void store4(const MatmulArgs &g, uint32_t row, uint32
  * VEC: a, b 16-byte aligned with lda, ldb, K, N multiples of 4, so a 16-byte
  * piece is either entirely inside or entirely outside the matrices.
  * ROPE: rotate pairs of the first g.rope_cols columns in the epilogue. */
-template <bool VEC, bool ROPE, int WT>
-__global__ __launch_bounds__(256, 2) void matmul_mfma_kernel(MatmulArgs g) {
-    constexpr int BM = TM * WT, BN = TN * WT, BK = TK / WT, KH = BK / 2;
-    constexpr int AP = BK + 4; /* floats per LDS row of the a tile: 16-byte fragment reads of 32 rows hit all banks */
-    constexpr int BP = BN + 4;
-    __shared__ __attribute__((aligned(16))) float sa[2][BM * AP];
-    __shared__ __attribute__((aligned(16))) float sb[2][BK * BP];
+template <int WT, int NW>
+struct MfmaShape {
+    static constexpr int BM = TM * WT, BN = TN * WT, BK = TK / WT, THREADS = 64 * NW;
+    static constexpr int AP = BK + 4; /* floats per LDS row of the a tile: 16-byte fragment reads of 32 rows hit all banks */
+    static constexpr int BP = BN + 4;
+    static constexpr int NP = BM * BK / 4 / THREADS; /* 16-byte pieces of each tile a thread moves per step */
+    static constexpr int KW = BK / 2 / (NW / 4);     /* k values of a step per half of a wave */
+    static constexpr size_t LDS_BYTES = (2 * BM * AP + 2 * BK * BP) * sizeof(float);
+    static_assert(BM * BK == BK * BN && NP * 4 * THREADS == BM * BK, "a thread moves the same number of pieces of both tiles");
+    static_assert(NW == 4 || (NW == 8 && WT == 1), "eight waves: the small tile only");
+    static_assert(NW == 4 || 4 * 16 * 64 * sizeof(float) <= LDS_BYTES, "the second group's sums pass through the tile buffers");
+};
+
+/* NW = 8 (small tile): a second group of four waves takes the other half of every K step, so each
+ * SIMD holds two waves of the workgroup and one's waits (LDS, memory, barrier) fall into the
+ * other's matrix instructions; with one workgroup per compute unit and four waves those waits
+ * left the matrix cores idle 46 % of the time.  The groups' sums meet in LDS at the end. */
+template <bool VEC, bool ROPE, int WT, int NW = 4>
+__global__ __launch_bounds__(64 * NW, 2) void matmul_mfma_kernel(MatmulArgs g) {
+    using Shape = MfmaShape<WT, NW>;
+    constexpr int BM = Shape::BM, BN = Shape::BN, BK = Shape::BK, KW = Shape::KW, NP = Shape::NP;
+    constexpr int AP = Shape::AP, BP = Shape::BP, THREADS = Shape::THREADS;
+    extern __shared__ __attribute__((aligned(16))) float mm_lds[];
+    float (*sa)[BM * AP] = reinterpret_cast<float (*)[BM * AP]>(mm_lds);
+    float (*sb)[BK * BP] = reinterpret_cast<float (*)[BK * BP]>(mm_lds + 2 * BM * AP);
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
     const uint32_t h = lane >> 5, c = lane & 31u;
-    const uint32_t wr = wave >> 1, wc = wave & 1u; /* wave's quadrant of the tile */
+    const uint32_t wr = (wave & 3u) >> 1, wc = wave & 1u; /* wave's quadrant of the tile */
+    const uint32_t kg = wave >> 2;                         /* its half of a K step (eight waves) */
     const uint32_t row0 = blockIdx.y * BM, col0 = blockIdx.x * BN;
 
-    /* pieces of 4 floats this thread moves per K step: two of the a tile, two of the b tile.
+    /* pieces of 4 floats this thread moves per K step: NP of the a tile, NP of the b tile.
      * Loads go to clamped addresses and land in registers untouched; pieces outside the matrices
      * are zeroed only when they are parked in LDS, after the step's matrix instructions, so that
      * nothing between the requests and those instructions waits for memory. */
-    float pa[2][4], pb[2][4];
-    auto request = [&](uint32_t k0) __attribute__((always_inline)) {
+    auto request = [&](float (&pa)[NP][4], float (&pb)[NP][4], uint32_t k0) __attribute__((always_inline)) {
 #pragma unroll
-        for (int u = 0; u < 2; u++) {
-            const uint32_t e = threadIdx.x + 256u * u;
+        for (int u = 0; u < NP; u++) {
+            const uint32_t e = threadIdx.x + (uint32_t)THREADS * u;
             {
                 const uint32_t r = row0 + e / (BK / 4), k = k0 + 4u * (e % (BK / 4));
                 const float *src = g.a + (size_t)min(r, g.m - 1u) * g.lda;
@@ -135,10 +153,11 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_kernel(MatmulArgs g) {
             }
         }
     };
-    auto park = [&](uint32_t buf, uint32_t k0) __attribute__((always_inline)) {
+    auto park = [&](const float (&pa)[NP][4], const float (&pb)[NP][4], uint32_t buf, uint32_t k0)
+                    __attribute__((always_inline)) {
 #pragma unroll
-        for (int u = 0; u < 2; u++) {
-            const uint32_t e = threadIdx.x + 256u * u;
+        for (int u = 0; u < NP; u++) {
+            const uint32_t e = threadIdx.x + (uint32_t)THREADS * u;
             const uint32_t ka = k0 + 4u * (e % (BK / 4));
             const uint32_t kb = k0 + e / (BN / 4), col = col0 + 4u * (e % (BN / 4));
             float va[4], vb[4];
@@ -162,39 +181,71 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_kernel(MatmulArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
+    /* Two register sets take turns: the pieces of step s+1 and s+2 are on their way while step s
+     * runs, so a request has two steps of matrix work to arrive in (one step is less than the
+     * memory latency when a wave is alone on its SIMD).  Requests and parks are unconditional --
+     * addresses are clamped, pieces past K parked as zeros -- so that no load sits behind a branch
+     * and no wait has to assume the worst at a join. */
     const uint32_t steps = (g.k + BK - 1u) / BK;
-    request(0);
-    park(0, 0);
+    float pa0[NP][4], pb0[NP][4], pa1[NP][4], pb1[NP][4];
+    request(pa0, pb0, 0);
+    request(pa1, pb1, BK);
+    /* the requests keep the order they have in the loop (one whole set after the other): the wait
+     * counts inside the loop are the worst case of both ways into it */
+    __builtin_amdgcn_sched_barrier(0);
+    park(pa0, pb0, 0, 0);
+    request(pa0, pb0, 2u * BK);
     __syncthreads();
-    for (uint32_t s = 0; s < steps; s++) {
+    auto step = [&](uint32_t s, float (&pa)[NP][4], float (&pb)[NP][4]) __attribute__((always_inline)) {
+        /* (pa, pb) hold the pieces of step s+1 */
         const uint32_t buf = s & 1u;
-        if (s + 1u < steps) request((s + 1u) * BK);
-        /* MFMA A operand (rows of D = output columns): b[k][col], k = KH*h + t
-         * MFMA B operand (columns of D = output rows):  a[row][k]            */
-        const float *ar = &sa[buf][(wr * (32u * WT) + c) * AP + KH * h];
-        const float *bc = &sb[buf][(KH * h) * BP + wc * (32u * WT) + c];
+        /* MFMA A operand (rows of D = output columns): b[k][col], k = KW*(2*kg + h) + t
+         * MFMA B operand (columns of D = output rows):  a[row][k]                       */
+        const float *ar = &sa[buf][(wr * (32u * WT) + c) * AP + KW * (2u * kg + h)];
+        const float *bc = &sb[buf][(KW * (2u * kg + h)) * BP + wc * (32u * WT) + c];
+        /* every fragment of the step is requested from LDS before its first matrix instruction:
+         * read just in time, each pair of instructions waited for the next read */
+        float av[WT][KW], bv[WT][KW];
 #pragma unroll
-        for (int t4 = 0; t4 < KH; t4 += 4) {
-            float av[WT][4];
+        for (int t4 = 0; t4 < KW; t4 += 4) {
 #pragma unroll
             for (int i = 0; i < WT; i++) {
                 const float4 t = *reinterpret_cast<const float4 *>(ar + 32 * i * AP + t4);
-                av[i][0] = t.x, av[i][1] = t.y, av[i][2] = t.z, av[i][3] = t.w;
+                av[i][t4 + 0] = t.x, av[i][t4 + 1] = t.y, av[i][t4 + 2] = t.z, av[i][t4 + 3] = t.w;
             }
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
-                float bv[WT];
+            for (int t = 0; t < 4; t++)
 #pragma unroll
-                for (int j = 0; j < WT; j++) bv[j] = bc[(t4 + t) * BP + 32 * j];
-#pragma unroll
-                for (int i = 0; i < WT; i++)
-#pragma unroll
-                    for (int j = 0; j < WT; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j], av[i][t], acc[i][j], 0, 0, 0);
-            }
+                for (int j = 0; j < WT; j++) bv[j][t4 + t] = bc[(t4 + t) * BP + 32 * j];
         }
-        if (s + 1u < steps) park(buf ^ 1u, (s + 1u) * BK);
+        __builtin_amdgcn_sched_barrier(0); /* the compiler would sink the reads back between the instructions */
+#pragma unroll
+        for (int t = 0; t < KW; t++)
+#pragma unroll
+            for (int i = 0; i < WT; i++)
+#pragma unroll
+                for (int j = 0; j < WT; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j][t], av[i][t], acc[i][j], 0, 0, 0);
+        park(pa, pb, buf ^ 1u, (s + 1u) * BK); /* past K this parks zeros in the buffer nobody reads again */
+        request(pa, pb, (s + 3u) * BK);
         __syncthreads();
+    };
+    /* steps in pairs, one per register set; an odd count ends with a step over zeros */
+    for (uint32_t s = 0; s < steps; s += 2u) {
+        step(s, pa1, pb1);
+        step(s + 1u, pa0, pb0);
+    }
+
+    if constexpr (NW == 8) { /* the loop ended on a barrier: the tile buffers are free */
+        float *meet = mm_lds + (wave & 3u) * (16u * 64u);
+        if (kg == 1u) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) meet[r * 64 + lane] = acc[0][0][r];
+        }
+        __syncthreads();
+        if (kg == 1u) return;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[0][0][r] = acc[0][0][r] + meet[r * 64 + lane];
     }
 
     /* lane (h, c) holds out[row0 + 32*(WT*wr + i) + c][col0 + 32*(WT*wc + j) + 8*q + 4*h + 0..3] in acc[i][j][4q..4q+3] */
@@ -639,6 +690,30 @@ void matmul_f32_launch_pair(const MatmulArgs &g0, const MatmulArgs &g1, hipStrea
     else blt_launch("matmul_splitk", matmul_splitk_pair_kernel<false>, grid, dim3(256), 0, s, g0, g1, rows0);
 }
 
+namespace {
+template <bool VEC, bool ROPE, int WT, int NW>
+void launch_mfma_as(dim3 grid, hipStream_t s, const MatmulArgs &g) {
+    constexpr size_t lds = MfmaShape<WT, NW>::LDS_BYTES;
+    static_assert(lds <= 64u * 1024u, "above 64 KB a kernel has to ask for its LDS first");
+    blt_launch("matmul_mfma", matmul_mfma_kernel<VEC, ROPE, WT, NW>, grid, dim3(64 * NW), lds, s, g);
+}
+template <bool VEC, bool ROPE, int WT>
+void launch_mfma(dim3 grid, hipStream_t s, const MatmulArgs &g) {
+    /* BLT_HIP_MATMUL_WAVES=4 keeps four waves per small tile: tuning hook */
+    static const bool eight = [] {
+        const char *e = getenv("BLT_HIP_MATMUL_WAVES");
+        return !(e && atoi(e) == 4);
+    }();
+    if constexpr (WT == 1) {
+        if (eight && g.k >= 256u) { /* from eight K steps on: below, the meeting of the sums costs what the overlap gains */
+            launch_mfma_as<VEC, ROPE, 1, 8>(grid, s, g);
+            return;
+        }
+    }
+    launch_mfma_as<VEC, ROPE, WT, 4>(grid, s, g);
+}
+} // namespace
+
 void matmul_f32_launch(const MatmulArgs &g, hipStream_t s) {
     if (g.m == 0 || g.n == 0) return;
     const bool rope = g.rope_cos != nullptr && g.rope_cols > 0;
@@ -683,21 +758,21 @@ void matmul_f32_launch(const MatmulArgs &g, hipStream_t s) {
     if (big_ok && (uint64_t)tx * ty >= 512u) {
         const dim3 grid(tx, ty);
         if (rope) {
-            if (vec) blt_launch("matmul_mfma", matmul_mfma_kernel<true, true, 2>, grid, block, 0, s, g);
-            else blt_launch("matmul_mfma", matmul_mfma_kernel<false, true, 2>, grid, block, 0, s, g);
+            if (vec) launch_mfma<true, true, 2>(grid, s, g);
+            else launch_mfma<false, true, 2>(grid, s, g);
         } else {
-            if (vec) blt_launch("matmul_mfma", matmul_mfma_kernel<true, false, 2>, grid, block, 0, s, g);
-            else blt_launch("matmul_mfma", matmul_mfma_kernel<false, false, 2>, grid, block, 0, s, g);
+            if (vec) launch_mfma<true, false, 2>(grid, s, g);
+            else launch_mfma<false, false, 2>(grid, s, g);
         }
         return;
     }
     const dim3 grid((g.n + TN - 1) / TN, (g.m + TM - 1) / TM);
     if (rope) {
-        if (vec) blt_launch("matmul_mfma", matmul_mfma_kernel<true, true, 1>, grid, block, 0, s, g);
-        else blt_launch("matmul_mfma", matmul_mfma_kernel<false, true, 1>, grid, block, 0, s, g);
+        if (vec) launch_mfma<true, true, 1>(grid, s, g);
+        else launch_mfma<false, true, 1>(grid, s, g);
     } else {
-        if (vec) blt_launch("matmul_mfma", matmul_mfma_kernel<true, false, 1>, grid, block, 0, s, g);
-        else blt_launch("matmul_mfma", matmul_mfma_kernel<false, false, 1>, grid, block, 0, s, g);
+        if (vec) launch_mfma<true, false, 1>(grid, s, g);
+        else launch_mfma<false, false, 1>(grid, s, g);
     }
 }
 

@@ -846,7 +846,8 @@ def _dev_tensor(t, shape=None):
                                           (3, 1100, 70, True), (1, 7, 300, True), (9, 528, 257, True),
                                           (16, 128, 512, True), (33, 64, 64, False), (64, 128, 384, False),
                                           (512, 128, 384, False), (100, 70, 50, False), (513, 129, 130, False),
-                                          (2048, 512, 1536, False), (4100, 70, 2050, False), (4096, 96, 2048, False)])
+                                          (2048, 512, 1536, False), (4100, 70, 2050, False), (4096, 96, 2048, False),
+                                          (1500, 300, 600, False), (1100, 257, 1030, False), (2048, 2048, 512, False)])
 def test_matmul(m, k, n, exact, oracle, dev):
     """blt_matmul: up to 32 rows bit-identical to the reference loop, above that fp32 tolerance."""
     import torch
