@@ -60,13 +60,13 @@ typedef struct host_block {
 static host_block *g_host_blocks = NULL;
 static pthread_mutex_t g_host_blocks_lock = PTHREAD_MUTEX_INITIALIZER;
 
-/* Frees the arena's host blocks that were handed out above `keep_to` (all of them for 0 with
+/* Frees the arena's host blocks that were handed out at or above `keep_to` (all of them with
  * `all` set).  Caller holds the lock. */
 static void host_blocks_release(const blt_arena *a, size_t keep_to, int all) {
     host_block **link = &g_host_blocks;
     while (*link) {
         host_block *b = *link;
-        if (b->arena == a && (all || b->at > keep_to)) {
+        if (b->arena == a && (all || b->at >= keep_to)) {
             *link = b->next;
             free(b);
         } else {
@@ -113,10 +113,11 @@ void *blt_arena_alloc(blt_arena *a, size_t bytes, size_t alignment) {
  * model structs (csrc/models/local_decoder.c:76-80, transformer_stack.c:85).  On the CPU backend
  * they live in the arena (csrc/core/tensor.c:154); for a device arena the reference hands out
  * zeroed host memory instead (tensor.c:156-162, backend.c:494-501) and never releases it.  Here a
- * block belongs to its arena: it is released when the arena is reset or destroyed, or once the
- * caller has rewound the arena's offset below the point the block was handed out at
- * (csrc/infer/self_speculation.c:359-401 rewinds that way), which is when a container of the CPU
- * backend would be dead too. */
+ * block belongs to its arena and takes a 64-byte token of it, which gives the block a place in the
+ * arena's order: it is released when the arena is reset or destroyed, or once the caller has
+ * rewound the arena's offset to or below its token (csrc/infer/self_speculation.c:359-401 rewinds
+ * that way), which is when a container of the CPU backend would be dead too.  A loop that rewinds
+ * to a marker every round therefore holds one round's blocks at most. */
 void *blt_container_alloc(blt_arena *a, size_t bytes) {
     if (!a || !a->buffer) BLT_FATAL("invalid arena");
     if (a->backend != BLT_BACKEND_HIP) return blt_arena_alloc(a, bytes, 64);
@@ -129,10 +130,11 @@ void *blt_container_alloc(blt_arena *a, size_t bytes) {
     b->arena = a;
     b->at = a->offset;
     pthread_mutex_lock(&g_host_blocks_lock);
-    host_blocks_release(a, a->offset, 0);
+    host_blocks_release(a, a->offset, 0); /* whatever sat at or above this point was rewound over */
     b->next = g_host_blocks;
     g_host_blocks = b;
     pthread_mutex_unlock(&g_host_blocks_lock);
+    (void)blt_arena_alloc(a, 64, 1); /* the token */
     return (char *)b + HOST_BLOCK_HEADER;
 }
 

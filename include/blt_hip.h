@@ -192,9 +192,9 @@ void blt_arena_reset(blt_arena *arena);
 void *blt_arena_alloc(blt_arena *arena, size_t bytes, size_t alignment);
 /* csrc/core/allocator.h:33 (tensor.c:154-162, backend.c:494-501).  Memory the caller fills and
  * reads on the host (group-id arrays, weight-view and model structs): arena memory on the CPU
- * backend, zeroed host memory for a device arena.  A device arena's blocks are released with
- * blt_arena_reset / blt_arena_destroy, or once the arena's offset has been rewound below the
- * point they were handed out at. */
+ * backend, zeroed host memory for a device arena, plus a 64-byte token of the arena that marks the
+ * block's place in it.  A device arena's blocks are released with blt_arena_reset /
+ * blt_arena_destroy, or once the arena's offset has been rewound to or below their token. */
 void *blt_container_alloc(blt_arena *arena, size_t bytes);
 blt_tensor blt_tensor_create(blt_arena *arena, const size_t *shape, size_t ndim, blt_dtype dtype);
 blt_tensor blt_tensor_create_uninit(blt_arena *arena, const size_t *shape, size_t ndim, blt_dtype dtype);

@@ -308,7 +308,7 @@ def test_host_arena_and_tensor():
 
 def test_containers_are_host_memory_for_a_device_arena():
     """blt_container_alloc (csrc/core/tensor.c:154-162): arena memory on the CPU backend; for a device arena zeroed,
-    64-byte aligned host memory that leaves the arena's offset alone, released with the arena's reset.  The device
+    64-byte aligned host memory plus a 64-byte token of the arena, released with the arena's reset or a rewind.  The device
     arena here is a hand-made struct whose buffer is never touched, so this runs without a GPU."""
     lib = api.load()
     host = lib.blt_arena_create(4096, abi.BLT_BACKEND_CPU)
@@ -318,18 +318,27 @@ def test_containers_are_host_memory_for_a_device_arena():
 
     dev = abi.BltArena()
     dev.buffer, dev.capacity, dev.offset, dev.backend = 0x10000, 1 << 20, 0, abi.BLT_BACKEND_HIP
-    blocks = []
-    for at, size in ((0, 100), (512, 8), (512, 4000), (256, 64), (256, 1)):  # the fourth follows a rewind
-        dev.offset = at
+
+    def take(size):
+        before = dev.offset
         q = lib.blt_container_alloc(C.byref(dev), size)
-        assert q % 64 == 0 and dev.offset == at
+        assert q % 64 == 0 and dev.offset == before + 64  # the block's token in the arena
         view = (C.c_ubyte * size).from_address(q)
         assert not any(view)
         for i in range(size):
             view[i] = 0xA5  # host-writable
-        blocks.append(q)
-    first = (C.c_ubyte * 100).from_address(blocks[0])
-    assert all(b == 0xA5 for b in first)  # handed out below the rewind point: still alive
+        return q
+
+    keep = take(100)
+    marker = dev.offset
+    for _ in range(3):  # a caller that rewinds to its marker every round (csrc/infer/self_speculation.c:359-401)
+        take(8)
+        dev.offset += 4096
+        take(4000)
+        take(1)
+        dev.offset = marker
+    take(64)
+    assert all(b == 0xA5 for b in (C.c_ubyte * 100).from_address(keep))  # handed out below the marker: still alive
     lib.blt_arena_reset(C.byref(dev))
     assert dev.offset == 0
 
