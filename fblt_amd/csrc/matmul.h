@@ -50,6 +50,13 @@ struct MatmulArgs {
      * the matrix cores with K split over the waves (the whole decoder step sets it: a one-row
      * step takes 72 us instead of 112). */
     uint32_t tolerant;
+    /* Set by the launcher, never by callers.  slices > 1: the K range is also split over slices
+     * workgroups per output tile (grid z); each leaves its 32x32 sums in slice_sums
+     * [tile][slice][1024] and the one that draws the last of the tile's tickets adds them in slice
+     * order and runs the epilogue. */
+    uint32_t slices;
+    float *slice_sums;
+    uint32_t *slice_tickets;
 };
 
 void matmul_f32_launch(const MatmulArgs &g, hipStream_t s);

@@ -42,6 +42,9 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <algorithm>
+#include <map>
+
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -328,11 +331,16 @@ __device__ __forceinline__ void splitk_tile(const MatmulArgs &g, const uint32_t 
     floatx16 acc, acc2;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.f, acc2[r] = 0.f;
-    const uint32_t chunks = (g.k + 31u) / 32u;
+    uint32_t chunks = (g.k + 31u) / 32u, first = 0u;
+    if (g.slices > 1u) { /* this workgroup's share of the chunks */
+        const uint32_t per = (chunks + g.slices - 1u) / g.slices;
+        first = min(blockIdx.z * per, chunks);
+        chunks = min(first + per, chunks);
+    }
     float fa[16], fb[16], fg[GATED ? 16 : 1];
     float dummy[GATED ? 1 : 16]; /* stands in for the gate fragment when there is none */
     (void)dummy;
-    uint32_t ch = wave;
+    uint32_t ch = first + wave;
     if (ch < chunks) {
         if constexpr (GATED) fetch(ch * 32u, fa, fb, fg);
         else fetch(ch * 32u, fa, fb, dummy);
@@ -392,6 +400,29 @@ __device__ __forceinline__ void splitk_tile(const MatmulArgs &g, const uint32_t 
             if (g.out2) second[i] = gate; /* two products, two outputs */
             else v4[i] = silu_times(gate, v4[i]);
         }
+    }
+    if (!GATED && !CROSS && g.slices > 1u) {
+        /* Device-scope stores and loads, and the barrier's wait on outstanding memory operations
+         * between this workgroup's stores and its ticket, as for the split softmax states of the
+         * KV step (kv_step.h).  The waves past the fourth have left. */
+        __shared__ uint32_t ticket;
+        const uint32_t tile = by * gridDim.x + bx;
+        float *sums = g.slice_sums + (size_t)tile * g.slices * 1024u + 4u * threadIdx.x;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            __hip_atomic_store(sums + (size_t)blockIdx.z * 1024u + i, v4[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (threadIdx.x == 0)
+            ticket = __hip_atomic_fetch_add(&g.slice_tickets[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (ticket != g.slices - 1u) return;
+        if (threadIdx.x == 0) g.slice_tickets[tile] = 0u; /* re-armed for the next launch */
+#pragma unroll
+        for (int i = 0; i < 4; i++) v4[i] = __hip_atomic_load(sums + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (uint32_t z = 1; z < g.slices; z++) /* slice order, whoever comes last */
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                v4[i] += __hip_atomic_load(sums + (size_t)z * 1024u + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (CROSS) {
         /* The tile is the projected query of 32 rows for head bx: park it, then wave w takes rows
@@ -626,20 +657,80 @@ Path choose_path(const MatmulArgs &g) {
         return e && *e ? (uint32_t)atoi(e) : 32u;
     }();
     if (g.m <= exact_rows && !rope && !g.tolerant) return PATH_SKINNY;
-    /* fewer 64x64 tiles than half the compute units: quarter tiles, K split over the waves
-     * (BLT_HIP_MATMUL_SPLITK_BELOW moves the limit: tuning hook) */
+    /* up to 143 64x64 tiles (a bit over half the compute units): quarter tiles, K split over the
+     * waves.  Measured at K = 512 ... 4096: a fifth faster than the 64x64 kernel at 128 tiles, level
+     * with it at 144 ... 192, a quarter slower at 256 (BLT_HIP_MATMUL_SPLITK_BELOW moves the limit:
+     * tuning hook) */
     static const uint64_t splitk_below = [] {
         const char *e = getenv("BLT_HIP_MATMUL_SPLITK_BELOW");
-        return e && *e ? (uint64_t)atoll(e) : (uint64_t)128u;
+        return e && *e ? (uint64_t)atoll(e) : (uint64_t)144u;
     }();
     if ((uint64_t)((g.n + TN - 1) / TN) * ((g.m + TM - 1) / TM) < splitk_below) return PATH_SPLITK;
     return PATH_MFMA;
 }
 
+/* Sums and tickets of the K slices, per (thread, stream) like the scratch of the KV step: launches
+ * on one stream follow each other, launches on two streams never share them. */
+struct SliceScratch {
+    float *sums = nullptr;
+    size_t sum_floats = 0;
+    uint32_t *tickets = nullptr;
+    size_t ticket_count = 0;
+};
+__global__ void clear_words_kernel(uint32_t *w, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256u + threadIdx.x;
+    if (i < n) w[i] = 0u;
+}
+/* false: the scratch would have to grow while a graph capture is open (the launch then runs unsliced) */
+bool slice_scratch(MatmulArgs &g, size_t tiles, hipStream_t s) {
+    static thread_local std::map<hipStream_t, SliceScratch> by_stream;
+    SliceScratch &sc = by_stream[blt_stream_key()];
+    const size_t floats = tiles * g.slices * 1024u;
+    if (blt_stream_capturing() && (floats > sc.sum_floats || tiles > sc.ticket_count)) return false;
+    /* outgrown buffers are left to the process: a launch still in flight may be using them */
+    if (floats > sc.sum_floats) {
+        sc.sum_floats = std::max(floats, 2 * sc.sum_floats);
+        HIP_CHECK(hipMalloc((void **)&sc.sums, sc.sum_floats * sizeof(float)));
+    }
+    if (tiles > sc.ticket_count) {
+        sc.ticket_count = std::max<size_t>(2 * tiles, 1024);
+        HIP_CHECK(hipMalloc((void **)&sc.tickets, sc.ticket_count * sizeof(uint32_t)));
+        /* a fill kernel, not a memset, on the stream the launches follow */
+        hipLaunchKernelGGL(clear_words_kernel, dim3((unsigned)((sc.ticket_count + 255) / 256)), dim3(256), 0,
+                           s ? s : blt_stream(), sc.tickets, sc.ticket_count);
+    }
+    g.slice_sums = sc.sums;
+    g.slice_tickets = sc.tickets;
+    return true;
+}
+
+/* Slices of K per output tile: long K over few tiles leaves most of the chip idle and every wave
+ * with a serial chain of chunk loads (2048 x 512 weights under 118 rows: 64 tiles, eight chunks per
+ * wave).  As many slices as keep one chunk per wave and give one workgroup per compute unit: measured
+ * over 12 ... 256 tiles and K = 1024 ... 4096, the best count was the one that brought the launch
+ * to about 256 workgroups, and more made it slower again.
+ * BLT_HIP_MATMUL_KSLICES=1 switches them off, n > 1 forces n: tuning hook. */
+uint32_t slices_for(const MatmulArgs &g, dim3 grid, bool eight) {
+    static const int forced = [] {
+        const char *e = getenv("BLT_HIP_MATMUL_KSLICES");
+        return e && *e ? atoi(e) : 0;
+    }();
+    if (g.b2 || g.cross_k || g.norm_w) return 1u;
+    const uint32_t chunks = (g.k + 31u) / 32u, tiles = grid.x * grid.y;
+    const uint32_t room = chunks / (eight ? 8u : 4u);
+    if (forced >= 1) return std::max(1u, std::min((uint32_t)forced, std::min(room, 64u)));
+    if (chunks < 32u || tiles > 128u) return 1u;
+    return std::max(1u, std::min(room, 256u / tiles));
+}
+
 template <bool VEC, bool ROPE>
-void launch_splitk(const MatmulArgs &g, dim3 grid, hipStream_t s) {
+void launch_splitk(const MatmulArgs &g_in, dim3 grid, hipStream_t s) {
     /* eight waves once every wave still gets a chunk (K >= 256) and the launch leaves the chip room for them */
-    const bool eight = g.k >= 256u && (uint64_t)grid.x * grid.y <= 512u;
+    const bool eight = g_in.k >= 256u && (uint64_t)grid.x * grid.y <= 512u;
+    MatmulArgs g = g_in;
+    g.slices = slices_for(g, grid, eight);
+    if (g.slices > 1u && slice_scratch(g, (size_t)grid.x * grid.y, s)) grid.z = g.slices;
+    else g.slices = 1u;
     if (g.cross_k) {
         if constexpr (VEC && !ROPE)
             blt_launch("matmul_splitk_cross", matmul_splitk_kernel<true, false, false, 4, true>, grid, dim3(256), 0, s, g);

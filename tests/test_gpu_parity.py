@@ -847,7 +847,8 @@ def _dev_tensor(t, shape=None):
                                           (16, 128, 512, True), (33, 64, 64, False), (64, 128, 384, False),
                                           (512, 128, 384, False), (100, 70, 50, False), (513, 129, 130, False),
                                           (2048, 512, 1536, False), (4100, 70, 2050, False), (4096, 96, 2048, False),
-                                          (1500, 300, 600, False), (1100, 257, 1030, False), (2048, 2048, 512, False)])
+                                          (1500, 300, 600, False), (1100, 257, 1030, False), (2048, 2048, 512, False),
+                                          (118, 2048, 512, False), (64, 4096, 256, False), (100, 3000, 70, False), (33, 1025, 40, False)])
 def test_matmul(m, k, n, exact, oracle, dev):
     """blt_matmul: up to 32 rows bit-identical to the reference loop, above that fp32 tolerance."""
     import torch
@@ -867,6 +868,33 @@ def test_matmul(m, k, n, exact, oracle, dev):
         assert got.tobytes() == ref.tobytes()
     else:
         assert_close(got, ref, "matmul %dx%dx%d" % (m, k, n))
+
+
+def test_matmul_k_slices_back_to_back(dev):
+    """Long-K products over few output tiles split K over several workgroups per tile, which meet through
+    per-stream sums and tickets: launches of different shapes issued back to back, without a wait in between,
+    must each find the tickets re-armed and must give the same bits every time (the slices are added in slice
+    order whichever workgroup comes last)."""
+    import torch
+    lib = api.load()
+    torch.manual_seed(5)
+    shapes = [(118, 2048, 512), (64, 4096, 256), (100, 3000, 70), (40, 1024, 2048), (118, 2048, 512)]
+    ops = []
+    for m, k, n in shapes:
+        a = torch.randn(m, k, device="cuda")
+        b = torch.randn(k, n, device="cuda") / k ** 0.5
+        outs = [torch.full((m, n), 3.0, device="cuda") for _ in range(3)]
+        ops.append((a, b, outs))
+    for rnd in range(3):
+        for a, b, outs in ops:
+            va, vb, vo = _dev_tensor(a), _dev_tensor(b), _dev_tensor(outs[rnd])
+            lib.blt_matmul(C.byref(va), C.byref(vb), C.byref(vo))
+    lib.blt_backend_pass_sync_hip()
+    for (m, k, n), (a, b, outs) in zip(shapes, ops):
+        want = (a.double() @ b.double()).float().cpu().numpy()
+        got = [o.cpu().numpy() for o in outs]
+        assert_close(got[0], want, "sliced matmul %dx%dx%d" % (m, k, n))
+        assert got[0].tobytes() == got[1].tobytes() == got[2].tobytes(), (m, k, n)
 
 
 def test_rope_apply_bit_exact(oracle, dev):
