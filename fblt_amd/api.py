@@ -24,7 +24,7 @@ class BltAttentionProblem(C.Structure):
     _fields_ = [
         ("head", abi.BltAttentionHeadArgs),
         ("mask_kind", C.c_uint32),
-        ("reserved", C.c_uint32),
+        ("row_span", C.c_uint32),
         ("causal_offset", C.c_size_t),
         ("window", C.c_size_t),
         ("row_lo", C.c_void_p),
@@ -258,10 +258,11 @@ def head_args(q_ptr, k_ptr, v_ptr, out_ptr, nq, nk, hd, scale, q_stride, k_strid
     return a
 
 
-def problem(head, kind=BLT_ATTN_MASK_FROM_HEAD, causal_offset=0, window=0, row_lo=None, row_hi=None):
+def problem(head, kind=BLT_ATTN_MASK_FROM_HEAD, causal_offset=0, window=0, row_lo=None, row_hi=None, row_span=0):
     p = BltAttentionProblem()
     p.head = head
     p.mask_kind = kind
+    p.row_span = row_span
     p.causal_offset = causal_offset
     p.window = window
     p.row_lo = row_lo

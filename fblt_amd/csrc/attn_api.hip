@@ -97,6 +97,7 @@ AttnProb translate(const blt_attention_problem &pr, bool need_score_buffer, cons
         d.vis = ATTN_VIS_RANGE;
         d.row_lo = pr.row_lo;
         d.row_hi = pr.row_hi;
+        d.range_span = pr.row_span;
         break;
     default:
         BLT_FATAL("%s: unknown mask_kind %u", what, pr.mask_kind);

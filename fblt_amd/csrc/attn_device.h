@@ -38,7 +38,8 @@ struct AttnProb {
     uint32_t causal_off, window;
     float scale;
     uint32_t flags;
-    uint32_t reserved0, reserved1;
+    uint32_t range_span; /* ATTN_VIS_RANGE: longest range of a row if the caller said so, else 0 */
+    uint32_t reserved1;
 };
 
 static_assert(sizeof(AttnProb) == 128, "AttnProb is staged to the device as raw bytes");

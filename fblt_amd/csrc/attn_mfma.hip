@@ -576,7 +576,16 @@ bool attn_mfma_can(const AttnProb &d) { return d.hd <= 128u && d.nk >= 1u && d.n
 /* shapes it is the better choice for */
 bool attn_mfma_takes(const AttnProb &d) {
     if (!attn_mfma_can(d)) return false;
-    if (d.vis == ATTN_VIS_RANGE) return false; /* per-row ranges are short: the rows family reads less */
+    /* per-row ranges are short (a patch's bytes) unless the caller says otherwise: the rows family
+     * reads less.  Document-causal self-attention comes as ranges as long as the document: measured
+     * at 128 ... 2048 rows, both head widths, the two families are level at ranges of 16 keys, this
+     * one is 1.5 times faster at 32 and 9 ... 13 times at 512 and more
+     * (BLT_HIP_RANGE_SPAN_MIN moves the limit: tuning hook). */
+    static const uint32_t span_min = [] {
+        const char *e = getenv("BLT_HIP_RANGE_SPAN_MIN");
+        return e && *e ? (uint32_t)atol(e) : 24u;
+    }();
+    if (d.vis == ATTN_VIS_RANGE && d.range_span < span_min) return false;
     return d.nq >= 16u;
 }
 

@@ -45,7 +45,8 @@ __device__ __forceinline__ void affine_problem(AttnProb &p, const AttnAffine &af
     p.q_stride = f.q_stride, p.k_stride = f.k_stride, p.v_stride = f.v_stride, p.out_stride = f.out_stride;
     p.nq = f.nq, p.nk = f.nk, p.hd = f.hd, p.vis = f.vis;
     p.causal_off = f.causal_off, p.window = f.window, p.scale = f.scale, p.flags = f.flags;
-    p.reserved0 = p.reserved1 = 0;
+    p.range_span = f.range_span;
+    p.reserved1 = 0;
 }
 
 /* Keys any of the query rows [first, last] can see, [tlo, thi), and keys all

@@ -19,6 +19,7 @@
 #include "launch.h"
 #include "matmul.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 #include <vector>
@@ -137,6 +138,7 @@ void mha_run(const blt_tensor *input, const blt_tensor *weight_qkv, const blt_te
     const uint32_t *row_lo = nullptr, *row_hi = nullptr;
     bool causal_desc = false;
     size_t causal_off = 0, window = 0;
+    uint32_t row_span = 0;
     if (mc != NULL) {
         BLT_REQUIRE(mc->seq_len_q == T && mc->seq_len_kv == T,
                     "blt_multihead_attention: mask_config seq_len_q/seq_len_kv must match input seq_len ");
@@ -154,8 +156,10 @@ void mha_run(const blt_tensor *input, const blt_tensor *weight_qkv, const blt_te
              * the pinned ring; the dense matrix from the device builder otherwise */
             std::vector<uint32_t> lohi(2 * T);
             if (blt_mask_config_row_ranges(mc, lohi.data(), lohi.data() + T) == 1) {
-                for (size_t i = 0; i < T; i++) /* the dense builder refuses such a mask (mask_builder_cpu.c:93) */
+                for (size_t i = 0; i < T; i++) { /* the dense builder refuses such a mask (mask_builder_cpu.c:93) */
                     BLT_REQUIRE(lohi[i] < lohi[T + i], "blt_build_attention_mask: query position has no valid key");
+                    row_span = std::max(row_span, lohi[T + i] - lohi[i]);
+                }
                 uint32_t *dev = (uint32_t *)blt_arena_alloc(arena, 2 * T * sizeof(uint32_t), 64);
                 blt_upload_staged(dev, lohi.data(), 2 * T * sizeof(uint32_t));
                 row_lo = dev, row_hi = dev + T;
@@ -190,6 +194,7 @@ void mha_run(const blt_tensor *input, const blt_tensor *weight_qkv, const blt_te
             p.mask_kind = BLT_ATTN_MASK_ROW_RANGE;
             p.row_lo = row_lo;
             p.row_hi = row_hi;
+            p.row_span = row_span;
         } else {
             p.mask_kind = BLT_ATTN_MASK_FROM_HEAD;
             p.head.mask = dense;
@@ -393,11 +398,14 @@ extern "C" void blt_cross_attention_forward_hip(const blt_tensor *query_in, cons
     /* 3. mask as row ranges when it reduces, then every head in one launch */
     const uint32_t *row_lo = nullptr, *row_hi = nullptr;
     const float *dense = nullptr;
+    uint32_t row_span = 0;
     {
         std::vector<uint32_t> lohi(2 * P);
         if (blt_mask_config_row_ranges(mc, lohi.data(), lohi.data() + P) == 1) {
-            for (size_t i = 0; i < P; i++) /* the dense builder refuses such a mask (mask_builder_cpu.c:93) */
+            for (size_t i = 0; i < P; i++) { /* the dense builder refuses such a mask (mask_builder_cpu.c:93) */
                 BLT_REQUIRE(lohi[i] < lohi[P + i], "blt_build_attention_mask: query position has no valid key");
+                row_span = std::max(row_span, lohi[P + i] - lohi[i]);
+            }
             uint32_t *dev = (uint32_t *)blt_arena_alloc(arena, 2 * P * sizeof(uint32_t), 64);
             blt_upload_staged(dev, lohi.data(), 2 * P * sizeof(uint32_t));
             row_lo = dev, row_hi = dev + P;
@@ -428,6 +436,7 @@ extern "C" void blt_cross_attention_forward_hip(const blt_tensor *query_in, cons
             p.mask_kind = BLT_ATTN_MASK_ROW_RANGE;
             p.row_lo = row_lo;
             p.row_hi = row_hi;
+            p.row_span = row_span;
         } else {
             p.mask_kind = BLT_ATTN_MASK_FROM_HEAD;
             p.head.mask = dense;

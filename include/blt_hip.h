@@ -305,7 +305,9 @@ typedef enum {
 typedef struct {
     blt_attention_head_args head;
     uint32_t mask_kind; /* blt_attn_mask_kind */
-    uint32_t reserved;
+    uint32_t row_span;  /* BLT_ATTN_MASK_ROW_RANGE: the longest range of any row when the caller knows it (it built
+                           the ranges on the host); 0 = unknown, taken as short.  Short ranges (a patch's bytes) run
+                           one row per wave; long ones (document-causal self-attention) on the matrix cores. */
     size_t causal_offset;
     size_t window;
     const uint32_t *row_lo; /* device, [nq] */

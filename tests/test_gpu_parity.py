@@ -870,6 +870,54 @@ def test_matmul(m, k, n, exact, oracle, dev):
         assert_close(got, ref, "matmul %dx%dx%d" % (m, k, n))
 
 
+@pytest.mark.parametrize("T,H,hd,docs", [(200, 2, 32, [0, 7, 90, 150]), (512, 4, 32, [0, 300]), (128, 8, 64, [0]),
+                                         (96, 2, 64, [0, 20, 40, 60, 80])])
+def test_document_causal_ranges_take_the_matrix_cores(T, H, hd, docs, oracle, dev):
+    """Row-range problems whose caller states a long row_span (document-causal self-attention: row i sees
+    [start of its document, i]) run on the matrix-core family, short or unstated spans one row per wave; both
+    against the restated core under the equivalent dense mask (csrc/ops/mask_builder_cpu.c:21-98)."""
+    import torch
+    lib = api.load()
+    rs = np.random.RandomState(T + hd)
+    E = H * hd
+    qkv = rs.randn(T, 3 * E).astype(np.float32)
+    start = np.zeros(T, dtype=np.uint32)
+    for d0 in docs:
+        start[d0:] = d0
+    lo, hi = start, (np.arange(T) + 1).astype(np.uint32)
+    mask = np.full((T, T), -np.inf, dtype=np.float32)
+    for i in range(T):
+        mask[i, lo[i]:hi[i]] = 0.0
+    ref = np.zeros((T, E), dtype=np.float32)
+    wts = np.zeros((T, T), dtype=np.float32)
+    flat = qkv.reshape(-1)
+    for h in range(H):
+        a = binding.head_args(flat, flat, flat, ref.reshape(-1), T, T, hd, 1.0 / np.sqrt(hd), 3 * E, 3 * E, 3 * E, E,
+                              h * hd, q_off=h * hd, k_off=E + h * hd, v_off=2 * E + h * hd, weights=wts.reshape(-1),
+                              mask=mask.reshape(-1))
+        assert oracle.orc_attention_head_core(C.byref(a)) == 0
+    tq = torch.from_numpy(qkv).cuda()
+    dlo, dhi = torch.from_numpy(lo.view(np.int32)).cuda(), torch.from_numpy(hi.view(np.int32)).cuda()
+    span = int((hi - lo).max())
+    for stated, kernel in ((span, "attn_mfma" if span >= 24 else "attn_rows"), (0, "attn_rows")):
+        to = torch.zeros((T, E), dtype=torch.float32, device="cuda")
+        probs = []
+        for h in range(H):
+            a = abi.BltAttentionHeadArgs()
+            a.q, a.k, a.v = tq.data_ptr() + 4 * h * hd, tq.data_ptr() + 4 * (E + h * hd), tq.data_ptr() + 4 * (2 * E + h * hd)
+            a.q_stride = a.k_stride = a.v_stride = 3 * E
+            a.combined, a.combined_stride, a.combined_col_offset = to.data_ptr(), E, h * hd
+            a.nq = a.nk = T
+            a.head_dim, a.scale = hd, 1.0 / np.sqrt(hd)
+            probs.append(api.problem(a, api.BLT_ATTN_MASK_ROW_RANGE, row_lo=dlo.data_ptr(), row_hi=dhi.data_ptr(),
+                                     row_span=stated))
+        lib.blt_hip_profile_begin()
+        lib.blt_attention_batch_hip(api.problem_array(probs), H)
+        launched = api.profile_end()
+        assert list(launched) == [kernel], (launched, stated)
+        assert_close(to.cpu().numpy(), ref, "document-causal ranges T=%d span stated %d" % (T, stated))
+
+
 def test_matmul_k_slices_back_to_back(dev):
     """Long-K products over few output tiles split K over several workgroups per tile, which meet through
     per-stream sums and tickets: launches of different shapes issued back to back, without a wait in between,
