@@ -328,12 +328,24 @@ void plan_build(blt_attention_plan &pl, const blt_attention_problem *problems, s
     pl.host.reserve(count);
     std::vector<std::pair<uint64_t, AttnProb>> keyed;
     keyed.reserve(count);
+    bool any_mfma = false;
     for (size_t t = 0; t < count; t++) {
         AttnProb d = translate(problems[t], need_score_buffer, what);
         if (d.nq == 0) continue; /* nothing to write */
         const Family f = choose_family(d);
+        any_mfma = any_mfma || f == FAM_MFMA;
         const uint64_t vec4 = (d.flags & ATTN_FLAG_VEC4) ? 1u : 0u, dense = d.vis == ATTN_VIS_DENSE ? 1u : 0u;
         keyed.emplace_back(((uint64_t)f << 40) | ((uint64_t)d.hd << 8) | (vec4 << 1) | dense, d);
+    }
+    /* Problems that went to the rows family only for their few rows (the short documents of a
+     * document-causal batch) join the matrix-core launch the batch has anyway rather than cost a
+     * launch of their own. */
+    if (any_mfma && family_override() == 0) {
+        for (auto &kd : keyed) {
+            const AttnProb &d = kd.second;
+            if ((Family)(kd.first >> 40) == FAM_ROWS && d.vis != ATTN_VIS_RANGE && attn_mfma_can(d))
+                kd.first = (kd.first & ((1ull << 40) - 1u)) | ((uint64_t)FAM_MFMA << 40);
+        }
     }
     std::stable_sort(keyed.begin(), keyed.end(),
                      [](const std::pair<uint64_t, AttnProb> &x, const std::pair<uint64_t, AttnProb> &y) {

@@ -139,14 +139,33 @@ void mha_run(const blt_tensor *input, const blt_tensor *weight_qkv, const blt_te
     bool causal_desc = false;
     size_t causal_off = 0, window = 0;
     uint32_t row_span = 0;
+    std::vector<size_t> doc_start; /* document-causal: first row of every document, then T */
     if (mc != NULL) {
         BLT_REQUIRE(mc->seq_len_q == T && mc->seq_len_kv == T,
                     "blt_multihead_attention: mask_config seq_len_q/seq_len_kv must match input seq_len ");
         const bool plain = mc->doc_boundaries == NULL && mc->query_group_ids == NULL && mc->kv_group_ids == NULL;
+        const bool documents = mc->doc_boundaries != NULL && mc->num_docs > 0 && mc->query_group_ids == NULL &&
+                               mc->kv_group_ids == NULL;
         if (plain && mc->is_causal) {
             causal_desc = true;
             causal_off = mc->causal_offset;
             window = mc->sliding_window;
+        } else if (documents && mc->is_causal && mc->causal_offset == 0) {
+            /* Document-causal (csrc/ops/mask_builder_cpu.c:10-19, 52-79: same document, not after the
+             * row, inside the window): a row never looks past the start of its document, so every
+             * document is a causal problem of its own over its own rows -- the shape the causal
+             * kernels are built for, with no key outside the document ever touched.  Documents are
+             * runs of the position -> document map the builder uses. */
+            causal_desc = true;
+            window = mc->sliding_window;
+            size_t d = 0;
+            doc_start.push_back(0);
+            for (size_t pos = 0; pos < T; pos++) {
+                const size_t before = d;
+                while (d + 1 < mc->num_docs && pos >= mc->doc_boundaries[d]) d++;
+                if (d != before && pos != 0) doc_start.push_back(pos);
+            }
+            doc_start.push_back(T);
         } else if (plain && mc->sliding_window == 0) {
             /* nothing masked */
         } else {
@@ -171,19 +190,22 @@ void mha_run(const blt_tensor *input, const blt_tensor *weight_qkv, const blt_te
             }
         }
     }
-    std::vector<blt_attention_problem> pr(H);
+    if (doc_start.empty()) doc_start = {0, T}; /* one problem per head over all rows */
+    const size_t docs = doc_start.size() - 1;
+    std::vector<blt_attention_problem> pr(docs * H);
     const float scale = 1.0f / sqrtf((float)hd);
-    for (size_t head = 0; head < H; head++) {
-        blt_attention_problem &p = pr[head];
+    for (size_t t = 0; t < docs * H; t++) {
+        const size_t head = t % H, first = doc_start[t / H], rows = doc_start[t / H + 1] - first;
+        blt_attention_problem &p = pr[t];
         std::memset(&p, 0, sizeof(p));
-        p.head.q = qkv + head * hd;
-        p.head.k = qkv + E + head * hd;
-        p.head.v = qkv + 2 * E + head * hd;
+        p.head.q = qkv + first * 3 * E + head * hd;
+        p.head.k = qkv + first * 3 * E + E + head * hd;
+        p.head.v = qkv + first * 3 * E + 2 * E + head * hd;
         p.head.q_stride = p.head.k_stride = p.head.v_stride = 3 * E;
-        p.head.combined = combined;
+        p.head.combined = combined + first * E;
         p.head.combined_stride = E;
         p.head.combined_col_offset = head * hd;
-        p.head.nq = p.head.nk = T;
+        p.head.nq = p.head.nk = rows;
         p.head.head_dim = hd;
         p.head.scale = scale;
         if (causal_desc) {
@@ -201,7 +223,7 @@ void mha_run(const blt_tensor *input, const blt_tensor *weight_qkv, const blt_te
             p.head.is_causal = mc == NULL && config->is_causal;
         }
     }
-    blt_attention_batch_hip(pr.data(), H);
+    blt_attention_batch_hip(pr.data(), pr.size());
 
     /* 3. output projection (+ residual) */
     std::memset(&g, 0, sizeof(g));

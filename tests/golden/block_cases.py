@@ -127,7 +127,8 @@ def diffusion_inputs(name):
 def transformer_case(rs, T, E, H, hidden, mask):
     """Seeded inputs of one RMSNorm + SwiGLU block and its mask configuration: "causal" (the
     decoder's), "window" (causal + sliding window), "docs" (document-causal: the patch transformer's,
-    csrc/models/global_transformer.c:19-33), "docs_window" (the local encoder's)."""
+    csrc/models/global_transformer.c:19-33), "docs_window" (the local encoder's); "docs_edge[_window]": document boundaries at the edges of what
+    csrc/ops/mask_builder_cpu.c:10-19 accepts."""
     x = rs.randn(T, E).astype(np.float32)
     w = {"norm1": (1.0 + 0.1 * rs.randn(E)).astype(np.float32), "qkv": (rs.randn(E, 3 * E) / np.sqrt(E)).astype(np.float32),
          "proj": (rs.randn(E, E) / np.sqrt(E)).astype(np.float32), "norm2": (1.0 + 0.1 * rs.randn(E)).astype(np.float32),
@@ -142,6 +143,8 @@ def transformer_case(rs, T, E, H, hidden, mask):
         cfg.sliding_window = max(2, T // 5)
     if "docs" in mask:
         cuts = sorted(set(int(v) for v in rs.randint(1, T, size=3))) if T > 4 else [1]
+        if "edge" in mask:  # a boundary at 0, a repeated one, one-row documents, a boundary past the end
+            cuts = [0, 1, 1, 5, T - 1, T + 3]
         keep = abi.size_array(cuts)
         cfg.doc_boundaries, cfg.num_docs = keep, len(cuts) + 1
     return x, w, cfg, keep

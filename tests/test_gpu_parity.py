@@ -1346,7 +1346,8 @@ def test_kv_decode_step_single_sequence(case, impl, oracle, dev):
 
 @pytest.mark.parametrize("impl", IMPLS)
 @pytest.mark.parametrize("shape", [(2, 8, 2, 12, "causal"), (33, 32, 4, 48, "window"), (70, 48, 3, 64, "docs"),
-                                   (40, 64, 2, 96, "docs_window"),
+                                   (40, 64, 2, 96, "docs_window"), (64, 64, 2, 96, "docs_edge"),
+                                   (200, 128, 4, 256, "docs_edge_window"),
                                    (512, 128, 4, 512, "docs_window"),    # a byte layer of the local encoder at C1 size
                                    (128, 512, 8, 1024, "docs"),          # a layer of the patch transformer at C2 size
                                    (300, 256, 4, 768, "causal")])
