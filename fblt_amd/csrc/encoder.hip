@@ -25,6 +25,14 @@
 #include <cstring>
 #include <vector>
 
+/* blt_cross_attention_forward_hip with the steps either side of it in a caller's layer folded in
+ * (mha.hip): norm_w, when set, is the weight of the RMSNorm that makes query_in's rows the queries
+ * (taken inside the query projection), residual [rows, embed] is added to the projected output. */
+void blt_cross_attention_run(const blt_tensor *query_in, const blt_tensor *kv_in,
+                             const blt_cross_attention_weights *weights, blt_tensor *output,
+                             const blt_cross_attention_config *config, blt_arena *arena, const float *norm_w,
+                             const float *residual);
+
 namespace {
 
 constexpr int IDX_PER_LAUNCH = 512; /* index entries a launch carries in its arguments */
@@ -349,18 +357,17 @@ extern "C" void blt_local_encoder_forward_hip(const blt_local_encoder *model, co
         h = h_next;
         if (!blt_local_cross_attn_fires(cfg.cross_attn_placement, cfg.cross_attn_all_layers, cfg.num_layers, l)) continue;
 
+        /* P_{l+1} = P_l + cross(RMSNorm(P_l), h) (local_encoder.c:255-272), the norm inside the query
+         * projection and the sum in the epilogue of the output projection: three launches */
         blt_tensor p_rows = view_2d(p.data, num_patches * k, E);
-        blt_tensor query = blt_tensor_create_uninit(arena, sub_shape, 2, BLT_DTYPE_FP32);
-        blt_rmsnorm_forward_hip(&p_rows, &s->cross_norm_weight, &query);
         blt_cross_attention_weights xw;
         xw.weight_q = &s->cross_weight_q, xw.weight_k = &s->cross_weight_k, xw.weight_v = &s->cross_weight_v;
         xw.weight_proj = &s->cross_weight_proj;
-        blt_tensor cross_out = blt_tensor_create_uninit(arena, sub_shape, 2, BLT_DTYPE_FP32);
-        blt_cross_attention_forward_hip(&query, &h, &xw, &cross_out, &cross_cfg, arena);
-        blt_tensor cross_rows = view_2d(cross_out.data, num_patches, patch_dim);
         blt_tensor p_next = l == last_cross ? view_2d(patch_out->data, num_patches, patch_dim)
                                             : blt_tensor_create_uninit(arena, patch_shape, 2, BLT_DTYPE_FP32);
-        blt_add_hip(&p, &cross_rows, &p_next);
+        blt_tensor next_rows = view_2d(p_next.data, num_patches * k, E);
+        blt_cross_attention_run(&p_rows, &h, &xw, &next_rows, &cross_cfg, arena,
+                                (const float *)s->cross_norm_weight.data, (const float *)p.data);
         p = p_next;
     }
     if (last_cross == cfg.num_layers) /* no cross block fired: P_0 is the result */

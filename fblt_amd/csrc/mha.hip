@@ -353,9 +353,10 @@ extern "C" void blt_transformer_forward_hip(const blt_tensor *input, const blt_t
  *
  * A patch that owns no byte is fatal, as in the reference's mask builder.
  */
-extern "C" void blt_cross_attention_forward_hip(const blt_tensor *query_in, const blt_tensor *kv_in,
-                                                const blt_cross_attention_weights *weights, blt_tensor *output,
-                                                const blt_cross_attention_config *config, blt_arena *arena) {
+void blt_cross_attention_run(const blt_tensor *query_in, const blt_tensor *kv_in,
+                             const blt_cross_attention_weights *weights, blt_tensor *output,
+                             const blt_cross_attention_config *config, blt_arena *arena, const float *norm_w,
+                             const float *residual) {
     BLT_REQUIRE(config != NULL && arena != NULL, "blt_cross_attention: config and arena cannot be NULL");
     BLT_REQUIRE(config->mask_config != NULL,
                 "blt_cross_attention: mask_config is required (block-diagonal patch mask)");
@@ -396,6 +397,17 @@ extern "C" void blt_cross_attention_forward_hip(const blt_tensor *query_in, cons
     g.m = (uint32_t)P, g.k = (uint32_t)E, g.n = (uint32_t)E;
     g.lda = g.ldb = g.ldo = (uint32_t)E;
     MatmulArgs gkv = g;
+    g.norm_w = norm_w; /* the query rows only */
+    if (norm_w != nullptr && !matmul_takes_norm(g)) { /* shapes the fused norm does not cover: a pass of its own */
+        blt_tensor normed = blt_tensor_create_uninit(arena, query_in->shape, 2, BLT_DTYPE_FP32);
+        blt_tensor wt;
+        std::memset(&wt, 0, sizeof(wt));
+        wt.data = const_cast<float *>(norm_w), wt.ndim = 1, wt.shape[0] = E, wt.strides[0] = 1, wt.numel = E;
+        wt.dtype = BLT_DTYPE_FP32, wt.backend = BLT_BACKEND_HIP, wt.is_view = true;
+        blt_rmsnorm_forward_hip(query_in, &wt, &normed);
+        g.a = (const float *)normed.data;
+        g.norm_w = nullptr;
+    }
     gkv.a = (const float *)kv_in->data;
     gkv.b = (const float *)weights->weight_k->data;
     gkv.out = k;
@@ -471,8 +483,15 @@ extern "C" void blt_cross_attention_forward_hip(const blt_tensor *query_in, cons
     g.a = combined;
     g.b = (const float *)weights->weight_proj->data;
     g.out = (float *)output->data;
+    g.residual = residual;
     g.m = (uint32_t)P, g.k = (uint32_t)E, g.n = (uint32_t)E;
     g.lda = g.ldb = g.ldo = (uint32_t)E;
     matmul_f32_launch(g, 0);
     HIP_CHECK_LAUNCH("blt_cross_attention_forward");
+}
+
+extern "C" void blt_cross_attention_forward_hip(const blt_tensor *query_in, const blt_tensor *kv_in,
+                                                const blt_cross_attention_weights *weights, blt_tensor *output,
+                                                const blt_cross_attention_config *config, blt_arena *arena) {
+    blt_cross_attention_run(query_in, kv_in, weights, output, config, arena, nullptr, nullptr);
 }
