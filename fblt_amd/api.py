@@ -146,6 +146,13 @@ SYMBOLS = {
     "blt_local_encoder_forward": (None, [C.POINTER(abi.BltLocalEncoder), C.POINTER(abi.BltTensor),
                                          C.POINTER(abi.BltPatchInfo), C.c_size_t, abi.c_size_p, C.c_size_t,
                                          C.POINTER(abi.BltTensor), C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)]),
+    "blt_local_decoder_forward_ext_hip": (None, [C.POINTER(abi.BltLocalDecoder), C.POINTER(abi.BltTensor),
+                                                 C.POINTER(abi.BltTensor), C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t,
+                                                 C.c_int, C.POINTER(abi.BltTensor), C.POINTER(abi.BltArena)]),
+    "blt_local_decoder_forward_ext": (None, [C.POINTER(abi.BltLocalDecoder), C.POINTER(abi.BltTensor),
+                                             C.POINTER(abi.BltTensor), C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p,
+                                             C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.POINTER(abi.BltTensor),
+                                             C.c_void_p, C.POINTER(abi.BltArena)]),
     "blt_local_encoder_forward_hip": (None, [C.POINTER(abi.BltLocalEncoder), C.POINTER(abi.BltTensor),
                                              C.POINTER(abi.BltPatchInfo), C.c_size_t, abi.c_size_p, C.c_size_t,
                                              C.POINTER(abi.BltTensor), C.POINTER(abi.BltTensor),

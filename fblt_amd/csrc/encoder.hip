@@ -343,7 +343,6 @@ extern "C" void blt_local_encoder_forward_hip(const blt_local_encoder *model, co
     size_t last_cross = cfg.num_layers; /* none */
     for (size_t l = 0; l < cfg.num_layers; l++)
         if (blt_local_cross_attn_fires(cfg.cross_attn_placement, cfg.cross_attn_all_layers, cfg.num_layers, l)) last_cross = l;
-    const size_t sub_shape[2] = {num_patches * k, E};
     for (size_t l = 0; l < cfg.num_layers; l++) {
         const blt_local_layer_storage *s = &model->layers[l];
         blt_transformer_weights w;
@@ -375,4 +374,116 @@ extern "C" void blt_local_encoder_forward_hip(const blt_local_encoder *model, co
                              num_patches * patch_dim, 1, num_patches * patch_dim);
     /* the host index arrays of the masks are consumed by the calls above (ranges are staged, dense
      * masks are built before the attention launch is issued): nothing outlives this call */
+}
+
+/*
+ * blt_local_decoder_forward_ext without D_0 options and loss (reference: csrc/models/
+ * local_decoder.c:233-351).  D_0 is byte_hidden_in itself; per layer B = D + cross(RMSNorm(D),
+ * patch sub-tokens) where the cross block fires (norm inside the query projection, sum in the
+ * output projection's epilogue: three launches), D = byte block(B) under the causal, windowed,
+ * per-document mask (five launches); logits = D_final * lm_head.  A byte reads the latent the
+ * paper's rule gives it (blt_patch_decoder_latent_at, the last byte of the window its own patch's
+ * when trailing_closed): one sub-token group per row, so the cross mask travels as key ranges.
+ */
+extern "C" void blt_local_decoder_forward_ext_hip(const blt_local_decoder *model, const blt_tensor *byte_hidden_in,
+                                                  const blt_tensor *patch_in, const blt_patch_info *patches,
+                                                  size_t num_patches, const size_t *doc_boundaries, size_t num_docs,
+                                                  int trailing_closed, blt_tensor *logits_out, blt_arena *arena) {
+    BLT_REQUIRE(model != NULL && byte_hidden_in != NULL && patch_in != NULL && patches != NULL && arena != NULL,
+                "blt_local_decoder_forward_ext: model, byte_hidden_in, patch_in, patches and arena cannot be NULL");
+    BLT_REQUIRE(logits_out != NULL, "blt_local_decoder_forward_ext: logits_out cannot be NULL");
+    BLT_REQUIRE(arena->backend == BLT_BACKEND_HIP, "blt_local_decoder_forward_ext: HIP implementation needs a device arena");
+    const blt_local_decoder_config &cfg = model->config;
+    const size_t E = cfg.embed_dim, V = cfg.vocab_size;
+    BLT_REQUIRE(cfg.num_heads != 0 && E % cfg.num_heads == 0 && (E / cfg.num_heads) % 2 == 0,
+                "blt_local_decoder_forward_ext: embed_dim / num_heads must be an even head width");
+    BLT_REQUIRE(byte_hidden_in->ndim == 2 && byte_hidden_in->dtype == BLT_DTYPE_FP32 && byte_hidden_in->shape[1] == E &&
+                    byte_hidden_in->backend == BLT_BACKEND_HIP,
+                "blt_local_decoder_forward_ext: byte_hidden_in must be [seq_len, embed_dim] FP32");
+    const size_t seq_len = byte_hidden_in->shape[0];
+    BLT_REQUIRE(seq_len >= 1 && seq_len <= cfg.max_seq_len,
+                "blt_local_decoder_forward_ext: seq_len must be in [1, max_seq_len]");
+    BLT_REQUIRE(num_patches >= 1, "blt_local_decoder_forward_ext: num_patches must be >= 1");
+    const size_t patch_dim = cfg.patch_dim == 0 ? E : cfg.patch_dim;
+    BLT_REQUIRE(patch_dim % E == 0, "blt_local_decoder_forward_ext: patch_dim must be a multiple of embed_dim");
+    const size_t k = patch_dim / E, half = E / cfg.num_heads / 2;
+    check_2d(patch_in, num_patches, patch_dim, "blt_local_decoder_forward_ext: patch_in must be [num_patches, patch_dim] FP32");
+    check_2d(logits_out, seq_len, V, "blt_local_decoder_forward_ext: logits_out must be [seq_len, vocab_size] FP32");
+    check_2d(&model->lm_head_weight, E, V, "blt_local_decoder_forward_ext: lm_head_weight must be [embed_dim, vocab_size] FP32");
+    check_2d(&model->rope_cos_cache, cfg.max_seq_len, half, "blt_local_decoder_forward_ext: rope_cos_cache");
+    check_2d(&model->rope_sin_cache, cfg.max_seq_len, half, "blt_local_decoder_forward_ext: rope_sin_cache");
+    size_t covered = 0;
+    for (size_t j = 0; j < num_patches; j++) { /* patches tile [0, seq_len) (patch_pool_cpu.c:98-118) */
+        BLT_REQUIRE(patches[j].start_idx == covered && patches[j].length >= 1,
+                    "blt_local_decoder_forward_ext: patches must tile the window without gaps");
+        covered += patches[j].length;
+    }
+    BLT_REQUIRE(covered == seq_len, "blt_local_decoder_forward_ext: patches must tile [0, seq_len) exactly");
+
+    /* ---- masks (local_decoder.c:64-121): host metadata ---- */
+    std::vector<size_t> byte_groups(seq_len), kv_groups(num_patches * k);
+    for (size_t i = 0; i < seq_len; i++) byte_groups[i] = blt_patch_decoder_latent_at(patches, num_patches, i);
+    if (trailing_closed) byte_groups[seq_len - 1] = num_patches - 1;
+    for (size_t j = 0; j < num_patches * k; j++) kv_groups[j] = j / k;
+    blt_mask_config local_mask, cross_mask;
+    std::memset(&local_mask, 0, sizeof(local_mask));
+    std::memset(&cross_mask, 0, sizeof(cross_mask));
+    local_mask.seq_len_q = local_mask.seq_len_kv = seq_len;
+    local_mask.sliding_window = cfg.local_window;
+    local_mask.doc_boundaries = doc_boundaries;
+    local_mask.num_docs = num_docs;
+    local_mask.is_causal = true;
+    cross_mask.seq_len_q = seq_len;
+    cross_mask.seq_len_kv = num_patches * k;
+    cross_mask.query_group_ids = byte_groups.data();
+    cross_mask.kv_group_ids = kv_groups.data();
+    cross_mask.bidirectional_within_group = true;
+    blt_tensor cos_view = view_2d(model->rope_cos_cache.data, seq_len, half);
+    blt_tensor sin_view = view_2d(model->rope_sin_cache.data, seq_len, half);
+    blt_transformer_config layer_cfg;
+    std::memset(&layer_cfg, 0, sizeof(layer_cfg));
+    layer_cfg.attn_config.embed_dim = E;
+    layer_cfg.attn_config.num_heads = cfg.num_heads;
+    layer_cfg.attn_config.is_causal = true;
+    layer_cfg.attn_config.use_rope = true;
+    layer_cfg.attn_config.rope_theta = cfg.rope_theta;
+    layer_cfg.attn_config.rope_cos_cache = &cos_view;
+    layer_cfg.attn_config.rope_sin_cache = &sin_view;
+    layer_cfg.attn_config.mask_config = &local_mask;
+    layer_cfg.hidden_dim = cfg.hidden_dim;
+    layer_cfg.norm_type = BLT_NORM_RMSNORM;
+    layer_cfg.activation_type = BLT_ACTIVATION_SWIGLU;
+    blt_cross_attention_config cross_cfg;
+    std::memset(&cross_cfg, 0, sizeof(cross_cfg));
+    cross_cfg.embed_dim = E;
+    cross_cfg.patch_dim = patch_dim;
+    cross_cfg.split_mode = k == 1 ? BLT_CROSS_ATTN_NO_SPLIT : BLT_CROSS_ATTN_SPLIT_KV;
+    cross_cfg.num_heads = cfg.cross_attn_heads;
+    cross_cfg.mask_config = &cross_mask;
+
+    /* ---- layers ---- */
+    const size_t byte_shape[2] = {seq_len, E};
+    blt_tensor latents = view_2d(patch_in->data, num_patches * k, E);
+    blt_tensor d = view_2d(byte_hidden_in->data, seq_len, E);
+    for (size_t l = 0; l < cfg.num_layers; l++) {
+        blt_local_layer_storage *s = &model->layers[l];
+        blt_tensor b = d;
+        if (blt_local_cross_attn_fires(cfg.cross_attn_placement, cfg.cross_attn_all_layers, cfg.num_layers, l)) {
+            blt_cross_attention_weights xw;
+            xw.weight_q = &s->cross_weight_q, xw.weight_k = &s->cross_weight_k, xw.weight_v = &s->cross_weight_v;
+            xw.weight_proj = &s->cross_weight_proj;
+            b = blt_tensor_create_uninit(arena, byte_shape, 2, BLT_DTYPE_FP32);
+            blt_cross_attention_run(&d, &latents, &xw, &b, &cross_cfg, arena, (const float *)s->cross_norm_weight.data,
+                                    (const float *)d.data);
+        }
+        blt_transformer_weights w;
+        std::memset(&w, 0, sizeof(w));
+        w.norm1_weight = &s->norm1_weight, w.norm2_weight = &s->norm2_weight;
+        w.attn_qkv_w = &s->attn_qkv_w, w.attn_proj_w = &s->attn_proj_w;
+        w.ffn_up_w = &s->ffn_up_w, w.ffn_gate_w = &s->ffn_gate_w, w.ffn_down_w = &s->ffn_down_w;
+        blt_tensor d_next = blt_tensor_create_uninit(arena, byte_shape, 2, BLT_DTYPE_FP32);
+        blt_transformer_forward_hip(&b, &w, &d_next, &layer_cfg, arena);
+        d = d_next;
+    }
+    blt_matmul_hip(&d, &model->lm_head_weight, logits_out);
 }

@@ -454,6 +454,25 @@ void blt_local_encoder_forward(const blt_local_encoder *model, const blt_tensor 
                                   byte_hidden_out, arena);
 }
 
+void blt_local_decoder_forward_ext(const blt_local_decoder *model, const blt_tensor *byte_hidden_in,
+                                   const blt_tensor *patch_in, const blt_patch_info *patches, size_t num_patches,
+                                   const blt_tensor *bytes_in, const blt_tensor *targets, const size_t *doc_boundaries,
+                                   size_t num_docs, const blt_local_decoder_d0_opts *d0_opts, int trailing_closed,
+                                   blt_tensor *logits_out, blt_tensor *loss_out, blt_arena *arena) {
+    (void)targets;
+    BLT_REQUIRE(logits_out != NULL, "blt_local_decoder_forward_ext: logits_out cannot be NULL");
+    BLT_REQUIRE(loss_out != NULL || bytes_in == NULL,
+                "blt_local_decoder_forward_ext: bytes_in is only used for the loss; pass NULL when loss_out is NULL");
+    BLT_DEVICE_ONLY(logits_out->backend, "blt_local_decoder_forward_ext");
+    BLT_REQUIRE(loss_out == NULL,
+                "blt_local_decoder_forward_ext: the HIP backend runs the inference form only (loss_out must be NULL)");
+    BLT_REQUIRE(d0_opts == NULL || d0_opts->d0_mode == BLT_D0_HFINAL,
+                "blt_local_decoder_forward_ext: D_0 modes other than BLT_D0_HFINAL go through "
+                "blt_local_decoder_forward_diffusion_infer on the HIP backend");
+    blt_local_decoder_forward_ext_hip(model, byte_hidden_in, patch_in, patches, num_patches, doc_boundaries, num_docs,
+                                      trailing_closed, logits_out, arena);
+}
+
 void blt_add(const blt_tensor *a, const blt_tensor *b, blt_tensor *out) {
     BLT_REQUIRE(a != NULL, "blt_add: input tensors must be FP32 with matching element count");
     BLT_DEVICE_ONLY(a->backend, "blt_add");

@@ -280,6 +280,13 @@ typedef enum {
     BLT_D0_LEARNED     /* block rows read d0_embed_weight[token] */
 } blt_d0_mode;
 
+/* csrc/models/local_decoder.h:48-54 */
+typedef struct {
+    blt_d0_mode d0_mode;
+    size_t num_hfinal_rows;
+    const uint32_t *d0_extra_tokens;
+} blt_local_decoder_d0_opts;
+
 #define BLT_MASK_TOKEN_ID 256u /* csrc/models/block_diffusion.h:32 */
 
 /* csrc/models/block_diffusion.h:37-86: the block section behind a clean prefix.  The inference

@@ -164,6 +164,12 @@ void blt_transformer_forward_hip(const blt_tensor *input, const blt_transformer_
  * weights, outputs and the arena are device memory; patches, doc_boundaries are HOST arrays.
  * Unlike the reference's body on a device arena, sub-token splits (patch_dim = k * embed_dim,
  * k > 1) work: the expanded group ids are host memory here. */
+/* csrc/models/local_decoder.c:233-351 on the device: per layer the cross block (when it fires)
+ * in three launches and the byte block in five, then the LM head. */
+void blt_local_decoder_forward_ext_hip(const blt_local_decoder *model, const blt_tensor *byte_hidden_in,
+                                       const blt_tensor *patch_in, const blt_patch_info *patches, size_t num_patches,
+                                       const size_t *doc_boundaries, size_t num_docs, int trailing_closed,
+                                       blt_tensor *logits_out, blt_arena *arena);
 void blt_local_encoder_forward_hip(const blt_local_encoder *model, const blt_tensor *bytes_in,
                                    const blt_patch_info *patches, size_t num_patches, const size_t *doc_boundaries,
                                    size_t num_docs, blt_tensor *patch_out, blt_tensor *byte_hidden_out,
@@ -250,6 +256,14 @@ void blt_cross_attention_forward(const blt_tensor *query_in, const blt_tensor *k
 void blt_transformer_forward(const blt_tensor *input, const blt_transformer_weights *weights, blt_tensor *output,
                              const blt_transformer_config *config, blt_arena *arena);
 /* csrc/models/local_encoder.h:71-73 */
+/* csrc/models/local_decoder.h:112-125 (local_decoder.c:233-361), the inference form: loss_out
+ * must be NULL (the loss is a training op) and d0_opts NULL or BLT_D0_HFINAL (block rows with
+ * their own D_0 go through blt_local_decoder_forward_diffusion_infer). */
+void blt_local_decoder_forward_ext(const blt_local_decoder *model, const blt_tensor *byte_hidden_in,
+                                   const blt_tensor *patch_in, const blt_patch_info *patches, size_t num_patches,
+                                   const blt_tensor *bytes_in, const blt_tensor *targets, const size_t *doc_boundaries,
+                                   size_t num_docs, const blt_local_decoder_d0_opts *d0_opts, int trailing_closed,
+                                   blt_tensor *logits_out, blt_tensor *loss_out, blt_arena *arena);
 void blt_local_encoder_forward(const blt_local_encoder *model, const blt_tensor *bytes_in, const blt_patch_info *patches,
                                size_t num_patches, const size_t *doc_boundaries, size_t num_docs, blt_tensor *patch_out,
                                blt_tensor *byte_hidden_out, blt_arena *arena);

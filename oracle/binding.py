@@ -28,7 +28,7 @@ def build(ref=True):
     if ref and os.path.isdir(os.environ.get("REF_ROOT", "/root/reference")):
         subprocess.check_call(["make", "-s", "-B", "-C", HERE, "ref"])
         if os.path.exists(os.path.join(HERE, "..", "fblt_amd", "lib", "libfblt_hip.so")):
-            subprocess.check_call(["make", "-s", "-C", HERE, "callers", "stack_callers", "model_callers"])
+            subprocess.check_call(["make", "-s", "-C", HERE, "callers", "stack_callers", "model_callers", "model_driver"])
 
 
 def load_oracle():
@@ -358,6 +358,22 @@ def load_ref_model_callers():
         return None
     load_ref()
     lib = C.CDLL(MODEL_CALLERS_SO)
+    _model_entry(lib)
+    return lib
+
+
+MODEL_DRIVER_SO = os.path.join(HERE, "_ref", "libblt_ref_model_driver.so")
+
+
+def load_ref_model_driver():
+    """The reference's whole-model driver and patch transformer alone, compiled unmodified and
+    linked against the HIP library without the reference's encoder and decoder sources: both local
+    models run through the library's own entries (`make -C oracle model_driver`); None where that
+    was never built."""
+    if not os.path.exists(MODEL_DRIVER_SO) or not os.path.exists(REF_SO):
+        return None
+    load_ref()
+    lib = C.CDLL(MODEL_DRIVER_SO)
     _model_entry(lib)
     return lib
 

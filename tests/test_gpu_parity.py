@@ -1276,6 +1276,49 @@ def _decoders(oracle, c, seed):
     return host, device
 
 
+@pytest.mark.parametrize("case", range(len(STEP_CASES)))
+@pytest.mark.parametrize("closed,docs,impl", [(0, [], "public"), (1, [], "twin"), (0, [5, 11], "public"),
+                                              (1, [0, 1, 1, 30], "twin")])
+def test_local_decoder_forward(case, closed, docs, impl, oracle, dev):
+    """The library's own blt_local_decoder_forward_ext (inference form: no loss, D_0 = the encoder's rows) against
+    the restated forward (csrc/models/local_decoder.c:233-351): every decoder configuration of the step tests
+    (sub-token split, window, placements), trailing_closed, document boundaries in the byte mask; through the
+    public name and through the device twin."""
+    import torch
+    from fblt_amd import decoder
+    lib = api.load()
+    c = STEP_CASES[case]
+    host, device = _decoders(oracle, c, 900 + case)
+    rs = np.random.RandomState(900 + case)
+    lengths = [3, 4, 2, 5, 1, 6, 9] if c["max_len"] < 64 else [3, 4, 2, 5, 1, 6, 9, 16, 2, 12]
+    T, P, E, V = sum(lengths), len(lengths), c["E"], c["V"]
+    patches = decoder.patch_table(lengths)
+    hidden = rs.randn(T, E).astype(np.float32)
+    patch_in = rs.randn(P, E * c["k"]).astype(np.float32)
+    bounds = abi.size_array(docs) if docs else None
+    num_docs = len(docs) + 1 if docs else 0
+    want = np.zeros((T, V), dtype=np.float32)
+    assert oracle.orc_local_decoder_forward(host.ptr, binding.fptr(hidden.reshape(-1)), T,
+                                            binding.fptr(patch_in.reshape(-1)), patches, P, bounds, num_docs, closed,
+                                            binding.fptr(want.reshape(-1))) == 0
+    th, tp = torch.from_numpy(hidden).cuda(), torch.from_numpy(patch_in).cuda()
+    tl = torch.full((T, V), 7.0, dtype=torch.float32, device="cuda")
+    vh, vp, vl = _dev_tensor(th), _dev_tensor(tp), _dev_tensor(tl)
+    arena = lib.blt_arena_create(64 << 20, abi.BLT_BACKEND_HIP)
+    try:
+        if impl == "public":
+            lib.blt_local_decoder_forward_ext(device.ptr, C.byref(vh), C.byref(vp), patches, P, None, None, bounds,
+                                              num_docs, None, closed, C.byref(vl), None, arena)
+        else:
+            lib.blt_local_decoder_forward_ext_hip(device.ptr, C.byref(vh), C.byref(vp), patches, P, bounds, num_docs,
+                                                  closed, C.byref(vl), arena)
+        lib.blt_backend_pass_sync_hip()
+    finally:
+        lib.blt_arena_destroy(arena)
+    assert np.isfinite(want).all() and np.abs(want).max() > 1e-3
+    assert_close(tl.cpu().numpy(), want, "decoder forward case %d closed %d docs %s" % (case, closed, docs))
+
+
 def _tier(lib, cache, name, layer, rows, E):
     out = np.empty((rows, E), dtype=np.float32)
     lib.blt_hip_memcpy_d2h(out.ctypes.data, getattr(cache.contents, name)[layer].data, out.nbytes)
@@ -1825,7 +1868,7 @@ def test_local_encoder_forward(name, impl, oracle, dev):
 
 
 
-@pytest.mark.parametrize("driver", ["reference_encoder", "library_encoder"])
+@pytest.mark.parametrize("driver", ["reference_encoder", "library_encoder", "library_stages"])
 @pytest.mark.parametrize("name", ["model_T96", "model_T200_docs_window"])
 def test_model_forward_on_the_library(name, driver, oracle, dev):
     """The reference's whole-model inference forward -- blt_model_encode + blt_model_decode of
@@ -1836,11 +1879,13 @@ def test_model_forward_on_the_library(name, driver, oracle, dev):
     against the composition of the restated stages, which tests/test_oracle_vs_ref.py pins bit for
     bit against the reference's CPU build.  `library_encoder`: the same driver built without the
     reference's encoder sources, so that blt_model_encode runs this library's own
-    blt_local_encoder_forward."""
+    blt_local_encoder_forward; `library_stages`: without its decoder sources either
+    (blt_local_decoder_forward_ext is the library's too)."""
     from fblt_amd import decoder
     from tests import model_runs
     lib = api.load()
-    stack_lib = binding.load_ref_stack_callers() if driver == "reference_encoder" else binding.load_ref_model_callers()
+    stack_lib = {"reference_encoder": binding.load_ref_stack_callers, "library_encoder": binding.load_ref_model_callers,
+                 "library_stages": binding.load_ref_model_driver}[driver]()
     if stack_lib is None or not hasattr(stack_lib, "blt_model_encode"):
         pytest.skip("oracle/_ref does not hold the model driver build (needs the reference sources)")
     args = model_runs.inputs(name)

@@ -132,6 +132,8 @@ int main(void) {
     O(blt_transformer_config, norm_type); O(blt_transformer_config, activation_type); O(blt_transformer_config, use_bf16);
     S(blt_block_batch); O(blt_block_batch, t); O(blt_block_batch, tokens); O(blt_block_batch, positions);
     O(blt_block_batch, groups); O(blt_block_batch, loss_scale); O(blt_block_batch, trailing_closed);
+    S(blt_local_decoder_d0_opts); O(blt_local_decoder_d0_opts, num_hfinal_rows);
+    O(blt_local_decoder_d0_opts, d0_extra_tokens);
     S(blt_hash_ngram_config); O(blt_hash_ngram_config, num_ngram_sizes); O(blt_hash_ngram_config, per_ngram_vocab);
     O(blt_hash_ngram_config, hash_prime); O(blt_hash_ngram_config, normalize); O(blt_hash_ngram_config, embed_dim);
     S(blt_hash_ngram_weights); O(blt_hash_ngram_weights, num_tables);
