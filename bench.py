@@ -782,6 +782,86 @@ def bench_encoder(steps, warmup, cpu_budget_s):
     return res
 
 
+def bench_decoder_forward(steps, warmup, cpu_budget_s, T=512, L=2, E=128, H=4, hidden=512, V=256):
+    """The local decoder's plain forward in its inference form (csrc/models/local_decoder.c:233-351:
+    D_0 = the encoder's rows, cross block and byte block per layer, LM head) at C1's caller size:
+    this library's blt_local_decoder_forward_ext, and the restated forward on one host core."""
+    import ctypes as C
+    import numpy as np
+    import torch
+    from fblt_amd import abi, api, decoder
+    lib = api.load()
+    hd, half = E // H, E // H // 2
+    rs = np.random.RandomState(41)
+    lengths = []
+    while sum(lengths) < T:
+        lengths.append(int(min(T - sum(lengths), rs.poisson(3) + 1)))
+    P = len(lengths)
+    weights = decoder.random_weights(E, hidden, L, V, 43)
+    view = lambda t: abi.tensor_view(t.data_ptr(), tuple(t.shape), abi.BLT_BACKEND_HIP)
+    cos, sin = torch.zeros((T, half), device="cuda"), torch.zeros((T, half), device="cuda")
+    vc, vs = view(cos), view(sin)
+    rcfg = abi.BltRopeConfig(500000.0, hd)
+    lib.blt_rope_precompute(T, C.byref(rcfg), C.byref(vc), C.byref(vs))
+    tables = (cos.cpu().numpy(), sin.cpu().numpy())
+    args = (E, H, H, hidden, V, T)
+    dev = decoder.bind(weights, *tables, abi.BLT_BACKEND_HIP, decoder.device_place, *args)
+    patches = decoder.patch_table(lengths)
+    hidden_in = rs.randn(T, E).astype(np.float32)
+    latents = rs.randn(P, E).astype(np.float32)
+    th, tp = torch.from_numpy(hidden_in).cuda(), torch.from_numpy(latents).cuda()
+    tl = torch.zeros((T, V), device="cuda")
+    vh, vp, vl = view(th), view(tp), view(tl)
+    arena = lib.blt_arena_create(256 << 20, abi.BLT_BACKEND_HIP)
+
+    def run(count):
+        for _ in range(count):
+            arena.contents.offset = 0
+            lib.blt_local_decoder_forward_ext(dev.ptr, C.byref(vh), C.byref(vp), patches, P, None, None, None, 0, None, 0,
+                                              C.byref(vl), None, arena)
+    steps = max(10, steps // 5)
+    run(warmup)
+    lib.blt_backend_pass_sync_hip()
+    lib.blt_hip_profile_begin()
+    run(steps)
+    lib.blt_backend_pass_sync_hip()
+    prof = api.profile_end()
+    t0 = time.perf_counter()
+    run(steps)
+    lib.blt_backend_pass_sync_hip()
+    wall = (time.perf_counter() - t0) / steps
+    lib.blt_arena_destroy(arena)
+    per_kernel = {k: v[1] * 1e3 / steps for k, v in prof.items()}
+    kernel_us = sum(per_kernel.values())
+    flops = L * (2.0 * T * (E * 3 * E + E * E + 3 * E * hidden) + 4.0 * E * T * (T + 1) / 2 +
+                 2.0 * (T * 2 * E * E + P * 2 * E * E) + 4.0 * E * T) + 2.0 * T * E * V
+    nbytes = 4.0 * (L * (E * 3 * E + E * E + 3 * E * hidden + 4 * E * E + 6 * T * E) + E * V + T * V)
+    res = {"workload": "local decoder forward: %d bytes, %d patches, %d layers (cross block in each), E=%d, H=%d, "
+                       "hidden=%d, V=%d" % (T, P, L, E, H, hidden, V),
+           "entry": "blt_local_decoder_forward_ext", "kernel": "+".join(sorted(per_kernel)),
+           "launches_per_step": sum(v[0] for v in prof.values()) / steps, "tokens_per_step": T, "us_per_step": wall * 1e6,
+           "kernel_us_avg": kernel_us, "kernel_us_min": min(per_kernel.values()), "per_kernel_us": per_kernel,
+           "tokens_per_s": T / wall, "flops": flops, "bytes": nbytes,
+           "roofline_hbm": roofline("hbm", nbytes, kernel_us * 1e-6), "roofline_mfma": roofline("mfma", flops, kernel_us * 1e-6)}
+    res["roofline"] = res["roofline_mfma"]
+    if cpu_budget_s > 0:
+        from oracle import binding
+        orc = binding.load_oracle()
+        host = decoder.bind(weights, *tables, abi.BLT_BACKEND_CPU, decoder.host_place, *args)
+        out = np.zeros((T, V), dtype=np.float32)
+        t0, passes = time.perf_counter(), 0
+        while passes == 0 or time.perf_counter() - t0 < cpu_budget_s:
+            assert orc.orc_local_decoder_forward(host.ptr, binding.fptr(hidden_in.reshape(-1)), T,
+                                                 binding.fptr(latents.reshape(-1)), patches, P, None, 0, 0,
+                                                 binding.fptr(out.reshape(-1))) == 0
+            passes += 1
+        dt = (time.perf_counter() - t0) / passes
+        res["cpu_baseline"] = {"value": T / dt, "unit": "tokens/s", "cores": 1, "kind": "port",
+                               "sample": "%d passes of the restated forward, %.1f s" % (passes, dt * passes),
+                               "ms_per_pass": dt * 1e3}
+    return res
+
+
 def bench_draft_pass(steps, warmup, cpu_budget_s, N=400, B=8, L=2, E=128, H=4, hidden=512, V=256):
     """One denoising pass of the reference's draft loop (csrc/infer/block_generation.c:156-266: one
     sequence, N clean bytes, a block of B [MASK] rows on the last latent) three ways: the reference's
@@ -1125,6 +1205,8 @@ def main():
         log("draft_pass", json.dumps(others["draft_pass"]))
         others["encoder"] = bench_encoder(K, W, 0.0 if args.no_cpu else 2.0 * cs)
         log("encoder", json.dumps(others["encoder"]))
+        others["decoder_forward"] = bench_decoder_forward(K, W, 0.0 if args.no_cpu else 2.0 * cs)
+        log("decoder_forward", json.dumps(others["decoder_forward"]))
 
     # the dense-mask builders the callers still use
     if want("masks"):
@@ -1200,7 +1282,7 @@ def compact_line(head, others, cpu_head, K, W, detail_path):
                         "c5_B16_b128_L2048", "c5_B16_b128_L2048_host_lens") if k in others}
     # whole decoder step (all layers + LM head): [launches per step, device us, wall us]
     steps_ = {k: [others[k]["launches_per_step"], _sig(others[k]["kernel_us_avg"]), _sig(others[k]["us_per_step"])]
-              for k in ("decode_step", "decode_step_b1", "draft_pass", "encoder") if k in others}
+              for k in ("decode_step", "decode_step_b1", "draft_pass", "encoder", "decoder_forward") if k in others}
     if "reference_call" in others.get("draft_pass", {}):   # the reference's call (prefix recomputed per pass) beside the cached block step
         c = others["draft_pass"]["reference_call"]
         steps_["draft_pass_reference_call"] = [c["launches_per_pass"], _sig(c["kernel_us_per_pass"]),
