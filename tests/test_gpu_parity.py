@@ -1742,6 +1742,36 @@ def test_graph_replay_of_a_plan_and_a_decode_layer(oracle, dev):
     lib.blt_hip_graph_destroy(graph)
 
 
+def test_sliced_product_replays_in_a_graph(dev):
+    """A product whose K is split over workgroups, recorded into a graph after an eager run has sized its sums and
+    tickets: three replays, each with an eager sliced product of another shape in between (same tickets), give the
+    eager bits."""
+    import torch
+    lib = api.load()
+    torch.manual_seed(9)
+    a, b = torch.randn(118, 2048, device="cuda"), torch.randn(2048, 512, device="cuda") / 45.0
+    a2, b2 = torch.randn(64, 4096, device="cuda"), torch.randn(4096, 256, device="cuda") / 64.0
+    o, o2 = torch.zeros(118, 512, device="cuda"), torch.zeros(64, 256, device="cuda")
+    va, vb, vo, va2, vb2, vo2 = (_dev_tensor(t) for t in (a, b, o, a2, b2, o2))
+    lib.blt_matmul(C.byref(va), C.byref(vb), C.byref(vo))          # eager: scratch gets allocated here
+    lib.blt_matmul(C.byref(va2), C.byref(vb2), C.byref(vo2))
+    lib.blt_backend_pass_sync_hip()
+    want, want2 = o.cpu().numpy().copy(), o2.cpu().numpy().copy()
+    assert_close(want, (a.double() @ b.double()).float().cpu().numpy(), "sliced product")
+    lib.blt_hip_capture_begin()
+    lib.blt_matmul(C.byref(va), C.byref(vb), C.byref(vo))
+    graph = lib.blt_hip_capture_end()
+    for _ in range(3):
+        o.zero_()
+        o2.zero_()
+        torch.cuda.synchronize()
+        lib.blt_hip_graph_launch(graph)
+        lib.blt_matmul(C.byref(va2), C.byref(vb2), C.byref(vo2))
+        lib.blt_backend_pass_sync_hip()
+        assert o.cpu().numpy().tobytes() == want.tobytes() and o2.cpu().numpy().tobytes() == want2.tobytes()
+    lib.blt_hip_graph_destroy(graph)
+
+
 def test_library_follows_the_chosen_stream(oracle, dev):
     """blt_hip_set_stream: launches go to the caller's stream; results are the null-stream results."""
     import torch
