@@ -847,7 +847,11 @@ void matmul_f32_launch(const MatmulArgs &g, hipStream_t s) {
         return !(e && atoi(e) == 64);
     }();
     const uint32_t tx = (g.n + 2 * TN - 1) / (2 * TN), ty = (g.m + 2 * TM - 1) / (2 * TM);
-    if (big_ok && (uint64_t)tx * ty >= 512u) {
+    static const uint64_t big_from = [] { /* BLT_HIP_MATMUL_BIG_FROM: tuning hook */
+        const char *e = getenv("BLT_HIP_MATMUL_BIG_FROM");
+        return e && *e ? (uint64_t)atoll(e) : (uint64_t)512u;
+    }();
+    if (big_ok && (uint64_t)tx * ty >= big_from) {
         const dim3 grid(tx, ty);
         if (rope) {
             if (vec) launch_mfma<true, true, 2>(grid, s, g);
