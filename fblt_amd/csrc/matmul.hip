@@ -851,7 +851,13 @@ void matmul_f32_launch(const MatmulArgs &g, hipStream_t s) {
         const char *e = getenv("BLT_HIP_MATMUL_BIG_FROM");
         return e && *e ? (uint64_t)atoll(e) : (uint64_t)512u;
     }();
-    if (big_ok && (uint64_t)tx * ty >= big_from) {
+    /* Two large tiles are resident per compute unit, 512 at a time: a last round that fills less
+     * than three eighths of the chip costs more than the large tile gains (576 tiles, 6144 x 512 .
+     * 512 x 1536: 106 us against 92 with the small tile; 640: 106 / 104; 960: 142 / 151) until the
+     * rounds are many. */
+    const uint64_t big_tiles = (uint64_t)tx * ty, last_round = big_tiles % 512u;
+    const bool short_tail = big_tiles < 2048u && last_round != 0u && last_round < 192u;
+    if (big_ok && big_tiles >= big_from && !short_tail) {
         const dim3 grid(tx, ty);
         if (rope) {
             if (vec) launch_mfma<true, true, 2>(grid, s, g);
