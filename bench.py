@@ -71,19 +71,25 @@ def roofline(bound, work, avg_s, traffic=None):
             "traffic": traffic}
 
 
-def step_percentiles(lib, api, one_step, count):
-    """Device time of `count` further steps, one profile per step (kernel durations of the
-    step's launches summed; each step ends with a device sync): mean / p50 / p90 / p99 in us."""
+MIN_SAMPLES = 200   # event-timed launches behind every kernel duration, whatever --steps says
+WARM_MS = 100.0     # back-to-back work before anything at the BASELINE sizes is timed, whatever --warmup says
+
+
+def sample_stats(samples_us):
+    """mean / p50 / p90 / p99 / min / max of per-step device times in us (nearest-rank percentiles)."""
     import numpy as np
-    samples = []
-    for s in range(count):
-        lib.blt_hip_profile_begin()
-        one_step(s)
-        samples.append(sum(v[1] for v in api.profile_end().values()) * 1e3)
-    a = np.sort(np.array(samples))
+    a = np.sort(np.array(samples_us, dtype=np.float64))
     pick = lambda q: float(a[min(len(a) - 1, int(q * len(a)))])
     return {"n": len(a), "mean": float(a.mean()), "p50": pick(0.50), "p90": pick(0.90), "p99": pick(0.99),
             "min": float(a[0]), "max": float(a[-1])}
+
+
+def per_step_us(launch_ms, steps):
+    """Per-launch durations (ms, issue order) of `steps` equal steps -> device us per step."""
+    per = len(launch_ms) // steps if steps and len(launch_ms) % steps == 0 else 0
+    if per <= 1:
+        return [v * 1e3 for v in launch_ms]
+    return [sum(launch_ms[i * per:(i + 1) * per]) * 1e3 for i in range(steps)]
 
 
 def warm_up(lib, one_call, calls, warm_ms=0.0):
@@ -101,54 +107,61 @@ def warm_up(lib, one_call, calls, warm_ms=0.0):
         lib.blt_backend_pass_sync_hip()
 
 
-def time_plan(lib, api, plan, steps, warmup, warm_ms=0.0):
-    """(wall seconds for `steps` launches, {tag: (launches, total_ms, min, max)})."""
-    warm_up(lib, lambda: lib.blt_attention_plan_run_hip(plan), warmup, warm_ms)
+def time_plan(lib, api, plan, steps, warmup, warm_ms=WARM_MS):
+    """Warm-up (`warmup` launches, then by time), then two regions of back-to-back launches:
+    exactly `steps` plain launches bracketed by device syncs (the whole-job wall time), and
+    max(steps, MIN_SAMPLES) launches with a start / stop event pair attached to each (the kernel's
+    own durations).  Returns (wall seconds of the plain region, {tag: (launches, total_ms, min,
+    max)} of one launch, per-launch durations in ms of the event-timed region, its wall seconds)."""
+    run = lambda: lib.blt_attention_plan_run_hip(plan)
+    warm_up(lib, run, warmup, warm_ms)
     lib.blt_hip_profile_begin()
+    run()
+    tags = api.profile_end()
+    lib.blt_backend_pass_sync_hip()
     t0 = time.perf_counter()
     for _ in range(steps):
-        lib.blt_attention_plan_run_hip(plan)
+        run()
     lib.blt_backend_pass_sync_hip()
-    wall = time.perf_counter() - t0
-    return wall, api.profile_end()
+    wall_plain = time.perf_counter() - t0
+    n = max(steps, MIN_SAMPLES)
+    lib.blt_hip_profile_begin()
+    t0 = time.perf_counter()
+    for _ in range(n):
+        run()
+    lib.blt_backend_pass_sync_hip()
+    wall_events = time.perf_counter() - t0
+    return wall_plain, tags, api.profile_end_list(), wall_events
 
 
-def bench_dense(make, steps, warmup, bound, mask_mode="descriptor", warm_ms=0.0, caller_path=False):
+def bench_dense(make, steps, warmup, bound, mask_mode="descriptor", warm_ms=WARM_MS, caller_path=False):
     from fblt_amd import api, runner
     lib = api.load()
     w = make()
     d = runner.DeviceWorkload(w)
     plan = d.make_plan(mask_mode)
     kernel = lib.blt_attention_plan_kernel_hip(plan).decode()
-    wall, prof = time_plan(lib, api, plan, steps, warmup, warm_ms)
-    # the same launches without events attached: the whole-job rate
-    lib.blt_backend_pass_sync_hip()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        lib.blt_attention_plan_run_hip(plan)
-    lib.blt_backend_pass_sync_hip()
-    wall_plain = time.perf_counter() - t0
-    pct = step_percentiles(lib, api, lambda s_: lib.blt_attention_plan_run_hip(plan), min(steps, 256))
+    wall_plain, tags, launch_ms, wall_events = time_plan(lib, api, plan, steps, warmup, warm_ms)
     lib.blt_attention_plan_destroy_hip(plan)
     caller = bench_caller_path(w, d, steps, warmup) if caller_path else None
     d.close()
-    launches = sum(v[0] for v in prof.values())
-    kern_ms = sum(v[1] for v in prof.values())
-    avg_s = kern_ms / 1e3 / steps       # device time of one step (all its launches)
+    per_launch = sum(v[0] for v in tags.values())          # launches of one step
+    samples = per_step_us(launch_ms, len(launch_ms) // per_launch)
+    pct = sample_stats(samples)
+    avg_s = pct["mean"] * 1e-6                               # device time of one step (all its launches)
     res = {
-        "workload": w.name, "kernel": kernel, "launches_per_step": launches / steps,
+        "workload": w.name, "kernel": kernel, "launches_per_step": per_launch,
         "tokens_per_step": w.tokens, "ms_per_step": wall_plain / steps * 1e3,
-        "ms_per_step_with_events": wall / steps * 1e3,
-        "kernel_us_avg": avg_s * 1e6, "kernel_us_min": min(v[2] for v in prof.values()) * 1e3,
-        "kernel_us_percentiles": pct,
+        "ms_per_step_with_events": wall_events / len(samples) * 1e3,
+        "kernel_us_avg": pct["mean"], "kernel_us_p50": pct["p50"], "kernel_us_min": pct["min"],
+        "kernel_us_samples": pct["n"], "kernel_us_percentiles": pct,
         "tokens_per_s": w.tokens * steps / wall_plain,
         "tokens_per_s_kernel": w.tokens / avg_s,
         "flops": w.flops, "bytes": w.bytes,
         "roofline_hbm": roofline("hbm", w.bytes, avg_s, MEASURED_TRAFFIC_BYTES.get(w.name)),
         "roofline_mfma": roofline("mfma", w.flops, avg_s),
     }
-    if warm_ms:
-        res["warmup_ms"] = warm_ms
+    res["warmup_ms"] = warm_ms
     if caller:
         res["reference_call_pattern"] = caller
     res["roofline"] = res["roofline_" + bound]
@@ -185,10 +198,8 @@ def bench_caller_path(w, d, steps, warmup):
             for a in args:
                 a.mask = t.data
                 lib.blt_attention_head_core(abi.BLT_BACKEND_HIP, C.byref(a))
-    n = max(5, steps // 10)
-    for _ in range(max(2, warmup // 4)):
-        one_pass()
-    lib.blt_backend_pass_sync_hip()
+    n = max(10, steps // 10)
+    warm_up(lib, one_pass, max(2, warmup // 4), WARM_MS / 2)
     lib.blt_hip_profile_begin()
     for _ in range(n):
         one_pass()
@@ -217,32 +228,37 @@ def bench_kv(kw, steps, warmup, warm_ms=0.0, lens="device"):
     d = runner.DeviceKvWorkload(kw, lens=lens)
     idx = (lambda s: s) if kw.commit else (lambda s: 0)
 
-    def one_pass(profiled):
+    def one_pass(profiled, count=steps):
+        """reset, `warmup` steps, then `count` timed steps; (wall seconds, per-launch ms or None)"""
         d.reset()
         for s in range(warmup):
             d.step(idx(s))
         lib.blt_backend_pass_sync_hip()
-        if warm_ms and not kw.commit:
-            warm_up(lib, lambda: d.step(0), 0, warm_ms)
         if profiled:
             lib.blt_hip_profile_begin()
         t0 = time.perf_counter()
-        for s in range(warmup, warmup + steps):
+        for s in range(warmup, warmup + count):
             d.step(idx(s))
         lib.blt_backend_pass_sync_hip()
         wall = time.perf_counter() - t0
-        return wall, (api.profile_end() if profiled else None)
+        return wall, (api.profile_end_list() if profiled else None)
 
-    wall, prof = one_pass(True)
-    wall_plain, _ = one_pass(False)
+    # warm by time: a non-committing step repeats; a committing workload repeats whole passes
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < max(warm_ms, WARM_MS):
+        one_pass(False)
     d.reset()
-    for s in range(warmup):
-        d.step(idx(s))
-    lib.blt_backend_pass_sync_hip()
-    pct = step_percentiles(lib, api, lambda s_: d.step(idx(warmup + s_)), min(steps, 256))
-    kern_ms = sum(v[1] for v in prof.values())
-    launches = sum(v[0] for v in prof.values())
-    avg_s = kern_ms / 1e3 / steps
+    lib.blt_hip_profile_begin()
+    d.step(idx(0))
+    tags = api.profile_end()
+    wall_plain, _ = one_pass(False)
+    # a committing workload has exactly `steps` steps to time; a repeating one gives as many samples as asked
+    timed = steps if kw.commit else max(steps, MIN_SAMPLES)
+    wall, launch_ms = one_pass(True, timed)
+    per_launch = sum(v[0] for v in tags.values())
+    samples = per_step_us(launch_ms, len(launch_ms) // per_launch)
+    pct = sample_stats(samples)
+    avg_s = pct["mean"] * 1e-6
     # algorithmic work of an average timed step: lengths grow by n per committed step
     E, n = kw.E, kw.n
     base = float(kw.lens.astype("int64").sum())
@@ -253,10 +269,10 @@ def bench_kv(kw, steps, warmup, warm_ms=0.0, lens="device"):
     bytes_step = 4.0 * (2 * E * mean_keys + rows * 2 * E + (rows * 2 * E if kw.commit else 0))
     flops_step = 4.0 * kw.hd * kw.H * n * mean_keys
     res = {
-        "workload": kw.name, "kernel": "+".join(sorted(prof)), "launches_per_step": launches / steps,
+        "workload": kw.name, "kernel": "+".join(sorted(tags)), "launches_per_step": per_launch,
         "tokens_per_step": kw.tokens, "us_per_step": wall_plain / steps * 1e6,
-        "us_per_step_with_events": wall / steps * 1e6, "kernel_us_avg": avg_s * 1e6,
-        "kernel_us_min": min(v[2] for v in prof.values()) * 1e3, "kernel_us_percentiles": pct,
+        "us_per_step_with_events": wall / timed * 1e6, "kernel_us_avg": pct["mean"], "kernel_us_p50": pct["p50"],
+        "kernel_us_min": pct["min"], "kernel_us_samples": pct["n"], "kernel_us_percentiles": pct,
         "tokens_per_s": kw.tokens * steps / wall_plain, "tokens_per_s_kernel": kw.tokens / avg_s,
         "flops": flops_step, "bytes": bytes_step,
         "roofline_hbm": roofline("hbm", bytes_step, avg_s, MEASURED_TRAFFIC_BYTES.get(kw.name)),
@@ -264,8 +280,7 @@ def bench_kv(kw, steps, warmup, warm_ms=0.0, lens="device"):
         "entry": ("blt_kv_attend_step_lens_hip (lengths on the host, carried in the kernel arguments)"
                   if lens == "host" else "blt_kv_attend_step_hip / blt_kv_rope_attend_step_hip (lengths in device memory)"),
     }
-    if warm_ms and not kw.commit:
-        res["warmup_ms"] = warm_ms
+    res["warmup_ms"] = max(warm_ms, WARM_MS)
     res["roofline"] = res["roofline_hbm"]
     return res, kw
 
@@ -1047,10 +1062,6 @@ def main():
     ap.add_argument("--detail", default=DETAIL_FILE, help="file the full per-workload records are written to")
     ap.add_argument("--probe-copy-mib", type=int, default=0,
                     help="only run the plain streaming copy of this many MiB --steps times (counter yardstick)")
-    ap.add_argument("--probe-read-mib", default="",
-                    help="only run the plain streaming read over buffers of these sizes (comma list of MiB)")
-    ap.add_argument("--probe-issue", action="store_true",
-                    help="only run the matrix / vector issue probe (do fp32 MFMA and VALU overlap on a SIMD?)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the workload shards by sequence "
@@ -1077,35 +1088,14 @@ def main():
                           "GBps_read_plus_write": 2.0 * nbytes * args.steps / dt / 1e9}), flush=True)
         return
 
-    if args.probe_read_mib:
-        from fblt_amd import probes
-        lib = probes.load()
-        sizes = [int(x) for x in args.probe_read_mib.split(",") if x]
-        buf = torch.ones((max(sizes) << 20) // 4, dtype=torch.float32, device="cuda")
-        torch.cuda.synchronize()
-        out = []
-        for mib in sizes:
-            ms = lib.blt_probe_stream_read(buf.data_ptr(), mib << 20, 10)
-            out.append({"MiB": mib, "us_per_launch": ms * 1e3, "GBps": (mib << 20) / ms / 1e6,
-                        "frac_of_hbm_peak": (mib << 20) / ms / 1e6 / HBM_PEAK_GBS})
-        print(json.dumps({"probe": "stream_read", "results": out}), flush=True)
-        return
-    if args.probe_issue:
-        from fblt_amd import probes
-        lib = probes.load()
-        groups = 4000
-        ms = {m: min(lib.blt_probe_issue(m, groups) for _ in range(3)) for m in (1, 2, 3)}
-        tflops = 256 * 4 * groups * 8 * 4096 / (ms[1] * 1e-3) / 1e12   # one matrix wave per SIMD
-        print(json.dumps({"probe": "issue", "groups": groups, "ms_matrix_only": ms[1], "ms_vector_only": ms[2],
-                          "ms_both": ms[3], "both_over_sum": ms[3] / (ms[1] + ms[2]),
-                          "both_over_max": ms[3] / max(ms[1], ms[2]), "matrix_only_TFLOPs": tflops}), flush=True)
-        return
-
     only = set(x for x in args.only.split(",") if x)
     want = lambda c: not only or c in only
     K, W = args.steps, args.warmup
     cs = args.cpu_scale
 
+    from fblt_amd import probes
+    floor = _sig(probes.launch_floor(300))
+    log("launch_floor", json.dumps(floor))
     head, w2 = bench_dense(workloads.config2, K, W, "hbm", caller_path=True)
     log("c2", json.dumps(head))
     others = {}
@@ -1131,6 +1121,10 @@ def main():
         for B in (4, 8, 16):
             others["c5_B%d" % B], k5 = bench_kv(workloads.config5(B=B), K, W)
             log("c5_B%d" % B, json.dumps(others["c5_B%d" % B]))
+            # the same block with the lengths where the reference keeps them (on the host,
+            # csrc/infer/kv_cache.h:56-60; csrc/infer/block_generation.c:156-266)
+            others["c5_B%d_host_lens" % B], _ = bench_kv(workloads.config5(B=B), K, W, lens="host")
+            log("c5_B%d_host_lens" % B, json.dumps(others["c5_B%d_host_lens" % B]))
         # the sibling shape the reference's KV path really runs: a chunk-causal block of 16 new rows
         # over the cached prefix (a prefill chunk, kv_cache.c:229-236), not committed so that it repeats
         others["c5_chunk_causal_n16"], _ = bench_kv(_chunk_causal(workloads.config5(B=16)), K, W)
@@ -1240,7 +1234,7 @@ def main():
         detail_path = os.path.relpath(args.detail, ROOT)
     except OSError as e:
         log("detail file not written:", e)
-    print(json.dumps(compact_line(head, others, cpu_head, K, W, detail_path)), flush=True)
+    print(json.dumps(compact_line(head, others, cpu_head, K, W, detail_path, floor)), flush=True)
 
 
 def _sig(x, digits=4):
@@ -1252,41 +1246,41 @@ def _sig(x, digits=4):
     return x
 
 
-def compact_line(head, others, cpu_head, K, W, detail_path):
+def compact_line(head, others, cpu_head, K, W, detail_path, floor=None):
     """The one JSON object printed last on stdout: headline figures in full precision, one short
     summary row per attention shape (kernel, its device microseconds, fraction of the binding
     roofline, the reference call pattern beside it, CPU figure)."""
     def row(r):
+        """kernel, device us per step (mean and median of the event samples), bound and fraction of its
+        roofline, tokens/s; where measured: HBM traffic over algorithmic bytes, the reference's call pattern
+        on this library's ops as [launches, device us, wall us] per pass, the CPU figure."""
         if r is None:
             return None
-        o = {"kernel": r["kernel"][:40], "launches": r["launches_per_step"], "kernel_us": r["kernel_us_avg"],
-             "bound": r["roofline"]["bound"], "frac": r["roofline"]["frac"],
-             "tokens_per_s": r["tokens_per_s"]}
+        c_dense = "reference_call_pattern" in r   # the dense configurations: tokens/s of the KV rows are lifted to the top
+        o = {"kernel": r["kernel"][:24], "us": r["kernel_us_avg"], "p50": r.get("kernel_us_p50"),
+             "bound": r["roofline"]["bound"], "frac": r["roofline"]["frac"]}
+        if c_dense:
+            o["tok_s"] = r["tokens_per_s"]
+        if r["launches_per_step"] != 1:
+            o["launches"] = r["launches_per_step"]
         if r.get("roofline_hbm", {}).get("traffic"):
             o["traffic_x"] = r["roofline_hbm"]["traffic"] / r["bytes"]   # measured HBM bytes over algorithmic bytes
         c = r.get("reference_call_pattern")
         if c:
-            # the reference's call pattern on this library's ops: [launches, device us, wall us] per pass
             o["caller"] = [c["launches_per_pass"], _sig(c["kernel_us_per_pass"]), _sig(c["wall_us_per_pass"])]
         b = r.get("cpu_baseline")
         if b:
             o["cpu"] = [_sig(b["value"]), b["unit"]]
         return _sig(o)
     per = {"c2": row(head)}
-    for k in ("c1", "c3", "c4", "c4_host_lens", "c4_rope", "c5_B4", "c5_B8", "c5_B16"):
+    for k in ("c1", "c3", "c4", "c4_host_lens", "c4_rope", "c5_B4", "c5_B4_host_lens", "c5_B8", "c5_B8_host_lens",
+              "c5_B16", "c5_B16_host_lens"):
         if k in others:
             per[k] = row(others[k])
     # the same kernels away from the launch floor: [kernel us, binding roofline, fraction of it]
     scaled = {k: [_sig(others[k]["kernel_us_avg"]), others[k]["roofline"]["bound"], _sig(others[k]["roofline"]["frac"])]
               for k in ("c1_x64", "c2_x8", "c1_T4096", "c2_P2048", "c4_b128_L2048", "c4_b128_L2048_host_lens",
                         "c5_B16_b128_L2048", "c5_B16_b128_L2048_host_lens") if k in others}
-    # whole decoder step (all layers + LM head): [launches per step, device us, wall us]
-    steps_ = {k: [others[k]["launches_per_step"], _sig(others[k]["kernel_us_avg"]), _sig(others[k]["us_per_step"])]
-              for k in ("decode_step", "decode_step_b1", "draft_pass", "encoder", "decoder_forward") if k in others}
-    if "reference_call" in others.get("draft_pass", {}):   # the reference's call (prefix recomputed per pass) beside the cached block step
-        c = others["draft_pass"]["reference_call"]
-        steps_["draft_pass_reference_call"] = [c["launches_per_pass"], _sig(c["kernel_us_per_pass"]),
-                                               _sig(c["wall_us_per_pass"])]
     return {
         "metric": "attn_tokens_per_s", "value": head["tokens_per_s"], "unit": "tokens/s",
         "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": head["ms_per_step"],
@@ -1297,6 +1291,11 @@ def compact_line(head, others, cpu_head, K, W, detail_path):
                    "kernel": head["kernel"], "tokens_per_step": head["tokens_per_step"]},
         "kernel_us_avg": head["kernel_us_avg"],
         "kernel_us_p50": head["kernel_us_percentiles"]["p50"],
+        "kernel_us_samples": head["kernel_us_samples"],
+        # an empty kernel timed the same way (events on the dispatch) and by the host clock back to back: an
+        # event-timed duration includes dispatch overhead that overlaps the previous kernel in a back-to-back
+        # loop, so kernel_us can exceed ms_per_step for kernels close to the floor
+        "launch_floor": floor,
         "roofline": head["roofline"],
         "roofline_mfma": head["roofline_mfma"],
         "cpu_baseline": cpu_head,
@@ -1306,10 +1305,11 @@ def compact_line(head, others, cpu_head, K, W, detail_path):
         # reference's blt_kv_decode_step (the device-length entry, which graphs can replay, is beside it)
         "decode_us_per_step": others["c4_host_lens"]["us_per_step"] if "c4_host_lens" in others else None,
         "decode_us_per_step_device_lens": others["c4"]["us_per_step"] if "c4" in others else None,
-        "verify_tokens_per_s": {k: others[k]["tokens_per_s"] for k in ("c5_B4", "c5_B8", "c5_B16") if k in others} or None,
+        # verify: query rows per second of the block step, lengths on the host as the reference keeps them
+        "verify_tokens_per_s": {k[:-10]: others[k]["tokens_per_s"] for k in
+                                ("c5_B4_host_lens", "c5_B8_host_lens", "c5_B16_host_lens") if k in others} or None,
         "per_config": per,
         "at_scale": scaled or None,
-        "decoder_step": steps_ or None,
         "detail": detail_path,
     }
 

@@ -217,6 +217,7 @@ SYMBOLS = {
     "blt_hip_graph_destroy": (None, [C.c_void_p]),
     "blt_hip_profile_begin": (None, []),
     "blt_hip_profile_end": (C.c_size_t, [C.POINTER(BltHipKernelTime), C.c_size_t]),
+    "blt_hip_profile_end_list": (C.c_size_t, [C.POINTER(C.c_float), C.c_size_t]),
     "blt_hip_build_info": (C.c_char_p, []),
 }
 
@@ -282,6 +283,13 @@ def problem_array(problems):
     for i, p in enumerate(problems):
         arr[i] = p
     return arr
+
+
+def profile_end_list(capacity=1 << 16):
+    """Close the open profile: the duration of every launch since `begin`, in milliseconds, in issue order."""
+    buf = (C.c_float * capacity)()
+    n = load().blt_hip_profile_end_list(buf, capacity)
+    return [buf[i] for i in range(min(n, capacity))]
 
 
 def profile_end():

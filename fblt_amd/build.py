@@ -1,5 +1,5 @@
 """Builds fblt_amd/lib/libfblt_hip.so: host C99 (gcc) + gfx950 HIP (hipcc); and the
-bench-only yardsticks fblt_amd/lib/libfblt_probes.so.
+bench-only counter yardstick fblt_amd/lib/libfblt_probes.so.
 
 `python -m fblt_amd.build` or `fblt_amd.build.build()`.  Objects go to
 fblt_amd/lib/obj; nothing is compiled at import time, and loading the library
@@ -16,7 +16,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(LIBDIR, "obj")
 LIB = os.path.join(LIBDIR, "libfblt_hip.so")
-# measurement yardsticks of bench.py's --probe-* modes: their own small library, not in the backend's ABI
+# the counter yardstick of bench.py's --probe-copy-mib mode: its own small library, not in the backend's ABI
 PROBES_SRC = os.path.join(HERE, "probes", "probes.hip")
 PROBES_LIB = os.path.join(LIBDIR, "libfblt_probes.so")
 

@@ -484,7 +484,10 @@ void kv_step_run(const blt_kv_attn_cache *cache, const float *q_rows, size_t q_s
                       combined + row0 * combined_stride, combined_stride, rows, n, row0, step_kind, last ? commit : 0,
                       max_len_hint - (n - row0 - rows), static_scratch, host_lens);
     }
-    if (!host_lens) g_unchecked_steps.fetch_add(1, std::memory_order_relaxed);
+    if (!host_lens) {
+        g_unchecked_steps.fetch_add(1, std::memory_order_relaxed);
+        blt_stream_note_device_length_step(); /* replays of a graph that holds this step arm the check themselves */
+    }
 }
 
 /* Query capacity of the per-split record layout a launch of `nq` rows uses: the VALU kernel's
@@ -722,6 +725,8 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
 
 /* Reads the sticky device error word when a device-length step was issued since the last look;
  * called by the library's synchronising entry points after their wait. */
+void blt_kv_arm_device_error_check() { g_unchecked_steps.fetch_add(1, std::memory_order_relaxed); }
+
 void blt_kv_check_device_errors() {
     if (g_unchecked_steps.exchange(0, std::memory_order_relaxed) == 0) return;
     uint32_t word = 0;

@@ -32,13 +32,6 @@
 #include <cstring>
 #include <type_traits>
 
-#ifdef BLT_MARKS
-__device__ unsigned long long blt_marks[16 * 65536];
-extern "C" void blt_marks_read(unsigned long long *out, size_t count) {
-    HIP_CHECK(hipMemcpyFromSymbol(out, HIP_SYMBOL(blt_marks), count * sizeof(unsigned long long)));
-}
-#endif
-
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -464,7 +457,6 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
     const uint32_t hsafe = head_ok ? head : 0u;
     const uint32_t g = lane >> 4;
     const uint32_t c = lane & 15u;
-    BLT_MARK(0);
 
     const uint32_t len = kv_len_of(a, lens, b) + a.len_bias;
     const uint32_t nk = len + a.n;
@@ -478,7 +470,6 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
     const uint32_t per_split = a.splits == 1u ? total_subs : (total_subs + a.splits - 1u) / a.splits;
     const uint32_t s_begin = split * per_split;
     const uint32_t s_end = min(s_begin + per_split, total_subs);
-    BLT_MARK(1);
 
     const float *const cache_k = a.cache_k + slab * a.embed_dim + hsafe * HD;
     const float *const cache_v = a.cache_v + slab * a.embed_dim + hsafe * HD;
@@ -524,7 +515,6 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
     float kf[2][QD];
     float vf[DT][8];
     request(kf, vf, si);
-    BLT_MARK(3);
 
     /* query fragment: row c of the block (clamped), columns [g*QD, (g+1)*QD) of the head */
     const uint32_t qi = a.q0 + c;
@@ -554,7 +544,6 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
     }
     if (!q_ok) vis_hi = 0;
     const float scale2 = a.scale * LOG2E;
-    BLT_MARK(2);
 
     floatx4 oacc[DT];
 #pragma unroll
@@ -562,8 +551,6 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
 #pragma unroll
         for (int r = 0; r < 4; r++) oacc[d][r] = 0.f;
     float m = neg_inf(), l = 0.f;
-    uint32_t mark_it = 0; /* sub-chunks done (cycle marks of experiment builds) */
-    (void)mark_it;
 
     while (si < s_end) {
         float kn[2][QD];
@@ -604,7 +591,6 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
                 }
             }
         }
-        BLT_MARK(8 + (mark_it < 3u ? mark_it : 3u));
 
         floatx4 sacc[2];
 #pragma unroll
@@ -660,11 +646,8 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
         for (int d = 0; d < DT; d++)
 #pragma unroll
             for (int u = 0; u < 8; u++) vf[d][u] = vn[d][u];
-        BLT_MARK(12 + (mark_it < 3u ? mark_it : 3u));
-        mark_it++;
         si += a.slices;
     }
-    BLT_MARK(4);
 
     /* the four lane groups of a column carry the same m, their sums add */
     l = swap32(swap16(l, OpSum()), OpSum());
@@ -685,13 +668,10 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
                 make_float4(oacc[0][r], oacc[1][r], oacc[2][r], oacc[3][r]);
     }
     if (g == 0) *reinterpret_cast<float2 *>(mine + c * LPR + HD) = make_float2(m * LN2, l); /* merges work in natural units */
-    BLT_MARK(5);
     __syncthreads();
-    BLT_MARK(6);
     const uint32_t early_ticket = kv_draw_early_ticket(a, b); /* as in the 32-wide kernel */
 
     kv_merge_slices<HD, WAVES, LPR, (int)ROWS>(a, sm_o, hshift, wave, b, split, newrow0, zblock);
-    BLT_MARK(7);
 
     kv_finish_sequence<HD>(a, (uint32_t)SLOTS, b, nk, &sm_ticket, early_ticket);
 }
@@ -739,7 +719,6 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
     const uint32_t li = lane & 3u;   /* i of the A operand, j (query) of B and D in S^T */
     const uint32_t half = lane >> 5; /* which 32 keys of a sub-chunk this lane contracts in O */
     const uint32_t dcol = lane & 31u;
-    BLT_MARK(0);
 
     const uint32_t len = kv_len_of(a, lens, b) + a.len_bias;
     const uint32_t nk = len + a.n;
@@ -755,7 +734,6 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
         s_end = min(s_begin + per_split, total_subs);
     }
 
-    BLT_MARK(1);
     const char *const cache_k = reinterpret_cast<const char *>(a.cache_k + slab * a.embed_dim + hsafe * HD);
     const char *const cache_v = reinterpret_cast<const char *>(a.cache_v + slab * a.embed_dim + hsafe * HD);
     const char *const new_k = reinterpret_cast<const char *>(a.k_rows + newrow0 * a.k_stride + hsafe * HD);
@@ -808,7 +786,6 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
     float4 kr[8];
     float vr[32];
     if (LOOP || si < s_end) request(kr, vr, si); /* before anything waits for memory */
-    BLT_MARK(3);
 
     const uint32_t qi = a.q0 + li;
     const bool q_ok = qi < a.n;
@@ -820,7 +797,6 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
     }
     if (!q_ok) vis_hi = 0;
     const float scale2 = a.scale * LOG2E;
-    BLT_MARK(2);
 
     floatx4 oacc; /* register i: O[query i][column dcol], this half's keys */
 #pragma unroll
@@ -853,7 +829,6 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
             }
         }
 
-        BLT_MARK(8);
         /* S[query, key]: A = block 0's query rows for every block (cbsz:4 abid:0), B = the lane's K
          * row; two chains (even and odd columns) so that no instruction waits for the one before.
          * Register i of lane (blk, j) ends up with query i against key j0 + 4 blk + j. */
@@ -900,7 +875,6 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
             x[r] = vis ? t : neg_inf();
             mt = fmaxf(mt, x[r]);
         }
-        BLT_MARK(9);
         mt = across_keys<4>(mt, OpMax()); /* over the sixteen blocks, query by query */
         const float mn = fmaxf(m, mt);
         const float ms = mn == neg_inf() ? 0.f : mn;
@@ -925,7 +899,6 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
     oacc = __builtin_amdgcn_mfma_f32_4x4x1f32(x[3], vr[4 * BETA + 3], oacc, 3, BETA, 0);
         BLT_O_STEP(0) BLT_O_STEP(1) BLT_O_STEP(2) BLT_O_STEP(3) BLT_O_STEP(4) BLT_O_STEP(5) BLT_O_STEP(6) BLT_O_STEP(7)
 #undef BLT_O_STEP
-        BLT_MARK(12);
     };
 
     if constexpr (!LOOP) {
@@ -945,7 +918,6 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
         }
     }
 
-    BLT_MARK(4);
     /* the two halves of the keys meet; the sixteen blocks' sums of weights meet; m is already common */
 #pragma unroll
     for (int r = 0; r < 4; r++) oacc[r] = swap32(oacc[r], OpSum());
@@ -957,12 +929,9 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
         for (int i = 0; i < 4; i++) mine[i * LPR + dcol] = oacc[i];
         if (blk == 0u) *reinterpret_cast<float2 *>(mine + li * LPR + HD) = make_float2(m * LN2, l);
     }
-    BLT_MARK(5);
     __syncthreads();
-    BLT_MARK(6);
     const uint32_t early_ticket = kv_draw_early_ticket(a, b);
     kv_merge_slices<HD, WAVES, LPR, (int)ROWS>(a, sm_o, hshift, wave, b, split, newrow0, blockIdx.z);
-    BLT_MARK(7);
     kv_finish_sequence<HD>(a, (uint32_t)SLOTS, b, nk, &sm_ticket, early_ticket);
 }
 

@@ -19,4 +19,11 @@
         if (blt_hip_err_ != hipSuccess) BLT_FATAL("%s failed: %s", what, hipGetErrorString(blt_hip_err_));         \
     } while (0)
 
+/* The calling wave's outstanding vector-memory operations have completed when this returns
+ * (device-scope write-through stores are then visible to the other workgroups of the launch).
+ * Placed between a workgroup's published data and the barrier before its ticket, so that the
+ * order "data, then ticket" rests on a wait the source states rather than on one the compiler
+ * happens to emit for the barrier. */
+__device__ __forceinline__ void blt_vector_memory_done() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 #endif

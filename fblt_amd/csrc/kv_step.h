@@ -8,19 +8,8 @@
 #define FBLT_AMD_KV_STEP_H
 
 #include "attn_device.h"
+#include "hip_check.h"
 #include "rope_device.h"
-
-#ifdef BLT_MARKS /* experiment builds only: cycle marks of wave 0 of every workgroup */
-extern __device__ unsigned long long blt_marks[];
-#define BLT_MARK(i)                                                                                        \
-    do {                                                                                                   \
-        if (threadIdx.x == 0)                                                                              \
-            blt_marks[((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 16 + (i)] =       \
-                __builtin_readcyclecounter();                                                              \
-    } while (0)
-#else
-#define BLT_MARK(i) do { } while (0)
-#endif
 
 constexpr int SUB = 32;        /* keys per sub-chunk (one wave, one head)       */
 constexpr int MAX_SPLITS = 16; /* workgroups per sequence                        */
@@ -144,8 +133,8 @@ __device__ __forceinline__ float observe(const float *p) {
  *
  * The per-split states were stored with device-scope write-through stores and
  * are read back with device-scope loads, so they never sit dirty or stale in
- * one die's L2 and no cache write-back or invalidate is needed; the barrier's
- * wait on outstanding memory operations orders the stores before this
+ * one die's L2 and no cache write-back or invalidate is needed; each wave waits
+ * for its own stores to complete before the barrier that precedes the
  * workgroup's ticket. */
 /* The step commits, has one split per sequence but several workgroups (head
  * groups): all that has to be known is when every workgroup of the sequence
@@ -179,6 +168,7 @@ __device__ __forceinline__ void kv_finish_sequence(const StepArgs &a, uint32_t s
         }
         return;
     }
+    blt_vector_memory_done(); /* every wave's published records are out before thread 0 draws the ticket */
     __syncthreads();
     if (threadIdx.x == 0)
         *sm_ticket = __hip_atomic_fetch_add(&a.tickets[b], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -30,6 +30,12 @@ void blt_upload_staged(void *dst, const void *src, size_t bytes);
  * only when such a step was issued since the last look.  Called after a host wait
  * (attn_decode.hip). */
 void blt_kv_check_device_errors();
+/* Makes the next call of blt_kv_check_device_errors read the word: for device-length steps that
+ * are issued without passing through the step's entry point (replays of a captured graph). */
+void blt_kv_arm_device_error_check();
+/* Tells an open capture on this thread that it recorded a KV step with device-resident lengths
+ * (stream.hip); no effect outside a capture. */
+void blt_stream_note_device_length_step();
 /* A fresh (start, stop) event pair owned by the open profile, booked under `tag`. */
 void blt_profile_book(const char *tag, hipEvent_t *start, hipEvent_t *stop);
 

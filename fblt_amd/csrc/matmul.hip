@@ -402,8 +402,8 @@ __device__ __forceinline__ void splitk_tile(const MatmulArgs &g, const uint32_t 
         }
     }
     if (!GATED && !CROSS && g.slices > 1u) {
-        /* Device-scope stores and loads, and the barrier's wait on outstanding memory operations
-         * between this workgroup's stores and its ticket, as for the split softmax states of the
+        /* Device-scope stores and loads, and an explicit wait for the stores' completion before the
+         * barrier that precedes this workgroup's ticket, as for the split softmax states of the
          * KV step (kv_step.h).  The waves past the fourth have left. */
         __shared__ uint32_t ticket;
         const uint32_t tile = by * gridDim.x + bx;
@@ -411,6 +411,7 @@ __device__ __forceinline__ void splitk_tile(const MatmulArgs &g, const uint32_t 
 #pragma unroll
         for (int i = 0; i < 4; i++)
             __hip_atomic_store(sums + (size_t)blockIdx.z * 1024u + i, v4[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        blt_vector_memory_done(); /* every wave's sums are out before thread 0 draws the ticket */
         __syncthreads();
         if (threadIdx.x == 0)
             ticket = __hip_atomic_fetch_add(&g.slice_tickets[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

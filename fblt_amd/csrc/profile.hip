@@ -39,6 +39,23 @@ extern "C" void blt_hip_profile_begin(void) {
     g_open = true;
 }
 
+extern "C" size_t blt_hip_profile_end_list(float *ms_out, size_t capacity) {
+    BLT_REQUIRE(g_open, "blt_hip_profile_end_list: no profile is open");
+    g_open = false;
+    HIP_CHECK(hipDeviceSynchronize());
+    size_t at = 0;
+    for (const Booking &b : g_bookings) {
+        float ms = 0.f;
+        HIP_CHECK(hipEventElapsedTime(&ms, b.start, b.stop));
+        HIP_CHECK(hipEventDestroy(b.start));
+        HIP_CHECK(hipEventDestroy(b.stop));
+        if (ms_out && at < capacity) ms_out[at] = ms;
+        at++;
+    }
+    g_bookings.clear();
+    return at;
+}
+
 extern "C" size_t blt_hip_profile_end(blt_hip_kernel_time *out, size_t capacity) {
     BLT_REQUIRE(g_open, "blt_hip_profile_end: no profile is open");
     g_open = false;

@@ -25,6 +25,7 @@ namespace {
 thread_local hipStream_t t_stream = nullptr;
 thread_local hipStream_t t_saved = nullptr;
 thread_local bool t_capturing = false;
+thread_local bool t_captured_device_length_step = false; /* the open capture recorded a KV step that reads self_len on the device */
 hipStream_t g_capture_stream = nullptr; /* default priority, non-blocking; lives until the process ends */
 
 } // namespace
@@ -32,11 +33,18 @@ hipStream_t g_capture_stream = nullptr; /* default priority, non-blocking; lives
 struct blt_hip_graph {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
+    /* The graph holds a KV step with device-resident lengths: a replay can outgrow what the
+     * captured launch was sized for, which its kernels report through the sticky device error
+     * word; every replay therefore arms the host's look at that word. */
+    bool device_length_step = false;
 };
 
 hipStream_t blt_stream() { return t_stream; }
 hipStream_t blt_stream_key() { return t_capturing ? t_saved : t_stream; }
 bool blt_stream_capturing() { return t_capturing; }
+void blt_stream_note_device_length_step() {
+    if (t_capturing) t_captured_device_length_step = true;
+}
 
 extern "C" void blt_hip_set_stream(void *stream) {
     BLT_REQUIRE(!t_capturing, "blt_hip_set_stream: a capture is open on this thread");
@@ -54,6 +62,7 @@ extern "C" void blt_hip_capture_begin(void) {
     t_stream = g_capture_stream;
     HIP_CHECK(hipStreamBeginCapture(g_capture_stream, hipStreamCaptureModeThreadLocal));
     t_capturing = true;
+    t_captured_device_length_step = false;
 }
 
 extern "C" blt_hip_graph *blt_hip_capture_end(void) {
@@ -64,6 +73,7 @@ extern "C" blt_hip_graph *blt_hip_capture_end(void) {
     t_stream = t_saved;
     if (e != hipSuccess || g->graph == nullptr) BLT_FATAL("blt_hip_capture_end: capture failed: %s", hipGetErrorString(e));
     HIP_CHECK(hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0));
+    g->device_length_step = t_captured_device_length_step;
     return g;
 }
 
@@ -71,6 +81,7 @@ extern "C" void blt_hip_graph_launch(const blt_hip_graph *g) {
     BLT_REQUIRE(g != NULL && g->exec != nullptr, "blt_hip_graph_launch: graph must not be NULL");
     BLT_REQUIRE(!t_capturing, "blt_hip_graph_launch: a capture is open on this thread");
     HIP_CHECK(hipGraphLaunch(g->exec, t_stream));
+    if (g->device_length_step) blt_kv_arm_device_error_check();
 }
 
 extern "C" void blt_hip_graph_destroy(blt_hip_graph *g) {

@@ -1,5 +1,6 @@
-"""ctypes binding of libfblt_probes.so: the measurement yardsticks bench.py's --probe-* modes run
-(plain streaming copy and read, matrix / vector issue probe).  Not part of the attention backend."""
+"""ctypes binding of libfblt_probes.so: the two yardsticks bench.py runs (a plain streaming copy of
+known size for the hardware counters, an empty kernel for the launch floor).  Not part of the
+attention backend."""
 import ctypes as C
 import os
 
@@ -16,7 +17,14 @@ def load():
         import torch  # noqa: F401  (one HIP runtime per process: torch's comes first)
         lib = C.CDLL(LIB_PATH)
         lib.blt_probe_stream_copy.restype, lib.blt_probe_stream_copy.argtypes = None, [C.c_void_p, C.c_void_p, C.c_size_t]
-        lib.blt_probe_stream_read.restype, lib.blt_probe_stream_read.argtypes = C.c_float, [C.c_void_p, C.c_size_t, C.c_int]
-        lib.blt_probe_issue.restype, lib.blt_probe_issue.argtypes = C.c_float, [C.c_int, C.c_int]
+        fp = C.POINTER(C.c_float)
+        lib.blt_probe_launch_floor.restype, lib.blt_probe_launch_floor.argtypes = None, [C.c_int, fp, fp, fp]
         _lib = lib
     return _lib
+
+
+def launch_floor(launches=300):
+    """{event_us_mean, event_us_median, back_to_back_wall_us} of an empty kernel."""
+    mean, med, wall = C.c_float(), C.c_float(), C.c_float()
+    load().blt_probe_launch_floor(launches, C.byref(mean), C.byref(med), C.byref(wall))
+    return {"event_us_mean": mean.value, "event_us_median": med.value, "back_to_back_wall_us": wall.value}

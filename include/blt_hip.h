@@ -547,6 +547,10 @@ typedef struct {
 } blt_hip_kernel_time;
 void blt_hip_profile_begin(void);
 size_t blt_hip_profile_end(blt_hip_kernel_time *out, size_t capacity);
+/* The same close, launch by launch: the duration in milliseconds of every launch since `begin`, in
+ * the order they were issued (up to `capacity` of them); returns the number of launches seen.
+ * For medians and percentiles of a kernel's duration. */
+size_t blt_hip_profile_end_list(float *ms_out, size_t capacity);
 
 /* Library build tag and the architecture its kernels were compiled for. */
 const char *blt_hip_build_info(void);

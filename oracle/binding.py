@@ -62,11 +62,6 @@ def load_oracle():
     lib.orc_kv_slot.argtypes = [C.c_size_t] * 7
     lib.orc_kv_self_mask.restype = None
     lib.orc_kv_self_mask.argtypes = [_fp, C.c_size_t, C.c_size_t, C.c_size_t]
-    lib.orc_kv_step_group_ids.restype = None
-    lib.orc_kv_step_group_ids.argtypes = [C.POINTER(abi.BltPatchInfo), C.c_size_t, C.c_size_t, C.c_size_t,
-                                          C.c_size_t, C.c_int, _sp, _sp]
-    lib.orc_kv_cross_mask.restype = None
-    lib.orc_kv_cross_mask.argtypes = [_fp, _sp, C.c_size_t, _sp, C.c_size_t]
     lib.orc_kv_attend_step.restype = C.c_int
     lib.orc_kv_attend_step.argtypes = [_fp, _fp, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t,
                                        C.c_size_t, C.c_size_t, _fp, _fp, _fp, _fp]

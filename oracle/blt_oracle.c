@@ -258,21 +258,6 @@ void orc_kv_self_mask(float *out, size_t n, size_t base, size_t window) {
     }
 }
 
-/* csrc/infer/kv_cache.c:203-218 */
-void orc_kv_step_group_ids(const blt_patch_info *patches, size_t num_patches, size_t k_split, size_t base,
-                           size_t n, int trailing_closed, size_t *q_ids, size_t *kv_ids) {
-    for (size_t r = 0; r < n; r++) q_ids[r] = orc_patch_decoder_latent_at(patches, num_patches, base + r);
-    if (trailing_closed && num_patches >= 1) q_ids[n - 1] = num_patches - 1;
-    for (size_t p = 0; p < num_patches; p++)
-        for (size_t s = 0; s < k_split; s++) kv_ids[p * k_split + s] = p;
-}
-
-/* csrc/infer/kv_cache.c:240-251 */
-void orc_kv_cross_mask(float *out, const size_t *q_ids, size_t n, const size_t *kv_ids, size_t total_sub) {
-    for (size_t r = 0; r < n; r++)
-        for (size_t j = 0; j < total_sub; j++) out[r * total_sub + j] = kv_ids[j] == q_ids[r] ? 0.0f : -INFINITY;
-}
-
 /* csrc/infer/kv_cache.c:343-390 (attention statements only) */
 int orc_kv_attend_step(float *self_k, float *self_v, size_t max_seq_len, size_t E, size_t H, size_t b,
                        size_t base, size_t n, size_t window, const float *q_rows, const float *k_rows,

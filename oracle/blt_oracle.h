@@ -155,14 +155,6 @@ size_t orc_kv_slot(size_t b, size_t pos, size_t head, size_t d, size_t max_seq_l
  * columns; allowed = j <= base+r and (window == 0 or base+r-j < window). */
 void orc_kv_self_mask(float *out, size_t n, size_t base, size_t window);
 
-/* Query/KV group ids of a decode step, kv_cache.c:203-218. */
-void orc_kv_step_group_ids(const blt_patch_info *patches, size_t num_patches, size_t k_split, size_t base,
-                           size_t n, int trailing_closed, size_t *q_group_ids, size_t *kv_group_ids);
-
-/* Cross-attention step mask, kv_cache.c:240-251. */
-void orc_kv_cross_mask(float *out, const size_t *q_group_ids, size_t n, const size_t *kv_group_ids,
-                       size_t total_sub);
-
 /* The attention part of one decode step for one sequence, kv_cache.c:343-390
  * without the projections and RoPE: `q_rows`, `k_rows`, `v_rows` are the n new
  * rows [n, E] (K already rotated).  K/V rows are written through to slab rows

@@ -577,12 +577,13 @@ def test_zero_weight_key_with_non_finite_value_row(oracle, dev):
         assert_close(mid[fin], out_ref[first_tile_row:bad_key, bad_col][fin], "finite cells of the key's tile")
 
 
-@pytest.mark.parametrize("mode", ["hint", "slab", "tables"])
+@pytest.mark.parametrize("mode", ["hint", "slab", "tables", "graph"])
 def test_kv_step_length_beyond_capacity_is_reported(mode):
     """The lengths of the KV step live on the device; the host sizes the launch from a hint.  A
     sequence that outgrew the hint, its slab or the rotation tables is left alone by the kernels
     (which all exit normally) and the next synchronising call ends with the reference's "exceeds
-    cache capacity" error (csrc/infer/kv_cache.c:191).  Runs in its own process: the error is fatal."""
+    cache capacity" error (csrc/infer/kv_cache.c:191).  "graph": the same for a committing step that is
+    replayed from a HIP graph past its captured hint.  Runs in its own process: the error is fatal."""
     import os
     import subprocess
     import sys
@@ -590,6 +591,7 @@ def test_kv_step_length_beyond_capacity_is_reported(mode):
     p = subprocess.run([sys.executable, "-u", os.path.join(here, "kv_guard_case.py"), mode], capture_output=True,
                        text=True, timeout=300)
     assert "CHECKED" in p.stdout and "NOT REACHED" not in p.stdout, p.stdout[-2000:] + p.stderr[-2000:]
+    assert mode != "graph" or "REPLAY 1 QUIET" in p.stdout, p.stdout[-2000:]
     assert p.returncode == 1 and "exceeds cache capacity" in p.stderr, (p.returncode, p.stderr[-2000:])
 
 
