@@ -2,7 +2,7 @@
  * Entry points of the attention forward path: the per-head device twin the
  * reference's dispatcher binds, the whole-batch launch and the resident plan.
  * Host code only (argument checks, descriptor translation, kernel choice);
- * the kernels live in attn_rows.hip, attn_mfma.hip, attn_wide.hip and attn_fine.hip.
+ * the kernels live in attn_rows.hip, attn_mfma.hip, attn_wide.hip, attn_fine.hip and attn_once.hip.
  */
 #include "blt_hip.h"
 #include "blt_fatal.h"
@@ -14,12 +14,13 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <string>
 #include <vector>
 
 namespace {
 
 /* Kernel family a problem is routed to. */
-enum Family : uint32_t { FAM_ROWS = 0, FAM_MFMA = 1, FAM_WIDE = 2, FAM_FINE = 3 };
+enum Family : uint32_t { FAM_ROWS = 0, FAM_MFMA = 1, FAM_WIDE = 2, FAM_FINE = 3, FAM_ONCE = 4, FAM_COUNT = 5 };
 
 struct Bucket {
     Family fam;
@@ -33,7 +34,7 @@ struct Bucket {
     uint32_t max_nq;
     uint32_t tiles;   /* mfma: number of work items; first item index in tile array = tile_base */
     uint32_t tile_base;
-    uint32_t span;    /* fine: keys the longest 32-row tile needs */
+    uint32_t span;    /* fine: keys the longest 32-row tile needs; once: 16-key tiles the longest 16-row tile spans */
     bool tall;        /* fine: 16-row workgroups of sixteen waves */
     bool whole;       /* fine: one four-wave workgroup per whole problem (strided batches) */
 };
@@ -109,7 +110,7 @@ AttnProb translate(const blt_attention_problem &pr, bool need_score_buffer, cons
     return d;
 }
 
-/* BLT_HIP_ATTN_FAMILY=rows|mfma|wide|fine pins the kernel family wherever the
+/* BLT_HIP_ATTN_FAMILY=rows|mfma|wide|fine|once pins the kernel family wherever the
  * shape allows it (tuning and test hook); unset or anything else = automatic. */
 int family_override() {
     static const int cached = [] {
@@ -118,6 +119,7 @@ int family_override() {
         if (e && std::strcmp(e, "mfma") == 0) return 2;
         if (e && std::strcmp(e, "wide") == 0) return 3;
         if (e && std::strcmp(e, "fine") == 0) return 4;
+        if (e && std::strcmp(e, "once") == 0) return 5;
         return 0;
     }();
     return cached;
@@ -126,6 +128,7 @@ int family_override() {
 Family choose_family(const AttnProb &d) {
     const int forced = family_override();
     if (forced == 1) return FAM_ROWS;
+    if (forced == 5) return attn_once_can(d) || attn_mfma_takes(d) ? FAM_MFMA : FAM_ROWS;
     if (forced >= 2 && attn_mfma_can(d)) return FAM_MFMA;
     if (attn_mfma_takes(d)) return FAM_MFMA;
     return FAM_ROWS;
@@ -150,7 +153,7 @@ uint32_t wide_min_groups(uint32_t max_nk) {
 /* Do problems p[0..n), all routed to the mfma family, go to the wide kernel instead? */
 bool choose_wide(const AttnProb *p, uint32_t n) {
     const int forced = family_override();
-    if (forced == 1 || forced == 2 || forced == 4) return false;
+    if (forced == 1 || forced == 2 || forced == 4 || forced == 5) return false;
     uint64_t groups = 0;
     uint32_t max_nk = 0;
     for (uint32_t i = 0; i < n; i++) {
@@ -207,6 +210,25 @@ bool choose_fine(const AttnProb *p, uint32_t n, bool strided, uint32_t &span, bo
     if (span > attn_fine_fill_max(p[0].hd)) return tiles > 448u && tiles <= 512u;
     if (tiles <= 256u && span > 64u) return false;
     return groups < (max_nk <= 64u ? 640u : 448u);
+}
+
+/* Do problems p[0..n), all routed to the mfma family, go to the once kernel (16-row tiles whose keys
+ * are all in flight at once)?  `span` gets the 16-key tiles its longest tile spans.  The kernel is
+ * built for launches one trip to memory deep: it is chosen while the launch gives a compute unit
+ * at most one workgroup. */
+bool choose_once(const AttnProb *p, uint32_t n, uint32_t &span) {
+    const int forced = family_override();
+    if (forced != 0 && forced != 5) return false;
+    uint64_t tiles = 0;
+    uint32_t most = 0;
+    for (uint32_t i = 0; i < n; i++) {
+        if (!attn_once_can(p[i])) return false;
+        most = std::max(most, attn_once_span_tiles(p[i]));
+        tiles += (p[i].nq + 15u) / 16u;
+    }
+    if (forced == 0 && tiles > 256u) return false;
+    span = most;
+    return true;
 }
 
 /* Does a strided batch of n problems like `d` go to the fine family's whole-problem shape (one
@@ -315,7 +337,7 @@ struct blt_attention_plan {
     std::vector<AttnTile> tiles;  /* mfma work items, all buckets */
     AttnProb *dev = nullptr;      /* resident plans: descriptors in device memory */
     AttnTile *dev_tiles = nullptr;
-    const char *kernel = "none";
+    std::string kernel_name = "none";
 };
 
 namespace {
@@ -382,28 +404,37 @@ void plan_build(blt_attention_plan &pl, const blt_attention_problem *problems, s
         b.affine = detect_affine(pl.host.data() + b.base, b.count, b.aff);
         b.whole = choose_whole(pl.host[b.base], b.count, b.affine);
         if (b.whole) b.fam = FAM_FINE;
+        else if (choose_once(pl.host.data() + b.base, b.count, b.span)) b.fam = FAM_ONCE;
         else if (choose_fine(pl.host.data() + b.base, b.count, b.affine, b.span, b.tall)) b.fam = FAM_FINE;
         else if (choose_wide(pl.host.data() + b.base, b.count)) b.fam = FAM_WIDE;
         if (b.affine) continue; /* no descriptor or tile memory needed */
         b.tile_base = (uint32_t)pl.tiles.size();
         if (b.fam == FAM_WIDE) attn_wide_make_tiles(pl.host.data(), b.base, b.count, pl.tiles);
         else if (b.fam == FAM_FINE) attn_fine_make_tiles(pl.host.data(), b.base, b.count, pl.tiles);
+        else if (b.fam == FAM_ONCE) attn_once_make_tiles(pl.host.data(), b.base, b.count, pl.tiles);
         else attn_mfma_make_tiles(pl.host.data(), b.base, b.count, pl.tiles);
         b.tiles = (uint32_t)pl.tiles.size() - b.tile_base;
     }
-    bool any[4] = {false, false, false, false};
+    bool any[FAM_COUNT] = {false, false, false, false, false};
     for (const Bucket &b : pl.buckets) any[b.fam] = true;
-    static const char *const names[16] = {"none",           "rows",           "mfma",           "mfma+rows",
-                                          "wide",           "wide+rows",      "wide+mfma",      "wide+mfma+rows",
-                                          "fine",           "fine+rows",      "fine+mfma",      "fine+mfma+rows",
-                                          "fine+wide",      "fine+wide+rows", "fine+wide+mfma", "fine+wide+mfma+rows"};
-    pl.kernel = names[(any[FAM_ROWS] ? 1 : 0) | (any[FAM_MFMA] ? 2 : 0) | (any[FAM_WIDE] ? 4 : 0) |
-                      (any[FAM_FINE] ? 8 : 0)];
+    /* the families the plan launches, joined by '+': "fine", "mfma+rows", ... */
+    static const char *const names[FAM_COUNT] = {"rows", "mfma", "wide", "fine", "once"};
+    pl.kernel_name.clear();
+    for (int f = FAM_COUNT - 1; f >= 0; f--) {
+        if (!any[f]) continue;
+        if (!pl.kernel_name.empty()) pl.kernel_name += "+";
+        pl.kernel_name += names[f];
+    }
+    if (pl.kernel_name.empty()) pl.kernel_name = "none";
 }
 
 void plan_launch(const blt_attention_plan &pl, const AttnProb *dev, const AttnTile *dev_tiles) {
     for (const Bucket &b : pl.buckets) {
-        if (b.fam == FAM_WIDE && b.affine)
+        if (b.fam == FAM_ONCE && b.affine)
+            attn_once_launch_affine(b.aff, 0);
+        else if (b.fam == FAM_ONCE)
+            attn_once_launch(dev, dev_tiles + b.tile_base, b.tiles, b.hd, b.span, b.dense, 0);
+        else if (b.fam == FAM_WIDE && b.affine)
             attn_wide_launch_affine(b.aff, 0);
         else if (b.fam == FAM_WIDE)
             attn_wide_launch(dev, dev_tiles + b.tile_base, b.tiles, b.hd, b.dense, 0);
@@ -488,7 +519,8 @@ extern "C" void blt_attention_head_core_hip(blt_backend backend, const blt_atten
     const Family f = choose_family(d);
     uint32_t span = 0;
     bool tall = false;
-    if (f == FAM_MFMA && choose_fine(&d, 1, true, span, tall)) attn_fine_launch_single(d, tall, 0);
+    if (f == FAM_MFMA && choose_once(&d, 1, span)) attn_once_launch_single(d, 0);
+    else if (f == FAM_MFMA && choose_fine(&d, 1, true, span, tall)) attn_fine_launch_single(d, tall, 0);
     else if (f == FAM_MFMA && choose_wide(&d, 1)) attn_wide_launch_single(d, 0);
     else if (f == FAM_MFMA) attn_mfma_launch_single(d, 0);
     else attn_rows_launch_single(d, 0);
@@ -533,5 +565,5 @@ extern "C" void blt_attention_plan_destroy_hip(blt_attention_plan *plan) {
 }
 
 extern "C" const char *blt_attention_plan_kernel_hip(const blt_attention_plan *plan) {
-    return plan ? plan->kernel : "none";
+    return plan ? plan->kernel_name.c_str() : "none";
 }

@@ -71,4 +71,15 @@ void attn_fine_launch_affine(const AttnAffine &aff, bool tall, hipStream_t s);
 bool attn_whole_can(const AttnProb &d);
 void attn_whole_launch_affine(const AttnAffine &aff, hipStream_t s);
 
+/* once family: 16-row tiles whose keys are all in flight at once, exact softmax, weights in the same
+ * sweep (attn_once.hip) */
+bool attn_once_can(const AttnProb &d);
+uint32_t attn_once_tiles_max(uint32_t hd);
+uint32_t attn_once_span_tiles(const AttnProb &d);
+void attn_once_make_tiles(const AttnProb *host, uint32_t base, uint32_t count, std::vector<AttnTile> &tiles);
+void attn_once_launch(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t ntiles, uint32_t hd, uint32_t span_tiles,
+                      bool dense, hipStream_t s);
+void attn_once_launch_single(const AttnProb &single, hipStream_t s);
+void attn_once_launch_affine(const AttnAffine &aff, hipStream_t s);
+
 #endif

@@ -751,7 +751,7 @@ def test_kv_step_kernel_families_agree(kernel):
     assert p.returncode == 0 and "OK" in p.stdout, p.stdout[-2000:] + p.stderr[-2000:]
 
 
-@pytest.mark.parametrize("family", ["rows", "mfma", "wide", "fine", "fine16", "fine128"])
+@pytest.mark.parametrize("family", ["rows", "mfma", "wide", "fine", "fine16", "fine128", "once"])
 def test_attention_kernel_families(family):
     """Every attention kernel family on the same cases (causal, chunked prefill, sliding window,
     dense masks, lse output), pinned through BLT_HIP_ATTN_FAMILY in a fresh process; the fine
@@ -778,7 +778,7 @@ def test_attention_kernel_families(family):
         assert ("attn_whole" in launched) == (shape == "fine128"), launched
 
 
-@pytest.mark.parametrize("family", ["auto", "rows", "mfma", "wide", "fine", "fine16", "fine128"])
+@pytest.mark.parametrize("family", ["auto", "rows", "mfma", "wide", "fine", "fine16", "fine128", "once"])
 def test_attention_random_shapes(family):
     """72 randomly shaped strided batches per routing (automatic, and every family / workgroup shape
     pinned wherever the shape allows it) through the one-shot batch entry and a plan, against the
@@ -799,6 +799,8 @@ def test_attention_random_shapes(family):
     launched = [ln for ln in p.stdout.splitlines() if ln.startswith("LAUNCHED")][0].split()[1].split(",")
     if family == "fine128":
         assert "attn_whole" in launched, launched
+    if family == "once":
+        assert "attn_once" in launched, launched
 
 
 @pytest.mark.parametrize("case", ["decode", "chunk5", "block16", "packed"])
