@@ -599,7 +599,8 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
             const size_t nb = std::min<size_t>(KARG_SEQS, cache->batch - b0);
             uint32_t longest = 0;
             for (size_t b = 0; b < nb; b++) longest = std::max(longest, host_lens[b0 + b] + 1u);
-            kv_row_launch(chunk_of(a, b0), (uint32_t)nb, (uint32_t)hd, host_lens + b0, longest, 0);
+            BLT_REQUIRE(kv_row_launch(chunk_of(a, b0), (uint32_t)nb, (uint32_t)hd, host_lens + b0, longest, 0),
+                        "blt_kv_attend_step_lens: internal: head_dim %zu not taken by the row kernel", hd);
         }
         HIP_CHECK_LAUNCH("blt_kv_attend_step_lens");
         return;
@@ -618,7 +619,8 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
         a.splits = 1, a.span = 0, a.q0 = 0, a.write_through = 1, a.commit = commit;
         a.cap = (uint32_t)std::min<size_t>((size_t)cache->max_seq_len, rope_cos ? rope_positions : (size_t)UINT32_MAX);
         acquire_scratch(a, 0, cache->batch, static_scratch);
-        kv_row_launch(a, (uint32_t)cache->batch, (uint32_t)hd, nullptr, (uint32_t)max_len_hint, 0);
+        BLT_REQUIRE(kv_row_launch(a, (uint32_t)cache->batch, (uint32_t)hd, nullptr, (uint32_t)max_len_hint, 0),
+                    "blt_kv_attend_step: internal: head_dim %zu not taken by the row kernel", hd);
         HIP_CHECK_LAUNCH("blt_kv_attend_step");
         return;
     }
@@ -696,10 +698,12 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
             a.self_len = nullptr;
             for (size_t b0 = 0; b0 < cache->batch; b0 += KARG_SEQS) {
                 const size_t nb = std::min<size_t>(KARG_SEQS, cache->batch - b0);
-                kv_block_mfma_launch(chunk_of(a, b0), (uint32_t)nb, (uint32_t)hd, host_lens + b0, 0);
+                BLT_REQUIRE(kv_block_mfma_launch(chunk_of(a, b0), (uint32_t)nb, (uint32_t)hd, host_lens + b0, 0),
+                            "blt_kv_attend_step_lens: internal: head_dim %zu not taken by the block kernels", hd);
             }
         } else {
-            kv_block_mfma_launch(a, (uint32_t)cache->batch, (uint32_t)hd, nullptr, 0);
+            BLT_REQUIRE(kv_block_mfma_launch(a, (uint32_t)cache->batch, (uint32_t)hd, nullptr, 0),
+                        "blt_kv_attend_step: internal: head_dim %zu not taken by the block kernels", hd);
         }
         HIP_CHECK_LAUNCH("blt_kv_attend_step");
         return;

@@ -300,6 +300,7 @@ __global__ __launch_bounds__(64 * WAVES, 4) void attn_fine_kernel(const AttnProb
     extern __shared__ __attribute__((aligned(16))) float sm[];
     float *const sm_k = sm;
     float *const sm_v = sm + (size_t)kc * ROW;
+    float *const sm_q = sm + (size_t)2 * kc * ROW; /* the tile's query rows, ROWS x ROW */
 
     if (SRC != SRC_TILES) {
         /* every kernel argument the workgroup will read is asked for here, in one go: left to
@@ -381,16 +382,19 @@ __global__ __launch_bounds__(64 * WAVES, 4) void attn_fine_kernel(const AttnProb
         for (int r = 0; r < 4; r++) oacc[d][r] = 0.f;
     float m = neg_inf(), l = 0.f;
 
-    /* the query fragment: row c of the half, columns [g*QD, (g+1)*QD) */
+    /* The tile's query rows: one 16-byte piece per thread, consecutive lanes on consecutive pieces of
+     * a row (a load whose lanes each touch another row is served at a quarter of the rate, and a
+     * fragment read straight from global memory is such a load), parked with the first stage's
+     * rows and read back as fragments -- row c of the half, columns [g*QD, (g+1)*QD) -- after the
+     * barrier that stage has anyway.  Threads past the tile's pieces repeat one (no branch around
+     * the request) and park nothing. */
+    constexpr uint32_t QPIECES = ROWS * (uint32_t)LPR4;
+    static_assert(QPIECES <= FINE_THREADS, "one query piece per thread at most");
     float qf[QD];
-    {
-        const float *qrow = p.q + (size_t)qi * p.q_stride + g * QD;
-#pragma unroll
-        for (int s = 0; s < QD; s += 4) {
-            const float4 t = *reinterpret_cast<const float4 *>(qrow + s);
-            qf[s + 0] = t.x, qf[s + 1] = t.y, qf[s + 2] = t.z, qf[s + 3] = t.w;
-        }
-    }
+    const uint32_t qe = tid % QPIECES;
+    const floatx4 q_piece = *reinterpret_cast<const floatx4 *>(
+        p.q + (size_t)min(q0 + qe / LPR4, p.nq - 1u) * p.q_stride + 4u * (qe % LPR4));
+    bool q_ready = false; /* uniform: the fragment has been read */
 
     /* ---- fill: rows [c0, c0 + kc) of K and V, clamped to the last row the tile needs; the first
      * fill is requested here, the later ones at the end of the loop's body, so that nothing at the
@@ -410,11 +414,10 @@ __global__ __launch_bounds__(64 * WAVES, 4) void attn_fine_kernel(const AttnProb
     };
     uint32_t c0 = t0 * 16u;
     request(c0); /* unconditionally: a branch here would make the code after it wait for every request */
-    /* the query fragment is pinned down here, where the compiler still counts the requests in flight
-     * one by one: inside the loops below a use of a value that is still on its way makes it wait for
-     * every request, the later pieces of the fill included */
-#pragma unroll
-    for (int s = 0; s < QD; s++) asm volatile("" : "+v"(qf[s]));
+    /* the query piece is parked here, where the compiler still counts the requests in flight one by
+     * one: inside the loops below a use of a value that is still on its way makes it wait for every
+     * request, the later pieces of the fill included */
+    if (tid < QPIECES) *reinterpret_cast<floatx4 *>(sm_q + (qe / LPR4) * ROW + 4u * (qe % LPR4)) = q_piece;
     while (c0 < key_end) {
         /* ---- the pieces land in the order they were requested: piece by piece, park it and work
          * on the key tiles it completes while the later pieces are still on their way ---- */
@@ -433,6 +436,15 @@ __global__ __launch_bounds__(64 * WAVES, 4) void attn_fine_kernel(const AttnProb
         /* one stage = the units of the key tiles that pieces [0, pieces_done) complete */
         auto stage = [&](const uint32_t pieces_done) __attribute__((always_inline)) {
             __syncthreads();
+            if (!q_ready) { /* first barrier of the workgroup: the query rows are parked */
+                const float *qrow = sm_q + (16u * half + c) * ROW + g * QD;
+#pragma unroll
+                for (int s = 0; s < QD; s += 4) {
+                    const float4 t = *reinterpret_cast<const float4 *>(qrow + s);
+                    qf[s + 0] = t.x, qf[s + 1] = t.y, qf[s + 2] = t.z, qf[s + 3] = t.w;
+                }
+                q_ready = true;
+            }
             const uint32_t stage_end = min(c0 + RPP * pieces_done, fill_end);
             while (kt < my1 && kt * 16u < stage_end) {
                 const uint32_t k0 = kt * 16u;
@@ -671,11 +683,12 @@ void fine_launch_as(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t nbl
                     uint32_t span, hipStream_t s) {
     using Shape = FineShape<HD, HALVES, WAVES>;
     const uint32_t kc = fine_fill_keys<Shape>(span);
-    const size_t lds = (size_t)2 * kc * Shape::ROW * sizeof(float);
+    /* K and V rows of a fill, then the tile's query rows */
+    const size_t lds = ((size_t)2 * kc + 16u * HALVES) * Shape::ROW * sizeof(float);
     static const bool raised = [] { /* more than the 64 KB a kernel may use without asking */
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_fine_kernel<HD, SRC, HALVES, WAVES>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      2 * (int)Shape::KC_MAX * Shape::ROW * (int)sizeof(float)));
+                                      (2 * (int)Shape::KC_MAX + 16 * HALVES) * Shape::ROW * (int)sizeof(float)));
         return true;
     }();
     (void)raised;

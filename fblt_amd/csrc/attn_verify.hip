@@ -346,8 +346,8 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
  * lane does not grow with the number of slices (a loop over the slices in one thread did: 1900
  * cycles at 8 slices, by cycle marks).  With one split the output rows are written, otherwise the
  * workgroup's per-split records. */
-template <int HD, int WAVES, int LPR, int ROWCAP>
-__device__ __forceinline__ void kv_merge_slices(const StepArgs &a, const float (*sm_o)[ROWCAP * LPR], uint32_t hshift,
+template <int HD, int WAVES, int LPR, int ROWCAP, int STRIDE = ROWCAP * LPR> /* STRIDE: floats between the waves' tiles */
+__device__ __forceinline__ void kv_merge_slices(const StepArgs &a, const float (*sm_o)[STRIDE], uint32_t hshift,
                                                 uint32_t wave, uint32_t b, uint32_t split, size_t newrow0,
                                                 const uint32_t zblock) {
     static_assert(WAVES == 4 || WAVES == 8 || WAVES == 16, "slices map onto lane groups of a wave");
@@ -431,8 +431,16 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
     constexpr int DT = HD / 16; /* 16-row tiles of O^T */
     constexpr int LPR = HD + 4; /* a result row [HD columns, max, sum] parked in LDS, rows 16-byte aligned */
     constexpr uint32_t ROWS = 16;
+    constexpr int KROW = HD + 4;      /* a K row on its way to fragments: the same padded row */
+    constexpr int KL = HD / 4;        /* lanes per K row when the wave moves a sub-chunk, 16 bytes each */
+    constexpr int KRI = 64 / KL;      /* K rows one load instruction covers */
+    constexpr int KNV = 32 / KRI;     /* load instructions per 32-key sub-chunk */
 
-    __shared__ __attribute__((aligned(16))) float sm_o[WAVES][ROWS * LPR];
+    /* per wave: the sub-chunk's 32 K rows between their coalesced loads and the fragment reads; after the
+     * loop the first half of the same area holds the wave's result rows */
+    __shared__ __attribute__((aligned(16))) float sm_kt[WAVES][32 * KROW];
+    float(*const sm_o)[32 * KROW] = sm_kt;
+    static_assert(ROWS * LPR <= 32 * KROW, "the result rows fit the K tile they overlay");
     __shared__ uint32_t sm_ticket;
 
     /* Which (sequence, head group) the workgroup takes.  Launches by length walk the pairs sequence
@@ -479,22 +487,22 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
     const uint32_t last_cached = len > 0u ? len - 1u : 0u, last_new = a.n - 1u;
     const uint32_t lane_k = g * (QD * 4u), lane_v = c * (DT * 4u); /* byte offsets inside a row */
 
-    /* K fragment of sub-chunk si: tile t holds its row 16 t + c, columns g*QD ...;
-     * V fragment: element (e, 4 t + r) is column DT c + e of its row 16 t + 4 g + r */
-    auto request = [&](float (&kf)[2][QD], float (&vf)[DT][8], uint32_t si) __attribute__((always_inline)) {
+    /* K rows of sub-chunk si as the wave moves them: load v covers rows KRI v ... KRI v + KRI - 1 with
+     * consecutive lanes on consecutive 16-byte pieces of a row (lanes that each touch another row
+     * are served at a quarter of the rate); they become fragments through the wave's LDS tile.
+     * V fragment: element (e, 4 t + r) is column DT c + e of row 16 t + 4 g + r -- sixteen lanes on one
+     * row's contiguous bytes as it is. */
+    const uint32_t krow_l = lane / KL, kpiece = lane % KL;
+    auto request = [&](floatx4 (&kg)[KNV], float (&vf)[DT][8], uint32_t si) __attribute__((always_inline)) {
         const bool fresh = si >= cached_subs; /* wave-uniform: scalar selects */
         const char *kb = reinterpret_cast<const char *>(fresh ? new_k : cache_k);
         const char *vb = reinterpret_cast<const char *>(fresh ? new_v : cache_v);
         const uint32_t kp = fresh ? newk_pitch : cache_pitch, vp = fresh ? newv_pitch : cache_pitch;
         const uint32_t row0 = fresh ? 0u : si * 32u, limit = fresh ? last_new : last_cached;
 #pragma unroll
-        for (int t = 0; t < 2; t++) {
-            const uint32_t off = min(row0 + 16u * t + c, limit) * kp + lane_k;
-#pragma unroll
-            for (int s = 0; s < QD; s += 4) {
-                const float4 x = *reinterpret_cast<const float4 *>(kb + off + 4 * s);
-                kf[t][s + 0] = x.x, kf[t][s + 1] = x.y, kf[t][s + 2] = x.z, kf[t][s + 3] = x.w;
-            }
+        for (int v = 0; v < KNV; v++) {
+            const uint32_t off = min(row0 + (uint32_t)(KRI * v) + krow_l, limit) * kp + 16u * kpiece;
+            kg[v] = *reinterpret_cast<const floatx4 *>(kb + off);
         }
 #pragma unroll
         for (int u = 0; u < 8; u++) {
@@ -512,9 +520,9 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
 
     /* the first sub-chunk's rows are requested before anything else waits for memory */
     uint32_t si = s_begin + slice;
-    float kf[2][QD];
+    floatx4 kg[KNV];
     float vf[DT][8];
-    request(kf, vf, si);
+    request(kg, vf, si);
 
     /* query fragment: row c of the block (clamped), columns [g*QD, (g+1)*QD) of the head */
     const uint32_t qi = a.q0 + c;
@@ -552,32 +560,24 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
         for (int r = 0; r < 4; r++) oacc[d][r] = 0.f;
     float m = neg_inf(), l = 0.f;
 
+    float *const my_kt = sm_kt[wave];
     while (si < s_end) {
-        float kn[2][QD];
-        float vn[DT][8];
-        request(kn, vn, si + a.slices);
-        __builtin_amdgcn_sched_barrier(0); /* the requests stay ahead of the arithmetic */
-
         const bool fresh = si >= cached_subs;
         const uint32_t j0 = fresh ? len : si * 32u; /* absolute position of the sub-chunk's first key */
         const uint32_t j_end = fresh ? nk : len;    /* rows past it are clamped repeats */
         if (fresh) { /* the new rows: rotate their keys at their own positions, write keys and values through */
 #pragma unroll
-            for (int t = 0; t < 2; t++) {
-                const uint32_t r = 16u * t + c;
+            for (int v = 0; v < KNV; v++) {
+                const uint32_t r = (uint32_t)(KRI * v) + krow_l;
                 const bool real = r < a.n;
-#pragma unroll
-                for (int s = 0; s < QD; s += 4) {
-                    float4 piece = make_float4(kf[t][s + 0], kf[t][s + 1], kf[t][s + 2], kf[t][s + 3]);
-                    if (a.rope_cos && real) {
-                        const size_t at = (size_t)(len + r) * HALF + (g * QD + s) / 2;
-                        piece = rope_rotate4(piece, a.rope_cos + at, a.rope_sin + at);
-                        kf[t][s + 0] = piece.x, kf[t][s + 1] = piece.y, kf[t][s + 2] = piece.z, kf[t][s + 3] = piece.w;
-                    }
-                    if (a.write_through && head_ok && real)
-                        *reinterpret_cast<float4 *>(a.cache_k + (slab + len + r) * a.embed_dim + head * HD + g * QD + s) =
-                            piece;
+                if (a.rope_cos && real) {
+                    const size_t at = (size_t)(len + r) * HALF + 2u * kpiece;
+                    const float4 t = rope_rotate4(make_float4(kg[v][0], kg[v][1], kg[v][2], kg[v][3]), a.rope_cos + at,
+                                                  a.rope_sin + at);
+                    kg[v][0] = t.x, kg[v][1] = t.y, kg[v][2] = t.z, kg[v][3] = t.w;
                 }
+                if (a.write_through && head_ok && real)
+                    *reinterpret_cast<floatx4 *>(a.cache_k + (slab + len + r) * a.embed_dim + head * HD + 4u * kpiece) = kg[v];
             }
             if (a.write_through && head_ok) {
 #pragma unroll
@@ -591,6 +591,24 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
                 }
             }
         }
+        /* rows -> fragments through the wave's own tile (LDS serves a wave's requests in order: no
+         * barrier): tile t holds row 16 t + c, columns g QD ... */
+#pragma unroll
+        for (int v = 0; v < KNV; v++)
+            *reinterpret_cast<floatx4 *>(my_kt + ((uint32_t)(KRI * v) + krow_l) * KROW + 4u * kpiece) = kg[v];
+        float kf[2][QD];
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int s = 0; s < QD; s += 4) {
+                const float4 x = *reinterpret_cast<const float4 *>(my_kt + (16u * t + c) * KROW + g * QD + s);
+                kf[t][s + 0] = x.x, kf[t][s + 1] = x.y, kf[t][s + 2] = x.z, kf[t][s + 3] = x.w;
+            }
+        /* the next sub-chunk's rows travel while this one is worked on: the raw rows have left their
+         * registers, the values move into a second set */
+        float vn[DT][8];
+        request(kg, vn, si + a.slices);
+        __builtin_amdgcn_sched_barrier(0); /* the requests stay ahead of the arithmetic */
 
         floatx4 sacc[2];
 #pragma unroll
@@ -639,10 +657,6 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
                 oacc[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[d][u], x[u], oacc[d], 0, 0, 0);
 
 #pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int s = 0; s < QD; s++) kf[t][s] = kn[t][s];
-#pragma unroll
         for (int d = 0; d < DT; d++)
 #pragma unroll
             for (int u = 0; u < 8; u++) vf[d][u] = vn[d][u];
@@ -671,7 +685,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
     __syncthreads();
     const uint32_t early_ticket = kv_draw_early_ticket(a, b); /* as in the 32-wide kernel */
 
-    kv_merge_slices<HD, WAVES, LPR, (int)ROWS>(a, sm_o, hshift, wave, b, split, newrow0, zblock);
+    kv_merge_slices<HD, WAVES, LPR, (int)ROWS, 32 * KROW>(a, sm_o, hshift, wave, b, split, newrow0, zblock);
 
     kv_finish_sequence<HD>(a, (uint32_t)SLOTS, b, nk, &sm_ticket, early_ticket);
 }
@@ -1037,11 +1051,7 @@ uint32_t kv_block_heads_per_group(uint32_t batch, uint32_t subs, uint32_t num_he
  * 32 query rows per launch: a.q0 .. a.q0 + 31. */
 bool kv_block_mfma_launch(const StepArgs &a, uint32_t batch, uint32_t head_dim, const uint32_t *host_lens,
                           hipStream_t s) {
-    /* the per-wave K tiles bound the 32-wide kernel's workgroup: 8 waves of 4.6 KB or 4 of 8.7 KB */
-    static const int narrow_waves = [] {
-        const char *e = getenv("BLT_HIP_BLOCK_WAVES");
-        return e && *e ? atoi(e) : 8;
-    }();
+    /* the per-wave K tiles bound the workgroups: 8 waves of 4.6 KB or 4 of 8.7 KB */
     /* BLT_HIP_BLOCK_TILE=16 keeps blocks of up to four rows on the 16-wide tiles (test hook) */
     static const bool no_tile4 = [] {
         const char *e = getenv("BLT_HIP_BLOCK_TILE");
@@ -1050,7 +1060,6 @@ bool kv_block_mfma_launch(const StepArgs &a, uint32_t batch, uint32_t head_dim, 
     if (head_dim == 32u) {
         if (a.n - a.q0 <= 4u && !no_tile4) launch_block4(a, batch, host_lens, s);
         else if (!narrow_block(a)) launch_block_as<32, 8, false>(a, batch, host_lens, s);
-        else if (narrow_waves >= 16) launch_block_as<32, 16, true>(a, batch, host_lens, s);
         else launch_block_as<32, 8, true>(a, batch, host_lens, s);
     } else if (head_dim == 64u) {
         if (!narrow_block(a)) launch_block_as<64, 4, false>(a, batch, host_lens, s);

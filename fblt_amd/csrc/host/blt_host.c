@@ -53,7 +53,8 @@ blt_arena *blt_arena_create(size_t capacity_bytes, blt_backend backend) {
 typedef struct host_block {
     struct host_block *next;
     const blt_arena *arena;
-    size_t at; /* the arena's offset when the block was handed out */
+    size_t at;   /* the arena's offset when the block was handed out */
+    size_t seen; /* the arena's offset after the newest allocation this library saw (kept in the newest block) */
 } host_block;
 #define HOST_BLOCK_HEADER 64 /* keeps the payload 64-byte aligned, as arena containers are */
 
@@ -73,6 +74,27 @@ static void host_blocks_release(const blt_arena *a, size_t keep_to, int all) {
             link = &b->next;
         }
     }
+}
+
+/* Called before every allocation from a device arena: an offset below what the last allocation
+ * left behind means the caller has rewound the arena since, and the blocks handed out at or above
+ * the new offset are dead, as their arena-resident twins of the CPU backend would be.  Then notes
+ * where this allocation will leave the offset.  Costs a pointer comparison while the arena has no
+ * blocks. */
+static void host_blocks_sweep(const blt_arena *a, size_t offset_after) {
+    if (!g_host_blocks) return; /* racy peek: a block list that is empty needs no sweep */
+    pthread_mutex_lock(&g_host_blocks_lock);
+    host_block *newest = g_host_blocks;
+    while (newest && newest->arena != a) newest = newest->next;
+    if (newest) {
+        if (a->offset < newest->seen) {
+            host_blocks_release(a, a->offset, 0);
+            newest = g_host_blocks;
+            while (newest && newest->arena != a) newest = newest->next;
+        }
+        if (newest) newest->seen = offset_after;
+    }
+    pthread_mutex_unlock(&g_host_blocks_lock);
 }
 
 void blt_arena_destroy(blt_arena *a) {
@@ -105,6 +127,7 @@ void *blt_arena_alloc(blt_arena *a, size_t bytes, size_t alignment) {
     if (at + bytes > a->capacity)
         BLT_FATAL("arena allocation exceeded capacity: need %zu (aligned %zu), offset %zu, capacity %zu", bytes, at,
                   a->offset, a->capacity);
+    if (a->backend == BLT_BACKEND_HIP) host_blocks_sweep(a, at + bytes);
     a->offset = at + bytes;
     return (char *)a->buffer + at;
 }
@@ -113,11 +136,14 @@ void *blt_arena_alloc(blt_arena *a, size_t bytes, size_t alignment) {
  * model structs (csrc/models/local_decoder.c:76-80, transformer_stack.c:85).  On the CPU backend
  * they live in the arena (csrc/core/tensor.c:154); for a device arena the reference hands out
  * zeroed host memory instead (tensor.c:156-162, backend.c:494-501) and never releases it.  Here a
- * block belongs to its arena and takes a 64-byte token of it, which gives the block a place in the
- * arena's order: it is released when the arena is reset or destroyed, or once the caller has
- * rewound the arena's offset to or below its token (csrc/infer/self_speculation.c:359-401 rewinds
- * that way), which is when a container of the CPU backend would be dead too.  A loop that rewinds
- * to a marker every round therefore holds one round's blocks at most. */
+ * block belongs to its arena and takes ONE BYTE of it as a token, which gives the block a place
+ * in the arena's order (a run of containers costs the arena at most the 63 bytes the next
+ * tensor's alignment would have skipped anyway): the block is released when the arena is reset
+ * or destroyed, or at the first allocation after the caller has rewound the arena's offset to or
+ * below its token (csrc/infer/self_speculation.c:359-401 rewinds that way), which is when a
+ * container of the CPU backend would be dead too.  Every allocation from the arena looks for
+ * such a rewind, so a loop that rewinds to a marker every round holds one round's blocks at
+ * most, whether its first allocation of a round is a container or a tensor. */
 void *blt_container_alloc(blt_arena *a, size_t bytes) {
     if (!a || !a->buffer) BLT_FATAL("invalid arena");
     if (a->backend != BLT_BACKEND_HIP) return blt_arena_alloc(a, bytes, 64);
@@ -128,13 +154,13 @@ void *blt_container_alloc(blt_arena *a, size_t bytes) {
     host_block *b = (host_block *)raw;
     memset(b, 0, HOST_BLOCK_HEADER + bytes);
     b->arena = a;
-    b->at = a->offset;
+    (void)blt_arena_alloc(a, 1, 1); /* the token; sweeps the blocks a rewind has killed */
+    b->at = a->offset - 1;
+    b->seen = a->offset;
     pthread_mutex_lock(&g_host_blocks_lock);
-    host_blocks_release(a, a->offset, 0); /* whatever sat at or above this point was rewound over */
     b->next = g_host_blocks;
     g_host_blocks = b;
     pthread_mutex_unlock(&g_host_blocks_lock);
-    (void)blt_arena_alloc(a, 64, 1); /* the token */
     return (char *)b + HOST_BLOCK_HEADER;
 }
 

@@ -310,7 +310,8 @@ def test_host_arena_and_tensor():
 
 def test_containers_are_host_memory_for_a_device_arena():
     """blt_container_alloc (csrc/core/tensor.c:154-162): arena memory on the CPU backend; for a device arena zeroed,
-    64-byte aligned host memory plus a 64-byte token of the arena, released with the arena's reset or a rewind.  The device
+    64-byte aligned host memory plus a one-byte token of the arena, released with the arena's reset or at the first
+    allocation (container or tensor) after a rewind.  The device
     arena here is a hand-made struct whose buffer is never touched, so this runs without a GPU."""
     lib = api.load()
     host = lib.blt_arena_create(4096, abi.BLT_BACKEND_CPU)
@@ -324,7 +325,7 @@ def test_containers_are_host_memory_for_a_device_arena():
     def take(size):
         before = dev.offset
         q = lib.blt_container_alloc(C.byref(dev), size)
-        assert q % 64 == 0 and dev.offset == before + 64  # the block's token in the arena
+        assert q % 64 == 0 and dev.offset == before + 1  # the block's token in the arena
         view = (C.c_ubyte * size).from_address(q)
         assert not any(view)
         for i in range(size):

@@ -39,6 +39,10 @@ def _cases():
     yield "block16", workloads.config5(batch=9, B=16)
     yield "block8_long_prefix", workloads.config5(batch=2, B=8, len_lo=2500, len_hi=3000, max_seq_len=3072)
     yield "block4_smaller", workloads.config5(batch=3, B=4)
+    # 20 block rows at head width 16: the vector kernel in two launches of at most 16 rows that share the
+    # fixed per-split records
+    wide = workloads.config5(batch=4, B=20, H=4, hd=16, len_lo=600, len_hi=900, max_seq_len=1024)
+    yield "block20_head16_two_launches", wide
 
 
 def test_noalloc_entry_matches_the_allocating_one(oracle):
@@ -52,6 +56,40 @@ def test_noalloc_entry_matches_the_allocating_one(oracle):
         assert (err <= 1e-5 + 1e-4 * np.abs(ref_out)).all(), "%s: max err %.3e" % (name, float(err.max()))
         assert got[1].tobytes() == ref_k.tobytes() and got[2].tobytes() == ref_v.tobytes(), name
         assert (got[3] == kw.lens.astype(np.int64) + (kw.steps * kw.n if kw.commit else 0)).all(), name
+
+
+def test_noalloc_entry_replays_from_a_graph(oracle):
+    """The entry's own use: recorded into a HIP graph (after one eager call, which looks up the fixed array's
+    address) and replayed three times with eager work in between; every replay gives the allocating entry's bits."""
+    import torch
+    from fblt_amd import runner
+    lib = api.load()
+    kw = workloads.config4(batch=24, steps=1, len_lo=300, len_hi=700, max_seq_len=720)
+    kw.commit = False
+    want = _run(kw, "blt_kv_attend_step_hip")
+    d = runner.DeviceKvWorkload(kw)
+    E = kw.E
+
+    def step():
+        lib.blt_kv_attend_step_noalloc_hip(C.byref(d.c), d.q_new[0].data_ptr(), E, d.k_new[0].data_ptr(), E,
+                                           d.v_new[0].data_ptr(), E, d.out[0].data_ptr(), E, kw.n, d.kind, 0,
+                                           d.host_max_len + kw.n)
+    step()
+    lib.blt_backend_pass_sync_hip()
+    lib.blt_hip_capture_begin()
+    step()
+    graph = lib.blt_hip_capture_end()
+    other = workloads.config5(batch=3, B=4)
+    for _ in range(3):
+        d.out.zero_()
+        torch.cuda.synchronize()
+        lib.blt_hip_graph_launch(graph)
+        lib.blt_backend_pass_sync_hip()
+        got = d.results()
+        for g, w, what in zip(got, want, ("out", "cache_k", "cache_v", "lens")):
+            assert g.tobytes() == w.tobytes(), "replay: %s differs from the allocating entry point" % what
+        _run(other, "blt_kv_attend_step_noalloc_hip")   # eager work on the same fixed array between replays
+    lib.blt_hip_graph_destroy(graph)
 
 
 def test_noalloc_entry_rejects_what_the_fixed_scratch_cannot_hold():
