@@ -114,8 +114,15 @@ __global__ __launch_bounds__(64 * W) void attn_once_kernel(const AttnProb *__res
         p = aff.first;
         qtile = gridDim.x - 1u - blockIdx.x; /* the long tiles of a causal problem first */
     } else {
-        const uint32_t prob = blockIdx.x % aff.count;
-        qtile = (aff.first.nq + 15u) / 16u - 1u - blockIdx.x / aff.count;
+        /* Workgroups are handed to the chip's eight dies in turn, each die with an L2 of its own.  A
+         * batch of few problems (aff.reserved = 8: eight slots per round, the slots past the
+         * problems exit at once) therefore keeps every problem on one die, whose L2 then fetches
+         * the problem's K and V rows once for all of its tiles; otherwise the problems of a tile
+         * index follow each other. */
+        const uint32_t slots = aff.reserved ? aff.reserved : aff.count;
+        const uint32_t prob = blockIdx.x % slots;
+        if (prob >= aff.count) return; /* uniform over the workgroup, before any barrier */
+        qtile = (aff.first.nq + 15u) / 16u - 1u - blockIdx.x / slots;
         affine_problem(p, aff, prob, DENSE);
     }
 
@@ -532,8 +539,14 @@ void attn_once_launch_single(const AttnProb &single, hipStream_t s) {
 }
 
 void attn_once_launch_affine(const AttnAffine &aff, hipStream_t s) {
-    const uint32_t nblocks = aff.count * ((aff.first.nq + 15u) / 16u);
-    if (nblocks == 0) return;
-    once_launch_shape<SRC_AFFINE>(nullptr, nullptr, aff, nblocks, aff.first.hd, attn_once_span_tiles(aff.first),
+    const uint32_t nqt = (aff.first.nq + 15u) / 16u;
+    if (aff.count == 0 || nqt == 0) return;
+    AttnAffine a = aff;
+    /* Fewer problems than dies, and no more tiles per problem than a die has compute units: one die per
+     * problem (eight workgroup slots per tile index, see the kernel).  Measured at 4 heads x 512 rows:
+     * the launch fetches K and V once instead of twice. */
+    a.reserved = aff.count < 8u && nqt <= 32u ? 8u : 0u;
+    const uint32_t nblocks = (a.reserved ? a.reserved : aff.count) * nqt;
+    once_launch_shape<SRC_AFFINE>(nullptr, nullptr, a, nblocks, aff.first.hd, attn_once_span_tiles(aff.first),
                                   aff.first.vis == ATTN_VIS_DENSE, s);
 }

@@ -717,8 +717,10 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
     constexpr int LPR = HD + 4; /* a parked result row in LDS, 16-byte aligned */
     constexpr uint32_t ROWS = 4, CH = 64;
 
+    constexpr int KROW = HD + 4; /* a K row on its way from its coalesced load to the lane that contracts it */
     __shared__ __attribute__((aligned(16))) float sm_o[WAVES][ROWS * LPR];
     __shared__ uint32_t sm_ticket;
+    extern __shared__ __attribute__((aligned(16))) float sm_kt4[]; /* per wave: 32 K rows, KROW floats each */
 
     const uint32_t b = blockIdx.y;
     const uint32_t split = blockIdx.x;
@@ -755,17 +757,21 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
     const uint32_t cache_pitch = a.embed_dim * 4u, newk_pitch = a.k_stride * 4u, newv_pitch = a.v_stride * 4u;
     const uint32_t last_cached = len > 0u ? len - 1u : 0u, last_new = a.n - 1u;
 
-    /* kr: the K row of the sub-chunk's row `lane`; vr[4 beta + r]: column dcol of its row 32 half +
-     * 4 beta + r.  Rows past the last one are clamped to it (their weights are zero).  Base, pitch
-     * and limit are scalar selects: every load is scalar base + 32-bit lane offset. */
-    auto request = [&](float4 (&kr)[8], float (&vr)[32], uint32_t si) __attribute__((always_inline)) {
+    /* kg[v]: piece lane % 8 of the sub-chunk's row 8 v + lane / 8 -- consecutive lanes on consecutive
+     * 16-byte pieces of a row; a load whose lanes each touch another row (lane = key, as the S^T
+     * product wants the rows) is served at a quarter of the rate, and eight of those per sub-chunk
+     * were most of what the longest sequences waited for.  vr[4 beta + r]: column dcol of row
+     * 32 half + 4 beta + r.  Rows past the last one are clamped to it (their weights are zero).
+     * Base, pitch and limit are scalar selects: every load is scalar base + 32-bit lane offset. */
+    const uint32_t krow_l = lane >> 3, kpiece = lane & 7u;
+    auto request = [&](floatx4 (&kg)[8], float (&vr)[32], uint32_t si) __attribute__((always_inline)) {
         const bool fresh = si >= cached_subs;
         const char *kb = fresh ? new_k : cache_k, *vb = fresh ? new_v : cache_v;
         const uint32_t kp = fresh ? newk_pitch : cache_pitch, vp = fresh ? newv_pitch : cache_pitch;
         const uint32_t row0 = fresh ? 0u : si * CH, limit = fresh ? last_new : last_cached;
-        const uint32_t koff = __umul24(min(row0 + lane, limit), kp);
 #pragma unroll
-        for (int e = 0; e < 8; e++) kr[e] = *reinterpret_cast<const float4 *>(kb + koff + 16 * e);
+        for (int v = 0; v < 8; v++)
+            kg[v] = *reinterpret_cast<const floatx4 *>(kb + __umul24(min(row0 + 8u * v + krow_l, limit), kp) + 16u * kpiece);
         const uint32_t vrow0 = min(row0 + 32u * half, limit);
         const uint32_t room = limit - vrow0; /* rows this half may step forward */
         const uint32_t voff0 = __umul24(vrow0, vp) + 4u * dcol;
@@ -797,9 +803,10 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
      * unit's vector memory path (64 bytes a cycle) is what the longest sequences wait for -- and
      * park a neutral record.  LOOP = true: sub-chunks round-robin, the next one requested ahead. */
     uint32_t si = s_begin + slice;
-    float4 kr[8];
+    floatx4 kg[8];
     float vr[32];
-    if (LOOP || si < s_end) request(kr, vr, si); /* before anything waits for memory */
+    if (LOOP || si < s_end) request(kg, vr, si); /* before anything waits for memory */
+    float *const my_kt = sm_kt4 + wave * (32 * KROW);
 
     const uint32_t qi = a.q0 + li;
     const bool q_ok = qi < a.n;
@@ -818,28 +825,41 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
     float m = neg_inf(), l = 0.f;
 
     /* one sub-chunk whose rows sit in kr / vr */
-    auto attend = [&](float4 (&kr)[8], float (&vr)[32], uint32_t si) __attribute__((always_inline)) {
+    auto attend = [&](floatx4 (&kg)[8], float (&vr)[32], uint32_t si) __attribute__((always_inline)) {
         const bool fresh = si >= cached_subs;
         const uint32_t j0 = fresh ? len : si * CH; /* absolute position of the sub-chunk's first key */
         const uint32_t j_end = fresh ? nk : len;   /* rows past it are clamped repeats */
         if (fresh) { /* the new rows (wave-uniform): rotate their keys, write keys and values through */
-            const bool real = lane < a.n;
-            if (a.rope_cos && real) {
-                const size_t at = (size_t)(len + lane) * HALF;
 #pragma unroll
-                for (int e = 0; e < 8; e++) kr[e] = rope_rotate4(kr[e], a.rope_cos + at + 2 * e, a.rope_sin + at + 2 * e);
+            for (int v = 0; v < 8; v++) {
+                const uint32_t r = 8u * v + krow_l;
+                const bool real = r < a.n;
+                if (a.rope_cos && real) {
+                    const size_t at = (size_t)(len + r) * HALF + 2u * kpiece;
+                    const float4 t = rope_rotate4(make_float4(kg[v][0], kg[v][1], kg[v][2], kg[v][3]), a.rope_cos + at,
+                                                  a.rope_sin + at);
+                    kg[v][0] = t.x, kg[v][1] = t.y, kg[v][2] = t.z, kg[v][3] = t.w;
+                }
+                if (a.write_through && head_ok && real)
+                    *reinterpret_cast<floatx4 *>(a.cache_k + (slab + len + r) * a.embed_dim + head * HD + 4u * kpiece) = kg[v];
             }
-            if (a.write_through && head_ok) {
-                if (real) {
-                    float *dst = a.cache_k + (slab + len + lane) * a.embed_dim + head * HD;
+            if (a.write_through && head_ok && half == 0u) {
 #pragma unroll
-                    for (int e = 0; e < 8; e++) *reinterpret_cast<float4 *>(dst + 4 * e) = kr[e];
-                }
-                if (half == 0u) {
+                for (int r = 0; r < 4; r++)
+                    if ((uint32_t)r < a.n) a.cache_v[(slab + len + r) * a.embed_dim + head * HD + dcol] = vr[r];
+            }
+        }
+        /* rows -> the lanes that contract them, 32 rows at a time through the wave's own LDS tile (LDS
+         * serves a wave's requests in order: no barrier): lane l ends up with row l whole */
+        float4 kr[8];
 #pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        if ((uint32_t)r < a.n) a.cache_v[(slab + len + r) * a.embed_dim + head * HD + dcol] = vr[r];
-                }
+        for (int h2 = 0; h2 < 2; h2++) {
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+                *reinterpret_cast<floatx4 *>(my_kt + (8u * v + krow_l) * KROW + 4u * kpiece) = kg[4 * h2 + v];
+            if (half == (uint32_t)h2) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) kr[e] = *reinterpret_cast<const float4 *>(my_kt + (lane & 31u) * KROW + 4 * e);
             }
         }
 
@@ -916,16 +936,16 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
     };
 
     if constexpr (!LOOP) {
-        if (si < s_end) attend(kr, vr, si);
+        if (si < s_end) attend(kg, vr, si);
     } else {
         while (si < s_end) {
-            float4 kn[8];
+            floatx4 kn[8];
             float vn[32];
             request(kn, vn, si + a.slices); /* past the end the clamped rows hit the cache; no branch */
             __builtin_amdgcn_sched_barrier(0);
-            attend(kr, vr, si);
+            attend(kg, vr, si);
 #pragma unroll
-            for (int e = 0; e < 8; e++) kr[e] = kn[e];
+            for (int e = 0; e < 8; e++) kg[e] = kn[e];
 #pragma unroll
             for (int t = 0; t < 32; t++) vr[t] = vn[t];
             si += a.slices;
@@ -999,12 +1019,28 @@ template <int WAVES, int MAXW, bool LOOP>
 void launch_block4_as(const StepArgs &a, uint32_t batch, const uint32_t *host_lens, hipStream_t s) {
     dim3 grid(a.splits, batch, (a.num_heads + a.hpb - 1) / a.hpb);
     const dim3 block(64 * a.hpb * a.slices);
+    /* the waves' K tiles: 32 rows of 36 floats each; with sixteen waves more than the 64 KB a kernel
+     * may use without asking (the static result rows come on top) */
+    constexpr size_t kt_bytes = (size_t)MAXW * 32 * 36 * sizeof(float);
     if (host_lens) {
+        static const bool raised = [] {
+            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&kv_block4_mfma_kernel<WAVES, MAXW, LOOP, true>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kt_bytes));
+            return true;
+        }();
+        (void)raised;
         KargLens lens;
         for (uint32_t b = 0; b < batch; b++) lens.v[b] = host_lens[b];
-        blt_launch("kv_block4_mfma", kv_block4_mfma_kernel<WAVES, MAXW, LOOP, true>, grid, block, 0, s, a, lens);
+        blt_launch("kv_block4_mfma", kv_block4_mfma_kernel<WAVES, MAXW, LOOP, true>, grid, block, kt_bytes, s, a, lens);
     } else {
-        blt_launch("kv_block4_mfma", kv_block4_mfma_kernel<WAVES, MAXW, LOOP, false>, grid, block, 0, s, a, DeviceLens{0u});
+        static const bool raised = [] {
+            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&kv_block4_mfma_kernel<WAVES, MAXW, LOOP, false>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kt_bytes));
+            return true;
+        }();
+        (void)raised;
+        blt_launch("kv_block4_mfma", kv_block4_mfma_kernel<WAVES, MAXW, LOOP, false>, grid, block, kt_bytes, s, a,
+                   DeviceLens{0u});
     }
 }
 
