@@ -39,6 +39,15 @@ __device__ __forceinline__ float4 load4(const float *row, uint32_t d, uint32_t h
     return r;
 }
 
+/* The same for 16-byte aligned rows with head_dim a multiple of four, without a branch around the
+ * load: a branch there makes the compiler wait for every load in flight before the next one is
+ * issued, and a trip's loads are meant to travel together. */
+__device__ __forceinline__ float4 load4_aligned(const float *row, uint32_t d, uint32_t hd) {
+    const bool in = d < hd;
+    const float4 t = *reinterpret_cast<const float4 *>(row + (in ? d : 0u));
+    return in ? t : make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
 __device__ __forceinline__ void store4(float *row, uint32_t d, uint32_t hd, bool vec4, float4 x) {
     if (vec4) {
         if (d < hd) *reinterpret_cast<float4 *>(row + d) = x;
@@ -52,52 +61,19 @@ __device__ __forceinline__ void store4(float *row, uint32_t d, uint32_t hd, bool
 
 __device__ __forceinline__ float dot4(float4 a, float4 b) { return a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w; }
 
-/* SRC: where the workgroup finds its problem (attn_tile.h): a device array, the kernel arguments
- * (one problem), or the kernel arguments of a strided batch -- the last two need no trip to memory
- * before the row ranges and the rows themselves can be requested. */
-template <int G, int T, int SRC>
-__global__ __launch_bounds__(256) void attn_rows_kernel(const AttnProb *__restrict__ probs, uint32_t prob_base,
-                                                        AttnAffine aff) {
-    constexpr int ROWS_PER_WAVE = 64 / G;
-    constexpr int ROWS_PER_BLOCK = 4 * ROWS_PER_WAVE;
-
-    AttnProb p;
-    if (SRC == SRC_TILES) p = probs[prob_base + blockIdx.y];
-    else if (SRC == SRC_SINGLE) p = aff.first;
-    else affine_problem(p, aff, prob_base + blockIdx.y, aff.first.vis == ATTN_VIS_DENSE);
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t wave = threadIdx.x >> 6;
-    const uint32_t g = lane % G;
-    const uint32_t row = blockIdx.x * ROWS_PER_BLOCK + wave * ROWS_PER_WAVE + lane / G;
-    /* whole wave past the end: leave (uniform per wave) */
-    if (blockIdx.x * ROWS_PER_BLOCK + wave * ROWS_PER_WAVE >= p.nq) return;
-
-    const bool live = row < p.nq;
-    const uint32_t i = live ? row : p.nq - 1;
-    const bool vec4 = (p.flags & ATTN_FLAG_VEC4) != 0;
-
-    uint32_t lo, hi;
-    row_key_range(p, i, lo, hi);
-    if (!live) hi = lo;
-
-    float4 q[T], o[T];
-    const float *qrow = p.q + (size_t)i * p.q_stride;
-#pragma unroll
-    for (int t = 0; t < T; t++) {
-        q[t] = load4(qrow, 4u * (g + G * t), p.hd, vec4);
-        o[t] = make_float4(0.f, 0.f, 0.f, 0.f);
-    }
-
-    /* every group walks its own range, U keys per trip with all 2*U*T loads
-     * of the trip issued before any arithmetic; the wave makes as many trips
-     * as its longest row needs */
-    constexpr int U = T > 2 ? 1 : 4; /* very wide heads keep one key in flight: registers */
+/* One group's walk over its row's key range [lo, hi): U keys per trip with all loads of the trip
+ * issued before any arithmetic; the wave makes as many trips as its longest row needs.  A trip is
+ * a trip to memory -- at the sizes this kernel is the fast path for (a patch's 1..16 bytes per row)
+ * the whole range goes out in ONE, so U is sixteen for aligned rows at the common head widths.
+ * Rows with fewer keys repeat their last one (clamped address, weight zero): nothing in the trip
+ * sits behind a branch. */
+template <int G, int T, bool VEC4>
+__device__ __forceinline__ void rows_walk(const AttnProb &p, const float4 (&q)[T], float4 (&o)[T], float &m, float &l,
+                                          const uint32_t lo, const uint32_t hi, const float *mrow, const uint32_t g) {
+    constexpr int U = !VEC4 ? (T > 2 ? 1 : 4) : (T > 2 ? 1 : (T == 2 ? 4 : 16)); /* wide heads: fewer keys in flight (registers) */
     uint32_t trips = (hi - lo + U - 1) / U;
 #pragma unroll
     for (int off = G; off < 64; off <<= 1) trips = max(trips, (uint32_t)__shfl_xor((int)trips, off, 64));
-
-    float m = neg_inf(), l = 0.f;
-    const float *mrow = p.vis == ATTN_VIS_DENSE ? p.mask + (size_t)i * p.nk : nullptr;
     const uint32_t last = hi > lo ? hi - 1u : 0u; /* a readable key of this row (row 0 when it has none) */
 
     for (uint32_t trip = 0; trip < trips; trip++) {
@@ -112,8 +88,13 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const AttnProb *__restri
             const float *vrow = p.v + (size_t)jr * p.v_stride;
 #pragma unroll
             for (int t = 0; t < T; t++) {
-                kk[u][t] = load4(krow, 4u * (g + G * t), p.hd, vec4);
-                vv[u][t] = load4(vrow, 4u * (g + G * t), p.hd, vec4);
+                if constexpr (VEC4) {
+                    kk[u][t] = load4_aligned(krow, 4u * (g + G * t), p.hd);
+                    vv[u][t] = load4_aligned(vrow, 4u * (g + G * t), p.hd);
+                } else {
+                    kk[u][t] = load4(krow, 4u * (g + G * t), p.hd, false);
+                    vv[u][t] = load4(vrow, 4u * (g + G * t), p.hd, false);
+                }
             }
             bias[u] = mrow ? mrow[jr] : 0.f;
         }
@@ -154,6 +135,49 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const AttnProb *__restri
             m = mn;
         }
     }
+}
+
+/* SRC: where the workgroup finds its problem (attn_tile.h): a device array, the kernel arguments
+ * (one problem), or the kernel arguments of a strided batch -- the last two need no trip to memory
+ * before the row ranges and the rows themselves can be requested. */
+template <int G, int T, int SRC>
+__global__ __launch_bounds__(256) void attn_rows_kernel(const AttnProb *__restrict__ probs, uint32_t prob_base,
+                                                        AttnAffine aff) {
+    constexpr int ROWS_PER_WAVE = 64 / G;
+    constexpr int ROWS_PER_BLOCK = 4 * ROWS_PER_WAVE;
+
+    AttnProb p;
+    if (SRC == SRC_TILES) p = probs[prob_base + blockIdx.y];
+    else if (SRC == SRC_SINGLE) p = aff.first;
+    else affine_problem(p, aff, prob_base + blockIdx.y, aff.first.vis == ATTN_VIS_DENSE);
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t g = lane % G;
+    const uint32_t row = blockIdx.x * ROWS_PER_BLOCK + wave * ROWS_PER_WAVE + lane / G;
+    /* whole wave past the end: leave (uniform per wave) */
+    if (blockIdx.x * ROWS_PER_BLOCK + wave * ROWS_PER_WAVE >= p.nq) return;
+
+    const bool live = row < p.nq;
+    const uint32_t i = live ? row : p.nq - 1;
+    const bool vec4 = (p.flags & ATTN_FLAG_VEC4) != 0;
+
+    /* the query row is requested before the row's key range is read: the two travel together, and the
+     * keys' addresses wait for the range only */
+    float4 q[T], o[T];
+    const float *qrow = p.q + (size_t)i * p.q_stride;
+#pragma unroll
+    for (int t = 0; t < T; t++) {
+        q[t] = vec4 ? load4_aligned(qrow, 4u * (g + G * t), p.hd) : load4(qrow, 4u * (g + G * t), p.hd, false);
+        o[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    uint32_t lo, hi;
+    row_key_range(p, i, lo, hi);
+    if (!live) hi = lo;
+
+    float m = neg_inf(), l = 0.f;
+    const float *mrow = p.vis == ATTN_VIS_DENSE ? p.mask + (size_t)i * p.nk : nullptr;
+    if (vec4) rows_walk<G, T, true>(p, q, o, m, l, lo, hi, mrow, g);
+    else rows_walk<G, T, false>(p, q, o, m, l, lo, hi, mrow, g);
 
     if (live) {
         const float inv = l > 0.f ? 1.0f / l : 0.f;
