@@ -215,7 +215,7 @@ bool choose_fine(const AttnProb *p, uint32_t n, bool strided, uint32_t &span, bo
 /* Do problems p[0..n), all routed to the mfma family, go to the once kernel (16-row tiles whose keys
  * are all in flight at once)?  `span` gets the 16-key tiles its longest tile spans.  The kernel is
  * built for launches one trip to memory deep: it is chosen while the launch gives a compute unit
- * at most one workgroup. */
+ * one workgroup, or two short ones. */
 bool choose_once(const AttnProb *p, uint32_t n, uint32_t &span) {
     const int forced = family_override();
     if (forced != 0 && forced != 5) return false;
@@ -226,7 +226,10 @@ bool choose_once(const AttnProb *p, uint32_t n, uint32_t &span) {
         most = std::max(most, attn_once_span_tiles(p[i]));
         tiles += (p[i].nq + 15u) / 16u;
     }
-    if (forced == 0 && tiles > 256u) return false;
+    /* measured against the other matrix-core kernels (4 heads of 32 over 256 ... 1024 rows, 8 heads of 64
+     * over 128 rows, 1 ... 16 sequences): ahead up to 256 tiles whatever the rows' length (one workgroup
+     * per compute unit), up to 512 tiles while a row has at most 128 keys, behind beyond */
+    if (forced == 0 && tiles > (most <= 8u ? 512u : 256u)) return false;
     span = most;
     return true;
 }

@@ -423,7 +423,7 @@ __global__ __launch_bounds__(64 * W) void attn_once_kernel(const AttnProb *__res
 
 template <int HD, int W, int T, int SRC, bool DENSE>
 void once_launch_kernel(const AttnProb *dprobs, const AttnTile *dtiles, const AttnAffine &aff, uint32_t nblocks,
-                        hipStream_t s) {
+                        bool pieces, hipStream_t s) {
     using Shape = OnceShape<HD, W>;
     static const bool raised = [] { /* more than the 64 KB a kernel may use without asking */
         if (Shape::BYTES > 64u * 1024u)
@@ -432,31 +432,34 @@ void once_launch_kernel(const AttnProb *dprobs, const AttnTile *dtiles, const At
         return true;
     }();
     (void)raised;
-    blt_launch("attn_once", attn_once_kernel<HD, W, T, SRC, DENSE>, dim3(nblocks), dim3(64 * W), Shape::BYTES, s, dprobs,
-               dtiles, aff);
+    /* the piece tiles (mask in, weights out) sit at the end of the workgroup's LDS: a launch with neither
+     * does without them, and a fourth workgroup of eight waves then fits a compute unit */
+    const size_t lds = DENSE || pieces ? Shape::BYTES : Shape::BYTES - (size_t)W * 16 * Shape::MROW * sizeof(float);
+    blt_launch("attn_once", attn_once_kernel<HD, W, T, SRC, DENSE>, dim3(nblocks), dim3(64 * W), lds, s, dprobs, dtiles,
+               aff);
 }
 
 template <int HD, int W, int T, int SRC>
 void once_launch_as(const AttnProb *dprobs, const AttnTile *dtiles, const AttnAffine &aff, uint32_t nblocks, bool dense,
-                    hipStream_t s) {
-    if (dense) once_launch_kernel<HD, W, T, SRC, true>(dprobs, dtiles, aff, nblocks, s);
-    else once_launch_kernel<HD, W, T, SRC, false>(dprobs, dtiles, aff, nblocks, s);
+                    bool pieces, hipStream_t s) {
+    if (dense) once_launch_kernel<HD, W, T, SRC, true>(dprobs, dtiles, aff, nblocks, pieces, s);
+    else once_launch_kernel<HD, W, T, SRC, false>(dprobs, dtiles, aff, nblocks, pieces, s);
 }
 
 /* `tiles` = 16-key tiles the longest 16-row tile of the launch spans: sizes the workgroups */
 template <int SRC>
 void once_launch_shape(const AttnProb *dprobs, const AttnTile *dtiles, const AttnAffine &aff, uint32_t nblocks,
-                       uint32_t hd, uint32_t tiles, bool dense, hipStream_t s) {
+                       uint32_t hd, uint32_t tiles, bool dense, bool pieces, hipStream_t s) {
     BLT_REQUIRE(tiles <= attn_once_tiles_max(hd), "attention: internal: the once kernel was given rows it does not hold");
     if (hd == 32u) {
-        if (tiles <= 8u) once_launch_as<32, 8, 1, SRC>(dprobs, dtiles, aff, nblocks, dense, s);
-        else if (tiles <= 16u) once_launch_as<32, 16, 1, SRC>(dprobs, dtiles, aff, nblocks, dense, s);
-        else if (tiles <= 32u) once_launch_as<32, 16, 2, SRC>(dprobs, dtiles, aff, nblocks, dense, s);
-        else once_launch_as<32, 16, 4, SRC>(dprobs, dtiles, aff, nblocks, dense, s);
+        if (tiles <= 8u) once_launch_as<32, 8, 1, SRC>(dprobs, dtiles, aff, nblocks, dense, pieces, s);
+        else if (tiles <= 16u) once_launch_as<32, 16, 1, SRC>(dprobs, dtiles, aff, nblocks, dense, pieces, s);
+        else if (tiles <= 32u) once_launch_as<32, 16, 2, SRC>(dprobs, dtiles, aff, nblocks, dense, pieces, s);
+        else once_launch_as<32, 16, 4, SRC>(dprobs, dtiles, aff, nblocks, dense, pieces, s);
     } else {
-        if (tiles <= 8u) once_launch_as<64, 8, 1, SRC>(dprobs, dtiles, aff, nblocks, dense, s);
-        else if (tiles <= 16u) once_launch_as<64, 16, 1, SRC>(dprobs, dtiles, aff, nblocks, dense, s);
-        else once_launch_as<64, 16, 2, SRC>(dprobs, dtiles, aff, nblocks, dense, s);
+        if (tiles <= 8u) once_launch_as<64, 8, 1, SRC>(dprobs, dtiles, aff, nblocks, dense, pieces, s);
+        else if (tiles <= 16u) once_launch_as<64, 16, 1, SRC>(dprobs, dtiles, aff, nblocks, dense, pieces, s);
+        else once_launch_as<64, 16, 2, SRC>(dprobs, dtiles, aff, nblocks, dense, pieces, s);
     }
 }
 
@@ -525,7 +528,8 @@ void attn_once_launch(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t n
     if (ntiles == 0) return;
     AttnAffine none;
     __builtin_memset(&none, 0, sizeof(none));
-    once_launch_shape<SRC_TILES>(dprobs, dtiles, none, ntiles, hd, span_tiles, dense, s);
+    /* a list may hold problems that want their weights: the piece tiles stay */
+    once_launch_shape<SRC_TILES>(dprobs, dtiles, none, ntiles, hd, span_tiles, dense, true, s);
 }
 
 void attn_once_launch_single(const AttnProb &single, hipStream_t s) {
@@ -535,7 +539,7 @@ void attn_once_launch_single(const AttnProb &single, hipStream_t s) {
     __builtin_memset(&a, 0, sizeof(a));
     a.first = single;
     once_launch_shape<SRC_SINGLE>(nullptr, nullptr, a, nblocks, single.hd, attn_once_span_tiles(single),
-                                  single.vis == ATTN_VIS_DENSE, s);
+                                  single.vis == ATTN_VIS_DENSE, single.weights != nullptr, s);
 }
 
 void attn_once_launch_affine(const AttnAffine &aff, hipStream_t s) {
@@ -548,5 +552,5 @@ void attn_once_launch_affine(const AttnAffine &aff, hipStream_t s) {
     a.reserved = aff.count < 8u && nqt <= 32u ? 8u : 0u;
     const uint32_t nblocks = (a.reserved ? a.reserved : aff.count) * nqt;
     once_launch_shape<SRC_AFFINE>(nullptr, nullptr, a, nblocks, aff.first.hd, attn_once_span_tiles(aff.first),
-                                  aff.first.vis == ATTN_VIS_DENSE, s);
+                                  aff.first.vis == ATTN_VIS_DENSE, aff.first.weights != nullptr, s);
 }
