@@ -138,15 +138,8 @@ Family choose_family(const AttnProb &d) {
  * unit one (short rows: few key tiles per item) or two (long rows: the
  * latency-oriented mfma kernel, which splits the keys of a 32-row tile over
  * its waves, keeps the shorter serial chain for longer) -- measured
- * crossovers: 128..256 items at 128 keys, 256..512 items at 512 keys.
- * BLT_HIP_WIDE_MIN_GROUPS overrides the threshold. */
+ * crossovers: 128..256 items at 128 keys, 256..512 items at 512 keys. */
 uint32_t wide_min_groups(uint32_t max_nk) {
-    static const uint32_t pinned = [] {
-        const char *e = getenv("BLT_HIP_WIDE_MIN_GROUPS");
-        const long v = e ? std::atol(e) : 0;
-        return v > 0 ? (uint32_t)v : 0u;
-    }();
-    if (pinned) return pinned;
     return max_nk <= 256u ? 256u : 512u;
 }
 
@@ -238,22 +231,16 @@ bool choose_once(const AttnProb *p, uint32_t n, uint32_t &span) {
  * four-wave workgroup per problem of at most 128 rows whose keys fit one LDS fill)?  It fetches
  * K and V once per problem and balances the causal triangle inside the workgroup, which pays once
  * the batch is several workgroups deep on every compute unit.  BLT_HIP_FINE_ROWS=128 pins it
- * wherever the shape allows (tuning and test hook), BLT_HIP_WHOLE_MIN moves the threshold. */
+ * wherever the shape allows (tuning and test hook). */
 bool choose_whole(const AttnProb &d, uint32_t n, bool strided) {
     static const int rows_pinned = [] {
         const char *e = getenv("BLT_HIP_FINE_ROWS");
         return e ? std::atoi(e) : 0;
     }();
-    static const uint32_t min_problems = [] {
-        const char *e = getenv("BLT_HIP_WHOLE_MIN");
-        const long v = e ? std::atol(e) : 0;
-        return v > 0 ? (uint32_t)v : 0u;
-    }();
     const int forced = family_override();
     if (!strided || (forced != 0 && forced != 4) || !attn_whole_can(d)) return false;
     if (rows_pinned != 0) return rows_pinned == 128;
     if (forced != 0 || d.nq < 48u) return false; /* three row halves and fewer leave most of the waves idle */
-    if (min_problems) return n >= min_problems;
     /* measured against the family's other shapes and the wide kernel (8 heads of 64 and 4 heads
      * of 32): 128 rows ahead from 144 problems on (11.9 against 12.4 us; 12.5 against 15.6 at
      * 256, 38.7 against 45.5 at 1024, 72.5 against 86 at 2048), 64 rows from 768 on */

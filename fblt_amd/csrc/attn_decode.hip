@@ -407,19 +407,11 @@ void launch_step(StepArgs a, uint32_t batch, hipStream_t s) {
     blt_launch("kv_step", kv_step_kernel<G, NQ, WAVES>, grid, dim3(64 * waves), lds, s, a);
 }
 
-/* tuning hooks: BLT_HIP_DECODE_WAVES = 4|8|16 waves per workgroup (decode
- * rows only), BLT_HIP_DECODE_SPAN = sub-chunks of 32 keys per split */
-int env_int(const char *name, int fallback) {
-    const char *e = getenv(name);
-    return e && *e ? atoi(e) : fallback;
-}
-
 template <int G>
 void dispatch_nq(const StepArgs &a, uint32_t nq, uint32_t batch, hipStream_t s) {
     /* single rows: one wave per head, and a second slice of waves once a split
      * holds enough keys to keep both busy */
-    static const int pinned_waves = env_int("BLT_HIP_DECODE_WAVES", 0);
-    const int waves = pinned_waves > 0 ? pinned_waves : (a.hpb == 1u ? 16 : a.span >= 256u ? 8 : 4);
+    const int waves = a.hpb == 1u ? 16 : a.span >= 256u ? 8 : 4;
     if (nq <= 1) {
         if (waves >= 16) launch_step<G, 1, 16>(a, batch, s);
         else if (waves >= 8) launch_step<G, 1, 8>(a, batch, s);
@@ -579,7 +571,6 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
     a.block_kind = step_kind == BLT_KV_STEP_BLOCK;
     a.hpb = 0, a.slices = 1;
 
-    static const int span_env = env_int("BLT_HIP_DECODE_SPAN", 0);
     const size_t subs = (max_len_hint + SUB - 1) / SUB;
 
     /* Lengths on the host (the reference keeps self_len there, csrc/infer/kv_cache.h:56-60): they
@@ -607,15 +598,13 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
     }
     /* Single rows of a batch that one workgroup per (sequence, head) spreads over the chip: the
      * waves of a workgroup slice one head's keys and meet once in LDS, nothing crosses workgroups
-     * but the length ticket.  BLT_HIP_DECODE_ROW=0 keeps the split layout (tuning hook). */
-    static const int row_env = env_int("BLT_HIP_DECODE_ROW", 1);
-    /* measured against the split layout at 32 / 64 / 128 sequences of 4 heads: ahead or level up to
+     * but the length ticket.
+     * Measured against the split layout at 32 / 64 / 128 sequences of 4 heads: ahead or level up to
      * 8192 cached keys with up to 256 (sequence, head) pairs (21.2 against 24.2 us at 32 x 2048..4096,
      * 35.5 against 39.4 at 64), with 512 pairs ahead at 2048 keys (33.2 against 39.2) and behind at
      * 4096 (86.1 against 81.8) */
     const size_t pairs = cache->batch * H;
-    if (n_seq == 1 && span_env == 0 &&
-        (row_env == 2 || (row_env == 1 && subs >= 4 && pairs >= 128 && pairs <= 512 && subs <= (pairs <= 256 ? 256u : 96u)))) {
+    if (n_seq == 1 && subs >= 4 && pairs >= 128 && pairs <= 512 && subs <= (pairs <= 256 ? 256u : 96u)) {
         a.splits = 1, a.span = 0, a.q0 = 0, a.write_through = 1, a.commit = commit;
         a.cap = (uint32_t)std::min<size_t>((size_t)cache->max_seq_len, rope_cos ? rope_positions : (size_t)UINT32_MAX);
         acquire_scratch(a, 0, cache->batch, static_scratch);
@@ -630,7 +619,6 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
      * sub-chunks */
     size_t splits = (1024 + cache->batch - 1) / cache->batch;
     splits = std::min<size_t>(splits, (subs + 1) / 2);
-    if (span_env > 0) splits = (subs + span_env - 1) / span_env;
     splits = std::max<size_t>(1, std::min<size_t>(splits, MAX_SPLITS));
     const size_t span_subs = (subs + splits - 1) / splits;
     splits = (subs + span_subs - 1) / span_subs;
@@ -639,10 +627,8 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
     a.hpb = 0;
     /* Single rows of a batch that one workgroup per (sequence, head) already
      * spreads over the chip: all 16 waves of a workgroup slice one head's keys
-     * and merge through LDS, so nothing crosses workgroups but the ticket.
-     * BLT_HIP_DECODE_HPB=0 keeps the split layout (tuning hook). */
-    static const int hpb_env = env_int("BLT_HIP_DECODE_HPB", 1);
-    if (hpb_env == 1 && a.n == 1u && span_env == 0 && subs >= 4 && subs <= 64 && cache->batch * H >= 128 &&
+     * and merge through LDS, so nothing crosses workgroups but the ticket. */
+    if (a.n == 1u && subs >= 4 && subs <= 64 && cache->batch * H >= 128 &&
         cache->batch * H <= 512) {
         a.hpb = 1;
         a.splits = 1;
@@ -675,8 +661,7 @@ void kv_step_slice(const blt_kv_attn_cache *cache, const float *q_rows, size_t q
          * (measured at 1..16 sequences: 10.4 against 17.8 us at 500 keys, 13.6 against 18.1 at
          * 1000, even at 2000; 16.7 against 30 us at 4000 keys with 16 sub-chunks per split). */
         size_t bs = 1;
-        if (span_env > 0) bs = (subs + span_env - 1) / span_env;
-        else if (subs > 64) bs = std::min<size_t>((256 + cache->batch * zblocks - 1) / (cache->batch * zblocks), (subs + 15) / 16);
+        if (subs > 64) bs = std::min<size_t>((256 + cache->batch * zblocks - 1) / (cache->batch * zblocks), (subs + 15) / 16);
         bs = std::max<size_t>(1, std::min<size_t>(bs, MAX_SPLITS));
         const size_t bspan = (subs + bs - 1) / bs;
         a.splits = (uint32_t)((subs + bspan - 1) / bspan);

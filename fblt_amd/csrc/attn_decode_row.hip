@@ -193,11 +193,6 @@ __global__ __launch_bounds__(64 * W) void kv_row_kernel(StepArgs a, LensArg<KARG
     }
 }
 
-int env_int(const char *name, int fallback) {
-    const char *e = getenv(name);
-    return e && *e ? atoi(e) : fallback;
-}
-
 template <int G, int W>
 void launch_row(const StepArgs &a, uint32_t batch, const uint32_t *host_lens, hipStream_t s) {
     dim3 grid(a.num_heads, batch, 1);
@@ -222,14 +217,12 @@ void launch_row_waves(const StepArgs &a, uint32_t batch, const uint32_t *host_le
 /* One new row per sequence, one workgroup per (sequence, head).  `host_lens` (batch entries, at
  * most KARG_SEQS) or NULL for the device lengths in a.self_len.  max_keys sizes the
  * workgroups (measured at 64 sequences x 4 heads x <= 790 keys: 5.2 us with 8 waves, 5.5 with 16,
- * 6.0 with 4; at 128 sequences x 1024..2048 keys: 33.8 us with 16 waves, 34.4 with 8, 35.8 with 4;
- * BLT_HIP_ROW_WAVES pins the count). */
+ * 6.0 with 4; at 128 sequences x 1024..2048 keys: 33.8 us with 16 waves, 34.4 with 8, 35.8 with 4). */
 bool kv_row_launch(const StepArgs &a, uint32_t batch, uint32_t head_dim, const uint32_t *host_lens, uint32_t max_keys,
                    hipStream_t s) {
-    static const int pinned = env_int("BLT_HIP_ROW_WAVES", 0);
     const uint32_t keys_per_wave = head_dim >= 128 ? 8u : head_dim >= 64 ? 16u : head_dim >= 8 ? 32u : 64u;
     const uint32_t rounds = (max_keys + keys_per_wave - 1) / keys_per_wave;
-    const uint32_t waves = pinned > 0 ? (uint32_t)pinned : rounds > 32 ? 16u : rounds > 4 ? 8u : 4u;
+    const uint32_t waves = rounds > 32 ? 16u : rounds > 4 ? 8u : 4u;
     switch (head_dim) {
     case 4: launch_row_waves<1>(a, batch, host_lens, waves, s); break;
     case 8: launch_row_waves<2>(a, batch, host_lens, waves, s); break;

@@ -534,11 +534,8 @@ void launch_variant(const AttnProb *dprobs, const AttnTile *dtiles, uint32_t nbl
     const dim3 grid(nblocks);
     if constexpr (HD == 32) {
         /* fewer workgroups than the compute units can spread: eight waves each (their K tiles fit
-         * LDS at this head dim).  BLT_HIP_MFMA_WAVES8_BELOW overrides the workgroup count (tuning hook). */
-        static const uint32_t below = [] {
-            const char *e = getenv("BLT_HIP_MFMA_WAVES8_BELOW");
-            return e && *e ? (uint32_t)atoi(e) : 320u; /* measured: ahead up to 256 workgroups, level at 512 */
-        }();
+         * LDS at this head dim); measured: ahead up to 256 workgroups, level at 512 */
+        constexpr uint32_t below = 320u;
         if (exact && nblocks < below) {
             if (dense)
                 blt_launch("attn_mfma", attn_mfma_kernel<HD, SRC, true, true, 8>, grid, dim3(512), 0, s, dprobs, dtiles,
@@ -579,12 +576,8 @@ bool attn_mfma_takes(const AttnProb &d) {
     /* per-row ranges are short (a patch's bytes) unless the caller says otherwise: the rows family
      * reads less.  Document-causal self-attention comes as ranges as long as the document: measured
      * at 128 ... 2048 rows, both head widths, the two families are level at ranges of 16 keys, this
-     * one is 1.5 times faster at 32 and 9 ... 13 times at 512 and more
-     * (BLT_HIP_RANGE_SPAN_MIN moves the limit: tuning hook). */
-    static const uint32_t span_min = [] {
-        const char *e = getenv("BLT_HIP_RANGE_SPAN_MIN");
-        return e && *e ? (uint32_t)atol(e) : 24u;
-    }();
+     * one is 1.5 times faster at 32 and 9 ... 13 times at 512 and more. */
+    constexpr uint32_t span_min = 24u;
     if (d.vis == ATTN_VIS_RANGE && d.range_span < span_min) return false;
     return d.nq >= 16u;
 }

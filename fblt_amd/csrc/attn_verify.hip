@@ -979,20 +979,15 @@ void launch_block_as(StepArgs a, uint32_t batch, const uint32_t *host_lens, hipS
     /* Long sequences of unequal lengths, more (sequence, head) pairs than compute units, lengths
      * known here: a launch of one workgroup per sequence and head pair ends with its longest
      * sequence (2032 keys against a mean of 1528 is a quarter of the time lost), so the pairs
-     * become workgroups of their own, handed out longest first.  BLT_HIP_BLOCK_BY_LENGTH=0|1
-     * switches it off / on wherever it applies (tuning and test hook). */
+     * become workgroups of their own, handed out longest first. */
     KargLens lens;
     a.by_length = 0;
     if (NARROW && host_lens && a.splits == 1u && a.num_heads >= 2u && batch >= 2u) {
-        static const int pinned = [] {
-            const char *e = getenv("BLT_HIP_BLOCK_BY_LENGTH");
-            return e && *e ? atoi(e) : -1;
-        }();
         uint32_t shortest = host_lens[0], longest = host_lens[0];
         for (uint32_t b = 1; b < batch; b++)
             shortest = std::min(shortest, host_lens[b]), longest = std::max(longest, host_lens[b]);
         const bool pays = (uint64_t)batch * a.num_heads > 256u && subs >= 32u && (longest - shortest) * 5u >= longest;
-        if (pinned < 0 ? pays : pinned != 0) {
+        if (pays) {
             a.by_length = 1;
             a.hpb = 1;
             uint32_t idx[KARG_SEQS];

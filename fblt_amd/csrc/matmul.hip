@@ -652,20 +652,13 @@ enum Path { PATH_SKINNY, PATH_SPLITK, PATH_MFMA };
 Path choose_path(const MatmulArgs &g) {
     const bool rope = g.rope_cos != nullptr && g.rope_cols > 0;
     /* up to this many rows the thread-per-column kernel, whose sums run in the reference's order
-     * (bit-identical results); BLT_HIP_EXACT_PRODUCT_ROWS lowers it (0: matrix cores for every shape) */
-    static const uint32_t exact_rows = [] {
-        const char *e = getenv("BLT_HIP_EXACT_PRODUCT_ROWS");
-        return e && *e ? (uint32_t)atoi(e) : 32u;
-    }();
+     * (bit-identical results) */
+    constexpr uint32_t exact_rows = 32u;
     if (g.m <= exact_rows && !rope && !g.tolerant) return PATH_SKINNY;
     /* up to 143 64x64 tiles (a bit over half the compute units): quarter tiles, K split over the
      * waves.  Measured at K = 512 ... 4096: a fifth faster than the 64x64 kernel at 128 tiles, level
-     * with it at 144 ... 192, a quarter slower at 256 (BLT_HIP_MATMUL_SPLITK_BELOW moves the limit:
-     * tuning hook) */
-    static const uint64_t splitk_below = [] {
-        const char *e = getenv("BLT_HIP_MATMUL_SPLITK_BELOW");
-        return e && *e ? (uint64_t)atoll(e) : (uint64_t)144u;
-    }();
+     * with it at 144 ... 192, a quarter slower at 256 */
+    constexpr uint64_t splitk_below = 144u;
     if ((uint64_t)((g.n + TN - 1) / TN) * ((g.m + TM - 1) / TM) < splitk_below) return PATH_SPLITK;
     return PATH_MFMA;
 }
@@ -709,17 +702,11 @@ bool slice_scratch(MatmulArgs &g, size_t tiles, hipStream_t s) {
  * with a serial chain of chunk loads (2048 x 512 weights under 118 rows: 64 tiles, eight chunks per
  * wave).  As many slices as keep one chunk per wave and give one workgroup per compute unit: measured
  * over 12 ... 256 tiles and K = 1024 ... 4096, the best count was the one that brought the launch
- * to about 256 workgroups, and more made it slower again.
- * BLT_HIP_MATMUL_KSLICES=1 switches them off, n > 1 forces n: tuning hook. */
+ * to about 256 workgroups, and more made it slower again. */
 uint32_t slices_for(const MatmulArgs &g, dim3 grid, bool eight) {
-    static const int forced = [] {
-        const char *e = getenv("BLT_HIP_MATMUL_KSLICES");
-        return e && *e ? atoi(e) : 0;
-    }();
     if (g.b2 || g.cross_k || g.norm_w) return 1u;
     const uint32_t chunks = (g.k + 31u) / 32u, tiles = grid.x * grid.y;
     const uint32_t room = chunks / (eight ? 8u : 4u);
-    if (forced >= 1) return std::max(1u, std::min((uint32_t)forced, std::min(room, 64u)));
     if (chunks < 32u || tiles > 128u) return 1u;
     return std::max(1u, std::min(room, 256u / tiles));
 }
@@ -792,13 +779,8 @@ void launch_mfma_as(dim3 grid, hipStream_t s, const MatmulArgs &g) {
 }
 template <bool VEC, bool ROPE, int WT>
 void launch_mfma(dim3 grid, hipStream_t s, const MatmulArgs &g) {
-    /* BLT_HIP_MATMUL_WAVES=4 keeps four waves per small tile: tuning hook */
-    static const bool eight = [] {
-        const char *e = getenv("BLT_HIP_MATMUL_WAVES");
-        return !(e && atoi(e) == 4);
-    }();
     if constexpr (WT == 1) {
-        if (eight && g.k >= 256u) { /* from eight K steps on: below, the meeting of the sums costs what the overlap gains */
+        if (g.k >= 256u) { /* from eight K steps on: below, the meeting of the sums costs what the overlap gains */
             launch_mfma_as<VEC, ROPE, 1, 8>(grid, s, g);
             return;
         }
@@ -841,24 +823,16 @@ void matmul_f32_launch(const MatmulArgs &g, hipStream_t s) {
         }
         return;
     }
-    /* 128x128 tiles once there are enough of them to load every compute unit twice over
-     * (BLT_HIP_MATMUL_TILE=64 keeps the 64x64 tiles: tuning hook) */
-    static const bool big_ok = [] {
-        const char *e = getenv("BLT_HIP_MATMUL_TILE");
-        return !(e && atoi(e) == 64);
-    }();
+    /* 128x128 tiles once there are enough of them to load every compute unit twice over */
     const uint32_t tx = (g.n + 2 * TN - 1) / (2 * TN), ty = (g.m + 2 * TM - 1) / (2 * TM);
-    static const uint64_t big_from = [] { /* BLT_HIP_MATMUL_BIG_FROM: tuning hook */
-        const char *e = getenv("BLT_HIP_MATMUL_BIG_FROM");
-        return e && *e ? (uint64_t)atoll(e) : (uint64_t)512u;
-    }();
+    constexpr uint64_t big_from = 512u;
     /* Two large tiles are resident per compute unit, 512 at a time: a last round that fills less
      * than three eighths of the chip costs more than the large tile gains (576 tiles, 6144 x 512 .
      * 512 x 1536: 106 us against 92 with the small tile; 640: 106 / 104; 960: 142 / 151) until the
      * rounds are many. */
     const uint64_t big_tiles = (uint64_t)tx * ty, last_round = big_tiles % 512u;
     const bool short_tail = big_tiles < 2048u && last_round != 0u && last_round < 192u;
-    if (big_ok && big_tiles >= big_from && !short_tail) {
+    if (big_tiles >= big_from && !short_tail) {
         const dim3 grid(tx, ty);
         if (rope) {
             if (vec) launch_mfma<true, true, 2>(grid, s, g);
