@@ -21,7 +21,7 @@ PROBES_SRC = os.path.join(HERE, "probes", "probes.hip")
 PROBES_LIB = os.path.join(LIBDIR, "libfblt_probes.so")
 
 HIP_SOURCES = ["memory.hip", "mask_builder.hip", "vecmath.hip", "attn_rows.hip", "attn_mfma.hip", "attn_wide.hip", "attn_fine.hip", "attn_once.hip", "matmul.hip", "rope.hip", "mha.hip", "layer_ops.hip", "encoder.hip", "stream.hip",
-               "attn_decode.hip", "attn_decode_row.hip", "attn_verify.hip", "attn_api.hip", "profile.hip"]
+               "attn_decode.hip", "attn_decode_row.hip", "attn_verify.hip", "attn_verify_once.hip", "attn_api.hip", "profile.hip"]
 C_SOURCES = ["host/blt_host.c"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

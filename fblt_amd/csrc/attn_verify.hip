@@ -703,9 +703,9 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
  *                    column; register r of lane (block, j) ends up with key 4 block + r, query j;
  *   O[query, d]:     instruction (beta, r) broadcasts the weights of key 4 beta + r (lower eight
  *                    blocks) and key 32 + 4 beta + r (upper eight) as A; lane l supplies column
- *                    l % 32 of that key's V row as B (32 lanes = the row's 128 bytes, one dword
- *                    load); register i of lane l accumulates O[query i][column l % 32] over the
- *                    lane's half of the keys.  One accumulator of four registers; the two halves
+ *                    l % 32 of that key's V row as B (the V rows reach the lanes like the K rows:
+ *                    coalesced loads, then the wave's LDS tile); register i of lane l accumulates
+ *                    O[query i][column l % 32] over the lane's half of the keys.  One accumulator of four registers; the two halves
  *                    meet once, after the loop, with one row swap.
  *
  * The sequence is walked as ceil(len / 64) sub-chunks of cached rows followed by one with the new
@@ -760,11 +760,14 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
     /* kg[v]: piece lane % 8 of the sub-chunk's row 8 v + lane / 8 -- consecutive lanes on consecutive
      * 16-byte pieces of a row; a load whose lanes each touch another row (lane = key, as the S^T
      * product wants the rows) is served at a quarter of the rate, and eight of those per sub-chunk
-     * were most of what the longest sequences waited for.  vr[4 beta + r]: column dcol of row
-     * 32 half + 4 beta + r.  Rows past the last one are clamped to it (their weights are zero).
-     * Base, pitch and limit are scalar selects: every load is scalar base + 32-bit lane offset. */
+     * were most of what the longest sequences waited for.  vg[v]: the same piece of the same row of V
+     * (the O product wants column dcol of row 32 half + 4 beta + r in lane (half, dcol): a load of that
+     * shape moves 256 bytes per instruction, and thirty-two of them per sub-chunk kept the compute
+     * unit's vector memory path busier than the K rows did).  Rows past the last one are clamped to it
+     * (their weights are zero).  Base, pitch and limit are scalar selects: every load is scalar base +
+     * 32-bit lane offset. */
     const uint32_t krow_l = lane >> 3, kpiece = lane & 7u;
-    auto request = [&](floatx4 (&kg)[8], float (&vr)[32], uint32_t si) __attribute__((always_inline)) {
+    auto request = [&](floatx4 (&kg)[8], floatx4 (&vg)[8], uint32_t si) __attribute__((always_inline)) {
         const bool fresh = si >= cached_subs;
         const char *kb = fresh ? new_k : cache_k, *vb = fresh ? new_v : cache_v;
         const uint32_t kp = fresh ? newk_pitch : cache_pitch, vp = fresh ? newv_pitch : cache_pitch;
@@ -772,11 +775,9 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
 #pragma unroll
         for (int v = 0; v < 8; v++)
             kg[v] = *reinterpret_cast<const floatx4 *>(kb + __umul24(min(row0 + 8u * v + krow_l, limit), kp) + 16u * kpiece);
-        const uint32_t vrow0 = min(row0 + 32u * half, limit);
-        const uint32_t room = limit - vrow0; /* rows this half may step forward */
-        const uint32_t voff0 = __umul24(vrow0, vp) + 4u * dcol;
 #pragma unroll
-        for (int t = 0; t < 32; t++) vr[t] = *reinterpret_cast<const float *>(vb + (__umul24(min((uint32_t)t, room), vp) + voff0));
+        for (int v = 0; v < 8; v++)
+            vg[v] = *reinterpret_cast<const floatx4 *>(vb + __umul24(min(row0 + 8u * v + krow_l, limit), vp) + 16u * kpiece);
     };
 
     /* The query rows: lanes 0..3 (block 0) hold row `lane` whole; the S^T instructions hand block
@@ -803,9 +804,8 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
      * unit's vector memory path (64 bytes a cycle) is what the longest sequences wait for -- and
      * park a neutral record.  LOOP = true: sub-chunks round-robin, the next one requested ahead. */
     uint32_t si = s_begin + slice;
-    floatx4 kg[8];
-    float vr[32];
-    if (LOOP || si < s_end) request(kg, vr, si); /* before anything waits for memory */
+    floatx4 kg[8], vg[8];
+    if (LOOP || si < s_end) request(kg, vg, si); /* before anything waits for memory */
     float *const my_kt = sm_kt4 + wave * (32 * KROW);
 
     const uint32_t qi = a.q0 + li;
@@ -824,8 +824,8 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
     for (int r = 0; r < 4; r++) oacc[r] = 0.f;
     float m = neg_inf(), l = 0.f;
 
-    /* one sub-chunk whose rows sit in kr / vr */
-    auto attend = [&](floatx4 (&kg)[8], float (&vr)[32], uint32_t si) __attribute__((always_inline)) {
+    /* one sub-chunk whose rows sit in kg / vg */
+    auto attend = [&](floatx4 (&kg)[8], floatx4 (&vg)[8], uint32_t si) __attribute__((always_inline)) {
         const bool fresh = si >= cached_subs;
         const uint32_t j0 = fresh ? len : si * CH; /* absolute position of the sub-chunk's first key */
         const uint32_t j_end = fresh ? nk : len;   /* rows past it are clamped repeats */
@@ -840,13 +840,11 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
                                                   a.rope_sin + at);
                     kg[v][0] = t.x, kg[v][1] = t.y, kg[v][2] = t.z, kg[v][3] = t.w;
                 }
-                if (a.write_through && head_ok && real)
-                    *reinterpret_cast<floatx4 *>(a.cache_k + (slab + len + r) * a.embed_dim + head * HD + 4u * kpiece) = kg[v];
-            }
-            if (a.write_through && head_ok && half == 0u) {
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-                    if ((uint32_t)r < a.n) a.cache_v[(slab + len + r) * a.embed_dim + head * HD + dcol] = vr[r];
+                if (a.write_through && head_ok && real) {
+                    const size_t at = (slab + len + r) * a.embed_dim + head * HD + 4u * kpiece;
+                    *reinterpret_cast<floatx4 *>(a.cache_k + at) = kg[v];
+                    *reinterpret_cast<floatx4 *>(a.cache_v + at) = vg[v];
+                }
             }
         }
         /* rows -> the lanes that contract them, 32 rows at a time through the wave's own LDS tile (LDS
@@ -860,6 +858,18 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
             if (half == (uint32_t)h2) {
 #pragma unroll
                 for (int e = 0; e < 8; e++) kr[e] = *reinterpret_cast<const float4 *>(my_kt + (lane & 31u) * KROW + 4 * e);
+            }
+        }
+        /* the V rows the same way: lane (half, dcol) ends up with column dcol of rows 32 half ... 32 half + 31 */
+        float vr[32];
+#pragma unroll
+        for (int h2 = 0; h2 < 2; h2++) {
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+                *reinterpret_cast<floatx4 *>(my_kt + (8u * v + krow_l) * KROW + 4u * kpiece) = vg[4 * h2 + v];
+            if (half == (uint32_t)h2) {
+#pragma unroll
+                for (int t = 0; t < 32; t++) vr[t] = my_kt[t * KROW + dcol];
             }
         }
 
@@ -936,18 +946,15 @@ __global__ __launch_bounds__(64 * MAXW, 1) void kv_block4_mfma_kernel(StepArgs a
     };
 
     if constexpr (!LOOP) {
-        if (si < s_end) attend(kg, vr, si);
+        if (si < s_end) attend(kg, vg, si);
     } else {
         while (si < s_end) {
-            floatx4 kn[8];
-            float vn[32];
+            floatx4 kn[8], vn[8];
             request(kn, vn, si + a.slices); /* past the end the clamped rows hit the cache; no branch */
             __builtin_amdgcn_sched_barrier(0);
-            attend(kg, vr, si);
+            attend(kg, vg, si);
 #pragma unroll
-            for (int e = 0; e < 8; e++) kg[e] = kn[e];
-#pragma unroll
-            for (int t = 0; t < 32; t++) vr[t] = vn[t];
+            for (int e = 0; e < 8; e++) kg[e] = kn[e], vg[e] = vn[e];
             si += a.slices;
         }
     }
@@ -1083,11 +1090,20 @@ uint32_t kv_block_heads_per_group(uint32_t batch, uint32_t subs, uint32_t num_he
 bool kv_block_mfma_launch(const StepArgs &a, uint32_t batch, uint32_t head_dim, const uint32_t *host_lens,
                           hipStream_t s) {
     /* the per-wave K tiles bound the workgroups: 8 waves of 4.6 KB or 4 of 8.7 KB */
-    /* BLT_HIP_BLOCK_TILE=16 keeps blocks of up to four rows on the 16-wide tiles (test hook) */
-    static const bool no_tile4 = [] {
+    /* BLT_HIP_BLOCK_TILE=16 keeps blocks of up to four rows on the 16-wide tiles, =4 keeps the looping
+     * kernels (4x4x1 tiles up to four rows, 16-wide above), =once takes the all-at-once kernel wherever
+     * the shape allows (test hooks) */
+    static const int pin = [] {
         const char *e = getenv("BLT_HIP_BLOCK_TILE");
-        return e && (strcmp(e, "16") == 0 || strcmp(e, "32") == 0);
+        return !e ? 0 : strcmp(e, "once") == 0 ? 1 : strcmp(e, "4") == 0 ? 4 : strcmp(e, "16") == 0 ? 16 : strcmp(e, "32") == 0 ? 32 : 0;
     }();
+    const bool no_tile4 = pin == 16 || pin == 32;
+    /* All at once wherever the shape allows, ahead of the looping 16-wide kernel (64 sequences x 4 heads
+     * over 64 ... 508 cached keys: 7.0 against 8.0 us at 8 rows, 7.2 against 8.6 at 16); up to four rows
+     * of head width 32 the 4x4x1 kernel, which has no padding rows to multiply, stays ahead (6.4 against
+     * 6.9 us). */
+    const bool small = head_dim == 32u && a.n - a.q0 <= 4u;
+    if ((pin == 1 || (pin == 0 && !small)) && kv_block_once_launch(a, batch, head_dim, host_lens, s)) return true;
     if (head_dim == 32u) {
         if (a.n - a.q0 <= 4u && !no_tile4) launch_block4(a, batch, host_lens, s);
         else if (!narrow_block(a)) launch_block_as<32, 8, false>(a, batch, host_lens, s);

@@ -220,6 +220,11 @@ uint32_t kv_block_heads_per_group(uint32_t batch, uint32_t subs, uint32_t num_he
 bool kv_block_mfma_launch(const StepArgs &a, uint32_t batch, uint32_t head_dim, const uint32_t *host_lens,
                           hipStream_t s);
 
+/* block steps of at most 16 rows over a prefix short enough to be requested all at once
+ * (attn_verify_once.hip); false when it does not take the shape */
+bool kv_block_once_launch(const StepArgs &a, uint32_t batch, uint32_t head_dim, const uint32_t *host_lens,
+                          hipStream_t s);
+
 /* single-row steps with one workgroup per (sequence, head) (attn_decode_row.hip): lengths from
  * `host_lens` (at most KARG_SEQS sequences, carried in the kernel arguments; nothing is
  * committed) or, when NULL, from a.self_len with the commit through a.tickets; max_keys sizes

@@ -733,19 +733,21 @@ def test_rope_position_gather(dev):
     assert (got_c == cos[pos]).all() and (got_s == sin[pos]).all()
 
 
-@pytest.mark.parametrize("kernel", ["valu", "mfma", "mfma32"])
+@pytest.mark.parametrize("kernel", ["valu", "mfma", "mfma_once", "mfma_loop", "mfma32"])
 def test_kv_step_kernel_families_agree(kernel):
-    """The kernels behind the KV step entry points (VALU, matrix-core with 16-wide tiles for blocks of
-    up to 16 rows, matrix-core with 32-wide tiles only) on the same cases -- block rows, prefill
-    chunks, rotation fused in or not -- pinned through BLT_HIP_BLOCK_KERNEL / BLT_HIP_BLOCK_TILE in a
-    fresh process (the hooks are read once)."""
+    """The kernels behind the KV step entry points (VALU; matrix-core as routed; the all-at-once kernel
+    wherever it takes the shape; the looping kernels only -- 4x4x1 tiles up to four rows, 16-wide tiles
+    up to 16; 32-wide tiles only) on the same cases -- block rows, prefill chunks, rotation fused in or
+    not -- pinned through BLT_HIP_BLOCK_KERNEL / BLT_HIP_BLOCK_TILE in a fresh process (the hooks are
+    read once)."""
     import subprocess
     import sys
     import os
     here = os.path.dirname(os.path.abspath(__file__))
     env = dict(os.environ, BLT_HIP_BLOCK_KERNEL=kernel[:4])
-    if kernel == "mfma32":
-        env["BLT_HIP_BLOCK_TILE"] = "32"
+    tile = {"mfma32": "32", "mfma_once": "once", "mfma_loop": "4"}.get(kernel)
+    if tile:
+        env["BLT_HIP_BLOCK_TILE"] = tile
     p = subprocess.run([sys.executable, "-u", os.path.join(here, "kv_family_cases.py")], capture_output=True,
                        text=True, timeout=600, env=env)
     assert p.returncode == 0 and "OK" in p.stdout, p.stdout[-2000:] + p.stderr[-2000:]
