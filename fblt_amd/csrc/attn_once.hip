@@ -152,10 +152,11 @@ __global__ __launch_bounds__(64 * W) void attn_once_kernel(const AttnProb *__res
     const uint32_t ntiles = (p.nk + 15u) / 16u;
     const uint32_t last_key = p.nk - 1u;
 
-    /* ---- every request of the wave, before anything waits.  Rows of Q, K and the mask are asked
+    /* ---- every request of the wave, before anything waits.  Rows of Q, K, V and the mask are asked
      * for with consecutive lanes on consecutive 16-byte pieces of a row (a load whose lanes each
-     * touch another row is served at a quarter of the rate) and turned into matrix fragments
-     * through the wave's own LDS tile; V rows are contiguous per sixteen lanes as they are. ---- */
+     * touch another row is served at a quarter of the rate, and the compute unit's one vector memory
+     * path is what a tile with many keys waits for: the fewest instructions that move the bytes) and
+     * turned into matrix fragments through the wave's own LDS tile. ---- */
     constexpr int LPR = HD / 4;   /* lanes per row when the wave moves a tile */
     constexpr int RPI = 64 / LPR; /* rows one load instruction covers         */
     const uint32_t prow = lane / LPR, pf = lane % LPR;
@@ -163,11 +164,10 @@ __global__ __launch_bounds__(64 * W) void attn_once_kernel(const AttnProb *__res
     float *const tile = sm_o + wave * (16 * ROW);          /* becomes the wave's partial output later */
     float *const mtile = sm_o + W * (16 * ROW) + wave * (16 * Shape::MROW);
 
-    floatx4 qg[NV], kg[T][NV], mg[T]; /* native vectors: arrays of the float4 struct were kept in scratch memory */
+    floatx4 qg[NV], kg[T][NV], vg[T][NV], mg[T]; /* native vectors: arrays of the float4 struct were kept in scratch memory */
 #pragma unroll
     for (int v = 0; v < NV; v++)
         qg[v] = *reinterpret_cast<const floatx4 *>(p.q + (size_t)min(q0 + prow + (uint32_t)(RPI * v), p.nq - 1u) * p.q_stride + 4u * pf);
-    float vf[T][DT][4];
     /* A tile past the span repeats the span's last tile: the loads hit the cache, nothing is computed.
      * The mask pieces go first: theirs is the only branch among the requests, and what is requested
      * after it is counted exactly when the scores wait for K but not yet for V. */
@@ -198,17 +198,9 @@ __global__ __launch_bounds__(64 * W) void attn_once_kernel(const AttnProb *__res
     for (int u = 0; u < T; u++) {
         const uint32_t kt = min(t0 + wave + (uint32_t)(W * u), t1 > 0u ? t1 - 1u : 0u);
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const float *vrow = p.v + (size_t)min(16u * kt + 4u * g + r, last_key) * p.v_stride + DT * c;
-            if constexpr (DT == 2) {
-                const float2 t = *reinterpret_cast<const float2 *>(vrow);
-                vf[u][0][r] = t.x, vf[u][1][r] = t.y;
-            } else {
-                static_assert(DT == 4, "head widths 32 and 64");
-                const float4 t = *reinterpret_cast<const float4 *>(vrow);
-                vf[u][0][r] = t.x, vf[u][1][r] = t.y, vf[u][2][r] = t.z, vf[u][3][r] = t.w;
-            }
-        }
+        for (int v = 0; v < NV; v++)
+            vg[u][v] = *reinterpret_cast<const floatx4 *>(
+                p.v + (size_t)min(16u * kt + prow + (uint32_t)(RPI * v), last_key) * p.v_stride + 4u * pf);
     }
 
     /* ---- fragments: lane (g, c) holds floats [g QD, (g + 1) QD) of row c.  The tile is the wave's
@@ -292,6 +284,28 @@ __global__ __launch_bounds__(64 * W) void attn_once_kernel(const AttnProb *__res
 #pragma unroll
                     for (int a = 0; a < NA; a++)
                         sa[u][a] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[u][s + a], qf[s + a], sa[u][a], 0, 0, 0);
+            }
+        }
+    }
+    /* while the matrix cores work on the scores: the V rows -> fragments through the same tile; element
+     * (d, r) of tile u is column DT c + d of row 4 g + r -- the key whose weight register r of the scores
+     * holds, so P^T needs no exchange */
+    float vf[T][DT][4];
+#pragma unroll
+    for (int u = 0; u < T; u++) {
+#pragma unroll
+        for (int v = 0; v < NV; v++)
+            *reinterpret_cast<floatx4 *>(tile + (prow + (uint32_t)(RPI * v)) * ROW + 4u * pf) = vg[u][v];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const float *vrow = tile + (4u * g + r) * ROW + DT * c;
+            if constexpr (DT == 2) {
+                const float2 t = *reinterpret_cast<const float2 *>(vrow);
+                vf[u][0][r] = t.x, vf[u][1][r] = t.y;
+            } else {
+                static_assert(DT == 4, "head widths 32 and 64");
+                const float4 t = *reinterpret_cast<const float4 *>(vrow);
+                vf[u][0][r] = t.x, vf[u][1][r] = t.y, vf[u][2][r] = t.z, vf[u][3][r] = t.w;
             }
         }
     }
