@@ -485,15 +485,16 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
     const float *const new_v = a.v_rows + newrow0 * a.v_stride + hsafe * HD;
     const uint32_t cache_pitch = a.embed_dim * 4u, newk_pitch = a.k_stride * 4u, newv_pitch = a.v_stride * 4u;
     const uint32_t last_cached = len > 0u ? len - 1u : 0u, last_new = a.n - 1u;
-    const uint32_t lane_k = g * (QD * 4u), lane_v = c * (DT * 4u); /* byte offsets inside a row */
+    const uint32_t lane_k = g * (QD * 4u); /* byte offset inside a row */
 
     /* K rows of sub-chunk si as the wave moves them: load v covers rows KRI v ... KRI v + KRI - 1 with
      * consecutive lanes on consecutive 16-byte pieces of a row (lanes that each touch another row
      * are served at a quarter of the rate); they become fragments through the wave's LDS tile.
-     * V fragment: element (e, 4 t + r) is column DT c + e of row 16 t + 4 g + r -- sixteen lanes on one
-     * row's contiguous bytes as it is. */
+     * The V rows the same way (as fragments -- element (e, 4 t + r) is column DT c + e of row
+     * 16 t + 4 g + r -- a load moves half the bytes per instruction at head width 32, and the
+     * compute unit's vector memory path is what a long sequence waits for). */
     const uint32_t krow_l = lane / KL, kpiece = lane % KL;
-    auto request = [&](floatx4 (&kg)[KNV], float (&vf)[DT][8], uint32_t si) __attribute__((always_inline)) {
+    auto request = [&](floatx4 (&kg)[KNV], floatx4 (&vg)[KNV], uint32_t si) __attribute__((always_inline)) {
         const bool fresh = si >= cached_subs; /* wave-uniform: scalar selects */
         const char *kb = reinterpret_cast<const char *>(fresh ? new_k : cache_k);
         const char *vb = reinterpret_cast<const char *>(fresh ? new_v : cache_v);
@@ -505,24 +506,16 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
             kg[v] = *reinterpret_cast<const floatx4 *>(kb + off);
         }
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
-            const uint32_t off = min(row0 + 16u * (u >> 2) + (u & 3) + 4u * g, limit) * vp + lane_v;
-            if constexpr (DT == 2) {
-                const float2 x = *reinterpret_cast<const float2 *>(vb + off);
-                vf[0][u] = x.x, vf[1][u] = x.y;
-            } else {
-                static_assert(DT == 4, "head widths 32 and 64");
-                const float4 x = *reinterpret_cast<const float4 *>(vb + off);
-                vf[0][u] = x.x, vf[1][u] = x.y, vf[2][u] = x.z, vf[3][u] = x.w;
-            }
+        for (int v = 0; v < KNV; v++) {
+            const uint32_t off = min(row0 + (uint32_t)(KRI * v) + krow_l, limit) * vp + 16u * kpiece;
+            vg[v] = *reinterpret_cast<const floatx4 *>(vb + off);
         }
     };
 
     /* the first sub-chunk's rows are requested before anything else waits for memory */
     uint32_t si = s_begin + slice;
-    floatx4 kg[KNV];
-    float vf[DT][8];
-    request(kg, vf, si);
+    floatx4 kg[KNV], vg[KNV];
+    request(kg, vg, si);
 
     /* query fragment: row c of the block (clamped), columns [g*QD, (g+1)*QD) of the head */
     const uint32_t qi = a.q0 + c;
@@ -576,18 +569,10 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
                                                   a.rope_sin + at);
                     kg[v][0] = t.x, kg[v][1] = t.y, kg[v][2] = t.z, kg[v][3] = t.w;
                 }
-                if (a.write_through && head_ok && real)
-                    *reinterpret_cast<floatx4 *>(a.cache_k + (slab + len + r) * a.embed_dim + head * HD + 4u * kpiece) = kg[v];
-            }
-            if (a.write_through && head_ok) {
-#pragma unroll
-                for (int u = 0; u < 8; u++) {
-                    const uint32_t r = 16u * (u >> 2) + 4u * g + (u & 3);
-                    if (r < a.n) {
-                        float *dst = a.cache_v + (slab + len + r) * a.embed_dim + head * HD + DT * c;
-                        if constexpr (DT == 2) *reinterpret_cast<float2 *>(dst) = make_float2(vf[0][u], vf[1][u]);
-                        else *reinterpret_cast<float4 *>(dst) = make_float4(vf[0][u], vf[1][u], vf[2][u], vf[3][u]);
-                    }
+                if (a.write_through && head_ok && real) {
+                    const size_t at = (slab + len + r) * a.embed_dim + head * HD + 4u * kpiece;
+                    *reinterpret_cast<floatx4 *>(a.cache_k + at) = kg[v];
+                    *reinterpret_cast<floatx4 *>(a.cache_v + at) = vg[v];
                 }
             }
         }
@@ -604,10 +589,25 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
                 const float4 x = *reinterpret_cast<const float4 *>(my_kt + (16u * t + c) * KROW + g * QD + s);
                 kf[t][s + 0] = x.x, kf[t][s + 1] = x.y, kf[t][s + 2] = x.z, kf[t][s + 3] = x.w;
             }
+        float vf[DT][8];
+#pragma unroll
+        for (int v = 0; v < KNV; v++)
+            *reinterpret_cast<floatx4 *>(my_kt + ((uint32_t)(KRI * v) + krow_l) * KROW + 4u * kpiece) = vg[v];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const float *vrow = my_kt + (16u * (u >> 2) + (u & 3) + 4u * g) * KROW + DT * c;
+            if constexpr (DT == 2) {
+                const float2 x = *reinterpret_cast<const float2 *>(vrow);
+                vf[0][u] = x.x, vf[1][u] = x.y;
+            } else {
+                static_assert(DT == 4, "head widths 32 and 64");
+                const float4 x = *reinterpret_cast<const float4 *>(vrow);
+                vf[0][u] = x.x, vf[1][u] = x.y, vf[2][u] = x.z, vf[3][u] = x.w;
+            }
+        }
         /* the next sub-chunk's rows travel while this one is worked on: the raw rows have left their
-         * registers, the values move into a second set */
-        float vn[DT][8];
-        request(kg, vn, si + a.slices);
+         * registers */
+        request(kg, vg, si + a.slices);
         __builtin_amdgcn_sched_barrier(0); /* the requests stay ahead of the arithmetic */
 
         floatx4 sacc[2];
@@ -655,11 +655,6 @@ __global__ __launch_bounds__(64 * WAVES, 1) void kv_block16_mfma_kernel(StepArgs
 #pragma unroll
             for (int d = 0; d < DT; d++)
                 oacc[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[d][u], x[u], oacc[d], 0, 0, 0);
-
-#pragma unroll
-        for (int d = 0; d < DT; d++)
-#pragma unroll
-            for (int u = 0; u < 8; u++) vf[d][u] = vn[d][u];
         si += a.slices;
     }
 
