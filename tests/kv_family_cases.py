@@ -46,6 +46,13 @@ CASES = {
     "chunk70_window_hd64": lambda: chunked(70, True, hd=64, window=50),
     "block8_rope": lambda: workloads.config5(batch=9, B=8, rope=True),
     "block16_rope_hd64": lambda: workloads.config5(batch=5, B=16, H=2, hd=64, rope=True),
+    # the shapes around the all-at-once kernel's limits: caches of one or two rows (one cached tile and
+    # the tile of new rows, four waves), a prefix of four tiles per wave, one past what it holds (the looping kernels
+    # take over), a block of one row short of a tile at head width 64
+    "block7_tiny_cache": lambda: workloads.config5(batch=6, B=7, len_lo=1, len_hi=2, max_seq_len=64),
+    "block16_prefix_900": lambda: workloads.config5(batch=3, B=16, len_lo=700, len_hi=990, max_seq_len=1024),
+    "block16_prefix_1100": lambda: workloads.config5(batch=3, B=16, len_lo=1000, len_hi=1100, max_seq_len=1200),
+    "block15_hd64_prefix_400": lambda: workloads.config5(batch=4, B=15, H=2, hd=64, len_lo=100, len_hi=400, max_seq_len=512),
 }
 
 
