@@ -523,16 +523,18 @@ __global__ __launch_bounds__(64 * WAVES, 4) void attn_fine_kernel(const AttnProb
 }
 
 /* Whole short problems (at most 128 query rows, keys that fit one fill), for strided batches of
- * so many of them that throughput matters and the launch floor does not: the workgroup -- four
+ * so many of them that throughput matters and the launch floor does not: the workgroup -- eight
  * waves -- fetches the problem's K and V rows ONCE into LDS, meets once, and from there on its
- * waves run on their own.  Wave w takes the row halves (of 16 rows) n-1-w and w, one after the
- * other: under a causal mask the two add up to the same number of units for every wave, and a
- * half's keys are all the wave's own, so nothing is merged; the finished rows go to global
- * memory straight from the accumulators.  Two workgroups fit a compute unit (LDS), so one
- * fetches while the other computes. */
+ * waves run on their own.  A wave takes one row half (of 16 rows): wave w the half n-1-w, wave
+ * w + 4, which shares its SIMD, the half w -- under a causal mask the two add up to the same
+ * number of units on every SIMD, and a half's keys are all the wave's own, so nothing is merged;
+ * the finished rows go to global memory straight from the accumulators.  Two workgroups fit a
+ * compute unit (LDS), four waves on every SIMD: a wave's softmax and LDS waits are another's
+ * matrix instructions (four waves of two halves each, one after the other: 22.5 / 36.3 / 72.5 us
+ * at 512 / 1024 / 2048 problems of 128 rows x 64 columns against 20.4 / 35.2 / 62.0 now). */
 template <int HD>
 struct WholeShape {
-    static constexpr uint32_t THREADS = 256;
+    static constexpr uint32_t THREADS = 512;
     static constexpr uint32_t MAX_ROWS = 128;
     static constexpr uint32_t KC_MAX = FineShape<HD, 2, 8>::KC_MAX;
     static constexpr int ROW = HD + 4, LPR4 = HD / 4;
@@ -540,7 +542,7 @@ struct WholeShape {
 };
 
 template <int HD>
-__global__ __launch_bounds__(256, 2) void attn_whole_kernel(AttnAffine aff, uint32_t kc) {
+__global__ __launch_bounds__(512, 2) void attn_whole_kernel(AttnAffine aff, uint32_t kc) {
     using Shape = WholeShape<HD>;
     constexpr int ROW = Shape::ROW, LPR4 = Shape::LPR4, QD = HD / 4, DT = HD / 16;
     extern __shared__ __attribute__((aligned(16))) float sm[];
@@ -570,10 +572,12 @@ __global__ __launch_bounds__(256, 2) void attn_whole_kernel(AttnAffine aff, uint
     const uint32_t key_end = thi > tlo ? (thi + 15u) / 16u * 16u : 0u;
     const uint32_t last_key = min(max(key_end, 1u), p.nk) - 1u;
 
-    /* the wave's two row halves; hb == NONE: one half, ha == NONE: nothing */
+    /* The wave's row half, NONE: nothing.  Waves w and w + 4 sit on one SIMD: w takes half n-1-w, w + 4
+     * takes half w, which under a causal mask add up to the same number of units on every SIMD. */
     constexpr uint32_t NONE = 0xFFFFFFFFu;
-    const uint32_t ha = wave < halves && halves - 1u - wave >= wave ? halves - 1u - wave : NONE;
-    const uint32_t hb = ha != NONE && ha > wave ? wave : NONE;
+    const uint32_t pw = wave & 3u;
+    const uint32_t far = pw < halves && halves - 1u - pw >= pw ? halves - 1u - pw : NONE;
+    const uint32_t ha = wave < 4u ? far : (far != NONE && far > pw ? pw : NONE);
 
     auto load_q = [&](float (&qf)[QD], const uint32_t half) __attribute__((always_inline)) {
         const uint32_t row = min(16u * (half == NONE ? 0u : half) + c, p.nq - 1u);
@@ -584,9 +588,8 @@ __global__ __launch_bounds__(256, 2) void attn_whole_kernel(AttnAffine aff, uint
             qf[s + 0] = t.x, qf[s + 1] = t.y, qf[s + 2] = t.z, qf[s + 3] = t.w;
         }
     };
-    float qa[QD], qb[QD];
+    float qa[QD];
     load_q(qa, ha);
-    load_q(qb, hb);
 
     /* ---- the fill: every piece is requested, then parked in the order it was requested ---- */
     float4 kp[Shape::PIECES], vp[Shape::PIECES];
@@ -599,7 +602,7 @@ __global__ __launch_bounds__(256, 2) void attn_whole_kernel(AttnAffine aff, uint
         vp[t] = *reinterpret_cast<const float4 *>(p.v + (size_t)j * p.v_stride + 4u * f);
     }
 #pragma unroll
-    for (int s = 0; s < QD; s++) asm volatile("" : "+v"(qa[s]), "+v"(qb[s]));
+    for (int s = 0; s < QD; s++) asm volatile("" : "+v"(qa[s]));
     /* the pieces go to the lambda by value: indexed inside it, the arrays would live in scratch memory */
     auto park = [&](const uint32_t pc, const float4 k_piece, const float4 v_piece) __attribute__((always_inline)) {
         const uint32_t e = tid + Shape::THREADS * pc;
@@ -668,7 +671,6 @@ __global__ __launch_bounds__(256, 2) void attn_whole_kernel(AttnAffine aff, uint
         }
     };
     if (ha != NONE) run_half(qa, ha);
-    if (hb != NONE) run_half(qb, hb);
 }
 
 /* keys per fill for a launch whose longest tile needs `span` keys */
@@ -784,7 +786,7 @@ void attn_whole_launch_affine(const AttnAffine &aff, hipStream_t s) {
             return true;
         }();
         (void)raised;
-        blt_launch("attn_whole", attn_whole_kernel<32>, dim3(aff.count), dim3(256), lds, s, aff, kc);
+        blt_launch("attn_whole", attn_whole_kernel<32>, dim3(aff.count), dim3(WholeShape<32>::THREADS), lds, s, aff, kc);
     } else {
         const size_t lds = (size_t)2 * kc * WholeShape<64>::ROW * sizeof(float);
         static const bool raised = [] {
@@ -794,7 +796,7 @@ void attn_whole_launch_affine(const AttnAffine &aff, hipStream_t s) {
             return true;
         }();
         (void)raised;
-        blt_launch("attn_whole", attn_whole_kernel<64>, dim3(aff.count), dim3(256), lds, s, aff, kc);
+        blt_launch("attn_whole", attn_whole_kernel<64>, dim3(aff.count), dim3(WholeShape<64>::THREADS), lds, s, aff, kc);
     }
 }
 
