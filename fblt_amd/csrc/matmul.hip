@@ -795,7 +795,6 @@ void matmul_f32_launch(const MatmulArgs &g, hipStream_t s) {
     const Path path = choose_path(g);
     BLT_REQUIRE(g.b2 == nullptr || path != PATH_MFMA, "matmul: the gated product is not available for this shape");
     BLT_REQUIRE(g.norm_w == nullptr || matmul_takes_norm(g), "matmul: the fused row norm is not available for this shape");
-    const dim3 block(256);
     if (path == PATH_SKINNY) {
         BLT_REQUIRE(g.cross_k == nullptr || (matmul_takes_cross(g) && g.cross_v && g.cross_out && g.cross_lo &&
                                              g.cross_hi && g.cross_rows_per_seq >= 1u),
