@@ -13,8 +13,8 @@ CPU baseline (the reference's own attention core where its build travelled
 with the tree, else the checker under oracle/; one host core, bounded sample),
 the other two parts of the composite metric (decode us/step, verify tokens/s)
 and one summary row per attention shape under "per_config".  The full
-per-workload records go to stderr as they are measured and, together, to
-gpurun_out/bench_detail.json.
+per-workload records go to stderr as they are measured and, together, to the
+file --detail names.
 """
 import argparse
 import json
